@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Benchmark of the headline metric: Hyrax row commitment of a quantised weight matrix
+(BASELINE.json configs[1]) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one full commitment of a 4096 x 4096 int16-range matrix (sigma = 2^10, clipped) against
+4096 seeded generators through the C ABI (grape_commit_i32, small-scalar fast path), inputs
+already resident in HBM.  One JSON line is printed with the throughput in Mpoints/s
+(points = matrix elements), the roofline of the dominant kernel (accumulation kernel; its
+duration is measured live with HIP events on the launch stream) and the CPU oracle timed on a
+bounded sample of rows of the same workload on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+ROWS = 4096
+COLS = 4096
+SIGMA = 1024.0
+SEED_W = 20240001
+SEED_G = 20240002
+RADIX_BITS = 16        # one signed 16-bit digit per scalar
+K_DIGIT = 32768
+
+# Algorithmic work per committed point, the reference's algorithm (two non-zero byte windows of an
+# int16 scalar, each a mixed XYZZ addition of 8M+2S, 300 32x32 multiplies per 12-limb Montgomery
+# product): 2 * 10 * 300.
+ALG_MULS_PER_POINT = 6000
+# What the fast path executes: one mixed addition per point.
+EXEC_MULS_PER_POINT = 3000
+# lane-level 32x32 multiplies per second if every SIMD issued one v_mad_u64_u32 per cycle:
+# 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz
+PEAK_MULS_NOMINAL = 256 * 64 * 2.4e9
+
+
+def gaussian_i16(shape, seed, sigma=SIGMA):
+    rng = np.random.default_rng(seed)
+    x = np.rint(rng.normal(0.0, sigma, size=shape))
+    return np.clip(x, -32768, 32767).astype(np.int32)
+
+
+def seeded_scalars(n, seed):
+    """n canonical scalars < r from a seeded generator (rejection sampling of 255-bit draws)."""
+    from gpuutil import rand_fr
+    return rand_fr(n, seed)
+
+
+def cpu_baseline(W, gens_dev, ops, budget_s=15.0):
+    """The CPU oracle (reference algorithm: byte-window table, OpenMP over rows) on a bounded
+    sample of rows of the same matrix; also checks the GPU result of those rows."""
+    import orc
+    table_dev = ops.g1_table_gen(gens_dev, 256)
+    ops.sync()
+    table = ops.g1_to_host(table_dev)          # 256 x 4096 affine points, the reference's table format
+    del table_dev
+    threads = orc.lib().orc_num_threads()
+    probe = max(threads, 8)
+    t0 = time.perf_counter()
+    first = orc.commit_i32(W[:probe], table, COLS, COLS)
+    dt = time.perf_counter() - t0
+    rows = int(min(ROWS, max(probe, (budget_s / max(dt, 1e-6)) * probe)))
+    rows -= rows % probe
+    rows = max(rows, probe)
+    t0 = time.perf_counter()
+    out = orc.commit_i32(W[:rows], table, COLS, COLS)
+    dt = time.perf_counter() - t0
+    assert np.array_equal(out[:probe], first)
+    return {"value": rows * COLS / dt / 1e6, "unit": "Mpoints/s", "cores": threads, "kind": "port",
+            "sample": "first %d of %d rows (x %d columns) of the same matrix, %.1f s" % (rows, ROWS, COLS, dt)}, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
+              "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
+        return 2
+
+    import torch
+    from grape_amd import ops
+    ops.init(0)
+
+    # ---- synthetic inputs, resident in HBM before the timed region
+    W = gaussian_i16((ROWS, COLS), SEED_W)
+    dW = torch.from_numpy(W).cuda()
+    gens = ops.g1_make_generators(seeded_scalars(COLS, SEED_G))
+    ops.sync()
+    t0 = time.perf_counter()
+    table = ops.g1_wide_table_gen(gens, RADIX_BITS, 1, K_DIGIT)
+    ops.sync()
+    table_gen_s = time.perf_counter() - t0
+    out = ops.g1_empty(ROWS)
+
+    def step():
+        ops.commit_i32(dW, COLS, table, COLS, RADIX_BITS, 1, K_DIGIT, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    points = ROWS * COLS
+    value = points / (ms_per_step * 1e-3) / 1e6
+
+    # ---- dominant kernel, HIP events on the launch stream inside the library
+    ops.profile_enable(True)
+    kern_ms = []
+    for _ in range(max(3, min(args.steps, 10))):
+        step()
+        kern_ms.append(ops.profile_last())
+    ops.profile_enable(False)
+    acc_ms = float(np.mean([k[0] for k in kern_ms]))
+    red_ms = float(np.mean([k[1] for k in kern_ms]))
+    peak_measured = ops.bench_mad(16384, 512, 5)
+    achieved_alg = ALG_MULS_PER_POINT * points / (acc_ms * 1e-3)
+    achieved_exec = EXEC_MULS_PER_POINT * points / (acc_ms * 1e-3)
+    roofline = {
+        "bound": "valu_int32_mul",
+        "kernel": "commit_wide_kernel<int32>",
+        "achieved": achieved_alg / 1e12,
+        "peak": peak_measured / 1e12,
+        "unit": "Tmul/s",
+        "frac": achieved_alg / peak_measured,
+        "traffic": None,
+        "achieved_executed": achieved_exec / 1e12,
+        "frac_executed": achieved_exec / peak_measured,
+        "peak_nominal": PEAK_MULS_NOMINAL / 1e12,
+        "peak_source": "v_mad_u64_u32 issue-rate microbenchmark measured in this run "
+                       "(no published integer-multiply peak exists for MI355X)",
+        "kernel_ms": acc_ms,
+        "reduce_kernel_ms": red_ms,
+    }
+
+    result = {
+        "metric": "hyrax_commit_throughput",
+        "value": value,
+        "unit": "Mpoints/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: Hyrax commit of a 4096x4096 int16-range matrix "
+                               "(Gaussian sigma=2^10, clipped), 4096 seeded G1 generators, "
+                               "small-scalar path, 4096 affine outputs",
+                   "rows": ROWS, "cols": COLS, "radix_bits": RADIX_BITS,
+                   "table_bytes": int(table.numel()) * 4, "table_gen_s": table_gen_s},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu_baseline:
+        base, cpu_out = cpu_baseline(W, gens, ops)
+        got = ops.g1_to_host(out)[: cpu_out.shape[0]]
+        if not np.array_equal(got, cpu_out):
+            print("bench.py: GPU commitments differ from the CPU oracle on the sampled rows", file=sys.stderr)
+            return 1
+        result["cpu_baseline"] = base
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,55 @@
+// Shared host-side plumbing of the C-ABI translation units: error reporting, launch geometry
+// and the per-device scratch pool.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/grape_hip.h"
+#include "curve.hpp"
+#include "field.hpp"
+
+namespace grape {
+
+void set_error(const char* fmt, ...);
+
+#define GRAPE_HIP_CHECK(expr)                                                              \
+    do {                                                                                   \
+        hipError_t _e = (expr);                                                            \
+        if (_e != hipSuccess) {                                                            \
+            ::grape::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),      \
+                               __FILE__, __LINE__);                                        \
+            return GRAPE_EHIP;                                                             \
+        }                                                                                  \
+    } while (0)
+
+#define GRAPE_REQUIRE(cond, msg)                                                           \
+    do {                                                                                   \
+        if (!(cond)) {                                                                     \
+            ::grape::set_error("%s: %s", __func__, msg);                                   \
+            return GRAPE_EINVAL;                                                           \
+        }                                                                                  \
+    } while (0)
+
+#define GRAPE_LAUNCH_CHECK() GRAPE_HIP_CHECK(hipGetLastError())
+
+static inline hipStream_t as_stream(grape_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+constexpr int kBlock = 256;          // 4 wave64 per workgroup
+constexpr int kNumCU = 256;          // MI355X
+static inline unsigned blocks_for(size_t n, int per_block = kBlock) {
+    return (unsigned)((n + per_block - 1) / per_block);
+}
+
+// Scratch pool: one growing device allocation per slot, reused across calls so the hot path
+// never allocates.  Slots are independent buffers (a call may use several at once).
+enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kNumSlots = 5 };
+int scratch_get(ScratchSlot slot, size_t bytes, void** out);
+bool initialised();
+
+// Optional per-kernel event timing (see grape_profile_enable).
+bool profiling();
+void profile_begin();                     // forget the previous call's marks
+int profile_mark(hipStream_t s);          // record an event; kernels sit between consecutive marks
+
+}  // namespace grape

@@ -12,6 +12,47 @@
 
 namespace grape {
 
+// Fp products used by the group law.  A translation unit may route them through out-of-line
+// device functions (GRAPE_FP_MUL_OUTLINE) to keep kernels small: one shared multiplier body
+// instead of a copy per call site.  The default is the inline multiplier.
+#if defined(GRAPE_FP_MUL_OUTLINE) && defined(__HIP_DEVICE_COMPILE__)
+__device__ __noinline__ Fp fp_mul_outline(Fp a, Fp b);
+__device__ __noinline__ Fp fp_sqr_outline(Fp a);
+__device__ __forceinline__ Fp fmul(const Fp& a, const Fp& b) { return fp_mul_outline(a, b); }
+__device__ __forceinline__ Fp fsqr(const Fp& a) { return fp_sqr_outline(a); }
+#else
+GRAPE_HD Fp fmul(const Fp& a, const Fp& b) { return mul(a, b); }
+GRAPE_HD Fp fsqr(const Fp& a) { return sqr(a); }
+#endif
+
+// a^(p-2) with the hooked multiplier (4-bit fixed windows, rolled loops).
+GRAPE_HD Fp fp_inverse(const Fp& a) {
+    Fp tbl[16];
+    tbl[0] = Fp::one();
+    tbl[1] = a;
+    for (int i = 2; i < 16; i++) tbl[i] = fmul(tbl[i - 1], a);
+    Fp acc = Fp::one();
+    bool started = false;
+    for (int limb = 11; limb >= 0; limb--) {
+        uint32_t e = 0;
+        for (int k = 0; k < 12; k++) e = (k == limb) ? FpParams::pm2(k) : e;
+        for (int nib = 7; nib >= 0; nib--) {
+            if (started) {
+                acc = fsqr(acc);
+                acc = fsqr(acc);
+                acc = fsqr(acc);
+                acc = fsqr(acc);
+            }
+            uint32_t w = (e >> (4 * nib)) & 15u;
+            if (w) {
+                acc = fmul(acc, tbl[w]);
+                started = true;
+            }
+        }
+    }
+    return acc;
+}
+
 struct alignas(16) G1Affine {
     Fp x, y;
     GRAPE_HD bool is_inf() const { return x.is_zero() & y.is_zero(); }
@@ -68,28 +109,28 @@ GRAPE_HD void xyzz_add_affine(G1Xyzz& acc, const G1Affine& p, bool negate) {
         acc.zzz = Fp::one();
         return;
     }
-    Fp P = sub(mul(p.x, acc.zz), acc.x);   // U2 - X1
-    Fp R = sub(mul(py, acc.zzz), acc.y);   // S2 - Y1
+    Fp P = sub(fmul(p.x, acc.zz), acc.x);   // U2 - X1
+    Fp R = sub(fmul(py, acc.zzz), acc.y);   // S2 - Y1
     if (!P.is_zero()) {
-        Fp PP = sqr(P);
-        Fp PPP = mul(P, PP);
-        Fp Q = mul(acc.x, PP);
-        Fp X3 = sub(sub(sub(sqr(R), PPP), Q), Q);
-        Fp Y3 = sub(mul(R, sub(Q, X3)), mul(acc.y, PPP));
-        acc.zz = mul(acc.zz, PP);
-        acc.zzz = mul(acc.zzz, PPP);
+        Fp PP = fsqr(P);
+        Fp PPP = fmul(P, PP);
+        Fp Q = fmul(acc.x, PP);
+        Fp X3 = sub(sub(sub(fsqr(R), PPP), Q), Q);
+        Fp Y3 = sub(fmul(R, sub(Q, X3)), fmul(acc.y, PPP));
+        acc.zz = fmul(acc.zz, PP);
+        acc.zzz = fmul(acc.zzz, PPP);
         acc.x = X3;
         acc.y = Y3;
     } else if (R.is_zero()) {
         // same point: double the affine operand
         Fp U = dbl(py);
-        Fp V = sqr(U);
-        Fp W = mul(U, V);
-        Fp S = mul(p.x, V);
-        Fp M = sqr(p.x);
+        Fp V = fsqr(U);
+        Fp W = fmul(U, V);
+        Fp S = fmul(p.x, V);
+        Fp M = fsqr(p.x);
         M = add(add(M, M), M);
-        Fp X3 = sub(sub(sqr(M), S), S);
-        Fp Y3 = sub(mul(M, sub(S, X3)), mul(W, py));
+        Fp X3 = sub(sub(fsqr(M), S), S);
+        Fp Y3 = sub(fmul(M, sub(S, X3)), fmul(W, py));
         acc.x = X3;
         acc.y = Y3;
         acc.zz = V;
@@ -107,17 +148,17 @@ GRAPE_HD void xyzz_dbl(G1Xyzz& acc) {
         acc = G1Xyzz::inf();
         return;
     }
-    Fp V = sqr(U);
-    Fp W = mul(U, V);
-    Fp S = mul(acc.x, V);
-    Fp M = sqr(acc.x);
+    Fp V = fsqr(U);
+    Fp W = fmul(U, V);
+    Fp S = fmul(acc.x, V);
+    Fp M = fsqr(acc.x);
     M = add(add(M, M), M);
-    Fp X3 = sub(sub(sqr(M), S), S);
-    Fp Y3 = sub(mul(M, sub(S, X3)), mul(W, acc.y));
+    Fp X3 = sub(sub(fsqr(M), S), S);
+    Fp Y3 = sub(fmul(M, sub(S, X3)), fmul(W, acc.y));
     acc.x = X3;
     acc.y = Y3;
-    acc.zz = mul(V, acc.zz);
-    acc.zzz = mul(W, acc.zzz);
+    acc.zz = fmul(V, acc.zz);
+    acc.zzz = fmul(W, acc.zzz);
 }
 
 // acc += q, both XYZZ. 12M + 2S on the common path.
@@ -127,18 +168,18 @@ GRAPE_HD void xyzz_add(G1Xyzz& acc, const G1Xyzz& q) {
         acc = q;
         return;
     }
-    Fp U1 = mul(acc.x, q.zz);
-    Fp S1 = mul(acc.y, q.zzz);
-    Fp P = sub(mul(q.x, acc.zz), U1);
-    Fp R = sub(mul(q.y, acc.zzz), S1);
+    Fp U1 = fmul(acc.x, q.zz);
+    Fp S1 = fmul(acc.y, q.zzz);
+    Fp P = sub(fmul(q.x, acc.zz), U1);
+    Fp R = sub(fmul(q.y, acc.zzz), S1);
     if (!P.is_zero()) {
-        Fp PP = sqr(P);
-        Fp PPP = mul(P, PP);
-        Fp Q = mul(U1, PP);
-        Fp X3 = sub(sub(sub(sqr(R), PPP), Q), Q);
-        Fp Y3 = sub(mul(R, sub(Q, X3)), mul(S1, PPP));
-        acc.zz = mul(mul(acc.zz, q.zz), PP);
-        acc.zzz = mul(mul(acc.zzz, q.zzz), PPP);
+        Fp PP = fsqr(P);
+        Fp PPP = fmul(P, PP);
+        Fp Q = fmul(U1, PP);
+        Fp X3 = sub(sub(sub(fsqr(R), PPP), Q), Q);
+        Fp Y3 = sub(fmul(R, sub(Q, X3)), fmul(S1, PPP));
+        acc.zz = fmul(fmul(acc.zz, q.zz), PP);
+        acc.zzz = fmul(fmul(acc.zzz, q.zzz), PPP);
         acc.x = X3;
         acc.y = Y3;
     } else if (R.is_zero()) {
@@ -148,14 +189,13 @@ GRAPE_HD void xyzz_add(G1Xyzz& acc, const G1Xyzz& q) {
     }
 }
 
-// XYZZ -> Jacobian without inversion: (X*ZZ, Y*ZZZ, Z) with Z := ZZZ/ZZ is not available
-// division-free, but (X*ZZ^2... ) is not needed: the triple (X*ZZ, Y*ZZZ, ZZ) satisfies
-// x = X*ZZ/ZZ^2, y = Y*ZZZ/ZZ^3 because ZZZ^2 = ZZ^3.
+// XYZZ -> Jacobian without inversion: the triple (X*ZZ, Y*ZZZ, ZZ) is a Jacobian representative
+// with Z = ZZ, since x = X*ZZ/ZZ^2 and y = Y*ZZZ/ZZ^3 = Y/ZZZ (ZZZ^2 = ZZ^3).
 GRAPE_HD G1Jac xyzz_to_jac(const G1Xyzz& p) {
     if (p.is_inf()) return G1Jac::inf();
     G1Jac r;
-    r.x = mul(p.x, p.zz);
-    r.y = mul(p.y, p.zzz);
+    r.x = fmul(p.x, p.zz);
+    r.y = fmul(p.y, p.zzz);
     r.z = p.zz;
     return r;
 }
@@ -165,35 +205,35 @@ GRAPE_HD G1Xyzz jac_to_xyzz(const G1Jac& p) {
     G1Xyzz r;
     r.x = p.x;
     r.y = p.y;
-    r.zz = sqr(p.z);
-    r.zzz = mul(r.zz, p.z);
+    r.zz = fsqr(p.z);
+    r.zzz = fmul(r.zz, p.z);
     return r;
 }
 
 // Affine image given the inverse of ZZZ: 1/Z = ZZ/ZZZ, x = X/Z^2, y = Y/ZZZ.
 GRAPE_HD G1Affine xyzz_to_affine_with_inv(const G1Xyzz& p, const Fp& zzz_inv) {
     if (p.is_inf()) return G1Affine::inf();
-    Fp zinv = mul(zzz_inv, p.zz);
+    Fp zinv = fmul(zzz_inv, p.zz);
     G1Affine r;
-    r.x = mul(p.x, sqr(zinv));
-    r.y = mul(p.y, zzz_inv);
+    r.x = fmul(p.x, fsqr(zinv));
+    r.y = fmul(p.y, zzz_inv);
     return r;
 }
 
 GRAPE_HD G1Affine xyzz_to_affine(const G1Xyzz& p) {
     if (p.is_inf()) return G1Affine::inf();
-    return xyzz_to_affine_with_inv(p, inverse(p.zzz));
+    return xyzz_to_affine_with_inv(p, fp_inverse(p.zzz));
 }
 
 // Jacobian -> affine: x = X/Z^2, y = Y/Z^3; infinity maps to (0,0)
 // (include/curve/jacobian_t.cuh:33-41).
 GRAPE_HD G1Affine jac_to_affine(const G1Jac& p) {
     if (p.is_inf()) return G1Affine::inf();
-    Fp zi = inverse(p.z);
-    Fp zi2 = sqr(zi);
+    Fp zi = fp_inverse(p.z);
+    Fp zi2 = fsqr(zi);
     G1Affine r;
-    r.x = mul(p.x, zi2);
-    r.y = mul(p.y, mul(zi2, zi));
+    r.x = fmul(p.x, zi2);
+    r.y = fmul(p.y, fmul(zi2, zi));
     return r;
 }
 

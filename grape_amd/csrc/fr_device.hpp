@@ -1,0 +1,75 @@
+// Device-side helpers shared by the Fr kernels: 16-byte vector load/store of 32-byte elements
+// and wave64 / workgroup tree sums.
+#pragma once
+#include "common.hpp"
+
+namespace grape {
+
+__device__ __forceinline__ Fr ld_fr(const uint32_t* base, size_t i) {
+    const uint4* p = reinterpret_cast<const uint4*>(base) + 2 * i;
+    uint4 lo = p[0], hi = p[1];
+    Fr r;
+    r.v[0] = lo.x; r.v[1] = lo.y; r.v[2] = lo.z; r.v[3] = lo.w;
+    r.v[4] = hi.x; r.v[5] = hi.y; r.v[6] = hi.z; r.v[7] = hi.w;
+    return r;
+}
+__device__ __forceinline__ void st_fr(uint32_t* base, size_t i, const Fr& a) {
+    uint4* p = reinterpret_cast<uint4*>(base) + 2 * i;
+    p[0] = make_uint4(a.v[0], a.v[1], a.v[2], a.v[3]);
+    p[1] = make_uint4(a.v[4], a.v[5], a.v[6], a.v[7]);
+}
+
+__device__ __forceinline__ Fr shfl_down_fr(const Fr& a, int off) {
+    Fr r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.v[i] = __shfl_down(a.v[i], off, 64);
+    return r;
+}
+// wave64 tree: lane 0 ends with the sum of all 64 lanes
+__device__ __forceinline__ Fr wave_sum(Fr a) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) a = add(a, shfl_down_fr(a, off));
+    return a;
+}
+// Workgroup sum of NV values per thread; result valid in thread 0.  lds holds NV*(kBlock/64) Fr.
+template <int NV>
+__device__ __forceinline__ void block_sum(Fr* vals, Fr* lds) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int NW = kBlock / 64;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        Fr s = wave_sum(vals[k]);
+        if (lane == 0) lds[k * NW + wave] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            Fr s = lds[k * NW];
+            for (int w = 1; w < NW; w++) s = add(s, lds[k * NW + w]);
+            vals[k] = s;
+        }
+    }
+}
+
+// NV interleaved partial arrays: partial[b*NV + k]; out[k] = sum_b partial[b*NV + k]
+template <int NV>
+__global__ void __launch_bounds__(kBlock) final_sum_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
+    __shared__ Fr lds[NV * (kBlock / 64)];
+    Fr acc[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) acc[k] = Fr::zero();
+    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) acc[k] = add(acc[k], ld_fr(partial, (size_t)b * NV + k));
+    }
+    block_sum<NV>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) st_fr(out, k, acc[k]);
+    }
+}
+
+#define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")
+
+}  // namespace grape

@@ -1,0 +1,467 @@
+// Fr tensor kernels: element-wise field ops, integer embedding, Montgomery in/out, padding,
+// reductions, batched inversion and the multilinear fold.
+//
+// Layout: a tensor is an array of 32-byte elements (the reference's fr_t array); every lane moves
+// one element with two 16-byte vector accesses, so a wave64 covers 2 KiB of contiguous memory per
+// element index and both halves of every 128-byte line are consumed back to back.
+#include "fr_device.hpp"
+
+namespace grape {
+
+// ------------------------------------------------------------------------------------------------
+// element-wise
+// ------------------------------------------------------------------------------------------------
+enum BinOp { OP_ADD, OP_SUB, OP_MUL };
+
+template <int OP>
+__device__ __forceinline__ Fr apply(const Fr& a, const Fr& b) {
+    if (OP == OP_ADD) return add(a, b);
+    if (OP == OP_SUB) return sub(a, b);
+    return mul(a, b);
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kBlock) ew_kernel(uint32_t* out, const uint32_t* a, const uint32_t* b, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, apply<OP>(ld_fr(a, i), ld_fr(b, i)));
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kBlock) bcast_kernel(uint32_t* out, const uint32_t* a, const uint32_t* x, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, apply<OP>(ld_fr(a, i), ld_fr(x, 0)));
+}
+
+__global__ void __launch_bounds__(kBlock) from_i32_kernel(uint32_t* out, const int32_t* in, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, fr_from_i32(in[i]));
+}
+__global__ void __launch_bounds__(kBlock) from_u32_kernel(uint32_t* out, const uint32_t* in, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, fr_from_u32(in[i]));
+}
+template <bool TO>
+__global__ void __launch_bounds__(kBlock) mont_kernel(uint32_t* out, const uint32_t* in, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    Fr a = ld_fr(in, i);
+    st_fr(out, i, TO ? to_mont(a) : from_mont(a));
+}
+
+__global__ void __launch_bounds__(kBlock) pad_fr_kernel(uint32_t* out, const uint32_t* in, uint32_t N, uint32_t pad_N,
+                                                        size_t size, const uint32_t* pad_val) {
+    size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= size) return;
+    size_t row = g / pad_N;
+    uint32_t col = (uint32_t)(g % pad_N);
+    st_fr(out, g, col < N ? ld_fr(in, row * N + col) : ld_fr(pad_val, 0));
+}
+__global__ void __launch_bounds__(kBlock) pad_i32_kernel(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t size) {
+    size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= size) return;
+    size_t row = g / pad_N;
+    uint32_t col = (uint32_t)(g % pad_N);
+    out[g] = col < N ? in[row * N + col] : 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// reductions
+// ------------------------------------------------------------------------------------------------
+// stage 1: grid-stride partial sums, one Fr per block; stage 2: the same kernel with one block.
+__global__ void __launch_bounds__(kBlock) sum_kernel(uint32_t* out, const uint32_t* in, size_t n) {
+    __shared__ Fr lds[kBlock / 64];
+    Fr acc = Fr::zero();
+    size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) acc = add(acc, ld_fr(in, i));
+    block_sum<1>(&acc, lds);
+    if (threadIdx.x == 0) st_fr(out, blockIdx.x, acc);
+}
+
+__global__ void __launch_bounds__(kBlock) sum_by_dim_kernel(uint32_t* out, const uint32_t* in, size_t rows, size_t dim) {
+    // one wave per row: strided partial sums, wave tree, broadcast back
+    const int lane = threadIdx.x & 63;
+    size_t row = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+    if (row >= rows) return;
+    Fr acc = Fr::zero();
+    for (size_t i = lane; i < dim; i += 64) acc = add(acc, ld_fr(in, row * dim + i));
+    acc = wave_sum(acc);
+    Fr tot;
+#pragma unroll
+    for (int k = 0; k < 8; k++) tot.v[k] = __shfl(acc.v[k], 0, 64);
+    for (size_t i = lane; i < dim; i += 64) st_fr(out, row * dim + i, tot);
+}
+
+// ------------------------------------------------------------------------------------------------
+// batched inversion (Montgomery's trick), three levels:
+//   chunk products -> (recursive inversion of the products) -> back-substitution.
+// Zero inputs are skipped in the products and produce zero outputs.
+// ------------------------------------------------------------------------------------------------
+constexpr int kInvChunk = 8;
+
+// prod[t] = product of the non-zero elements of chunk t (beta added first when given)
+__global__ void __launch_bounds__(kBlock) inv_prod_kernel(uint32_t* prod, const uint32_t* in, const uint32_t* beta, size_t n) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    size_t nchunks = (n + kInvChunk - 1) / kInvChunk;
+    if (t >= nchunks) return;
+    Fr acc = Fr::one();
+    Fr bt = beta ? ld_fr(beta, 0) : Fr::zero();
+    // chunk t owns elements t, t + nchunks, t + 2*nchunks, ... so that lanes stay coalesced
+#pragma unroll
+    for (int k = 0; k < kInvChunk; k++) {
+        size_t i = t + (size_t)k * nchunks;
+        if (i < n) {
+            Fr x = ld_fr(in, i);
+            if (beta) x = add(x, bt);
+            if (!x.is_zero()) acc = mul(acc, x);
+        }
+    }
+    st_fr(prod, t, acc);
+}
+// given inv_prod[t] = 1/prod[t], write the individual inverses
+__global__ void __launch_bounds__(kBlock) inv_back_kernel(uint32_t* out, const uint32_t* in, const uint32_t* beta,
+                                                          const uint32_t* inv_prod, size_t n) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    size_t nchunks = (n + kInvChunk - 1) / kInvChunk;
+    if (t >= nchunks) return;
+    Fr bt = beta ? ld_fr(beta, 0) : Fr::zero();
+    Fr x[kInvChunk];
+    Fr pre[kInvChunk];   // pre[k] = product of non-zero x[0..k-1]
+    Fr acc = Fr::one();
+#pragma unroll
+    for (int k = 0; k < kInvChunk; k++) {
+        size_t i = t + (size_t)k * nchunks;
+        x[k] = Fr::zero();
+        if (i < n) {
+            x[k] = ld_fr(in, i);
+            if (beta) x[k] = add(x[k], bt);
+        }
+        pre[k] = acc;
+        if (!x[k].is_zero()) acc = mul(acc, x[k]);
+    }
+    Fr inv = ld_fr(inv_prod, t);   // 1 / product of all non-zero x
+#pragma unroll
+    for (int k = kInvChunk - 1; k >= 0; k--) {
+        size_t i = t + (size_t)k * nchunks;
+        if (i < n) {
+            if (x[k].is_zero()) {
+                st_fr(out, i, Fr::zero());
+            } else {
+                st_fr(out, i, mul(inv, pre[k]));
+                inv = mul(inv, x[k]);
+            }
+        }
+    }
+}
+// direct inversion, used for the last (small) level
+__global__ void __launch_bounds__(kBlock) inv_direct_kernel(uint32_t* out, const uint32_t* in, const uint32_t* beta, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    Fr x = ld_fr(in, i);
+    if (beta) x = add(x, ld_fr(beta, 0));
+    st_fr(out, i, inverse(x));
+}
+
+// ------------------------------------------------------------------------------------------------
+// fold.  One pass binds the TOP b bits of the folded axis (the multilinear extension does not
+// care in which order variables are bound, and binding high bits keeps every access contiguous):
+//   out[o][i_lo][g] = sum_{i_hi} w[i_hi] * t[o][i_hi*c_lo + i_lo][g],   i_hi*c_lo + i_lo < c
+// with w[i_hi] = prod_k eq(x[k], bit_k(i_hi)) over the b challenges of those bits.
+// ------------------------------------------------------------------------------------------------
+constexpr int kFoldMaxBits = 6;
+
+__global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* out, const uint32_t* in, const uint32_t* x_top,
+                                                           uint32_t b, size_t outer, size_t c, size_t c_lo, size_t gap) {
+    __shared__ Fr w[1 << kFoldMaxBits];
+    const uint32_t nw = 1u << b;
+    if (threadIdx.x < nw) {
+        Fr acc = Fr::one();
+        for (uint32_t k = 0; k < b; k++) {
+            Fr xk = ld_fr(x_top, k);
+            acc = mul(acc, ((threadIdx.x >> k) & 1) ? xk : sub(Fr::one(), xk));
+        }
+        w[threadIdx.x] = acc;
+    }
+    __syncthreads();
+    const size_t c_out = c < c_lo ? c : c_lo;       // surviving extent of the axis
+    const size_t inner = c_out * gap;               // outputs per outer index
+    const size_t total = outer * inner;
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (tid >= total) return;
+    const size_t o = tid / inner;
+    const size_t p = tid - o * inner;               // i_lo*gap + g
+    const size_t i_lo = p / gap;
+    const uint32_t* src = in + 8 * (o * c * gap + p);
+    const size_t hi_stride = c_lo * gap;            // elements between consecutive i_hi
+    // number of i_hi with i_hi*c_lo + i_lo < c
+    const size_t n_hi = (c - i_lo + c_lo - 1) / c_lo;
+    Fr acc = Fr::zero();
+    for (size_t h = 0; h < n_hi; h++) acc = add(acc, mul(ld_fr(src, h * hi_stride), w[h]));
+    st_fr(out, o * inner + p, acc);
+}
+
+// Small-tensor finish: one workgroup holds the whole [c][gap] slab of one outer index in LDS
+// and binds the remaining bits top-down with a barrier per level.
+constexpr int kFoldSmallElems = 2048;   // 64 KiB of LDS
+
+__global__ void __launch_bounds__(kBlock) fold_small_kernel(uint32_t* out, const uint32_t* in, const uint32_t* x,
+                                                            uint32_t L, size_t c, size_t gap) {
+    __shared__ Fr buf[kFoldSmallElems];
+    const size_t o = blockIdx.x;
+    const size_t n = c * gap;
+    for (size_t i = threadIdx.x; i < n; i += kBlock) buf[i] = ld_fr(in, o * n + i);
+    __syncthreads();
+    size_t cur = c;
+    for (int lvl = (int)L - 1; lvl >= 0; lvl--) {
+        const size_t half = (size_t)1 << lvl;        // axis indices >= half fold onto [0, half)
+        if (cur > half) {
+            const Fr xv = ld_fr(x, lvl);
+            const size_t nlow = half * gap;
+            for (size_t i = threadIdx.x; i < nlow; i += kBlock) {
+                const size_t j = i + nlow;
+                Fr lo = buf[i];
+                Fr hi = (j < cur * gap) ? buf[j] : Fr::zero();
+                buf[i] = add(lo, mul(xv, sub(hi, lo)));
+            }
+            cur = half;
+        } else {
+            // the whole upper half is padding: value *= (1 - x)
+            const Fr xv = sub(Fr::one(), ld_fr(x, lvl));
+            for (size_t i = threadIdx.x; i < cur * gap; i += kBlock) buf[i] = mul(buf[i], xv);
+        }
+        __syncthreads();
+    }
+    for (size_t i = threadIdx.x; i < gap; i += kBlock) st_fr(out, o * gap + i, buf[i]);
+}
+
+static uint32_t log2ceil(size_t n) {
+    uint32_t r = 0;
+    while (((size_t)1 << r) < n) r++;
+    return r;
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+
+template <int OP>
+static int launch_ew(uint32_t* out, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(a); CHECK_PTR16(b);
+    ew_kernel<OP><<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, a, b, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+template <int OP>
+static int launch_bcast(uint32_t* out, const uint32_t* a, const uint32_t* x, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(a); CHECK_PTR16(x);
+    bcast_kernel<OP><<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, a, x, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+// shared by grape_fr_batch_inverse / grape_fr_shift_inverse
+static int batch_inverse_impl(uint32_t* out, const uint32_t* in, const uint32_t* beta, size_t n, hipStream_t s) {
+    if (n == 0) return GRAPE_OK;
+    if (n <= 4096) {
+        inv_direct_kernel<<<blocks_for(n), kBlock, 0, s>>>(out, in, beta, n);
+        GRAPE_LAUNCH_CHECK();
+        return GRAPE_OK;
+    }
+    // levels of chunk products live back to back in one scratch buffer
+    size_t sizes[16];
+    int levels = 0;
+    size_t cur = n, total = 0;
+    while (cur > 4096) {
+        cur = (cur + kInvChunk - 1) / kInvChunk;
+        sizes[levels++] = cur;
+        total += cur;
+    }
+    void* ws;
+    int rc = scratch_get(kSlotInv, total * 32, &ws);
+    if (rc) return rc;
+    uint32_t* lvl[16];
+    {
+        uint32_t* p = (uint32_t*)ws;
+        for (int l = 0; l < levels; l++) {
+            lvl[l] = p;
+            p += 8 * sizes[l];
+        }
+    }
+    // forward: products
+    inv_prod_kernel<<<blocks_for(sizes[0]), kBlock, 0, s>>>(lvl[0], in, beta, n);
+    for (int l = 1; l < levels; l++)
+        inv_prod_kernel<<<blocks_for(sizes[l]), kBlock, 0, s>>>(lvl[l], lvl[l - 1], nullptr, sizes[l - 1]);
+    // top: direct inversion in place
+    inv_direct_kernel<<<blocks_for(sizes[levels - 1]), kBlock, 0, s>>>(lvl[levels - 1], lvl[levels - 1], nullptr, sizes[levels - 1]);
+    // backward: each level's inverses from the level above (in place over the products)
+    for (int l = levels - 1; l >= 1; l--)
+        inv_back_kernel<<<blocks_for(sizes[l]), kBlock, 0, s>>>(lvl[l - 1], lvl[l - 1], nullptr, lvl[l], sizes[l - 1]);
+    inv_back_kernel<<<blocks_for(sizes[0]), kBlock, 0, s>>>(out, in, beta, lvl[0], n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+extern "C" {
+
+int grape_fr_add(uint32_t* o, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t s) { return launch_ew<OP_ADD>(o, a, b, n, s); }
+int grape_fr_sub(uint32_t* o, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t s) { return launch_ew<OP_SUB>(o, a, b, n, s); }
+int grape_fr_mul(uint32_t* o, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t s) { return launch_ew<OP_MUL>(o, a, b, n, s); }
+int grape_fr_bcast_add(uint32_t* o, const uint32_t* a, const uint32_t* x, size_t n, grape_stream_t s) { return launch_bcast<OP_ADD>(o, a, x, n, s); }
+int grape_fr_bcast_mul(uint32_t* o, const uint32_t* a, const uint32_t* x, size_t n, grape_stream_t s) { return launch_bcast<OP_MUL>(o, a, x, n, s); }
+
+int grape_fr_from_i32(uint32_t* out, const int32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out);
+    GRAPE_REQUIRE(in != nullptr, "null input");
+    from_i32_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_fr_from_u32(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out);
+    GRAPE_REQUIRE(in != nullptr, "null input");
+    from_u32_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_fr_to_mont(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    mont_kernel<true><<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_fr_from_mont(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    mont_kernel<false><<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_fr_batch_inverse(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    return batch_inverse_impl(out, in, nullptr, n, as_stream(st));
+}
+int grape_fr_shift_inverse(uint32_t* out, const uint32_t* in, const uint32_t* beta, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in); CHECK_PTR16(beta);
+    return batch_inverse_impl(out, in, beta, n, as_stream(st));
+}
+
+int grape_fr_sum(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    CHECK_PTR16(out);
+    hipStream_t s = as_stream(st);
+    if (n == 0) {
+        GRAPE_HIP_CHECK(hipMemsetAsync(out, 0, 32, s));
+        return GRAPE_OK;
+    }
+    CHECK_PTR16(in);
+    unsigned nb = blocks_for(n);
+    if (nb > kNumCU * 8) nb = kNumCU * 8;
+    if (nb == 1) {
+        sum_kernel<<<1, kBlock, 0, s>>>(out, in, n);
+    } else {
+        void* ws;
+        int rc = scratch_get(kSlotReduce, (size_t)nb * 32, &ws);
+        if (rc) return rc;
+        sum_kernel<<<nb, kBlock, 0, s>>>((uint32_t*)ws, in, n);
+        final_sum_kernel<1><<<1, kBlock, 0, s>>>(out, (const uint32_t*)ws, nb);
+    }
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_sum_by_dim(uint32_t* out, const uint32_t* in, size_t rows, size_t dim, grape_stream_t st) {
+    if (rows == 0 || dim == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    sum_by_dim_kernel<<<blocks_for(rows * 64), kBlock, 0, as_stream(st)>>>(out, in, rows, dim);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_pad(uint32_t* out, const uint32_t* in, uint32_t N, uint32_t pad_N, size_t pad_size, const uint32_t* pad_val, grape_stream_t st) {
+    if (pad_size == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in); CHECK_PTR16(pad_val);
+    GRAPE_REQUIRE(N <= pad_N && pad_N > 0 && out != in, "need N <= pad_N and distinct buffers");
+    pad_fr_kernel<<<blocks_for(pad_size), kBlock, 0, as_stream(st)>>>(out, in, N, pad_N, pad_size, pad_val);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_i32_pad(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t pad_size, grape_stream_t st) {
+    if (pad_size == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(out && in && N <= pad_N && pad_N > 0 && out != in, "need N <= pad_N and distinct buffers");
+    pad_i32_kernel<<<blocks_for(pad_size), kBlock, 0, as_stream(st)>>>(out, in, N, pad_N, pad_size);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
+    CHECK_PTR16(t); CHECK_PTR16(x);
+    GRAPE_REQUIRE(c >= 1 && gap >= 1 && N >= (size_t)c * gap && N % ((size_t)c * gap) == 0, "N must be a multiple of c*gap");
+    hipStream_t s = as_stream(st);
+    const size_t outer = N / ((size_t)c * gap);
+    uint32_t L = log2ceil(c);
+    if (L == 0) return GRAPE_OK;   // c == 1: nothing to bind, data already compact
+    const uint32_t* xs = x + 8 * (size_t)id;
+    size_t cur_c = c;
+    const uint32_t* src = t;
+    // With a single outer index a pass can run in place (thread p reads p + k*stride only).
+    // Otherwise passes ping-pong through scratch and the result is copied to the front.
+    uint32_t* ws[2] = {nullptr, nullptr};
+    int which = 0;
+    while (L > 0) {
+        if (cur_c * gap <= (size_t)kFoldSmallElems) {
+            uint32_t* dst = t;
+            if (outer > 1 && src == t) {
+                // reading slabs o*cur_c*gap while writing o*gap would race across workgroups
+                void* p;
+                int rc = scratch_get(kSlotFold, outer * gap * 32 * 2 + 64, &p);
+                if (rc) return rc;
+                dst = (uint32_t*)p;
+            }
+            fold_small_kernel<<<(unsigned)outer, kBlock, 0, s>>>(dst, src, xs, L, cur_c, gap);
+            GRAPE_LAUNCH_CHECK();
+            if (dst != t) GRAPE_HIP_CHECK(hipMemcpyAsync(t, dst, outer * gap * 32, hipMemcpyDeviceToDevice, s));
+            return GRAPE_OK;
+        }
+        // pick b: as many bits as possible while keeping >= 2^17 output threads
+        uint32_t b = L < (uint32_t)kFoldMaxBits ? L : (uint32_t)kFoldMaxBits;
+        while (b > 1 && outer * gap * ((size_t)1 << (L - b)) < ((size_t)1 << 17)) b--;
+        const size_t c_lo = (size_t)1 << (L - b);
+        const size_t c_out = cur_c < c_lo ? cur_c : c_lo;
+        uint32_t* dst;
+        if (outer == 1) {
+            dst = t;   // in place (src == t always holds here)
+        } else {
+            if (!ws[0]) {
+                void* p;
+                // two buffers, each large enough for the first pass output
+                size_t each = outer * c_out * gap * 32;
+                int rc = scratch_get(kSlotFold, 2 * each + 64, &p);
+                if (rc) return rc;
+                ws[0] = (uint32_t*)p;
+                ws[1] = (uint32_t*)((char*)p + each);
+            }
+            dst = ws[which];
+            which ^= 1;
+        }
+        const size_t total = outer * c_out * gap;
+        fold_pass_kernel<<<blocks_for(total), kBlock, 0, s>>>(dst, src, xs + 8 * (size_t)(L - b), b, outer, cur_c, c_lo, gap);
+        GRAPE_LAUNCH_CHECK();
+        src = dst;
+        cur_c = c_out;
+        L -= b;
+    }
+    if (src != t) GRAPE_HIP_CHECK(hipMemcpyAsync(t, src, outer * gap * 32, hipMemcpyDeviceToDevice, s));
+    return GRAPE_OK;
+}
+
+}  // extern "C"

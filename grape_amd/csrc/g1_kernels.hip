@@ -1,0 +1,510 @@
+// G1 kernels: generator derivation, fixed-base tables and the Hyrax row-commitment kernels.
+//
+// Commitment design (one GPU, 288 GB of HBM): all rows of a matrix are committed against the
+// SAME generators, so the work per scalar is bought down with memory — a table of
+// k * 2^(c*w) * G_i for every digit value k and window w turns each signed radix-2^c digit into
+// exactly one mixed addition into a single per-lane accumulator (no per-window accumulators,
+// no doubling chain at the end).  For int16-range weights c = 16 makes that one addition per
+// matrix element.  Lanes own columns (coalesced scalar reads), accumulate in extended Jacobian
+// (XYZZ) coordinates, and a second kernel folds the 64 lane partials of each row and maps the
+// result to affine coordinates.
+#define GRAPE_FP_MUL_OUTLINE 1
+#include "common.hpp"
+
+namespace grape {
+
+// The one shared body of the Fp multiplier / squarer (about a thousand instructions each, so
+// every branch inside stays short-range).
+__device__ __noinline__ Fp fp_mul_outline(Fp a, Fp b) { return mul(a, b); }
+__device__ __noinline__ Fp fp_sqr_outline(Fp a) { return sqr(a); }
+
+__device__ __forceinline__ Fp ld_fp(const uint32_t* p) {
+    const uint4* q = reinterpret_cast<const uint4*>(p);
+    uint4 a = q[0], b = q[1], c = q[2];
+    Fp r;
+    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
+    r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
+    r.v[8] = c.x; r.v[9] = c.y; r.v[10] = c.z; r.v[11] = c.w;
+    return r;
+}
+__device__ __forceinline__ void st_fp(uint32_t* p, const Fp& a) {
+    uint4* q = reinterpret_cast<uint4*>(p);
+    q[0] = make_uint4(a.v[0], a.v[1], a.v[2], a.v[3]);
+    q[1] = make_uint4(a.v[4], a.v[5], a.v[6], a.v[7]);
+    q[2] = make_uint4(a.v[8], a.v[9], a.v[10], a.v[11]);
+}
+__device__ __forceinline__ G1Affine ld_affine(const uint32_t* base, size_t i) {
+    G1Affine r;
+    r.x = ld_fp(base + 24 * i);
+    r.y = ld_fp(base + 24 * i + 12);
+    return r;
+}
+__device__ __forceinline__ void st_affine(uint32_t* base, size_t i, const G1Affine& p) {
+    st_fp(base + 24 * i, p.x);
+    st_fp(base + 24 * i + 12, p.y);
+}
+__device__ __forceinline__ G1Xyzz ld_xyzz(const uint32_t* base, size_t i) {
+    G1Xyzz r;
+    r.x = ld_fp(base + 48 * i);
+    r.y = ld_fp(base + 48 * i + 12);
+    r.zz = ld_fp(base + 48 * i + 24);
+    r.zzz = ld_fp(base + 48 * i + 36);
+    return r;
+}
+__device__ __forceinline__ void st_xyzz(uint32_t* base, size_t i, const G1Xyzz& p) {
+    st_fp(base + 48 * i, p.x);
+    st_fp(base + 48 * i + 12, p.y);
+    st_fp(base + 48 * i + 24, p.zz);
+    st_fp(base + 48 * i + 36, p.zzz);
+}
+__device__ __forceinline__ Fr ld_fr8(const uint32_t* base, size_t i) {
+    const uint4* p = reinterpret_cast<const uint4*>(base) + 2 * i;
+    uint4 lo = p[0], hi = p[1];
+    Fr r;
+    r.v[0] = lo.x; r.v[1] = lo.y; r.v[2] = lo.z; r.v[3] = lo.w;
+    r.v[4] = hi.x; r.v[5] = hi.y; r.v[6] = hi.z; r.v[7] = hi.w;
+    return r;
+}
+
+__device__ __forceinline__ G1Xyzz shfl_down_xyzz(const G1Xyzz& a, int off) {
+    G1Xyzz r;
+#pragma unroll
+    for (int i = 0; i < 12; i++) {
+        r.x.v[i] = __shfl_down(a.x.v[i], off, 64);
+        r.y.v[i] = __shfl_down(a.y.v[i], off, 64);
+        r.zz.v[i] = __shfl_down(a.zz.v[i], off, 64);
+        r.zzz.v[i] = __shfl_down(a.zzz.v[i], off, 64);
+    }
+    return r;
+}
+
+// The group operations are always inlined into the kernels; only the Fp multiplier and squarer
+// are out-of-line.  An out-of-line device function large enough to need far branches is not
+// safe: the compiler's far-branch expansion inside a non-kernel function borrows s[30:31] - the
+// return address - so such a function never returns once the far path is taken (seen in the
+// generated code of an out-of-line mixed addition: the "accumulator is at infinity for every
+// active lane" path jumped through s[30:31] and the final s_setpc_b64 s[30:31] then looped
+// forever).  Kernels have no return address to lose, and the multiplier body is far below the
+// +-128 KiB range of a short branch.
+__device__ __forceinline__ void madd(G1Xyzz& acc, const G1Affine& p, bool negate) { xyzz_add_affine(acc, p, negate); }
+__device__ __forceinline__ void padd(G1Xyzz& acc, const G1Xyzz& q) { xyzz_add(acc, q); }
+__device__ __forceinline__ void pdbl(G1Xyzz& acc) { xyzz_dbl(acc); }
+__device__ __forceinline__ G1Affine to_affine(const G1Xyzz& p) { return xyzz_to_affine(p); }
+
+// k * P for a 256-bit canonical scalar held in 8 limbs
+__device__ __forceinline__ G1Xyzz scalar_mul(const G1Affine& p, const uint32_t* k, int top_bit) {
+    G1Xyzz acc = G1Xyzz::inf();
+    for (int i = top_bit; i >= 0; i--) {
+        pdbl(acc);
+        if ((k[i >> 5] >> (i & 31)) & 1) madd(acc, p, false);
+    }
+    return acc;
+}
+
+__global__ void __launch_bounds__(64) scalar_mul_base_kernel(uint32_t* out, const uint32_t* k, const uint32_t* base, size_t n) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n) return;
+    uint32_t kk[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) kk[j] = k[8 * i + j];
+    G1Affine p = ld_affine(base, 0);
+    st_affine(out, i, to_affine(scalar_mul(p, kk, 255)));
+}
+
+// reference-format table: out[w*N + i] = w*G_i (naive_msm)
+__global__ void __launch_bounds__(64) ref_table_kernel(uint32_t* out, const uint32_t* gens, size_t N, uint32_t W) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= N) return;
+    G1Affine g = ld_affine(gens, i);
+    G1Xyzz res = G1Xyzz::inf();
+    for (uint32_t w = 0; w < W; w++) {
+        st_affine(out, (size_t)w * N + i, to_affine(res));
+        madd(res, g, false);
+    }
+}
+
+// bases[w*N + i] = 2^(c*w) * G_i, affine
+__global__ void __launch_bounds__(64) window_bases_kernel(uint32_t* bases, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= N) return;
+    G1Affine g = ld_affine(gens, i);
+    st_affine(bases, i, g);
+    G1Xyzz cur = G1Xyzz::from_affine(g);
+    for (uint32_t w = 1; w < nw; w++) {
+        for (uint32_t d = 0; d < c; d++) pdbl(cur);
+        st_affine(bases, (size_t)w * N + i, to_affine(cur));
+    }
+}
+
+// One thread per (window w, generator i, chunk j): XYZZ multiples k*B for k = j*CH+1 .. j*CH+CH
+// (clipped to K) into tmp[((j - j0)*CH + t) * (nw*N) + w*N + i].
+__global__ void __launch_bounds__(64) wide_chain_kernel(uint32_t* tmp, const uint32_t* bases, size_t N, uint32_t nw, uint32_t K,
+                                                        uint32_t CH, uint32_t j0, uint32_t nj) {
+    size_t tid = (size_t)blockIdx.x * 64 + threadIdx.x;
+    size_t per_chunk = (size_t)nw * N;
+    if (tid >= per_chunk * nj) return;
+    uint32_t jj = (uint32_t)(tid / per_chunk);
+    size_t wi = tid - (size_t)jj * per_chunk;       // w*N + i
+    uint32_t j = j0 + jj;
+    G1Affine B = ld_affine(bases, wi);
+    uint32_t kstart[8] = {j * CH + 1, 0, 0, 0, 0, 0, 0, 0};
+    G1Xyzz acc = scalar_mul(B, kstart, 31 - __clz((int)kstart[0]));
+    for (uint32_t t = 0; t < CH; t++) {
+        uint32_t k = j * CH + 1 + t;
+        if (k > K) break;
+        st_xyzz(tmp, ((size_t)jj * CH + t) * per_chunk + wi, acc);
+        madd(acc, B, false);
+    }
+}
+
+// Batched XYZZ -> affine (Montgomery's trick over 8 entries per thread, strided so that lanes
+// stay adjacent).  Entry e of tmp goes to dst[map(e)] where, for the wide table,
+// e = (jj*CH + t)*(nw*N) + w*N + i  ->  ((w*K) + (j0*CH + jj*CH + t))*N + i.
+constexpr int kNormChunk = 8;
+__global__ void __launch_bounds__(64) wide_normalize_kernel(uint32_t* table, const uint32_t* tmp, size_t N, uint32_t nw, uint32_t K,
+                                                            uint32_t CH, uint32_t j0, size_t n_entries) {
+    size_t t0 = (size_t)blockIdx.x * 64 + threadIdx.x;
+    size_t nthreads = (n_entries + kNormChunk - 1) / kNormChunk;
+    if (t0 >= nthreads) return;
+    Fp pre[kNormChunk];
+    Fp acc = Fp::one();
+#pragma unroll
+    for (int k = 0; k < kNormChunk; k++) {
+        size_t e = t0 + (size_t)k * nthreads;
+        pre[k] = acc;
+        if (e < n_entries) {
+            Fp zzz = ld_fp(tmp + 48 * e + 36);
+            if (!zzz.is_zero()) acc = fmul(acc, zzz);
+        }
+    }
+    Fp inv = fp_inverse(acc);
+    const size_t per_chunk = (size_t)nw * N;
+#pragma unroll
+    for (int k = kNormChunk - 1; k >= 0; k--) {
+        size_t e = t0 + (size_t)k * nthreads;
+        if (e >= n_entries) continue;
+        G1Xyzz p = ld_xyzz(tmp, e);
+        size_t kk = e / per_chunk;                  // jj*CH + t
+        size_t wi = e - kk * per_chunk;
+        size_t w = wi / N, i = wi - w * N;
+        size_t kidx = (size_t)j0 * CH + kk;         // k - 1
+        if (kidx >= K) continue;
+        G1Affine a = G1Affine::inf();
+        if (!p.zzz.is_zero()) {
+            Fp zi = fmul(inv, pre[k]);
+            inv = fmul(inv, p.zzz);
+            a = xyzz_to_affine_with_inv(p, zi);
+        }
+        st_affine(table, (w * K + kidx) * N + i, a);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// commitment, wide table
+// ------------------------------------------------------------------------------------------------
+// Each wave owns one row segment of `seg` columns; lane l takes columns l, l+64, ...
+// partial[(row*nseg + s)*64 + lane] receives the lane's XYZZ accumulator.
+template <bool FR>
+__global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, const void* scalars, uint32_t rowlen, size_t rows,
+                                                             uint32_t seg, uint32_t nseg, const uint32_t* table, size_t N,
+                                                             uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+    if (wave >= rows * nseg) return;
+    const size_t row = wave / nseg;
+    const uint32_t s = (uint32_t)(wave - row * nseg);
+    const uint32_t col_end = (s + 1) * seg < rowlen ? (s + 1) * seg : rowlen;
+    const uint32_t half = 1u << (c - 1), mask = (c == 32) ? 0xffffffffu : ((1u << c) - 1u);
+    G1Xyzz acc = G1Xyzz::inf();
+    for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
+        if (FR) {
+            const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
+            uint32_t carry = 0;
+            for (uint32_t w = 0; w < nw; w++) {
+                const uint32_t bit = w * c;
+                if (bit >= 256) break;
+                // c <= 16 bits starting at `bit`, possibly straddling two limbs
+                const uint32_t limb = bit >> 5, sh = bit & 31;
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    lo = (q == (int)limb) ? k.v[q] : lo;
+                    hi = (q == (int)limb + 1) ? k.v[q] : hi;
+                }
+                uint64_t both = ((uint64_t)hi << 32) | lo;
+                uint32_t d = ((uint32_t)(both >> sh) & mask) + carry;
+                bool neg = d > half;                 // digit in (half, 2^c] -> d - 2^c, carry 1
+                carry = neg ? 1u : 0u;
+                uint32_t mag = neg ? (mask + 1u - d) : d;
+                if (mag != 0) {
+                    if (mag > K) { *err_flag = 1; continue; }
+                    G1Affine p = ld_affine(table, ((size_t)w * K + (mag - 1)) * N + col);
+                    madd(acc, p, neg);
+                }
+            }
+            if (carry) *err_flag = 1;               // cannot happen for canonical 255-bit scalars when nw*c >= 256
+        } else {
+            int64_t v = ((const int32_t*)scalars)[row * rowlen + col];
+            for (uint32_t w = 0; w < nw; w++) {
+                int64_t d = v & (int64_t)mask;
+                v >>= c;                            // arithmetic shift keeps the sign
+                // digits above half go negative with a carry; exactly half goes negative only
+                // when what remains is negative (so that -2^(c-1) recodes to one digit)
+                if (d > (int64_t)half || (d == (int64_t)half && v < 0)) {
+                    d -= (int64_t)mask + 1;
+                    v += 1;
+                }
+                const bool neg = d < 0;
+                const uint32_t mag = (uint32_t)(neg ? -d : d);
+                if (mag != 0) {
+                    if (mag > K) { *err_flag = 1; continue; }
+                    G1Affine p = ld_affine(table, ((size_t)w * K + (mag - 1)) * N + col);
+                    madd(acc, p, neg);
+                }
+            }
+            if (v != 0) *err_flag = 1;              // scalar does not fit nw windows
+        }
+    }
+    st_xyzz(partial, wave * 64 + lane, acc);
+}
+
+// Row epilogue: 8 lanes per row, each sums nparts/8 partials serially, then a 3-step tree over
+// the 8 lanes; the leader converts to affine.
+__global__ void __launch_bounds__(64) commit_reduce_kernel(uint32_t* out, const uint32_t* partial, size_t rows, uint32_t nparts) {
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & 7;
+    const size_t row = (size_t)blockIdx.x * 8 + (lane >> 3);
+    G1Xyzz acc = G1Xyzz::inf();
+    if (row < rows) {
+        for (uint32_t j = sub; j < nparts; j += 8) padd(acc, ld_xyzz(partial, row * nparts + j));
+    }
+#pragma unroll
+    for (int off = 4; off >= 1; off >>= 1) {
+        G1Xyzz o = shfl_down_xyzz(acc, off);
+        if (sub + off < 8) padd(acc, o);
+    }
+    if (row < rows && sub == 0) st_affine(out, row, to_affine(acc));
+}
+
+// ------------------------------------------------------------------------------------------------
+// commitment through the reference-format table (k*G_i, k < 256): one wave per row, byte windows
+// from the top, 8 doublings between windows.  Compatibility path, not tuned.
+// ------------------------------------------------------------------------------------------------
+template <bool FR>
+__global__ void __launch_bounds__(64) commit_ref_kernel(uint32_t* out, const void* scalars, uint32_t rowlen, size_t rows,
+                                                        const uint32_t* table, size_t npoints) {
+    const int lane = threadIdx.x;
+    const size_t row = blockIdx.x;
+    if (row >= rows) return;
+    const int nwin = FR ? 32 : 4;
+    G1Xyzz total = G1Xyzz::inf();
+    for (int w = nwin - 1; w >= 0; w--) {
+        G1Xyzz acc = G1Xyzz::inf();
+        for (uint32_t col = lane; col < rowlen; col += 64) {
+            uint32_t idx;
+            bool neg = false;
+            if (FR) {
+                const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
+                uint32_t limb = 0;
+#pragma unroll
+                for (int q = 0; q < 8; q++) limb = (q == (w >> 2)) ? k.v[q] : limb;
+                idx = (limb >> (8 * (w & 3))) & 255u;
+            } else {
+                int32_t sv = ((const int32_t*)scalars)[row * rowlen + col];
+                neg = sv < 0;
+                uint32_t a = neg ? (uint32_t)0 - (uint32_t)sv : (uint32_t)sv;
+                idx = (a >> (8 * w)) & 255u;
+            }
+            if (idx) madd(acc, ld_affine(table, (size_t)idx * npoints + col), neg);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            G1Xyzz o = shfl_down_xyzz(acc, off);
+            if (lane + off < 64) padd(acc, o);
+        }
+        // lane 0 carries the running Horner value; other lanes follow along harmlessly
+        for (int d = 0; d < 8; d++) pdbl(total);
+        padd(total, acc);
+    }
+    if (lane == 0) st_affine(out, row, to_affine(total));
+}
+
+__global__ void __launch_bounds__(64) affine_to_jac_kernel(uint32_t* out, const uint32_t* in, size_t n) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n) return;
+    G1Affine a = ld_affine(in, i);
+    bool inf = a.is_inf();
+    st_fp(out + 36 * i, a.x);
+    st_fp(out + 36 * i + 12, a.y);
+    st_fp(out + 36 * i + 24, inf ? Fp::zero() : Fp::one());
+}
+__global__ void __launch_bounds__(64) jac_to_affine_kernel(uint32_t* out, const uint32_t* in, size_t n) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n) return;
+    G1Jac p;
+    p.x = ld_fp(in + 36 * i);
+    p.y = ld_fp(in + 36 * i + 12);
+    p.z = ld_fp(in + 36 * i + 24);
+    st_affine(out, i, jac_to_affine(p));
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+#define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")
+
+static const uint32_t kGenX[12] = {0xfd530c16u, 0x5cb38790u, 0x9976fff5u, 0x7817fc67u, 0x143ba1c1u, 0x154f95c7u,
+                                   0xf3d0e747u, 0xf0ae6acdu, 0x21dbf440u, 0xedce6eccu, 0x9e0bfb75u, 0x12017741u};
+static const uint32_t kGenY[12] = {0x0ce72271u, 0xbaac93d5u, 0x7918fd8eu, 0x8c22631au, 0x570725ceu, 0xdd595f13u,
+                                   0x50405194u, 0x51ac5829u, 0xad0059c0u, 0x0e1c8c3fu, 0x5008a26au, 0x0bbc3efcu};
+
+template <bool FR>
+static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                            uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
+    GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
+    GRAPE_REQUIRE(c >= 2 && c <= 16 && nw >= 1 && K >= (1u << (c - 1)), "need 2 <= c <= 16 and K >= 2^(c-1)");
+    if (FR) GRAPE_REQUIRE((uint64_t)nw * c >= 256, "Fr scalars need nw*c >= 256");
+    const size_t rows = size / rowlen;
+    if (rows == 0) return GRAPE_OK;
+    hipStream_t s = as_stream(st);
+    // segments: enough waves to fill the chip (>= 4 per SIMD) but at least 64 columns per lane-sweep
+    uint32_t nseg = 1;
+    while (rows * nseg < 4096 && rowlen / (nseg * 2) >= 64) nseg *= 2;
+    const uint32_t seg = (rowlen + nseg - 1) / nseg;
+    const size_t nwaves = rows * nseg;
+    void* ws;
+    int rc = scratch_get(kSlotMsm, nwaves * 64 * 192 + 64, &ws);
+    if (rc) return rc;
+    int* err = (int*)((char*)ws + nwaves * 64 * 192);
+    GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
+    profile_begin();
+    profile_mark(s);
+    commit_wide_kernel<FR><<<blocks_for(nwaves * 64), kBlock, 0, s>>>((uint32_t*)ws, scalars, rowlen, rows, seg, nseg, table, N, c, nw, K, err);
+    profile_mark(s);
+    commit_reduce_kernel<<<(unsigned)((rows + 7) / 8), 64, 0, s>>>(out, (const uint32_t*)ws, rows, nseg * 64);
+    profile_mark(s);
+    GRAPE_LAUNCH_CHECK();
+    int h_err = 0;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(&h_err, err, sizeof(int), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    if (h_err) {
+        set_error("commit: a scalar does not fit the table's digit range (c=%u, nw=%u, K=%u)", c, nw, K);
+        return GRAPE_EINVAL;
+    }
+    return GRAPE_OK;
+}
+
+extern "C" {
+
+int grape_g1_generator(uint32_t* out) {
+    GRAPE_REQUIRE(out != nullptr, "null output");
+    for (int i = 0; i < 12; i++) {
+        out[i] = kGenX[i];
+        out[12 + i] = kGenY[i];
+    }
+    return GRAPE_OK;
+}
+
+int grape_g1_scalar_mul_base(uint32_t* out, const uint32_t* k, const uint32_t* base, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(k); CHECK_PTR16(base);
+    scalar_mul_base_kernel<<<blocks_for(n, 64), 64, 0, as_stream(st)>>>(out, k, base, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_g1_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t W, grape_stream_t st) {
+    if (N == 0 || W == 0) return GRAPE_OK;
+    CHECK_PTR16(table); CHECK_PTR16(gens);
+    ref_table_kernel<<<blocks_for(N, 64), 64, 0, as_stream(st)>>>(table, gens, N, W);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K) { return (size_t)nw * K * N * 96; }
+
+int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    CHECK_PTR16(table); CHECK_PTR16(gens);
+    GRAPE_REQUIRE(N >= 1 && c >= 1 && c <= 16 && nw >= 1 && K >= 1 && K <= (1u << 16), "bad table shape");
+    hipStream_t s = as_stream(st);
+    const size_t per_chunk = (size_t)nw * N;
+    // chunk length: long enough to amortise the start-up scalar multiplication, short enough
+    // to expose nw*N*(K/CH) threads
+    uint32_t CH = 64;
+    if (K < CH) CH = K;
+    const uint32_t nchunks = (K + CH - 1) / CH;
+    // slab the chunk index so that the XYZZ staging buffer stays below ~1.5 GiB
+    size_t slab_chunks = ((size_t)3 << 29) / (per_chunk * CH * 192);
+    if (slab_chunks < 1) slab_chunks = 1;
+    if (slab_chunks > nchunks) slab_chunks = nchunks;
+    void* ws;
+    const size_t bases_bytes = per_chunk * 96;
+    const size_t tmp_bytes = slab_chunks * CH * per_chunk * 192;
+    int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes, &ws);
+    if (rc) return rc;
+    uint32_t* bases = (uint32_t*)ws;
+    uint32_t* tmp = (uint32_t*)((char*)ws + bases_bytes);
+    window_bases_kernel<<<blocks_for(N, 64), 64, 0, s>>>(bases, gens, N, c, nw);
+    GRAPE_LAUNCH_CHECK();
+    for (uint32_t j0 = 0; j0 < nchunks; j0 += (uint32_t)slab_chunks) {
+        uint32_t nj = nchunks - j0 < slab_chunks ? nchunks - j0 : (uint32_t)slab_chunks;
+        size_t nthreads = per_chunk * nj;
+        wide_chain_kernel<<<blocks_for(nthreads, 64), 64, 0, s>>>(tmp, bases, N, nw, K, CH, j0, nj);
+        size_t k_hi = (size_t)(j0 + nj) * CH < K ? (size_t)(j0 + nj) * CH : K;
+        size_t n_entries = (k_hi - (size_t)j0 * CH) * per_chunk;
+        size_t nthr2 = (n_entries + kNormChunk - 1) / kNormChunk;
+        wide_normalize_kernel<<<blocks_for(nthr2, 64), 64, 0, s>>>(table, tmp, N, nw, K, CH, j0, n_entries);
+        GRAPE_LAUNCH_CHECK();
+    }
+    return GRAPE_OK;
+}
+
+int grape_commit_i32(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                     uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    return commit_wide_impl<false>(out, scalars, size, rowlen, table, N, c, nw, K, st);
+}
+int grape_commit_fr(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                    uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    return commit_wide_impl<true>(out, scalars, size, rowlen, table, N, c, nw, K, st);
+}
+
+int grape_commit_i32_ref_table(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table,
+                               size_t npoints, grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
+    size_t rows = size / rowlen;
+    if (rows == 0) return GRAPE_OK;
+    commit_ref_kernel<false><<<(unsigned)rows, 64, 0, as_stream(st)>>>(out, scalars, rowlen, rows, table, npoints);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_commit_fr_ref_table(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table,
+                              size_t npoints, grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
+    size_t rows = size / rowlen;
+    if (rows == 0) return GRAPE_OK;
+    commit_ref_kernel<true><<<(unsigned)rows, 64, 0, as_stream(st)>>>(out, scalars, rowlen, rows, table, npoints);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_g1_affine_to_jacobian(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    affine_to_jac_kernel<<<blocks_for(n, 64), 64, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_g1_jacobian_to_affine(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    jac_to_affine_kernel<<<blocks_for(n, 64), 64, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,329 @@
+// Protocol kernels: fused sumcheck rounds (prove.cu) and the logUp / tlookup kernels (tlookup.cu).
+// Every round kernel streams its operands once and leaves per-workgroup partial sums that a
+// one-block kernel finishes; nothing here allocates.
+#include "fr_device.hpp"
+
+namespace grape {
+
+// hi operand of the MSB split: X[g + h] or zero when that index is past the live extent
+__device__ __forceinline__ Fr ld_hi(const uint32_t* X, size_t g, size_t h, size_t in_size) {
+    return (g + h < in_size) ? ld_fr(X, g + h) : Fr::zero();
+}
+
+template <bool COEFFS>
+__global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
+                                                           uint32_t in_size, uint32_t out_size, const uint32_t* v,
+                                                           uint32_t* partial) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    const Fr vv = ld_fr(v, 0);
+    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < out_size; g += stride) {
+        const Fr Ab = ld_fr(A, g), Bb = ld_fr(B, g);
+        const Fr Aa = sub(ld_hi(A, g, out_size, in_size), Ab);
+        const Fr Ba = sub(ld_hi(B, g, out_size, in_size), Bb);
+        st_fr(A, g, add(mul(Aa, vv), Ab));
+        st_fr(B, g, add(mul(Ba, vv), Bb));
+        const Fr c0 = mul(Ab, Bb);
+        const Fr c1 = add(mul(Aa, Bb), mul(Ab, Ba));
+        const Fr c2 = mul(Aa, Ba);
+        if (COEFFS) {
+            st_fr(cc, g, c0);
+            st_fr(cb, g, c1);
+            st_fr(ca, g, c2);
+        }
+        acc[0] = add(acc[0], c0);
+        acc[1] = add(acc[1], c1);
+        acc[2] = add(acc[2], c2);
+    }
+    if (partial) {
+        block_sum<3>(acc, lds);
+        if (threadIdx.x == 0) {
+            st_fr(partial, (size_t)blockIdx.x * 3 + 0, acc[0]);
+            st_fr(partial, (size_t)blockIdx.x * 3 + 1, acc[1]);
+            st_fr(partial, (size_t)blockIdx.x * 3 + 2, acc[2]);
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) sumcheck1_kernel(uint32_t* X, uint32_t* a, uint32_t* b, uint32_t in_size,
+                                                           uint32_t out_size, const uint32_t* v) {
+    size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= out_size) return;
+    const Fr Xb = ld_fr(X, g);
+    const Fr Xa = sub(ld_hi(X, g, out_size, in_size), Xb);
+    st_fr(X, g, add(mul(Xa, ld_fr(v, 0)), Xb));
+    st_fr(b, g, Xb);
+    st_fr(a, g, Xa);
+}
+
+// ---------------------------------------------------------------- tlookup
+__global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    // (v - low) is a small non-negative integer for an in-range witness; leave Montgomery form
+    // and take the low limb, rejecting anything with higher limbs set.
+    Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
+    uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
+    if (hi == 0 && d.v[0] < len) atomicAdd(&hist[d.v[0]], 1u);
+}
+
+__global__ void __launch_bounds__(kBlock) tl_table_kernel(uint32_t* T, const uint32_t* map, const uint32_t* r, int32_t low, uint32_t len) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= len) return;
+    Fr t = add(fr_from_u32((uint32_t)i), fr_from_i32(low));
+    if (map) t = add(t, mul(ld_fr(map, i), ld_fr(r, 0)));
+    st_fr(T, i, t);
+}
+
+__global__ void __launch_bounds__(kBlock) tl_poly_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
+                                                         uint32_t* o0, uint32_t* o1, uint32_t* o2, size_t n_out) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n_out) return;
+    const Fr c00 = ld_fr(A, t);
+    const Fr c01 = sub(ld_fr(A, t + n_out), c00);
+    const Fr s0 = ld_fr(S, t);
+    const Fr c10 = beta ? add(s0, ld_fr(beta, 0)) : s0;
+    const Fr c11 = sub(ld_fr(S, t + n_out), s0);
+    st_fr(o0, t, mul(c00, c10));
+    st_fr(o1, t, add(mul(c01, c10), mul(c00, c11)));
+    st_fr(o2, t, mul(c01, c11));
+}
+
+__global__ void __launch_bounds__(kBlock) tl_poly_sum_kernel(const uint32_t* A, uint32_t* o0, uint32_t* o1, size_t n_out) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n_out) return;
+    const Fr a0 = ld_fr(A, t);
+    st_fr(o0, t, a0);
+    st_fr(o1, t, sub(ld_fr(A, t + n_out), a0));
+}
+
+// 5 sums per round: eq-weighted coefficients of (A0+tA1)(S0+beta+tS1), and plain sums of A0, A1
+__global__ void __launch_bounds__(kBlock) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
+                                                          const uint32_t* eq, size_t n_out, uint32_t* partial) {
+    __shared__ Fr lds[5 * (kBlock / 64)];
+    const Fr bt = beta ? ld_fr(beta, 0) : Fr::zero();
+    Fr acc[5];
+#pragma unroll
+    for (int k = 0; k < 5; k++) acc[k] = Fr::zero();
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
+        const Fr a0 = ld_fr(A, t);
+        const Fr a1 = sub(ld_fr(A, t + n_out), a0);
+        const Fr s0r = ld_fr(S, t);
+        const Fr s0 = add(s0r, bt);
+        const Fr s1 = sub(ld_fr(S, t + n_out), s0r);
+        const Fr e = ld_fr(eq, t);
+        const Fr ea0 = mul(e, a0), ea1 = mul(e, a1);
+        acc[0] = add(acc[0], mul(ea0, s0));
+        acc[1] = add(acc[1], add(mul(ea1, s0), mul(ea0, s1)));
+        acc[2] = add(acc[2], mul(ea1, s1));
+        acc[3] = add(acc[3], a0);
+        acc[4] = add(acc[4], a1);
+    }
+    block_sum<5>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 5; k++) st_fr(partial, (size_t)blockIdx.x * 5 + k, acc[k]);
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* partial) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
+        const Fr m0 = ld_fr(m, t);
+        const Fr m1 = sub(ld_fr(m, t + n_out), m0);
+        const Fr b0 = ld_fr(B, t);
+        const Fr b1 = sub(ld_fr(B, t + n_out), b0);
+        acc[0] = add(acc[0], mul(m0, b0));
+        acc[1] = add(acc[1], add(mul(m1, b0), mul(m0, b1)));
+        acc[2] = add(acc[2], mul(m1, b1));
+    }
+    block_sum<3>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 3; k++) st_fr(partial, (size_t)blockIdx.x * 3 + k, acc[k]);
+    }
+}
+
+// eq table by doubling: level j turns e[0..2^j) into e[0..2^(j+1)) with
+// e[i + 2^j] = e[i]*u_j, e[i] = e[i] - e[i + 2^j]   (= e[i]*(1-u_j))
+__global__ void __launch_bounds__(kBlock) eq_level_kernel(uint32_t* e, const uint32_t* u, uint32_t j) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    size_t half = (size_t)1 << j;
+    if (i >= half) return;
+    const Fr lo = ld_fr(e, i);
+    const Fr hi = mul(lo, ld_fr(u, j));
+    st_fr(e, i + half, hi);
+    st_fr(e, i, sub(lo, hi));
+}
+__global__ void eq_init_kernel(uint32_t* e) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) st_fr(e, 0, Fr::one());
+}
+__global__ void __launch_bounds__(kBlock) eq_halve_kernel(uint32_t* e, size_t n_out) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_out) return;
+    st_fr(e, i, add(ld_fr(e, i), ld_fr(e, i + n_out)));
+}
+
+struct PtrPack { uint32_t* p[8]; };
+__global__ void __launch_bounds__(kBlock) fold_msb_multi_kernel(PtrPack pk, uint32_t k, size_t n_out, const uint32_t* v) {
+    size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= n_out) return;
+    const Fr vv = ld_fr(v, 0);
+    for (uint32_t j = 0; j < k; j++) {
+        uint32_t* X = pk.p[j];
+        const Fr lo = ld_fr(X, g);
+        st_fr(X, g, add(lo, mul(vv, sub(ld_fr(X, g + n_out), lo))));
+    }
+}
+
+static unsigned reduce_grid(size_t n) {
+    unsigned nb = blocks_for(n);
+    unsigned cap = kNumCU * 8;
+    return nb > cap ? cap : nb;
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+// defined in fr_kernels.hip
+extern "C" int grape_fr_shift_inverse(uint32_t*, const uint32_t*, const uint32_t*, size_t, grape_stream_t);
+
+template <bool COEFFS>
+static int sumcheck2_impl(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, uint32_t* c, uint32_t in_size, uint32_t out_size,
+                          const uint32_t* v, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(B); CHECK_PTR16(v);
+    GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * out_size, "need out_size <= in_size <= 2*out_size");
+    hipStream_t s = as_stream(st);
+    unsigned nb = reduce_grid(out_size);
+    uint32_t* partial = nullptr;
+    if (sums) {
+        CHECK_PTR16(sums);
+        void* ws;
+        int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws);
+        if (rc) return rc;
+        partial = (uint32_t*)ws;
+    }
+    sumcheck2_kernel<COEFFS><<<nb, kBlock, 0, s>>>(A, B, a, b, c, in_size, out_size, v, partial);
+    if (sums) final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+extern "C" {
+
+int grape_sumcheck_round2(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {
+    GRAPE_REQUIRE(sums != nullptr, "d_sums is required");
+    return sumcheck2_impl<false>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, sums, st);
+}
+int grape_sumcheck_round2_coeffs(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, uint32_t* c, uint32_t in_size,
+                                 uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(a); CHECK_PTR16(b); CHECK_PTR16(c);
+    return sumcheck2_impl<true>(A, B, a, b, c, in_size, out_size, v, sums, st);
+}
+int grape_sumcheck_round1(uint32_t* X, uint32_t* a, uint32_t* b, uint32_t in_size, uint32_t out_size, const uint32_t* v, grape_stream_t st) {
+    CHECK_PTR16(X); CHECK_PTR16(a); CHECK_PTR16(b); CHECK_PTR16(v);
+    GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * out_size, "need out_size <= in_size <= 2*out_size");
+    sumcheck1_kernel<<<blocks_for(out_size), kBlock, 0, as_stream(st)>>>(X, a, b, in_size, out_size, v);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t low, uint32_t len, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(hist != nullptr && len > 0, "bad histogram buffer");
+    CHECK_PTR16(vals);
+    hist_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(hist, vals, n, low, len);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_init(uint32_t* T, uint32_t* B, int32_t low, uint32_t len, const uint32_t* beta, const uint32_t* map,
+                       const uint32_t* r, grape_stream_t st) {
+    CHECK_PTR16(T); CHECK_PTR16(B); CHECK_PTR16(beta);
+    GRAPE_REQUIRE(len > 0, "empty table");
+    if (map) { CHECK_PTR16(map); CHECK_PTR16(r); }
+    tl_table_kernel<<<blocks_for(len), kBlock, 0, as_stream(st)>>>(T, map, r, low, len);
+    GRAPE_LAUNCH_CHECK();
+    return grape_fr_shift_inverse(B, T, beta, len, st);
+}
+
+int grape_tlookup_poly(const uint32_t* A, const uint32_t* S, const uint32_t* beta, uint32_t* o0, uint32_t* o1, uint32_t* o2,
+                       size_t n_out, grape_stream_t st) {
+    if (n_out == 0) return GRAPE_OK;
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(o0); CHECK_PTR16(o1); CHECK_PTR16(o2);
+    tl_poly_kernel<<<blocks_for(n_out), kBlock, 0, as_stream(st)>>>(A, S, beta, o0, o1, o2, n_out);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_tlookup_poly_sum(const uint32_t* A, uint32_t* o0, uint32_t* o1, size_t n_out, grape_stream_t st) {
+    if (n_out == 0) return GRAPE_OK;
+    CHECK_PTR16(A); CHECK_PTR16(o0); CHECK_PTR16(o1);
+    tl_poly_sum_kernel<<<blocks_for(n_out), kBlock, 0, as_stream(st)>>>(A, o0, o1, n_out);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_round_sums(const uint32_t* A, const uint32_t* S, const uint32_t* beta, const uint32_t* eq, size_t n_out,
+                             uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(eq); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(n_out >= 1, "empty round");
+    hipStream_t s = as_stream(st);
+    unsigned nb = reduce_grid(n_out);
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nb * 5 * 32, &ws);
+    if (rc) return rc;
+    tl_round_kernel<<<nb, kBlock, 0, s>>>(A, S, beta, eq, n_out, (uint32_t*)ws);
+    final_sum_kernel<5><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_tlookup_mb_sums(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(m); CHECK_PTR16(B); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(n_out >= 1, "empty round");
+    hipStream_t s = as_stream(st);
+    unsigned nb = reduce_grid(n_out);
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws);
+    if (rc) return rc;
+    tl_mb_kernel<<<nb, kBlock, 0, s>>>(m, B, n_out, (uint32_t*)ws);
+    final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_eq_table(uint32_t* e, const uint32_t* u, uint32_t nu, grape_stream_t st) {
+    CHECK_PTR16(e);
+    GRAPE_REQUIRE(nu <= 30, "too many variables");
+    hipStream_t s = as_stream(st);
+    eq_init_kernel<<<1, 64, 0, s>>>(e);
+    if (nu) CHECK_PTR16(u);
+    for (uint32_t j = 0; j < nu; j++) eq_level_kernel<<<blocks_for((size_t)1 << j), kBlock, 0, s>>>(e, u, j);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_eq_table_halve(uint32_t* e, size_t n_out, grape_stream_t st) {
+    if (n_out == 0) return GRAPE_OK;
+    CHECK_PTR16(e);
+    eq_halve_kernel<<<blocks_for(n_out), kBlock, 0, as_stream(st)>>>(e, n_out);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_fold_msb_multi(uint32_t* const* ptrs, uint32_t k, size_t n_out, const uint32_t* v, grape_stream_t st) {
+    GRAPE_REQUIRE(ptrs != nullptr && k >= 1 && k <= 8, "1..8 tensors");
+    CHECK_PTR16(v);
+    if (n_out == 0) return GRAPE_OK;
+    PtrPack pk;
+    for (uint32_t j = 0; j < 8; j++) pk.p[j] = j < k ? ptrs[j] : nullptr;
+    for (uint32_t j = 0; j < k; j++) CHECK_PTR16(pk.p[j]);
+    fold_msb_multi_kernel<<<blocks_for(n_out), kBlock, 0, as_stream(st)>>>(pk, k, n_out, v);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+}  // extern "C"

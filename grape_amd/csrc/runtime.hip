@@ -1,0 +1,223 @@
+// Runtime part of the C ABI: device selection, error text, memory helpers, the scratch pool and
+// the two roofline micro-benchmarks (stream copy, v_mad_u64_u32 issue rate).
+#include <stdarg.h>
+#include <string.h>
+#include "common.hpp"
+
+namespace grape {
+
+static thread_local char g_err[512] = "";
+static bool g_init = false;
+static void* g_scratch[kNumSlots] = {nullptr};
+static size_t g_scratch_bytes[kNumSlots] = {0};
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+}
+bool initialised() { return g_init; }
+
+static bool g_prof = false;
+static hipEvent_t g_prof_ev[8];
+static int g_prof_n = 0, g_prof_cap = 0;
+bool profiling() { return g_prof; }
+void profile_begin() { g_prof_n = 0; }
+int profile_mark(hipStream_t s) {
+    if (!g_prof || g_prof_n >= 8) return GRAPE_OK;
+    if (g_prof_n >= g_prof_cap) {
+        GRAPE_HIP_CHECK(hipEventCreate(&g_prof_ev[g_prof_cap]));
+        g_prof_cap++;
+    }
+    GRAPE_HIP_CHECK(hipEventRecord(g_prof_ev[g_prof_n], s));
+    g_prof_n++;
+    return GRAPE_OK;
+}
+
+int scratch_get(ScratchSlot slot, size_t bytes, void** out) {
+    if (bytes > g_scratch_bytes[slot]) {
+        if (g_scratch[slot]) {
+            GRAPE_HIP_CHECK(hipDeviceSynchronize());
+            GRAPE_HIP_CHECK(hipFree(g_scratch[slot]));
+            g_scratch[slot] = nullptr;
+            g_scratch_bytes[slot] = 0;
+        }
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        hipError_t e = hipMalloc(&g_scratch[slot], want);
+        if (e != hipSuccess) {
+            set_error("scratch allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
+            return GRAPE_ENOMEM;
+        }
+        g_scratch_bytes[slot] = want;
+    }
+    *out = g_scratch[slot];
+    return GRAPE_OK;
+}
+
+// 16-byte-per-lane streaming copy, grid-stride
+__global__ void __launch_bounds__(256) copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+// 8 independent multiply-add chains per lane keep the multiplier pipe full; each chain feeds
+// its own low word back as the multiplicand so nothing can be hoisted or shared.
+__global__ void __launch_bounds__(256) mad_kernel(uint64_t* out, int inner, uint32_t seed) {
+    uint32_t a = threadIdx.x * 2654435761u + seed, b = (blockIdx.x * 40503u + 12345u + seed) | 1u;
+    uint64_t c[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) c[k] = (uint64_t)(a + k) * 0x9e3779b97f4a7c15ull;
+    for (int it = 0; it < inner; it++) {
+#pragma unroll
+        for (int rep = 0; rep < 8; rep++) {
+#pragma unroll
+            for (int k = 0; k < 8; k++) c[k] = (uint64_t)(uint32_t)c[k] * b + c[k];
+        }
+    }
+    uint64_t r = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) r ^= c[k];
+    if (r == 0x123456789abcdefull) out[0] = r;   // practically never; keeps the chains alive
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+extern "C" {
+
+int grape_init(int device) {
+    GRAPE_HIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    GRAPE_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("grape_init: device %d is %s, this library is built for gfx950 only", device, prop.gcnArchName);
+        return GRAPE_EINVAL;
+    }
+    g_init = true;
+    return GRAPE_OK;
+}
+const char* grape_last_error(void) { return g_err; }
+int grape_stream_sync(grape_stream_t s) {
+    GRAPE_HIP_CHECK(hipStreamSynchronize(as_stream(s)));
+    return GRAPE_OK;
+}
+int grape_malloc(void** p, size_t bytes) {
+    GRAPE_REQUIRE(p != nullptr, "null output pointer");
+    hipError_t e = hipMalloc(p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        set_error("hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        return GRAPE_ENOMEM;
+    }
+    return GRAPE_OK;
+}
+int grape_free(void* p) {
+    if (p) GRAPE_HIP_CHECK(hipFree(p));
+    return GRAPE_OK;
+}
+int grape_memcpy_h2d(void* d, const void* s, size_t bytes, grape_stream_t st) {
+    if (!bytes) return GRAPE_OK;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(d, s, bytes, hipMemcpyHostToDevice, as_stream(st)));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(as_stream(st)));   // the host buffer may be reused at once
+    return GRAPE_OK;
+}
+int grape_memcpy_d2h(void* d, const void* s, size_t bytes, grape_stream_t st) {
+    if (!bytes) return GRAPE_OK;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(d, s, bytes, hipMemcpyDeviceToHost, as_stream(st)));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(as_stream(st)));
+    return GRAPE_OK;
+}
+int grape_memcpy_d2d(void* d, const void* s, size_t bytes, grape_stream_t st) {
+    if (!bytes) return GRAPE_OK;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(d, s, bytes, hipMemcpyDeviceToDevice, as_stream(st)));
+    return GRAPE_OK;
+}
+int grape_memset_zero(void* d, size_t bytes, grape_stream_t st) {
+    if (!bytes) return GRAPE_OK;
+    GRAPE_HIP_CHECK(hipMemsetAsync(d, 0, bytes, as_stream(st)));
+    return GRAPE_OK;
+}
+
+int grape_profile_enable(int on) {
+    g_prof = on != 0;
+    g_prof_n = 0;
+    return GRAPE_OK;
+}
+int grape_profile_last(float* ms, int cap, int* n) {
+    GRAPE_REQUIRE(ms != nullptr && n != nullptr, "null output");
+    *n = 0;
+    for (int i = 0; i + 1 < g_prof_n && i < cap; i++) {
+        GRAPE_HIP_CHECK(hipEventSynchronize(g_prof_ev[i + 1]));
+        GRAPE_HIP_CHECK(hipEventElapsedTime(&ms[i], g_prof_ev[i], g_prof_ev[i + 1]));
+        *n = i + 1;
+    }
+    return GRAPE_OK;
+}
+
+int grape_event_create(void** ev) {
+    hipEvent_t e;
+    GRAPE_HIP_CHECK(hipEventCreate(&e));
+    *ev = e;
+    return GRAPE_OK;
+}
+int grape_event_destroy(void* ev) {
+    GRAPE_HIP_CHECK(hipEventDestroy((hipEvent_t)ev));
+    return GRAPE_OK;
+}
+int grape_event_record(void* ev, grape_stream_t s) {
+    GRAPE_HIP_CHECK(hipEventRecord((hipEvent_t)ev, as_stream(s)));
+    return GRAPE_OK;
+}
+int grape_event_elapsed_ms(float* ms, void* a, void* b) {
+    GRAPE_HIP_CHECK(hipEventSynchronize((hipEvent_t)b));
+    GRAPE_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b));
+    return GRAPE_OK;
+}
+
+int grape_bench_copy(void* d_dst, const void* d_src, size_t bytes, int iters, float* ms, grape_stream_t st) {
+    GRAPE_REQUIRE(d_dst && d_src && ms && iters > 0 && bytes % 16 == 0, "bad arguments");
+    hipEvent_t e0, e1;
+    GRAPE_HIP_CHECK(hipEventCreate(&e0));
+    GRAPE_HIP_CHECK(hipEventCreate(&e1));
+    size_t n16 = bytes / 16;
+    unsigned grid = kNumCU * 16;
+    copy_kernel<<<grid, 256, 0, as_stream(st)>>>((uint4*)d_dst, (const uint4*)d_src, n16);   // warm-up
+    GRAPE_HIP_CHECK(hipEventRecord(e0, as_stream(st)));
+    for (int i = 0; i < iters; i++) copy_kernel<<<grid, 256, 0, as_stream(st)>>>((uint4*)d_dst, (const uint4*)d_src, n16);
+    GRAPE_HIP_CHECK(hipEventRecord(e1, as_stream(st)));
+    GRAPE_HIP_CHECK(hipEventSynchronize(e1));
+    GRAPE_LAUNCH_CHECK();
+    float t;
+    GRAPE_HIP_CHECK(hipEventElapsedTime(&t, e0, e1));
+    *ms = t / iters;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return GRAPE_OK;
+}
+
+int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double* mads_per_s, grape_stream_t st) {
+    GRAPE_REQUIRE(blocks > 0 && inner > 0 && iters > 0 && mads_per_s, "bad arguments");
+    void* out;
+    int rc = scratch_get(kSlotMisc, 64, &out);
+    if (rc) return rc;
+    hipEvent_t e0, e1;
+    GRAPE_HIP_CHECK(hipEventCreate(&e0));
+    GRAPE_HIP_CHECK(hipEventCreate(&e1));
+    mad_kernel<<<blocks, 256, 0, as_stream(st)>>>((uint64_t*)out, inner, 1u);
+    GRAPE_HIP_CHECK(hipEventRecord(e0, as_stream(st)));
+    for (int i = 0; i < iters; i++) mad_kernel<<<blocks, 256, 0, as_stream(st)>>>((uint64_t*)out, inner, (uint32_t)i);
+    GRAPE_HIP_CHECK(hipEventRecord(e1, as_stream(st)));
+    GRAPE_HIP_CHECK(hipEventSynchronize(e1));
+    GRAPE_LAUNCH_CHECK();
+    float t;
+    GRAPE_HIP_CHECK(hipEventElapsedTime(&t, e0, e1));
+    double mads = (double)blocks * 256.0 * (double)inner * 64.0 * (double)iters;
+    *mads_per_s = mads / (t * 1e-3);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return GRAPE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,354 @@
+"""Thin Python helpers over the C ABI for tests and benchmarks.
+
+Device memory comes from torch (plumbing only): an Fr tensor of n elements is a CUDA int32
+tensor of shape (n, 8) whose bytes are the fr_t array; affine G1 points are (n, 24), XYZZ
+(n, 48).  Host-side values travel as numpy uint64 arrays of shape (n, 4) / (n, 12).
+Every helper enqueues on torch's current stream.
+"""
+import ctypes
+import numpy as np
+import torch
+
+from . import _capi
+
+_initialised = False
+
+
+def init(device=0):
+    global _initialised
+    lib = _capi.load()
+    if not _initialised:
+        torch.cuda.set_device(device)
+        _capi.check(lib.grape_init(device))
+        _initialised = True
+    return lib
+
+
+def _s():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous()
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def sync():
+    _capi.check(init().grape_stream_sync(_s()))
+
+
+# ------------------------------------------------------------------ host <-> device
+def to_dev(a):
+    """numpy array (any integer dtype) -> device tensor viewing the same bytes as int32."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint64:
+        t = torch.from_numpy(a.view(np.int64)).cuda().view(torch.int32)
+        return t.reshape(a.shape[0], -1) if a.ndim == 2 else t
+    if a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32)).cuda()
+    return torch.from_numpy(a).cuda()
+
+
+def fr_to_host(t):
+    """device (n,8) int32 -> numpy uint64 (n,4)."""
+    return t.detach().cpu().contiguous().numpy().view(np.uint64).reshape(-1, 4)
+
+
+def g1_to_host(t):
+    return t.detach().cpu().contiguous().numpy().view(np.uint64).reshape(-1, 12)
+
+
+def fr_empty(n):
+    return torch.empty((max(int(n), 0), 8), dtype=torch.int32, device="cuda")
+
+
+def g1_empty(n):
+    return torch.empty((int(n), 24), dtype=torch.int32, device="cuda")
+
+
+# ------------------------------------------------------------------ Fr tensors
+def _ew(name, a, b, out=None):
+    lib = init()
+    out = fr_empty(a.shape[0]) if out is None else out
+    _capi.check(getattr(lib, name)(_p(out), _p(a), _p(b), a.shape[0], _s()))
+    return out
+
+
+def fr_add(a, b, out=None): return _ew("grape_fr_add", a, b, out)
+def fr_sub(a, b, out=None): return _ew("grape_fr_sub", a, b, out)
+def fr_mul(a, b, out=None): return _ew("grape_fr_mul", a, b, out)
+def fr_bcast_add(a, x, out=None): return _ew("grape_fr_bcast_add", a, x, out)
+def fr_bcast_mul(a, x, out=None): return _ew("grape_fr_bcast_mul", a, x, out)
+
+
+def fr_from_i32(x):
+    lib = init()
+    out = fr_empty(x.numel())
+    _capi.check(lib.grape_fr_from_i32(_p(out), _p(x), x.numel(), _s()))
+    return out
+
+
+def fr_from_u32(x):
+    lib = init()
+    out = fr_empty(x.numel())
+    _capi.check(lib.grape_fr_from_u32(_p(out), _p(x), x.numel(), _s()))
+    return out
+
+
+def fr_to_mont(a):
+    lib = init()
+    out = fr_empty(a.shape[0])
+    _capi.check(lib.grape_fr_to_mont(_p(out), _p(a), a.shape[0], _s()))
+    return out
+
+
+def fr_from_mont(a):
+    lib = init()
+    out = fr_empty(a.shape[0])
+    _capi.check(lib.grape_fr_from_mont(_p(out), _p(a), a.shape[0], _s()))
+    return out
+
+
+def fr_batch_inverse(a, out=None):
+    lib = init()
+    out = fr_empty(a.shape[0]) if out is None else out
+    _capi.check(lib.grape_fr_batch_inverse(_p(out), _p(a), a.shape[0], _s()))
+    return out
+
+
+def fr_shift_inverse(a, beta, out=None):
+    lib = init()
+    out = fr_empty(a.shape[0]) if out is None else out
+    _capi.check(lib.grape_fr_shift_inverse(_p(out), _p(a), _p(beta), a.shape[0], _s()))
+    return out
+
+
+def fr_sum(a, n=None):
+    lib = init()
+    out = fr_empty(1)
+    n = a.shape[0] if n is None else n
+    _capi.check(lib.grape_fr_sum(_p(out), _p(a), n, _s()))
+    return out
+
+
+def fr_sum_by_dim(a, rows, dim):
+    lib = init()
+    out = fr_empty(rows * dim)
+    _capi.check(lib.grape_fr_sum_by_dim(_p(out), _p(a), rows, dim, _s()))
+    return out
+
+
+def fr_pad(a, N, pad_N, pad_size, pad_val):
+    lib = init()
+    out = fr_empty(pad_size)
+    _capi.check(lib.grape_fr_pad(_p(out), _p(a), N, pad_N, pad_size, _p(pad_val), _s()))
+    return out
+
+
+def i32_pad(a, N, pad_N, pad_size):
+    lib = init()
+    out = torch.empty(pad_size, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_i32_pad(_p(out), _p(a), N, pad_N, pad_size, _s()))
+    return out
+
+
+def fr_fold(t, N, x, c, idx, gap):
+    """in place; the result is t[: N // c]."""
+    lib = init()
+    _capi.check(lib.grape_fr_fold(_p(t), N, _p(x), c, idx, gap, _s()))
+    return t
+
+
+# ------------------------------------------------------------------ sumcheck / tlookup
+def sumcheck_round2(A, B, in_size, out_size, v):
+    lib = init()
+    sums = fr_empty(3)
+    _capi.check(lib.grape_sumcheck_round2(_p(A), _p(B), in_size, out_size, _p(v), _p(sums), _s()))
+    return sums
+
+
+def sumcheck_round2_coeffs(A, B, a, b, c, in_size, out_size, v, want_sums=True):
+    lib = init()
+    sums = fr_empty(3) if want_sums else None
+    _capi.check(lib.grape_sumcheck_round2_coeffs(_p(A), _p(B), _p(a), _p(b), _p(c), in_size, out_size, _p(v), _p(sums), _s()))
+    return sums
+
+
+def sumcheck_round1(X, a, b, in_size, out_size, v):
+    lib = init()
+    _capi.check(lib.grape_sumcheck_round1(_p(X), _p(a), _p(b), in_size, out_size, _p(v), _s()))
+
+
+def tlookup_hist(vals, low, length, hist=None):
+    lib = init()
+    if hist is None:
+        hist = torch.zeros(length, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_tlookup_hist(_p(hist), _p(vals), vals.shape[0], low, length, _s()))
+    return hist
+
+
+def tlookup_init(low, length, beta, map_t=None, r=None):
+    lib = init()
+    T, B = fr_empty(length), fr_empty(length)
+    _capi.check(lib.grape_tlookup_init(_p(T), _p(B), low, length, _p(beta), _p(map_t), _p(r), _s()))
+    return T, B
+
+
+def tlookup_poly(A, S, beta, n_out):
+    lib = init()
+    o = [fr_empty(n_out) for _ in range(3)]
+    _capi.check(lib.grape_tlookup_poly(_p(A), _p(S), _p(beta), _p(o[0]), _p(o[1]), _p(o[2]), n_out, _s()))
+    return o
+
+
+def tlookup_poly_sum(A, n_out):
+    lib = init()
+    o = [fr_empty(n_out) for _ in range(2)]
+    _capi.check(lib.grape_tlookup_poly_sum(_p(A), _p(o[0]), _p(o[1]), n_out, _s()))
+    return o
+
+
+def tlookup_round_sums(A, S, beta, eq, n_out):
+    lib = init()
+    sums = fr_empty(8)
+    _capi.check(lib.grape_tlookup_round_sums(_p(A), _p(S), _p(beta), _p(eq), n_out, _p(sums), _s()))
+    return sums
+
+
+def tlookup_mb_sums(m, B, n_out):
+    lib = init()
+    sums = fr_empty(3)
+    _capi.check(lib.grape_tlookup_mb_sums(_p(m), _p(B), n_out, _p(sums), _s()))
+    return sums
+
+
+def eq_table(u, nu=None):
+    lib = init()
+    nu = u.shape[0] if nu is None else nu
+    e = fr_empty(1 << nu)
+    _capi.check(lib.grape_eq_table(_p(e), _p(u) if nu else None, nu, _s()))
+    return e
+
+
+def eq_table_halve(e, n_out):
+    lib = init()
+    _capi.check(lib.grape_eq_table_halve(_p(e), n_out, _s()))
+
+
+def fr_fold_msb_multi(tensors, n_out, v):
+    lib = init()
+    arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+    _capi.check(lib.grape_fr_fold_msb_multi(arr, len(tensors), n_out, _p(v), _s()))
+
+
+# ------------------------------------------------------------------ G1
+def g1_generator():
+    lib = init()
+    out = np.zeros(12, dtype=np.uint64)
+    _capi.check(lib.grape_g1_generator(out.ctypes.data_as(ctypes.c_void_p)))
+    return out
+
+
+def g1_make_generators(k_plain):
+    """k_plain: numpy uint64 (n,4) canonical scalars -> device affine points (n,24)."""
+    lib = init()
+    k = to_dev(np.ascontiguousarray(k_plain, dtype=np.uint64).reshape(-1, 4))
+    base = to_dev(g1_generator().reshape(1, 12))
+    out = g1_empty(k.shape[0])
+    _capi.check(lib.grape_g1_scalar_mul_base(_p(out), _p(k), _p(base), k.shape[0], _s()))
+    return out
+
+
+def g1_table_gen(gens, W):
+    lib = init()
+    n = gens.shape[0]
+    out = g1_empty(W * n)
+    _capi.check(lib.grape_g1_table_gen(_p(out), _p(gens), n, W, _s()))
+    return out
+
+
+def g1_wide_table_gen(gens, c, nw, K):
+    lib = init()
+    n = gens.shape[0]
+    out = g1_empty(nw * K * n)
+    _capi.check(lib.grape_g1_wide_table_gen(_p(out), _p(gens), n, c, nw, K, _s()))
+    return out
+
+
+def commit_i32(scalars, rowlen, table, N, c, nw, K, out=None):
+    lib = init()
+    size = scalars.numel()
+    out = g1_empty(size // rowlen) if out is None else out
+    _capi.check(lib.grape_commit_i32(_p(out), _p(scalars), size, rowlen, _p(table), N, c, nw, K, _s()))
+    return out
+
+
+def commit_fr(scalars, rowlen, table, N, c, nw, K, out=None):
+    lib = init()
+    size = scalars.shape[0]
+    out = g1_empty(size // rowlen) if out is None else out
+    _capi.check(lib.grape_commit_fr(_p(out), _p(scalars), size, rowlen, _p(table), N, c, nw, K, _s()))
+    return out
+
+
+def commit_i32_ref_table(scalars, rowlen, table, npoints):
+    lib = init()
+    size = scalars.numel()
+    out = g1_empty(size // rowlen)
+    _capi.check(lib.grape_commit_i32_ref_table(_p(out), _p(scalars), size, rowlen, _p(table), npoints, _s()))
+    return out
+
+
+def commit_fr_ref_table(scalars, rowlen, table, npoints):
+    lib = init()
+    size = scalars.shape[0]
+    out = g1_empty(size // rowlen)
+    _capi.check(lib.grape_commit_fr_ref_table(_p(out), _p(scalars), size, rowlen, _p(table), npoints, _s()))
+    return out
+
+
+def g1_affine_to_jacobian(a):
+    lib = init()
+    out = torch.empty((a.shape[0], 36), dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_g1_affine_to_jacobian(_p(out), _p(a), a.shape[0], _s()))
+    return out
+
+
+def g1_jacobian_to_affine(a):
+    lib = init()
+    out = g1_empty(a.shape[0])
+    _capi.check(lib.grape_g1_jacobian_to_affine(_p(out), _p(a), a.shape[0], _s()))
+    return out
+
+
+# ------------------------------------------------------------------ measurement
+def bench_copy(nbytes, iters=10):
+    lib = init()
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    src.zero_()
+    ms = ctypes.c_float(0)
+    _capi.check(lib.grape_bench_copy(_p(dst), _p(src), nbytes, iters, ctypes.byref(ms), _s()))
+    return ms.value
+
+
+def bench_mad(blocks=4096, inner=256, iters=5):
+    lib = init()
+    r = ctypes.c_double(0)
+    _capi.check(lib.grape_bench_mad_u64_u32(blocks, inner, iters, ctypes.byref(r), _s()))
+    return r.value
+
+
+def profile_enable(on=True):
+    _capi.check(init().grape_profile_enable(1 if on else 0))
+
+
+def profile_last():
+    """kernel durations (ms) of the most recent profiled call, in launch order."""
+    lib = init()
+    buf = (ctypes.c_float * 8)()
+    n = ctypes.c_int(0)
+    _capi.check(lib.grape_profile_last(buf, 8, ctypes.byref(n)))
+    return [buf[i] for i in range(n.value)]

@@ -1,0 +1,221 @@
+/*
+ * grape_hip.h — C ABI of the MI355X (gfx950) kernels behind Grape's proving hot path.
+ *
+ * Everything the host-side classes (FrTensor, Hyrax, prove_matmul, tLookupRange, ...) need from
+ * the GPU goes through these functions; they are the only place HIP is used.  Conventions:
+ *
+ *   - every pointer named d_* is DEVICE memory, everything else is host memory;
+ *   - an Fr element is 8 x u32 little-endian limbs (32 bytes, 32-byte aligned arrays) holding the
+ *     canonical Montgomery residue x*2^256 mod r — the reference's fr_t image
+ *     (include/field/mont_t.cuh:33, include/field/bls12-381.cuh:24-45), which is also the image
+ *     of the host Fr (4 x u64), so values move between host and device by plain copies as in
+ *     src/fr-tensor.cu:214,352,437;
+ *   - an Fp element is 12 x u32 (x*2^384 mod p); an affine G1 point is {x,y} = 96 bytes with
+ *     infinity = all zero (include/curve/affine_t.cuh:28-39); a Jacobian point is {X,Y,Z} = 144
+ *     bytes with Z = 0 for infinity; an XYZZ accumulator is {X,Y,ZZ,ZZZ} = 192 bytes;
+ *   - every function returns 0 on success and a negative GRAPE_E* code otherwise;
+ *     grape_last_error() gives the message.  Nothing is printed, nothing throws;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Kernels are only
+ *     enqueued; results are ready after grape_stream_sync(stream).  Functions that return a value
+ *     to the host say so and synchronise the stream themselves;
+ *   - one host thread per stream; calls on the same device share an internal scratch pool, so
+ *     calls issued from different host threads must not overlap.
+ */
+#ifndef GRAPE_HIP_H
+#define GRAPE_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GRAPE_OK 0
+#define GRAPE_EINVAL (-1)   /* bad argument (null pointer, size mismatch, unsupported shape) */
+#define GRAPE_EHIP (-2)     /* a HIP runtime call failed */
+#define GRAPE_ENOMEM (-3)   /* device allocation failed */
+
+typedef void *grape_stream_t;
+
+/* ------------------------------------------------------------------ runtime ------------------ */
+/* Select the device and create the per-device scratch pool.  Must be called once before use. */
+int grape_init(int device);
+const char *grape_last_error(void);
+int grape_stream_sync(grape_stream_t stream);
+/* Thin allocation / copy helpers so host code needs no HIP headers (replace the reference's
+ * direct cudaMalloc / cudaMemcpy / cudaFree calls, e.g. src/fr-tensor.cu:371-374,322-328). */
+int grape_malloc(void **d_ptr, size_t bytes);
+int grape_free(void *d_ptr);
+int grape_memcpy_h2d(void *d_dst, const void *src, size_t bytes, grape_stream_t stream);
+int grape_memcpy_d2h(void *dst, const void *d_src, size_t bytes, grape_stream_t stream); /* syncs */
+int grape_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, grape_stream_t stream);
+int grape_memset_zero(void *d_ptr, size_t bytes, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ Fr tensors --------------- */
+/* out[i] = a[i] (+,-,*) b[i]; out may alias a or b.
+ * Fr_elementwise_add/sub/mul, src/fr-tensor.cu:74-101. */
+int grape_fr_add(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_b, size_t n, grape_stream_t stream);
+int grape_fr_sub(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_b, size_t n, grape_stream_t stream);
+int grape_fr_mul(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_b, size_t n, grape_stream_t stream);
+/* out[i] = a[i] (+,*) x[0], x one device element.  Fr_broadcast_add/mul, src/fr-tensor.cu:88-108. */
+int grape_fr_bcast_add(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_x, size_t n, grape_stream_t stream);
+int grape_fr_bcast_mul(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_x, size_t n, grape_stream_t stream);
+/* Integer embedding, negatives as r-|v|.  int_to_fr / uint_to_fr, src/fr-tensor.cu:30-46. */
+int grape_fr_from_i32(uint32_t *d_out, const int32_t *d_in, size_t n, grape_stream_t stream);
+int grape_fr_from_u32(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
+/* Enter / leave Montgomery form, in place allowed.  to_kernel / from_kernel, src/fr-tensor.cu:110-120. */
+int grape_fr_to_mont(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
+int grape_fr_from_mont(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
+/* out[i] = 1/in[i], 1/0 = 0, by batched Montgomery inversion (same values as the per-element
+ * reciprocal of inverse_kernel, src/fr-tensor.cu:122-126).  out may alias in. */
+int grape_fr_batch_inverse(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
+/* out[i] = 1/(in[i] + beta[0]).  tlookup_inv_kernel, src/tlookup.cu:52-62. */
+int grape_fr_shift_inverse(uint32_t *d_out, const uint32_t *d_in, const uint32_t *d_beta, size_t n, grape_stream_t stream);
+/* d_out[0] = sum of the first n elements; the input is left untouched (the reference's
+ * FrTensor::sum, src/fr-tensor.cu:415-440, clobbers it for n > 256 — not reproduced). */
+int grape_fr_sum(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
+/* Row sums broadcast back over each row of `dim` columns.  sum_by_dim_kernel, src/fr-tensor.cu:155-163. */
+int grape_fr_sum_by_dim(uint32_t *d_out, const uint32_t *d_in, size_t rows, size_t dim, grape_stream_t stream);
+/* Row padding N -> pad_N columns, pad_size output elements.  pad_fr_kernel / pad_int_kernel,
+ * src/fr-tensor.cu:18-28.  out must not alias in. */
+int grape_fr_pad(uint32_t *d_out, const uint32_t *d_in, uint32_t N, uint32_t pad_N, size_t pad_size,
+                 const uint32_t *d_pad_val, grape_stream_t stream);
+int grape_i32_pad(int32_t *d_out, const int32_t *d_in, uint32_t N, uint32_t pad_N, size_t pad_size, grape_stream_t stream);
+/*
+ * Fold (partial multilinear evaluation) in place: view the first N elements of t as
+ * [N/(c*gap)][c][gap], bind the c axis with challenges x[id], x[id+1], ... (index bit j of the
+ * axis pairs with x[id+j]; a missing partner of an odd tail counts as zero) and leave the
+ * [N/(c*gap)][gap] result contiguous at the front of t.
+ * FrTensor::partial_eval, src/fr-tensor.cu:330-344 with Fr_partial_me :168-188 and
+ * Fr_partial_eval_kernel :53-72.  x is a device array of challenges.
+ */
+int grape_fr_fold(uint32_t *d_t, size_t N, const uint32_t *d_x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ sumcheck ----------------- */
+/*
+ * One round of the two-tensor sumcheck kernel (sumcheck_kernel, src/prove.cu:29-46) fused with the
+ * three reductions the reference runs afterwards (src/prove.cu:101-105): for g < out_size with
+ * hi = X[g+out_size] (zero when g+out_size >= in_size): Xa = hi - X[g], Xb = X[g];
+ * A[g] = Aa*v + Ab, B[g] = Ba*v + Bb (in place) and
+ * d_sums[0] = sum Ab*Bb, d_sums[1] = sum (Aa*Bb + Ab*Ba), d_sums[2] = sum Aa*Ba.
+ */
+int grape_sumcheck_round2(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size,
+                          const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
+/* As above but also materialises the coefficient arrays a, b, c (needed by phase 1, which folds
+ * them over the remaining layer bits, src/prove.cu:64-66).  d_sums may be NULL. */
+int grape_sumcheck_round2_coeffs(uint32_t *d_A, uint32_t *d_B, uint32_t *d_a, uint32_t *d_b, uint32_t *d_c,
+                                 uint32_t in_size, uint32_t out_size, const uint32_t *d_v,
+                                 uint32_t *d_sums, grape_stream_t stream);
+/* Single-tensor round (sumcheck_kernel, src/prove.cu:14-27): X[g] = Xa*v + Xb, a[g] = Xa, b[g] = Xb. */
+int grape_sumcheck_round1(uint32_t *d_X, uint32_t *d_a, uint32_t *d_b, uint32_t in_size, uint32_t out_size,
+                          const uint32_t *d_v, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ tlookup / logUp ---------- */
+/* hist[(v - low) as integer] += 1 for n values (Montgomery Fr); hist has `len` u32 counters and
+ * is NOT cleared here.  Values outside [low, low+len) are ignored.
+ * get_histogram_kernel, src/tlookup.cu:5-14. */
+int grape_tlookup_hist(uint32_t *d_hist, const uint32_t *d_vals, size_t n, int32_t low, uint32_t len, grape_stream_t stream);
+/* T[i] = low + i (+ r*map[i] when d_map != NULL), B[i] = 1/(T[i] + beta).
+ * tlookuprange_init_kernel / tLookupRangeMapping_init_kernel, src/tlookup.cu:16-50. */
+int grape_tlookup_init(uint32_t *d_T, uint32_t *d_B, int32_t low, uint32_t len, const uint32_t *d_beta,
+                       const uint32_t *d_map, const uint32_t *d_r, grape_stream_t stream);
+/* out0 = A0*(S0+beta), out1 = A1*(S0+beta) + A0*S1, out2 = A1*S1 with X0 = X[t], X1 = X[t+n_out]-X[t].
+ * tLookup_poly_kernel, src/tlookup.cu:64-78.  d_beta may be NULL (beta = 0, as :181). */
+int grape_tlookup_poly(const uint32_t *d_A, const uint32_t *d_S, const uint32_t *d_beta, uint32_t *d_out0,
+                       uint32_t *d_out1, uint32_t *d_out2, size_t n_out, grape_stream_t stream);
+/* out0 = A[t], out1 = A[t+n_out] - A[t].  tLookup_poly_sum_kernel, src/tlookup.cu:80-88. */
+int grape_tlookup_poly_sum(const uint32_t *d_A, uint32_t *d_out0, uint32_t *d_out1, size_t n_out, grape_stream_t stream);
+/*
+ * Fused round of the logUp sumcheck: with X_t = X0 + t*X1 on the MSB split of size n_out and
+ * e[x] = eq(u_low, x) held in d_eq (n_out entries), writes into d_sums (8 elements):
+ *   [0..2] sum_x e[x] * coefficients of (A0 + tA1)(S0 + beta + tS1)      (src/tlookup.cu:129-138)
+ *   [3..4] sum_x A0, sum_x A1                                           (:142-146)
+ * Nothing is modified.  This replaces tLookup_poly_kernel + three full multilinear evaluations
+ * + tLookup_poly_sum_kernel + two sums of the reference with one pass over A, S and e.
+ */
+int grape_tlookup_round_sums(const uint32_t *d_A, const uint32_t *d_S, const uint32_t *d_beta, const uint32_t *d_eq,
+                             size_t n_out, uint32_t *d_sums, grape_stream_t stream);
+/* d_sums[0..2] = sums of the coefficients of (m0 + t m1)(B0 + t B1) (src/tlookup.cu:180-185). */
+int grape_tlookup_mb_sums(const uint32_t *d_m, const uint32_t *d_B, size_t n_out, uint32_t *d_sums, grape_stream_t stream);
+/* e[i] = prod_j (u_j if bit_j(i) else 1 - u_j) for i < 2^nu; u is a device array of nu challenges. */
+int grape_eq_table(uint32_t *d_eq, const uint32_t *d_u, uint32_t nu, grape_stream_t stream);
+/* e'[x] = e[x] + e[x + n_out] for x < n_out: the table of the remaining variables after the
+ * top one is dropped. */
+int grape_eq_table_halve(uint32_t *d_eq, size_t n_out, grape_stream_t stream);
+/* MSB fold of k tensors at once: X[g] = X[g] + v*(X[g+n_out]-X[g]) for each of the k device
+ * pointers in d_ptrs (host array of device pointers), in place.
+ * tLookup_phase2_reduce_kernel, src/tlookup.cu:100-113; FrTensor::partial_eval(size,v,2,0,size/2). */
+int grape_fr_fold_msb_multi(uint32_t *const *ptrs, uint32_t k, size_t n_out, const uint32_t *d_v, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ G1 / Hyrax --------------- */
+/* The standard BLS12-381 G1 generator, affine Montgomery, to host memory (96 bytes). */
+int grape_g1_generator(uint32_t *out_affine);
+/* out[i] = k[i] * base for n canonical (non-Montgomery) 256-bit scalars k and one affine base
+ * point; used to derive seeded generators (the reference draws bn128::random_element(),
+ * src/ec_operation.cu:31-36). */
+int grape_g1_scalar_mul_base(uint32_t *d_out_affine, const uint32_t *d_k_plain, const uint32_t *d_base_affine,
+                             size_t n, grape_stream_t stream);
+/* The reference's generator table: table[w*N + i] = w*G_i for w < W as affine points, entry
+ * w = 0 is infinity.  precompute_generators + naive_msm, src/ec_operation.cu:15-49. */
+int grape_g1_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, size_t N, uint32_t W, grape_stream_t stream);
+/*
+ * Wide fixed-base table for the commitment kernels:
+ *   table[(w*K + (k-1))*N + i] = k * 2^(c*w) * G_i,  k = 1..K, w < nw
+ * (affine).  With c = 16, nw = 1, K = 32768 a signed 16-bit scalar is ONE mixed addition;
+ * with c = 8, nw = 32, K = 128 a 255-bit scalar is 32 signed-digit additions into a single
+ * accumulator.  Size: nw*K*N*96 bytes.
+ */
+int grape_g1_wide_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, size_t N, uint32_t c, uint32_t nw,
+                            uint32_t K, grape_stream_t stream);
+size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K);
+/*
+ * Row commitments of an integer matrix: for each of size/rowlen rows,
+ * C_row = sum_i s[row*rowlen + i] * G_i, i < rowlen, written as AFFINE points (96 bytes each).
+ * Hyrax::commit(int*, size, N), src/Hyrax.cu:312-333 (int_windows_sum :46-65, int_windows_reduce
+ * :67-87); rowlen is the reference's N*com_scale.  The wide table must have been built for
+ * N >= rowlen generators with radix 2^c, nw windows and K >= 2^(c-1); scalars are recoded into
+ * signed radix-2^c digits, so any int32 is accepted when nw*c >= 33, and the int16 fast path
+ * (c = 16, nw = 1) requires -32768 <= s <= 32767 (checked on device: returns GRAPE_EINVAL after
+ * synchronising if violated).
+ */
+int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
+                     const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/* Same for full-width Fr scalars (Montgomery form in, left untouched — the reference's
+ * tensor.from()/to() round trip of src/Hyrax.cu:347,356 is not needed).
+ * Hyrax::commit(FrTensor&, size, N), src/Hyrax.cu:335-359. Requires nw*c >= 256. */
+int grape_commit_fr(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
+                    const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/* Commitments through the reference-format table (k*G_i, k < 256, byte windows of |s| resp. of
+ * the canonical scalar) — the reference's own algorithm, kept for tables loaded from its
+ * points.bin.  Output affine. */
+int grape_commit_i32_ref_table(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
+                               const uint32_t *d_table_affine, size_t npoints, grape_stream_t stream);
+int grape_commit_fr_ref_table(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
+                              const uint32_t *d_table_affine, size_t npoints, grape_stream_t stream);
+/* Format conversions for callers that keep the reference's jacob_t arrays. */
+int grape_g1_affine_to_jacobian(uint32_t *d_out_jac, const uint32_t *d_in_affine, size_t n, grape_stream_t stream);
+int grape_g1_jacobian_to_affine(uint32_t *d_out_affine, const uint32_t *d_in_jac, size_t n, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ measurement -------------- */
+/* Device-to-device copy of `bytes` with the library's own streaming kernel, `iters` times;
+ * returns the average time per copy in milliseconds in *ms (HIP events on `stream`). */
+int grape_bench_copy(void *d_dst, const void *d_src, size_t bytes, int iters, float *ms, grape_stream_t stream);
+/* Dependency-free v_mad_u64_u32 throughput: every lane of `blocks` x 256 threads runs
+ * `inner` x 64 multiply-adds; *mads_per_s receives lane-level 32x32 multiplies per second. */
+int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double *mads_per_s, grape_stream_t stream);
+/* Kernel-level timing: when enabled, the commitment entry points bracket each kernel they launch
+ * with HIP events on the caller's stream.  grape_profile_last() synchronises and returns the
+ * durations (ms) of the kernels of the most recent call, in launch order (for grape_commit_*:
+ * [0] accumulation kernel, [1] row-reduction kernel); *n receives how many were written. */
+int grape_profile_enable(int on);
+int grape_profile_last(float *ms, int cap, int *n);
+/* Event timing helpers on a stream (HIP events), for benchmarks that live above this ABI. */
+int grape_event_create(void **ev);
+int grape_event_destroy(void *ev);
+int grape_event_record(void *ev, grape_stream_t stream);
+int grape_event_elapsed_ms(float *ms, void *ev_start, void *ev_stop); /* syncs on ev_stop */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

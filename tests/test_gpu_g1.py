@@ -1,0 +1,179 @@
+"""GPU parity of the G1 / Hyrax commitment kernels against the CPU oracle (affine, bit-exact)."""
+import numpy as np
+import pytest
+import bigref as br
+import orc
+from gpuutil import rand_fr, gaussian_i16, assert_same
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from grape_amd import ops as o
+    o.init(0)
+    return o
+
+
+def _scalars(n, seed):
+    """canonical (non-Montgomery) scalars < r for generator derivation."""
+    return rand_fr(n, seed)
+
+
+@pytest.fixture(scope="module")
+def gens64(ops):
+    k = _scalars(64, 100)
+    host = orc.g1_make_generators(k)
+    dev = ops.g1_make_generators(k)
+    return k, host, dev
+
+
+def test_generator_constant(ops):
+    assert_same(ops.g1_generator(), orc.g1_generator(), "generator")
+
+
+def test_make_generators(ops, gens64):
+    k, host, dev = gens64
+    assert_same(ops.g1_to_host(dev), host, "k*G")
+    # special scalars: 0 -> infinity (0,0), 1 -> G, r-1 -> -G
+    ks = br.ints_to_limbs([0, 1, br.R_MOD - 1, 2], 4)
+    got = br.g1_unpack(ops.g1_to_host(ops.g1_make_generators(ks)))
+    assert got == [None, br.G1, br.g1_neg(br.G1), br.g1_add(br.G1, br.G1)]
+
+
+def test_reference_table(ops, gens64):
+    k, host, dev = gens64
+    n, W = 16, 256
+    got = ops.g1_to_host(ops.g1_table_gen(dev[:n].contiguous(), W))
+    assert_same(got, orc.g1_table(host[:n], W), "table")
+    assert not got[:n].any()                  # w = 0 row is infinity
+
+
+def test_wide_table_entries(ops, gens64):
+    k, host, dev = gens64
+    n, c, nw, K = 8, 8, 3, 128
+    tab = br.g1_unpack(ops.g1_to_host(ops.g1_wide_table_gen(dev[:n].contiguous(), c, nw, K)))
+    pts = br.g1_unpack(host[:n])
+    for (w, kk, i) in [(0, 1, 0), (0, 128, 7), (1, 1, 3), (1, 77, 2), (2, 128, 5), (2, 2, 0), (0, 65, 1), (1, 64, 6)]:
+        assert tab[(w * K + (kk - 1)) * n + i] == br.g1_mul(kk << (c * w), pts[i])
+
+
+def test_commit_i32_small_vs_oracle_and_bigint(ops, gens64):
+    import torch
+    k, host, dev = gens64
+    n, rows = 64, 6
+    rng = np.random.default_rng(5)
+    S = rng.integers(-2**31, 2**31, size=(rows, n)).astype(np.int32)
+    S[0] = 0
+    S[1] = 0
+    S[1, 3] = -1
+    S[2, :8] = [-2**31, 2**31 - 1, 65535, -65536, 32768, -32768, 32767, -32767]
+    table_ref = orc.g1_table(host, 256)
+    want = orc.commit_i32(S, table_ref, n, n)
+    dS = torch.from_numpy(S).cuda()
+    # general int32: radix 2^8 signed digits, 5 windows
+    wide = ops.g1_wide_table_gen(dev, 8, 5, 128)
+    assert_same(ops.g1_to_host(ops.commit_i32(dS, n, wide, n, 8, 5, 128)), want, "commit i32 c=8")
+    # radix 2^16, 3 windows
+    wide16 = ops.g1_wide_table_gen(dev[:16].contiguous(), 16, 3, 32768)
+    S16 = S[:, :16].copy()
+    want16 = orc.commit_i32(S16, orc.g1_table(host[:16], 256), 16, 16)
+    assert_same(ops.g1_to_host(ops.commit_i32(torch.from_numpy(S16).cuda(), 16, wide16, 16, 16, 3, 32768)), want16, "commit i32 c=16")
+    # reference-format table path
+    dtab = ops.g1_table_gen(dev, 256)
+    assert_same(ops.g1_to_host(ops.commit_i32_ref_table(dS, n, dtab, n)), want, "commit i32 ref table")
+    got = br.g1_unpack(want)
+    assert got[0] is None and got[1] == br.g1_neg(br.g1_unpack(host[3:4])[0])
+
+
+def test_commit_int16_fast_path(ops, gens64):
+    import torch
+    k, host, dev = gens64
+    n, rows = 32, 40
+    W = gaussian_i16((rows, n), 6)
+    W[0, :4] = [-32768, 32767, 0, 1]
+    wide = ops.g1_wide_table_gen(dev[:n].contiguous(), 16, 1, 32768)
+    got = ops.g1_to_host(ops.commit_i32(torch.from_numpy(W).cuda(), n, wide, n, 16, 1, 32768))
+    want = orc.commit_i32(W, orc.g1_table(host[:n], 256), n, n)
+    assert_same(got, want, "int16 fast path")
+    # a value outside int16 range is rejected, not silently mis-committed
+    W[3, 3] = 40000
+    from grape_amd import GrapeError
+    with pytest.raises(GrapeError):
+        ops.commit_i32(torch.from_numpy(W).cuda(), n, wide, n, 16, 1, 32768)
+
+
+def test_commit_fr_config1_shape(ops):
+    # BASELINE config 1: the 2^16 products committed as a 256 x 256 matrix with 256 generators
+    k = _scalars(256, 101)
+    host = orc.g1_make_generators(k)
+    dev = ops.g1_make_generators(k)
+    a, b = rand_fr(1 << 16, 1), rand_fr(1 << 16, 2)
+    prod = orc.vec2("orc_fr_vec_mul", a, b)
+    rows_checked = 6                              # the oracle takes ~1 s per row
+    want = orc.commit_fr(prod[: rows_checked * 256], orc.g1_table(host, 256), 256, 256)
+    wide = ops.g1_wide_table_gen(dev, 8, 32, 128)
+    dprod = ops.fr_mul(ops.to_dev(a), ops.to_dev(b))
+    got = ops.g1_to_host(ops.commit_fr(dprod, 256, wide, 256, 8, 32, 128))
+    assert got.shape[0] == 256
+    assert_same(got[:rows_checked], want, "commit fr")
+    # every output is on the curve
+    for pt in br.g1_unpack(got[::37]):
+        assert br.g1_on_curve(pt)
+    # the tensor is still in Montgomery form afterwards
+    assert_same(ops.fr_to_host(dprod), prod, "scalars untouched")
+    # reference-format table path on a few rows
+    dtab = ops.g1_table_gen(dev, 256)
+    got2 = ops.g1_to_host(ops.commit_fr_ref_table(dprod[: 3 * 256].contiguous(), 256, dtab, 256))
+    assert_same(got2, want[:3], "commit fr ref table")
+
+
+def test_commit_fr_edge_scalars_and_int_path_agreement(ops, gens64):
+    import torch
+    k, host, dev = gens64
+    n = 16
+    vals = [0, 1, br.R_MOD - 1, 255, 256, 128, 127, 129, (1 << 254), br.R_MOD - 128, 0x80808080, 2**64 - 1,
+            2**128, 0x7f7f7f7f7f7f7f7f, 3, 5]
+    s = br.fr_pack(vals)
+    wide = ops.g1_wide_table_gen(dev[:n].contiguous(), 8, 32, 128)
+    got = br.g1_unpack(ops.g1_to_host(ops.commit_fr(ops.to_dev(s), n, wide, n, 8, 32, 128)))[0]
+    assert got == br.g1_msm(vals, br.g1_unpack(host[:n]))
+    small = np.array([[5, -7, 300, -70000, 0, 0, 1, -1, 9, 8, 7, 6, 5, 4, 3, 2]], dtype=np.int32)
+    a = ops.g1_to_host(ops.commit_fr(ops.fr_from_i32(torch.from_numpy(small).cuda()), n, wide, n, 8, 32, 128))
+    wide5 = ops.g1_wide_table_gen(dev[:n].contiguous(), 8, 5, 128)
+    b = ops.g1_to_host(ops.commit_i32(torch.from_numpy(small).cuda(), n, wide5, n, 8, 5, 128))
+    assert_same(a, b, "int path == Fr path")
+
+
+def test_commit_linearity_medium(ops):
+    # size-independent property on a larger shape: com(a + b) = com(a) + com(b)
+    import torch
+    n, rows = 512, 64
+    k = _scalars(n, 102)
+    dev = ops.g1_make_generators(k)
+    wide = ops.g1_wide_table_gen(dev, 16, 1, 32768)
+    a = gaussian_i16((rows, n), 7, sigma=512)
+    b = gaussian_i16((rows, n), 8, sigma=512)
+    ca = br.g1_unpack(ops.g1_to_host(ops.commit_i32(torch.from_numpy(a).cuda(), n, wide, n, 16, 1, 32768)))
+    cb = br.g1_unpack(ops.g1_to_host(ops.commit_i32(torch.from_numpy(b).cuda(), n, wide, n, 16, 1, 32768)))
+    cab = br.g1_unpack(ops.g1_to_host(ops.commit_i32(torch.from_numpy(a + b).cuda(), n, wide, n, 16, 1, 32768)))
+    for x, y, z in zip(ca, cb, cab):
+        assert z == br.g1_add(x, y)
+    # rows shorter than the generator set (table stride N > rowlen)
+    c2 = ops.g1_to_host(ops.commit_i32(torch.from_numpy(a[:, :128].copy()).cuda(), 128, wide, n, 16, 1, 32768))
+    host = orc.g1_make_generators(k[:128])
+    assert_same(c2[:4], orc.commit_i32(a[:4, :128].copy(), orc.g1_table(host, 256), 128, 128), "stride")
+
+
+def test_jacobian_conversions(ops, gens64):
+    k, host, dev = gens64
+    jac = ops.g1_affine_to_jacobian(dev)
+    back = ops.g1_jacobian_to_affine(jac)
+    assert_same(ops.g1_to_host(back), host, "affine -> jacobian -> affine")
+    hj = jac.cpu().numpy().view(np.uint64).reshape(-1, 18)
+    want = np.zeros((64, 12), dtype=np.uint64)
+    orc.lib().orc_g1_jac_to_affine(orc.P(want), orc.P(np.ascontiguousarray(hj)), orc.c64(64))
+    assert_same(want, host, "oracle jacobian -> affine")

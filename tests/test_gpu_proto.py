@@ -1,0 +1,191 @@
+"""GPU parity of the sumcheck-round and tlookup kernels against the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import bigref as br
+import orc
+from gpuutil import rand_fr, assert_same
+
+pytestmark = pytest.mark.gpu
+R = br.R_MOD
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from grape_amd import ops as o
+    o.init(0)
+    return o
+
+
+def _oracle_round2(A, B, in_size, out_size, v):
+    A, B = A.copy(), B.copy()
+    a = np.zeros((out_size, 4), dtype=np.uint64)
+    b = np.zeros_like(a)
+    c = np.zeros_like(a)
+    orc.lib().orc_sumcheck_round2(orc.P(A), orc.P(B), orc.P(a), orc.P(b), orc.P(c), orc.c32(in_size), orc.c32(out_size), orc.P(v))
+    return A, B, a, b, c
+
+
+@pytest.mark.parametrize("in_size,out_size", [(2, 1), (8, 4), (6, 4), (5, 4), (4096, 2048), (3000, 2048), (1 << 17, 1 << 16), (100000, 65536)])
+def test_sumcheck_round2(ops, in_size, out_size):
+    A, B = rand_fr(in_size, 1 + in_size), rand_fr(in_size, 2 + in_size)
+    v = rand_fr(1, 3)
+    wA, wB, wa, wb, wc = _oracle_round2(A, B, in_size, out_size, v)
+    dA, dB = ops.to_dev(A), ops.to_dev(B)
+    sums = ops.fr_to_host(ops.sumcheck_round2(dA, dB, in_size, out_size, ops.to_dev(v)))
+    assert_same(ops.fr_to_host(dA)[:out_size], wA[:out_size], "folded A")
+    assert_same(ops.fr_to_host(dB)[:out_size], wB[:out_size], "folded B")
+    assert_same(sums[0], orc.fr_sum(wc), "sum c")
+    assert_same(sums[1], orc.fr_sum(wb), "sum b")
+    assert_same(sums[2], orc.fr_sum(wa), "sum a")
+    # coefficient-array variant
+    dA, dB = ops.to_dev(A), ops.to_dev(B)
+    da, db, dc = ops.fr_empty(out_size), ops.fr_empty(out_size), ops.fr_empty(out_size)
+    sums2 = ops.fr_to_host(ops.sumcheck_round2_coeffs(dA, dB, da, db, dc, in_size, out_size, ops.to_dev(v)))
+    assert_same(ops.fr_to_host(da), wa, "a")
+    assert_same(ops.fr_to_host(db), wb, "b")
+    assert_same(ops.fr_to_host(dc), wc, "c")
+    assert_same(sums2, sums, "sums")
+
+
+def test_sumcheck_round1(ops):
+    in_size, out_size = 1000, 512
+    X = rand_fr(in_size, 11)
+    v = rand_fr(1, 12)
+    dX = ops.to_dev(X)
+    da, db = ops.fr_empty(out_size), ops.fr_empty(out_size)
+    ops.sumcheck_round1(dX, da, db, in_size, out_size, ops.to_dev(v))
+    Xi = br.fr_unpack(X)
+    vi = br.fr_unpack(v)[0]
+    hi = [Xi[g + out_size] if g + out_size < in_size else 0 for g in range(out_size)]
+    assert br.fr_unpack(ops.fr_to_host(db)) == Xi[:out_size]
+    assert br.fr_unpack(ops.fr_to_host(da)) == [(h - l) % R for h, l in zip(hi, Xi)]
+    assert br.fr_unpack(ops.fr_to_host(dX)[:out_size]) == [(l + vi * (h - l)) % R for h, l in zip(hi, Xi)]
+
+
+def test_full_phase2_chain_matches_oracle_transcript(ops):
+    # run 12 fused rounds on K = 4096 (BASELINE config 3's phase 2) and compare every round's
+    # sums with the oracle's prove_matmul transcript for L = N = M = 1
+    K = 4096
+    A, B = rand_fr(K, 21), rand_fr(K, 22)
+    v = rand_fr(12, 23)
+    u = rand_fr(1, 24)[:0]
+    prod = orc.vec2("orc_fr_vec_mul", A, B)
+    claim = orc.fr_sum(prod)
+    st, tr, final_claim, ac, bc = orc.prove_matmul(A, B, 1, 1, 1, K, u, v, claim)
+    assert st == 0 and tr.shape[0] == 12
+    dA, dB, dv = ops.to_dev(A), ops.to_dev(B), ops.to_dev(v)
+    in_size, out_size = K, K // 2
+    for i in range(12):
+        vi = dv[12 - 1 - i: 12 - i].contiguous()
+        sums = ops.fr_to_host(ops.sumcheck_round2(dA, dB, in_size, out_size, vi))
+        assert_same(sums, tr[i][:3], "round %d" % i)
+        in_size, out_size = out_size, out_size // 2
+    assert_same(ops.fr_to_host(dA)[0], ac, "A(v)")
+    assert_same(ops.fr_to_host(dB)[0], bc, "B(v)")
+
+
+def test_histogram(ops):
+    import torch
+    low, length = -32768, 65536
+    rng = np.random.default_rng(31)
+    s = rng.integers(low, low + length, size=200000).astype(np.int32)
+    vals = ops.fr_from_i32(torch.from_numpy(s).cuda())
+    h = ops.tlookup_hist(vals, low, length).cpu().numpy().view(np.uint32)
+    assert np.array_equal(h, np.bincount(s.astype(np.int64) - low, minlength=length).astype(np.uint32))
+    assert_same(h[:, None], orc.histogram(orc.from_i32(s), low, length)[:, None], "hist vs oracle")
+    # heavy collisions: everything in one bin
+    same = ops.fr_from_i32(torch.full((100000,), 5, dtype=torch.int32, device="cuda"))
+    h2 = ops.tlookup_hist(same, 0, 16).cpu().numpy()
+    assert h2[5] == 100000 and h2.sum() == 100000
+    # out-of-range values are ignored
+    oob = ops.fr_from_i32(torch.tensor([100, -1, 3], dtype=torch.int32, device="cuda"))
+    h3 = ops.tlookup_hist(oob, 0, 16).cpu().numpy()
+    assert h3.sum() == 1 and h3[3] == 1
+
+
+def test_table_init(ops):
+    low, length = -32768, 65536
+    beta = br.fr_pack([length])
+    T, B = ops.tlookup_init(low, length, ops.to_dev(beta))
+    wT, wB = orc.tlookup_init(low, length, beta[0])
+    assert_same(ops.fr_to_host(T), wT, "T")
+    assert_same(ops.fr_to_host(B), wB, "B")
+    mp = rand_fr(1024, 41)
+    r = rand_fr(1, 42)
+    T, B = ops.tlookup_init(-512, 1024, ops.to_dev(br.fr_pack([1024])), ops.to_dev(mp), ops.to_dev(r))
+    wT, wB = orc.tlookup_init(-512, 1024, br.fr_pack([1024])[0], mp, r[0])
+    assert_same(ops.fr_to_host(T), wT, "T mapped")
+    assert_same(ops.fr_to_host(B), wB, "B mapped")
+
+
+def test_tlookup_poly_kernels_and_fused_round(ops):
+    n_out = 3000
+    A, S = rand_fr(2 * n_out, 51), rand_fr(2 * n_out, 52)
+    beta = rand_fr(1, 53)
+    Ai, Si, bi = br.fr_unpack(A), br.fr_unpack(S), br.fr_unpack(beta)[0]
+    o = [br.fr_unpack(ops.fr_to_host(t)) for t in ops.tlookup_poly(ops.to_dev(A), ops.to_dev(S), ops.to_dev(beta), n_out)]
+    c00 = Ai[:n_out]
+    c01 = [(Ai[t + n_out] - Ai[t]) % R for t in range(n_out)]
+    c10 = [(Si[t] + bi) % R for t in range(n_out)]
+    c11 = [(Si[t + n_out] - Si[t]) % R for t in range(n_out)]
+    assert o[0] == [a * b % R for a, b in zip(c00, c10)]
+    assert o[1] == [(a * b + c * d) % R for a, b, c, d in zip(c01, c10, c00, c11)]
+    assert o[2] == [a * b % R for a, b in zip(c01, c11)]
+    p = [br.fr_unpack(ops.fr_to_host(t)) for t in ops.tlookup_poly_sum(ops.to_dev(A), n_out)]
+    assert p[0] == c00 and p[1] == c01
+    # beta = NULL means zero
+    o2 = [br.fr_unpack(ops.fr_to_host(t)) for t in ops.tlookup_poly(ops.to_dev(A), ops.to_dev(S), None, n_out)]
+    assert o2[0] == [a * b % R for a, b in zip(c00, Si[:n_out])]
+
+
+def test_fused_round_sums_equal_reference_steps(ops):
+    # the fused kernel must give what the reference's poly kernel + three multilinear
+    # evaluations + poly-sum kernel + two sums give (oracle restatement of those steps)
+    logh = 12
+    n_out = 1 << logh
+    A, S = rand_fr(2 * n_out, 61), rand_fr(2 * n_out, 62)
+    beta = rand_fr(1, 63)
+    u = rand_fr(logh, 64)
+    eq = ops.eq_table(ops.to_dev(u))
+    sums = ops.fr_to_host(ops.tlookup_round_sums(ops.to_dev(A), ops.to_dev(S), ops.to_dev(beta), eq, n_out))
+    o = [ops.fr_to_host(t) for t in ops.tlookup_poly(ops.to_dev(A), ops.to_dev(S), ops.to_dev(beta), n_out)]
+    for k in range(3):
+        assert_same(sums[k], orc.mle_eval(o[k], u), "weighted coefficient %d" % k)
+    p = [ops.fr_to_host(t) for t in ops.tlookup_poly_sum(ops.to_dev(A), n_out)]
+    assert_same(sums[3], orc.fr_sum(p[0]), "sum A0")
+    assert_same(sums[4], orc.fr_sum(p[1]), "sum A1")
+    m, B = rand_fr(2 * n_out, 65), rand_fr(2 * n_out, 66)
+    mb = ops.fr_to_host(ops.tlookup_mb_sums(ops.to_dev(m), ops.to_dev(B), n_out))
+    o = [ops.fr_to_host(t) for t in ops.tlookup_poly(ops.to_dev(m), ops.to_dev(B), None, n_out)]
+    for k in range(3):
+        assert_same(mb[k], orc.fr_sum(o[k]), "m*B coefficient %d" % k)
+
+
+def test_eq_table_and_halving(ops):
+    u = rand_fr(10, 71)
+    ui = br.fr_unpack(u)
+    e = ops.eq_table(ops.to_dev(u))
+    got = br.fr_unpack(ops.fr_to_host(e))
+    for i in (0, 1, 2, 513, 1023, 77):
+        assert got[i] == br.eq_weight(i, ui)
+    assert sum(got) % R == 1
+    ops.eq_table_halve(e, 512)
+    got2 = br.fr_unpack(ops.fr_to_host(e)[:512])
+    for i in (0, 1, 511, 77):
+        assert got2[i] == br.eq_weight(i, ui[:9])
+    e0 = ops.eq_table(ops.to_dev(u), 0)
+    assert br.fr_unpack(ops.fr_to_host(e0)) == [1]
+
+
+def test_fold_msb_multi(ops):
+    n_out = 5000
+    ts = [rand_fr(2 * n_out, 80 + j) for j in range(5)]
+    v = rand_fr(1, 90)
+    dts = [ops.to_dev(t) for t in ts]
+    ops.fr_fold_msb_multi(dts, n_out, ops.to_dev(v))
+    for t, dt in zip(ts, dts):
+        want = orc.partial_eval(t, 2 * n_out, v, 2, 0, n_out)[:n_out]
+        assert_same(ops.fr_to_host(dt)[:n_out], want, "msb fold")
