@@ -1,0 +1,178 @@
+"""ctypes binding of the C entry points over the C++ host classes (grape_amd/host/host_capi.h)."""
+import ctypes
+import os
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "host", "libgrape_host.so")
+_lib = None
+
+NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_prove_matmul", "grape_host_prove_elemul",
+         "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
+         "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
+         "grape_host_fr_op", "grape_host_g1_mul_generator"]
+
+
+class HostError(RuntimeError):
+    pass
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HostError("%s not found: build it with `python grape_amd/host/build.py`" % LIB_PATH)
+        from . import _capi
+        _capi.load()                       # the kernel library first (dependency)
+        lib = ctypes.CDLL(LIB_PATH)
+        for n in NAMES:
+            getattr(lib, n)
+        lib.grape_host_last_error.restype = ctypes.c_char_p
+        lib.grape_host_seed.argtypes = [ctypes.c_uint64]
+        _lib = lib
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise HostError(load().grape_host_last_error().decode())
+
+
+def _hp(a):
+    """pointer to a host numpy array (or None)"""
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _dp(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _fr(a, n=None):
+    a = np.ascontiguousarray(a, dtype=np.uint64).reshape(-1, 4)
+    if n is not None:
+        assert a.shape[0] == n
+    return a
+
+
+def prove_matmul(dA, dB, L, N, M, K, u, v, claim):
+    lib = load()
+    u, v = _fr(u), _fr(v)
+    claim = np.array(claim, dtype=np.uint64).reshape(4)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    ac, bc = np.zeros(4, dtype=np.uint64), np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_prove_matmul(_dp(dA), _dp(dB), L, N, M, K, _hp(u), u.shape[0], _hp(v), v.shape[0], _hp(claim),
+                                       _hp(tr), ctypes.byref(nr), _hp(ac), _hp(bc)))
+    return tr[: nr.value].copy(), claim, ac, bc
+
+
+def prove_elemul(dA, dB, L, M, N, u, v, claim):
+    lib = load()
+    u, v = _fr(u), _fr(v)
+    claim = np.array(claim, dtype=np.uint64).reshape(4)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    ac, bc = np.zeros(4, dtype=np.uint64), np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_prove_elemul(_dp(dA), _dp(dB), L, M, N, _hp(u), u.shape[0], _hp(v), v.shape[0], _hp(claim),
+                                       _hp(tr), ctypes.byref(nr), _hp(ac), _hp(bc)))
+    return tr[: nr.value].copy(), claim, ac, bc
+
+
+def combine_claims(dX, size, claims, us, v):
+    lib = load()
+    claims, v = _fr(claims), _fr(v)
+    us = np.ascontiguousarray(us, dtype=np.uint64).reshape(claims.shape[0], v.shape[0], 4)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    res = np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_combine_claims(_dp(dX), size, _hp(claims), claims.shape[0], _hp(us), _hp(v), v.shape[0],
+                                         _hp(tr), ctypes.byref(nr), _hp(res)))
+    return tr[: nr.value].copy(), res
+
+
+def mle_eval(dT, size, u):
+    lib = load()
+    u = _fr(u)
+    out = np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_mle_eval(_dp(dT), size, _hp(u), u.shape[0], _hp(out)))
+    return out
+
+
+def hyrax_commit_i32(d_scalars, size, N, d_table, npoints, com_scale=16, layer_num=1):
+    lib = load()
+    rows = size // (N * com_scale)
+    out = np.zeros((rows, 12), dtype=np.uint64)
+    _check(lib.grape_host_hyrax_commit_i32(_dp(d_scalars), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(out)))
+    return out
+
+
+def hyrax_commit_fr(d_scalars, size, N, d_table, npoints, com_scale=16, layer_num=1):
+    lib = load()
+    rows = size // (N * com_scale)
+    out = np.zeros((rows, 12), dtype=np.uint64)
+    _check(lib.grape_host_hyrax_commit_fr(_dp(d_scalars), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(out)))
+    return out
+
+
+def hyrax_open_verify(d_tensor, size, N, d_table, npoints, eval_point, c, com_scale=16, layer_num=1):
+    lib = load()
+    pt = _fr(eval_point)
+    c = _fr(c, 1)
+    res = np.zeros(4, dtype=np.uint64)
+    ok = ctypes.c_int(0)
+    _check(lib.grape_host_hyrax_open_verify(_dp(d_tensor), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(pt),
+                                            pt.shape[0], _hp(c), _hp(res), ctypes.byref(ok)))
+    return res, bool(ok.value)
+
+
+def tlookup_range_prove(dS, D, low, length, alpha, u, v, d_table, npoints, com_scale, msm_size, want_commitments=False):
+    lib = load()
+    alpha, u, v = _fr(alpha, 1), _fr(u), _fr(v)
+    size = 1 << max(0, (length - 1).bit_length())
+    m = np.zeros((size, 4), dtype=np.uint64)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    sc = np.zeros(4, dtype=np.uint64)
+    Dp = 1 << max(0, (D - 1).bit_length())
+    comA = np.zeros((Dp // (msm_size * com_scale), 12), dtype=np.uint64) if want_commitments else None
+    logn = (size - 1).bit_length()
+    mN = 1 << (logn // 2)
+    comm = np.zeros((size // (mN * com_scale), 12), dtype=np.uint64) if want_commitments else None
+    ct = ctypes.c_double(0)
+    _check(lib.grape_host_tlookup_range_prove(_dp(dS), D, low, length, _hp(alpha), _hp(u), _hp(v), u.shape[0], _dp(d_table),
+                                              npoints, com_scale, msm_size, _hp(m), _hp(tr), ctypes.byref(nr), _hp(sc),
+                                              _hp(comA), _hp(comm), ctypes.byref(ct)))
+    return {"m": m, "transcript": tr[: nr.value].copy(), "S_claim": sc, "com_A": comA, "com_m": comm, "commit_s": ct.value}
+
+
+def tlookup_mapping_prove(dS_in, dS_out, D, low, length, table, alpha, r, u, v, d_table, npoints, com_scale, msm_size):
+    lib = load()
+    alpha, r, u, v = _fr(alpha, 1), _fr(r, 1), _fr(u), _fr(v)
+    table = np.ascontiguousarray(table, dtype=np.int32)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    sc = np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_tlookup_mapping_prove(_dp(dS_in), _dp(dS_out), D, low, length, _hp(table), _hp(alpha), _hp(r),
+                                                _hp(u), _hp(v), u.shape[0], _dp(d_table), npoints, com_scale, msm_size,
+                                                _hp(tr), ctypes.byref(nr), _hp(sc)))
+    return tr[: nr.value].copy(), sc
+
+
+def fr_op(op, a, b=None):
+    lib = load()
+    a = _fr(a, 1)
+    b = _fr(b, 1) if b is not None else None
+    out = np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_fr_op(op, _hp(a), _hp(b), _hp(out)))
+    return out
+
+
+def g1_mul_generator(k_mont):
+    lib = load()
+    k = _fr(k_mont, 1)
+    out = np.zeros(12, dtype=np.uint64)
+    _check(lib.grape_host_g1_mul_generator(_hp(k), _hp(out)))
+    return out

@@ -1,0 +1,144 @@
+#include "fr.hpp"
+#include <ostream>
+#include <iomanip>
+
+namespace {
+struct Xoshiro {
+    uint64_t s[4];
+    static uint64_t splitmix(uint64_t& x) {
+        uint64_t z = (x += 0x9e3779b97f4a7c15ull);
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+    }
+    void seed(uint64_t x) { for (int i = 0; i < 4; i++) s[i] = splitmix(x); }
+    static uint64_t rotl(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+    uint64_t next() {
+        uint64_t r = rotl(s[1] * 5, 7) * 9, t = s[1] << 17;
+        s[2] ^= s[0]; s[3] ^= s[1]; s[1] ^= s[2]; s[0] ^= s[3]; s[2] ^= t; s[3] = rotl(s[3], 45);
+        return r;
+    }
+};
+Xoshiro& rng() {
+    static Xoshiro g = [] { Xoshiro x; x.seed(0x47524150452d4d49ull); return x; }();
+    return g;
+}
+bool below_modulus(const uint32_t* a) {
+    for (int i = 7; i >= 0; i--) {
+        uint32_t m = grape::FrParams::mod(i);
+        if (a[i] < m) return true;
+        if (a[i] > m) return false;
+    }
+    return false;
+}
+}  // namespace
+
+Fr::Fr(long x) {
+    unsigned long ax = x < 0 ? 0ul - (unsigned long)x : (unsigned long)x;
+    fr_t raw = grape::Fr::zero();
+    raw.v[0] = (uint32_t)ax;
+    raw.v[1] = (uint32_t)(ax >> 32);
+    v = grape::to_mont(raw);
+    if (x < 0) v = grape::neg(v);
+}
+
+void Fr::seed(uint64_t s) { rng().seed(s); }
+
+Fr Fr::random_element() {
+    for (;;) {
+        fr_t raw;
+        for (int i = 0; i < 4; i++) {
+            uint64_t w = rng().next();
+            raw.v[2 * i] = (uint32_t)w;
+            raw.v[2 * i + 1] = (uint32_t)(w >> 32);
+        }
+        raw.v[7] &= 0x7fffffffu;
+        if (below_modulus(raw.v)) return Fr(raw);   // a uniform residue read as Montgomery form is uniform
+    }
+}
+
+Fr& Fr::invert() {
+    v = grape::inverse(v);
+    return *this;
+}
+
+void Fr::to_plain(uint32_t out[8]) const {
+    fr_t t = grape::from_mont(v);
+    for (int i = 0; i < 8; i++) out[i] = t.v[i];
+}
+
+std::ostream& operator<<(std::ostream& os, const Fr& x) {
+    uint32_t w[8];
+    x.to_plain(w);
+    std::ios_base::fmtflags f = os.flags();
+    os << "0x";
+    for (int i = 7; i >= 0; i--) os << std::hex << std::setw(8) << std::setfill('0') << w[i];
+    os.flags(f);
+    return os;
+}
+
+// ------------------------------------------------------------------ G1
+static const uint32_t kGenX[12] = {0xfd530c16u, 0x5cb38790u, 0x9976fff5u, 0x7817fc67u, 0x143ba1c1u, 0x154f95c7u,
+                                   0xf3d0e747u, 0xf0ae6acdu, 0x21dbf440u, 0xedce6eccu, 0x9e0bfb75u, 0x12017741u};
+static const uint32_t kGenY[12] = {0x0ce72271u, 0xbaac93d5u, 0x7918fd8eu, 0x8c22631au, 0x570725ceu, 0xdd595f13u,
+                                   0x50405194u, 0x51ac5829u, 0xad0059c0u, 0x0e1c8c3fu, 0x5008a26au, 0x0bbc3efcu};
+
+G1::G1(const affine_t& a) {
+    if (a.is_inf()) {
+        p = grape::G1Jac::inf();
+    } else {
+        p.x = a.x;
+        p.y = a.y;
+        p.z = grape::Fp::one();
+    }
+}
+
+G1 G1::one() {
+    affine_t a;
+    for (int i = 0; i < 12; i++) {
+        a.x.v[i] = kGenX[i];
+        a.y.v[i] = kGenY[i];
+    }
+    return G1(a);
+}
+
+G1 G1::random_element() { return Fr::random_element() * G1::one(); }
+
+affine_t G1::to_affine() const { return grape::jac_to_affine(p); }
+
+G1 G1::operator+(const G1& o) const {
+    grape::G1Xyzz a = grape::jac_to_xyzz(p);
+    grape::xyzz_add(a, grape::jac_to_xyzz(o.p));
+    return G1(grape::xyzz_to_jac(a));
+}
+G1 G1::operator-() const {
+    G1 r(*this);
+    r.p.y = grape::neg(r.p.y);
+    return r;
+}
+G1 G1::operator-(const G1& o) const { return *this + (-o); }
+G1 G1::dbl() const {
+    grape::G1Xyzz a = grape::jac_to_xyzz(p);
+    grape::xyzz_dbl(a);
+    return G1(grape::xyzz_to_jac(a));
+}
+bool G1::operator==(const G1& o) const {
+    if (is_zero() || o.is_zero()) return is_zero() && o.is_zero();
+    // X1*Z2^2 == X2*Z1^2 and Y1*Z2^3 == Y2*Z1^3
+    using namespace grape;
+    Fp z1 = sqr(p.z), z2 = sqr(o.p.z);
+    if (mul(p.x, z2) != mul(o.p.x, z1)) return false;
+    return mul(p.y, mul(z2, o.p.z)) == mul(o.p.y, mul(z1, p.z));
+}
+
+G1 operator*(const Fr& k, const G1& pt) {
+    uint32_t w[8];
+    k.to_plain(w);
+    grape::G1Xyzz base = grape::jac_to_xyzz(pt.p);
+    grape::G1Xyzz acc = grape::G1Xyzz::inf();
+    for (int i = 255; i >= 0; i--) {
+        grape::xyzz_dbl(acc);
+        if ((w[i >> 5] >> (i & 31)) & 1) grape::xyzz_add(acc, base);
+    }
+    return G1(grape::xyzz_to_jac(acc));
+}

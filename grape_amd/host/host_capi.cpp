@@ -1,0 +1,227 @@
+#include "host_capi.h"
+#include <cstring>
+#include <string>
+#include "../../include/grape_hip.h"
+#include "ec_operation.hpp"
+#include "fr_tensor.hpp"
+#include "hyrax.hpp"
+#include "prove.hpp"
+#include "tlookup.hpp"
+
+static thread_local std::string g_err;
+
+#define GUARD_BEGIN try {
+#define GUARD_END                      \
+    }                                  \
+    catch (const std::exception& e) {  \
+        g_err = e.what();              \
+        return 1;                      \
+    }                                  \
+    return 0;
+
+static std::vector<Fr> vec_from(const uint32_t* p, uint32_t n) {
+    std::vector<Fr> v(n);
+    if (n) std::memcpy(v.data(), p, 32 * (size_t)n);
+    return v;
+}
+static Fr fr_from(const uint32_t* p) {
+    Fr x;
+    std::memcpy(&x, p, 32);
+    return x;
+}
+static void fr_to(uint32_t* p, const Fr& x) { std::memcpy(p, &x, 32); }
+static FrTensor tensor_from_device(const uint32_t* d, uint32_t n, uint32_t capacity = 0) {
+    FrTensor t(capacity > n ? capacity : n);
+    t.set_size(n);
+    grape_host::check(grape_memcpy_d2d(t.gpu_data, d, 32 * (size_t)n, nullptr), "grape_memcpy_d2d");
+    return t;
+}
+static void put_transcript(const SumcheckTranscript& tr, uint32_t* out, uint32_t* n_rounds) {
+    *n_rounds = (uint32_t)tr.rounds.size();
+    for (size_t r = 0; r < tr.rounds.size(); r++) {
+        std::memset(out + 32 * r, 0, 128);
+        const auto& c = tr.rounds[r].coefficients();
+        for (size_t i = 0; i < c.size() && i < 4; i++) fr_to(out + 32 * r + 8 * i, c[i]);
+    }
+}
+
+extern "C" {
+
+const char* grape_host_last_error(void) { return g_err.c_str(); }
+void grape_host_seed(uint64_t seed) { Fr::seed(seed); }
+
+int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int N, int M, int K, const uint32_t* u, uint32_t nu,
+                            const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
+                            uint32_t* A_claim, uint32_t* B_claim) {
+    GUARD_BEGIN
+    FrTensor A = tensor_from_device(d_A, (uint32_t)(L * N * K));
+    FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * K));
+    Fr claim = fr_from(claim_inout);
+    SumcheckTranscript tr;
+    auto res = prove_matmul(A, B, L, N, M, K, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    fr_to(claim_inout, claim);
+    fr_to(A_claim, res.first);
+    fr_to(B_claim, res.second);
+    put_transcript(tr, transcript, n_rounds);
+    GUARD_END
+}
+
+int grape_host_prove_elemul(const uint32_t* d_A, const uint32_t* d_B, int L, int M, int N, const uint32_t* u, uint32_t nu,
+                            const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
+                            uint32_t* A_claim, uint32_t* B_claim) {
+    GUARD_BEGIN
+    FrTensor A = tensor_from_device(d_A, (uint32_t)(L * M * N));
+    FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * N));
+    Fr claim = fr_from(claim_inout);
+    SumcheckTranscript tr;
+    auto res = prove_eleMul(A, B, L, M, N, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    fr_to(claim_inout, claim);
+    fr_to(A_claim, res.first);
+    fr_to(B_claim, res.second);
+    put_transcript(tr, transcript, n_rounds);
+    GUARD_END
+}
+
+int grape_host_combine_claims(const uint32_t* d_X, uint32_t size, const uint32_t* claims, uint32_t num, const uint32_t* u,
+                              const uint32_t* v, uint32_t nv, uint32_t* transcript, uint32_t* n_rounds, uint32_t* result) {
+    GUARD_BEGIN
+    FrTensor X = tensor_from_device(d_X, size);
+    std::vector<std::vector<Fr>> us(num);
+    for (uint32_t j = 0; j < num; j++) us[j] = vec_from(u + 8 * (size_t)j * nv, nv);
+    SumcheckTranscript tr;
+    Fr r = combine_claims(X, vec_from(claims, num), us, vec_from(v, nv), size, &tr);
+    fr_to(result, r);
+    put_transcript(tr, transcript, n_rounds);
+    GUARD_END
+}
+
+int grape_host_mle_eval(const uint32_t* d_T, uint32_t size, const uint32_t* u, uint32_t nu, uint32_t* out) {
+    GUARD_BEGIN
+    FrTensor T = tensor_from_device(d_T, size);
+    fr_to(out, T(vec_from(u, nu)));
+    GUARD_END
+}
+
+int grape_host_hyrax_commit_i32(const int32_t* d_scalars, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
+                                uint32_t com_scale, uint32_t layer_num, uint32_t* out_affine) {
+    GUARD_BEGIN
+    bn128 G = bn128::one();
+    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    affine_t* c = hyrax.commit_affine(const_cast<int*>(d_scalars), size, N);
+    uint32_t rows = size / (N * com_scale);
+    grape_host::check(grape_memcpy_d2h(out_affine, c, sizeof(affine_t) * (size_t)rows, nullptr), "d2h");
+    grape_free(c);
+    GUARD_END
+}
+
+int grape_host_hyrax_commit_fr(const uint32_t* d_scalars, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
+                               uint32_t com_scale, uint32_t layer_num, uint32_t* out_affine) {
+    GUARD_BEGIN
+    bn128 G = bn128::one();
+    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    FrTensor t = tensor_from_device(d_scalars, size);
+    // through the Jacobian-returning entry point, to cover the reference's return format
+    jacob_t* cj = hyrax.commit(t, size, N);
+    uint32_t rows = size / (N * com_scale);
+    affine_t* ca = nullptr;
+    grape_host::check(grape_malloc((void**)&ca, sizeof(affine_t) * (size_t)rows), "grape_malloc");
+    grape_host::check(grape_g1_jacobian_to_affine((uint32_t*)ca, (const uint32_t*)cj, rows, nullptr), "jac->affine");
+    grape_host::check(grape_memcpy_d2h(out_affine, ca, sizeof(affine_t) * (size_t)rows, nullptr), "d2h");
+    grape_free(ca);
+    grape_free(cj);
+    GUARD_END
+}
+
+int grape_host_hyrax_open_verify(const uint32_t* d_tensor, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
+                                 uint32_t com_scale, uint32_t layer_num, const uint32_t* eval_point, uint32_t n_eval,
+                                 const uint32_t* c, uint32_t* result, int* verified) {
+    GUARD_BEGIN
+    bn128 G = bn128::one();
+    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    FrTensor t = tensor_from_device(d_tensor, size);
+    jacob_t* com = hyrax.commit(t, size, N);
+    std::vector<Fr> pt = vec_from(eval_point, n_eval);
+    Hyrax_proof proof = hyrax.open(t, pt, fr_from(c), size, N);
+    fr_to(result, proof.result);
+    *verified = hyrax.verify(proof, com, pt, fr_from(c), size, N) ? 1 : 0;
+    grape_free(com);
+    GUARD_END
+}
+
+int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low, uint32_t len, const uint32_t* alpha,
+                                   const uint32_t* u, const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints,
+                                   uint32_t com_scale, uint32_t msm_size, uint32_t* m_out, uint32_t* transcript, uint32_t* n_rounds,
+                                   uint32_t* S_claim, uint32_t* com_A_out, uint32_t* com_m_out, double* commit_seconds) {
+    GUARD_BEGIN
+    bn128 G = bn128::one();
+    Hyrax hyrax(1, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    tLookupRange lk(low, len);
+    lk.alpha = fr_from(alpha);
+    lk.set_u(vec_from(u, nuv));
+    uint32_t Dp = 1u << Log2(D);
+    FrTensor S = tensor_from_device(d_S, D, Dp);
+    FrTensor A(Dp);
+    double ct = 0;
+    Fr sc = lk.prove(S, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    fr_to(S_claim, sc);
+    put_transcript(lk.last_transcript, transcript, n_rounds);
+    if (m_out) grape_host::check(grape_memcpy_d2h(m_out, lk.m.gpu_data, 32 * (size_t)lk.m.size, nullptr), "d2h");
+    if (com_A_out) grape_host::check(grape_memcpy_d2h(com_A_out, lk.com_A, sizeof(affine_t) * (size_t)lk.com_A_rows, nullptr), "d2h");
+    if (com_m_out) grape_host::check(grape_memcpy_d2h(com_m_out, lk.com_m, sizeof(affine_t) * (size_t)lk.com_m_rows, nullptr), "d2h");
+    if (commit_seconds) *commit_seconds = ct;
+    GUARD_END
+}
+
+int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S_out, uint32_t D, int32_t low, uint32_t len,
+                                     const int32_t* map, const uint32_t* alpha, const uint32_t* r, const uint32_t* u,
+                                     const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints, uint32_t com_scale,
+                                     uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim) {
+    GUARD_BEGIN
+    bn128 G = bn128::one();
+    Hyrax hyrax(1, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    // r is drawn in the constructor; to pin it, seed-independent, rebuild the table with the given r
+    struct Pinned : tLookupRangeMapping {
+        Pinned(int low, uint len, const int* map, const Fr& r_) : tLookupRangeMapping(low, len, map) {
+            r = r_;
+            grape_host::check(grape_tlookup_init((uint32_t*)T.gpu_data, (uint32_t*)B.gpu_data, low, len,
+                                                 (uint32_t*)grape_host::device_scalar(beta), (uint32_t*)mapped_vals.gpu_data,
+                                                 (uint32_t*)grape_host::device_scalar(r), nullptr),
+                              "grape_tlookup_init");
+        }
+    } lk(low, len, map, fr_from(r));
+    lk.alpha = fr_from(alpha);
+    lk.set_u(vec_from(u, nuv));
+    uint32_t Dp = 1u << Log2(D);
+    FrTensor S_in = tensor_from_device(d_S_in, D);
+    FrTensor S_out = tensor_from_device(d_S_out, D);
+    FrTensor A(Dp);
+    double ct = 0;
+    Fr sc = lk.prove(S_in, S_out, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    fr_to(S_claim, sc);
+    put_transcript(lk.last_transcript, transcript, n_rounds);
+    GUARD_END
+}
+
+int grape_host_fr_op(int op, const uint32_t* a, const uint32_t* b, uint32_t* out) {
+    GUARD_BEGIN
+    Fr x = fr_from(a), y = b ? fr_from(b) : Fr::zero(), r;
+    switch (op) {
+        case 0: r = x + y; break;
+        case 1: r = x - y; break;
+        case 2: r = x * y; break;
+        case 3: r = x.inverse(); break;
+        default: throw std::runtime_error("bad op");
+    }
+    fr_to(out, r);
+    GUARD_END
+}
+
+int grape_host_g1_mul_generator(const uint32_t* k_mont, uint32_t* out_affine) {
+    GUARD_BEGIN
+    bn128 p = fr_from(k_mont) * bn128::one();
+    affine_t a = p.to_affine();
+    std::memcpy(out_affine, &a, sizeof a);
+    GUARD_END
+}
+
+}  // extern "C"

@@ -1,0 +1,70 @@
+/*
+ * C entry points over the C++ host classes (FrTensor, Hyrax, prove_matmul, tLookupRange, ...),
+ * for callers without a C++ toolchain (the Python test-suite and benchmark bind these with
+ * ctypes).  Every function returns 0 on success and 1 after a C++ exception, whose message
+ * grape_host_last_error() returns.  Pointers named d_* are device memory; field elements in
+ * host memory are 8 x u32 Montgomery limbs, affine points 24 x u32.
+ */
+#ifndef GRAPE_HOST_CAPI_H
+#define GRAPE_HOST_CAPI_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char *grape_host_last_error(void);
+void grape_host_seed(uint64_t seed);
+
+/* prove_matmul on copies of the device tensors d_A (L*N*K) and d_B (L*M*K).  transcript receives
+ * 4 coefficients (8 u32 each) per round. */
+int grape_host_prove_matmul(const uint32_t *d_A, const uint32_t *d_B, int L, int N, int M, int K, const uint32_t *u,
+                            uint32_t nu, const uint32_t *v, uint32_t nv, uint32_t *claim_inout, uint32_t *transcript,
+                            uint32_t *n_rounds, uint32_t *A_claim, uint32_t *B_claim);
+int grape_host_prove_elemul(const uint32_t *d_A, const uint32_t *d_B, int L, int M, int N, const uint32_t *u, uint32_t nu,
+                            const uint32_t *v, uint32_t nv, uint32_t *claim_inout, uint32_t *transcript,
+                            uint32_t *n_rounds, uint32_t *A_claim, uint32_t *B_claim);
+/* combine_claims: num claims about d_X (size elements) at points u (num x nv elements, row-major). */
+int grape_host_combine_claims(const uint32_t *d_X, uint32_t size, const uint32_t *claims, uint32_t num, const uint32_t *u,
+                              const uint32_t *v, uint32_t nv, uint32_t *transcript, uint32_t *n_rounds, uint32_t *result);
+/* FrTensor::operator()(u) on a copy of d_T. */
+int grape_host_mle_eval(const uint32_t *d_T, uint32_t size, const uint32_t *u, uint32_t nu, uint32_t *out);
+
+/* Hyrax over a reference-format device table (k*G_i, k < 256, stride npoints_total).
+ * Commits d_scalars (int32) and writes rows = size/(N*com_scale) affine points to out_affine (host). */
+int grape_host_hyrax_commit_i32(const int32_t *d_scalars, uint32_t size, uint32_t N, const uint32_t *d_table,
+                                uint32_t npoints, uint32_t com_scale, uint32_t layer_num, uint32_t *out_affine);
+int grape_host_hyrax_commit_fr(const uint32_t *d_scalars, uint32_t size, uint32_t N, const uint32_t *d_table,
+                               uint32_t npoints, uint32_t com_scale, uint32_t layer_num, uint32_t *out_affine);
+/* commit + open at eval_point with blinding challenge c, then verify; *verified = 1/0,
+ * result = the opened evaluation, which also equals the multilinear extension at eval_point. */
+int grape_host_hyrax_open_verify(const uint32_t *d_tensor, uint32_t size, uint32_t N, const uint32_t *d_table,
+                                 uint32_t npoints, uint32_t com_scale, uint32_t layer_num, const uint32_t *eval_point,
+                                 uint32_t n_eval, const uint32_t *c, uint32_t *result, int *verified);
+
+/*
+ * tLookupRange(low, len).prove on a copy of the witness d_S (D elements).  alpha, u, v are host
+ * values (u, v: nuv elements).  Outputs: multiplicities as len Fr elements (host), the
+ * transcript, S(v), and the commitments of A and m (affine, host; pass NULL to skip).
+ * d_table/npoints/com_scale describe the Hyrax used for those commitments.
+ */
+int grape_host_tlookup_range_prove(const uint32_t *d_S, uint32_t D, int32_t low, uint32_t len, const uint32_t *alpha,
+                                   const uint32_t *u, const uint32_t *v, uint32_t nuv, const uint32_t *d_table,
+                                   uint32_t npoints, uint32_t com_scale, uint32_t msm_size, uint32_t *m_out,
+                                   uint32_t *transcript, uint32_t *n_rounds, uint32_t *S_claim, uint32_t *com_A_out,
+                                   uint32_t *com_m_out, double *commit_seconds);
+/* tLookupRangeMapping with table map[len] (host int32) and random combiner r. */
+int grape_host_tlookup_mapping_prove(const uint32_t *d_S_in, const uint32_t *d_S_out, uint32_t D, int32_t low,
+                                     uint32_t len, const int32_t *map, const uint32_t *alpha, const uint32_t *r,
+                                     const uint32_t *u, const uint32_t *v, uint32_t nuv, const uint32_t *d_table,
+                                     uint32_t npoints, uint32_t com_scale, uint32_t msm_size, uint32_t *transcript,
+                                     uint32_t *n_rounds, uint32_t *S_claim);
+/* Host-side scalar arithmetic checks: out = a op b with op in {0:+, 1:-, 2:*, 3: a^-1}. */
+int grape_host_fr_op(int op, const uint32_t *a, const uint32_t *b, uint32_t *out);
+/* k * G as a host computation (affine out) */
+int grape_host_g1_mul_generator(const uint32_t *k_mont, uint32_t *out_affine);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,196 @@
+#include "hyrax.hpp"
+#include <cassert>
+#include "../../include/grape_hip.h"
+
+using grape_host::check;
+static inline uint32_t* W(void* p) { return reinterpret_cast<uint32_t*>(p); }
+static inline const uint32_t* W(const void* p) { return reinterpret_cast<const uint32_t*>(p); }
+
+Hyrax_proof::Hyrax_proof(Fr result_, size_t z_len, bn128 commit_d_, bn128 commit_ad_)
+    : z_size(z_len), result(result_), commit_d(commit_d_), commit_ad(commit_ad_) {
+    z = new Fr[z_size];
+}
+Hyrax_proof::~Hyrax_proof() { delete[] z; }
+Hyrax_proof::Hyrax_proof(const Hyrax_proof& o) : z_size(o.z_size), result(o.result), commit_d(o.commit_d), commit_ad(o.commit_ad) {
+    z = new Fr[z_size];
+    for (size_t i = 0; i < z_size; i++) z[i] = o.z[i];
+}
+Hyrax_proof& Hyrax_proof::operator=(const Hyrax_proof& o) {
+    if (this != &o) {
+        delete[] z;
+        z_size = o.z_size;
+        result = o.result;
+        commit_d = o.commit_d;
+        commit_ad = o.commit_ad;
+        z = new Fr[z_size];
+        for (size_t i = 0; i < z_size; i++) z[i] = o.z[i];
+    }
+    return *this;
+}
+
+Hyrax::Hyrax(uint layer_num_, uint npoints_, affine_t* g, bn128& G_, uint com_scale_)
+    : com_scale(com_scale_), layer_num(layer_num_), npoints(npoints_ * com_scale_), G(G_), g_affine(g) {
+    grape_host::ensure_init();
+}
+Hyrax::~Hyrax() {
+    grape_free(int16_table_.d);
+    grape_free(int32_table_.d);
+    grape_free(fr_table_.d);
+}
+
+// src/Hyrax.cu:314-315 / :337-338
+void Hyrax::check_shape(uint size, uint N) const {
+    if (size / N / com_scale < layer_num) throw std::runtime_error("Size too small: size < N * com_scale * layer_num");
+    if (N != (1u << Log2(N))) throw std::runtime_error("N must be a power of 2");
+}
+
+// Builds (once) the wide table over the first `rowlen` generators; false when it exceeds the budget.
+bool Hyrax::ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K) {
+    if (t.d && t.ngen >= rowlen && t.c == c && t.nw == nw) return true;
+    size_t bytes = grape_g1_wide_table_bytes(rowlen, nw, K);
+    if (bytes > table_budget_) return false;
+    if (rowlen > npoints) throw std::runtime_error("row longer than the generator set");
+    grape_free(t.d);
+    t = WideTable();
+    check(grape_malloc((void**)&t.d, bytes), "grape_malloc");
+    // generators are row k = 1 of the reference-format table
+    check(grape_g1_wide_table_gen(W(t.d), W(g_affine + npoints), rowlen, c, nw, K, nullptr), "grape_g1_wide_table_gen");
+    t.ngen = rowlen;
+    t.c = c;
+    t.nw = nw;
+    t.K = K;
+    return true;
+}
+
+affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
+    check_shape(size, N);
+    const uint rowlen = N * com_scale;
+    const uint rows = size / rowlen;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
+    // small-scalar fast path: one signed 16-bit digit per scalar, one mixed addition per element
+    if (int16_ok_ && ensure_table(int16_table_, rowlen, 16, 1, 32768)) {
+        int rc = grape_commit_i32(W(out), tensor, size, rowlen, W(int16_table_.d), int16_table_.ngen, 16, 1, 32768, nullptr);
+        if (rc == GRAPE_OK) return out;
+        if (rc != GRAPE_EINVAL) check(rc, "grape_commit_i32");
+        int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
+    }
+    if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
+        check(grape_commit_i32(W(out), tensor, size, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr), "grape_commit_i32");
+    } else {
+        check(grape_commit_i32_ref_table(W(out), tensor, size, rowlen, W(g_affine), npoints, nullptr), "grape_commit_i32_ref_table");
+    }
+    return out;
+}
+
+affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
+    check_shape(size, N);
+    const uint rowlen = N * com_scale;
+    const uint rows = size / rowlen;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
+    if (ensure_table(fr_table_, rowlen, 8, 32, 128)) {
+        check(grape_commit_fr(W(out), W(tensor.gpu_data), size, rowlen, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    } else {
+        check(grape_commit_fr_ref_table(W(out), W(tensor.gpu_data), size, rowlen, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
+    }
+    return out;
+}
+
+static jacob_t* to_jacobian(affine_t* aff, uint rows) {
+    jacob_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(jacob_t) * (size_t)rows), "grape_malloc");
+    check(grape_g1_affine_to_jacobian(W(out), W(aff), rows, nullptr), "grape_g1_affine_to_jacobian");
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(aff);
+    return out;
+}
+jacob_t* Hyrax::commit(int* tensor, uint size, uint N) {
+    affine_t* a = commit_affine(tensor, size, N);
+    return to_jacobian(a, size / (N * com_scale));
+}
+jacob_t* Hyrax::commit(FrTensor& tensor, uint size, uint N) {
+    affine_t* a = commit_affine(tensor, size, N);
+    return to_jacobian(a, size / (N * com_scale));
+}
+
+// Hyrax::open, src/Hyrax.cu:237-305: fold the tensor down to one row x of length new_N at the
+// outer variables of the point, blind it as z = c*x + d with a random row d, commit d, and send
+// <a,d>*G where a is the eq-vector of the inner variables.
+Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N) {
+    if (size / N / com_scale < layer_num) throw std::runtime_error("Size too small: size < N * com_scale * layer_num");
+    uint pad_N = 1u << Log2(N);
+    uint new_N = pad_N * com_scale;
+    assert(eval_point_.size() == Log2(size));
+    fr_t* eval_point = grape_host::upload(eval_point_);
+
+    std::vector<Fr> host_d(new_N);
+    for (uint i = 0; i < new_N; i++) host_d[i] = Fr::random_element();
+    FrTensor d = FrTensor::from_host(host_d);
+
+    // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185)
+    affine_t* com_d_dev = nullptr;
+    check(grape_malloc((void**)&com_d_dev, sizeof(affine_t)), "grape_malloc");
+    if (ensure_table(fr_table_, new_N, 8, 32, 128)) {
+        check(grape_commit_fr(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    } else {
+        check(grape_commit_fr_ref_table(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
+    }
+
+    FrTensor x(new_N);
+    tensor.partial_eval(size, eval_point, (size / layer_num) / (N * com_scale), Log2(N * com_scale), N * com_scale);
+    tensor.partial_eval((N * com_scale) * layer_num, eval_point, layer_num, Log2(size / layer_num), N * com_scale);
+    x = tensor;
+    if (pad_N != N) x.pad(tensor, N, pad_N, new_N, Fr::zero());
+
+    tensor.partial_eval(new_N, eval_point, new_N, 0, 1);
+    Fr result = grape_host::download(tensor.gpu_data);
+
+    FrTensor z(new_N);
+    z = x;
+    z *= c;
+    z += d;
+
+    d.partial_eval(d.size, eval_point, new_N, 0, 1);
+    Fr sum_ad = grape_host::download(d.gpu_data);
+    bn128 commit_ad = sum_ad * G;
+
+    affine_t host_com_d;
+    check(grape_memcpy_d2h(&host_com_d, com_d_dev, sizeof(affine_t), nullptr), "d2h");
+    Hyrax_proof proof(result, new_N, bn128(host_com_d), commit_ad);
+    check(grape_memcpy_d2h(proof.z, z.gpu_data, sizeof(fr_t) * (size_t)new_N, nullptr), "d2h");
+    grape_free(com_d_dev);
+    grape_free(eval_point);
+    return proof;
+}
+
+// The driver-side verification of test/HyraxTest.cu:87-125: fold the row commitments at the outer
+// variables, then check  c*C + com_d == com(z)  and  (c*result)*G + com_ad == <a,z>*G.
+bool Hyrax::verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N) {
+    const uint rowlen = N * com_scale;
+    const uint rows = size / rowlen;
+    const uint new_N = (uint)proof.z_size;
+    std::vector<jacob_t> raw(rows);
+    check(grape_memcpy_d2h(raw.data(), commitment, sizeof(jacob_t) * (size_t)rows, nullptr), "d2h");
+    std::vector<bn128> coms(rows);
+    for (uint i = 0; i < rows; i++) coms[i] = bn128(raw[i]);
+    const uint inner = Log2(rowlen);
+    bn128 C = host_partial_me<bn128>(coms.data(), rows, eval_point.begin() + inner, eval_point.end());
+    // com(z) on the device
+    std::vector<Fr> zv(proof.z, proof.z + new_N);
+    FrTensor z = FrTensor::from_host(zv);
+    affine_t* com_z_dev = nullptr;
+    check(grape_malloc((void**)&com_z_dev, sizeof(affine_t)), "grape_malloc");
+    if (ensure_table(fr_table_, new_N, 8, 32, 128)) {
+        check(grape_commit_fr(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    } else {
+        check(grape_commit_fr_ref_table(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
+    }
+    affine_t com_z;
+    check(grape_memcpy_d2h(&com_z, com_z_dev, sizeof(affine_t), nullptr), "d2h");
+    grape_free(com_z_dev);
+    if (!(c * C + proof.commit_d == bn128(com_z))) return false;
+    std::vector<Fr> inner_point(eval_point.begin(), eval_point.begin() + inner);
+    Fr az = z(inner_point);
+    return (c * proof.result) * G + proof.commit_ad == az * G;
+}

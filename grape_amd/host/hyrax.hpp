@@ -1,0 +1,63 @@
+// Hyrax row commitments: the interface of the reference's include/Hyrax.cuh:57-86.
+#pragma once
+#include <vector>
+#include "ec_operation.hpp"
+#include "fr_tensor.hpp"
+
+class Hyrax_proof {
+public:
+    size_t z_size;
+    Fr result;
+    Fr* z;
+    bn128 commit_d;
+    bn128 commit_ad;
+
+    Hyrax_proof(Fr result_, size_t z_len, bn128 commit_d_, bn128 commit_ad_);
+    ~Hyrax_proof();
+    Hyrax_proof(const Hyrax_proof& other);
+    Hyrax_proof& operator=(const Hyrax_proof& other);
+};
+
+class Hyrax {
+public:
+    uint com_scale;
+    uint layer_num;
+    uint npoints;          // generators available = npoints_ * com_scale (also the table stride)
+    bn128 G;
+    affine_t* g_affine;    // reference-format table: g_affine[k*npoints + i] = k*G_i, k < 256 (not owned)
+
+    // com_scale is hard-wired to 16 in the reference (src/Hyrax.cu:229); it is a parameter here
+    // with that default.
+    Hyrax(uint layer_num_, uint npoints_, affine_t* g, bn128& G_, uint com_scale_ = 16);
+    ~Hyrax();
+    Hyrax(const Hyrax&) = delete;
+    Hyrax& operator=(const Hyrax&) = delete;
+
+    // Row commitments as a device array of Jacobian points (Z = 1); the caller frees it with
+    // grape_free, as the reference's callers cudaFree it (test/commit.cu:72).
+    jacob_t* commit(int* tensor, uint size, uint N);
+    jacob_t* commit(FrTensor& tensor, uint size, uint N);
+    // The same commitments as affine points (what the kernels produce).
+    affine_t* commit_affine(int* tensor, uint size, uint N);
+    affine_t* commit_affine(FrTensor& tensor, uint size, uint N);
+
+    Hyrax_proof open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
+    // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
+    // the reference's own verify is an empty stub (src/Hyrax.cu:307-310).
+    bool verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
+
+    // Upper bound for the wide fixed-base tables this object may build (default 64 GiB).  When a
+    // table would not fit, commitments go through the reference-format table instead.
+    void set_table_budget(size_t bytes) { table_budget_ = bytes; }
+
+private:
+    struct WideTable {
+        affine_t* d = nullptr;
+        uint ngen = 0, c = 0, nw = 0, K = 0;
+    };
+    bool ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K);
+    void check_shape(uint size, uint N) const;
+    WideTable int16_table_, int32_table_, fr_table_;
+    bool int16_ok_ = true;
+    size_t table_budget_ = (size_t)64 << 30;
+};

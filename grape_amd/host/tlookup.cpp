@@ -1,0 +1,222 @@
+#include "tlookup.hpp"
+#include <cassert>
+#include <chrono>
+#include <cstdio>
+#include "../../include/grape_hip.h"
+
+using grape_host::check;
+static inline uint32_t* W(fr_t* p) { return reinterpret_cast<uint32_t*>(p); }
+static inline const uint32_t* W(const fr_t* p) { return reinterpret_cast<const uint32_t*>(p); }
+
+// src/tlookup.cu:247: beta is the table size, alpha is random
+tLookup::tLookup(const uint size) : alpha(Fr::random_element()), beta(Fr((long)size)), T(size), B(size), m(size) {}
+tLookup::~tLookup() {
+    grape_free(com_A);
+    grape_free(com_m);
+}
+
+static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
+    uint32_t* hist = nullptr;
+    check(grape_malloc((void**)&hist, sizeof(uint32_t) * (size_t)m.size), "grape_malloc");
+    check(grape_memset_zero(hist, sizeof(uint32_t) * (size_t)m.size, nullptr), "grape_memset_zero");
+    check(grape_tlookup_hist(hist, W(vals.gpu_data), vals.size, low, m.size, nullptr), "grape_tlookup_hist");
+    // src/tlookup.cu:276-281: padding a witness of non-power-of-two length adds zeros
+    if (vals.size != (1u << Log2(vals.size))) {
+        uint32_t zero_count = 0;
+        check(grape_memcpy_d2h(&zero_count, hist + (-low), sizeof(uint32_t), nullptr), "d2h");
+        zero_count += (1u << Log2(vals.size)) - vals.size;
+        check(grape_memcpy_h2d(hist + (-low), &zero_count, sizeof(uint32_t), nullptr), "h2d");
+    }
+    m.get_data(m.size, hist);
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(hist);
+}
+
+// src/tlookup.cu:250-263
+tLookupRange::tLookupRange(int low_, uint len) : tLookup(1u << Log2(len)), low(low_) {
+    // the table always covers the whole power-of-two range T.size (the reference initialises
+    // only the first len entries and leaves the rest unset)
+    check(grape_tlookup_init(W(T.gpu_data), W(B.gpu_data), low, T.size, W(grape_host::device_scalar(beta)), nullptr, nullptr, nullptr),
+          "grape_tlookup_init");
+}
+tLookupRange::~tLookupRange() {}
+
+void tLookupRange::prep(const FrTensor& vals) { histogram_to_m(m, vals, low); }
+
+// Shared body of tLookupRange::prove (src/tlookup.cu:288-343) and tLookupRangeMapping::prove
+// (:397-456) from the inversion on, with tLookup_phase1 (:216-244) and tLookup_phase2 (:192-214).
+// Per round the reference runs tLookup_poly_kernel, three full multilinear evaluations,
+// tLookup_poly_sum_kernel and two sums (:117-151, :153-190); here one fused pass per operand
+// pair produces the same coefficients, weighted by a table of eq(u_low, x) that is halved
+// between rounds.
+Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
+    const uint D = S.size;
+    const uint N = T.size;
+    std::vector<Fr> u = forced_u_.empty() ? random_vec(Log2(D)) : forced_u_;
+    forced_u_.clear();
+    if (u.size() != v.size()) throw std::runtime_error("u.size() != v.size()");
+    if (v.size() != Log2(D)) throw std::runtime_error("u.size() != ceilLog2(D)");
+    if (D % msm_size != 0) throw std::runtime_error("D % msm_size != 0");
+    last_transcript = SumcheckTranscript();
+
+    fr_t* d_beta = grape_host::device_scalar(beta);
+    check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
+    A.set_size(D);
+
+    {   // commitments of A and m (kept, not dropped)
+        auto t0 = std::chrono::steady_clock::now();
+        grape_free(com_A);
+        grape_free(com_m);
+        com_A = hyrax.commit_affine(A, D, msm_size);
+        com_A_rows = D / (msm_size * hyrax.com_scale);
+        uint m_N = 1u << (Log2(N) / 2);
+        com_m = hyrax.commit_affine(m, N, m_N);
+        com_m_rows = N / (m_N * hyrax.com_scale);
+        check(grape_stream_sync(nullptr), "sync");
+        commit_time += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    }
+
+    FrTensor Bm(B);
+    Bm *= m;
+    Fr alpha_sq = alpha * alpha;
+    Fr C = alpha_sq - Bm.sum(N);
+    Fr claim = alpha + alpha_sq;
+    Fr N_div_D = Fr((long)N) * Fr((long)D).invert();
+    const Fr two_inv = Fr(2).invert();
+    const uint logN = Log2(N);
+
+    // eq(u[0 .. nu-2], x) for x < D/2
+    const uint nu = (uint)u.size();
+    FrTensor E(D / 2 ? D / 2 : 1);
+    {
+        fr_t* d_u = grape_host::upload(u);
+        check(grape_eq_table(W(E.gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_table");
+        check(grape_stream_sync(nullptr), "sync");
+        grape_free(d_u);
+    }
+    FrTensor sums(8);
+    Fr alpha_run = alpha;
+    uint cur = D;
+    int ui = (int)nu - 1;      // index of the variable bound in this round (u.back())
+    Fr h[8];
+    // phase 1: D -> N, challenges v[logN ..] from the back
+    for (int vi = (int)v.size() - 1; vi >= (int)logN; vi--, ui--) {
+        const uint half = cur / 2;
+        check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
+              "grape_tlookup_round_sums");
+        check(grape_memcpy_d2h(h, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
+        Polynomial p0({h[0], h[1], h[2]});
+        p0 = p0 * alpha_run;
+        p0 *= Polynomial::eq(u[ui]);
+        Polynomial p1({h[3], h[4]});
+        Polynomial p = p0 + p1 + Polynomial(C * two_inv);
+        if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase1: claim != p(0) + p(1)");
+        claim = p(v[vi]);
+        last_transcript.rounds.push_back(p);
+        last_transcript.claims.push_back(claim);
+        uint32_t* ptrs[2] = {W(A.gpu_data), W(S.gpu_data)};
+        check(grape_fr_fold_msb_multi(ptrs, 2, half, W(grape_host::device_scalar(v[vi])), nullptr), "grape_fr_fold_msb_multi");
+        A.set_size(half);
+        S.set_size(half);
+        if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
+        alpha_run *= Polynomial::eq(u[ui], v[vi]);
+        C = C * two_inv;
+        cur = half;
+    }
+    // phase 2: bind the table variables; T, B, m of this object stay intact
+    FrTensor Bw(B), Tw(T), mw(m);
+    Fr alpha_sq_run = alpha_sq;
+    for (int vi = (int)logN - 1; vi >= 0; vi--, ui--) {
+        const uint half = cur / 2;
+        Fr a3[5], b3[5], c3[3];
+        check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
+              "grape_tlookup_round_sums");
+        check(grape_memcpy_d2h(a3, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
+        check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
+              "grape_tlookup_round_sums");
+        check(grape_memcpy_d2h(b3, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
+        check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(sums.gpu_data), nullptr), "grape_tlookup_mb_sums");
+        check(grape_memcpy_d2h(c3, sums.gpu_data, 3 * sizeof(fr_t), nullptr), "d2h");
+        Polynomial p0({a3[0], a3[1], a3[2]});
+        p0 = p0 * alpha_run;
+        Fr coef = N_div_D * alpha_sq_run;
+        p0 += Polynomial({b3[0] * coef, b3[1] * coef, b3[2] * coef});
+        Polynomial p1({a3[3], a3[4]});
+        Polynomial p2({c3[0], c3[1], c3[2]});
+        Polynomial p = Polynomial::eq(u[ui]) * p0 + p1 - p2 * N_div_D;
+        if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase2: claim != p(0) + p(1)");
+        claim = p(v[vi]);
+        last_transcript.rounds.push_back(p);
+        last_transcript.claims.push_back(claim);
+        uint32_t* ptrs[5] = {W(A.gpu_data), W(S.gpu_data), W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
+        check(grape_fr_fold_msb_multi(ptrs, 5, half, W(grape_host::device_scalar(v[vi])), nullptr), "grape_fr_fold_msb_multi");
+        A.set_size(half);
+        S.set_size(half);
+        if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
+        Fr e = Polynomial::eq(u[ui], v[vi]);
+        alpha_run *= e;
+        alpha_sq_run *= e;
+        cur = half;
+    }
+    return S(0u);
+}
+
+Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
+    uint D = S.size;
+    prep(S);
+    if (D != (1u << Log2(D))) {
+        // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
+        Fr pad_value = Fr::zero();
+        S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
+    }
+    return run(S, A, v, hyrax, msm_size, commit_time);
+}
+
+// ------------------------------------------------------------------ mapping lookup
+void tLookupRangeMapping::init_from_host(const int* host_table, uint len) {
+    if (len != (1u << Log2(len))) throw std::runtime_error("tLookupRangeMapping: len must be a power of two");
+    int* d_int = nullptr;
+    check(grape_malloc((void**)&d_int, sizeof(int) * (size_t)len), "grape_malloc");
+    check(grape_memcpy_h2d(d_int, host_table, sizeof(int) * (size_t)len, nullptr), "h2d");
+    mapped_vals.get_data(len, d_int);
+    check(grape_tlookup_init(W(T.gpu_data), W(B.gpu_data), low, len, W(grape_host::device_scalar(beta)), W(mapped_vals.gpu_data),
+                             W(grape_host::device_scalar(r)), nullptr),
+          "grape_tlookup_init");
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(d_int);
+}
+
+// src/tlookup.cu:350-372
+tLookupRangeMapping::tLookupRangeMapping(const int low_, const uint len, const std::string& filename)
+    : tLookup(len), r(Fr::random_element()), low(low_), mapped_vals(len) {
+    std::vector<int> host(len);
+    FILE* f = std::fopen(filename.c_str(), "rb");
+    if (!f) throw std::runtime_error("tLookupRangeMapping: cannot open " + filename);
+    size_t got = std::fread(host.data(), sizeof(int), len, f);
+    std::fclose(f);
+    if (got != len) throw std::runtime_error("tLookupRangeMapping: short table file " + filename);
+    init_from_host(host.data(), len);
+}
+tLookupRangeMapping::tLookupRangeMapping(const int low_, const uint len, const int* host_table)
+    : tLookup(len), r(Fr::random_element()), low(low_), mapped_vals(len) {
+    init_from_host(host_table, len);
+}
+
+void tLookupRangeMapping::prep(const FrTensor& vals) { histogram_to_m(m, vals, low); }
+
+// src/tlookup.cu:397-456
+Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax,
+                              uint msm_size, double& commit_time) {
+    uint D = S_in.size;
+    prep(S_in);
+    FrTensor S(1u << Log2(D));
+    S.set_size(D);
+    S = S_out;
+    S *= r;
+    S.add_with_size(D, S_in);
+    if (D != (1u << Log2(D))) {
+        Fr pad_value = mapped_vals((uint)(-low)) * r;
+        S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
+    }
+    return run(S, A, v, hyrax, msm_size, commit_time);
+}

@@ -1,0 +1,67 @@
+// tlookup / logUp range and mapping proofs: the interface of the reference's
+// include/tlookup.cuh:37-79.
+#pragma once
+#include <string>
+#include <vector>
+#include "fr_tensor.hpp"
+#include "hyrax.hpp"
+#include "polynomial.hpp"
+#include "prove.hpp"
+
+class tLookup {
+public:
+    Fr alpha, beta;
+    FrTensor T;
+    FrTensor B;
+    FrTensor m;
+
+    tLookup(const uint size);
+
+    // The reference draws the prover's point u inside prove() from an unseeded generator
+    // (src/tlookup.cu:293); by default it comes from the seeded generator of Fr::random_element,
+    // and a caller that needs a reproducible transcript can fix it here (consumed by the next prove).
+    void set_u(const std::vector<Fr>& u) { forced_u_ = u; }
+    // Round polynomials of the most recent prove (the reference keeps none).
+    SumcheckTranscript last_transcript;
+    // Device commitments of A and m made inside prove (affine points); the reference computes
+    // and drops them (src/tlookup.cu:320-321).  Owned by this object.
+    affine_t* com_A = nullptr;
+    affine_t* com_m = nullptr;
+    uint com_A_rows = 0, com_m_rows = 0;
+    ~tLookup();
+
+protected:
+    Fr run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
+    std::vector<Fr> forced_u_;
+};
+
+class tLookupRange : public tLookup {
+public:
+    const int low;
+
+    tLookupRange(int low, uint len);
+    ~tLookupRange();
+
+    void prep(const FrTensor& vals);
+    // Proves every element of S lies in [low, low+len); returns S(v).  S and A are scratch-mutated.
+    Fr prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
+};
+
+class tLookupRangeMapping : public tLookup {
+public:
+    Fr r;
+    int low;
+    FrTensor mapped_vals;
+
+    // table_file holds len raw little-endian int32 values f(low), f(low+1), ...
+    tLookupRangeMapping(const int low, const uint len, const std::string& table_file);
+    // same from host memory
+    tLookupRangeMapping(const int low, const uint len, const int* host_table);
+
+    void prep(const FrTensor& vals);
+    Fr prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size,
+             double& commit_time);
+
+private:
+    void init_from_host(const int* host_table, uint len);
+};

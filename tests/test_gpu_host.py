@@ -1,0 +1,258 @@
+"""GPU parity of the C++ host classes (FrTensor, Hyrax, prove_matmul, tLookupRange, ...) against
+the CPU oracle: transcripts, claims, multiplicities and commitments, bit-exact."""
+import random
+import numpy as np
+import pytest
+import bigref as br
+import orc
+from gpuutil import rand_fr, gaussian_i16, assert_same
+
+pytestmark = pytest.mark.gpu
+R = br.R_MOD
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from grape_amd import ops as o
+    o.init(0)
+    return o
+
+
+@pytest.fixture(scope="module")
+def host():
+    from grape_amd import _host
+    _host.load()
+    return _host
+
+
+@pytest.fixture(scope="module")
+def gens(ops):
+    k = rand_fr(256, 500)
+    h = orc.g1_make_generators(k)
+    d = ops.g1_make_generators(k)
+    return h, d
+
+
+def _int_tensor(shape, seed):
+    rng = np.random.default_rng(seed)
+    return rng.integers(-2**15, 2**15, size=shape).astype(np.int32)
+
+
+@pytest.mark.parametrize("L,N,M,K", [(1, 4, 8, 16), (2, 4, 4, 8), (4, 2, 4, 4), (1, 3, 5, 6), (1, 8, 4, 1),
+                                     (1, 64, 128, 512), (2, 16, 32, 256), (1, 172, 64, 96)])
+def test_prove_matmul_vs_oracle(ops, host, L, N, M, K):
+    import torch
+    A = _int_tensor(L * N * K, 1 + N)
+    B = _int_tensor(L * M * K, 2 + M)
+    lM, lN, lL, lK = br.log2ceil(M), br.log2ceil(N), br.log2ceil(L), br.log2ceil(K)
+    u = rand_fr(br.log2ceil(L * N * M), 3)
+    v = rand_fr(br.log2ceil(L * K), 4)
+    assert u.shape[0] == lM + lN + lL or (N & (N - 1)) or (M & (M - 1))
+    # claim = Y(u): exact integer matmul, embedded, evaluated by the oracle's own fold
+    Y = np.einsum("lnk,lmk->lnm", A.reshape(L, N, K).astype(np.int64), B.reshape(L, M, K).astype(np.int64))
+    Mp, Np, Lp = 1 << lM, 1 << lN, 1 << lL
+    Ypad = np.zeros((Lp, Np, Mp), dtype=np.int64)
+    Ypad[:L, :N, :M] = Y
+    yf = br.fr_pack([int(x) % R for x in Ypad.reshape(-1)]) if Ypad.size <= 4096 else None
+    if yf is None:
+        # larger case: embed through two int32 halves (|Y| < 2^42)
+        lo = (Ypad.reshape(-1) & 0xffff).astype(np.int32)
+        hi = (Ypad.reshape(-1) >> 16).astype(np.int32)
+        sh = br.fr_pack([1 << 16])[0]
+        yf = orc.vec2("orc_fr_vec_add", orc.vec_bcast("orc_fr_vec_bcast_mul", orc.from_i32(hi), sh), orc.from_i32(lo))
+    upad = rand_fr(lM + lN + lL, 3) if u.shape[0] != lM + lN + lL else u
+    if u.shape[0] != lM + lN + lL:
+        pytest.skip("shape whose Log2(L*N*M) differs from the sum of logs")
+    claim0 = orc.mle_eval(yf, upad)
+    Af, Bf = orc.from_i32(A), orc.from_i32(B)
+    st, wtr, wclaim, wac, wbc = orc.prove_matmul(Af, Bf, L, N, M, K, u, v, claim0)
+    assert st == 0
+    dA = ops.fr_from_i32(torch.from_numpy(A).cuda())
+    dB = ops.fr_from_i32(torch.from_numpy(B).cuda())
+    tr, claim, ac, bc = host.prove_matmul(dA, dB, L, N, M, K, u, v, claim0)
+    assert_same(tr, wtr, "transcript")
+    assert_same(claim, wclaim, "final claim")
+    assert_same(ac, wac, "A(v)")
+    assert_same(bc, wbc, "B(v)")
+
+
+def test_prove_matmul_rejects_wrong_claim(ops, host):
+    import torch
+    A, B = _int_tensor(2 * 4, 5), _int_tensor(2 * 4, 6)
+    dA = ops.fr_from_i32(torch.from_numpy(A).cuda())
+    dB = ops.fr_from_i32(torch.from_numpy(B).cuda())
+    with pytest.raises(host.HostError, match="matmul_phase2"):
+        host.prove_matmul(dA, dB, 1, 2, 2, 4, rand_fr(2, 7), rand_fr(2, 8), br.fr_pack([12345])[0])
+
+
+def test_mle_eval_operator(ops, host):
+    t = rand_fr(4096, 11)
+    u = rand_fr(12, 12)
+    assert_same(host.mle_eval(ops.to_dev(t), 4096, u), orc.mle_eval(t, u), "T(u)")
+    # rows of 11008 read as zero-extended to 16384
+    t = orc.from_i32(_int_tensor(2 * 11008, 13))
+    u = rand_fr(15, 14)
+    assert_same(host.mle_eval(ops.to_dev(t), 2 * 11008, u), orc.mle_eval(t, u), "T(u), 11008 columns")
+
+
+@pytest.mark.parametrize("logD,logN,low", [(4, 2, -2), (5, 3, -4), (3, 3, 0), (12, 6, -32), (14, 8, -128), (16, 16, -32768)])
+def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low):
+    import torch
+    hg, dg = gens
+    D, N = 1 << logD, 1 << logN
+    rng = np.random.default_rng(logD * 7 + logN)
+    S = rng.integers(low, low + N, size=D).astype(np.int32)
+    alpha, u, v = rand_fr(1, 21), rand_fr(logD, 22), rand_fr(logD, 23)
+    beta = br.fr_pack([N])[0]
+    Sp = orc.from_i32(S)
+    T, B = orc.tlookup_init(low, N, beta)
+    m = orc.tlookup_prep(Sp, low, N)
+    st, wtr, wsc = orc.tlookup_prove(Sp, T, B, m, alpha[0], beta, u, v)
+    assert st == 0
+    table = ops.g1_table_gen(dg, 256)               # 256 generators: com(m) uses rows of 2^(logN/2)
+    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
+    msm = min(D, 16)
+    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 256, 1, msm, want_commitments=(logD <= 5))
+    assert_same(res["m"], m, "multiplicities")
+    assert_same(res["transcript"], wtr, "transcript")
+    assert_same(res["S_claim"], wsc, "S(v)")
+    assert br.fr_unpack(res["m"]) == [int(x) for x in np.bincount(S.astype(np.int64) - low, minlength=N)]
+    if logD <= 5:
+        # the commitments of A = 1/(S+beta) and of m made inside prove
+        Ainv = orc.vec1("orc_fr_vec_inv", orc.vec_bcast("orc_fr_vec_bcast_add", Sp, beta))
+        tab = orc.g1_table(hg, 256)
+        assert_same(res["com_A"], orc.commit_fr(Ainv, tab, msm, 256), "com(A)")
+        mN = 1 << (logN // 2)
+        assert_same(res["com_m"], orc.commit_fr(m, tab, mN, 256), "com(m)")
+
+
+def test_tlookup_range_rejects_out_of_range(ops, host, gens):
+    import torch
+    hg, dg = gens
+    S = np.array([0, 1, 2, 3, 9, 1, 2, 3, 0, 0, 1, 1, 2, 2, 3, 3], dtype=np.int32)
+    table = ops.g1_table_gen(dg[:16].contiguous(), 256)
+    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
+    with pytest.raises(host.HostError, match="tLookup_phase"):
+        host.tlookup_range_prove(dS, 16, 0, 4, rand_fr(1, 31), rand_fr(4, 32), rand_fr(4, 33), table, 16, 1, 16)
+
+
+def test_tlookup_pads_11008_rows(ops, host, gens):
+    # a witness of 2 x 11008 values is padded to 2 x 16384 with zeros, which are counted in m
+    import torch
+    hg, dg = gens
+    D, low, N = 2 * 11008, -8, 16
+    rng = np.random.default_rng(41)
+    S = rng.integers(low, low + N, size=D).astype(np.int32)
+    alpha, u, v = rand_fr(1, 42), rand_fr(15, 43), rand_fr(15, 44)
+    beta = br.fr_pack([N])[0]
+    Sp = orc.from_i32(S)
+    m = orc.tlookup_prep(Sp, low, N)
+    Spad = np.zeros((32768, 4), dtype=np.uint64)
+    orc.lib().orc_fr_pad(orc.P(Spad), orc.P(Sp), orc.c32(11008), orc.c32(16384), orc.c64(32768), orc.P(np.zeros(4, dtype=np.uint64)))
+    T, B = orc.tlookup_init(low, N, beta)
+    st, wtr, wsc = orc.tlookup_prove(Spad, T, B, m, alpha[0], beta, u, v)
+    assert st == 0
+    table = ops.g1_table_gen(dg[:16].contiguous(), 256)
+    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
+    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 16, 1, 16)
+    assert_same(res["m"], m, "multiplicities with pad fix-up")
+    assert_same(res["transcript"], wtr, "transcript")
+    assert_same(res["S_claim"], wsc, "S(v)")
+
+
+def test_tlookup_mapping_prove_vs_oracle(ops, host, gens):
+    import torch
+    hg, dg = gens
+    logD, logN, low = 10, 6, -32
+    D, N = 1 << logD, 1 << logN
+    rng = np.random.default_rng(51)
+    fmap = rng.integers(-1000, 1000, size=N).astype(np.int32)      # a seeded synthetic table x -> f(x)
+    S_in = rng.integers(low, low + N, size=D).astype(np.int32)
+    S_out = fmap[S_in - low]
+    alpha, r, u, v = rand_fr(1, 52), rand_fr(1, 53), rand_fr(logD, 54), rand_fr(logD, 55)
+    beta = br.fr_pack([N])[0]
+    T, B = orc.tlookup_init(low, N, beta, orc.from_i32(fmap), r[0])
+    m = orc.tlookup_prep(orc.from_i32(S_in), low, N)
+    S = orc.vec2("orc_fr_vec_add", orc.vec_bcast("orc_fr_vec_bcast_mul", orc.from_i32(S_out), r[0]), orc.from_i32(S_in))
+    st, wtr, wsc = orc.tlookup_prove(S, T, B, m, alpha[0], beta, u, v)
+    assert st == 0
+    table = ops.g1_table_gen(dg[:16].contiguous(), 256)
+    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
+    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
+    tr, sc = host.tlookup_mapping_prove(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
+    assert_same(tr, wtr, "transcript")
+    assert_same(sc, wsc, "S(v)")
+    # a wrong output value is caught
+    S_out2 = S_out.copy()
+    S_out2[5] += 1
+    with pytest.raises(host.HostError, match="tLookup_phase"):
+        host.tlookup_mapping_prove(dSi, ops.fr_from_i32(torch.from_numpy(S_out2).cuda()), D, low, N, fmap, alpha, r, u, v,
+                                   table, 16, 1, 16)
+
+
+def test_hyrax_class_commits(ops, host, gens):
+    import torch
+    hg, dg = gens
+    npoints = 256
+    table = ops.g1_table_gen(dg, 256)
+    htab = orc.g1_table(hg, 256)
+    # com_scale = 16 (the reference's value): rows of N*16
+    W = gaussian_i16((8, 256), 61)
+    got = host.hyrax_commit_i32(torch.from_numpy(W).cuda(), W.size, 16, table, npoints, com_scale=16)
+    assert_same(got, orc.commit_i32(W, htab, 256, npoints), "Hyrax::commit(int*) int16 path")
+    # values outside int16 fall back to the general int32 tables
+    W2 = _int_tensor((4, 256), 62) * 40000
+    got = host.hyrax_commit_i32(torch.from_numpy(W2).cuda(), W2.size, 16, table, npoints, com_scale=16)
+    assert_same(got, orc.commit_i32(W2, htab, 256, npoints), "Hyrax::commit(int*) int32 path")
+    # com_scale = 1, shorter rows than the generator set
+    W3 = gaussian_i16((16, 64), 63)
+    got = host.hyrax_commit_i32(torch.from_numpy(W3).cuda(), W3.size, 64, table, npoints, com_scale=1)
+    assert_same(got, orc.commit_i32(W3, htab, 64, npoints), "com_scale = 1")
+    s = rand_fr(2 * 64, 64)
+    got = host.hyrax_commit_fr(ops.to_dev(s), 128, 4, table, npoints, com_scale=16)
+    assert_same(got, orc.commit_fr(s, htab, 64, npoints), "Hyrax::commit(FrTensor&)")
+    with pytest.raises(host.HostError, match="power of 2"):
+        host.hyrax_commit_i32(torch.from_numpy(W).cuda(), W.size, 12, table, npoints, com_scale=16)
+    with pytest.raises(host.HostError, match="Size too small"):
+        host.hyrax_commit_i32(torch.from_numpy(W).cuda(), 128, 16, table, npoints, com_scale=16)
+
+
+def test_hyrax_open_and_verify(ops, host, gens):
+    hg, dg = gens
+    npoints = 64
+    table = ops.g1_table_gen(dg[:64].contiguous(), 256)
+    size, N = 64 * 8, 4                   # 8 rows of 4*16 = 64
+    t = rand_fr(size, 71)
+    pt = rand_fr(9, 72)
+    c = rand_fr(1, 73)
+    res, ok = host.hyrax_open_verify(ops.to_dev(t), size, N, table, npoints, pt, c, com_scale=16)
+    assert ok
+    assert_same(res, orc.mle_eval(t, pt), "opened value = T(point)")
+
+
+def test_elemul_and_combine_claims_invariants(ops, host):
+    # no oracle restatement exists for these two; they are checked against the definition:
+    # the returned evaluations are the multilinear extensions at v and the claim chain closes
+    rng = random.Random(81)
+    L, M, N = 1, 4, 8
+    n = L * M * N
+    A = [rng.randrange(R) for _ in range(n)]
+    B = [rng.randrange(R) for _ in range(n)]
+    u = [rng.randrange(R) for _ in range(5)]
+    v = [rng.randrange(R) for _ in range(5)]
+    claim0 = sum(br.eq_weight(i, u) * A[i] * B[i] for i in range(n)) % R
+    tr, claim, ac, bc = host.prove_elemul(ops.to_dev(br.fr_pack(A)), ops.to_dev(br.fr_pack(B)), L, M, N, br.fr_pack(u), br.fr_pack(v),
+                                          br.fr_pack([claim0])[0])
+    assert tr.shape[0] == 5
+    assert br.fr_unpack(ac)[0] == br.mle_eval(A, v) and br.fr_unpack(bc)[0] == br.mle_eval(B, v)
+    X = [rng.randrange(R) for _ in range(16)]
+    us = [[rng.randrange(R) for _ in range(4)] for _ in range(3)]
+    vv = [rng.randrange(R) for _ in range(4)]
+    claims = [br.mle_eval(X, uj) for uj in us]
+    tr, res = host.combine_claims(ops.to_dev(br.fr_pack(X)), 16, br.fr_pack(claims),
+                                  np.stack([br.fr_pack(uj) for uj in us]), br.fr_pack(vv))
+    assert tr.shape[0] == 4
+    assert br.fr_unpack(res)[0] == br.mle_eval(X, vv)
