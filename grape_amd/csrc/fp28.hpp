@@ -1,0 +1,331 @@
+// BLS12-381 Fp on 14 signed limbs of 28 bits with lazy reduction - the working form of the
+// commitment kernels.
+//
+// Why: on gfx950 a 32x32+64 multiply-add (v_mad_i64_i32 / v_mad_u64_u32) issues at the same rate
+// as an addition, so the cost of a field product is its instruction count, and with saturated
+// 32-bit limbs two thirds of the instructions are carry handling.  With 28-bit limbs every limb
+// product is < 2^58, a whole column of an (a*b + m*p) row set fits a 64-bit accumulator, and a
+// limb product is exactly ONE instruction; signed limbs make subtraction limb-wise, with no
+// borrow chain and no bias.
+//
+// Representation: x = sum_i v[i] * 2^(28 i), v[i] signed 32-bit.  "Normalised" means
+// 0 <= v[i] < 2^28 for i < 13 (the top limb carries the sign and the overflow).  A value stands
+// for its residue mod p; arithmetic is Montgomery with radix R' = 2^392.  The canonical memory
+// form elsewhere in the library is the reference's: 12 x 32-bit limbs, radix 2^384
+// (include/field/mont_t.cuh, include/field/bls12-381.cuh:7-23); conversion is exact both ways.
+//
+// Bounds (checked by the callers' comments): mul28(a, b) needs |a| < alpha*p, |b| < beta*p with
+// alpha*beta <= 2^11 and limb magnitudes with 14 * 2^(la+lb) < 2^62, i.e. la + lb <= 58; its
+// result is normalised and lies in (0, 3p).
+#pragma once
+#include "curve.hpp"
+
+namespace grape {
+
+struct Fp28 {
+    int32_t v[14];
+};
+
+namespace fp28 {
+
+constexpr int N = 14;
+constexpr int W = 28;
+constexpr uint32_t MASK = (1u << W) - 1;
+constexpr uint32_t PINV = 0xffcfffdu;   // -p^-1 mod 2^28
+
+GRAPE_HD int32_t P(int i) {
+    constexpr int32_t t[14] = {0xfffaaab, 0xfefffff, 0x3ffffb9, 0xfffeb15, 0x6241eab, 0xa0f6b0f, 0xf6730d2,
+                               0xf38512b, 0x4774b84, 0x4bacd76, 0xba7b643, 0xe69a4b1, 0x1ea397f, 0x001a011};
+    return t[i];
+}
+GRAPE_HD int32_t P2(int i) {   // 2p
+    constexpr int32_t t[14] = {0xfff5556, 0xfdfffff, 0x7ffff73, 0xfffd62a, 0xc483d57, 0x41ed61e, 0xece61a5,
+                               0xe70a257, 0x8ee9709, 0x9759aec, 0x74f6c86, 0xcd34963, 0x3d472ff, 0x0034022};
+    return t[i];
+}
+GRAPE_HD int32_t ONE(int i) {   // 2^392 mod p
+    constexpr int32_t t[14] = {0x347fcb8, 0xd800000, 0x002b119, 0x0cde6d2, 0xc7212e0, 0x83a2090, 0x037669f,
+                               0xda0f73e, 0x9b09b42, 0x1297bb0, 0x515d98f, 0x012ca7c, 0x659fcfa, 0x000577a};
+    return t[i];
+}
+GRAPE_HD int32_t C384(int i) {   // 2^384 mod p: mul28(x*2^392, C384) = x*2^384
+    constexpr int32_t t[14] = {0x002fffd, 0x0900000, 0xc000276, 0x000bc40, 0x8baebf4, 0x5753c75, 0x55f4898,
+                               0x7052574, 0x7ce5853, 0x56ec6d7, 0x71a97a2, 0xe4935c0, 0xec3fa80, 0x0015f65};
+    return t[i];
+}
+// Montgomery (radix 2^384) form of 2^8, 32-bit limbs: mul(x*2^384, M256) = x*2^392 mod p
+GRAPE_HD uint32_t M256(int i) {
+    constexpr uint32_t t[12] = {0x0347fcb8u, 0x19d80000u, 0x6d2002b1u, 0x12e00cdeu, 0xa2090c72u, 0x37669f83u,
+                                0xda0f73e0u, 0x09b09b42u, 0x8f1297bbu, 0xa7c515d9u, 0xfcfa012cu, 0x0577a659u};
+    return t[i];
+}
+
+GRAPE_HD Fp28 one() {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = ONE(i);
+    return r;
+}
+GRAPE_HD Fp28 zero() {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = 0;
+    return r;
+}
+
+// limb-wise, no carries: the caller tracks magnitudes
+GRAPE_HD Fp28 add(const Fp28& a, const Fp28& b) {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = a.v[i] + b.v[i];
+    return r;
+}
+GRAPE_HD Fp28 sub(const Fp28& a, const Fp28& b) {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = a.v[i] - b.v[i];
+    return r;
+}
+GRAPE_HD Fp28 neg(const Fp28& a) {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = -a.v[i];
+    return r;
+}
+GRAPE_HD Fp28 cneg(const Fp28& a, bool flag) {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = flag ? -a.v[i] : a.v[i];
+    return r;
+}
+
+// signed carry propagation: same value, limbs 0..12 in [0, 2^28)
+GRAPE_HD Fp28 normalize(const Fp28& a) {
+    Fp28 r;
+    int32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < N - 1; i++) {
+        int32_t t = a.v[i] + c;
+        r.v[i] = t & (int32_t)MASK;
+        c = t >> W;   // arithmetic
+    }
+    r.v[N - 1] = a.v[N - 1] + c;
+    return r;
+}
+
+// Montgomery product a*b/2^392 (mod p), result normalised in (0, 3p).
+GRAPE_HD Fp28 mul(const Fp28& a, const Fp28& b) {
+    int64_t C[2 * N];
+#pragma unroll
+    for (int k = 0; k < 2 * N; k++) C[k] = 0;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)a.v[j] * (int64_t)b.v[i];
+        const int32_t m = (int32_t)(((uint32_t)C[i] * PINV) & MASK);
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)m * (int64_t)P(j);
+        C[i + 1] += C[i] >> W;   // C[i] is now a multiple of 2^28
+    }
+    // the quotient may be slightly negative: add p, then carry-propagate
+    Fp28 r;
+    int64_t c = 0;
+#pragma unroll
+    for (int k = 0; k < N - 1; k++) {
+        int64_t t = C[N + k] + (int64_t)P(k) + c;
+        r.v[k] = (int32_t)((uint32_t)t & MASK);
+        c = t >> W;
+    }
+    r.v[N - 1] = (int32_t)(C[2 * N - 1] + (int64_t)P(N - 1) + c);
+    return r;
+}
+
+// a^2/2^392: the off-diagonal limb products are taken once with a doubled operand.
+GRAPE_HD Fp28 sqr(const Fp28& a) {
+    int64_t C[2 * N];
+#pragma unroll
+    for (int k = 0; k < 2 * N; k++) C[k] = 0;
+    int32_t a2[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) a2[i] = a.v[i] * 2;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        C[2 * i] += (int64_t)a.v[i] * (int64_t)a.v[i];
+#pragma unroll
+        for (int j = i + 1; j < N; j++) C[i + j] += (int64_t)a2[i] * (int64_t)a.v[j];
+    }
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        const int32_t m = (int32_t)(((uint32_t)C[i] * PINV) & MASK);
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)m * (int64_t)P(j);
+        C[i + 1] += C[i] >> W;
+    }
+    Fp28 r;
+    int64_t c = 0;
+#pragma unroll
+    for (int k = 0; k < N - 1; k++) {
+        int64_t t = C[N + k] + (int64_t)P(k) + c;
+        r.v[k] = (int32_t)((uint32_t)t & MASK);
+        c = t >> W;
+    }
+    r.v[N - 1] = (int32_t)(C[2 * N - 1] + (int64_t)P(N - 1) + c);
+    return r;
+}
+
+// Is a normalised value in [0, 3p) congruent to zero, i.e. one of 0, p, 2p?
+GRAPE_HD bool is_zero_mod_p(const Fp28& a) {
+    uint32_t z0 = 0, z1 = 0, z2 = 0;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        z0 |= (uint32_t)a.v[i];
+        z1 |= (uint32_t)(a.v[i] ^ P(i));
+        z2 |= (uint32_t)(a.v[i] ^ P2(i));
+    }
+    return (z0 == 0) | (z1 == 0) | (z2 == 0);
+}
+
+// ---- conversions with the canonical 12 x 32-bit, radix-2^384 Montgomery form ----
+// pure re-limbing of a 384-bit non-negative integer
+GRAPE_HD Fp28 pack(const Fp& x) {
+    Fp28 r;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        const int bit = W * k, q = bit >> 5, s = bit & 31;
+        uint64_t two = (uint64_t)x.v[q] | ((q + 1 < 12) ? ((uint64_t)x.v[q + 1] << 32) : 0);
+        r.v[k] = (int32_t)((uint32_t)(two >> s) & MASK);
+    }
+    return r;
+}
+// inverse of pack for a normalised, non-negative value below 2^384
+GRAPE_HD Fp unpack(const Fp28& a) {
+    Fp r;
+#pragma unroll
+    for (int q = 0; q < 12; q++) {
+        // word q covers bits [32q, 32q+32): limbs k0 = floor(32q/28) .. up to two more
+        const int k0 = (32 * q) / W;
+        uint64_t acc = 0;
+#pragma unroll
+        for (int t = 0; t < 3; t++) {
+            const int k = k0 + t;
+            if (k < N) {
+                const int sh = W * k - 32 * q;   // position of limb k relative to the word
+                if (sh >= 0) {
+                    if (sh < 32) acc |= (uint64_t)(uint32_t)a.v[k] << sh;
+                } else {
+                    acc |= (uint64_t)(uint32_t)a.v[k] >> (-sh);
+                }
+            }
+        }
+        r.v[q] = (uint32_t)acc;
+    }
+    return r;
+}
+// canonical x*2^384 (32-bit limbs) -> x*2^392 (28-bit limbs), canonical and normalised
+GRAPE_HD Fp28 from_canonical(const Fp& x) {
+    Fp m;
+#pragma unroll
+    for (int i = 0; i < 12; i++) m.v[i] = M256(i);
+    return pack(fmul(x, m));
+}
+// value in (-9p, 3p), any limb form -> canonical x*2^384, 32-bit limbs
+GRAPE_HD Fp to_canonical(const Fp28& a) {
+    Fp28 c;
+#pragma unroll
+    for (int i = 0; i < N; i++) c.v[i] = C384(i);
+    Fp28 t = mul(normalize(a), c);   // in (0, 3p), now with radix 2^384
+    // subtract p while the result stays non-negative (at most twice)
+#pragma unroll
+    for (int rep = 0; rep < 2; rep++) {
+        Fp28 d;
+#pragma unroll
+        for (int i = 0; i < N; i++) d.v[i] = t.v[i] - P(i);
+        d = normalize(d);
+        const bool ok = d.v[N - 1] >= 0;
+#pragma unroll
+        for (int i = 0; i < N; i++) t.v[i] = ok ? d.v[i] : t.v[i];
+    }
+    return unpack(t);
+}
+
+}  // namespace fp28
+
+// ------------------------------------------------------------------------------------------------
+// XYZZ accumulator in the 28-bit form.  Invariants between additions:
+//   x in (-9p, 3p) normalised (signed top limb); y in (-3p, 3p) with |limbs| < 2^28;
+//   zz, zzz in (0, 3p) normalised, never congruent to zero; `inf` marks the identity.
+// ------------------------------------------------------------------------------------------------
+struct Xyzz28 {
+    Fp28 x, y, zz, zzz;
+    bool inf;
+};
+struct Affine28 {   // canonical coordinates (in [0,p), normalised)
+    Fp28 x, y;
+};
+
+GRAPE_HD Xyzz28 xyzz28_inf() {
+    Xyzz28 r;
+    r.x = fp28::zero();
+    r.y = fp28::zero();
+    r.zz = fp28::zero();
+    r.zzz = fp28::zero();
+    r.inf = true;
+    return r;
+}
+
+GRAPE_HD G1Xyzz xyzz28_to_canonical(const Xyzz28& a) {
+    if (a.inf) return G1Xyzz::inf();
+    G1Xyzz r;
+    r.x = fp28::to_canonical(a.x);
+    r.y = fp28::to_canonical(a.y);
+    r.zz = fp28::to_canonical(a.zz);
+    r.zzz = fp28::to_canonical(a.zzz);
+    return r;
+}
+GRAPE_HD Xyzz28 xyzz28_from_canonical(const G1Xyzz& a) {
+    Xyzz28 r;
+    r.inf = a.is_inf();
+    r.x = fp28::from_canonical(a.x);
+    r.y = fp28::from_canonical(a.y);
+    r.zz = fp28::from_canonical(a.zz);
+    r.zzz = fp28::from_canonical(a.zzz);
+    return r;
+}
+
+// acc += (negate ? -p : p) for a finite affine point p (the caller skips the identity).
+// Returns false when the addition is one of the exceptional cases (p = +-acc): then acc is left
+// untouched and the caller must take the exact slow path.
+GRAPE_HD bool xyzz28_madd(Xyzz28& acc, const Affine28& p, bool negate) {
+    using namespace fp28;
+    if (acc.inf) {
+        acc.x = p.x;
+        acc.y = cneg(p.y, negate);
+        acc.zz = one();
+        acc.zzz = one();
+        acc.inf = false;
+        return true;
+    }
+    const Fp28 U2 = mul(p.x, acc.zz);                  // 1 * 3            -> (0,3p)
+    const Fp28 S2 = mul(p.y, acc.zzz);                 // 1 * 3            -> (0,3p)
+    const Fp28 Pd = sub(U2, acc.x);                    // (-3p,12p), |limb| < 2^29
+    const Fp28 R = sub(cneg(S2, negate), acc.y);       // (-6p, 6p), |limb| < 2^29
+    const Fp28 PP = sqr(Pd);                           // 144 <= 2^11, 29+29 <= 58
+    const Fp28 ZZ3 = mul(acc.zz, PP);                  // 9
+    if (is_zero_mod_p(ZZ3)) return false;              // PP = 0  <=>  P = 0: doubling or cancellation
+    const Fp28 PPP = mul(Pd, PP);                      // 12 * 3 = 36
+    const Fp28 Q = mul(acc.x, PP);                     // 9 * 3 = 27
+    const Fp28 RR = sqr(R);                            // 36
+    Fp28 X3;
+#pragma unroll
+    for (int i = 0; i < N; i++) X3.v[i] = RR.v[i] - PPP.v[i] - 2 * Q.v[i];   // (-9p, 3p), |limb| < 2^30
+    X3 = normalize(X3);
+    const Fp28 T = sub(Q, X3);                         // (-3p, 12p), |limb| < 2^29
+    const Fp28 Y3 = sub(mul(R, T), mul(acc.y, PPP));   // 6*12 = 72 ; 3*3 = 9 -> (-3p, 3p)
+    acc.zzz = mul(acc.zzz, PPP);                       // 9
+    acc.zz = ZZ3;
+    acc.x = X3;
+    acc.y = Y3;
+    return true;
+}
+
+}  // namespace grape

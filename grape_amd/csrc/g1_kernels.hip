@@ -10,6 +10,7 @@
 // result to affine coordinates.
 #define GRAPE_FP_MUL_OUTLINE 1
 #include "common.hpp"
+#include "fp28.hpp"
 
 namespace grape {
 
@@ -64,6 +65,56 @@ __device__ __forceinline__ Fr ld_fr8(const uint32_t* base, size_t i) {
     r.v[0] = lo.x; r.v[1] = lo.y; r.v[2] = lo.z; r.v[3] = lo.w;
     r.v[4] = hi.x; r.v[5] = hi.y; r.v[6] = hi.z; r.v[7] = hi.w;
     return r;
+}
+
+// Wide-table entry: an affine point in the 28-bit working form, x[14] then y[14] as 32-bit
+// words plus 16 bytes of padding = 128 bytes, so that every gather is exactly one cache line.
+constexpr int kWideEntryWords = 32;
+__device__ __forceinline__ Affine28 ld_entry28(const uint32_t* table, size_t e) {
+    const uint4* q = reinterpret_cast<const uint4*>(table + (size_t)kWideEntryWords * e);
+    uint4 w[7];
+#pragma unroll
+    for (int i = 0; i < 7; i++) w[i] = q[i];
+    const uint32_t* f = reinterpret_cast<const uint32_t*>(w);
+    Affine28 r;
+#pragma unroll
+    for (int i = 0; i < 14; i++) {
+        r.x.v[i] = (int32_t)f[i];
+        r.y.v[i] = (int32_t)f[14 + i];
+    }
+    return r;
+}
+__device__ __forceinline__ void st_entry28(uint32_t* table, size_t e, const G1Affine& a) {
+    Fp28 x = fp28::from_canonical(a.x), y = fp28::from_canonical(a.y);
+    uint32_t f[32];
+#pragma unroll
+    for (int i = 0; i < 14; i++) {
+        f[i] = (uint32_t)x.v[i];
+        f[14 + i] = (uint32_t)y.v[i];
+    }
+    f[28] = f[29] = f[30] = f[31] = 0;
+    uint4* q = reinterpret_cast<uint4*>(table + (size_t)kWideEntryWords * e);
+#pragma unroll
+    for (int i = 0; i < 8; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+}
+__device__ __forceinline__ bool entry_is_inf(const Affine28& a) {
+    uint32_t z = 0;
+#pragma unroll
+    for (int i = 0; i < 14; i++) z |= (uint32_t)a.x.v[i] | (uint32_t)a.y.v[i];
+    return z == 0;
+}
+// acc += +-entry through the 28-bit mixed addition; the rare exceptional step (entry = +-acc)
+// goes through the exact canonical-form addition.
+__device__ __forceinline__ void madd28(Xyzz28& acc, const Affine28& e, bool negate) {
+    if (entry_is_inf(e)) return;
+    if (!xyzz28_madd(acc, e, negate)) {
+        G1Xyzz c = xyzz28_to_canonical(acc);
+        G1Affine a;
+        a.x = fp28::to_canonical(e.x);
+        a.y = fp28::to_canonical(e.y);
+        xyzz_add_affine(c, a, negate);
+        acc = xyzz28_from_canonical(c);
+    }
 }
 
 __device__ __forceinline__ G1Xyzz shfl_down_xyzz(const G1Xyzz& a, int off) {
@@ -195,7 +246,7 @@ __global__ void __launch_bounds__(64) wide_normalize_kernel(uint32_t* table, con
             inv = fmul(inv, p.zzz);
             a = xyzz_to_affine_with_inv(p, zi);
         }
-        st_affine(table, (w * K + kidx) * N + i, a);
+        st_entry28(table, (w * K + kidx) * N + i, a);
     }
 }
 
@@ -215,7 +266,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
     const uint32_t s = (uint32_t)(wave - row * nseg);
     const uint32_t col_end = (s + 1) * seg < rowlen ? (s + 1) * seg : rowlen;
     const uint32_t half = 1u << (c - 1), mask = (c == 32) ? 0xffffffffu : ((1u << c) - 1u);
-    G1Xyzz acc = G1Xyzz::inf();
+    Xyzz28 acc = xyzz28_inf();
     for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
         if (FR) {
             const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
@@ -238,8 +289,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 uint32_t mag = neg ? (mask + 1u - d) : d;
                 if (mag != 0) {
                     if (mag > K) { *err_flag = 1; continue; }
-                    G1Affine p = ld_affine(table, ((size_t)w * K + (mag - 1)) * N + col);
-                    madd(acc, p, neg);
+                    madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
                 }
             }
             if (carry) *err_flag = 1;               // cannot happen for canonical 255-bit scalars when nw*c >= 256
@@ -258,14 +308,13 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 const uint32_t mag = (uint32_t)(neg ? -d : d);
                 if (mag != 0) {
                     if (mag > K) { *err_flag = 1; continue; }
-                    G1Affine p = ld_affine(table, ((size_t)w * K + (mag - 1)) * N + col);
-                    madd(acc, p, neg);
+                    madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
                 }
             }
             if (v != 0) *err_flag = 1;              // scalar does not fit nw windows
         }
     }
-    st_xyzz(partial, wave * 64 + lane, acc);
+    st_xyzz(partial, wave * 64 + lane, xyzz28_to_canonical(acc));
 }
 
 // Row epilogue: 8 lanes per row, each sums nparts/8 partials serially, then a 3-step tree over
@@ -424,7 +473,7 @@ int grape_g1_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t
     return GRAPE_OK;
 }
 
-size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K) { return (size_t)nw * K * N * 96; }
+size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K) { return (size_t)nw * K * N * 4 * kWideEntryWords; }
 
 int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     CHECK_PTR16(table); CHECK_PTR16(gens);

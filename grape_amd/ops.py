@@ -272,8 +272,23 @@ def g1_table_gen(gens, W):
 def g1_wide_table_gen(gens, c, nw, K):
     lib = init()
     n = gens.shape[0]
-    out = g1_empty(nw * K * n)
+    nbytes = lib.grape_g1_wide_table_bytes(n, nw, K)
+    out = torch.empty((nbytes // 128, 32), dtype=torch.int32, device="cuda")
     _capi.check(lib.grape_g1_wide_table_gen(_p(out), _p(gens), n, c, nw, K, _s()))
+    return out
+
+
+def wide_table_entries_to_host(table, idx):
+    """decode entries of a wide table into affine points (x, y) as Python integers
+    (None for the identity); for tests."""
+    P = 0x1a0111ea397fe69a4b1ba7b6434bacd764774b84f38512bf6730d2a0f6b0f6241eabfffeb153ffffb9feffffffffaaab
+    rinv = pow(1 << 392, -1, P)
+    rows = table[idx].cpu().numpy()
+    out = []
+    for r in rows:
+        x = sum(int(r[i]) << (28 * i) for i in range(14))
+        y = sum(int(r[14 + i]) << (28 * i) for i in range(14))
+        out.append(None if (x == 0 and y == 0) else (x * rinv % P, y * rinv % P))
     return out
 
 

@@ -161,9 +161,12 @@ int grape_g1_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, 
 /*
  * Wide fixed-base table for the commitment kernels:
  *   table[(w*K + (k-1))*N + i] = k * 2^(c*w) * G_i,  k = 1..K, w < nw
- * (affine).  With c = 16, nw = 1, K = 32768 a signed 16-bit scalar is ONE mixed addition;
- * with c = 8, nw = 32, K = 128 a 255-bit scalar is 32 signed-digit additions into a single
- * accumulator.  Size: nw*K*N*96 bytes.
+ * With c = 16, nw = 1, K = 32768 a signed 16-bit scalar is ONE mixed addition; with c = 8,
+ * nw = 32, K = 128 a 255-bit scalar is 32 signed-digit additions into a single accumulator.
+ * The table is private to this library (only the commitment entry points read it): each entry
+ * is 128 bytes - the affine coordinates as 14 limbs of 28 bits each, Montgomery radix 2^392,
+ * the working form of the commitment kernels - so a gather is exactly one cache line.
+ * Size: grape_g1_wide_table_bytes(N, nw, K) = nw*K*N*128 bytes.
  */
 int grape_g1_wide_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, size_t N, uint32_t c, uint32_t nw,
                             uint32_t K, grape_stream_t stream);

@@ -1,0 +1,118 @@
+"""CPU checks of the 28-bit-limb lazy Fp arithmetic used by the commitment kernels (host build of
+grape_amd/csrc/fp28.hpp): products, squares, conversions and lazily reduced expressions against
+Python integers; sums of points through the 28-bit mixed addition against textbook affine
+arithmetic, including the exceptional cases (doubling, cancellation, identity)."""
+import ctypes
+import os
+import random
+import subprocess
+import numpy as np
+import pytest
+import bigref as br
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "native", "fp28_host.cpp")
+LIB = os.path.join(HERE, "native", "libfp28_host.so")
+P = br.P_MOD
+
+
+@pytest.fixture(scope="module")
+def lib():
+    deps = [SRC] + [os.path.join(HERE, "..", "grape_amd", "csrc", f) for f in ("fp28.hpp", "curve.hpp", "field.hpp")]
+    if not os.path.exists(LIB) or any(os.path.getmtime(d) > os.path.getmtime(LIB) for d in deps):
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas", "-o", LIB, SRC])
+    return ctypes.CDLL(LIB)
+
+
+def _p32(vals):
+    """canonical values -> (n, 12) uint32 Montgomery (radix 2^384) limbs"""
+    return np.ascontiguousarray(br.fp_pack(vals).view(np.uint32).reshape(len(vals), 12))
+
+
+def _u32(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+
+
+def _val(a):
+    return br.fp_unpack(np.ascontiguousarray(a).view(np.uint64).reshape(1, 6))[0]
+
+
+EDGE = [0, 1, 2, P - 1, P - 2, (1 << 380), (1 << 381) % P, (1 << 28) - 1, 1 << 28, (1 << 364) - 1, P >> 1]
+
+
+def test_mul_sqr_roundtrip(lib):
+    rng = random.Random(1)
+    vals = EDGE + [rng.randrange(P) for _ in range(60)]
+    out = np.zeros(12, dtype=np.uint32)
+    for a in vals:
+        pa = _p32([a])[0]
+        lib.t28_roundtrip(_u32(pa), _u32(out))
+        assert _val(out) == a
+        lib.t28_sqr(_u32(pa), _u32(out))
+        assert _val(out) == a * a % P
+        for b in vals[:14] + vals[-4:]:
+            pb = _p32([b])[0]
+            lib.t28_mul(_u32(pa), _u32(pb), _u32(out))
+            assert _val(out) == a * b % P
+
+
+def test_lazy_expression(lib):
+    rng = random.Random(2)
+    out = np.zeros(12, dtype=np.uint32)
+    for _ in range(200):
+        a, b, c, d = (rng.choice(EDGE) if rng.random() < 0.3 else rng.randrange(P) for _ in range(4))
+        pa, pb, pc, pd = (_p32([x])[0] for x in (a, b, c, d))
+        lib.t28_lazy(_u32(pa), _u32(pb), _u32(pc), _u32(pd), _u32(out))
+        assert _val(out) == (a - b - 2 * c) * d % P
+
+
+def test_zero_detection(lib):
+    plain = lambda v: np.ascontiguousarray(br.ints_to_limbs([v], 6).view(np.uint32).reshape(12))
+    for k in (0, 1, 2):
+        assert lib.t28_is_zero(_u32(plain(0)), k) == 1
+        assert lib.t28_is_zero(_u32(plain(1)), k) == 0
+        assert lib.t28_is_zero(_u32(plain(P - 1)), k) == (1 if False else 0)
+
+
+def _points(ks):
+    return [br.g1_mul(k, br.G1) for k in ks]
+
+
+def _sum28(lib, pts, negs):
+    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 24))
+    neg = np.array(negs, dtype=np.int32)
+    xyzz = np.zeros(48, dtype=np.uint32)
+    slow = lib.t28_sum(_u32(arr), neg.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), len(pts), _u32(xyzz))
+    aff = np.zeros(24, dtype=np.uint32)
+    lib.t28_xyzz_to_affine(_u32(xyzz), _u32(aff))
+    return br.g1_unpack(aff.view(np.uint64).reshape(1, 12))[0], slow
+
+
+def test_point_sums_vs_textbook(lib):
+    rng = random.Random(3)
+    ks = [rng.randrange(1, br.R_MOD) for _ in range(40)]
+    pts = _points(ks)
+    negs = [rng.random() < 0.5 for _ in pts]
+    got, slow = _sum28(lib, pts, negs)
+    want = None
+    for p, n in zip(pts, negs):
+        want = br.g1_add(want, br.g1_neg(p) if n else p)
+    assert got == want and slow == 0
+
+
+def test_exceptional_cases_take_the_exact_path(lib):
+    a, b = br.g1_mul(5, br.G1), br.g1_mul(7, br.G1)
+    # doubling: a + a ; cancellation: a - a ; identity operands ; then keep adding
+    got, slow = _sum28(lib, [a, a, b], [False, False, False])
+    assert got == br.g1_add(br.g1_add(a, a), b) and slow == 1
+    got, slow = _sum28(lib, [a, a, b], [False, True, False])
+    assert got == b and slow == 1
+    got, slow = _sum28(lib, [None, a, None, b], [False] * 4)
+    assert got == br.g1_add(a, b) and slow == 0
+    got, slow = _sum28(lib, [a, a], [True, False])
+    assert got is None and slow == 1
+    got, slow = _sum28(lib, [], [])
+    assert got is None
+    # a long chain of the same point: 1,2,3,...: only the first addition doubles
+    got, slow = _sum28(lib, [a] * 9, [False] * 9)
+    assert got == br.g1_mul(45, br.G1) and slow == 1

@@ -55,10 +55,14 @@ def test_reference_table(ops, gens64):
 def test_wide_table_entries(ops, gens64):
     k, host, dev = gens64
     n, c, nw, K = 8, 8, 3, 128
-    tab = br.g1_unpack(ops.g1_to_host(ops.g1_wide_table_gen(dev[:n].contiguous(), c, nw, K)))
+    table = ops.g1_wide_table_gen(dev[:n].contiguous(), c, nw, K)
+    assert table.numel() * 4 == nw * K * n * 128
     pts = br.g1_unpack(host[:n])
-    for (w, kk, i) in [(0, 1, 0), (0, 128, 7), (1, 1, 3), (1, 77, 2), (2, 128, 5), (2, 2, 0), (0, 65, 1), (1, 64, 6)]:
-        assert tab[(w * K + (kk - 1)) * n + i] == br.g1_mul(kk << (c * w), pts[i])
+    cases = [(0, 1, 0), (0, 128, 7), (1, 1, 3), (1, 77, 2), (2, 128, 5), (2, 2, 0), (0, 65, 1), (1, 64, 6)]
+    idx = [(w * K + (kk - 1)) * n + i for (w, kk, i) in cases]
+    got = ops.wide_table_entries_to_host(table, idx)
+    for (w, kk, i), pt in zip(cases, got):
+        assert pt == br.g1_mul(kk << (c * w), pts[i])
 
 
 def test_commit_i32_small_vs_oracle_and_bigint(ops, gens64):
