@@ -248,6 +248,35 @@ GRAPE_HD Fp to_canonical(const Fp28& a) {
     return unpack(t);
 }
 
+// a^(p-2) in the 28-bit form (4-bit fixed windows, rolled loops); a in (-9p, 3p), a != 0 mod p.
+// Result normalised in (0, 3p).
+GRAPE_HD Fp28 inverse(const Fp28& a) {
+    Fp28 tbl[16];
+    tbl[0] = one();
+    tbl[1] = mul(normalize(a), one());      // bring into (0, 3p)
+    for (int i = 2; i < 16; i++) tbl[i] = mul(tbl[i - 1], tbl[1]);
+    Fp28 acc = one();
+    bool started = false;
+    for (int limb = 11; limb >= 0; limb--) {
+        uint32_t e = 0;
+        for (int k = 0; k < 12; k++) e = (k == limb) ? FpParams::pm2(k) : e;
+        for (int nib = 7; nib >= 0; nib--) {
+            if (started) {
+                acc = sqr(acc);
+                acc = sqr(acc);
+                acc = sqr(acc);
+                acc = sqr(acc);
+            }
+            uint32_t w = (e >> (4 * nib)) & 15u;
+            if (w) {
+                acc = mul(acc, tbl[w]);
+                started = true;
+            }
+        }
+    }
+    return acc;
+}
+
 }  // namespace fp28
 
 // ------------------------------------------------------------------------------------------------
@@ -326,6 +355,52 @@ GRAPE_HD bool xyzz28_madd(Xyzz28& acc, const Affine28& p, bool negate) {
     acc.x = X3;
     acc.y = Y3;
     return true;
+}
+
+// acc += q, both accumulators in the 28-bit form (12M + 2S).  Returns false, leaving acc
+// untouched, in the exceptional cases q = +-acc; identities are handled here.
+GRAPE_HD bool xyzz28_add(Xyzz28& acc, const Xyzz28& q) {
+    using namespace fp28;
+    if (q.inf) return true;
+    if (acc.inf) {
+        acc = q;
+        return true;
+    }
+    const Fp28 U1 = mul(acc.x, q.zz);                  // 9 * 3 = 27
+    const Fp28 U2 = mul(q.x, acc.zz);
+    const Fp28 S1 = mul(acc.y, q.zzz);                 // 3 * 3
+    const Fp28 S2 = mul(q.y, acc.zzz);
+    const Fp28 Pd = sub(U2, U1);                       // (-3p, 3p)
+    const Fp28 R = sub(S2, S1);                        // (-3p, 3p)
+    const Fp28 PP = sqr(Pd);                           // 9
+    const Fp28 ZZ3 = mul(mul(acc.zz, q.zz), PP);       // 9, 9
+    if (is_zero_mod_p(ZZ3)) return false;
+    const Fp28 PPP = mul(Pd, PP);                      // 9
+    const Fp28 Q = mul(U1, PP);                        // 9
+    const Fp28 RR = sqr(R);                            // 9
+    Fp28 X3;
+#pragma unroll
+    for (int i = 0; i < N; i++) X3.v[i] = RR.v[i] - PPP.v[i] - 2 * Q.v[i];   // (-9p, 3p)
+    X3 = normalize(X3);
+    const Fp28 T = sub(Q, X3);                         // (-3p, 12p)
+    const Fp28 Y3 = sub(mul(R, T), mul(S1, PPP));      // 36 ; 9
+    acc.zzz = mul(mul(acc.zzz, q.zzz), PPP);
+    acc.zz = ZZ3;
+    acc.x = X3;
+    acc.y = Y3;
+    return true;
+}
+
+// affine image in canonical 32-bit form; the identity maps to (0,0)
+GRAPE_HD G1Affine xyzz28_to_affine(const Xyzz28& a) {
+    using namespace fp28;
+    if (a.inf) return G1Affine::inf();
+    const Fp28 zzz_inv = inverse(a.zzz);
+    const Fp28 zinv = mul(zzz_inv, a.zz);             // 1/Z
+    G1Affine r;
+    r.x = to_canonical(mul(a.x, sqr(zinv)));
+    r.y = to_canonical(mul(a.y, zzz_inv));
+    return r;
 }
 
 }  // namespace grape

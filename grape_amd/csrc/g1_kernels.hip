@@ -103,6 +103,63 @@ __device__ __forceinline__ bool entry_is_inf(const Affine28& a) {
     for (int i = 0; i < 14; i++) z |= (uint32_t)a.x.v[i] | (uint32_t)a.y.v[i];
     return z == 0;
 }
+// Per-lane partial accumulator in memory: x, y, zz, zzz (14 words each), the identity flag and
+// padding = 64 words (256 bytes).
+constexpr int kPartialWords = 64;
+__device__ __forceinline__ void st_partial28(uint32_t* base, size_t i, const Xyzz28& a) {
+    uint32_t f[64];
+#pragma unroll
+    for (int k = 0; k < 14; k++) {
+        f[k] = (uint32_t)a.x.v[k];
+        f[14 + k] = (uint32_t)a.y.v[k];
+        f[28 + k] = (uint32_t)a.zz.v[k];
+        f[42 + k] = (uint32_t)a.zzz.v[k];
+    }
+    f[56] = a.inf ? 1u : 0u;
+#pragma unroll
+    for (int k = 57; k < 64; k++) f[k] = 0;
+    uint4* q = reinterpret_cast<uint4*>(base + (size_t)kPartialWords * i);
+#pragma unroll
+    for (int k = 0; k < 16; k++) q[k] = make_uint4(f[4 * k], f[4 * k + 1], f[4 * k + 2], f[4 * k + 3]);
+}
+__device__ __forceinline__ Xyzz28 ld_partial28(const uint32_t* base, size_t i) {
+    const uint4* q = reinterpret_cast<const uint4*>(base + (size_t)kPartialWords * i);
+    uint4 w[15];
+#pragma unroll
+    for (int k = 0; k < 15; k++) w[k] = q[k];
+    const uint32_t* f = reinterpret_cast<const uint32_t*>(w);
+    Xyzz28 a;
+#pragma unroll
+    for (int k = 0; k < 14; k++) {
+        a.x.v[k] = (int32_t)f[k];
+        a.y.v[k] = (int32_t)f[14 + k];
+        a.zz.v[k] = (int32_t)f[28 + k];
+        a.zzz.v[k] = (int32_t)f[42 + k];
+    }
+    a.inf = f[56] != 0;
+    return a;
+}
+__device__ __forceinline__ Xyzz28 shfl_down_xyzz28(const Xyzz28& a, int off) {
+    Xyzz28 r;
+#pragma unroll
+    for (int k = 0; k < 14; k++) {
+        r.x.v[k] = __shfl_down(a.x.v[k], off, 64);
+        r.y.v[k] = __shfl_down(a.y.v[k], off, 64);
+        r.zz.v[k] = __shfl_down(a.zz.v[k], off, 64);
+        r.zzz.v[k] = __shfl_down(a.zzz.v[k], off, 64);
+    }
+    r.inf = __shfl_down((int)a.inf, off, 64) != 0;
+    return r;
+}
+// acc += q for two 28-bit accumulators, exceptional cases through the canonical-form addition
+__device__ __forceinline__ void padd28(Xyzz28& acc, const Xyzz28& q) {
+    if (!xyzz28_add(acc, q)) {
+        G1Xyzz c = xyzz28_to_canonical(acc);
+        xyzz_add(c, xyzz28_to_canonical(q));
+        acc = xyzz28_from_canonical(c);
+    }
+}
+
 // acc += +-entry through the 28-bit mixed addition; the rare exceptional step (entry = +-acc)
 // goes through the exact canonical-form addition.
 __device__ __forceinline__ void madd28(Xyzz28& acc, const Affine28& e, bool negate) {
@@ -314,25 +371,33 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
             if (v != 0) *err_flag = 1;              // scalar does not fit nw windows
         }
     }
-    st_xyzz(partial, wave * 64 + lane, xyzz28_to_canonical(acc));
+    st_partial28(partial, wave * 64 + lane, acc);
 }
 
 // Row epilogue: 8 lanes per row, each sums nparts/8 partials serially, then a 3-step tree over
-// the 8 lanes; the leader converts to affine.
+// the 8 lanes; the leader maps the row sum to affine coordinates.  All in the 28-bit form.
 __global__ void __launch_bounds__(64) commit_reduce_kernel(uint32_t* out, const uint32_t* partial, size_t rows, uint32_t nparts) {
     const int lane = threadIdx.x & 63;
     const int sub = lane & 7;
     const size_t row = (size_t)blockIdx.x * 8 + (lane >> 3);
-    G1Xyzz acc = G1Xyzz::inf();
-    if (row < rows) {
-        for (uint32_t j = sub; j < nparts; j += 8) padd(acc, ld_xyzz(partial, row * nparts + j));
+    Xyzz28 acc = xyzz28_inf();
+    // one addition site serves both the serial part and the three tree steps (code size)
+    const uint32_t nserial = (nparts + 7) / 8;
+    for (uint32_t step = 0; step < nserial + 3; step++) {
+        Xyzz28 q;
+        bool doit;
+        if (step < nserial) {
+            const uint32_t j = sub + 8 * step;
+            doit = row < rows && j < nparts;
+            q = doit ? ld_partial28(partial, row * nparts + j) : xyzz28_inf();
+        } else {
+            const int off = 4 >> (step - nserial);
+            q = shfl_down_xyzz28(acc, off);
+            doit = sub + off < 8;
+        }
+        if (doit) padd28(acc, q);
     }
-#pragma unroll
-    for (int off = 4; off >= 1; off >>= 1) {
-        G1Xyzz o = shfl_down_xyzz(acc, off);
-        if (sub + off < 8) padd(acc, o);
-    }
-    if (row < rows && sub == 0) st_affine(out, row, to_affine(acc));
+    if (row < rows && sub == 0) st_affine(out, row, xyzz28_to_affine(acc));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -425,9 +490,9 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     const uint32_t seg = (rowlen + nseg - 1) / nseg;
     const size_t nwaves = rows * nseg;
     void* ws;
-    int rc = scratch_get(kSlotMsm, nwaves * 64 * 192 + 64, &ws);
+    int rc = scratch_get(kSlotMsm, nwaves * 64 * (size_t)(4 * kPartialWords) + 64, &ws);
     if (rc) return rc;
-    int* err = (int*)((char*)ws + nwaves * 64 * 192);
+    int* err = (int*)((char*)ws + nwaves * 64 * (size_t)(4 * kPartialWords));
     GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
     profile_begin();
     profile_mark(s);

@@ -66,6 +66,42 @@ int t28_sum(const uint32_t* points, const int* negate, int n, uint32_t* out_xyzz
     memcpy(out_xyzz, &r, 192);
     return slow;
 }
+// tree-style sum: partial sums of two halves combined with the accumulator+accumulator addition,
+// affine result through the 28-bit inversion
+int t28_sum_tree(const uint32_t* points, const int* negate, int n, uint32_t* out_affine) {
+    Xyzz28 part[2] = {xyzz28_inf(), xyzz28_inf()};
+    int slow = 0;
+    for (int i = 0; i < n; i++) {
+        G1Affine p;
+        memcpy(&p, points + 24 * i, 96);
+        if (p.is_inf()) continue;
+        Affine28 q;
+        q.x = fp28::from_canonical(p.x);
+        q.y = fp28::from_canonical(p.y);
+        Xyzz28& acc = part[i & 1];
+        if (!xyzz28_madd(acc, q, negate[i] != 0)) {
+            G1Xyzz c = xyzz28_to_canonical(acc);
+            xyzz_add_affine(c, p, negate[i] != 0);
+            acc = xyzz28_from_canonical(c);
+            slow++;
+        }
+    }
+    if (!xyzz28_add(part[0], part[1])) {
+        G1Xyzz c = xyzz28_to_canonical(part[0]);
+        xyzz_add(c, xyzz28_to_canonical(part[1]));
+        part[0] = xyzz28_from_canonical(c);
+        slow++;
+    }
+    G1Affine r = xyzz28_to_affine(part[0]);
+    memcpy(out_affine, &r, 96);
+    return slow;
+}
+void t28_inverse(const uint32_t* a, uint32_t* out) {
+    Fp x;
+    memcpy(&x, a, 48);
+    Fp r = fp28::to_canonical(fp28::inverse(fp28::from_canonical(x)));
+    memcpy(out, &r, 48);
+}
 void t28_xyzz_to_affine(const uint32_t* xyzz, uint32_t* out) {
     G1Xyzz a;
     memcpy(&a, xyzz, 192);

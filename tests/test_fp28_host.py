@@ -71,7 +71,7 @@ def test_zero_detection(lib):
     for k in (0, 1, 2):
         assert lib.t28_is_zero(_u32(plain(0)), k) == 1
         assert lib.t28_is_zero(_u32(plain(1)), k) == 0
-        assert lib.t28_is_zero(_u32(plain(P - 1)), k) == (1 if False else 0)
+        assert lib.t28_is_zero(_u32(plain(P - 1)), k) == 0
 
 
 def _points(ks):
@@ -116,3 +116,36 @@ def test_exceptional_cases_take_the_exact_path(lib):
     # a long chain of the same point: 1,2,3,...: only the first addition doubles
     got, slow = _sum28(lib, [a] * 9, [False] * 9)
     assert got == br.g1_mul(45, br.G1) and slow == 1
+
+
+def test_inverse(lib):
+    rng = random.Random(4)
+    out = np.zeros(12, dtype=np.uint32)
+    for a in [1, 2, P - 1, (1 << 380)] + [rng.randrange(1, P) for _ in range(10)]:
+        lib.t28_inverse(_u32(_p32([a])[0]), _u32(out))
+        assert _val(out) == pow(a, -1, P)
+
+
+def _sum_tree(lib, pts, negs):
+    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 24))
+    neg = np.array(negs, dtype=np.int32)
+    aff = np.zeros(24, dtype=np.uint32)
+    slow = lib.t28_sum_tree(_u32(arr), neg.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), len(pts), _u32(aff))
+    return br.g1_unpack(aff.view(np.uint64).reshape(1, 12))[0], slow
+
+
+def test_accumulator_plus_accumulator(lib):
+    rng = random.Random(5)
+    pts = _points([rng.randrange(1, br.R_MOD) for _ in range(21)])
+    negs = [rng.random() < 0.5 for _ in pts]
+    got, slow = _sum_tree(lib, pts, negs)
+    want = None
+    for p, n in zip(pts, negs):
+        want = br.g1_add(want, br.g1_neg(p) if n else p)
+    assert got == want and slow == 0
+    a, b = br.g1_mul(5, br.G1), br.g1_mul(7, br.G1)
+    # the two halves hold the same point / opposite points / one of them is the identity
+    assert _sum_tree(lib, [a, a], [False, False]) == (br.g1_add(a, a), 1)
+    assert _sum_tree(lib, [a, a], [False, True]) == (None, 1)
+    assert _sum_tree(lib, [a], [False]) == (a, 0)
+    assert _sum_tree(lib, [a, b, b, a], [False, False, True, True])[0] is None
