@@ -277,6 +277,181 @@ GRAPE_HD Fp28 inverse(const Fp28& a) {
     return acc;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Modular inversion by divsteps (Bernstein-Yang "safegcd"), batched 30 steps at a time on
+// signed 30-bit limbs.  About 800 divsteps for a 381-bit modulus, i.e. some 27 batches of a few
+// hundred instructions each - an order of magnitude fewer sequential instructions than the
+// a^(p-2) ladder, which matters because one inversion sits on the critical path of every row
+// epilogue.  The reference inverts with the same family of algorithm
+// (include/field/mont_t.cuh:1058-1120, ct_inverse_mod_x).
+// ------------------------------------------------------------------------------------------------
+namespace by {
+
+constexpr int L = 13;                       // 13 x 30 = 390 bits
+constexpr int32_t M30 = (1 << 30) - 1;
+constexpr uint32_t PINV30 = 0x00030003u;    // p^-1 mod 2^30
+
+GRAPE_HD int32_t P30(int i) {
+    constexpr int32_t t[13] = {0x3fffaaab, 0x27fbffff, 0x153ffffb, 0x2affffac, 0x30f6241e, 0x034a83da, 0x112bf673,
+                               0x12e13ce1, 0x2cd76477, 0x1ed90d2e, 0x29a4b1ba, 0x3a8e5ff9, 0x001a0111};
+    return t[i];
+}
+
+struct Mat { int32_t u, v, q, r; };
+
+// 30 divsteps on the low words; returns the transition matrix scaled by 2^30:
+//   u*f + v*g = 2^30 * f',   q*f + r*g = 2^30 * g'
+GRAPE_HD int32_t divsteps30(int32_t delta, uint32_t f, uint32_t g, Mat& t) {
+    int32_t u = 1, v = 0, q = 0, r = 1;
+    for (int i = 0; i < 30; i++) {
+        const bool swap = (delta > 0) & ((g & 1u) != 0);
+        // (f, g) <- (g, -f), rows of the matrix alike, delta <- -delta
+        const uint32_t nf = swap ? g : f;
+        const uint32_t ng = swap ? (0u - f) : g;
+        const int32_t nu = swap ? q : u, nv = swap ? r : v;
+        const int32_t nq = swap ? -u : q, nr = swap ? -v : r;
+        delta = swap ? -delta : delta;
+        f = nf; g = ng; u = nu; v = nv; q = nq; r = nr;
+        // make g even
+        const bool odd = (g & 1u) != 0;
+        g += odd ? f : 0u;
+        q += odd ? u : 0;
+        r += odd ? v : 0;
+        delta += 1;
+        g >>= 1;
+        u <<= 1;
+        v <<= 1;
+    }
+    t.u = u; t.v = v; t.q = q; t.r = r;
+    return delta;
+}
+
+// (f, g) <- t * (f, g) / 2^30, exact
+GRAPE_HD void update_fg(int32_t* f, int32_t* g, const Mat& t) {
+    int64_t cf = (int64_t)t.u * f[0] + (int64_t)t.v * g[0];
+    int64_t cg = (int64_t)t.q * f[0] + (int64_t)t.r * g[0];
+    cf >>= 30;   // the low 30 bits are zero by construction
+    cg >>= 30;
+#pragma unroll
+    for (int i = 1; i < L; i++) {
+        cf += (int64_t)t.u * f[i] + (int64_t)t.v * g[i];
+        cg += (int64_t)t.q * f[i] + (int64_t)t.r * g[i];
+        f[i - 1] = (int32_t)cf & M30;
+        g[i - 1] = (int32_t)cg & M30;
+        cf >>= 30;
+        cg >>= 30;
+    }
+    f[L - 1] = (int32_t)cf;
+    g[L - 1] = (int32_t)cg;
+}
+
+// (d, e) <- t * (d, e) / 2^30 mod p, keeping both in (-2p, p)
+GRAPE_HD void update_de(int32_t* d, int32_t* e, const Mat& t) {
+    const int32_t sd = d[L - 1] >> 31, se = e[L - 1] >> 31;   // all-ones when negative
+    // a negative d (e) is replaced by d + p (e + p): that adds u*p (v*p) to the first row
+    int32_t md = (t.u & sd) + (t.v & se);
+    int32_t me = (t.q & sd) + (t.r & se);
+    int64_t cd = (int64_t)t.u * d[0] + (int64_t)t.v * e[0];
+    int64_t ce = (int64_t)t.q * d[0] + (int64_t)t.r * e[0];
+    // choose the multiple of p that clears the low 30 bits
+    md -= (int32_t)((PINV30 * (uint32_t)cd + (uint32_t)md) & (uint32_t)M30);
+    me -= (int32_t)((PINV30 * (uint32_t)ce + (uint32_t)me) & (uint32_t)M30);
+    cd += (int64_t)P30(0) * md;
+    ce += (int64_t)P30(0) * me;
+    cd >>= 30;
+    ce >>= 30;
+#pragma unroll
+    for (int i = 1; i < L; i++) {
+        cd += (int64_t)t.u * d[i] + (int64_t)t.v * e[i] + (int64_t)P30(i) * md;
+        ce += (int64_t)t.q * d[i] + (int64_t)t.r * e[i] + (int64_t)P30(i) * me;
+        d[i - 1] = (int32_t)cd & M30;
+        e[i - 1] = (int32_t)ce & M30;
+        cd >>= 30;
+        ce >>= 30;
+    }
+    d[L - 1] = (int32_t)cd;
+    e[L - 1] = (int32_t)ce;
+}
+
+}  // namespace by
+
+// R'^3 mod p: turns the plain inverse of a Montgomery-form value back into Montgomery form
+GRAPE_HD int32_t R3(int i) {
+    constexpr int32_t t[14] = {0x1f7b890, 0x294cc4d, 0x9f3af22, 0xb5ba56c, 0xcb5c0cc, 0xc0d975c, 0xc89a8c5,
+                               0x6c968b4, 0x22672ea, 0x91de8c9, 0x35652a6, 0x84977c8, 0x424bbb9, 0x00141ab};
+    return t[i];
+}
+
+// 1/a in Montgomery form (radix 2^392) for a in (-9p, 3p), a != 0 mod p; result normalised in (0, 3p).
+GRAPE_HD Fp28 inverse_by(const Fp28& a) {
+    using namespace by;
+    // canonical integer of a (still carrying the Montgomery factor) in [0, p)
+    Fp28 t = mul(normalize(a), one());
+#pragma unroll
+    for (int rep = 0; rep < 2; rep++) {
+        Fp28 dd;
+#pragma unroll
+        for (int i = 0; i < N; i++) dd.v[i] = t.v[i] - P(i);
+        dd = normalize(dd);
+        const bool ok = dd.v[N - 1] >= 0;
+#pragma unroll
+        for (int i = 0; i < N; i++) t.v[i] = ok ? dd.v[i] : t.v[i];
+    }
+    // re-limb 14 x 28 -> 13 x 30
+    int32_t f[L], g[L], d[L], e[L];
+#pragma unroll
+    for (int k = 0; k < L; k++) {
+        const int bit = 30 * k, i0 = bit / W, sh = bit % W;
+        uint64_t w = (uint64_t)(uint32_t)t.v[i0] >> sh;
+        if (i0 + 1 < N) w |= (uint64_t)(uint32_t)t.v[i0 + 1] << (W - sh);
+        if (i0 + 2 < N && 2 * W - sh < 30) w |= (uint64_t)(uint32_t)t.v[i0 + 2] << (2 * W - sh);
+        g[k] = (int32_t)(w & (uint64_t)M30);
+        f[k] = P30(k);
+        d[k] = 0;
+        e[k] = 0;
+    }
+    e[0] = 1;
+    int32_t delta = 1;
+    // at most floor((49*384+57)/17) = 1110 divsteps are ever needed for 384-bit inputs
+    for (int batch = 0; batch < 37; batch++) {
+        uint32_t gz = 0;
+#pragma unroll
+        for (int k = 0; k < L; k++) gz |= (uint32_t)g[k];
+        if (gz == 0) break;
+        Mat m;
+        delta = divsteps30(delta, (uint32_t)f[0] | ((uint32_t)f[1] << 30), (uint32_t)g[0] | ((uint32_t)g[1] << 30), m);
+        update_de(d, e, m);
+        update_fg(f, g, m);
+    }
+    // now g = 0, f = +-1 and d * a = f (mod p): the inverse is d * f; bring it into [0, p)
+    const int32_t fneg = f[L - 1] >> 31;          // all-ones when f = -1
+    int64_t c = 0;
+    int32_t x[L];
+#pragma unroll
+    for (int k = 0; k < L; k++) x[k] = (d[k] ^ fneg) - fneg;   // limb-wise negation when f = -1
+    // x in (-2p, 2p): add 2p, then normalise (limbs to [0, 2^30), top signed but now positive)
+#pragma unroll
+    for (int k = 0; k < L - 1; k++) {
+        int64_t s = (int64_t)x[k] + 2 * (int64_t)P30(k) + c;
+        x[k] = (int32_t)s & M30;
+        c = s >> 30;
+    }
+    x[L - 1] = (int32_t)((int64_t)x[L - 1] + 2 * (int64_t)P30(L - 1) + c);
+    // re-limb 13 x 30 -> 14 x 28 (value in (0, 4p), below 2^384)
+    Fp28 r;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        const int bit = W * k, i0 = bit / 30, sh = bit % 30;
+        uint64_t w = (uint64_t)(uint32_t)x[i0] >> sh;
+        if (i0 + 1 < L) w |= (uint64_t)(uint32_t)x[i0 + 1] << (30 - sh);
+        r.v[k] = (int32_t)(w & (uint64_t)MASK);
+    }
+    Fp28 r3;
+#pragma unroll
+    for (int i = 0; i < N; i++) r3.v[i] = R3(i);
+    return mul(r, r3);   // 4 * 1 <= 2^11
+}
+
 }  // namespace fp28
 
 // ------------------------------------------------------------------------------------------------
@@ -395,7 +570,7 @@ GRAPE_HD bool xyzz28_add(Xyzz28& acc, const Xyzz28& q) {
 GRAPE_HD G1Affine xyzz28_to_affine(const Xyzz28& a) {
     using namespace fp28;
     if (a.inf) return G1Affine::inf();
-    const Fp28 zzz_inv = inverse(a.zzz);
+    const Fp28 zzz_inv = inverse_by(a.zzz);
     const Fp28 zinv = mul(zzz_inv, a.zz);             // 1/Z
     G1Affine r;
     r.x = to_canonical(mul(a.x, sqr(zinv)));

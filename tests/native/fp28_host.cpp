@@ -102,6 +102,12 @@ void t28_inverse(const uint32_t* a, uint32_t* out) {
     Fp r = fp28::to_canonical(fp28::inverse(fp28::from_canonical(x)));
     memcpy(out, &r, 48);
 }
+void t28_inverse_by(const uint32_t* a, uint32_t* out) {
+    Fp x;
+    memcpy(&x, a, 48);
+    Fp r = fp28::to_canonical(fp28::inverse_by(fp28::from_canonical(x)));
+    memcpy(out, &r, 48);
+}
 void t28_xyzz_to_affine(const uint32_t* xyzz, uint32_t* out) {
     G1Xyzz a;
     memcpy(&a, xyzz, 192);

@@ -126,6 +126,16 @@ def test_inverse(lib):
         assert _val(out) == pow(a, -1, P)
 
 
+def test_inverse_by_divsteps(lib):
+    rng = random.Random(6)
+    out = np.zeros(12, dtype=np.uint32)
+    vals = [1, 2, 3, P - 1, P - 2, (1 << 380), (1 << 381) % P, (P + 1) // 2, 0xffffffff, 1 << 64]
+    vals += [rng.randrange(1, P) for _ in range(300)]
+    for a in vals:
+        lib.t28_inverse_by(_u32(_p32([a])[0]), _u32(out))
+        assert _val(out) == pow(a, -1, P), hex(a)
+
+
 def _sum_tree(lib, pts, negs):
     arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 24))
     neg = np.array(negs, dtype=np.int32)
