@@ -9,6 +9,19 @@
 #include "tlookup.hpp"
 
 static thread_local std::string g_err;
+static double g_last_prove_s = 0;
+#include <chrono>
+struct ProveTimer {
+    std::chrono::steady_clock::time_point t0;
+    ProveTimer() {
+        grape_stream_sync(nullptr);
+        t0 = std::chrono::steady_clock::now();
+    }
+    ~ProveTimer() {
+        grape_stream_sync(nullptr);
+        g_last_prove_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    }
+};
 
 #define GUARD_BEGIN try {
 #define GUARD_END                      \
@@ -18,6 +31,24 @@ static thread_local std::string g_err;
         return 1;                      \
     }                                  \
     return 0;
+
+#include <map>
+#include <memory>
+#include <tuple>
+// Hyrax objects persist across calls (keyed by their table), so the wide fixed-base tables
+// they build are generated once per generator set, as in a long-running prover.
+static Hyrax& hyrax_for(const uint32_t* d_table, uint32_t npoints, uint32_t com_scale, uint32_t layer_num) {
+    typedef std::tuple<const uint32_t*, uint32_t, uint32_t, uint32_t> Key;
+    static std::map<Key, std::unique_ptr<Hyrax>> cache;
+    static bn128 G = bn128::one();
+    Key k(d_table, npoints, com_scale, layer_num);
+    auto it = cache.find(k);
+    if (it == cache.end()) {
+        if (cache.size() >= 4) cache.clear();   // bounded: drop old tables
+        it = cache.emplace(k, std::unique_ptr<Hyrax>(new Hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale))).first;
+    }
+    return *it->second;
+}
 
 static std::vector<Fr> vec_from(const uint32_t* p, uint32_t n) {
     std::vector<Fr> v(n);
@@ -48,6 +79,7 @@ static void put_transcript(const SumcheckTranscript& tr, uint32_t* out, uint32_t
 extern "C" {
 
 const char* grape_host_last_error(void) { return g_err.c_str(); }
+double grape_host_last_prove_seconds(void) { return g_last_prove_s; }
 void grape_host_seed(uint64_t seed) { Fr::seed(seed); }
 
 int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int N, int M, int K, const uint32_t* u, uint32_t nu,
@@ -58,7 +90,11 @@ int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int
     FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * K));
     Fr claim = fr_from(claim_inout);
     SumcheckTranscript tr;
-    auto res = prove_matmul(A, B, L, N, M, K, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    std::pair<Fr, Fr> res;
+    {
+        ProveTimer timer;
+        res = prove_matmul(A, B, L, N, M, K, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    }
     fr_to(claim_inout, claim);
     fr_to(A_claim, res.first);
     fr_to(B_claim, res.second);
@@ -105,8 +141,7 @@ int grape_host_mle_eval(const uint32_t* d_T, uint32_t size, const uint32_t* u, u
 int grape_host_hyrax_commit_i32(const int32_t* d_scalars, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
                                 uint32_t com_scale, uint32_t layer_num, uint32_t* out_affine) {
     GUARD_BEGIN
-    bn128 G = bn128::one();
-    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, layer_num);
     affine_t* c = hyrax.commit_affine(const_cast<int*>(d_scalars), size, N);
     uint32_t rows = size / (N * com_scale);
     grape_host::check(grape_memcpy_d2h(out_affine, c, sizeof(affine_t) * (size_t)rows, nullptr), "d2h");
@@ -117,8 +152,7 @@ int grape_host_hyrax_commit_i32(const int32_t* d_scalars, uint32_t size, uint32_
 int grape_host_hyrax_commit_fr(const uint32_t* d_scalars, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
                                uint32_t com_scale, uint32_t layer_num, uint32_t* out_affine) {
     GUARD_BEGIN
-    bn128 G = bn128::one();
-    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, layer_num);
     FrTensor t = tensor_from_device(d_scalars, size);
     // through the Jacobian-returning entry point, to cover the reference's return format
     jacob_t* cj = hyrax.commit(t, size, N);
@@ -136,8 +170,7 @@ int grape_host_hyrax_open_verify(const uint32_t* d_tensor, uint32_t size, uint32
                                  uint32_t com_scale, uint32_t layer_num, const uint32_t* eval_point, uint32_t n_eval,
                                  const uint32_t* c, uint32_t* result, int* verified) {
     GUARD_BEGIN
-    bn128 G = bn128::one();
-    Hyrax hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, layer_num);
     FrTensor t = tensor_from_device(d_tensor, size);
     jacob_t* com = hyrax.commit(t, size, N);
     std::vector<Fr> pt = vec_from(eval_point, n_eval);
@@ -153,8 +186,7 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
                                    uint32_t com_scale, uint32_t msm_size, uint32_t* m_out, uint32_t* transcript, uint32_t* n_rounds,
                                    uint32_t* S_claim, uint32_t* com_A_out, uint32_t* com_m_out, double* commit_seconds) {
     GUARD_BEGIN
-    bn128 G = bn128::one();
-    Hyrax hyrax(1, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
     tLookupRange lk(low, len);
     lk.alpha = fr_from(alpha);
     lk.set_u(vec_from(u, nuv));
@@ -162,7 +194,11 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
     FrTensor S = tensor_from_device(d_S, D, Dp);
     FrTensor A(Dp);
     double ct = 0;
-    Fr sc = lk.prove(S, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    Fr sc;
+    {
+        ProveTimer timer;
+        sc = lk.prove(S, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    }
     fr_to(S_claim, sc);
     put_transcript(lk.last_transcript, transcript, n_rounds);
     if (m_out) grape_host::check(grape_memcpy_d2h(m_out, lk.m.gpu_data, 32 * (size_t)lk.m.size, nullptr), "d2h");
@@ -177,8 +213,7 @@ int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S
                                      const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints, uint32_t com_scale,
                                      uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim) {
     GUARD_BEGIN
-    bn128 G = bn128::one();
-    Hyrax hyrax(1, npoints / com_scale, (affine_t*)d_table, G, com_scale);
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
     // r is drawn in the constructor; to pin it, seed-independent, rebuild the table with the given r
     struct Pinned : tLookupRangeMapping {
         Pinned(int low, uint len, const int* map, const Fr& r_) : tLookupRangeMapping(low, len, map) {

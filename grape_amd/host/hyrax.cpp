@@ -83,14 +83,30 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
     return out;
 }
 
+// Full-width scalars cost ceil(256/c) additions each, so the widest radix whose table fits the
+// budget is used: c = 13 is 20 additions per element against 32 for byte windows.
+bool Hyrax::ensure_fr_table(uint rowlen) {
+    if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
+    size_t used = 0;
+    if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
+    if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
+    for (uint c = 13; c >= 8; c--) {
+        uint nw = (256 + c - 1) / c, K = 1u << (c - 1);
+        if (used + grape_g1_wide_table_bytes(rowlen, nw, K) <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
+    }
+    return false;
+}
+
 affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;
     const uint rows = size / rowlen;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
-    if (ensure_table(fr_table_, rowlen, 8, 32, 128)) {
-        check(grape_commit_fr(W(out), W(tensor.gpu_data), size, rowlen, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    if (ensure_fr_table(rowlen)) {
+        check(grape_commit_fr(W(out), W(tensor.gpu_data), size, rowlen, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
+                              fr_table_.K, nullptr),
+              "grape_commit_fr");
     } else {
         check(grape_commit_fr_ref_table(W(out), W(tensor.gpu_data), size, rowlen, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
     }
@@ -131,8 +147,10 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185)
     affine_t* com_d_dev = nullptr;
     check(grape_malloc((void**)&com_d_dev, sizeof(affine_t)), "grape_malloc");
-    if (ensure_table(fr_table_, new_N, 8, 32, 128)) {
-        check(grape_commit_fr(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    if (ensure_fr_table(new_N)) {
+        check(grape_commit_fr(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
+                              fr_table_.K, nullptr),
+              "grape_commit_fr");
     } else {
         check(grape_commit_fr_ref_table(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
     }
@@ -181,8 +199,10 @@ bool Hyrax::verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr
     FrTensor z = FrTensor::from_host(zv);
     affine_t* com_z_dev = nullptr;
     check(grape_malloc((void**)&com_z_dev, sizeof(affine_t)), "grape_malloc");
-    if (ensure_table(fr_table_, new_N, 8, 32, 128)) {
-        check(grape_commit_fr(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, 8, 32, 128, nullptr), "grape_commit_fr");
+    if (ensure_fr_table(new_N)) {
+        check(grape_commit_fr(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
+                              fr_table_.K, nullptr),
+              "grape_commit_fr");
     } else {
         check(grape_commit_fr_ref_table(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
     }

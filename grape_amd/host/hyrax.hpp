@@ -46,7 +46,7 @@ public:
     // the reference's own verify is an empty stub (src/Hyrax.cu:307-310).
     bool verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
 
-    // Upper bound for the wide fixed-base tables this object may build (default 64 GiB).  When a
+    // Upper bound for the wide fixed-base tables this object may build (default 96 GiB of the 288 GB).  When a
     // table would not fit, commitments go through the reference-format table instead.
     void set_table_budget(size_t bytes) { table_budget_ = bytes; }
 
@@ -56,8 +56,9 @@ private:
         uint ngen = 0, c = 0, nw = 0, K = 0;
     };
     bool ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K);
+    bool ensure_fr_table(uint rowlen);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;
-    size_t table_budget_ = (size_t)64 << 30;
+    size_t table_budget_ = (size_t)96 << 30;
 };
