@@ -66,6 +66,7 @@ SIGNATURES = {
     "grape_g1_affine_to_jacobian": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_g1_jacobian_to_affine": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_bench_copy": [c_void_p, c_void_p, c_size_t, c_int, ctypes.POINTER(ctypes.c_float), c_void_p],
+    "grape_bench_copy_fr": [c_void_p, c_void_p, c_size_t, c_int, ctypes.POINTER(ctypes.c_float), c_void_p],
     "grape_bench_mad_u64_u32": [c_int, c_int, c_int, ctypes.POINTER(ctypes.c_double), c_void_p],
     "grape_profile_enable": [c_int],
     "grape_profile_last": [ctypes.POINTER(ctypes.c_float), c_int, ctypes.POINTER(c_int)],

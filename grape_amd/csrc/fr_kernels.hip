@@ -27,6 +27,13 @@ __global__ void __launch_bounds__(kBlock) ew_kernel(uint32_t* out, const uint32_
     st_fr(out, i, apply<OP>(ld_fr(a, i), ld_fr(b, i)));
 }
 
+// plain copy with the tensors' access pattern (one 32-byte element per lane, two 16-byte accesses)
+__global__ void __launch_bounds__(kBlock) copy_fr_kernel(uint32_t* out, const uint32_t* a, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, ld_fr(a, i));
+}
+
 template <int OP>
 __global__ void __launch_bounds__(kBlock) bcast_kernel(uint32_t* out, const uint32_t* a, const uint32_t* x, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -314,6 +321,27 @@ int grape_fr_sub(uint32_t* o, const uint32_t* a, const uint32_t* b, size_t n, gr
 int grape_fr_mul(uint32_t* o, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t s) { return launch_ew<OP_MUL>(o, a, b, n, s); }
 int grape_fr_bcast_add(uint32_t* o, const uint32_t* a, const uint32_t* x, size_t n, grape_stream_t s) { return launch_bcast<OP_ADD>(o, a, x, n, s); }
 int grape_fr_bcast_mul(uint32_t* o, const uint32_t* a, const uint32_t* x, size_t n, grape_stream_t s) { return launch_bcast<OP_MUL>(o, a, x, n, s); }
+
+int grape_bench_copy_fr(uint32_t* out, const uint32_t* in, size_t n, int iters, float* ms, grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(in);
+    GRAPE_REQUIRE(n > 0 && iters > 0 && ms != nullptr, "bad arguments");
+    hipStream_t s = as_stream(st);
+    hipEvent_t e0, e1;
+    GRAPE_HIP_CHECK(hipEventCreate(&e0));
+    GRAPE_HIP_CHECK(hipEventCreate(&e1));
+    copy_fr_kernel<<<blocks_for(n), kBlock, 0, s>>>(out, in, n);
+    GRAPE_HIP_CHECK(hipEventRecord(e0, s));
+    for (int i = 0; i < iters; i++) copy_fr_kernel<<<blocks_for(n), kBlock, 0, s>>>(out, in, n);
+    GRAPE_HIP_CHECK(hipEventRecord(e1, s));
+    GRAPE_HIP_CHECK(hipEventSynchronize(e1));
+    GRAPE_LAUNCH_CHECK();
+    float t;
+    GRAPE_HIP_CHECK(hipEventElapsedTime(&t, e0, e1));
+    *ms = t / iters;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return GRAPE_OK;
+}
 
 int grape_fr_from_i32(uint32_t* out, const int32_t* in, size_t n, grape_stream_t st) {
     if (n == 0) return GRAPE_OK;

@@ -349,6 +349,15 @@ def bench_copy(nbytes, iters=10):
     return ms.value
 
 
+def bench_copy_fr(n, iters=10):
+    lib = init()
+    src, dst = fr_empty(n), fr_empty(n)
+    src.zero_()
+    ms = ctypes.c_float(0)
+    _capi.check(lib.grape_bench_copy_fr(_p(dst), _p(src), n, iters, ctypes.byref(ms), _s()))
+    return ms.value
+
+
 def bench_mad(blocks=4096, inner=256, iters=5):
     lib = init()
     r = ctypes.c_double(0)

@@ -203,6 +203,9 @@ int grape_g1_jacobian_to_affine(uint32_t *d_out_affine, const uint32_t *d_in_jac
 /* Device-to-device copy of `bytes` with the library's own streaming kernel, `iters` times;
  * returns the average time per copy in milliseconds in *ms (HIP events on `stream`). */
 int grape_bench_copy(void *d_dst, const void *d_src, size_t bytes, int iters, float *ms, grape_stream_t stream);
+/* The same for an Fr tensor of n elements moved with the tensors' own access pattern (one 32-byte
+ * element per lane as two 16-byte accesses). */
+int grape_bench_copy_fr(uint32_t *d_out, const uint32_t *d_in, size_t n, int iters, float *ms, grape_stream_t stream);
 /* Dependency-free v_mad_u64_u32 throughput: every lane of `blocks` x 256 threads runs
  * `inner` x 64 multiply-adds; *mads_per_s receives lane-level 32x32 multiplies per second. */
 int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double *mads_per_s, grape_stream_t stream);
