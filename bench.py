@@ -79,17 +79,212 @@ def cpu_baseline(W, gens_dev, ops, budget_s=15.0):
             "sample": "first %d of %d rows (x %d columns) of the same matrix, %.1f s" % (rows, ROWS, COLS, dt)}, out
 
 
+def layer_workload(args):
+    """BASELINE.json configs[4]: one LLaMA-2-7B-shape decoder layer (d_model 4096, 32 heads of 128,
+    FFN 11008, seq_len 2048 by default) proved on one GPU with seeded synthetic int16 weights and
+    activations: Hyrax commitments of the 7 weight matrices, matmul sumchecks for Q/K/V/O/gate/up/
+    down and per-head QK^T / AV, range lookups on every rescaling remainder, mapping lookups for the
+    softmax exponential and SiLU.  Witnesses (exact integer products, quotients, remainders) are
+    produced with torch, as the reference produces its own with a Python model; all proving goes
+    through the C++ host classes.  One step = one whole layer; prints one JSON line."""
+    import torch
+    from grape_amd import ops, _host as host
+    from gpuutil import rand_fr
+    ops.init(0)
+    host.load()
+    host.lib_seed = host.load().grape_host_seed(12345)
+    T, D, H, HD, F = args.seq, 4096, 32, 128, 11008
+    SH = 16
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(777)
+
+    def gauss(*shape):
+        x = torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * SIGMA
+        return x.round().clamp_(-32768, 32767).to(torch.int32)
+
+    weights = {"q": gauss(D, D), "k": gauss(D, D), "v": gauss(D, D), "o": gauss(D, D),
+               "gate": gauss(F, D), "up": gauss(F, D), "down": gauss(D, F)}
+    gens = ops.g1_make_generators(seeded_scalars(4096, SEED_G))
+    table = ops.g1_table_gen(gens, 256)            # reference-format table handed to Hyrax
+    NPTS = 4096
+    fr_scale = ops.to_dev(np.ascontiguousarray(_fr_const(1 << SH)))
+    seed = [1000]
+
+    def chal(n):
+        seed[0] += 1
+        return rand_fr(n, seed[0])
+
+    def log2c(n):
+        return 0 if n <= 1 else (n - 1).bit_length()
+
+    times = {"commit_weights": 0.0, "matmul": 0.0, "lookup": 0.0, "lookup_commits": 0.0}
+    counts = {"matmul": 0, "lookup": 0}
+
+    def commit_weight(w):
+        flat = w.contiguous().view(-1)
+        n = flat.numel()
+        if w.shape[1] != 4096:                     # down: rows of 11008 padded to 16384
+            flat = ops.i32_pad(flat, w.shape[1], 16384, w.shape[0] * 16384)
+            n = flat.numel()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        host.hyrax_commit_i32(flat, n, 4096, table, NPTS, com_scale=1)
+        torch.cuda.synchronize()
+        times["commit_weights"] += time.perf_counter() - t0
+
+    def rescale(y):
+        """y exact int64 -> (quotient int32, remainder int32) with y = q*2^16 + r, r in [-2^15, 2^15)"""
+        q = (y + (1 << (SH - 1))) >> SH
+        r = y - (q << SH)
+        return q.to(torch.int32), r.to(torch.int32)
+
+    def range_lookup(r):
+        flat = r.contiguous().view(-1)
+        dS = ops.fr_from_i32(flat)
+        n = flat.numel()
+        res = host.tlookup_range_prove(dS, n, -(1 << 15), 1 << 16, chal(1), chal(log2c(n)), chal(log2c(n)), table, NPTS, 1, 4096)
+        times["lookup"] += host.last_prove_seconds()
+        times["lookup_commits"] += res["commit_s"]
+        counts["lookup"] += 1
+
+    def mapping_lookup(x_in, x_out, low, length, fmap):
+        a, b = x_in.contiguous().view(-1), x_out.contiguous().view(-1)
+        n = a.numel()
+        host.tlookup_mapping_prove(ops.fr_from_i32(a), ops.fr_from_i32(b), n, low, length, fmap, chal(1), chal(1),
+                                   chal(log2c(n)), chal(log2c(n)), table, NPTS, 1, 4096)
+        times["lookup"] += host.last_prove_seconds()
+        counts["lookup"] += 1
+
+    def matmul_proof(a_int, b_int, L, N, M, K, q, r):
+        """sumcheck for Y[l][n][m] = sum_k A[l][n][k] B[l][m][k] with claim Y(u), Y = q*2^16 + r"""
+        dA = ops.fr_from_i32(a_int.contiguous().view(-1))
+        dB = ops.fr_from_i32(b_int.contiguous().view(-1))
+        Y = ops.fr_add(ops.fr_bcast_mul(ops.fr_from_i32(q.contiguous().view(-1)), fr_scale), ops.fr_from_i32(r.contiguous().view(-1)))
+        if M != 1 << log2c(M):                     # zero-extend the m axis, as the fold does
+            Y = ops.fr_pad(Y, M, 1 << log2c(M), L * N * (1 << log2c(M)), ops.to_dev(np.zeros((1, 4), dtype=np.uint64)))
+        u = chal(log2c(L) + log2c(N) + log2c(M))
+        v = chal(log2c(K) + log2c(L))
+        claim = host.mle_eval(Y, Y.shape[0], u)
+        del Y
+        host.prove_matmul(dA, dB, L, N, M, K, u, v, claim)
+        times["matmul"] += host.last_prove_seconds()
+        counts["matmul"] += 1
+
+    def mm(a, b):      # exact: every product sum stays below 2^53
+        return torch.matmul(a.to(torch.float64), b.to(torch.float64).transpose(-1, -2)).to(torch.int64)
+
+    # synthetic tables for the two mapping lookups (the reference's own table files are not in its tree)
+    exp_low, exp_len = -(1 << 19), 1 << 20
+    xs = torch.arange(exp_len, dtype=torch.float64) + exp_low
+    exp_map = torch.round(4095.0 * torch.exp((xs - (exp_len // 2 - 1)) / float(1 << 16))).to(torch.int32).numpy()
+    silu_low, silu_len = -(1 << 18), 1 << 19
+    xs = (torch.arange(silu_len, dtype=torch.float64) + silu_low) / 1024.0
+    silu_map = torch.round(1024.0 * xs * torch.sigmoid(xs)).to(torch.int32).numpy()
+    d_exp_map, d_silu_map = torch.from_numpy(exp_map).cuda(), torch.from_numpy(silu_map).cuda()
+
+    def one_layer():
+        for k in times:
+            times[k] = 0.0
+        counts["matmul"] = counts["lookup"] = 0
+        x = gauss(T, D)
+        for w in weights.values():
+            commit_weight(w)
+        # attention projections
+        proj = {}
+        for name in ("q", "k", "v"):
+            y = mm(x, weights[name])
+            proj[name], rem = rescale(y)
+            matmul_proof(x, weights[name], 1, T, D, D, proj[name], rem)
+            range_lookup(rem)
+        qh = proj["q"].view(T, H, HD).permute(1, 0, 2).contiguous()
+        kh = proj["k"].view(T, H, HD).permute(1, 0, 2).contiguous()
+        vh = proj["v"].view(T, H, HD).permute(1, 2, 0).contiguous()       # [H][HD][T]
+        sc = mm(qh, kh)                                                    # [H][T][T]
+        sc_q, sc_r = rescale(sc)
+        del sc
+        matmul_proof(qh, kh, H, T, T, HD, sc_q, sc_r)
+        range_lookup(sc_r)
+        del sc_r
+        e_in = sc_q.clamp(exp_low, exp_low + exp_len - 1)
+        e_out = d_exp_map[(e_in - exp_low).long()]
+        mapping_lookup(e_in, e_out, exp_low, exp_len, exp_map)
+        del sc_q, e_in
+        av = mm(e_out, vh)                                                 # [H][T][HD]
+        av_q, av_r = rescale(av)
+        matmul_proof(e_out, vh, H, T, HD, T, av_q, av_r)
+        range_lookup(av_r)
+        del e_out
+        attn = av_q.permute(1, 0, 2).contiguous().view(T, D)
+        y = mm(attn, weights["o"])
+        o_q, o_r = rescale(y)
+        matmul_proof(attn, weights["o"], 1, T, D, D, o_q, o_r)
+        range_lookup(o_r)
+        # feed-forward
+        x2 = o_q
+        gq, gr = rescale(mm(x2, weights["gate"]))
+        matmul_proof(x2, weights["gate"], 1, T, F, D, gq, gr)
+        range_lookup(gr)
+        uq, ur = rescale(mm(x2, weights["up"]))
+        matmul_proof(x2, weights["up"], 1, T, F, D, uq, ur)
+        range_lookup(ur)
+        s_in = gq.clamp(silu_low, silu_low + silu_len - 1)
+        s_out = d_silu_map[(s_in - silu_low).long()]
+        mapping_lookup(s_in, s_out, silu_low, silu_len, silu_map)
+        hq, _ = rescale(s_out.to(torch.int64) * uq.to(torch.int64))
+        dq, dr = rescale(mm(hq, weights["down"]))
+        matmul_proof(hq, weights["down"], 1, T, D, F, dq, dr)
+        range_lookup(dr)
+        return times["commit_weights"] + times["matmul"] + times["lookup"]
+
+    for _ in range(args.warmup):
+        one_layer()
+    totals = []
+    for _ in range(args.steps):
+        totals.append(one_layer())
+    total = float(np.mean(totals))
+    weight_points = sum(int(w.numel()) for w in weights.values())
+    print(json.dumps({
+        "metric": "layer_prove_time", "value": total, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": total * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "configs[4]: LLaMA-2-7B-shape decoder layer proof, seq_len %d, d_model 4096, 32 heads x 128, "
+                               "FFN 11008, int16 weights/activations" % T,
+                   "breakdown_s": {k: float(v) for k, v in times.items()},
+                   "n_matmul_sumchecks": counts["matmul"], "n_lookups": counts["lookup"],
+                   "weight_points": weight_points,
+                   "note": "time inside the provers (commitments, sumchecks, lookups incl. their commitments of A and m); "
+                           "witness generation with torch is outside"}}))
+    return 0
+
+
+def _fr_const(x):
+    """Montgomery limbs of a small constant, as a (1, 4) uint64 array"""
+    r = 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001
+    v = (x << 256) % r
+    return np.array([[(v >> (64 * i)) & ((1 << 64) - 1) for i in range(4)]], dtype=np.uint64)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["commit", "layer"], default="commit",
+                    help="commit: configs[1], the metric's headline (default); layer: configs[4]")
+    ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
         return 2
+    if args.workload == "layer":
+        args.steps = 1 if args.steps is None else args.steps
+        args.warmup = 1 if args.warmup is None else args.warmup
+        return layer_workload(args)
+    args.steps = 20 if args.steps is None else args.steps
+    args.warmup = 3 if args.warmup is None else args.warmup
 
     import torch
     from grape_amd import ops

@@ -60,12 +60,31 @@ __global__ void __launch_bounds__(kBlock) sumcheck1_kernel(uint32_t* X, uint32_t
 // ---------------------------------------------------------------- tlookup
 __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    // (v - low) is a small non-negative integer for an in-range witness; leave Montgomery form
-    // and take the low limb, rejecting anything with higher limbs set.
-    Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
-    uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
-    if (hi == 0 && d.v[0] < len) atomicAdd(&hist[d.v[0]], 1u);
+    bool valid = false;
+    uint32_t idx = 0;
+    if (i < n) {
+        // (v - low) is a small non-negative integer for an in-range witness; leave Montgomery form
+        // and take the low limb, rejecting anything with higher limbs set.
+        Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
+        uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
+        valid = hi == 0 && d.v[0] < len;
+        idx = d.v[0];
+    }
+    // Wave-level aggregation: lanes holding the same bin are counted with one atomic.  Skewed
+    // witnesses (clipped activations, padding zeros) otherwise serialise on a few counters.
+    // Eight leaders are tried (enough to catch any bin that holds a sizeable share of the
+    // wave); whatever is left is taken to be spread out and issues plain atomics.
+    const int lane = threadIdx.x & 63;
+    unsigned long long todo = __ballot(valid);
+    for (int it = 0; it < 8 && todo != 0ull; it++) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const uint32_t lidx = __shfl(idx, leader, 64);
+        const unsigned long long same = __ballot(valid && idx == lidx) & todo;
+        const int cnt = __popcll(same);
+        if (lane == leader) atomicAdd(&hist[lidx], (uint32_t)cnt);
+        todo &= ~same;
+    }
+    if (valid && ((todo >> lane) & 1ull)) atomicAdd(&hist[idx], 1u);
 }
 
 __global__ void __launch_bounds__(kBlock) tl_table_kernel(uint32_t* T, const uint32_t* map, const uint32_t* r, int32_t low, uint32_t len) {
