@@ -46,6 +46,7 @@ SIGNATURES = {
     "grape_sumcheck_round2_coeffs": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round1": [c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p],
     "grape_tlookup_hist": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
+    "grape_tlookup_index": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
     "grape_tlookup_init": [c_void_p, c_void_p, c_i32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_tlookup_poly": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_poly_sum": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
@@ -59,6 +60,7 @@ SIGNATURES = {
     "grape_g1_table_gen": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p],
     "grape_g1_wide_table_gen": [c_void_p, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_g1_wide_table_bytes": [c_size_t, c_u32, c_u32],
+    "grape_g1_scaled_table_gen": [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_i32": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_fr": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_i32_ref_table": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_void_p],

@@ -174,6 +174,36 @@ __device__ __forceinline__ void madd28(Xyzz28& acc, const Affine28& e, bool nega
     }
 }
 
+// acc += k * G_col for a canonical (non-Montgomery) 255-bit scalar k: signed radix-2^c digits,
+// one gather and one mixed addition per non-zero digit.
+__device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k, const uint32_t* table, size_t N, uint32_t col,
+                                               uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
+    const uint32_t half = 1u << (c - 1), mask = (1u << c) - 1u;
+    uint32_t carry = 0;
+    for (uint32_t w = 0; w < nw; w++) {
+        const uint32_t bit = w * c;
+        if (bit >= 256) break;
+        // c <= 16 bits starting at `bit`, possibly straddling two limbs
+        const uint32_t limb = bit >> 5, sh = bit & 31;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            lo = (q == (int)limb) ? k.v[q] : lo;
+            hi = (q == (int)limb + 1) ? k.v[q] : hi;
+        }
+        uint64_t both = ((uint64_t)hi << 32) | lo;
+        uint32_t d = ((uint32_t)(both >> sh) & mask) + carry;
+        bool neg = d > half;                 // digit in (half, 2^c] -> d - 2^c, carry 1
+        carry = neg ? 1u : 0u;
+        uint32_t mag = neg ? (mask + 1u - d) : d;
+        if (mag != 0) {
+            if (mag > K) { *err_flag = 1; continue; }
+            madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
+        }
+    }
+    if (carry) *err_flag = 1;   // cannot happen for canonical 255-bit scalars when nw*c >= 256
+}
+
 __device__ __forceinline__ G1Xyzz shfl_down_xyzz(const G1Xyzz& a, int off) {
     G1Xyzz r;
 #pragma unroll
@@ -327,29 +357,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
     for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
         if (FR) {
             const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
-            uint32_t carry = 0;
-            for (uint32_t w = 0; w < nw; w++) {
-                const uint32_t bit = w * c;
-                if (bit >= 256) break;
-                // c <= 16 bits starting at `bit`, possibly straddling two limbs
-                const uint32_t limb = bit >> 5, sh = bit & 31;
-                uint32_t lo = 0, hi = 0;
-#pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    lo = (q == (int)limb) ? k.v[q] : lo;
-                    hi = (q == (int)limb + 1) ? k.v[q] : hi;
-                }
-                uint64_t both = ((uint64_t)hi << 32) | lo;
-                uint32_t d = ((uint32_t)(both >> sh) & mask) + carry;
-                bool neg = d > half;                 // digit in (half, 2^c] -> d - 2^c, carry 1
-                carry = neg ? 1u : 0u;
-                uint32_t mag = neg ? (mask + 1u - d) : d;
-                if (mag != 0) {
-                    if (mag > K) { *err_flag = 1; continue; }
-                    madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
-                }
-            }
-            if (carry) *err_flag = 1;               // cannot happen for canonical 255-bit scalars when nw*c >= 256
+            madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
         } else {
             int64_t v = ((const int32_t*)scalars)[row * rowlen + col];
             for (uint32_t w = 0; w < nw; w++) {
@@ -372,6 +380,52 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
         }
     }
     st_partial28(partial, wave * 64 + lane, acc);
+}
+
+// Scaled table: out[t*ncols + i] = s_t * G_i for a short list of scalars s_t (Montgomery Fr).
+// Stage 1 leaves XYZZ points (canonical form) in tmp[(t - t0)*ncols + i]; stage 2 normalises
+// 8 per thread and writes 128-byte working-form entries.
+__global__ void __launch_bounds__(kBlock) scaled_chain_kernel(uint32_t* tmp, const uint32_t* scalars, size_t t0, size_t nt,
+                                                              size_t ncols, const uint32_t* table, size_t N, uint32_t c,
+                                                              uint32_t nw, uint32_t K, int* err_flag) {
+    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (tid >= nt * ncols) return;
+    const size_t tt = tid / ncols;
+    const uint32_t col = (uint32_t)(tid - tt * ncols);
+    const Fr k = from_mont(ld_fr8(scalars, t0 + tt));
+    Xyzz28 acc = xyzz28_inf();
+    madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
+    st_xyzz(tmp, tid, xyzz28_to_canonical(acc));
+}
+__global__ void __launch_bounds__(64) scaled_normalize_kernel(uint32_t* out, const uint32_t* tmp, size_t e0, size_t n_entries) {
+    size_t t0 = (size_t)blockIdx.x * 64 + threadIdx.x;
+    size_t nthreads = (n_entries + kNormChunk - 1) / kNormChunk;
+    if (t0 >= nthreads) return;
+    Fp pre[kNormChunk];
+    Fp acc = Fp::one();
+#pragma unroll
+    for (int k = 0; k < kNormChunk; k++) {
+        size_t e = t0 + (size_t)k * nthreads;
+        pre[k] = acc;
+        if (e < n_entries) {
+            Fp zzz = ld_fp(tmp + 48 * e + 36);
+            if (!zzz.is_zero()) acc = fmul(acc, zzz);
+        }
+    }
+    Fp inv = fp_inverse(acc);
+#pragma unroll
+    for (int k = kNormChunk - 1; k >= 0; k--) {
+        size_t e = t0 + (size_t)k * nthreads;
+        if (e >= n_entries) continue;
+        G1Xyzz p = ld_xyzz(tmp, e);
+        G1Affine a = G1Affine::inf();
+        if (!p.zzz.is_zero()) {
+            Fp zi = fmul(inv, pre[k]);
+            inv = fmul(inv, p.zzz);
+            a = xyzz_to_affine_with_inv(p, zi);
+        }
+        st_entry28(out, e0 + e, a);
+    }
 }
 
 // Row epilogue: 8 lanes per row, each sums nparts/8 partials serially, then a 3-step tree over
@@ -479,7 +533,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
-    GRAPE_REQUIRE(c >= 2 && c <= 16 && nw >= 1 && K >= (1u << (c - 1)), "need 2 <= c <= 16 and K >= 2^(c-1)");
+    GRAPE_REQUIRE(c >= 2 && c <= (FR ? 16u : 24u) && nw >= 1 && K >= (1u << (c - 1)), "need 2 <= c <= 16 (24 for int32) and K >= 2^(c-1)");
     if (FR) GRAPE_REQUIRE((uint64_t)nw * c >= 256, "Fr scalars need nw*c >= 256");
     const size_t rows = size / rowlen;
     if (rows == 0) return GRAPE_OK;
@@ -572,6 +626,39 @@ int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uin
         size_t nthr2 = (n_entries + kNormChunk - 1) / kNormChunk;
         wide_normalize_kernel<<<blocks_for(nthr2, 64), 64, 0, s>>>(table, tmp, N, nw, K, CH, j0, n_entries);
         GRAPE_LAUNCH_CHECK();
+    }
+    return GRAPE_OK;
+}
+
+int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len, size_t ncols, const uint32_t* table, size_t N,
+                              uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(len >= 1 && ncols >= 1 && ncols <= N, "bad shape");
+    GRAPE_REQUIRE(c >= 2 && c <= 16 && (uint64_t)nw * c >= 256 && K >= (1u << (c - 1)), "need a full-width wide table");
+    hipStream_t s = as_stream(st);
+    // slabs of scalars so that the XYZZ staging buffer stays near 1.5 GiB
+    size_t slab = ((size_t)3 << 29) / (ncols * 192);
+    if (slab < 1) slab = 1;
+    if (slab > len) slab = len;
+    void* ws;
+    int rc = scratch_get(kSlotMsm, slab * ncols * 192 + 64, &ws);
+    if (rc) return rc;
+    int* err = (int*)((char*)ws + slab * ncols * 192);
+    GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
+    for (size_t t0 = 0; t0 < len; t0 += slab) {
+        size_t nt = len - t0 < slab ? len - t0 : slab;
+        size_t n_entries = nt * ncols;
+        scaled_chain_kernel<<<blocks_for(n_entries), kBlock, 0, s>>>((uint32_t*)ws, scalars, t0, nt, ncols, table, N, c, nw, K, err);
+        size_t nthr = (n_entries + kNormChunk - 1) / kNormChunk;
+        scaled_normalize_kernel<<<blocks_for(nthr, 64), 64, 0, s>>>(out, (const uint32_t*)ws, t0 * ncols, n_entries);
+        GRAPE_LAUNCH_CHECK();
+    }
+    int h_err = 0;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(&h_err, err, sizeof(int), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    if (h_err) {
+        set_error("scaled table: a scalar digit exceeds the wide table's range");
+        return GRAPE_EINVAL;
     }
     return GRAPE_OK;
 }

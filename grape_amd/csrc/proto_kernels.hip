@@ -87,6 +87,15 @@ __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint
     if (valid && ((todo >> lane) & 1ull)) atomicAdd(&hist[idx], 1u);
 }
 
+// out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
+__global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
+    uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
+    out[i] = (hi == 0 && d.v[0] < len) ? (int32_t)(d.v[0] + 1) : 0;
+}
+
 __global__ void __launch_bounds__(kBlock) tl_table_kernel(uint32_t* T, const uint32_t* map, const uint32_t* r, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= len) return;
@@ -257,6 +266,15 @@ int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t l
     GRAPE_REQUIRE(hist != nullptr && len > 0, "bad histogram buffer");
     CHECK_PTR16(vals);
     hist_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(hist, vals, n, low, len);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_index(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(out != nullptr && len > 0, "bad arguments");
+    CHECK_PTR16(vals);
+    index_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, vals, n, low, len);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

@@ -10,6 +10,7 @@
 
 static thread_local std::string g_err;
 static double g_last_prove_s = 0;
+static bool g_indexed_commit = true;
 #include <chrono>
 struct ProveTimer {
     std::chrono::steady_clock::time_point t0;
@@ -81,6 +82,7 @@ extern "C" {
 const char* grape_host_last_error(void) { return g_err.c_str(); }
 double grape_host_last_prove_seconds(void) { return g_last_prove_s; }
 void grape_host_seed(uint64_t seed) { Fr::seed(seed); }
+void grape_host_set_indexed_commit(int on) { g_indexed_commit = on != 0; }
 
 int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int N, int M, int K, const uint32_t* u, uint32_t nu,
                             const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
@@ -187,7 +189,17 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
                                    uint32_t* S_claim, uint32_t* com_A_out, uint32_t* com_m_out, double* commit_seconds) {
     GUARD_BEGIN
     Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
-    tLookupRange lk(low, len);
+    // lookup objects persist like Hyrax objects: their scaled table is built once
+    typedef std::tuple<int32_t, uint32_t, Hyrax*> LKey;
+    static std::map<LKey, std::unique_ptr<tLookupRange>> lcache;
+    LKey lkey(low, len, &hyrax);
+    auto lit = lcache.find(lkey);
+    if (lit == lcache.end()) {
+        if (lcache.size() >= 2) lcache.clear();
+        lit = lcache.emplace(lkey, std::unique_ptr<tLookupRange>(new tLookupRange(low, len))).first;
+    }
+    tLookupRange& lk = *lit->second;
+    lk.set_indexed_commit(g_indexed_commit);
     lk.alpha = fr_from(alpha);
     lk.set_u(vec_from(u, nuv));
     uint32_t Dp = 1u << Log2(D);

@@ -15,6 +15,9 @@ extern "C" {
 
 const char *grape_host_last_error(void);
 void grape_host_seed(uint64_t seed);
+/* tLookupRange objects made by the wrappers below commit A through the scaled table (1) or as a
+ * full-width tensor (0); default 1. */
+void grape_host_set_indexed_commit(int on);
 
 /* prove_matmul on copies of the device tensors d_A (L*N*K) and d_B (L*M*K).  transcript receives
  * 4 coefficients (8 u32 each) per round. */

@@ -113,6 +113,36 @@ affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
     return out;
 }
 
+affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
+    if (ncols > npoints) throw std::runtime_error("row longer than the generator set");
+    if (!ensure_fr_table(ncols)) return nullptr;
+    size_t bytes = (size_t)scalars.size * ncols * 128;
+    size_t used = scaled_bytes_ + grape_g1_wide_table_bytes(fr_table_.ngen, fr_table_.nw, fr_table_.K);
+    if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
+    if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
+    if (used + bytes > table_budget_) return nullptr;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, bytes), "grape_malloc");
+    check(grape_g1_scaled_table_gen(W(out), W(scalars.gpu_data), scalars.size, ncols, W(fr_table_.d), fr_table_.ngen, fr_table_.c,
+                                    fr_table_.nw, fr_table_.K, nullptr),
+          "grape_g1_scaled_table_gen");
+    scaled_bytes_ += bytes;
+    return out;
+}
+
+affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len) {
+    check_shape(size, N);
+    const uint rowlen = N * com_scale;
+    if (rowlen > ncols) throw std::runtime_error("row longer than the scaled table");
+    const uint rows = size / rowlen;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
+    // one unsigned "digit" idx+1 in [1, len]: radix 2^(log2(len)+1) keeps it below the sign threshold
+    const uint c = Log2(len) + 1;
+    check(grape_commit_i32(W(out), idx_plus1, size, rowlen, W(scaled_table), ncols, c, 1, len, nullptr), "grape_commit_i32 (indexed)");
+    return out;
+}
+
 static jacob_t* to_jacobian(affine_t* aff, uint rows) {
     jacob_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(jacob_t) * (size_t)rows), "grape_malloc");

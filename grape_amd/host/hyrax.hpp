@@ -46,6 +46,13 @@ public:
     // the reference's own verify is an empty stub (src/Hyrax.cu:307-310).
     bool verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
 
+    // Scaled table out[t*ncols + i] = scalars[t] * G_i over the first ncols generators (device,
+    // owned by the caller, freed with grape_free); nullptr when it would not fit the budget.
+    // With it, a tensor whose elements are scalars[idx] commits at one addition per element:
+    affine_t* build_scaled_table(const FrTensor& scalars, uint ncols);
+    // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
+    affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len);
+
     // Upper bound for the wide fixed-base tables this object may build (default 96 GiB of the 288 GB).  When a
     // table would not fit, commitments go through the reference-format table instead.
     void set_table_budget(size_t bytes) { table_budget_ = bytes; }
@@ -60,5 +67,6 @@ private:
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;
+    size_t scaled_bytes_ = 0;
     size_t table_budget_ = (size_t)96 << 30;
 };

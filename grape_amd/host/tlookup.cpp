@@ -13,6 +13,7 @@ tLookup::tLookup(const uint size) : alpha(Fr::random_element()), beta(Fr((long)s
 tLookup::~tLookup() {
     grape_free(com_A);
     grape_free(com_m);
+    grape_free(scaled_table_);
 }
 
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
@@ -34,6 +35,8 @@ static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
 
 // src/tlookup.cu:250-263
 tLookupRange::tLookupRange(int low_, uint len) : tLookup(1u << Log2(len)), low(low_) {
+    index_known_ = true;
+    index_low_ = low_;
     // the table always covers the whole power-of-two range T.size (the reference initialises
     // only the first len entries and leaves the rest unset)
     check(grape_tlookup_init(W(T.gpu_data), W(B.gpu_data), low, T.size, W(grape_host::device_scalar(beta)), nullptr, nullptr, nullptr),
@@ -67,7 +70,23 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         auto t0 = std::chrono::steady_clock::now();
         grape_free(com_A);
         grape_free(com_m);
-        com_A = hyrax.commit_affine(A, D, msm_size);
+        const uint rowlen = msm_size * hyrax.com_scale;
+        if (indexed_commit_ && index_known_ && (scaled_for_ != &hyrax || scaled_cols_ < rowlen)) {
+            grape_free(scaled_table_);
+            scaled_table_ = hyrax.build_scaled_table(B, rowlen);   // nullptr when over budget
+            scaled_cols_ = scaled_table_ ? rowlen : 0;
+            scaled_for_ = &hyrax;
+        }
+        if (indexed_commit_ && index_known_ && scaled_table_) {
+            int* d_idx = nullptr;
+            check(grape_malloc((void**)&d_idx, sizeof(int) * (size_t)D), "grape_malloc");
+            check(grape_tlookup_index(d_idx, W(S.gpu_data), D, index_low_, N, nullptr), "grape_tlookup_index");
+            com_A = hyrax.commit_indexed_affine(d_idx, D, msm_size, scaled_table_, scaled_cols_, N);
+            check(grape_stream_sync(nullptr), "sync");
+            grape_free(d_idx);
+        } else {
+            com_A = hyrax.commit_affine(A, D, msm_size);
+        }
         com_A_rows = D / (msm_size * hyrax.com_scale);
         uint m_N = 1u << (Log2(N) / 2);
         com_m = hyrax.commit_affine(m, N, m_N);

@@ -29,10 +29,21 @@ public:
     affine_t* com_m = nullptr;
     uint com_A_rows = 0, com_m_rows = 0;
     ~tLookup();
+    // The elements of A = 1/(S+beta) take only T.size distinct values B[t].  When enabled (the
+    // default) and the table fits the Hyrax object's budget, prove() commits A through a table of
+    // B[t]*G_i built once per object - one addition per element instead of one per scalar digit.
+    // The commitment is the same group element either way.
+    void set_indexed_commit(bool on) { indexed_commit_ = on; }
 
 protected:
     Fr run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
     std::vector<Fr> forced_u_;
+    bool indexed_commit_ = true;
+    bool index_known_ = false;          // set by tLookupRange: A's index is S - low
+    int index_low_ = 0;
+    affine_t* scaled_table_ = nullptr;  // B[t]*G_i, built on first use
+    uint scaled_cols_ = 0;
+    Hyrax* scaled_for_ = nullptr;
 };
 
 class tLookupRange : public tLookup {

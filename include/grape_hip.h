@@ -115,6 +115,11 @@ int grape_sumcheck_round1(uint32_t *d_X, uint32_t *d_a, uint32_t *d_b, uint32_t 
  * is NOT cleared here.  Values outside [low, low+len) are ignored.
  * get_histogram_kernel, src/tlookup.cu:5-14. */
 int grape_tlookup_hist(uint32_t *d_hist, const uint32_t *d_vals, size_t n, int32_t low, uint32_t len, grape_stream_t stream);
+/* out[i] = (v_i - low) + 1 as an int32 for n values (Montgomery Fr) inside [low, low+len), 0 for a
+ * value outside: the table index of each witness element, shifted by one (the index the
+ * reference derives inside get_histogram_kernel, src/tlookup.cu:9-12).  Feeds the indexed
+ * commitment of A = 1/(S+beta) below. */
+int grape_tlookup_index(int32_t *d_out, const uint32_t *d_vals, size_t n, int32_t low, uint32_t len, grape_stream_t stream);
 /* T[i] = low + i (+ r*map[i] when d_map != NULL), B[i] = 1/(T[i] + beta).
  * tlookuprange_init_kernel / tLookupRangeMapping_init_kernel, src/tlookup.cu:16-50. */
 int grape_tlookup_init(uint32_t *d_T, uint32_t *d_B, int32_t low, uint32_t len, const uint32_t *d_beta,
@@ -172,14 +177,25 @@ int grape_g1_wide_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_aff
                             uint32_t K, grape_stream_t stream);
 size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K);
 /*
+ * Scaled table out[t*ncols + i] = s_t * G_i for `len` scalars s_t (device, Montgomery Fr) and the
+ * first ncols generators, computed through a full-width wide table (c, nw, K as built above).
+ * Same 128-byte entry format, so grape_commit_i32(out, idx, size, rowlen, table = this, N = ncols,
+ * c = log2(len)+1, nw = 1, K = len) with idx = t+1 gives sum_i s_{t_i} * G_i at ONE addition per
+ * element.  Used for the logUp commitment of A = 1/(S+beta): its elements take only `len`
+ * distinct values B[t] (the reference commits A as a full-width tensor, src/tlookup.cu:320).
+ * No counterpart in the reference.  Size: len*ncols*128 bytes.
+ */
+int grape_g1_scaled_table_gen(uint32_t *d_out, const uint32_t *d_scalars_mont, size_t len, size_t ncols,
+                              const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/*
  * Row commitments of an integer matrix: for each of size/rowlen rows,
  * C_row = sum_i s[row*rowlen + i] * G_i, i < rowlen, written as AFFINE points (96 bytes each).
  * Hyrax::commit(int*, size, N), src/Hyrax.cu:312-333 (int_windows_sum :46-65, int_windows_reduce
  * :67-87); rowlen is the reference's N*com_scale.  The wide table must have been built for
  * N >= rowlen generators with radix 2^c, nw windows and K >= 2^(c-1); scalars are recoded into
- * signed radix-2^c digits, so any int32 is accepted when nw*c >= 33, and the int16 fast path
- * (c = 16, nw = 1) requires -32768 <= s <= 32767 (checked on device: returns GRAPE_EINVAL after
- * synchronising if violated).
+ * signed radix-2^c digits (2 <= c <= 24 here), so any int32 is accepted when nw*c >= 33, and the
+ * int16 fast path (c = 16, nw = 1) requires -32768 <= s <= 32767 (checked on device: returns
+ * GRAPE_EINVAL after synchronising if violated).
  */
 int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
                      const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
