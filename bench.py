@@ -154,6 +154,7 @@ def layer_workload(args):
         host.tlookup_mapping_prove(ops.fr_from_i32(a), ops.fr_from_i32(b), n, low, length, fmap, chal(1), chal(1),
                                    chal(log2c(n)), chal(log2c(n)), table, NPTS, 1, 4096)
         times["lookup"] += host.last_prove_seconds()
+        times["lookup_commits"] += host.last_commit_seconds()
         counts["lookup"] += 1
 
     def matmul_proof(a_int, b_int, L, N, M, K, q, r):

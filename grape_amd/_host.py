@@ -7,7 +7,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "host", "libgrape_host.so")
 _lib = None
 
-NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
+NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
          "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
          "grape_host_fr_op", "grape_host_g1_mul_generator"]
@@ -30,12 +30,17 @@ def load():
         lib.grape_host_last_error.restype = ctypes.c_char_p
         lib.grape_host_seed.argtypes = [ctypes.c_uint64]
         lib.grape_host_last_prove_seconds.restype = ctypes.c_double
+        lib.grape_host_last_commit_seconds.restype = ctypes.c_double
         _lib = lib
     return _lib
 
 
 def set_indexed_commit(on):
     load().grape_host_set_indexed_commit(1 if on else 0)
+
+
+def last_commit_seconds():
+    return load().grape_host_last_commit_seconds()
 
 
 def last_prove_seconds():

@@ -1,0 +1,250 @@
+// BLS12-381 Fr on 10 signed limbs of 26 bits with lazy accumulation - the working form of the
+// streaming Fr kernels (fold, sumcheck rounds, logUp rounds, element-wise products).
+//
+// Tensors stay in memory in the reference's format (8 x 32-bit limbs, canonical Montgomery
+// residue x*2^256 mod r, include/field/mont_t.cuh:33); a kernel re-limbs an element on load
+// (two instructions per limb) and multiplies in 26-bit limbs, where a limb product is < 2^52 and
+// a 64-bit column accumulator absorbs hundreds of them: a product costs 100 multiply-adds, a SUM
+// of products costs one Montgomery reduction in total, and differences are limb-wise.
+// On gfx950 a 32x32+64 multiply-add issues at full rate, so this turns the fold / round kernels
+// from instruction-bound (about 600 instructions per saturated 32-bit product) into HBM-bound.
+//
+// Radix bookkeeping.  The working Montgomery radix is 2^260, the memory radix 2^256:
+//   reduce(a*b) = a*b / 2^260.  With a = x*2^256 and b = y*2^256 (memory form) that is
+//   (x*y*2^256) / 16, so one operand carries an extra factor 16 (limbs times 16, or the constant
+//   X16 applied to a finished sum) and the result is again the memory form of x*y.
+#pragma once
+#include "field.hpp"
+
+namespace grape {
+namespace fr26 {
+
+constexpr int N = 10;
+constexpr int W = 26;
+constexpr uint32_t MASK = (1u << W) - 1;
+
+struct Limbs {
+    int32_t v[N];
+};
+struct Acc {            // columns of a double-width sum of limb products
+    int64_t c[2 * N];
+};
+
+GRAPE_HD int32_t R(int i) {   // the modulus r; R(0) = 1 and -r^-1 mod 2^26 = -1
+    constexpr int32_t t[10] = {0x0000001, 0x3ffffc0, 0x1bfefff, 0x00bfff9, 0x153bda4,
+                               0x2687601, 0x39d8080, 0x1f520cc, 0x353299d, 0x01cfb69};
+    return t[i];
+}
+GRAPE_HD int32_t X16(int i) {   // 16 * 2^260 mod r: reduce(t * X16) = 16 t
+    constexpr int32_t t[10] = {0x3fffdcb, 0x0008d3f, 0x3635000, 0x1840e7b, 0x22e7505,
+                               0x3738f0f, 0x163642b, 0x1fe9bc5, 0x175276a, 0x0091f6d};
+    return t[i];
+}
+GRAPE_HD int32_t C516(int i) {   // 2^516 mod r: reduce(x * C516) = x * 2^256 (into memory form)
+    constexpr int32_t t[10] = {0x329c6cf, 0x3a6440f, 0x263d999, 0x2d5e49d, 0x1631138,
+                               0x2e8703b, 0x37715f1, 0x1cf20a7, 0x246cc02, 0x00027fd};
+    return t[i];
+}
+
+// 8 x 32-bit canonical -> 10 x 26-bit, non-negative
+GRAPE_HD Limbs pack(const Fr& x) {
+    Limbs r;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        const int bit = W * k, q = bit >> 5, s = bit & 31;
+        uint64_t two = (uint64_t)x.v[q] | ((q + 1 < 8) ? ((uint64_t)x.v[q + 1] << 32) : 0);
+        r.v[k] = (int32_t)((uint32_t)(two >> s) & MASK);
+    }
+    return r;
+}
+// the same with every limb times 16 (the radix correction factor)
+GRAPE_HD Limbs pack16(const Fr& x) {
+    Limbs r = pack(x);
+#pragma unroll
+    for (int k = 0; k < N; k++) r.v[k] <<= 4;
+    return r;
+}
+// normalised non-negative limbs below 2^256 -> 8 x 32-bit
+GRAPE_HD Fr unpack(const Limbs& a) {
+    Fr r;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int k0 = (32 * q) / W;
+        uint64_t acc = 0;
+#pragma unroll
+        for (int t = 0; t < 3; t++) {
+            const int k = k0 + t;
+            if (k < N) {
+                const int sh = W * k - 32 * q;
+                if (sh >= 0) {
+                    if (sh < 32) acc |= (uint64_t)(uint32_t)a.v[k] << sh;
+                } else {
+                    acc |= (uint64_t)(uint32_t)a.v[k] >> (-sh);
+                }
+            }
+        }
+        r.v[q] = (uint32_t)acc;
+    }
+    return r;
+}
+
+GRAPE_HD Limbs sub(const Limbs& a, const Limbs& b) {
+    Limbs r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = a.v[i] - b.v[i];
+    return r;
+}
+GRAPE_HD Limbs add(const Limbs& a, const Limbs& b) {
+    Limbs r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = a.v[i] + b.v[i];
+    return r;
+}
+GRAPE_HD Limbs normalize(const Limbs& a) {
+    Limbs r;
+    int32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < N - 1; i++) {
+        int32_t t = a.v[i] + c;
+        r.v[i] = t & (int32_t)MASK;
+        c = t >> W;
+    }
+    r.v[N - 1] = a.v[N - 1] + c;
+    return r;
+}
+
+GRAPE_HD void acc_zero(Acc& C) {
+#pragma unroll
+    for (int k = 0; k < 2 * N; k++) C.c[k] = 0;
+}
+// C += a * b (100 multiply-adds).  The caller keeps |column| < 2^63: each call adds at most
+// 10 * max|a limb| * max|b limb| to a column.
+GRAPE_HD void mac(Acc& C, const Limbs& a, const Limbs& b) {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+#pragma unroll
+        for (int j = 0; j < N; j++) C.c[i + j] += (int64_t)a.v[i] * (int64_t)b.v[j];
+    }
+}
+// Montgomery reduction of a column sum V: returns (V + M*r)/2^260 + add_r*r with 0 <= M < 2^260,
+// limbs 0..8 normalised, top limb signed.  For |V| < B*r^2 the value lies in
+// (add_r - B/35.3)*r .. (add_r + 1 + B/35.3)*r   (r/2^260 = 2^-5.143 = 1/35.3).
+GRAPE_HD Limbs reduce(Acc& C, int add_r) {
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        const int32_t m = (int32_t)((0u - (uint32_t)C.c[i]) & MASK);   // -r^-1 = -1 mod 2^26
+        C.c[i] += (int64_t)m;                                          // m * R(0), R(0) = 1
+#pragma unroll
+        for (int j = 1; j < N; j++) C.c[i + j] += (int64_t)m * (int64_t)R(j);
+        C.c[i + 1] += C.c[i] >> W;
+    }
+    Limbs r;
+    int64_t c = 0;
+#pragma unroll
+    for (int k = 0; k < N - 1; k++) {
+        int64_t t = C.c[N + k] + (int64_t)add_r * (int64_t)R(k) + c;
+        r.v[k] = (int32_t)((uint32_t)t & MASK);
+        c = t >> W;
+    }
+    r.v[N - 1] = (int32_t)(C.c[2 * N - 1] + (int64_t)add_r * (int64_t)R(N - 1) + c);
+    return r;
+}
+// subtract r up to `times` times while the value stays non-negative: [0, (times+1) r) -> [0, r)
+GRAPE_HD Limbs canon(Limbs t, int times) {
+    for (int rep = 0; rep < times; rep++) {
+        Limbs d;
+#pragma unroll
+        for (int i = 0; i < N; i++) d.v[i] = t.v[i] - R(i);
+        d = normalize(d);
+        const bool ok = d.v[N - 1] >= 0;
+#pragma unroll
+        for (int i = 0; i < N; i++) t.v[i] = ok ? d.v[i] : t.v[i];
+    }
+    return t;
+}
+
+// canonical product of two memory-form elements (memory form out): 16ab < 16 r^2 -> (0, 1.46r)
+GRAPE_HD Fr mulc(const Fr& a, const Fr& b) {
+    Acc C;
+    acc_zero(C);
+    mac(C, pack16(a), pack(b));
+    return unpack(canon(reduce(C, 0), 1));
+}
+// a finished column sum of memory-form products (value/2^260 within (-lo_r, hi_r) multiples of
+// r, lo_r + hi_r + 1 <= 34) -> canonical memory form of the sum of products
+GRAPE_HD Fr finish_sum(Acc& C, int lo_r) {
+    Limbs t = reduce(C, lo_r);          // in (0, 34 r)
+    Limbs x;
+#pragma unroll
+    for (int i = 0; i < N; i++) x.v[i] = X16(i);
+    Acc D;
+    acc_zero(D);
+    mac(D, t, x);                        // < 34 r^2 -> (0, 1.97 r)
+    return unpack(canon(reduce(D, 0), 1));
+}
+// leave / enter memory (Montgomery) form
+GRAPE_HD Fr from_montc(const Fr& a) {    // x*2^256 -> x: reduce(16 * a) = a / 2^256
+    Acc C;
+    acc_zero(C);
+    const Limbs p = pack16(a);
+#pragma unroll
+    for (int i = 0; i < N; i++) C.c[i] = p.v[i];
+    return unpack(canon(reduce(C, 0), 1));
+}
+GRAPE_HD Fr to_montc(const Fr& a) {      // x -> x*2^256
+    Acc C;
+    acc_zero(C);
+    Limbs k;
+#pragma unroll
+    for (int i = 0; i < N; i++) k.v[i] = C516(i);
+    mac(C, pack(a), k);                  // < r^2 -> (0, 1.03 r)
+    return unpack(canon(reduce(C, 0), 1));
+}
+// small integer -> memory form; negatives as r - |x|
+GRAPE_HD Fr from_i32c(int32_t x) {
+    const uint32_t ax = x < 0 ? 0u - (uint32_t)x : (uint32_t)x;
+    Acc C;
+    acc_zero(C);
+    const int32_t l0 = (int32_t)(ax & MASK), l1 = (int32_t)(ax >> W);
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+        C.c[j] += (int64_t)l0 * (int64_t)C516(j);
+        C.c[j + 1] += (int64_t)l1 * (int64_t)C516(j);
+    }
+    Limbs t = canon(reduce(C, 0), 1);
+    // negate: r - t unless t = 0
+    uint32_t nz = 0;
+#pragma unroll
+    for (int i = 0; i < N; i++) nz |= (uint32_t)t.v[i];
+    if (x < 0 && nz != 0) {
+        Limbs d;
+#pragma unroll
+        for (int i = 0; i < N; i++) d.v[i] = R(i) - t.v[i];
+        t = normalize(d);
+    }
+    return unpack(t);
+}
+GRAPE_HD Fr from_u32c(uint32_t ax) {
+    Acc C;
+    acc_zero(C);
+    const int32_t l0 = (int32_t)(ax & MASK), l1 = (int32_t)(ax >> W);
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+        C.c[j] += (int64_t)l0 * (int64_t)C516(j);
+        C.c[j + 1] += (int64_t)l1 * (int64_t)C516(j);
+    }
+    return unpack(canon(reduce(C, 0), 1));
+}
+
+// 16 * w mod r as normalised limbs (below 2^26) for a canonical element w: four modular
+// doublings.  Use this (not pack16) for an operand that enters many accumulated products.
+GRAPE_HD Limbs weight16(const Fr& w) {
+    Fr t = grape::add(w, w);
+    t = grape::add(t, t);
+    t = grape::add(t, t);
+    t = grape::add(t, t);
+    return pack(t);
+}
+
+}  // namespace fr26
+}  // namespace grape

@@ -2,6 +2,7 @@
 // and wave64 / workgroup tree sums.
 #pragma once
 #include "common.hpp"
+#include "fr26.hpp"
 
 namespace grape {
 
@@ -17,6 +18,19 @@ __device__ __forceinline__ void st_fr(uint32_t* base, size_t i, const Fr& a) {
     uint4* p = reinterpret_cast<uint4*>(base) + 2 * i;
     p[0] = make_uint4(a.v[0], a.v[1], a.v[2], a.v[3]);
     p[1] = make_uint4(a.v[4], a.v[5], a.v[6], a.v[7]);
+}
+
+// element as 26-bit working limbs straight from memory
+__device__ __forceinline__ fr26::Limbs ld_l26(const uint32_t* base, size_t i) { return fr26::pack(ld_fr(base, i)); }
+
+// (1-v)*lo + v*hi in canonical memory form, with w0 = weight16(1-v), w1 = weight16(v):
+// the sum of two products is below 2 r^2, so one conditional subtraction finishes it.
+__device__ __forceinline__ Fr fold2(const fr26::Limbs& w0, const fr26::Limbs& w1, const fr26::Limbs& lo, const fr26::Limbs& hi) {
+    fr26::Acc F;
+    fr26::acc_zero(F);
+    fr26::mac(F, w0, lo);
+    fr26::mac(F, w1, hi);
+    return fr26::unpack(fr26::canon(fr26::reduce(F, 0), 1));
 }
 
 __device__ __forceinline__ Fr shfl_down_fr(const Fr& a, int off) {

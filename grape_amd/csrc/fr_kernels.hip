@@ -17,7 +17,7 @@ template <int OP>
 __device__ __forceinline__ Fr apply(const Fr& a, const Fr& b) {
     if (OP == OP_ADD) return add(a, b);
     if (OP == OP_SUB) return sub(a, b);
-    return mul(a, b);
+    return fr26::mulc(a, b);
 }
 
 template <int OP>
@@ -44,19 +44,19 @@ __global__ void __launch_bounds__(kBlock) bcast_kernel(uint32_t* out, const uint
 __global__ void __launch_bounds__(kBlock) from_i32_kernel(uint32_t* out, const int32_t* in, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    st_fr(out, i, fr_from_i32(in[i]));
+    st_fr(out, i, fr26::from_i32c(in[i]));
 }
 __global__ void __launch_bounds__(kBlock) from_u32_kernel(uint32_t* out, const uint32_t* in, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    st_fr(out, i, fr_from_u32(in[i]));
+    st_fr(out, i, fr26::from_u32c(in[i]));
 }
 template <bool TO>
 __global__ void __launch_bounds__(kBlock) mont_kernel(uint32_t* out, const uint32_t* in, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     Fr a = ld_fr(in, i);
-    st_fr(out, i, TO ? to_mont(a) : from_mont(a));
+    st_fr(out, i, TO ? fr26::to_montc(a) : fr26::from_montc(a));
 }
 
 __global__ void __launch_bounds__(kBlock) pad_fr_kernel(uint32_t* out, const uint32_t* in, uint32_t N, uint32_t pad_N,
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(kBlock) inv_prod_kernel(uint32_t* prod, const 
         if (i < n) {
             Fr x = ld_fr(in, i);
             if (beta) x = add(x, bt);
-            if (!x.is_zero()) acc = mul(acc, x);
+            if (!x.is_zero()) acc = fr26::mulc(acc, x);
         }
     }
     st_fr(prod, t, acc);
@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(kBlock) inv_back_kernel(uint32_t* out, const u
             if (beta) x[k] = add(x[k], bt);
         }
         pre[k] = acc;
-        if (!x[k].is_zero()) acc = mul(acc, x[k]);
+        if (!x[k].is_zero()) acc = fr26::mulc(acc, x[k]);
     }
     Fr inv = ld_fr(inv_prod, t);   // 1 / product of all non-zero x
 #pragma unroll
@@ -157,8 +157,8 @@ __global__ void __launch_bounds__(kBlock) inv_back_kernel(uint32_t* out, const u
             if (x[k].is_zero()) {
                 st_fr(out, i, Fr::zero());
             } else {
-                st_fr(out, i, mul(inv, pre[k]));
-                inv = mul(inv, x[k]);
+                st_fr(out, i, fr26::mulc(inv, pre[k]));
+                inv = fr26::mulc(inv, x[k]);
             }
         }
     }
@@ -182,7 +182,8 @@ constexpr int kFoldMaxBits = 6;
 
 __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* out, const uint32_t* in, const uint32_t* x_top,
                                                            uint32_t b, size_t outer, size_t c, size_t c_lo, size_t gap) {
-    __shared__ Fr w[1 << kFoldMaxBits];
+    // weights in the 26-bit working form, each carrying the radix factor 16 (reduced mod r)
+    __shared__ fr26::Limbs w[1 << kFoldMaxBits];
     const uint32_t nw = 1u << b;
     if (threadIdx.x < nw) {
         Fr acc = Fr::one();
@@ -190,7 +191,7 @@ __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* out, const 
             Fr xk = ld_fr(x_top, k);
             acc = mul(acc, ((threadIdx.x >> k) & 1) ? xk : sub(Fr::one(), xk));
         }
-        w[threadIdx.x] = acc;
+        w[threadIdx.x] = fr26::weight16(acc);
     }
     __syncthreads();
     const size_t c_out = c < c_lo ? c : c_lo;       // surviving extent of the axis
@@ -205,9 +206,12 @@ __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* out, const 
     const size_t hi_stride = c_lo * gap;            // elements between consecutive i_hi
     // number of i_hi with i_hi*c_lo + i_lo < c
     const size_t n_hi = (c - i_lo + c_lo - 1) / c_lo;
-    Fr acc = Fr::zero();
-    for (size_t h = 0; h < n_hi; h++) acc = add(acc, mul(ld_fr(src, h * hi_stride), w[h]));
-    st_fr(out, o * inner + p, acc);
+    // One double-width accumulator for the whole weighted sum: at most 64 products of values
+    // below r, so the column sums stay below 64 * 10 * 2^52 and the reduced value below 2.82 r.
+    fr26::Acc C;
+    fr26::acc_zero(C);
+    for (size_t h = 0; h < n_hi; h++) fr26::mac(C, w[h], ld_l26(src, h * hi_stride));
+    st_fr(out, o * inner + p, fr26::unpack(fr26::canon(fr26::reduce(C, 0), 2)));
 }
 
 // Small-tensor finish: one workgroup holds the whole [c][gap] slab of one outer index in LDS
@@ -231,13 +235,13 @@ __global__ void __launch_bounds__(kBlock) fold_small_kernel(uint32_t* out, const
                 const size_t j = i + nlow;
                 Fr lo = buf[i];
                 Fr hi = (j < cur * gap) ? buf[j] : Fr::zero();
-                buf[i] = add(lo, mul(xv, sub(hi, lo)));
+                buf[i] = add(lo, fr26::mulc(xv, sub(hi, lo)));
             }
             cur = half;
         } else {
             // the whole upper half is padding: value *= (1 - x)
             const Fr xv = sub(Fr::one(), ld_fr(x, lvl));
-            for (size_t i = threadIdx.x; i < cur * gap; i += kBlock) buf[i] = mul(buf[i], xv);
+            for (size_t i = threadIdx.x; i < cur * gap; i += kBlock) buf[i] = fr26::mulc(buf[i], xv);
         }
         __syncthreads();
     }

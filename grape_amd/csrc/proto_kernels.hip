@@ -10,33 +10,57 @@ __device__ __forceinline__ Fr ld_hi(const uint32_t* X, size_t g, size_t h, size_
     return (g + h < in_size) ? ld_fr(X, g + h) : Fr::zero();
 }
 
+// hi operand as working limbs (zero past the live extent)
+__device__ __forceinline__ fr26::Limbs ld_hi26(const uint32_t* X, size_t g, size_t h, size_t in_size) {
+    return fr26::pack(ld_hi(X, g, h, in_size));
+}
+
+// Iterations per thread of the round kernels: the three coefficient sums are kept as
+// double-width column accumulators across the grid-stride loop and reduced once per thread,
+// which bounds how many products a column may absorb (16 iterations x 2 products x 10 limb
+// products x 2^52 < 2^61).
+constexpr int kRoundIters = 16;
+
 template <bool COEFFS>
 __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
                                                            uint32_t in_size, uint32_t out_size, const uint32_t* v,
                                                            uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
     const Fr vv = ld_fr(v, 0);
-    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
+    fr26::Acc C0, C1, C2;
+    fr26::acc_zero(C0);
+    fr26::acc_zero(C1);
+    fr26::acc_zero(C2);
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < out_size; g += stride) {
-        const Fr Ab = ld_fr(A, g), Bb = ld_fr(B, g);
-        const Fr Aa = sub(ld_hi(A, g, out_size, in_size), Ab);
-        const Fr Ba = sub(ld_hi(B, g, out_size, in_size), Bb);
-        st_fr(A, g, add(mul(Aa, vv), Ab));
-        st_fr(B, g, add(mul(Ba, vv), Bb));
-        const Fr c0 = mul(Ab, Bb);
-        const Fr c1 = add(mul(Aa, Bb), mul(Ab, Ba));
-        const Fr c2 = mul(Aa, Ba);
+        const fr26::Limbs a0 = ld_l26(A, g), b0 = ld_l26(B, g);
+        const fr26::Limbs a1 = ld_hi26(A, g, out_size, in_size), b1 = ld_hi26(B, g, out_size, in_size);
+        st_fr(A, g, fold2(w0, w1, a0, a1));
+        st_fr(B, g, fold2(w0, w1, b0, b1));
+        const fr26::Limbs da = fr26::sub(a1, a0), db = fr26::sub(b1, b0);   // signed, |limb| < 2^26
         if (COEFFS) {
-            st_fr(cc, g, c0);
-            st_fr(cb, g, c1);
-            st_fr(ca, g, c2);
+            // materialised coefficient arrays (phase 1 folds them further)
+            fr26::Acc T;
+            fr26::acc_zero(T);
+            fr26::mac(T, a0, b0);
+            st_fr(cc, g, fr26::finish_sum(T, 0));
+            fr26::acc_zero(T);
+            fr26::mac(T, da, b0);
+            fr26::mac(T, a0, db);
+            st_fr(cb, g, fr26::finish_sum(T, 1));
+            fr26::acc_zero(T);
+            fr26::mac(T, da, db);
+            st_fr(ca, g, fr26::finish_sum(T, 1));
         }
-        acc[0] = add(acc[0], c0);
-        acc[1] = add(acc[1], c1);
-        acc[2] = add(acc[2], c2);
+        fr26::mac(C0, a0, b0);
+        fr26::mac(C1, da, b0);
+        fr26::mac(C1, a0, db);
+        fr26::mac(C2, da, db);
     }
     if (partial) {
+        // |sum| < 16 * 2 r^2 -> within (-0.91 r, 1.91 r) after reduction
+        Fr acc[3] = {fr26::finish_sum(C0, 2), fr26::finish_sum(C1, 2), fr26::finish_sum(C2, 2)};
         block_sum<3>(acc, lds);
         if (threadIdx.x == 0) {
             st_fr(partial, (size_t)blockIdx.x * 3 + 0, acc[0]);
@@ -50,11 +74,12 @@ __global__ void __launch_bounds__(kBlock) sumcheck1_kernel(uint32_t* X, uint32_t
                                                            uint32_t out_size, const uint32_t* v) {
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (g >= out_size) return;
+    const Fr vv = ld_fr(v, 0);
     const Fr Xb = ld_fr(X, g);
-    const Fr Xa = sub(ld_hi(X, g, out_size, in_size), Xb);
-    st_fr(X, g, add(mul(Xa, ld_fr(v, 0)), Xb));
+    const Fr Xh = ld_hi(X, g, out_size, in_size);
+    st_fr(X, g, fold2(fr26::weight16(sub(Fr::one(), vv)), fr26::weight16(vv), fr26::pack(Xb), fr26::pack(Xh)));
     st_fr(b, g, Xb);
-    st_fr(a, g, Xa);
+    st_fr(a, g, sub(Xh, Xb));
 }
 
 // ---------------------------------------------------------------- tlookup
@@ -65,7 +90,7 @@ __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint
     if (i < n) {
         // (v - low) is a small non-negative integer for an in-range witness; leave Montgomery form
         // and take the low limb, rejecting anything with higher limbs set.
-        Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
+        Fr d = fr26::from_montc(sub(ld_fr(vals, i), fr26::from_i32c(low)));
         uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
         valid = hi == 0 && d.v[0] < len;
         idx = d.v[0];
@@ -91,7 +116,7 @@ __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    Fr d = from_mont(sub(ld_fr(vals, i), fr_from_i32(low)));
+    Fr d = fr26::from_montc(sub(ld_fr(vals, i), fr26::from_i32c(low)));
     uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
     out[i] = (hi == 0 && d.v[0] < len) ? (int32_t)(d.v[0] + 1) : 0;
 }
@@ -99,8 +124,8 @@ __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint3
 __global__ void __launch_bounds__(kBlock) tl_table_kernel(uint32_t* T, const uint32_t* map, const uint32_t* r, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= len) return;
-    Fr t = add(fr_from_u32((uint32_t)i), fr_from_i32(low));
-    if (map) t = add(t, mul(ld_fr(map, i), ld_fr(r, 0)));
+    Fr t = add(fr26::from_u32c((uint32_t)i), fr26::from_i32c(low));
+    if (map) t = add(t, fr26::mulc(ld_fr(map, i), ld_fr(r, 0)));
     st_fr(T, i, t);
 }
 
@@ -113,9 +138,9 @@ __global__ void __launch_bounds__(kBlock) tl_poly_kernel(const uint32_t* A, cons
     const Fr s0 = ld_fr(S, t);
     const Fr c10 = beta ? add(s0, ld_fr(beta, 0)) : s0;
     const Fr c11 = sub(ld_fr(S, t + n_out), s0);
-    st_fr(o0, t, mul(c00, c10));
-    st_fr(o1, t, add(mul(c01, c10), mul(c00, c11)));
-    st_fr(o2, t, mul(c01, c11));
+    st_fr(o0, t, fr26::mulc(c00, c10));
+    st_fr(o1, t, add(fr26::mulc(c01, c10), fr26::mulc(c00, c11)));
+    st_fr(o2, t, fr26::mulc(c01, c11));
 }
 
 __global__ void __launch_bounds__(kBlock) tl_poly_sum_kernel(const uint32_t* A, uint32_t* o0, uint32_t* o1, size_t n_out) {
@@ -126,29 +151,43 @@ __global__ void __launch_bounds__(kBlock) tl_poly_sum_kernel(const uint32_t* A, 
     st_fr(o1, t, sub(ld_fr(A, t + n_out), a0));
 }
 
-// 5 sums per round: eq-weighted coefficients of (A0+tA1)(S0+beta+tS1), and plain sums of A0, A1
+// 5 sums per round: eq-weighted coefficients of (A0+tA1)(S0+beta+tS1), and plain sums of A0, A1.
+// e*A0 and e*A1 are reduced products; the three second-level products are accumulated
+// double-width over the thread's iterations and reduced once.
 __global__ void __launch_bounds__(kBlock) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
                                                           const uint32_t* eq, size_t n_out, uint32_t* partial) {
     __shared__ Fr lds[5 * (kBlock / 64)];
-    const Fr bt = beta ? ld_fr(beta, 0) : Fr::zero();
-    Fr acc[5];
-#pragma unroll
-    for (int k = 0; k < 5; k++) acc[k] = Fr::zero();
+    const Fr btc = beta ? ld_fr(beta, 0) : Fr::zero();
+    const fr26::Limbs bt = fr26::pack(btc);
+    fr26::Acc C0, C1, C2;
+    fr26::acc_zero(C0);
+    fr26::acc_zero(C1);
+    fr26::acc_zero(C2);
+    Fr sa0 = Fr::zero(), sa1 = Fr::zero();
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
-        const Fr a0 = ld_fr(A, t);
-        const Fr a1 = sub(ld_fr(A, t + n_out), a0);
-        const Fr s0r = ld_fr(S, t);
-        const Fr s0 = add(s0r, bt);
-        const Fr s1 = sub(ld_fr(S, t + n_out), s0r);
-        const Fr e = ld_fr(eq, t);
-        const Fr ea0 = mul(e, a0), ea1 = mul(e, a1);
-        acc[0] = add(acc[0], mul(ea0, s0));
-        acc[1] = add(acc[1], add(mul(ea1, s0), mul(ea0, s1)));
-        acc[2] = add(acc[2], mul(ea1, s1));
-        acc[3] = add(acc[3], a0);
-        acc[4] = add(acc[4], a1);
+        const Fr a0c = ld_fr(A, t), a1c = ld_fr(A, t + n_out);
+        const fr26::Limbs a0 = fr26::pack(a0c), a1 = fr26::pack(a1c);
+        const fr26::Limbs s0r = ld_l26(S, t);
+        const fr26::Limbs s0 = fr26::add(s0r, bt);                   // value < 2r, limbs < 2^27
+        const fr26::Limbs s1 = fr26::sub(ld_l26(S, t + n_out), s0r);   // signed
+        const fr26::Limbs e16 = fr26::pack16(ld_fr(eq, t));         // limbs < 2^30: one product per column set
+        fr26::Acc T;
+        fr26::acc_zero(T);
+        fr26::mac(T, e16, a0);
+        const fr26::Limbs ea0 = fr26::reduce(T, 0);                  // (0, 1.46 r)
+        fr26::acc_zero(T);
+        fr26::mac(T, e16, fr26::sub(a1, a0));
+        const fr26::Limbs ea1 = fr26::reduce(T, 1);                  // (0.54 r, 2.46 r)
+        fr26::mac(C0, ea0, s0);
+        fr26::mac(C1, ea1, s0);
+        fr26::mac(C1, ea0, s1);
+        fr26::mac(C2, ea1, s1);
+        sa0 = add(sa0, a0c);
+        sa1 = add(sa1, sub(a1c, a0c));
     }
+    // per iteration |C1| grows by at most (2.46*2 + 1.46) r^2; 16 iterations -> below 103 r^2 -> 2.9 r
+    Fr acc[5] = {fr26::finish_sum(C0, 4), fr26::finish_sum(C1, 4), fr26::finish_sum(C2, 4), sa0, sa1};
     block_sum<5>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
@@ -158,17 +197,20 @@ __global__ void __launch_bounds__(kBlock) tl_round_kernel(const uint32_t* A, con
 
 __global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
-    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    fr26::Acc C0, C1, C2;
+    fr26::acc_zero(C0);
+    fr26::acc_zero(C1);
+    fr26::acc_zero(C2);
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
-        const Fr m0 = ld_fr(m, t);
-        const Fr m1 = sub(ld_fr(m, t + n_out), m0);
-        const Fr b0 = ld_fr(B, t);
-        const Fr b1 = sub(ld_fr(B, t + n_out), b0);
-        acc[0] = add(acc[0], mul(m0, b0));
-        acc[1] = add(acc[1], add(mul(m1, b0), mul(m0, b1)));
-        acc[2] = add(acc[2], mul(m1, b1));
+        const fr26::Limbs m0 = ld_l26(m, t), b0 = ld_l26(B, t);
+        const fr26::Limbs m1 = fr26::sub(ld_l26(m, t + n_out), m0), b1 = fr26::sub(ld_l26(B, t + n_out), b0);
+        fr26::mac(C0, m0, b0);
+        fr26::mac(C1, m1, b0);
+        fr26::mac(C1, m0, b1);
+        fr26::mac(C2, m1, b1);
     }
+    Fr acc[3] = {fr26::finish_sum(C0, 2), fr26::finish_sum(C1, 2), fr26::finish_sum(C2, 2)};
     block_sum<3>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
@@ -183,7 +225,7 @@ __global__ void __launch_bounds__(kBlock) eq_level_kernel(uint32_t* e, const uin
     size_t half = (size_t)1 << j;
     if (i >= half) return;
     const Fr lo = ld_fr(e, i);
-    const Fr hi = mul(lo, ld_fr(u, j));
+    const Fr hi = fr26::mulc(lo, ld_fr(u, j));
     st_fr(e, i + half, hi);
     st_fr(e, i, sub(lo, hi));
 }
@@ -201,17 +243,21 @@ __global__ void __launch_bounds__(kBlock) fold_msb_multi_kernel(PtrPack pk, uint
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (g >= n_out) return;
     const Fr vv = ld_fr(v, 0);
+    const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
     for (uint32_t j = 0; j < k; j++) {
         uint32_t* X = pk.p[j];
-        const Fr lo = ld_fr(X, g);
-        st_fr(X, g, add(lo, mul(vv, sub(ld_fr(X, g + n_out), lo))));
+        st_fr(X, g, fold2(w0, w1, ld_l26(X, g), ld_l26(X, g + n_out)));
     }
 }
 
+// enough workgroups that no thread runs more than kRoundIters iterations, at most one element
+// per thread below that
 static unsigned reduce_grid(size_t n) {
     unsigned nb = blocks_for(n);
     unsigned cap = kNumCU * 8;
-    return nb > cap ? cap : nb;
+    if (nb <= cap) return nb;
+    unsigned need = blocks_for(n, kBlock * kRoundIters);
+    return need > cap ? need : cap;
 }
 
 }  // namespace grape

@@ -11,6 +11,7 @@
 static thread_local std::string g_err;
 static double g_last_prove_s = 0;
 static bool g_indexed_commit = true;
+static double g_last_commit_s = 0;
 #include <chrono>
 struct ProveTimer {
     std::chrono::steady_clock::time_point t0;
@@ -81,6 +82,7 @@ extern "C" {
 
 const char* grape_host_last_error(void) { return g_err.c_str(); }
 double grape_host_last_prove_seconds(void) { return g_last_prove_s; }
+double grape_host_last_commit_seconds(void) { return g_last_commit_s; }
 void grape_host_seed(uint64_t seed) { Fr::seed(seed); }
 void grape_host_set_indexed_commit(int on) { g_indexed_commit = on != 0; }
 
@@ -112,7 +114,11 @@ int grape_host_prove_elemul(const uint32_t* d_A, const uint32_t* d_B, int L, int
     FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * N));
     Fr claim = fr_from(claim_inout);
     SumcheckTranscript tr;
-    auto res = prove_eleMul(A, B, L, M, N, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    std::pair<Fr, Fr> res;
+    {
+        ProveTimer timer;
+        res = prove_eleMul(A, B, L, M, N, vec_from(u, nu), vec_from(v, nv), claim, &tr);
+    }
     fr_to(claim_inout, claim);
     fr_to(A_claim, res.first);
     fr_to(B_claim, res.second);
@@ -216,6 +222,7 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
     if (m_out) grape_host::check(grape_memcpy_d2h(m_out, lk.m.gpu_data, 32 * (size_t)lk.m.size, nullptr), "d2h");
     if (com_A_out) grape_host::check(grape_memcpy_d2h(com_A_out, lk.com_A, sizeof(affine_t) * (size_t)lk.com_A_rows, nullptr), "d2h");
     if (com_m_out) grape_host::check(grape_memcpy_d2h(com_m_out, lk.com_m, sizeof(affine_t) * (size_t)lk.com_m_rows, nullptr), "d2h");
+    g_last_commit_s = ct;
     if (commit_seconds) *commit_seconds = ct;
     GUARD_END
 }
@@ -243,7 +250,12 @@ int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S
     FrTensor S_out = tensor_from_device(d_S_out, D);
     FrTensor A(Dp);
     double ct = 0;
-    Fr sc = lk.prove(S_in, S_out, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    Fr sc;
+    {
+        ProveTimer timer;
+        sc = lk.prove(S_in, S_out, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    }
+    g_last_commit_s = ct;
     fr_to(S_claim, sc);
     put_transcript(lk.last_transcript, transcript, n_rounds);
     GUARD_END

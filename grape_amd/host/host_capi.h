@@ -27,6 +27,8 @@ int grape_host_prove_matmul(const uint32_t *d_A, const uint32_t *d_B, int L, int
 /* Seconds spent inside the most recent prove_matmul / tLookup prove proper (copies of the inputs
  * and allocations made by these wrappers excluded), device synchronised on both sides. */
 double grape_host_last_prove_seconds(void);
+/* Of which, for the lookup provers, seconds spent committing A and m. */
+double grape_host_last_commit_seconds(void);
 int grape_host_prove_elemul(const uint32_t *d_A, const uint32_t *d_B, int L, int M, int N, const uint32_t *u, uint32_t nu,
                             const uint32_t *v, uint32_t nv, uint32_t *claim_inout, uint32_t *transcript,
                             uint32_t *n_rounds, uint32_t *A_claim, uint32_t *B_claim);
