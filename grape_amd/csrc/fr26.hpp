@@ -162,6 +162,15 @@ GRAPE_HD Limbs canon(Limbs t, int times) {
     }
     return t;
 }
+// non-negative value below 32 r with limbs 0..8 normalised -> [0, r).  The quotient estimate
+// from the top limb (r = R(9) * 2^234 + ...) is the true quotient or one less.
+GRAPE_HD Limbs canon_wide(const Limbs& t) {
+    const int32_t q = t.v[N - 1] / (R(N - 1) + 1);
+    Limbs d;
+#pragma unroll
+    for (int i = 0; i < N; i++) d.v[i] = t.v[i] - q * R(i);
+    return canon(normalize(d), 1);
+}
 
 // canonical product of two memory-form elements (memory form out): 16ab < 16 r^2 -> (0, 1.46r)
 GRAPE_HD Fr mulc(const Fr& a, const Fr& b) {

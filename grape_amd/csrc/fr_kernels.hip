@@ -178,45 +178,125 @@ __global__ void __launch_bounds__(kBlock) inv_direct_kernel(uint32_t* out, const
 //   out[o][i_lo][g] = sum_{i_hi} w[i_hi] * t[o][i_hi*c_lo + i_lo][g],   i_hi*c_lo + i_lo < c
 // with w[i_hi] = prod_k eq(x[k], bit_k(i_hi)) over the b challenges of those bits.
 // ------------------------------------------------------------------------------------------------
-constexpr int kFoldMaxBits = 6;
+constexpr int kFoldMaxBits = 8;      // bits bound by one pass (at most 64 products per thread)
+constexpr int kFoldMaxPasses = 16;
 
-__global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* out, const uint32_t* in, const uint32_t* x_top,
-                                                           uint32_t b, size_t outer, size_t c, size_t c_lo, size_t gap) {
-    // weights in the 26-bit working form, each carrying the radix factor 16 (reduced mod r)
-    __shared__ fr26::Limbs w[1 << kFoldMaxBits];
-    const uint32_t nw = 1u << b;
-    if (threadIdx.x < nw) {
-        Fr acc = Fr::one();
-        for (uint32_t k = 0; k < b; k++) {
-            Fr xk = ld_fr(x_top, k);
-            acc = mul(acc, ((threadIdx.x >> k) & 1) ? xk : sub(Fr::one(), xk));
-        }
-        w[threadIdx.x] = fr26::weight16(acc);
+struct FoldPlan {
+    uint32_t npass;
+    uint32_t lo[kFoldMaxPasses];      // the pass binds challenges lo .. lo+b-1
+    uint32_t b[kFoldMaxPasses];
+    uint32_t off[kFoldMaxPasses];     // first weight of the pass in the weight buffer
+};
+
+// Weights of every pass of a fold, in the 26-bit working form with the radix factor 16 folded
+// in (reduced mod r): workgroup p writes w[i] = prod_k eq(x[lo+k], bit_k(i)) for i < 2^b.
+__global__ void __launch_bounds__(kBlock) fold_weights_kernel(int32_t* wts, const uint32_t* x, FoldPlan plan) {
+    const uint32_t p = blockIdx.x, b = plan.b[p];
+    if (threadIdx.x >= (1u << b)) return;
+    // all challenges first (one memory round trip), then a product tree of depth 3: the
+    // factors of one level are independent, which a single wave needs to issue at full rate
+    Fr f[kFoldMaxBits];
+#pragma unroll
+    for (uint32_t k = 0; k < (uint32_t)kFoldMaxBits; k++) f[k] = ld_fr(x, plan.lo[p] + (k < b ? k : 0));
+#pragma unroll
+    for (uint32_t k = 0; k < (uint32_t)kFoldMaxBits; k++)
+        f[k] = k < b ? (((threadIdx.x >> k) & 1) ? f[k] : sub(Fr::one(), f[k])) : Fr::one();
+#pragma unroll
+    for (int width = kFoldMaxBits / 2; width >= 1; width /= 2) {
+#pragma unroll
+        for (int k = 0; k < width; k++) f[k] = fr26::mulc(f[2 * k], f[2 * k + 1]);
     }
-    __syncthreads();
-    const size_t c_out = c < c_lo ? c : c_lo;       // surviving extent of the axis
-    const size_t inner = c_out * gap;               // outputs per outer index
-    const size_t total = outer * inner;
-    size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (tid >= total) return;
-    const size_t o = tid / inner;
-    const size_t p = tid - o * inner;               // i_lo*gap + g
-    const size_t i_lo = p / gap;
-    const uint32_t* src = in + 8 * (o * c * gap + p);
-    const size_t hi_stride = c_lo * gap;            // elements between consecutive i_hi
-    // number of i_hi with i_hi*c_lo + i_lo < c
-    const size_t n_hi = (c - i_lo + c_lo - 1) / c_lo;
-    // One double-width accumulator for the whole weighted sum: at most 64 products of values
-    // below r, so the column sums stay below 64 * 10 * 2^52 and the reduced value below 2.82 r.
+    const Fr acc = f[0];
+    const fr26::Limbs w = fr26::weight16(acc);
+    int32_t* dst = wts + (size_t)fr26::N * (plan.off[p] + threadIdx.x);
+#pragma unroll
+    for (int k = 0; k < fr26::N; k++) dst[k] = w.v[k];
+}
+
+// One pass.  A workgroup is 4 waves: 4/S groups of 64 outputs, each output summed by S waves
+// that take every S-th term; the partial sums meet in LDS.  The weight index is wave-uniform, so
+// the weights arrive through scalar loads and cost no vector registers.
+template <int S>
+__global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
+                                                           const int32_t* __restrict__ wts, uint32_t n_hi_max,
+                                                           uint32_t outer, uint32_t c, uint32_t lg_c_lo, uint32_t gap) {
+    constexpr int IW = 4 / S;                       // output groups per workgroup
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int iw = wave % IW, part = wave / IW;
+    // index arithmetic in 32 bits (the host checks that the output count fits)
+    const uint32_t c_lo = 1u << lg_c_lo;
+    const uint32_t c_out = c < c_lo ? c : c_lo;     // surviving extent of the axis
+    const uint32_t inner = c_out * gap;             // outputs per outer index
+    const uint32_t total = outer * inner;
+    const uint32_t tid = ((uint32_t)blockIdx.x * IW + iw) * 64 + lane;
+    const bool live = tid < total;
+    const uint32_t o = live ? tid / inner : 0;
+    const uint32_t p = live ? tid - o * inner : 0;  // i_lo*gap + g
+    const uint32_t i_lo = p / gap;
+    const uint32_t* src = in + 8 * ((size_t)o * c * gap + p);
+    const size_t hi_stride = (size_t)c_lo * gap;    // elements between consecutive i_hi
+    // number of i_hi with i_hi*c_lo + i_lo < c (zero for a dead lane)
+    const uint32_t n_hi = live ? (c - i_lo + c_lo - 1) >> lg_c_lo : 0;
+    // One double-width accumulator per thread: at most 64 products of values below r, so the
+    // column sums stay below 64 * 10 * 2^52 and the reduced value below 2.82 r.
     fr26::Acc C;
     fr26::acc_zero(C);
-    for (size_t h = 0; h < n_hi; h++) fr26::mac(C, w[h], ld_l26(src, h * hi_stride));
-    st_fr(out, o * inner + p, fr26::unpack(fr26::canon(fr26::reduce(C, 0), 2)));
+    // Terms below n_full = c / c_lo exist for every lane, so the main loop is branch-free with
+    // wave-uniform offsets and four loads in flight per lane (a dead lane reads the terms of
+    // output 0 and stores nothing).  A ragged last term (c not a multiple of c_lo) follows
+    // under a lane predicate, in the part whose turn it is.
+    constexpr int U = 4;
+    const uint32_t n_full = c >> lg_c_lo;
+    uint32_t h = (uint32_t)part;
+    for (; h + (U - 1) * S < n_full; h += U * S) {
+        Fr t[U];
+#pragma unroll
+        for (int k = 0; k < U; k++) t[k] = ld_fr(src, (size_t)(h + k * S) * hi_stride);
+#pragma unroll
+        for (int k = 0; k < U; k++) {
+            fr26::Limbs w;
+#pragma unroll
+            for (int j = 0; j < fr26::N; j++) w.v[j] = wts[(size_t)fr26::N * (h + k * S) + j];
+            fr26::mac(C, w, fr26::pack(t[k]));
+        }
+    }
+    for (; h < n_hi_max; h += S) {
+        if (h < n_hi) {
+            fr26::Limbs w;
+#pragma unroll
+            for (int j = 0; j < fr26::N; j++) w.v[j] = wts[(size_t)fr26::N * h + j];
+            fr26::mac(C, w, ld_l26(src, (size_t)h * hi_stride));
+        }
+    }
+    fr26::Limbs r = fr26::reduce(C, 0);
+    if (S > 1) {
+        __shared__ int32_t lds[fr26::N * (S > 1 ? S - 1 : 1) * IW * 64];
+        if (part > 0) {
+#pragma unroll
+            for (int k = 0; k < fr26::N; k++) lds[((k * (S - 1) + part - 1) * IW + iw) * 64 + lane] = r.v[k];
+        }
+        __syncthreads();
+        if (part == 0) {
+#pragma unroll
+            for (int q = 1; q < S; q++) {
+#pragma unroll
+                for (int k = 0; k < fr26::N; k++) r.v[k] += lds[((k * (S - 1) + q - 1) * IW + iw) * 64 + lane];
+            }
+            r = fr26::normalize(r);
+        }
+    }
+    // below 2.82 S r <= 11.3 r
+    if (part == 0 && live) st_fr(out, tid, fr26::unpack(fr26::canon_wide(r)));
 }
 
 // Small-tensor finish: one workgroup holds the whole [c][gap] slab of one outer index in LDS
 // and binds the remaining bits top-down with a barrier per level.
 constexpr int kFoldSmallElems = 2048;   // 64 KiB of LDS
+constexpr int kFoldSmallMaxOuter = 256; // one workgroup per outer index: worth it only for few
+static bool fold_small_fits(size_t outer, size_t c, size_t gap) {
+    return c * gap <= (size_t)kFoldSmallElems && outer <= (size_t)kFoldSmallMaxOuter;
+}
 
 __global__ void __launch_bounds__(kBlock) fold_small_kernel(uint32_t* out, const uint32_t* in, const uint32_t* x,
                                                             uint32_t L, size_t c, size_t gap) {
@@ -449,8 +529,60 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
     // Otherwise passes ping-pong through scratch and the result is copied to the front.
     uint32_t* ws[2] = {nullptr, nullptr};
     int which = 0;
+    // Plan the passes: each binds as many top bits as possible (6, or more when the outputs are
+    // too few to fill the chip and S waves share one output), until the slab of one outer index
+    // fits the LDS finish kernel.
+    struct FoldPass { uint32_t b, S, off; };
+    FoldPass passes[kFoldMaxPasses];
+    FoldPlan plan;
+    plan.npass = 0;
+    {
+        uint32_t l = L, off = 0;
+        size_t cc = c;
+        while (l > 0 && !fold_small_fits(outer, cc, gap)) {
+            // the most bits per pass that still leave 2^19 threads (8 waves per SIMD), sharing
+            // an output between up to four waves and keeping at most 64 terms per thread
+            uint32_t S = 0, b = 0;
+            for (uint32_t tb = l < 8 ? l : 8; tb >= 1 && S == 0; tb--) {
+                const size_t items = outer * gap * ((size_t)1 << (l - tb));
+                const uint32_t ts = items >= ((size_t)1 << 19) ? 1 : items * 2 >= ((size_t)1 << 19) ? 2 : 4;
+                if (items * ts >= ((size_t)1 << 19) && (1u << tb) <= 64 * ts) { S = ts; b = tb; }
+            }
+            if (S == 0) {
+                // too few outputs to fill the chip whatever the split: four waves per output and
+                // at most 16 terms per thread keep the pass short
+                S = 4; b = l < 6 ? l : 6;
+                // few, short slabs: stop as soon as the LDS finish kernel can take over
+                if (outer <= (size_t)kFoldSmallMaxOuter && gap <= (size_t)kFoldSmallElems) {
+                    uint32_t keep = 0;      // bits the finish kernel can bind
+                    while (keep < l && (((size_t)2 << keep) * gap) <= (size_t)kFoldSmallElems) keep++;
+                    if (l > keep && l - keep < b) b = l - keep;
+                }
+            }
+            GRAPE_REQUIRE(plan.npass < (uint32_t)kFoldMaxPasses, "fold: too many passes");
+            passes[plan.npass] = {b, S, off};
+            plan.lo[plan.npass] = id + (l - b);
+            plan.b[plan.npass] = b;
+            plan.off[plan.npass] = off;
+            plan.npass++;
+            off += 1u << b;
+            l -= b;
+            const size_t c_lo = (size_t)1 << l;
+            cc = cc < c_lo ? cc : c_lo;
+        }
+    }
+    const int32_t* wts = nullptr;
+    if (plan.npass) {
+        void* p;
+        int rc = scratch_get(kSlotFoldW, ((size_t)kFoldMaxPasses * (1u << kFoldMaxBits) + 64) * fr26::N * 4, &p);
+        if (rc) return rc;
+        fold_weights_kernel<<<plan.npass, kBlock, 0, s>>>((int32_t*)p, x, plan);
+        GRAPE_LAUNCH_CHECK();
+        wts = (const int32_t*)p;
+    }
+    uint32_t pi = 0;
     while (L > 0) {
-        if (cur_c * gap <= (size_t)kFoldSmallElems) {
+        if (fold_small_fits(outer, cur_c, gap)) {
             uint32_t* dst = t;
             if (outer > 1 && src == t) {
                 // reading slabs o*cur_c*gap while writing o*gap would race across workgroups
@@ -464,9 +596,8 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
             if (dst != t) GRAPE_HIP_CHECK(hipMemcpyAsync(t, dst, outer * gap * 32, hipMemcpyDeviceToDevice, s));
             return GRAPE_OK;
         }
-        // pick b: as many bits as possible while keeping >= 2^17 output threads
-        uint32_t b = L < (uint32_t)kFoldMaxBits ? L : (uint32_t)kFoldMaxBits;
-        while (b > 1 && outer * gap * ((size_t)1 << (L - b)) < ((size_t)1 << 17)) b--;
+        const FoldPass& ps = passes[pi++];
+        const uint32_t b = ps.b;
         const size_t c_lo = (size_t)1 << (L - b);
         const size_t c_out = cur_c < c_lo ? cur_c : c_lo;
         uint32_t* dst;
@@ -486,7 +617,15 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
             which ^= 1;
         }
         const size_t total = outer * c_out * gap;
-        fold_pass_kernel<<<blocks_for(total), kBlock, 0, s>>>(dst, src, xs + 8 * (size_t)(L - b), b, outer, cur_c, c_lo, gap);
+        GRAPE_REQUIRE(total < ((size_t)1 << 32) - 256, "fold: more than 2^32 outputs in one pass");
+        const uint32_t n_hi_max = (uint32_t)((cur_c + c_lo - 1) / c_lo);
+        const int32_t* w = wts + (size_t)fr26::N * ps.off;
+        if (ps.S == 1)
+            fold_pass_kernel<1><<<blocks_for(total, 256), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
+        else if (ps.S == 2)
+            fold_pass_kernel<2><<<blocks_for(total, 128), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
+        else
+            fold_pass_kernel<4><<<blocks_for(total, 64), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
         GRAPE_LAUNCH_CHECK();
         src = dst;
         cur_c = c_out;

@@ -32,4 +32,23 @@ void t26_weighted_sum(const uint32_t* w, const uint32_t* t, int n, uint32_t* out
     for (int i = 0; i < n; i++) fr26::mac(C, fr26::weight16(ld(w + 8 * i)), fr26::pack(ld(t + 8 * i)));
     st(out, fr26::unpack(fr26::canon(fr26::reduce(C, 0), 2)));   // 64/35.3 + 1 = 2.82 r
 }
+// the same over n <= 64*S terms, every S-th term into one of S accumulators whose reduced values
+// are added limb-wise and canonicalised by quotient estimate (split fold pattern)
+void t26_weighted_sum_split(const uint32_t* w, const uint32_t* t, int n, int S, uint32_t* out) {
+    fr26::Limbs r;
+    for (int k = 0; k < fr26::N; k++) r.v[k] = 0;
+    for (int q = 0; q < S; q++) {
+        fr26::Acc C;
+        fr26::acc_zero(C);
+        for (int i = q; i < n; i += S) fr26::mac(C, fr26::weight16(ld(w + 8 * i)), fr26::pack(ld(t + 8 * i)));
+        r = fr26::add(r, fr26::reduce(C, 0));
+    }
+    st(out, fr26::unpack(fr26::canon_wide(fr26::normalize(r))));
+}
+// k * a + b for canonical a, b and 0 <= k < 31, through canon_wide
+void t26_canon_wide(const uint32_t* a, const uint32_t* b, int k, uint32_t* out) {
+    fr26::Limbs A = fr26::pack(ld(a)), B = fr26::pack(ld(b)), r;
+    for (int i = 0; i < fr26::N; i++) r.v[i] = k * A.v[i] + B.v[i];
+    st(out, fr26::unpack(fr26::canon_wide(fr26::normalize(r))));
+}
 }

@@ -86,3 +86,19 @@ def test_weighted_sum_64(lib):
             t = [R - 1 if trial == 0 else rng.randrange(R) for _ in range(n)]
             lib.t26_weighted_sum(_u32(_p(w)), _u32(_p(t)), n, _u32(out))
             assert _val(out) == sum(x * y for x, y in zip(w, t)) % R
+
+
+def test_split_weighted_sum_and_wide_canon(lib):
+    rng = random.Random(4)
+    out = np.zeros(8, dtype=np.uint32)
+    for n, S in ((1, 2), (5, 4), (128, 2), (256, 4), (64, 1), (200, 4)):
+        for trial in range(6):
+            w = [R - 1 if trial == 0 else rng.randrange(R) for _ in range(n)]
+            t = [R - 1 if trial == 0 else rng.randrange(R) for _ in range(n)]
+            lib.t26_weighted_sum_split(_u32(_p(w)), _u32(_p(t)), n, S, _u32(out))
+            assert _val(out) == sum(x * y for x, y in zip(w, t)) % R
+    for k in (0, 1, 2, 15, 30):
+        for a in EDGE + [rng.randrange(R) for _ in range(10)]:
+            for b in (0, 1, R - 1, rng.randrange(R)):
+                lib.t26_canon_wide(_u32(_p([a % R])[0]), _u32(_p([b])[0]), k, _u32(out))
+                assert _val(out) == (k * (a % R) + b) % R
