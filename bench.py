@@ -41,6 +41,7 @@ EXEC_MULS_PER_POINT = 8 * (196 + 196 + 14) + 2 * (105 + 196 + 14)
 # lane-level 32x32 multiplies per second if every SIMD issued one v_mad_u64_u32 per cycle:
 # 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz
 PEAK_MULS_NOMINAL = 256 * 64 * 2.4e9
+HBM_PEAK_GBPS = 8000.0
 
 
 def gaussian_i16(shape, seed, sigma=SIGMA):
@@ -346,6 +347,40 @@ def main():
         "reduce_kernel_ms": red_ms,
     }
 
+    # ---- HBM side of the same kernel: one 128-byte table entry and one 4-byte scalar per point
+    roofline["hbm_view"] = {"bytes_per_point": 132, "achieved_GBps": 132.0 * points / (acc_ms * 1e-3) / 1e9,
+                            "peak_GBps": HBM_PEAK_GBPS, "frac": 132.0 * points / (acc_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+    # ---- plain copy of known size (the kernel the FETCH_SIZE / WRITE_SIZE counters are scaled by)
+    copy_bytes = 1 << 30
+    copy_ms = ops.bench_copy(copy_bytes, 5)
+    hbm_copy = {"kernel": "copy_kernel", "bytes_read": copy_bytes, "bytes_written": copy_bytes,
+                "GBps": 2.0 * copy_bytes / (copy_ms * 1e-3) / 1e9}
+
+    # ---- the streaming Fr kernels: first fold pass over a 2^25-element tensor (1 GiB, reference
+    # format, four times the Infinity Cache), duration from HIP events inside the library
+    n_fold, c_fold = 1 << 25, 64
+    t_fold = ops.fr_empty(n_fold)
+    t_fold.zero_()
+    x_fold = ops.to_dev(seeded_scalars(8, SEED_G + 1))
+    ops.profile_enable(True)
+    fold_ms = []
+    torch.cuda.synchronize()
+    for _ in range(6):
+        # the tensor is all zero and stays so; it is not rewritten between runs, so no dirty
+        # cache lines of a fill kernel are written back while the pass is timed
+        ops.fr_fold(t_fold, n_fold, x_fold, c_fold, 0, n_fold // c_fold)
+        fold_ms.append(ops.profile_last()[1])
+    fold_ms = fold_ms[1:]
+    ops.profile_enable(False)
+    fold_pass_ms = float(np.median(fold_ms))
+    fold_bytes = 32.0 * n_fold                                   # every element read once (writes: 1/32 more, not counted)
+    roofline_streaming = {"bound": "hbm", "kernel": "fold_pass_kernel<1> (first pass of grape_fr_fold, c=64)",
+                          "achieved": fold_bytes / (fold_pass_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                          "frac": fold_bytes / (fold_pass_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                          "kernel_ms": fold_pass_ms, "elements": n_fold}
+    del t_fold
+
     result = {
         "metric": "hyrax_commit_throughput",
         "value": value,
@@ -365,6 +400,8 @@ def main():
                    "rows": ROWS, "cols": COLS, "radix_bits": RADIX_BITS,
                    "table_bytes": int(table.numel()) * 4, "table_gen_s": table_gen_s},
         "roofline": roofline,
+        "roofline_streaming": roofline_streaming,
+        "hbm_copy": hbm_copy,
     }
 
     if not args.no_cpu_baseline:

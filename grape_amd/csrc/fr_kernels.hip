@@ -540,18 +540,24 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
         uint32_t l = L, off = 0;
         size_t cc = c;
         while (l > 0 && !fold_small_fits(outer, cc, gap)) {
-            // the most bits per pass that still leave 2^19 threads (8 waves per SIMD), sharing
-            // an output between up to four waves and keeping at most 64 terms per thread
+            // Measured on MI355X: a pass streams fastest with one thread per output, 16 to 64
+            // terms per thread and 2^20 threads; 2^19 threads come close.  Failing that, up to
+            // four waves share an output to reach 2^19 threads.
             uint32_t S = 0, b = 0;
-            for (uint32_t tb = l < 8 ? l : 8; tb >= 1 && S == 0; tb--) {
-                const size_t items = outer * gap * ((size_t)1 << (l - tb));
-                const uint32_t ts = items >= ((size_t)1 << 19) ? 1 : items * 2 >= ((size_t)1 << 19) ? 2 : 4;
-                if (items * ts >= ((size_t)1 << 19) && (1u << tb) <= 64 * ts) { S = ts; b = tb; }
+            auto items = [&](uint32_t tb) { return outer * gap * ((size_t)1 << (l - tb)); };
+            for (uint32_t want = 20; want >= 19 && S == 0; want--) {
+                for (uint32_t tb = l < 6 ? l : 6; tb >= 4 && S == 0; tb--) {
+                    if (items(tb) >= ((size_t)1 << want)) { S = 1; b = tb; }
+                }
+            }
+            for (uint32_t tb = l < 8 ? l : 8; tb >= 4 && S == 0; tb--) {
+                const uint32_t ts = items(tb) * 2 >= ((size_t)1 << 19) ? 2 : 4;
+                if (items(tb) * ts >= ((size_t)1 << 19) && (1u << tb) <= 64 * ts) { S = ts; b = tb; }
             }
             if (S == 0) {
                 // too few outputs to fill the chip whatever the split: four waves per output and
-                // at most 16 terms per thread keep the pass short
-                S = 4; b = l < 6 ? l : 6;
+                // at most 32 terms per thread keep the pass short
+                S = 4; b = l <= 7 ? l : 6;
                 // few, short slabs: stop as soon as the LDS finish kernel can take over
                 if (outer <= (size_t)kFoldSmallMaxOuter && gap <= (size_t)kFoldSmallElems) {
                     uint32_t keep = 0;      // bits the finish kernel can bind
@@ -576,8 +582,11 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
         void* p;
         int rc = scratch_get(kSlotFoldW, ((size_t)kFoldMaxPasses * (1u << kFoldMaxBits) + 64) * fr26::N * 4, &p);
         if (rc) return rc;
+        profile_begin();
+        profile_mark(s);
         fold_weights_kernel<<<plan.npass, kBlock, 0, s>>>((int32_t*)p, x, plan);
         GRAPE_LAUNCH_CHECK();
+        profile_mark(s);               // profiled intervals: the weight kernel, then one per pass
         wts = (const int32_t*)p;
     }
     uint32_t pi = 0;
@@ -627,6 +636,7 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
         else
             fold_pass_kernel<4><<<blocks_for(total, 64), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
         GRAPE_LAUNCH_CHECK();
+        profile_mark(s);
         src = dst;
         cur_c = c_out;
         L -= b;

@@ -228,7 +228,8 @@ int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double *mads_per_s
 /* Kernel-level timing: when enabled, the commitment entry points bracket each kernel they launch
  * with HIP events on the caller's stream.  grape_profile_last() synchronises and returns the
  * durations (ms) of the kernels of the most recent call, in launch order (for grape_commit_*:
- * [0] accumulation kernel, [1] row-reduction kernel); *n receives how many were written. */
+ * [0] accumulation kernel, [1] row-reduction kernel; for grape_fr_fold: [0] weight kernel, then
+ * one entry per pass); *n receives how many were written. */
 int grape_profile_enable(int on);
 int grape_profile_last(float *ms, int cap, int *n);
 /* Event timing helpers on a stream (HIP events), for benchmarks that live above this ABI. */
