@@ -42,6 +42,11 @@ EXEC_MULS_PER_POINT = 8 * (196 + 196 + 14) + 2 * (105 + 196 + 14)
 # 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz
 PEAK_MULS_NOMINAL = 256 * 64 * 2.4e9
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch read from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# same counter reads for the 1 GiB copy kernel below); the counters cannot be read from inside this
+# process, so these are the figures of the committed counter summary of this same command.
+COMMIT_KERNEL_TRAFFIC_BYTES = 2.207e9
+FOLD_KERNEL_TRAFFIC_BYTES = 1.110e9
 
 
 def gaussian_i16(shape, seed, sigma=SIGMA):
@@ -260,6 +265,81 @@ def layer_workload(args):
     return 0
 
 
+def matmul_workload(args):
+    """BASELINE.json configs[2]: prove_matmul of a 2048 x 4096 activation by a 4096 x 4096 weight
+    (both int16-range, seeded), 12 sumcheck rounds over k after folding the row variables of both
+    operands.  One step = one proof; the claim and the final evaluations are checked against
+    independent multilinear evaluations on the GPU."""
+    import torch
+    from grape_amd import ops, _host as host
+    from gpuutil import rand_fr
+    ops.init(0)
+    host.load()
+    N, M, K = 2048, 4096, 4096
+    dA = ops.fr_from_i32(torch.from_numpy(gaussian_i16((N, K), 31)).cuda())
+    dB = ops.fr_from_i32(torch.from_numpy(gaussian_i16((M, K), 32)).cuda())
+    u, v = rand_fr(23, 33), rand_fr(12, 34)
+    du = ops.to_dev(u)
+    a2, b2 = dA.clone(), dB.clone()
+    ops.fr_fold(a2, N * K, du, N, 12, K)
+    ops.fr_fold(b2, M * K, du, M, 0, K)
+    claim = ops.fr_to_host(ops.fr_sum(ops.fr_mul(a2[:K].contiguous(), b2[:K].contiguous())))[0]
+    del a2, b2
+    secs = []
+    for i in range(args.warmup + args.steps):
+        _, _, ac, bc = host.prove_matmul(dA, dB, 1, N, M, K, u, v, claim)
+        if i >= args.warmup:
+            secs.append(host.last_prove_seconds())
+    pa, pb = np.concatenate([v, u[12:23]]), np.concatenate([v, u[0:12]])
+    if not (np.array_equal(host.mle_eval(dA, N * K, pa), ac) and np.array_equal(host.mle_eval(dB, M * K, pb), bc)):
+        print("bench.py: final evaluations of prove_matmul differ from independent evaluations", file=sys.stderr)
+        return 1
+    t = float(np.mean(secs))
+    print(json.dumps({
+        "metric": "matmul_sumcheck_time", "value": t, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: prove_matmul 2048x4096 by 4096x4096 (int16-range operands as Fr tensors)",
+                   "operand_bytes": 32 * (N * K + M * K),
+                   "operand_read_GBps": 32.0 * (N * K + M * K) / t / 1e9}}))
+    return 0
+
+
+def lookup_workload(args):
+    """BASELINE.json configs[3]: tLookupRange proof of 2^24 values in a 2^16-entry range with its
+    commitments of A and m (4096 generators).  One step = one proof."""
+    import torch
+    from grape_amd import ops, _host as host
+    from gpuutil import rand_fr
+    import bigref as br
+    ops.init(0)
+    host.load()
+    D, N, low = 1 << 24, 1 << 16, -32768
+    S = np.random.default_rng(41).integers(low, low + N, size=D).astype(np.int32)
+    gens = ops.g1_make_generators(rand_fr(4096, 42))
+    table = ops.g1_table_gen(gens, 256)
+    alpha, u, v = rand_fr(1, 43), rand_fr(24, 44), rand_fr(24, 45)
+    secs, commits = [], []
+    for i in range(args.warmup + args.steps):
+        dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
+        res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 4096, 1, 4096)
+        if i >= args.warmup:
+            secs.append(host.last_prove_seconds())
+            commits.append(res["commit_s"])
+    if br.fr_unpack(res["m"]) != [int(x) for x in np.bincount(S.astype(np.int64) - low, minlength=N)]:
+        print("bench.py: multiplicities differ from numpy.bincount", file=sys.stderr)
+        return 1
+    t = float(np.mean(secs))
+    print(json.dumps({
+        "metric": "lookup_prove_time", "value": t, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: tLookupRange, 2^24 lookups into a 2^16 range, 4096 generators",
+                   "commit_s": float(np.mean(commits)),
+                   "note": "tables tied to the Hyrax and lookup objects (fixed-base tables, B[t]*G_i) are built in the warm-up proof"}}))
+    return 0
+
+
 def _fr_const(x):
     """Montgomery limbs of a small constant, as a (1, 4) uint64 array"""
     r = 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001
@@ -273,14 +353,19 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["commit", "layer"], default="commit",
-                    help="commit: configs[1], the metric's headline (default); layer: configs[4]")
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup"], default="commit",
+                    help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
+                         "lookup: configs[3]; layer: configs[4]")
     ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
         return 2
+    if args.workload in ("matmul", "lookup"):
+        args.steps = 5 if args.steps is None else args.steps
+        args.warmup = 1 if args.warmup is None else args.warmup
+        return matmul_workload(args) if args.workload == "matmul" else lookup_workload(args)
     if args.workload == "layer":
         args.steps = 1 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
@@ -337,7 +422,9 @@ def main():
         "peak": peak_measured / 1e12,
         "unit": "Tmul/s",
         "frac": achieved_alg / peak_measured,
-        "traffic": None,
+        "traffic": COMMIT_KERNEL_TRAFFIC_BYTES,
+        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the 1 GiB copy kernel "
+                          "(FETCH_SIZE unit 2 KiB, WRITE_SIZE unit 1 KiB); algorithmic bytes 2.28e9",
         "achieved_executed": achieved_exec / 1e12,
         "frac_executed": achieved_exec / peak_measured,
         "peak_nominal": PEAK_MULS_NOMINAL / 1e12,
@@ -377,7 +464,7 @@ def main():
     fold_bytes = 32.0 * n_fold                                   # every element read once (writes: 1/32 more, not counted)
     roofline_streaming = {"bound": "hbm", "kernel": "fold_pass_kernel<1> (first pass of grape_fr_fold, c=64)",
                           "achieved": fold_bytes / (fold_pass_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                          "frac": fold_bytes / (fold_pass_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                          "frac": fold_bytes / (fold_pass_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": FOLD_KERNEL_TRAFFIC_BYTES,
                           "kernel_ms": fold_pass_ms, "elements": n_fold}
     del t_fold
 

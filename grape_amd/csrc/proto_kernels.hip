@@ -112,6 +112,66 @@ __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint
     if (valid && ((todo >> lane) & 1ull)) atomicAdd(&hist[idx], 1u);
 }
 
+// Large histograms.  Device-wide atomics on a table of a million counters run at a few 10^9
+// per second on this part (they are resolved on the memory side of the XCDs' L2 caches), so a
+// long witness is counted in LDS instead: the witness is first reduced to 32-bit indices
+// (index_kernel), workgroup (g, p) then streams chunk g of the indices and counts the bins of
+// range p in LDS, and writes its counters with plain stores; a last kernel adds the chunks up.
+// Every chunk is read once per bin range - 4 bytes per element and range, all of it streaming.
+constexpr int kHistThreads = 1024;
+
+template <int BINS>
+__global__ void __launch_bounds__(kHistThreads) hist_lds_kernel(uint32_t* __restrict__ partial, const int32_t* __restrict__ idx1,
+                                                                size_t n, size_t per_chunk, uint32_t len) {
+    extern __shared__ uint32_t bins[];
+    for (int k = threadIdx.x; k < BINS; k += kHistThreads) bins[k] = 0;
+    __syncthreads();
+    const uint32_t base = blockIdx.y * (uint32_t)BINS;
+    const size_t lo = (size_t)blockIdx.x * per_chunk;            // per_chunk is a multiple of 4
+    const size_t hi = lo + per_chunk < n ? lo + per_chunk : n;
+    const int lane = threadIdx.x & 63;
+    for (size_t i0 = lo + 4 * (size_t)(threadIdx.x & ~63); i0 < hi; i0 += 4 * kHistThreads) {
+        // a wave takes 256 consecutive indices, four per lane (the trip count is wave-uniform)
+        const size_t i = i0 + 4 * (size_t)lane;
+        int4 v = make_int4(0, 0, 0, 0);
+        if (i + 4 <= hi) {
+            v = *reinterpret_cast<const int4*>(idx1 + i);
+        } else {
+            if (i < hi) v.x = idx1[i];
+            if (i + 1 < hi) v.y = idx1[i + 1];
+            if (i + 2 < hi) v.z = idx1[i + 2];
+        }
+        const int vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t b = (uint32_t)(vv[q] - 1) - base;      // 0 (out of range) wraps far away
+            const bool in = b < (uint32_t)BINS;
+            // lanes that share a bin are counted once: up to four leaders, then plain adds
+            unsigned long long todo = __ballot(in);
+            for (int it = 0; it < 4 && todo != 0ull; it++) {
+                const int leader = __ffsll((long long)todo) - 1;
+                const uint32_t lb = __shfl(b, leader, 64);
+                const unsigned long long same = __ballot(in && b == lb) & todo;
+                if (lane == leader) atomicAdd(&bins[lb], (uint32_t)__popcll(same));
+                todo &= ~same;
+            }
+            if (in && ((todo >> lane) & 1ull)) atomicAdd(&bins[b], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t* dst = partial + (size_t)blockIdx.x * len + base;
+    const uint32_t live = len - base < (uint32_t)BINS ? len - base : (uint32_t)BINS;
+    for (uint32_t k = threadIdx.x; k < live; k += kHistThreads) dst[k] = bins[k];
+}
+
+__global__ void __launch_bounds__(kBlock) hist_merge_kernel(uint32_t* hist, const uint32_t* partial, uint32_t chunks, uint32_t len) {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= len) return;
+    uint32_t s = 0;
+    for (uint32_t g = 0; g < chunks; g++) s += partial[(size_t)g * len + t];
+    hist[t] += s;
+}
+
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -311,7 +371,46 @@ int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t l
     if (n == 0) return GRAPE_OK;
     GRAPE_REQUIRE(hist != nullptr && len > 0, "bad histogram buffer");
     CHECK_PTR16(vals);
-    hist_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(hist, vals, n, low, len);
+    hipStream_t s = as_stream(st);
+    if (n < ((size_t)1 << 20)) {
+        hist_kernel<<<blocks_for(n), kBlock, 0, s>>>(hist, vals, n, low, len);
+        GRAPE_LAUNCH_CHECK();
+        return GRAPE_OK;
+    }
+    // LDS counting: 32768 bins (128 KiB) per workgroup when the device grants that much dynamic
+    // LDS, else 16384
+    static int bins = 0;
+    if (bins == 0) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&hist_lds_kernel<32768>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 32768 * 4);
+        if (e == hipSuccess) {
+            bins = 32768;
+        } else {
+            (void)hipGetLastError();
+            bins = 16384;
+        }
+    }
+    const uint32_t ranges = (len + (uint32_t)bins - 1) / (uint32_t)bins;
+    // chunks: enough workgroups to fill the chip, partial counters capped at 1 GiB
+    size_t chunks = 256;
+    while (chunks > 1 && chunks * (size_t)len * 4 > ((size_t)1 << 30)) chunks /= 2;
+    while (chunks > 1 && n / chunks < ((size_t)1 << 16)) chunks /= 2;
+    size_t per_chunk = (n + chunks - 1) / chunks;
+    per_chunk = (per_chunk + 3) & ~(size_t)3;
+    void *idx, *partial;
+    int rc = scratch_get(kSlotHistIdx, n * 4, &idx);
+    if (rc) return rc;
+    rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial);
+    if (rc) return rc;
+    index_kernel<<<blocks_for(n), kBlock, 0, s>>>((int32_t*)idx, vals, n, low, len);
+    GRAPE_LAUNCH_CHECK();
+    const dim3 grid((unsigned)chunks, ranges);
+    if (bins == 32768)
+        hist_lds_kernel<32768><<<grid, kHistThreads, 32768 * 4, s>>>((uint32_t*)partial, (const int32_t*)idx, n, per_chunk, len);
+    else
+        hist_lds_kernel<16384><<<grid, kHistThreads, 16384 * 4, s>>>((uint32_t*)partial, (const int32_t*)idx, n, per_chunk, len);
+    GRAPE_LAUNCH_CHECK();
+    hist_merge_kernel<<<blocks_for(len), kBlock, 0, s>>>(hist, (const uint32_t*)partial, (uint32_t)chunks, len);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

@@ -106,6 +106,33 @@ def test_histogram(ops):
     assert h3.sum() == 1 and h3[3] == 1
 
 
+def test_histogram_long_witness(ops):
+    """witnesses of 2^20 values and more take the LDS-counting path: ragged length, a table that
+    is not a multiple of the bins held in LDS, a clipped (heavily repeated) value, values outside
+    the table, and accumulation into a histogram that is not zero"""
+    import torch
+    low, length = -40000, 100003
+    n = (1 << 20) + 4099
+    rng = np.random.default_rng(32)
+    s = np.rint(rng.normal(0.0, 30000.0, size=n)).astype(np.int64)
+    s = np.clip(s, low - 50, low + length + 49)              # piles at both ends, 50 steps outside
+    s[::7] = 12345
+    s32 = s.astype(np.int32)
+    vals = ops.fr_from_i32(torch.from_numpy(s32).cuda())
+    inside = (s >= low) & (s < low + length)
+    want = np.bincount(s[inside] - low, minlength=length).astype(np.uint32)
+    h = ops.tlookup_hist(vals, low, length).cpu().numpy().view(np.uint32)
+    assert np.array_equal(h, want)
+    assert int(h.sum()) == int(inside.sum()) < n
+    pre = torch.full((length,), 3, dtype=torch.int32, device="cuda")
+    h2 = ops.tlookup_hist(vals, low, length, hist=pre).cpu().numpy().view(np.uint32)
+    assert np.array_equal(h2, want + 3)
+    # small table, everything in one bin
+    same = ops.fr_from_i32(torch.full(((1 << 20) + 1,), 5, dtype=torch.int32, device="cuda"))
+    h3 = ops.tlookup_hist(same, 0, 16).cpu().numpy()
+    assert h3[5] == (1 << 20) + 1 and h3.sum() == (1 << 20) + 1
+
+
 def test_table_init(ops):
     low, length = -32768, 65536
     beta = br.fr_pack([length])
