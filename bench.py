@@ -36,8 +36,9 @@ K_DIGIT = 32768
 # product): 2 * 10 * 300.
 ALG_MULS_PER_POINT = 6000
 # What the fast path executes: ONE mixed addition per point on 14 limbs of 28 bits:
-# 8 products of 14*14 + 14*14 + 14 multiply-adds and 2 squares of 105 + 14*14 + 14.
-EXEC_MULS_PER_POINT = 8 * (196 + 196 + 14) + 2 * (105 + 196 + 14)
+# 6 products of 14*14 + 14*14 + 14 multiply-adds, one fused difference of two products
+# (2*14*14 + 14*14 + 14) and 2 squares of 105 + 14*14 + 14.
+EXEC_MULS_PER_POINT = 6 * (196 + 196 + 14) + (3 * 196 + 14) + 2 * (105 + 196 + 14)
 # lane-level 32x32 multiplies per second if every SIMD issued one v_mad_u64_u32 per cycle:
 # 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz
 PEAK_MULS_NOMINAL = 256 * 64 * 2.4e9

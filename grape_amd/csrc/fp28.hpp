@@ -141,6 +141,39 @@ GRAPE_HD Fp28 mul(const Fp28& a, const Fp28& b) {
 }
 
 // a^2/2^392: the off-diagonal limb products are taken once with a doubled operand.
+// a*b - c*d with one Montgomery reduction: both products accumulate in the same columns.
+// Needs 14*(2^(la+lb) + 2^(lc+ld)) + 14*2^56 < 2^63 for the limb bounds and |ab| + |cd| <= 2^11 p^2
+// for the values; the result is normalised in (0, 3p) like a product.
+GRAPE_HD Fp28 mul_sub(const Fp28& a, const Fp28& b, const Fp28& c, const Fp28& d) {
+    int64_t C[2 * N];
+#pragma unroll
+    for (int k = 0; k < 2 * N; k++) C[k] = 0;
+    int32_t nc[N];                        // limb-wise negation keeps every step a multiply-add
+#pragma unroll
+    for (int j = 0; j < N; j++) nc[j] = -c.v[j];
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)a.v[j] * (int64_t)b.v[i];
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)nc[j] * (int64_t)d.v[i];
+        const int32_t m = (int32_t)(((uint32_t)C[i] * PINV) & MASK);
+#pragma unroll
+        for (int j = 0; j < N; j++) C[i + j] += (int64_t)m * (int64_t)P(j);
+        C[i + 1] += C[i] >> W;
+    }
+    Fp28 r;
+    int64_t cy = 0;
+#pragma unroll
+    for (int k = 0; k < N - 1; k++) {
+        int64_t t = C[N + k] + (int64_t)P(k) + cy;
+        r.v[k] = (int32_t)((uint32_t)t & MASK);
+        cy = t >> W;
+    }
+    r.v[N - 1] = (int32_t)(C[2 * N - 1] + (int64_t)P(N - 1) + cy);
+    return r;
+}
+
 GRAPE_HD Fp28 sqr(const Fp28& a) {
     int64_t C[2 * N];
 #pragma unroll
@@ -524,7 +557,7 @@ GRAPE_HD bool xyzz28_madd(Xyzz28& acc, const Affine28& p, bool negate) {
     for (int i = 0; i < N; i++) X3.v[i] = RR.v[i] - PPP.v[i] - 2 * Q.v[i];   // (-9p, 3p), |limb| < 2^30
     X3 = normalize(X3);
     const Fp28 T = sub(Q, X3);                         // (-3p, 12p), |limb| < 2^29
-    const Fp28 Y3 = sub(mul(R, T), mul(acc.y, PPP));   // 6*12 = 72 ; 3*3 = 9 -> (-3p, 3p)
+    const Fp28 Y3 = mul_sub(R, T, acc.y, PPP);         // 6*12 + 3*3 = 81 <= 2^11; limbs 29+29, 28+28 -> (0, 3p)
     acc.zzz = mul(acc.zzz, PPP);                       // 9
     acc.zz = ZZ3;
     acc.x = X3;
@@ -558,7 +591,7 @@ GRAPE_HD bool xyzz28_add(Xyzz28& acc, const Xyzz28& q) {
     for (int i = 0; i < N; i++) X3.v[i] = RR.v[i] - PPP.v[i] - 2 * Q.v[i];   // (-9p, 3p)
     X3 = normalize(X3);
     const Fp28 T = sub(Q, X3);                         // (-3p, 12p)
-    const Fp28 Y3 = sub(mul(R, T), mul(S1, PPP));      // 36 ; 9
+    const Fp28 Y3 = mul_sub(R, T, S1, PPP);            // 36 + 9
     acc.zzz = mul(mul(acc.zzz, q.zzz), PPP);
     acc.zz = ZZ3;
     acc.x = X3;

@@ -46,6 +46,7 @@ Fr matmul_sumcheck_phase1(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, Fr
 // src/prove.cu:87-117, with the three reductions fused into the round kernel
 void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* v, uint K, Fr& claim,
                             Fr& eq_accumulate, SumcheckTranscript* transcript) {
+    (void)a;
     (void)b;
     (void)c;
     uint rounds = Log2(K);
@@ -55,29 +56,25 @@ void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, 
     // all challenges of this phase in one copy
     std::vector<Fr> vs(rounds);
     check(grape_memcpy_d2h(vs.data(), v - rounds, sizeof(fr_t) * rounds, nullptr), "grape_memcpy_d2h");
-    fr_t* d_sums = a.gpu_data;   // a has at least K >= 3 elements whenever rounds >= 2; see below
-    fr_t* own = nullptr;
-    if (a.size < 3) {
-        check(grape_malloc((void**)&own, 3 * sizeof(fr_t)), "grape_malloc");
-        d_sums = own;
-    }
+    // The challenges are known before the first round, so all rounds are queued back to back,
+    // each leaving its three sums in its own slot, and read with one copy at the end (the
+    // reference copies and synchronises after every round).
+    FrTensor sums(3 * rounds);
     for (uint i = 0; i < rounds; i++) {
-        check(grape_sumcheck_round2(W(A.gpu_data), W(B.gpu_data), inputsize, outputsize, W(v - i - 1), W(d_sums), nullptr),
+        check(grape_sumcheck_round2(W(A.gpu_data), W(B.gpu_data), inputsize, outputsize, W(v - i - 1), W(sums.gpu_data + 3 * i), nullptr),
               "grape_sumcheck_round2");
-        Fr s[3];
-        read3(d_sums, s);
-        Polynomial p({s[0] * eq_accumulate, s[1] * eq_accumulate, s[2] * eq_accumulate});
-        if (p(0) + p(1) != claim) {
-            grape_free(own);
-            throw std::runtime_error("matmul_phase2: claim != p(0) + p(1)");
-        }
-        const Fr& v_now = vs[rounds - 1 - i];
-        claim = p(v_now);
-        record(transcript, p, claim);
         inputsize = outputsize;
         outputsize = outputsize / 2;
     }
-    grape_free(own);
+    std::vector<Fr> s(3 * (size_t)rounds);
+    check(grape_memcpy_d2h(s.data(), sums.gpu_data, sizeof(fr_t) * 3 * rounds, nullptr), "grape_memcpy_d2h");
+    for (uint i = 0; i < rounds; i++) {
+        Polynomial p({s[3 * i] * eq_accumulate, s[3 * i + 1] * eq_accumulate, s[3 * i + 2] * eq_accumulate});
+        if (p(0) + p(1) != claim) throw std::runtime_error("matmul_phase2: claim != p(0) + p(1)");
+        const Fr& v_now = vs[rounds - 1 - i];
+        claim = p(v_now);
+        record(transcript, p, claim);
+    }
 }
 
 // src/prove.cu:175-210

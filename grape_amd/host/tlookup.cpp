@@ -113,69 +113,77 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         check(grape_stream_sync(nullptr), "sync");
         grape_free(d_u);
     }
-    FrTensor sums(8);
-    Fr alpha_run = alpha;
-    uint cur = D;
-    int ui = (int)nu - 1;      // index of the variable bound in this round (u.back())
-    Fr h[8];
-    // phase 1: D -> N, challenges v[logN ..] from the back
-    for (int vi = (int)v.size() - 1; vi >= (int)logN; vi--, ui--) {
-        const uint half = cur / 2;
-        check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
-              "grape_tlookup_round_sums");
-        check(grape_memcpy_d2h(h, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
-        Polynomial p0({h[0], h[1], h[2]});
-        p0 = p0 * alpha_run;
-        p0 *= Polynomial::eq(u[ui]);
-        Polynomial p1({h[3], h[4]});
-        Polynomial p = p0 + p1 + Polynomial(C * two_inv);
-        if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase1: claim != p(0) + p(1)");
-        claim = p(v[vi]);
-        last_transcript.rounds.push_back(p);
-        last_transcript.claims.push_back(claim);
-        uint32_t* ptrs[2] = {W(A.gpu_data), W(S.gpu_data)};
-        check(grape_fr_fold_msb_multi(ptrs, 2, half, W(grape_host::device_scalar(v[vi])), nullptr), "grape_fr_fold_msb_multi");
-        A.set_size(half);
-        S.set_size(half);
-        if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
-        alpha_run *= Polynomial::eq(u[ui], v[vi]);
-        C = C * two_inv;
-        cur = half;
-    }
-    // phase 2: bind the table variables; T, B, m of this object stay intact
-    FrTensor Bw(B), Tw(T), mw(m);
-    Fr alpha_sq_run = alpha_sq;
-    for (int vi = (int)logN - 1; vi >= 0; vi--, ui--) {
-        const uint half = cur / 2;
-        Fr a3[5], b3[5], c3[3];
-        check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
-              "grape_tlookup_round_sums");
-        check(grape_memcpy_d2h(a3, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
-        check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(E.gpu_data), half, W(sums.gpu_data), nullptr),
-              "grape_tlookup_round_sums");
-        check(grape_memcpy_d2h(b3, sums.gpu_data, 5 * sizeof(fr_t), nullptr), "d2h");
-        check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(sums.gpu_data), nullptr), "grape_tlookup_mb_sums");
-        check(grape_memcpy_d2h(c3, sums.gpu_data, 3 * sizeof(fr_t), nullptr), "d2h");
-        Polynomial p0({a3[0], a3[1], a3[2]});
-        p0 = p0 * alpha_run;
-        Fr coef = N_div_D * alpha_sq_run;
-        p0 += Polynomial({b3[0] * coef, b3[1] * coef, b3[2] * coef});
-        Polynomial p1({a3[3], a3[4]});
-        Polynomial p2({c3[0], c3[1], c3[2]});
-        Polynomial p = Polynomial::eq(u[ui]) * p0 + p1 - p2 * N_div_D;
-        if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase2: claim != p(0) + p(1)");
-        claim = p(v[vi]);
-        last_transcript.rounds.push_back(p);
-        last_transcript.claims.push_back(claim);
-        uint32_t* ptrs[5] = {W(A.gpu_data), W(S.gpu_data), W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
-        check(grape_fr_fold_msb_multi(ptrs, 5, half, W(grape_host::device_scalar(v[vi])), nullptr), "grape_fr_fold_msb_multi");
-        A.set_size(half);
-        S.set_size(half);
-        if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
-        Fr e = Polynomial::eq(u[ui], v[vi]);
-        alpha_run *= e;
-        alpha_sq_run *= e;
-        cur = half;
+    // The prover's challenges are all known before the first round, so the rounds are queued
+    // back to back: every round leaves its 13 sums in its own slot of one device buffer, which
+    // is read once after the last round; the polynomials and the running claim follow on the
+    // host.  (The reference interleaves a device-to-host copy and a sync with every round.)
+    const uint rounds = (uint)v.size();
+    FrTensor sums(13 * (rounds ? rounds : 1));
+    fr_t* d_v = grape_host::upload(v);
+    FrTensor Bw(B), Tw(T), mw(m);          // phase 2 binds copies; T, B, m of this object stay intact
+    try {
+        uint cur = D;
+        uint k = 0;
+        for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
+            const uint half = cur / 2;
+            fr_t* slot = sums.gpu_data + 13 * (size_t)k;
+            check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(slot), nullptr),
+                  "grape_tlookup_round_sums");
+            if (vi >= (int)logN) {
+                // phase 1: D -> N
+                uint32_t* ptrs[2] = {W(A.gpu_data), W(S.gpu_data)};
+                check(grape_fr_fold_msb_multi(ptrs, 2, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
+            } else {
+                // phase 2: the table variables
+                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(E.gpu_data), half, W(slot + 5), nullptr),
+                      "grape_tlookup_round_sums");
+                check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(slot + 10), nullptr), "grape_tlookup_mb_sums");
+                uint32_t* ptrs[5] = {W(A.gpu_data), W(S.gpu_data), W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
+                check(grape_fr_fold_msb_multi(ptrs, 5, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
+            }
+            A.set_size(half);
+            S.set_size(half);
+            if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
+            cur = half;
+        }
+        std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1));
+        check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * 13 * (size_t)rounds, nullptr), "d2h");
+        grape_free(d_v);
+        d_v = nullptr;
+
+        Fr alpha_run = alpha, alpha_sq_run = alpha_sq;
+        int ui = (int)nu - 1;      // index of the variable bound in this round (u.back())
+        k = 0;
+        for (int vi = (int)rounds - 1; vi >= 0; vi--, ui--, k++) {
+            const Fr* a3 = &h[13 * (size_t)k];
+            const Fr* b3 = a3 + 5;
+            const Fr* c3 = a3 + 10;
+            Polynomial p0({a3[0], a3[1], a3[2]});
+            p0 = p0 * alpha_run;
+            Polynomial p1({a3[3], a3[4]});
+            Polynomial p;
+            if (vi >= (int)logN) {
+                p0 *= Polynomial::eq(u[ui]);
+                p = p0 + p1 + Polynomial(C * two_inv);
+                if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase1: claim != p(0) + p(1)");
+                C = C * two_inv;
+            } else {
+                Fr coef = N_div_D * alpha_sq_run;
+                p0 += Polynomial({b3[0] * coef, b3[1] * coef, b3[2] * coef});
+                Polynomial p2({c3[0], c3[1], c3[2]});
+                p = Polynomial::eq(u[ui]) * p0 + p1 - p2 * N_div_D;
+                if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase2: claim != p(0) + p(1)");
+            }
+            claim = p(v[vi]);
+            last_transcript.rounds.push_back(p);
+            last_transcript.claims.push_back(claim);
+            Fr e = Polynomial::eq(u[ui], v[vi]);
+            alpha_run *= e;
+            if (vi < (int)logN) alpha_sq_run *= e;
+        }
+    } catch (...) {
+        grape_free(d_v);
+        throw;
     }
     return S(0u);
 }

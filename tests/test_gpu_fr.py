@@ -148,6 +148,27 @@ def test_fold_vs_oracle(ops, outer, c, gap):
     assert_same(got, want, "fold")
 
 
+@pytest.mark.parametrize("outer,c,gap", [
+    (1, 16, 1 << 19),        # one thread per output: 2^19 outputs of 16 terms
+    (1, 16, 1 << 18),        # two waves share an output
+    (1, 16, 1 << 17),        # four waves share an output, partial sums meet in LDS
+    (1, 13, 1 << 17),        # ragged last term under a lane predicate
+    (300, 4096, 1),          # many outer slabs, contiguous axis, several passes through scratch
+    (1, 1 << 21, 1),         # a full evaluation: pass, pass, LDS finish
+])
+def test_fold_large_shapes_vs_oracle(ops, outer, c, gap):
+    """shapes large enough to take every pass variant of the fold (the small cases above all
+    run as four waves per output or in the LDS finish kernel)"""
+    n = outer * c * gap
+    t = rand_fr(n, 90 + (c % 97) + (gap % 89))
+    x = rand_fr(br.log2ceil(c) + 1, 91 + (c % 97))
+    dt = ops.to_dev(t)
+    ops.fr_fold(dt, n, ops.to_dev(x), c, 1, gap)
+    got = ops.fr_to_host(dt)[: outer * gap]
+    want = orc.partial_eval(t, n, x, c, 1, gap)[: outer * gap]
+    assert_same(got, want, "fold")
+
+
 def test_fold_full_eval_config3_shape_slice(ops):
     # the two folds of BASELINE config 3 at reduced token/feature counts but the real K = 4096
     # stride: A [N=64][K=4096] over N with id = log2(M), B [M=128][K=4096] over M with id = 0
