@@ -1,4 +1,5 @@
 #include "hyrax.hpp"
+#include <cstdlib>
 #include <cassert>
 #include "../../include/grape_hip.h"
 
@@ -31,6 +32,12 @@ Hyrax_proof& Hyrax_proof::operator=(const Hyrax_proof& o) {
 Hyrax::Hyrax(uint layer_num_, uint npoints_, affine_t* g, bn128& G_, uint com_scale_)
     : com_scale(com_scale_), layer_num(layer_num_), npoints(npoints_ * com_scale_), G(G_), g_affine(g) {
     grape_host::ensure_init();
+    // GRAPE_TABLE_BUDGET_GIB overrides the default budget of the fixed-base tables
+    if (const char* e = std::getenv("GRAPE_TABLE_BUDGET_GIB")) {
+        char* end = nullptr;
+        unsigned long long gib = std::strtoull(e, &end, 10);
+        if (end != e) table_budget_ = (size_t)gib << 30;
+    }
 }
 Hyrax::~Hyrax() {
     grape_free(int16_table_.d);
@@ -84,13 +91,17 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
 }
 
 // Full-width scalars cost ceil(256/c) additions each, so the widest radix whose table fits the
-// budget is used: c = 13 is 20 additions per element against 32 for byte windows.
+// budget is used.  For 4096 generators: c = 14 is 19 additions per element (82 GB, what the
+// default budget allows next to the other tables), c = 13 is 20 (43 GB), c = 15 is 17.5 on average
+// (155 GB; measured no faster than c = 14, its gathers miss more), against 32 plus a doubling
+// chain for the reference's byte windows.
 bool Hyrax::ensure_fr_table(uint rowlen) {
     if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
     size_t used = 0;
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
     if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
-    for (uint c = 13; c >= 8; c--) {
+    // ceil(256 / c) windows: the top signed digit of a 255-bit scalar may carry into one more
+    for (uint c = 15; c >= 8; c--) {
         uint nw = (256 + c - 1) / c, K = 1u << (c - 1);
         if (used + grape_g1_wide_table_bytes(rowlen, nw, K) <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }

@@ -68,5 +68,5 @@ private:
     WideTable int16_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;
     size_t scaled_bytes_ = 0;
-    size_t table_budget_ = (size_t)96 << 30;
+    size_t table_budget_ = (size_t)128 << 30;
 };
