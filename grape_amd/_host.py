@@ -10,7 +10,8 @@ _lib = None
 NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
          "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
-         "grape_host_fr_op", "grape_host_g1_mul_generator"]
+         "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
+         "grape_host_generate_data"]
 
 
 class HostError(RuntimeError):
@@ -31,6 +32,11 @@ def load():
         lib.grape_host_seed.argtypes = [ctypes.c_uint64]
         lib.grape_host_last_prove_seconds.restype = ctypes.c_double
         lib.grape_host_last_commit_seconds.restype = ctypes.c_double
+        lib.grape_host_findsize.restype = ctypes.c_ulong
+        lib.grape_host_findsize.argtypes = [ctypes.c_char_p]
+        lib.grape_host_bin_io.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        lib.grape_host_load_data.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_uint32)]
+        lib.grape_host_generate_data.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint32]
         _lib = lib
     return _lib
 
@@ -190,3 +196,29 @@ def g1_mul_generator(k_mont):
     out = np.zeros(12, dtype=np.uint64)
     _check(lib.grape_host_g1_mul_generator(_hp(k), _hp(out)))
     return out
+
+
+# ------------------------------------------------------------------ file helpers (ioutils.hpp)
+def savebin(filename, ptr, size, is_gpu=True):
+    _check(load().grape_host_bin_io(0, os.fsencode(filename), ctypes.c_void_p(ptr), size, 1 if is_gpu else 0))
+
+
+def loadbin(filename, ptr, size, is_gpu=True):
+    _check(load().grape_host_bin_io(1, os.fsencode(filename), ctypes.c_void_p(ptr), size, 1 if is_gpu else 0))
+
+
+def findsize(filename):
+    return load().grape_host_findsize(os.fsencode(filename))
+
+
+def load_data(filename):
+    """int32 file -> (device pointer, element count); release the pointer with grape_free"""
+    p, n = ctypes.c_void_p(0), ctypes.c_uint32(0)
+    _check(load().grape_host_load_data(os.fsencode(filename), ctypes.byref(p), ctypes.byref(n)))
+    return p.value, n.value
+
+
+def generate_data(size):
+    p = ctypes.c_void_p(0)
+    _check(load().grape_host_generate_data(ctypes.byref(p), size))
+    return p.value

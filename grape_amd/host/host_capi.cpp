@@ -1,4 +1,5 @@
 #include "host_capi.h"
+#include "ioutils.hpp"
 #include <cstring>
 #include <string>
 #include "../../include/grape_hip.h"
@@ -280,6 +281,28 @@ int grape_host_g1_mul_generator(const uint32_t* k_mont, uint32_t* out_affine) {
     bn128 p = fr_from(k_mont) * bn128::one();
     affine_t a = p.to_affine();
     std::memcpy(out_affine, &a, sizeof a);
+    GUARD_END
+}
+
+int grape_host_bin_io(int op, const char* filename, void* ptr, size_t size, int is_gpu) {
+    GUARD_BEGIN
+    if (op == 0) savebin(filename, ptr, size, is_gpu != 0);
+    else loadbin(filename, ptr, size, is_gpu != 0);
+    GUARD_END
+}
+unsigned long grape_host_findsize(const char* filename) { return findsize(filename); }
+int grape_host_load_data(const char* filename, int32_t** d_out, uint32_t* n) {
+    GUARD_BEGIN
+    int* p = nullptr;
+    *n = load_data(filename, &p);
+    *d_out = p;
+    GUARD_END
+}
+int grape_host_generate_data(int32_t** d_out, uint32_t size) {
+    GUARD_BEGIN
+    int* p = nullptr;
+    generate_data(&p, size);
+    *d_out = p;
     GUARD_END
 }
 

@@ -72,6 +72,14 @@ int grape_host_fr_op(int op, const uint32_t *a, const uint32_t *b, uint32_t *out
 /* k * G as a host computation (affine out) */
 int grape_host_g1_mul_generator(const uint32_t *k_mont, uint32_t *out_affine);
 
+/* File helpers (ioutils.hpp): op 0 = savebin, 1 = loadbin of `size` bytes at ptr (device memory
+ * when is_gpu != 0); findsize; load_data into a fresh device buffer (*d_out, *n elements);
+ * generate_data (std::mt19937(123456) int32) into a fresh device buffer. */
+int grape_host_bin_io(int op, const char *filename, void *ptr, size_t size, int is_gpu);
+unsigned long grape_host_findsize(const char *filename);
+int grape_host_load_data(const char *filename, int32_t **d_out, uint32_t *n);
+int grape_host_generate_data(int32_t **d_out, uint32_t size);
+
 #ifdef __cplusplus
 }
 #endif

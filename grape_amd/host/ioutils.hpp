@@ -1,0 +1,26 @@
+// File helpers of the reference's drivers (include/ioutils.cuh:52-64, src/ioutils.cu:3-160): raw
+// little-endian dumps of device or host buffers.  The formats are the reference's own:
+//   * int tensors  (data/{W,Q,R}/*.bin): int32, row-major;
+//   * Fr tensors:  fr_t[n], 32 bytes each, Montgomery form;
+//   * points.bin:  affine_t[256 * npoints], entry w * npoints + i = w * G_i, 96 bytes each;
+//   * commitments: jacob_t[rows], 144 bytes each.
+// (Files written for BN254 by the reference are not interchangeable with this BLS12-381 build.)
+#pragma once
+#include <string>
+
+typedef unsigned int uint;
+typedef unsigned long ulong;
+
+// writes `size` bytes; device memory is staged through the host.  Errors are reported on stderr
+// and the call returns, as in the reference.
+void savebin(const std::string& filename, const void* data, size_t size, bool is_gpu_data = true);
+// file size in bytes, 0 when the file cannot be read
+ulong findsize(const std::string& filename);
+// reads exactly `size` bytes into device (default) or host memory
+void loadbin(const std::string& filename, void* data, size_t size, bool is_gpu_data = true);
+// whole file of int32 into a fresh device buffer (an old *gpu_ptr is released first); returns the
+// element count.  A missing file throws std::runtime_error (the reference calls exit(1)).
+uint load_data(const std::string& filename, int** gpu_ptr);
+uint load_data(const std::string& filename, int** gpu_ptr, int** cpu_ptr);
+// `size` uniformly distributed int32 from std::mt19937(123456) into a fresh device buffer
+void generate_data(int** out_ptr, uint size);

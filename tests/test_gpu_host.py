@@ -261,3 +261,51 @@ def test_elemul_and_combine_claims_invariants(ops, host):
                                   np.stack([br.fr_pack(uj) for uj in us]), br.fr_pack(vv))
     assert tr.shape[0] == 4
     assert br.fr_unpack(res)[0] == br.mle_eval(X, vv)
+
+
+def test_file_helpers_and_on_disk_formats(ops, host, gens, tmp_path):
+    """the reference's on-disk artefacts through savebin / loadbin / load_data: an int32 weight
+    dump (data/W/*.bin), the generator table points.bin (256 x npoints affine points, entry
+    w*npoints + i = w*G_i) and an Fr tensor dump; a table read back from disk commits to the same
+    points as the oracle"""
+    import torch
+    from grape_amd import _capi
+    hg, dg = gens
+    npoints = 256
+    table = ops.g1_table_gen(dg, 256)
+    ops.sync()
+    f_pts = str(tmp_path / "points.bin")
+    host.savebin(f_pts, table.data_ptr(), table.numel() * 4)
+    assert host.findsize(f_pts) == 256 * npoints * 96
+    assert np.array_equal(np.fromfile(f_pts, dtype=np.uint64).reshape(-1, 12), orc.g1_table(hg, 256))
+    table2 = torch.zeros_like(table)
+    host.loadbin(f_pts, table2.data_ptr(), table2.numel() * 4)
+    assert torch.equal(table, table2)
+    # int32 weights: written by numpy as the reference's Python side does, read by load_data
+    W = gaussian_i16((8, 256), 71)
+    f_w = str(tmp_path / "w.bin")
+    W.astype("<i4").tofile(f_w)
+    ptr, n = host.load_data(f_w)
+    assert n == W.size
+    dW = torch.empty(W.size, dtype=torch.int32, device="cuda")
+    lib = _capi.load()
+    _capi.check(lib.grape_memcpy_d2d(dW.data_ptr(), ptr, W.size * 4, None))
+    _capi.check(lib.grape_stream_sync(None))
+    _capi.check(lib.grape_free(ptr))
+    assert np.array_equal(dW.cpu().numpy().reshape(W.shape), W)
+    got = host.hyrax_commit_i32(dW, W.size, 16, table2, npoints, com_scale=16)
+    assert_same(got, orc.commit_i32(W, orc.g1_table(hg, 256), 256, npoints), "commit from on-disk table and weights")
+    # Fr tensor dump: 32-byte Montgomery elements
+    s = rand_fr(100, 72)
+    ds = ops.to_dev(s)
+    f_fr = str(tmp_path / "fr.bin")
+    host.savebin(f_fr, ds.data_ptr(), 100 * 32)
+    assert np.array_equal(np.fromfile(f_fr, dtype=np.uint64).reshape(-1, 4), s)
+    # generate_data: deterministic, full int32 range
+    p1, p2 = host.generate_data(4096), host.generate_data(4096)
+    a, b = torch.empty(4096, dtype=torch.int32, device="cuda"), torch.empty(4096, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_memcpy_d2d(a.data_ptr(), p1, 4096 * 4, None))
+    _capi.check(lib.grape_memcpy_d2d(b.data_ptr(), p2, 4096 * 4, None))
+    _capi.check(lib.grape_stream_sync(None))
+    _capi.check(lib.grape_free(p1)); _capi.check(lib.grape_free(p2))
+    assert torch.equal(a, b) and a.min().item() < -2**30 and a.max().item() > 2**30

@@ -31,3 +31,21 @@ def test_host_g1_scalar_mul_vs_textbook():
     for k in (0, 1, 2, 12345678901234567890, br.R_MOD - 1):
         got = br.g1_unpack(_host.g1_mul_generator(br.fr_pack([k])))[0]
         assert got == br.g1_mul(k, br.G1)
+
+
+def test_file_helpers_on_host_memory(tmp_path):
+    """savebin / loadbin / findsize with host buffers (src/ioutils.cu:3-103): raw bytes, a short
+    file leaves the destination untouched, a missing file is size 0"""
+    from grape_amd import _host
+    a = np.arange(1000, dtype=np.int32) * 7 - 3
+    f = str(tmp_path / "t.bin")
+    _host.savebin(f, a.ctypes.data, a.nbytes, is_gpu=False)
+    assert _host.findsize(f) == a.nbytes
+    assert np.array_equal(np.fromfile(f, dtype=np.int32), a)
+    b = np.zeros_like(a)
+    _host.loadbin(f, b.ctypes.data, b.nbytes, is_gpu=False)
+    assert np.array_equal(a, b)
+    c = np.full(2000, -1, dtype=np.int32)
+    _host.loadbin(f, c.ctypes.data, c.nbytes, is_gpu=False)      # asks for more than the file holds
+    assert (c == -1).all()
+    assert _host.findsize(str(tmp_path / "absent.bin")) == 0
