@@ -14,6 +14,9 @@
  *                      incl. non-power-of-two extents                       (test_oracle_fold.py)
  *   sumcheck ......... brute-force round polynomials p(0),p(1),p(2);
  *                      first claim = Y(u) of an exact integer matmul        (test_oracle_sumcheck.py)
+ *   eleMul, claims ... brute-force round polynomials at t = 0..3, returned
+ *                      values = multilinear extensions at v                 (test_oracle_elemul.py)
+ *   all of the above . known-answer vectors written from the definitions    (test_golden.py)
  *   logUp ............ numpy.bincount; sum A = sum m*B; S(v) by brute force (test_oracle_tlookup.py)
  *
  * Citations are to files under the reference's root.
@@ -826,6 +829,146 @@ int orc_prove_matmul(u64 *A, u64 *B, uint32_t L, uint32_t N, uint32_t M, uint32_
     free(a);
     free(b);
     free(c);
+    return status;
+}
+
+/* sumcheck_kernel (one tensor) src/prove.cu:14-27 */
+static void sumcheck_round1(u64 *X, u64 *a, u64 *b, uint32_t in_size, uint32_t out_size, const u64 *v) {
+    for (uint32_t g = 0; g < out_size; g++) {
+        u64 Xa[4], Xb[4], t[4];
+        fr_cpy(Xb, X + 4 * (uint64_t)g);
+        if ((uint64_t)g + out_size < in_size) fr_sub(Xa, X + 4 * ((uint64_t)g + out_size), Xb);
+        else fr_neg(Xa, Xb);
+        fr_mul(t, Xa, v);
+        fr_add(X + 4 * (uint64_t)g, t, Xb);
+        fr_cpy(b + 4 * (uint64_t)g, Xb);
+        fr_cpy(a + 4 * (uint64_t)g, Xa);
+    }
+}
+
+/* prove_eleMul src/prove.cu:212-243 with eleMul_sumcheck :119-172.  A, B: L*M*N elements, are
+ * folded in place.  Status 1: a round check failed, 3: final product check failed, 4: first_size
+ * (= L*M) is not a power of two (the reference throws). */
+int orc_prove_elemul(u64 *A, u64 *B, uint32_t L, uint32_t M, uint32_t N, const u64 *u, uint32_t nu,
+                     const u64 *v, uint32_t nv, u64 *claim, u64 *transcript, uint32_t *n_rounds,
+                     u64 *A_claim, u64 *B_claim) {
+    (void)nu;
+    (void)nv;
+    const uint32_t size = L * M * N, first_size = L * M;
+    *n_rounds = 0;
+    if ((1u << orc_log2(first_size)) != first_size) return 4;
+    const u64 *uend = u + 4 * orc_log2(L * N * M);
+    const u64 *vend = v + 4 * orc_log2(L * M * N);
+    const uint32_t second_size = size / first_size;
+    const uint32_t rounds = orc_log2(size);
+    uint32_t in = size, out = size / 2;
+    uint64_t cap = size / 2 ? size / 2 : 1;
+    u64 *a = malloc(32 * cap), *b = malloc(32 * cap), *c = malloc(32 * cap);
+    u64 eq_acc[4];
+    fr_cpy(eq_acc, FR_ONE);
+    int status = 0;
+    for (uint32_t i = 0; i < rounds; i++) {
+        const u64 *v_now = vend - 4 * (i + 1);
+        const u64 *u_now = uend - 4 * (i + 1);
+        orc_sumcheck_round2(A, B, a, b, c, in, out, v_now);
+        u64 *arr[3] = {a, b, c};
+        for (int k = 0; k < 3; k++) {
+            if (in > second_size) {
+                orc_fr_partial_eval(arr[k], out, uend - 4 * orc_log2(first_size), out / second_size, 0, second_size);
+                orc_fr_partial_eval(arr[k], second_size, uend - 4 * orc_log2(size), second_size, 0, 1);
+            } else {
+                orc_fr_partial_eval(arr[k], out, uend - 4 * orc_log2(size), out, 0, 1);
+            }
+        }
+        poly_t p, e;
+        poly_zero(&p, 2);
+        fr_cpy(p.c[0], c);
+        fr_cpy(p.c[1], b);
+        fr_cpy(p.c[2], a);
+        poly_eq(&e, u_now);
+        poly_scale(&e, eq_acc);
+        poly_mul(&p, &p, &e);
+        transcript_put(transcript, i, &p);
+        u64 s[4], t[4];
+        poly_eval01sum(s, &p);
+        if (!fr_eq(s, claim) && !status) status = 1;
+        poly_eval(claim, &p, v_now);
+        in = out;
+        out = (out == second_size) ? (1u << (orc_log2(out) - 1)) : out / 2;
+        eq2(t, u_now, v_now);
+        fr_mul(eq_acc, eq_acc, t);
+    }
+    *n_rounds = rounds;
+    fr_cpy(A_claim, A);
+    fr_cpy(B_claim, B);
+    u64 t[4];
+    fr_mul(t, A_claim, B_claim);
+    fr_mul(t, t, eq_acc);
+    if (!fr_eq(t, claim) && !status) status = 3;
+    free(a);
+    free(b);
+    free(c);
+    return status;
+}
+
+/* combine_claims src/prove.cu:245-301: merges `num` claims X(u_j) = claims[j] into one claim
+ * X(v).  u holds num rows of nv challenges.  Returns X(v) in ret and every round polynomial
+ * (degree 2) in transcript.  Status 1: a round check failed, 3: the final check failed. */
+int orc_combine_claims(u64 *X, uint32_t size, const u64 *claims, uint32_t num, const u64 *u,
+                       const u64 *v, uint32_t nv, u64 *transcript, u64 *ret) {
+    u64 claim[4];
+    fr_zero(claim);
+    for (uint32_t j = 0; j < num; j++) fr_add(claim, claim, claims + 4 * j);
+    uint64_t cap = size / 2 ? size / 2 : 1;
+    u64 *a = malloc(32 * cap), *b = malloc(32 * cap), *ta = malloc(32 * cap), *tb = malloc(32 * cap);
+    u64 *eq_acc = malloc(32 * (size_t)(num ? num : 1));
+    for (uint32_t j = 0; j < num; j++) fr_cpy(eq_acc + 4 * j, FR_ONE);
+    uint32_t in = size, out = size / 2;
+    int status = 0;
+    for (uint32_t i = 0; i < nv; i++) {
+        const uint32_t left = nv - 1 - i;          /* challenges still unbound after this round */
+        const u64 *v_now = v + 4 * left;           /* new_v.back() */
+        sumcheck_round1(X, a, b, in, out, v_now);
+        poly_t p;
+        poly_zero(&p, 2);
+        for (uint32_t j = 0; j < num; j++) {
+            const u64 *uj = u + 4 * (uint64_t)j * nv;
+            const u64 *now_u = uj + 4 * left;      /* new_u[j].back() */
+            memcpy(ta, a, 32 * (size_t)out);
+            memcpy(tb, b, 32 * (size_t)out);
+            poly_t p1, e;
+            poly_zero(&p1, 1);
+            orc_fr_mle_eval(p1.c[0], tb, out, uj, left);
+            orc_fr_mle_eval(p1.c[1], ta, out, uj, left);
+            poly_eq(&e, now_u);
+            poly_mul(&p1, &p1, &e);
+            poly_scale(&p1, eq_acc + 4 * j);
+            poly_add(&p, &p, &p1);
+            u64 t[4];
+            eq2(t, now_u, v_now);
+            fr_mul(eq_acc + 4 * j, eq_acc + 4 * j, t);
+        }
+        transcript_put(transcript, i, &p);
+        u64 s[4];
+        poly_eval01sum(s, &p);
+        if (!fr_eq(s, claim) && !status) status = 1;
+        poly_eval(claim, &p, v_now);
+        in = out;
+        out = out / 2;
+    }
+    fr_cpy(ret, X);
+    u64 sum[4], t[4];
+    fr_zero(sum);
+    for (uint32_t j = 0; j < num; j++) {
+        fr_mul(t, eq_acc + 4 * j, ret);
+        fr_add(sum, sum, t);
+    }
+    if (!fr_eq(sum, claim) && !status) status = 3;
+    free(a);
+    free(b);
+    free(ta);
+    free(tb);
+    free(eq_acc);
     return status;
 }
 

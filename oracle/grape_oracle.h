@@ -99,6 +99,21 @@ int orc_prove_matmul(uint64_t *A, uint64_t *B, uint32_t L, uint32_t N, uint32_t 
                      uint64_t *claim, uint64_t *transcript, uint32_t *n_rounds,
                      uint64_t *A_claim, uint64_t *B_claim);
 
+/*
+ * prove_eleMul (src/prove.cu:212-243, eleMul_sumcheck :119-172).  A, B: L*M*N elements, consumed.
+ * Transcript as above (degree 3).  Returns 0, 1 (round check), 3 (final check) or 4 (L*M is not
+ * a power of two).
+ */
+int orc_prove_elemul(uint64_t *A, uint64_t *B, uint32_t L, uint32_t M, uint32_t N, const uint64_t *u,
+                     uint32_t nu, const uint64_t *v, uint32_t nv, uint64_t *claim, uint64_t *transcript,
+                     uint32_t *n_rounds, uint64_t *A_claim, uint64_t *B_claim);
+/*
+ * combine_claims (src/prove.cu:245-301): u holds num rows of nv challenges; X (size = 2^nv
+ * elements) is consumed; ret receives X(v).  Returns 0, 1 (round check) or 3 (final check).
+ */
+int orc_combine_claims(uint64_t *X, uint32_t size, const uint64_t *claims, uint32_t num, const uint64_t *u,
+                       const uint64_t *v, uint32_t nv, uint64_t *transcript, uint64_t *ret);
+
 /* ---- tlookup / logUp ---- */
 void orc_histogram(uint32_t *hist, const uint64_t *vals_mont, uint64_t n, int32_t low, uint32_t len);
 void orc_tlookup_prep(uint64_t *m_mont, const uint64_t *vals_mont, uint64_t n, int32_t low,

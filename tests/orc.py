@@ -201,6 +201,34 @@ def prove_matmul(A, B, L, N, M, K, u, v, claim):
     return st, tr[: nr.value].copy(), claim, ac, bc
 
 
+def prove_elemul(A, B, L, M, N, u, v, claim):
+    """returns (status, transcript[rounds,4,4], final_claim, A_claim, B_claim)."""
+    A = np.array(A, dtype=np.uint64).reshape(-1, 4)
+    B = np.array(B, dtype=np.uint64).reshape(-1, 4)
+    u = np.ascontiguousarray(u, dtype=np.uint64).reshape(-1, 4)
+    v = np.ascontiguousarray(v, dtype=np.uint64).reshape(-1, 4)
+    claim = np.array(claim, dtype=np.uint64).reshape(4)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    ac = np.zeros(4, dtype=np.uint64)
+    bc = np.zeros(4, dtype=np.uint64)
+    st = lib().orc_prove_elemul(P(A), P(B), c32(L), c32(M), c32(N), P(u), c32(u.shape[0]), P(v), c32(v.shape[0]),
+                                P(claim), P(tr), ctypes.byref(nr), P(ac), P(bc))
+    return st, tr[: nr.value].copy(), claim, ac, bc
+
+
+def combine_claims(X, claims, u_rows, v):
+    """returns (status, transcript[nv,4,4], X(v))."""
+    X = np.array(X, dtype=np.uint64).reshape(-1, 4)
+    claims = np.ascontiguousarray(claims, dtype=np.uint64).reshape(-1, 4)
+    v = np.ascontiguousarray(v, dtype=np.uint64).reshape(-1, 4)
+    u = np.ascontiguousarray(u_rows, dtype=np.uint64).reshape(claims.shape[0], v.shape[0], 4)
+    tr = np.zeros((max(v.shape[0], 1), 4, 4), dtype=np.uint64)
+    ret = np.zeros(4, dtype=np.uint64)
+    st = lib().orc_combine_claims(P(X), c32(X.shape[0]), P(claims), c32(claims.shape[0]), P(u), P(v), c32(v.shape[0]), P(tr), P(ret))
+    return st, tr[: v.shape[0]].copy(), ret
+
+
 def histogram(vals_mont, low, length):
     v = np.ascontiguousarray(vals_mont, dtype=np.uint64).reshape(-1, 4)
     h = np.zeros(length, dtype=np.uint32)

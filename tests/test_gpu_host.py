@@ -238,29 +238,41 @@ def test_hyrax_open_and_verify(ops, host, gens):
     assert_same(res, orc.mle_eval(t, pt), "opened value = T(point)")
 
 
-def test_elemul_and_combine_claims_invariants(ops, host):
-    # no oracle restatement exists for these two; they are checked against the definition:
-    # the returned evaluations are the multilinear extensions at v and the claim chain closes
-    rng = random.Random(81)
-    L, M, N = 1, 4, 8
+@pytest.mark.parametrize("L,M,N", [(1, 4, 8), (2, 2, 4), (1, 4, 6), (2, 1, 5), (1, 32, 64), (1, 2, 1)])
+def test_prove_elemul_vs_oracle(ops, host, L, M, N):
+    rng = random.Random(81 + L + M + N)
     n = L * M * N
+    Np = 1 << br.log2ceil(N)
+    k = br.log2ceil(n)
     A = [rng.randrange(R) for _ in range(n)]
     B = [rng.randrange(R) for _ in range(n)]
-    u = [rng.randrange(R) for _ in range(5)]
-    v = [rng.randrange(R) for _ in range(5)]
-    claim0 = sum(br.eq_weight(i, u) * A[i] * B[i] for i in range(n)) % R
-    tr, claim, ac, bc = host.prove_elemul(ops.to_dev(br.fr_pack(A)), ops.to_dev(br.fr_pack(B)), L, M, N, br.fr_pack(u), br.fr_pack(v),
-                                          br.fr_pack([claim0])[0])
-    assert tr.shape[0] == 5
-    assert br.fr_unpack(ac)[0] == br.mle_eval(A, v) and br.fr_unpack(bc)[0] == br.mle_eval(B, v)
-    X = [rng.randrange(R) for _ in range(16)]
-    us = [[rng.randrange(R) for _ in range(4)] for _ in range(3)]
-    vv = [rng.randrange(R) for _ in range(4)]
-    claims = [br.mle_eval(X, uj) for uj in us]
-    tr, res = host.combine_claims(ops.to_dev(br.fr_pack(X)), 16, br.fr_pack(claims),
-                                  np.stack([br.fr_pack(uj) for uj in us]), br.fr_pack(vv))
-    assert tr.shape[0] == 4
-    assert br.fr_unpack(res)[0] == br.mle_eval(X, vv)
+    u = [rng.randrange(R) for _ in range(k)]
+    v = [rng.randrange(R) for _ in range(k)]
+    pad = lambda X: [X[f * N + j] if j < N else 0 for f in range(L * M) for j in range(Np)]
+    claim0 = sum(br.eq_weight(i, u) * a * b for i, (a, b) in enumerate(zip(pad(A), pad(B)))) % R
+    pA, pB, pu, pv, pc = br.fr_pack(A), br.fr_pack(B), br.fr_pack(u), br.fr_pack(v), br.fr_pack([claim0])[0]
+    st, wtr, wclaim, wac, wbc = orc.prove_elemul(pA, pB, L, M, N, pu, pv, pc)
+    assert st == 0
+    tr, claim, ac, bc = host.prove_elemul(ops.to_dev(pA), ops.to_dev(pB), L, M, N, pu, pv, pc)
+    assert_same(tr, wtr, "round polynomials")
+    assert_same(claim, wclaim, "final claim")
+    assert_same(ac, wac, "A(v)")
+    assert_same(bc, wbc, "B(v)")
+    with pytest.raises(host.HostError, match="claim != p\\(0\\) \\+ p\\(1\\)"):
+        host.prove_elemul(ops.to_dev(pA), ops.to_dev(pB), L, M, N, pu, pv, br.fr_pack([claim0 + 1])[0])
+
+
+@pytest.mark.parametrize("nv,num", [(4, 3), (3, 1), (1, 2), (10, 4)])
+def test_combine_claims_vs_oracle(ops, host, nv, num):
+    X = rand_fr(1 << nv, 90 + nv)
+    us = [rand_fr(nv, 91 + nv + j) for j in range(num)]
+    vv = rand_fr(nv, 99 + nv)
+    claims = np.stack([orc.partial_eval(X, 1 << nv, uj, 1 << nv, 0, 1)[0] for uj in us])
+    st, wtr, wret = orc.combine_claims(X, claims, us, vv)
+    assert st == 0
+    tr, res = host.combine_claims(ops.to_dev(X), 1 << nv, claims, np.stack(us), vv)
+    assert_same(tr, wtr, "round polynomials")
+    assert_same(res, wret, "X(v)")
 
 
 def test_file_helpers_and_on_disk_formats(ops, host, gens, tmp_path):
