@@ -172,6 +172,15 @@ GRAPE_HD Limbs canon_wide(const Limbs& t) {
     return canon(normalize(d), 1);
 }
 
+// limb-wise sum of at most 16 packed elements or differences of packed elements (|limb| < 2^30,
+// value within (-add_r * r, (32 - add_r) * r)) -> canonical element of memory form
+GRAPE_HD Fr limb_sum_to_fr(const Limbs& s, int add_r) {
+    Limbs d;
+#pragma unroll
+    for (int i = 0; i < N; i++) d.v[i] = s.v[i] + add_r * R(i);
+    return unpack(canon_wide(normalize(d)));
+}
+
 // canonical product of two memory-form elements (memory form out): 16ab < 16 r^2 -> (0, 1.46r)
 GRAPE_HD Fr mulc(const Fr& a, const Fr& b) {
     Acc C;

@@ -28,9 +28,9 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t
     __shared__ Fr lds[3 * (kBlock / 64)];
     const Fr vv = ld_fr(v, 0);
     const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
-    fr26::Acc C0, C1, C2;
+    fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
-    fr26::acc_zero(C1);
+    fr26::acc_zero(Q);
     fr26::acc_zero(C2);
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < out_size; g += stride) {
@@ -44,23 +44,26 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t
             fr26::Acc T;
             fr26::acc_zero(T);
             fr26::mac(T, a0, b0);
-            st_fr(cc, g, fr26::finish_sum(T, 0));
-            fr26::acc_zero(T);
-            fr26::mac(T, da, b0);
-            fr26::mac(T, a0, db);
-            st_fr(cb, g, fr26::finish_sum(T, 1));
+            const Fr c_ = fr26::finish_sum(T, 0);
             fr26::acc_zero(T);
             fr26::mac(T, da, db);
-            st_fr(ca, g, fr26::finish_sum(T, 1));
+            const Fr a_ = fr26::finish_sum(T, 1);
+            fr26::acc_zero(T);
+            fr26::mac(T, a1, b1);
+            st_fr(cc, g, c_);
+            st_fr(cb, g, sub(sub(fr26::finish_sum(T, 0), c_), a_));
+            st_fr(ca, g, a_);
         }
+        // middle coefficient by Karatsuba: da*b0 + a0*db = a1*b1 - a0*b0 - da*db, so the value at
+        // t = 1 is accumulated with one product instead of two
         fr26::mac(C0, a0, b0);
-        fr26::mac(C1, da, b0);
-        fr26::mac(C1, a0, db);
+        fr26::mac(Q, a1, b1);
         fr26::mac(C2, da, db);
     }
     if (partial) {
-        // |sum| < 16 * 2 r^2 -> within (-0.91 r, 1.91 r) after reduction
-        Fr acc[3] = {fr26::finish_sum(C0, 2), fr26::finish_sum(C1, 2), fr26::finish_sum(C2, 2)};
+        // |sum| < 16 r^2 -> within (-0.46 r, 1.46 r) after reduction
+        const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2), q1 = fr26::finish_sum(Q, 2);
+        Fr acc[3] = {c0, sub(sub(q1, c0), c2), c2};
         block_sum<3>(acc, lds);
         if (threadIdx.x == 0) {
             st_fr(partial, (size_t)blockIdx.x * 3 + 0, acc[0]);
@@ -214,40 +217,48 @@ __global__ void __launch_bounds__(kBlock) tl_poly_sum_kernel(const uint32_t* A, 
 // 5 sums per round: eq-weighted coefficients of (A0+tA1)(S0+beta+tS1), and plain sums of A0, A1.
 // e*A0 and e*A1 are reduced products; the three second-level products are accumulated
 // double-width over the thread's iterations and reduced once.
-__global__ void __launch_bounds__(kBlock) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
+__global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
                                                           const uint32_t* eq, size_t n_out, uint32_t* partial) {
     __shared__ Fr lds[5 * (kBlock / 64)];
     const Fr btc = beta ? ld_fr(beta, 0) : Fr::zero();
     const fr26::Limbs bt = fr26::pack(btc);
-    fr26::Acc C0, C1, C2;
+    fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
-    fr26::acc_zero(C1);
+    fr26::acc_zero(Q);
     fr26::acc_zero(C2);
-    Fr sa0 = Fr::zero(), sa1 = Fr::zero();
+    // plain sums of A's halves as limb-wise sums (no carries: 16 terms of 26-bit limbs)
+    fr26::Limbs sa0, sa1;
+#pragma unroll
+    for (int k = 0; k < fr26::N; k++) sa0.v[k] = sa1.v[k] = 0;
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
-        const Fr a0c = ld_fr(A, t), a1c = ld_fr(A, t + n_out);
-        const fr26::Limbs a0 = fr26::pack(a0c), a1 = fr26::pack(a1c);
-        const fr26::Limbs s0r = ld_l26(S, t);
-        const fr26::Limbs s0 = fr26::add(s0r, bt);                   // value < 2r, limbs < 2^27
-        const fr26::Limbs s1 = fr26::sub(ld_l26(S, t + n_out), s0r);   // signed
+        // operands are consumed as early as possible so that few of them are live beside the
+        // three double-width accumulators
         const fr26::Limbs e16 = fr26::pack16(ld_fr(eq, t));         // limbs < 2^30: one product per column set
+        const fr26::Limbs a0 = ld_l26(A, t);
+        const fr26::Limbs s0r = ld_l26(S, t);
+        const fr26::Limbs s1 = fr26::sub(ld_l26(S, t + n_out), s0r);   // signed
+        const fr26::Limbs s0 = fr26::add(s0r, bt);                   // value < 2r, limbs < 2^27
         fr26::Acc T;
         fr26::acc_zero(T);
         fr26::mac(T, e16, a0);
         const fr26::Limbs ea0 = fr26::reduce(T, 0);                  // (0, 1.46 r)
-        fr26::acc_zero(T);
-        fr26::mac(T, e16, fr26::sub(a1, a0));
-        const fr26::Limbs ea1 = fr26::reduce(T, 1);                  // (0.54 r, 2.46 r)
         fr26::mac(C0, ea0, s0);
-        fr26::mac(C1, ea1, s0);
-        fr26::mac(C1, ea0, s1);
+        const fr26::Limbs d1 = fr26::sub(ld_l26(A, t + n_out), a0);  // a1 - a0, signed
+        sa0 = fr26::add(sa0, a0);
+        sa1 = fr26::add(sa1, d1);
+        fr26::acc_zero(T);
+        fr26::mac(T, e16, d1);
+        const fr26::Limbs ea1 = fr26::reduce(T, 1);                  // e*(a1-a0) in (0.54 r, 2.46 r)
         fr26::mac(C2, ea1, s1);
-        sa0 = add(sa0, a0c);
-        sa1 = add(sa1, sub(a1c, a0c));
+        // middle coefficient by Karatsuba: e*a0*s1 + e*(a1-a0)*s0 = (e*a1)*(s0+s1) - c0 - c2,
+        // so Q accumulates the value at t = 1 with one product instead of two
+        fr26::mac(Q, fr26::add(ea0, ea1), fr26::add(s0, s1));        // (0.54 r, 3.92 r) * (-r, 3r)
     }
-    // per iteration |C1| grows by at most (2.46*2 + 1.46) r^2; 16 iterations -> below 103 r^2 -> 2.9 r
-    Fr acc[5] = {fr26::finish_sum(C0, 4), fr26::finish_sum(C1, 4), fr26::finish_sum(C2, 4), sa0, sa1};
+    // per iteration |Q| grows by at most 3.92 * 3 r^2 = 11.8 r^2; 16 iterations -> below 189 r^2,
+    // i.e. within 5.4 r of zero after the reduction: finish_sum's window of 34 r holds with lo_r = 6
+    const Fr c0 = fr26::finish_sum(C0, 4), c2 = fr26::finish_sum(C2, 4), q1 = fr26::finish_sum(Q, 6);
+    Fr acc[5] = {c0, sub(sub(q1, c0), c2), c2, fr26::limb_sum_to_fr(sa0, 0), fr26::limb_sum_to_fr(sa1, 16)};
     block_sum<5>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
@@ -257,20 +268,21 @@ __global__ void __launch_bounds__(kBlock) tl_round_kernel(const uint32_t* A, con
 
 __global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
-    fr26::Acc C0, C1, C2;
+    fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
-    fr26::acc_zero(C1);
+    fr26::acc_zero(Q);
     fr26::acc_zero(C2);
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
         const fr26::Limbs m0 = ld_l26(m, t), b0 = ld_l26(B, t);
-        const fr26::Limbs m1 = fr26::sub(ld_l26(m, t + n_out), m0), b1 = fr26::sub(ld_l26(B, t + n_out), b0);
+        const fr26::Limbs mh = ld_l26(m, t + n_out), bh = ld_l26(B, t + n_out);
+        const fr26::Limbs m1 = fr26::sub(mh, m0), b1 = fr26::sub(bh, b0);
         fr26::mac(C0, m0, b0);
-        fr26::mac(C1, m1, b0);
-        fr26::mac(C1, m0, b1);
+        fr26::mac(Q, mh, bh);             // value at t = 1; the middle coefficient is Q - C0 - C2
         fr26::mac(C2, m1, b1);
     }
-    Fr acc[3] = {fr26::finish_sum(C0, 2), fr26::finish_sum(C1, 2), fr26::finish_sum(C2, 2)};
+    const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2), q1 = fr26::finish_sum(Q, 2);
+    Fr acc[3] = {c0, sub(sub(q1, c0), c2), c2};
     block_sum<3>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
