@@ -73,6 +73,41 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t
     }
 }
 
+// The last rounds of a two-tensor sumcheck in ONE launch: once a round has at most kBlock output
+// indices, one workgroup runs all remaining rounds back to back (a barrier between rounds
+// instead of a launch and a finishing kernel per round).  Round i takes its challenge from
+// v_end[-(i+1)] and leaves its three sums in sums[3i .. 3i+2].
+__global__ void __launch_bounds__(kBlock) sumcheck2_tail_kernel(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t rounds,
+                                                                const uint32_t* v_end, uint32_t* sums) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    uint32_t in = in_size;
+    uint32_t out = 1;
+    while (2 * out < in) out *= 2;                    // 2^(ceil(log2 in) - 1), at most kBlock
+    const uint32_t g = threadIdx.x;
+    for (uint32_t i = 0; i < rounds; i++) {
+        Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+        if (g < out) {
+            const Fr vv = ld_fr(v_end - 8 * (size_t)(i + 1), 0);
+            const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
+            const Fr a0c = ld_fr(A, g), b0c = ld_fr(B, g);
+            const Fr a1c = ld_hi(A, g, out, in), b1c = ld_hi(B, g, out, in);
+            acc[0] = fr26::mulc(a0c, b0c);
+            acc[2] = fr26::mulc(sub(a1c, a0c), sub(b1c, b0c));
+            acc[1] = sub(sub(fr26::mulc(a1c, b1c), acc[0]), acc[2]);
+            st_fr(A, g, fold2(w0, w1, fr26::pack(a0c), fr26::pack(a1c)));
+            st_fr(B, g, fold2(w0, w1, fr26::pack(b0c), fr26::pack(b1c)));
+        }
+        block_sum<3>(acc, lds);
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int k = 0; k < 3; k++) st_fr(sums, 3 * (size_t)i + k, acc[k]);
+        }
+        __syncthreads();                              // folded values and lds visible to the next round
+        in = out;
+        out = out / 2;
+    }
+}
+
 __global__ void __launch_bounds__(kBlock) sumcheck1_kernel(uint32_t* X, uint32_t* a, uint32_t* b, uint32_t in_size,
                                                            uint32_t out_size, const uint32_t* v) {
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -361,6 +396,19 @@ static int sumcheck2_impl(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, ui
 }
 
 extern "C" {
+
+int grape_sumcheck_round2_tail(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t rounds, const uint32_t* v_end, uint32_t* sums,
+                               grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(B); CHECK_PTR16(v_end); CHECK_PTR16(sums);
+    if (rounds == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(in_size >= 1 && in_size <= 2u * kBlock, "tail rounds start at 2 * 256 elements or fewer");
+    uint32_t lg = 0;
+    while ((1u << lg) < in_size) lg++;
+    GRAPE_REQUIRE(rounds <= (lg ? lg : 1), "more rounds than variables");
+    sumcheck2_tail_kernel<<<1, kBlock, 0, as_stream(st)>>>(A, B, in_size, rounds, v_end, sums);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
 
 int grape_sumcheck_round2(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {
     GRAPE_REQUIRE(sums != nullptr, "d_sums is required");

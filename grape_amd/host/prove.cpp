@@ -61,6 +61,12 @@ void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, 
     // reference copies and synchronises after every round).
     FrTensor sums(3 * rounds);
     for (uint i = 0; i < rounds; i++) {
+        if (inputsize <= 512) {
+            // short tensors: all remaining rounds in one launch
+            check(grape_sumcheck_round2_tail(W(A.gpu_data), W(B.gpu_data), inputsize, rounds - i, W(v - i), W(sums.gpu_data + 3 * i), nullptr),
+                  "grape_sumcheck_round2_tail");
+            break;
+        }
         check(grape_sumcheck_round2(W(A.gpu_data), W(B.gpu_data), inputsize, outputsize, W(v - i - 1), W(sums.gpu_data + 3 * i), nullptr),
               "grape_sumcheck_round2");
         inputsize = outputsize;

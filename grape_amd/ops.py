@@ -169,6 +169,16 @@ def sumcheck_round2(A, B, in_size, out_size, v):
     return sums
 
 
+def sumcheck_round2_tail(A, B, in_size, rounds, v, v_end_index):
+    """rounds from in_size (<= 512) down, challenges v[v_end_index - 1], v[v_end_index - 2], ...;
+    returns the sums as a (3 * rounds, 8) tensor"""
+    lib = init()
+    sums = fr_empty(3 * max(rounds, 1))
+    v_end = v.data_ptr() + 32 * v_end_index
+    _capi.check(lib.grape_sumcheck_round2_tail(_p(A), _p(B), in_size, rounds, ctypes.c_void_p(v_end), _p(sums), _s()))
+    return sums
+
+
 def sumcheck_round2_coeffs(A, B, a, b, c, in_size, out_size, v, want_sums=True):
     lib = init()
     sums = fr_empty(3) if want_sums else None

@@ -101,6 +101,13 @@ int grape_fr_fold(uint32_t *d_t, size_t N, const uint32_t *d_x, uint32_t c, uint
  */
 int grape_sumcheck_round2(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size,
                           const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
+/* The last rounds of the same sumcheck in one launch (one workgroup, a barrier between rounds):
+ * `rounds` successive rounds starting from in_size <= 512 elements, out_size = 2^(ceil(log2 in_size) - 1)
+ * and halving from there; round i takes its challenge from d_v_end[-(i+1)] (the reference walks
+ * its challenge array backwards, src/prove.cu:101) and leaves its three sums in d_sums[3i..3i+2].
+ * Same results as `rounds` calls of grape_sumcheck_round2. */
+int grape_sumcheck_round2_tail(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t rounds,
+                               const uint32_t *d_v_end, uint32_t *d_sums, grape_stream_t stream);
 /* As above but also materialises the coefficient arrays a, b, c (needed by phase 1, which folds
  * them over the remaining layer bits, src/prove.cu:64-66).  d_sums may be NULL. */
 int grape_sumcheck_round2_coeffs(uint32_t *d_A, uint32_t *d_B, uint32_t *d_a, uint32_t *d_b, uint32_t *d_c,

@@ -50,6 +50,28 @@ def test_sumcheck_round2(ops, in_size, out_size):
     assert_same(sums2, sums, "sums")
 
 
+@pytest.mark.parametrize("in_size", [512, 300, 257, 64, 3, 2, 1])
+def test_sumcheck_tail_rounds_match_single_rounds(ops, in_size):
+    """all remaining rounds in one launch give what the same rounds give one launch at a time"""
+    rounds = br.log2ceil(in_size)
+    A, B = rand_fr(in_size, 301 + in_size), rand_fr(in_size, 302 + in_size)
+    v = rand_fr(rounds + 2, 303)
+    dv = ops.to_dev(v)
+    dA, dB = ops.to_dev(A), ops.to_dev(B)
+    want = []
+    n_in, n_out = in_size, (1 << (rounds - 1)) if rounds else 0
+    for i in range(rounds):
+        vi = dv[rounds + 1 - i - 1: rounds + 1 - i].contiguous()           # v[rounds], v[rounds-1], ...
+        want.append(ops.fr_to_host(ops.sumcheck_round2(dA, dB, n_in, n_out, vi)))
+        n_in, n_out = n_out, n_out // 2
+    tA, tB = ops.to_dev(A), ops.to_dev(B)
+    got = ops.fr_to_host(ops.sumcheck_round2_tail(tA, tB, in_size, rounds, dv, rounds + 1))
+    if rounds:
+        assert_same(got[: 3 * rounds], np.concatenate(want), "sums of every round")
+        assert_same(ops.fr_to_host(tA)[:1], ops.fr_to_host(dA)[:1], "A bound at every challenge")
+        assert_same(ops.fr_to_host(tB)[:1], ops.fr_to_host(dB)[:1], "B bound at every challenge")
+
+
 def test_sumcheck_round1(ops):
     in_size, out_size = 1000, 512
     X = rand_fr(in_size, 11)
