@@ -48,6 +48,8 @@ SIGNATURES = {
     "grape_sumcheck_round1": [c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p],
     "grape_tlookup_hist": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
     "grape_tlookup_index": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
+    "grape_tlookup_hist_index": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p],
+    "grape_tlookup_inverse_by_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_u32, ctypes.POINTER(c_size_t), c_void_p],
     "grape_tlookup_init": [c_void_p, c_void_p, c_i32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_tlookup_poly": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_poly_sum": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],

@@ -210,6 +210,47 @@ __global__ void __launch_bounds__(kBlock) hist_merge_kernel(uint32_t* hist, cons
     hist[t] += s;
 }
 
+// histogram of precomputed indices (idx1 = index + 1, 0 = outside the table), short witnesses
+__global__ void __launch_bounds__(kBlock) hist_index_kernel(uint32_t* hist, const int32_t* idx1, size_t n, uint32_t len) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t j = i < n ? (uint32_t)idx1[i] : 0u;
+    const bool valid = j >= 1 && j <= len;
+    const uint32_t idx = j - 1;
+    const int lane = threadIdx.x & 63;
+    unsigned long long todo = __ballot(valid);
+    for (int it = 0; it < 8 && todo != 0ull; it++) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const uint32_t lidx = __shfl(idx, leader, 64);
+        const unsigned long long same = __ballot(valid && idx == lidx) & todo;
+        if (lane == leader) atomicAdd(&hist[lidx], (uint32_t)__popcll(same));
+        todo &= ~same;
+    }
+    if (valid && ((todo >> lane) & 1ull)) atomicAdd(&hist[idx], 1u);
+}
+
+// A[i] = 1 / (S[i] + beta) read from the table instead of computed: with B[t] = 1 / (T[t] + beta)
+// and S[i] = T[idx_i], A[i] = B[idx_i].  Every element is checked against T; an element that is
+// outside the table or differs from its entry is counted in *mismatches and left unwritten.
+__global__ void __launch_bounds__(kBlock) inverse_by_table_kernel(uint32_t* A, const uint32_t* S, const int32_t* idx1, const uint32_t* T,
+                                                                   const uint32_t* B, size_t n, uint32_t len, unsigned int* mismatches) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    bool bad = false;
+    if (i < n) {
+        const uint32_t j = (uint32_t)idx1[i];
+        bad = !(j >= 1 && j <= len);
+        if (!bad) {
+            const Fr s = ld_fr(S, i), t = ld_fr(T, j - 1);
+            uint32_t diff = 0;
+#pragma unroll
+            for (int k = 0; k < 8; k++) diff |= s.v[k] ^ t.v[k];
+            bad = diff != 0;
+            if (!bad) st_fr(A, i, ld_fr(B, j - 1));
+        }
+    }
+    const unsigned long long b = __ballot(bad);
+    if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
+}
+
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -427,18 +468,9 @@ int grape_sumcheck_round1(uint32_t* X, uint32_t* a, uint32_t* b, uint32_t in_siz
     return GRAPE_OK;
 }
 
-int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t low, uint32_t len, grape_stream_t st) {
-    if (n == 0) return GRAPE_OK;
-    GRAPE_REQUIRE(hist != nullptr && len > 0, "bad histogram buffer");
-    CHECK_PTR16(vals);
-    hipStream_t s = as_stream(st);
-    if (n < ((size_t)1 << 20)) {
-        hist_kernel<<<blocks_for(n), kBlock, 0, s>>>(hist, vals, n, low, len);
-        GRAPE_LAUNCH_CHECK();
-        return GRAPE_OK;
-    }
-    // LDS counting: 32768 bins (128 KiB) per workgroup when the device grants that much dynamic
-    // LDS, else 16384
+// LDS counting of n >= 2^20 precomputed indices (see hist_lds_kernel)
+static int hist_lds_from_index(uint32_t* hist, const int32_t* idx, size_t n, uint32_t len, hipStream_t s) {
+    // 32768 bins (128 KiB) per workgroup when the device grants that much dynamic LDS, else 16384
     static int bins = 0;
     if (bins == 0) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&hist_lds_kernel<32768>),
@@ -457,21 +489,68 @@ int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t l
     while (chunks > 1 && n / chunks < ((size_t)1 << 16)) chunks /= 2;
     size_t per_chunk = (n + chunks - 1) / chunks;
     per_chunk = (per_chunk + 3) & ~(size_t)3;
-    void *idx, *partial;
-    int rc = scratch_get(kSlotHistIdx, n * 4, &idx);
+    void* partial;
+    int rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial);
     if (rc) return rc;
-    rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial);
-    if (rc) return rc;
-    index_kernel<<<blocks_for(n), kBlock, 0, s>>>((int32_t*)idx, vals, n, low, len);
-    GRAPE_LAUNCH_CHECK();
     const dim3 grid((unsigned)chunks, ranges);
     if (bins == 32768)
-        hist_lds_kernel<32768><<<grid, kHistThreads, 32768 * 4, s>>>((uint32_t*)partial, (const int32_t*)idx, n, per_chunk, len);
+        hist_lds_kernel<32768><<<grid, kHistThreads, 32768 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len);
     else
-        hist_lds_kernel<16384><<<grid, kHistThreads, 16384 * 4, s>>>((uint32_t*)partial, (const int32_t*)idx, n, per_chunk, len);
+        hist_lds_kernel<16384><<<grid, kHistThreads, 16384 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len);
     GRAPE_LAUNCH_CHECK();
     hist_merge_kernel<<<blocks_for(len), kBlock, 0, s>>>(hist, (const uint32_t*)partial, (uint32_t)chunks, len);
     GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t low, uint32_t len, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(hist != nullptr && len > 0, "bad histogram buffer");
+    CHECK_PTR16(vals);
+    hipStream_t s = as_stream(st);
+    if (n < ((size_t)1 << 20)) {
+        hist_kernel<<<blocks_for(n), kBlock, 0, s>>>(hist, vals, n, low, len);
+        GRAPE_LAUNCH_CHECK();
+        return GRAPE_OK;
+    }
+    void* idx;
+    int rc = scratch_get(kSlotHistIdx, n * 4, &idx);
+    if (rc) return rc;
+    index_kernel<<<blocks_for(n), kBlock, 0, s>>>((int32_t*)idx, vals, n, low, len);
+    GRAPE_LAUNCH_CHECK();
+    return hist_lds_from_index(hist, (const int32_t*)idx, n, len, s);
+}
+
+int grape_tlookup_hist_index(uint32_t* hist, const int32_t* idx1, size_t n, uint32_t len, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(hist != nullptr && idx1 != nullptr && len > 0, "bad arguments");
+    GRAPE_REQUIRE((reinterpret_cast<uintptr_t>(idx1) & 15) == 0, "idx1 must be 16-byte aligned");
+    hipStream_t s = as_stream(st);
+    if (n < ((size_t)1 << 20)) {
+        hist_index_kernel<<<blocks_for(n), kBlock, 0, s>>>(hist, idx1, n, len);
+        GRAPE_LAUNCH_CHECK();
+        return GRAPE_OK;
+    }
+    return hist_lds_from_index(hist, idx1, n, len, s);
+}
+
+int grape_tlookup_inverse_by_table(uint32_t* A, const uint32_t* S, const int32_t* idx1, const uint32_t* T, const uint32_t* B, size_t n,
+                                   uint32_t len, size_t* mismatches, grape_stream_t st) {
+    GRAPE_REQUIRE(mismatches != nullptr && idx1 != nullptr && len > 0, "bad arguments");
+    *mismatches = 0;
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(T); CHECK_PTR16(B);
+    hipStream_t s = as_stream(st);
+    void* cnt;
+    int rc = scratch_get(kSlotMisc, 64, &cnt);
+    if (rc) return rc;
+    GRAPE_HIP_CHECK(hipMemsetAsync(cnt, 0, sizeof(unsigned int), s));
+    inverse_by_table_kernel<<<blocks_for(n), kBlock, 0, s>>>(A, S, idx1, T, B, n, len, (unsigned int*)cnt);
+    GRAPE_LAUNCH_CHECK();
+    unsigned int h = 0;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(&h, cnt, sizeof h, hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    *mismatches = h;
     return GRAPE_OK;
 }
 

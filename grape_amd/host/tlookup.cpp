@@ -14,6 +14,37 @@ tLookup::~tLookup() {
     grape_free(com_A);
     grape_free(com_m);
     grape_free(scaled_table_);
+    grape_free(d_idx_);
+}
+
+void tLookup::make_index(const FrTensor& vals, int low_) {
+    drop_index();
+    check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(vals.size ? vals.size : 1)), "grape_malloc");
+    check(grape_tlookup_index(d_idx_, W(vals.gpu_data), vals.size, low_, T.size, nullptr), "grape_tlookup_index");
+}
+void tLookup::drop_index() {
+    if (d_idx_) {
+        check(grape_stream_sync(nullptr), "sync");
+        grape_free(d_idx_);
+        d_idx_ = nullptr;
+    }
+}
+// multiplicities from the indices (get_histogram_kernel, src/tlookup.cu:5-14, with the padding
+// rule of :276-281)
+void tLookup::index_to_m(uint witness_size, int low_) {
+    uint32_t* hist = nullptr;
+    check(grape_malloc((void**)&hist, sizeof(uint32_t) * (size_t)m.size), "grape_malloc");
+    check(grape_memset_zero(hist, sizeof(uint32_t) * (size_t)m.size, nullptr), "grape_memset_zero");
+    check(grape_tlookup_hist_index(hist, d_idx_, witness_size, m.size, nullptr), "grape_tlookup_hist_index");
+    if (witness_size != (1u << Log2(witness_size))) {
+        uint32_t zero_count = 0;
+        check(grape_memcpy_d2h(&zero_count, hist + (-low_), sizeof(uint32_t), nullptr), "d2h");
+        zero_count += (1u << Log2(witness_size)) - witness_size;
+        check(grape_memcpy_h2d(hist + (-low_), &zero_count, sizeof(uint32_t), nullptr), "h2d");
+    }
+    m.get_data(m.size, hist);
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(hist);
 }
 
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
@@ -63,7 +94,17 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     last_transcript = SumcheckTranscript();
 
     fr_t* d_beta = grape_host::device_scalar(beta);
-    check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
+    // A = 1/(S + beta): read from B where the witness matches its table entry (every element of
+    // a valid witness does), computed by batched inversion otherwise (tlookup_inv_kernel,
+    // src/tlookup.cu:52-62, inverts per element)
+    bool from_table = false;
+    if (d_idx_) {
+        size_t mismatches = 0;
+        check(grape_tlookup_inverse_by_table(W(A.gpu_data), W(S.gpu_data), d_idx_, W(T.gpu_data), W(B.gpu_data), D, N, &mismatches, nullptr),
+              "grape_tlookup_inverse_by_table");
+        from_table = mismatches == 0;
+    }
+    if (!from_table) check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
     A.set_size(D);
 
     {   // commitments of A and m (kept, not dropped)
@@ -78,12 +119,14 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             scaled_for_ = &hyrax;
         }
         if (indexed_commit_ && index_known_ && scaled_table_) {
-            int* d_idx = nullptr;
-            check(grape_malloc((void**)&d_idx, sizeof(int) * (size_t)D), "grape_malloc");
-            check(grape_tlookup_index(d_idx, W(S.gpu_data), D, index_low_, N, nullptr), "grape_tlookup_index");
+            int* d_idx = d_idx_;
+            if (!d_idx) {
+                check(grape_malloc((void**)&d_idx, sizeof(int) * (size_t)D), "grape_malloc");
+                check(grape_tlookup_index(d_idx, W(S.gpu_data), D, index_low_, N, nullptr), "grape_tlookup_index");
+            }
             com_A = hyrax.commit_indexed_affine(d_idx, D, msm_size, scaled_table_, scaled_cols_, N);
             check(grape_stream_sync(nullptr), "sync");
-            grape_free(d_idx);
+            if (d_idx != d_idx_) grape_free(d_idx);
         } else {
             com_A = hyrax.commit_affine(A, D, msm_size);
         }
@@ -190,13 +233,23 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
 
 Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
     uint D = S.size;
-    prep(S);
+    make_index(S, low);
+    index_to_m(D, low);                       // what prep(S) computes, from the shared indices
     if (D != (1u << Log2(D))) {
         // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
+        drop_index();
         Fr pad_value = Fr::zero();
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
     }
-    return run(S, A, v, hyrax, msm_size, commit_time);
+    Fr ret;
+    try {
+        ret = run(S, A, v, hyrax, msm_size, commit_time);
+    } catch (...) {
+        drop_index();
+        throw;
+    }
+    drop_index();
+    return ret;
 }
 
 // ------------------------------------------------------------------ mapping lookup
@@ -235,15 +288,25 @@ void tLookupRangeMapping::prep(const FrTensor& vals) { histogram_to_m(m, vals, l
 Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax,
                               uint msm_size, double& commit_time) {
     uint D = S_in.size;
-    prep(S_in);
+    make_index(S_in, low);
+    index_to_m(D, low);                       // what prep(S_in) computes, from the shared indices
     FrTensor S(1u << Log2(D));
     S.set_size(D);
     S = S_out;
     S *= r;
     S.add_with_size(D, S_in);
     if (D != (1u << Log2(D))) {
+        drop_index();
         Fr pad_value = mapped_vals((uint)(-low)) * r;
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
     }
-    return run(S, A, v, hyrax, msm_size, commit_time);
+    Fr ret;
+    try {
+        ret = run(S, A, v, hyrax, msm_size, commit_time);
+    } catch (...) {
+        drop_index();
+        throw;
+    }
+    drop_index();
+    return ret;
 }

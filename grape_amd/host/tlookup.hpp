@@ -41,6 +41,13 @@ protected:
     bool indexed_commit_ = true;
     bool index_known_ = false;          // set by tLookupRange: A's index is S - low
     int index_low_ = 0;
+    // Table indices (+1, 0 = outside) of the witness of the proof in flight, made once by prove()
+    // and used for the multiplicities, for A = B[index] and for the indexed commitment of A.
+    // nullptr when the witness is padded (its indices then do not line up with the padded tensor).
+    int* d_idx_ = nullptr;
+    void make_index(const FrTensor& vals, int low_);
+    void drop_index();
+    void index_to_m(uint witness_size, int low_);
     affine_t* scaled_table_ = nullptr;  // B[t]*G_i, built on first use
     uint scaled_cols_ = 0;
     Hyrax* scaled_for_ = nullptr;

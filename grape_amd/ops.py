@@ -199,6 +199,30 @@ def tlookup_hist(vals, low, length, hist=None):
     return hist
 
 
+def tlookup_index(vals, low, length):
+    lib = init()
+    out = torch.empty(vals.shape[0], dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_tlookup_index(_p(out), _p(vals), vals.shape[0], low, length, _s()))
+    return out
+
+
+def tlookup_hist_index(idx1, length, hist=None):
+    lib = init()
+    if hist is None:
+        hist = torch.zeros(length, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_tlookup_hist_index(_p(hist), _p(idx1), idx1.shape[0], length, _s()))
+    return hist
+
+
+def tlookup_inverse_by_table(S, idx1, T, B, A=None):
+    """returns (A, mismatches)"""
+    lib = init()
+    A = fr_empty(S.shape[0]) if A is None else A
+    mm = ctypes.c_size_t(0)
+    _capi.check(lib.grape_tlookup_inverse_by_table(_p(A), _p(S), _p(idx1), _p(T), _p(B), S.shape[0], T.shape[0], ctypes.byref(mm), _s()))
+    return A, mm.value
+
+
 def tlookup_init(low, length, beta, map_t=None, r=None):
     lib = init()
     T, B = fr_empty(length), fr_empty(length)

@@ -127,6 +127,17 @@ int grape_tlookup_hist(uint32_t *d_hist, const uint32_t *d_vals, size_t n, int32
  * reference derives inside get_histogram_kernel, src/tlookup.cu:9-12).  Feeds the indexed
  * commitment of A = 1/(S+beta) below. */
 int grape_tlookup_index(int32_t *d_out, const uint32_t *d_vals, size_t n, int32_t low, uint32_t len, grape_stream_t stream);
+/* The same histogram from indices already made by grape_tlookup_index (d_idx1[i] = index + 1,
+ * 0 = outside the table): hist[d_idx1[i] - 1] += 1. */
+int grape_tlookup_hist_index(uint32_t *d_hist, const int32_t *d_idx1, size_t n, uint32_t len, grape_stream_t stream);
+/* A = 1/(S + beta) read from the lookup table instead of computed (tlookup_inv_kernel,
+ * src/tlookup.cu:52-62, is an inversion per element): where S[i] equals the table entry
+ * T[d_idx1[i] - 1], A[i] = B[d_idx1[i] - 1] with B = 1/(T + beta).  Elements outside the table or
+ * different from their entry are left unwritten and counted in *mismatches (host; the call
+ * synchronises); a caller that sees mismatches != 0 inverts the tensor with
+ * grape_fr_shift_inverse instead. */
+int grape_tlookup_inverse_by_table(uint32_t *d_A, const uint32_t *d_S, const int32_t *d_idx1, const uint32_t *d_T,
+                                   const uint32_t *d_B, size_t n, uint32_t len, size_t *mismatches, grape_stream_t stream);
 /* T[i] = low + i (+ r*map[i] when d_map != NULL), B[i] = 1/(T[i] + beta).
  * tlookuprange_init_kernel / tLookupRangeMapping_init_kernel, src/tlookup.cu:16-50. */
 int grape_tlookup_init(uint32_t *d_T, uint32_t *d_B, int32_t low, uint32_t len, const uint32_t *d_beta,

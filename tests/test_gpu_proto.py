@@ -155,6 +155,38 @@ def test_histogram_long_witness(ops):
     assert h3[5] == (1 << 20) + 1 and h3.sum() == (1 << 20) + 1
 
 
+@pytest.mark.parametrize("n", [5000, (1 << 20) + 77])
+def test_index_histogram_and_inverse_by_table(ops, n):
+    """indices made once serve the multiplicities and A = 1/(S+beta) = B[index]; elements that are
+    outside the table or differ from their entry are reported, not written"""
+    import torch
+    low, length = -300, 1000
+    rng = np.random.default_rng(33 + n)
+    s = rng.integers(low, low + length, size=n).astype(np.int32)
+    s[::11] = low + 5
+    vals = ops.fr_from_i32(torch.from_numpy(s).cuda())
+    idx1 = ops.tlookup_index(vals, low, length)
+    assert np.array_equal(idx1.cpu().numpy(), s - low + 1)
+    h = ops.tlookup_hist_index(idx1, length).cpu().numpy().view(np.uint32)
+    assert np.array_equal(h, np.bincount(s.astype(np.int64) - low, minlength=length).astype(np.uint32))
+    beta = ops.to_dev(br.fr_pack([length]))
+    T, B = ops.tlookup_init(low, length, beta)
+    A, mism = ops.tlookup_inverse_by_table(vals, idx1, T, B)
+    assert mism == 0
+    assert_same(ops.fr_to_host(A), ops.fr_to_host(ops.fr_shift_inverse(vals, beta)), "A from the table = batched inversion")
+    # one value outside the table, one inside whose tensor element was altered afterwards
+    s2 = s.copy()
+    s2[7] = low + length + 3
+    vals2 = ops.fr_from_i32(torch.from_numpy(s2).cuda())
+    idx2 = ops.tlookup_index(vals2, low, length)
+    assert idx2[7].item() == 0
+    vals2[100] = ops.fr_from_i32(torch.tensor([int(s2[100]) + 1], dtype=torch.int32, device="cuda"))[0]
+    A2, mism2 = ops.tlookup_inverse_by_table(vals2, idx2, T, B)
+    assert mism2 == 2
+    h2 = ops.tlookup_hist_index(idx2, length).cpu().numpy()
+    assert h2.sum() == n - 1
+
+
 def test_table_init(ops):
     low, length = -32768, 65536
     beta = br.fr_pack([length])
