@@ -237,9 +237,9 @@ Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax
     index_to_m(D, low);                       // what prep(S) computes, from the shared indices
     if (D != (1u << Log2(D))) {
         // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
-        drop_index();
         Fr pad_value = Fr::zero();
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
+        make_index(S, low);                   // indices of the padded witness
     }
     Fr ret;
     try {
