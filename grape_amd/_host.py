@@ -11,7 +11,7 @@ NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seco
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
          "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
          "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
-         "grape_host_generate_data"]
+         "grape_host_generate_data", "grape_host_single_commit"]
 
 
 class HostError(RuntimeError):
@@ -222,3 +222,9 @@ def generate_data(size):
     p = ctypes.c_void_p(0)
     _check(load().grape_host_generate_data(ctypes.byref(p), size))
     return p.value
+
+
+def single_commit(d_scalars, N, d_table, npoints):
+    out = np.zeros(12, dtype=np.uint64)
+    _check(load().grape_host_single_commit(_dp(d_scalars), N, _dp(d_table), npoints, _hp(out)))
+    return out

@@ -284,6 +284,19 @@ int grape_host_g1_mul_generator(const uint32_t* k_mont, uint32_t* out_affine) {
     GUARD_END
 }
 
+int grape_host_single_commit(const uint32_t* d_scalars, uint32_t N, const uint32_t* d_table, uint32_t npoints, uint32_t* out_affine) {
+    GUARD_BEGIN
+    jacob_t* com = nullptr;
+    grape_host::check(grape_malloc((void**)&com, sizeof(jacob_t)), "grape_malloc");
+    single_commit((fr_t*)d_scalars, (affine_t*)d_table, com, N, npoints);
+    affine_t* aff = nullptr;
+    grape_host::check(grape_malloc((void**)&aff, sizeof(affine_t)), "grape_malloc");
+    grape_host::check(grape_g1_jacobian_to_affine((uint32_t*)aff, (const uint32_t*)com, 1, nullptr), "grape_g1_jacobian_to_affine");
+    grape_host::check(grape_memcpy_d2h(out_affine, aff, sizeof(affine_t), nullptr), "grape_memcpy_d2h");
+    grape_free(aff);
+    grape_free(com);
+    GUARD_END
+}
 int grape_host_bin_io(int op, const char* filename, void* ptr, size_t size, int is_gpu) {
     GUARD_BEGIN
     if (op == 0) savebin(filename, ptr, size, is_gpu != 0);

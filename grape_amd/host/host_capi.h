@@ -72,6 +72,10 @@ int grape_host_fr_op(int op, const uint32_t *a, const uint32_t *b, uint32_t *out
 /* k * G as a host computation (affine out) */
 int grape_host_g1_mul_generator(const uint32_t *k_mont, uint32_t *out_affine);
 
+/* single_commit (src/Hyrax.cu:176-185): one row of N full-width scalars against the reference-format
+ * table; the Jacobian result is returned in affine form on the host. */
+int grape_host_single_commit(const uint32_t *d_scalars, uint32_t N, const uint32_t *d_table, uint32_t npoints,
+                             uint32_t *out_affine);
 /* File helpers (ioutils.hpp): op 0 = savebin, 1 = loadbin of `size` bytes at ptr (device memory
  * when is_gpu != 0); findsize; load_data into a fresh device buffer (*d_out, *n elements);
  * generate_data (std::mt19937(123456) int32) into a fresh device buffer. */

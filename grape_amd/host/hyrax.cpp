@@ -154,6 +154,16 @@ affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine
     return out;
 }
 
+void single_commit(fr_t* d, affine_t* g, jacob_t* com, uint N, uint npoints) {
+    grape_host::ensure_init();
+    affine_t* a = nullptr;
+    check(grape_malloc((void**)&a, sizeof(affine_t)), "grape_malloc");
+    check(grape_commit_fr_ref_table(W(a), W(d), N, N, W(g), npoints, nullptr), "grape_commit_fr_ref_table");
+    check(grape_g1_affine_to_jacobian(W(com), W(a), 1, nullptr), "grape_g1_affine_to_jacobian");
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(a);
+}
+
 static jacob_t* to_jacobian(affine_t* aff, uint rows) {
     jacob_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(jacob_t) * (size_t)rows), "grape_malloc");

@@ -18,6 +18,11 @@ public:
     Hyrax_proof& operator=(const Hyrax_proof& other);
 };
 
+// com[0] = sum_i d[i] * G_i over the first N generators of the reference-format table g
+// (entry w * npoints + i = w * G_i): the one-row commitment Hyrax::open makes of its blinding
+// vector (single_commit, src/Hyrax.cu:176-185).  d: device, Montgomery form; com: device.
+void single_commit(fr_t* d, affine_t* g, jacob_t* com, uint N, uint npoints);
+
 class Hyrax {
 public:
     uint com_scale;

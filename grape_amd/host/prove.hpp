@@ -12,6 +12,22 @@ struct SumcheckTranscript {
     std::vector<Fr> claims;           // running claim after each round
 };
 
+// Work tensors a driver keeps across the sumchecks of one layer (include/prove.cuh:13-26):
+// a, b, c hold tokens_size * 2^13 elements each, tmpw one FFN row of 11008.
+struct SumcheckWorkTmp {
+    FrTensor tmpw;
+    FrTensor a;
+    FrTensor b;
+    FrTensor c;
+    size_t tokens_size;
+
+    explicit SumcheckWorkTmp(size_t tokens_size_)
+        : tmpw(11008), a((uint)(tokens_size_ * (1u << 13))), b((uint)(tokens_size_ * (1u << 13))),
+          c((uint)(tokens_size_ * (1u << 13))), tokens_size(tokens_size_) {}
+    SumcheckWorkTmp(const SumcheckWorkTmp&) = delete;
+    SumcheckWorkTmp& operator=(const SumcheckWorkTmp&) = delete;
+};
+
 Fr matmul_sumcheck_phase1(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* u, fr_t* v, uint K,
                           uint size, Fr& claim, SumcheckTranscript* transcript = nullptr);
 void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* v, uint K, Fr& claim,

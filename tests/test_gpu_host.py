@@ -225,6 +225,14 @@ def test_hyrax_class_commits(ops, host, gens):
         host.hyrax_commit_i32(torch.from_numpy(W).cuda(), 128, 16, table, npoints, com_scale=16)
 
 
+def test_single_commit(ops, host, gens):
+    hg, dg = gens
+    table = ops.g1_table_gen(dg, 256)
+    s = rand_fr(64, 65)
+    got = host.single_commit(ops.to_dev(s), 64, table, 256)
+    assert_same(got, orc.commit_fr(s, orc.g1_table(hg, 256), 64, 256)[0], "single_commit")
+
+
 def test_hyrax_open_and_verify(ops, host, gens):
     hg, dg = gens
     npoints = 64
