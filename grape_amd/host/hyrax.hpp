@@ -58,7 +58,7 @@ public:
     // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
     affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len);
 
-    // Upper bound for the wide fixed-base tables this object may build (default 96 GiB of the 288 GB).  When a
+    // Upper bound for the wide fixed-base tables this object may build (default 128 GiB of the 288 GB; GRAPE_TABLE_BUDGET_GIB overrides).  When a
     // table would not fit, commitments go through the reference-format table instead.
     void set_table_budget(size_t bytes) { table_budget_ = bytes; }
 

@@ -1,0 +1,116 @@
+// A driver written the way the reference's test programs are (test/HyraxTest.cu, test/tlookupTest.cu,
+// the matmul block of test/llm.cu), against the host classes of this build: generators and table,
+// integer and field-element commitments, opening with a real verification, a matmul sumcheck and a
+// range lookup.  Compiled with g++ and linked with libgrape_host / libgrape_hip by the tests; prints
+// "driver_flow OK" when every check holds.
+#include <cstdio>
+#include <cstdlib>
+#include <stdexcept>
+#include <string>
+#include <vector>
+#include "../../include/grape_hip.h"
+#include "../../grape_amd/host/ec_operation.hpp"
+#include "../../grape_amd/host/fr_tensor.hpp"
+#include "../../grape_amd/host/hyrax.hpp"
+#include "../../grape_amd/host/ioutils.hpp"
+#include "../../grape_amd/host/polynomial.hpp"
+#include "../../grape_amd/host/prove.hpp"
+#include "../../grape_amd/host/timer.hpp"
+#include "../../grape_amd/host/tlookup.hpp"
+
+static void require(bool ok, const char* what) {
+    if (!ok) throw std::runtime_error(std::string("driver_flow: ") + what);
+}
+
+int main(int argc, char** argv) {
+    const std::string dir = argc > 1 ? argv[1] : "/tmp";
+    try {
+        Fr::seed(2024);
+        Timer timer;
+        timer.start();
+        const uint npoints = 1024, layer_num = 1, N = 4, com_scale = 16;   // rows of N * com_scale = 64
+        affine_t* points = nullptr;
+        require(grape_malloc((void**)&points, sizeof(affine_t) * 256 * npoints) == 0, "grape_malloc");
+        std::vector<bn128> cpu_points = precompute_generators(npoints, 256, points);
+        require(cpu_points.size() == npoints, "generator count");
+        savebin(dir + "/points.bin", points, sizeof(affine_t) * 256 * npoints);          // test/ppgen.cu writes this file
+        require(findsize(dir + "/points.bin") == sizeof(affine_t) * 256 * npoints, "points.bin size");
+
+        // ---- commitments of an int tensor and of the same values as field elements agree (test/HyraxTest.cu:57-67)
+        const uint size = 64 * 8;
+        int* tensor = nullptr;
+        generate_data(&tensor, size);
+        Hyrax hyrax(layer_num, npoints / com_scale, points, cpu_points[0]);
+        FrTensor fr_tensor(size, tensor);
+        jacob_t* com_int = hyrax.commit(tensor, size, N);
+        jacob_t* com_fr = hyrax.commit(fr_tensor, size, N);
+        const uint rows = size / N / com_scale;
+        std::vector<bn128> h_int(rows), h_fr(rows);
+        require(grape_memcpy_d2h(h_int.data(), com_int, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
+        require(grape_memcpy_d2h(h_fr.data(), com_fr, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
+        for (uint i = 0; i < rows; i++) require(h_int[i] == h_fr[i], "int path and Fr path commit to different points");
+
+        // ---- open at a random point, verify, and compare with the multilinear extension (test/HyraxTest.cu:76-125)
+        std::vector<Fr> eval_point = random_vec(Log2(size));
+        Fr c = Fr::random_element();
+        FrTensor copy1(fr_tensor), copy2(fr_tensor);
+        Hyrax_proof proof = hyrax.open(copy1, eval_point, c, size, N);
+        require(hyrax.verify(proof, com_fr, eval_point, c, size, N), "opening does not verify");
+        require(proof.result == copy2(eval_point), "opened value differs from the multilinear extension");
+
+        // ---- matmul sumcheck (the pattern of test/llm.cu): Y[n][m] = sum_k A[n][k] B[m][k]
+        const int Ln = 1, Nn = 8, Mn = 4, Kn = 16;
+        FrTensor A = FrTensor::random(Ln * Nn * Kn), B = FrTensor::random(Ln * Mn * Kn);
+        std::vector<Fr> hA = A.to_host(), hB = B.to_host(), hY((size_t)Nn * Mn);
+        for (int n = 0; n < Nn; n++)
+            for (int m = 0; m < Mn; m++) {
+                Fr s = Fr::zero();
+                for (int k = 0; k < Kn; k++) s += hA[n * Kn + k] * hB[m * Kn + k];
+                hY[n * Mn + m] = s;
+            }
+        FrTensor Y = FrTensor::from_host(hY);
+        std::vector<Fr> u = random_vec(Log2(Ln * Nn * Mn)), v = random_vec(Log2(Kn) + Log2(Ln));
+        Fr claim = Y(u);
+        SumcheckTranscript tr;
+        std::pair<Fr, Fr> ab = prove_matmul(A, B, Ln, Nn, Mn, Kn, u, v, claim, &tr);
+        require(tr.rounds.size() == Log2(Kn), "round count");
+        require(ab.first * ab.second == claim, "A(v) * B(v) != final claim");
+
+        // ---- range lookup (test/tlookupTest.cu): every value lies in [-512, 512)
+        const uint D = 4096;
+        std::vector<int> h_s(D);
+        for (uint i = 0; i < D; i++) h_s[i] = (int)((i * 37 + 11) % 1024) - 512;
+        int* d_s = nullptr;
+        require(grape_malloc((void**)&d_s, sizeof(int) * D) == 0, "grape_malloc");
+        require(grape_memcpy_h2d(d_s, h_s.data(), sizeof(int) * D, nullptr) == 0, "h2d");
+        FrTensor S(D, d_s), S_keep(D, d_s), Aux(D);
+        tLookupRange rs(-512, 1024);
+        std::vector<Fr> v2 = random_vec(Log2(D));
+        double commit_time = 0.0;
+        Fr lookup_value = rs.prove(S, Aux, v2, hyrax, N, commit_time);
+        require(lookup_value == S_keep(v2), "lookup value differs from S(v)");
+        // a witness with one value outside the range is rejected by the prover's own check
+        h_s[5] = 600;
+        require(grape_memcpy_h2d(d_s, h_s.data(), sizeof(int) * D, nullptr) == 0, "h2d");
+        FrTensor S_bad(D, d_s);
+        bool rejected = false;
+        try {
+            rs.prove(S_bad, Aux, v2, hyrax, N, commit_time);
+        } catch (const std::runtime_error&) {
+            rejected = true;
+        }
+        require(rejected, "out-of-range witness was not rejected");
+
+        grape_free(d_s);
+        grape_free(com_int);
+        grape_free(com_fr);
+        grape_free(tensor);
+        grape_free(points);
+        timer.stop("driver_flow");
+        std::printf("driver_flow OK\n");
+        return 0;
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "%s\n", e.what());
+        return 1;
+    }
+}

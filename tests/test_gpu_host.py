@@ -329,3 +329,14 @@ def test_file_helpers_and_on_disk_formats(ops, host, gens, tmp_path):
     _capi.check(lib.grape_stream_sync(None))
     _capi.check(lib.grape_free(p1)); _capi.check(lib.grape_free(p2))
     assert torch.equal(a, b) and a.min().item() < -2**30 and a.max().item() > 2**30
+
+
+def test_cpp_driver_runs(ops, tmp_path):
+    """the reference-style C++ driver (generators, table file, int and Fr commitments, opening and
+    verification, matmul sumcheck, range lookup incl. a rejected witness) end to end"""
+    import subprocess
+    import driver_build
+    exe = driver_build.build()
+    res = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=280)
+    assert res.returncode == 0, res.stderr
+    assert "driver_flow OK" in res.stdout

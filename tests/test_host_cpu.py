@@ -49,3 +49,12 @@ def test_file_helpers_on_host_memory(tmp_path):
     _host.loadbin(f, c.ctypes.data, c.nbytes, is_gpu=False)      # asks for more than the file holds
     assert (c == -1).all()
     assert _host.findsize(str(tmp_path / "absent.bin")) == 0
+
+
+def test_cpp_driver_compiles_against_the_host_headers():
+    """a driver in the reference's style builds with g++ against the host classes alone (no HIP
+    headers, no kernels); the GPU suite runs it"""
+    import driver_build
+    exe = driver_build.build()
+    import os
+    assert os.path.exists(exe)
