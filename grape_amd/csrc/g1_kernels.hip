@@ -176,31 +176,55 @@ __device__ __forceinline__ void madd28(Xyzz28& acc, const Affine28& e, bool nega
 
 // acc += k * G_col for a canonical (non-Montgomery) 255-bit scalar k: signed radix-2^c digits,
 // one gather and one mixed addition per non-zero digit.
+// One signed radix-2^c digit of a canonical scalar: window w, incoming carry -> magnitude, sign,
+// outgoing carry.
+__device__ __forceinline__ uint32_t fr_digit(const Fr& k, uint32_t w, uint32_t c, uint32_t& carry, bool& neg) {
+    const uint32_t half = 1u << (c - 1), mask = (1u << c) - 1u;
+    const uint32_t bit = w * c;
+    // c <= 16 bits starting at `bit`, possibly straddling two limbs
+    const uint32_t limb = bit >> 5, sh = bit & 31;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        lo = (q == (int)limb) ? k.v[q] : lo;
+        hi = (q == (int)limb + 1) ? k.v[q] : hi;
+    }
+    const uint64_t both = ((uint64_t)hi << 32) | lo;
+    const uint32_t d = ((uint32_t)(both >> sh) & mask) + carry;
+    neg = d > half;                      // digit in (half, 2^c] -> d - 2^c, carry 1
+    carry = neg ? 1u : 0u;
+    return neg ? (mask + 1u - d) : d;
+}
+
+// acc += k * G_col through the wide table: one gather and one mixed addition per non-zero digit.
+// While the addition of digit w runs, the table line of digit w+1 is already on its way (one
+// word of it is touched right after the entry of digit w has been requested).
 __device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k, const uint32_t* table, size_t N, uint32_t col,
                                                uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
-    const uint32_t half = 1u << (c - 1), mask = (1u << c) - 1u;
+    uint32_t nwin = nw;
+    while (nwin > 0 && (nwin - 1) * c >= 256) nwin--;     // windows that start inside the scalar
     uint32_t carry = 0;
-    for (uint32_t w = 0; w < nw; w++) {
-        const uint32_t bit = w * c;
-        if (bit >= 256) break;
-        // c <= 16 bits starting at `bit`, possibly straddling two limbs
-        const uint32_t limb = bit >> 5, sh = bit & 31;
-        uint32_t lo = 0, hi = 0;
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            lo = (q == (int)limb) ? k.v[q] : lo;
-            hi = (q == (int)limb + 1) ? k.v[q] : hi;
-        }
-        uint64_t both = ((uint64_t)hi << 32) | lo;
-        uint32_t d = ((uint32_t)(both >> sh) & mask) + carry;
-        bool neg = d > half;                 // digit in (half, 2^c] -> d - 2^c, carry 1
-        carry = neg ? 1u : 0u;
-        uint32_t mag = neg ? (mask + 1u - d) : d;
+    bool neg = false;
+    uint32_t mag = nwin ? fr_digit(k, 0, c, carry, neg) : 0;
+    uint32_t touch = 0;
+    for (uint32_t w = 0; w < nwin; w++) {
+        bool neg_n = false;
+        const uint32_t mag_n = (w + 1 < nwin) ? fr_digit(k, w + 1, c, carry, neg_n) : 0;
         if (mag != 0) {
-            if (mag > K) { *err_flag = 1; continue; }
-            madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
+            if (mag > K) {
+                *err_flag = 1;
+            } else {
+                const Affine28 e = ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col);
+                // unconditional, so that the compiler counts the outstanding loads exactly
+                const size_t nxt = (mag_n != 0 && mag_n <= K) ? ((size_t)(w + 1) * K + (mag_n - 1)) * N + col : (size_t)col;
+                touch = table[(size_t)kWideEntryWords * nxt];
+                madd28(acc, e, neg);
+            }
         }
+        mag = mag_n;
+        neg = neg_n;
     }
+    asm volatile("" ::"v"(touch));      // keeps the last touch alive until here
     if (carry) *err_flag = 1;   // cannot happen for canonical 255-bit scalars when nw*c >= 256
 }
 
@@ -354,12 +378,44 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
     const uint32_t col_end = (s + 1) * seg < rowlen ? (s + 1) * seg : rowlen;
     const uint32_t half = 1u << (c - 1), mask = (c == 32) ? 0xffffffffu : ((1u << c) - 1u);
     Xyzz28 acc = xyzz28_inf();
+    // int path: the scalars of the next two columns are kept in flight (the next one addresses
+    // the table line to touch, the one after is being loaded)
+    int32_t sc1 = 0, sc2 = 0;
+    if (!FR) {
+        const uint32_t c0 = s * seg + lane;
+        if (c0 + 64 < col_end) sc1 = ((const int32_t*)scalars)[row * rowlen + c0 + 64];
+        if (c0 + 128 < col_end) sc2 = ((const int32_t*)scalars)[row * rowlen + c0 + 128];
+    }
+    int32_t sc0 = (!FR && s * seg + lane < col_end) ? ((const int32_t*)scalars)[row * rowlen + s * seg + lane] : 0;
     for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
         if (FR) {
             const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
             madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
         } else {
-            int64_t v = ((const int32_t*)scalars)[row * rowlen + col];
+            int64_t v = sc0;
+            const int64_t v_next = sc1;
+            sc0 = sc1;
+            sc1 = sc2;
+            sc2 = (col + 192 < col_end) ? ((const int32_t*)scalars)[row * rowlen + col + 192] : 0;
+            // The table line of the NEXT column's first digit is touched (one word) right after
+            // this column's own entry is requested, so that it is in cache when its turn comes:
+            // with two waves per SIMD an exposed HBM round trip per addition costs issue slots.
+            // (the touch is unconditional - a column without a successor touches its own first
+            // table line - because the compiler counts outstanding loads exactly only in
+            // straight-line code; a conditional load after the entry's would make it wait for both)
+            size_t next_entry = col;
+            bool have_next = false;
+            if (col + 64 < col_end) {
+                int64_t vn = v_next;
+                int64_t dn = vn & (int64_t)mask;
+                vn >>= c;
+                if (dn > (int64_t)half || (dn == (int64_t)half && vn < 0)) dn -= (int64_t)mask + 1;
+                const uint32_t magn = (uint32_t)(dn < 0 ? -dn : dn);
+                have_next = magn != 0 && magn <= K;
+                if (have_next) next_entry = ((size_t)(magn - 1)) * N + col + 64;
+            }
+            const uint32_t* touch_ptr = table + (size_t)kWideEntryWords * next_entry;
+            uint32_t touch = 0;
             for (uint32_t w = 0; w < nw; w++) {
                 int64_t d = v & (int64_t)mask;
                 v >>= c;                            // arithmetic shift keeps the sign
@@ -373,9 +429,12 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 const uint32_t mag = (uint32_t)(neg ? -d : d);
                 if (mag != 0) {
                     if (mag > K) { *err_flag = 1; continue; }
-                    madd28(acc, ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col), neg);
+                    const Affine28 e = ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col);
+                    touch = *touch_ptr;
+                    madd28(acc, e, neg);
                 }
             }
+            asm volatile("" ::"v"(touch));          // keeps the touch alive until here
             if (v != 0) *err_flag = 1;              // scalar does not fit nw windows
         }
     }
