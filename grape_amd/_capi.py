@@ -41,6 +41,7 @@ SIGNATURES = {
     "grape_fr_sum_by_dim": [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p],
     "grape_fr_pad": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_void_p, c_void_p],
     "grape_i32_pad": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_void_p],
+    "grape_i32_pad_fill": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_i32, c_void_p],
     "grape_fr_fold": [c_void_p, c_size_t, c_void_p, c_u32, c_u32, c_u32, c_void_p],
     "grape_sumcheck_round2": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_tail": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],

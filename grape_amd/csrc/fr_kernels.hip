@@ -67,12 +67,13 @@ __global__ void __launch_bounds__(kBlock) pad_fr_kernel(uint32_t* out, const uin
     uint32_t col = (uint32_t)(g % pad_N);
     st_fr(out, g, col < N ? ld_fr(in, row * N + col) : ld_fr(pad_val, 0));
 }
-__global__ void __launch_bounds__(kBlock) pad_i32_kernel(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t size) {
+__global__ void __launch_bounds__(kBlock) pad_i32_kernel(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t size,
+                                                         int32_t fill) {
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (g >= size) return;
     size_t row = g / pad_N;
     uint32_t col = (uint32_t)(g % pad_N);
-    out[g] = col < N ? in[row * N + col] : 0;
+    out[g] = col < N ? in[row * N + col] : fill;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -510,7 +511,14 @@ int grape_fr_pad(uint32_t* out, const uint32_t* in, uint32_t N, uint32_t pad_N, 
 int grape_i32_pad(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t pad_size, grape_stream_t st) {
     if (pad_size == 0) return GRAPE_OK;
     GRAPE_REQUIRE(out && in && N <= pad_N && pad_N > 0 && out != in, "need N <= pad_N and distinct buffers");
-    pad_i32_kernel<<<blocks_for(pad_size), kBlock, 0, as_stream(st)>>>(out, in, N, pad_N, pad_size);
+    pad_i32_kernel<<<blocks_for(pad_size), kBlock, 0, as_stream(st)>>>(out, in, N, pad_N, pad_size, 0);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+int grape_i32_pad_fill(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad_N, size_t pad_size, int32_t fill, grape_stream_t st) {
+    if (pad_size == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(out && in && N <= pad_N && pad_N > 0 && out != in, "need N <= pad_N and distinct buffers");
+    pad_i32_kernel<<<blocks_for(pad_size), kBlock, 0, as_stream(st)>>>(out, in, N, pad_N, pad_size, fill);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

@@ -22,6 +22,15 @@ void tLookup::make_index(const FrTensor& vals, int low_) {
     check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(vals.size ? vals.size : 1)), "grape_malloc");
     check(grape_tlookup_index(d_idx_, W(vals.gpu_data), vals.size, low_, T.size, nullptr), "grape_tlookup_index");
 }
+void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
+    if (!d_idx_ || N == pad_N) return;
+    int* padded = nullptr;
+    check(grape_malloc((void**)&padded, sizeof(int) * (size_t)pad_size), "grape_malloc");
+    check(grape_i32_pad_fill(padded, d_idx_, N, pad_N, pad_size, fill, nullptr), "grape_i32_pad_fill");
+    check(grape_stream_sync(nullptr), "sync");
+    grape_free(d_idx_);
+    d_idx_ = padded;
+}
 void tLookup::drop_index() {
     if (d_idx_) {
         check(grape_stream_sync(nullptr), "sync");
@@ -296,9 +305,9 @@ Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, cons
     S *= r;
     S.add_with_size(D, S_in);
     if (D != (1u << Log2(D))) {
-        drop_index();
         Fr pad_value = mapped_vals((uint)(-low)) * r;
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
+        pad_index(11008, 16384, 1u << Log2(D), -low + 1);      // the padding value sits at table index -low
     }
     Fr ret;
     try {

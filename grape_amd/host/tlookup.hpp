@@ -47,6 +47,7 @@ protected:
     int* d_idx_ = nullptr;
     void make_index(const FrTensor& vals, int low_);
     void drop_index();
+    void pad_index(uint N, uint pad_N, uint pad_size, int fill);   // rows of N indices -> rows of pad_N
     void index_to_m(uint witness_size, int low_);
     affine_t* scaled_table_ = nullptr;  // B[t]*G_i, built on first use
     uint scaled_cols_ = 0;

@@ -81,6 +81,10 @@ int grape_fr_sum_by_dim(uint32_t *d_out, const uint32_t *d_in, size_t rows, size
 int grape_fr_pad(uint32_t *d_out, const uint32_t *d_in, uint32_t N, uint32_t pad_N, size_t pad_size,
                  const uint32_t *d_pad_val, grape_stream_t stream);
 int grape_i32_pad(int32_t *d_out, const int32_t *d_in, uint32_t N, uint32_t pad_N, size_t pad_size, grape_stream_t stream);
+/* The same with a fill value other than zero (pads the table indices of a lookup witness with the
+ * index of the padding value). */
+int grape_i32_pad_fill(int32_t *d_out, const int32_t *d_in, uint32_t N, uint32_t pad_N, size_t pad_size, int32_t fill,
+                       grape_stream_t stream);
 /*
  * Fold (partial multilinear evaluation) in place: view the first N elements of t as
  * [N/(c*gap)][c][gap], bind the c axis with challenges x[id], x[id+1], ... (index bit j of the

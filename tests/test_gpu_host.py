@@ -198,6 +198,33 @@ def test_tlookup_mapping_prove_vs_oracle(ops, host, gens):
                                    table, 16, 1, 16)
 
 
+def test_tlookup_mapping_pads_11008_rows(ops, host, gens):
+    # mapping lookup of 2 x 11008 pairs: padded to 2 x 16384 with the pair (0, f(0)), counted in m
+    import torch
+    hg, dg = gens
+    D, low, N = 2 * 11008, -16, 32
+    rng = np.random.default_rng(56)
+    fmap = rng.integers(-1000, 1000, size=N).astype(np.int32)
+    S_in = rng.integers(low, low + N, size=D).astype(np.int32)
+    S_out = fmap[S_in - low]
+    alpha, r, u, v = rand_fr(1, 57), rand_fr(1, 58), rand_fr(15, 59), rand_fr(15, 60)
+    beta = br.fr_pack([N])[0]
+    T, B = orc.tlookup_init(low, N, beta, orc.from_i32(fmap), r[0])
+    m = orc.tlookup_prep(orc.from_i32(S_in), low, N)             # includes the pad fix-up of the zero bin
+    S = orc.vec2("orc_fr_vec_add", orc.vec_bcast("orc_fr_vec_bcast_mul", orc.from_i32(S_out), r[0]), orc.from_i32(S_in))
+    pad_val = orc.fr_mul(orc.from_i32(fmap[-low: -low + 1])[0], r[0])
+    Spad = np.zeros((32768, 4), dtype=np.uint64)
+    orc.lib().orc_fr_pad(orc.P(Spad), orc.P(S), orc.c32(11008), orc.c32(16384), orc.c64(32768), orc.P(pad_val))
+    st, wtr, wsc = orc.tlookup_prove(Spad, T, B, m, alpha[0], beta, u, v)
+    assert st == 0
+    table = ops.g1_table_gen(dg[:16].contiguous(), 256)
+    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
+    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
+    tr, sc = host.tlookup_mapping_prove(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
+    assert_same(tr, wtr, "transcript")
+    assert_same(sc, wsc, "S(v)")
+
+
 def test_hyrax_class_commits(ops, host, gens):
     import torch
     hg, dg = gens
