@@ -99,7 +99,7 @@ def layer_workload(args):
     from gpuutil import rand_fr
     ops.init(0)
     host.load()
-    host.lib_seed = host.load().grape_host_seed(12345)
+    host.load().grape_host_seed(12345)          # seeds the host classes' challenge generator
     T, D, H, HD, F = args.seq, 4096, 32, 128, 11008
     SH = 16
     dev = "cuda"
