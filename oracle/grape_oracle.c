@@ -31,6 +31,29 @@
 typedef unsigned __int128 u128;
 typedef uint64_t u64;
 
+/* limbs of 64 bits of a base-field element: 6 for BLS12-381 (default), 4 for BN254 (-DORC_BN254) */
+#if defined(ORC_BN254)
+#define FPL 4
+/* ------------------------------------------------------------------------------------------ */
+/* constants: include/field/alt_bn128.cuh:11-45, re-derived from closed forms (2^k mod m);      */
+/* curve y^2 = x^3 + 3 with generator (1, 2)                                                    */
+/* ------------------------------------------------------------------------------------------ */
+static const u64 FR_MOD[4] = {0x43e1f593f0000001ull, 0x2833e84879b97091ull, 0xb85045b68181585dull, 0x30644e72e131a029ull};
+static const u64 FR_ONE[4] = {0xac96341c4ffffffbull, 0x36fc76959f60cd29ull, 0x666ea36f7879462eull, 0x0e0a77c19a07df2full};
+static const u64 FR_RR[4] = {0x1bb8e645ae216da7ull, 0x53fe3ab1e35c59e3ull, 0x8c49833d53bb8085ull, 0x0216d0b17f4e44a5ull};
+static const u64 FR_PM2[4] = {0x43e1f593efffffffull, 0x2833e84879b97091ull, 0xb85045b68181585dull, 0x30644e72e131a029ull};
+#define FR_M0 0xc2e1f593efffffffull
+static const u64 FP_MOD[FPL] = {0x3c208c16d87cfd47ull, 0x97816a916871ca8dull, 0xb85045b68181585dull, 0x30644e72e131a029ull};
+static const u64 FP_ONE[FPL] = {0xd35d438dc58f0d9dull, 0x0a78eb28f5c70b3dull, 0x666ea36f7879462cull, 0x0e0a77c19a07df2full};
+static const u64 FP_RR[FPL] = {0xf32cfc5b538afa89ull, 0xb5e71911d44501fbull, 0x47ab1eff0a417ff6ull, 0x06d89f71cab8351full};
+static const u64 FP_PM2[FPL] = {0x3c208c16d87cfd45ull, 0x97816a916871ca8dull, 0xb85045b68181585dull, 0x30644e72e131a029ull};
+#define FP_M0 0x87d20782e4866389ull
+static const u64 G1_GX[FPL] = {0xd35d438dc58f0d9dull, 0x0a78eb28f5c70b3dull, 0x666ea36f7879462cull, 0x0e0a77c19a07df2full};
+static const u64 G1_GY[FPL] = {0xa6ba871b8b1e1b3aull, 0x14f1d651eb8e167bull, 0xccdd46def0f28c58ull, 0x1c14ef83340fbe5eull};
+static const u64 G1_B[FPL] = {0x7a17caa950ad28d7ull, 0x1f6ac17ae15521b9ull, 0x334bea4e696bd284ull, 0x2a1f6744ce179d8eull};
+
+#else
+#define FPL 6
 /* ------------------------------------------------------------------------------------------ */
 /* constants: include/field/bls12-381.cuh:7-45, re-derived from closed forms (2^k mod m)        */
 /* ------------------------------------------------------------------------------------------ */
@@ -44,22 +67,24 @@ static const u64 FR_PM2[4] = {0xfffffffeffffffffull, 0x53bda402fffe5bfeull, 0x33
                               0x73eda753299d7d48ull};
 #define FR_M0 0xfffffffeffffffffull
 
-static const u64 FP_MOD[6] = {0xb9feffffffffaaabull, 0x1eabfffeb153ffffull, 0x6730d2a0f6b0f624ull,
+static const u64 FP_MOD[FPL] = {0xb9feffffffffaaabull, 0x1eabfffeb153ffffull, 0x6730d2a0f6b0f624ull,
                               0x64774b84f38512bfull, 0x4b1ba7b6434bacd7ull, 0x1a0111ea397fe69aull};
-static const u64 FP_ONE[6] = {0x760900000002fffdull, 0xebf4000bc40c0002ull, 0x5f48985753c758baull,
+static const u64 FP_ONE[FPL] = {0x760900000002fffdull, 0xebf4000bc40c0002ull, 0x5f48985753c758baull,
                               0x77ce585370525745ull, 0x5c071a97a256ec6dull, 0x15f65ec3fa80e493ull};
-static const u64 FP_RR[6] = {0xf4df1f341c341746ull, 0x0a76e6a609d104f1ull, 0x8de5476c4c95b6d5ull,
+static const u64 FP_RR[FPL] = {0xf4df1f341c341746ull, 0x0a76e6a609d104f1ull, 0x8de5476c4c95b6d5ull,
                              0x67eb88a9939d83c0ull, 0x9a793e85b519952dull, 0x11988fe592cae3aaull};
-static const u64 FP_PM2[6] = {0xb9feffffffffaaa9ull, 0x1eabfffeb153ffffull, 0x6730d2a0f6b0f624ull,
+static const u64 FP_PM2[FPL] = {0xb9feffffffffaaa9ull, 0x1eabfffeb153ffffull, 0x6730d2a0f6b0f624ull,
                               0x64774b84f38512bfull, 0x4b1ba7b6434bacd7ull, 0x1a0111ea397fe69aull};
 #define FP_M0 0x89f3fffcfffcfffdull
 /* standard G1 generator, Montgomery form */
-static const u64 G1_GX[6] = {0x5cb38790fd530c16ull, 0x7817fc679976fff5ull, 0x154f95c7143ba1c1ull,
+static const u64 G1_GX[FPL] = {0x5cb38790fd530c16ull, 0x7817fc679976fff5ull, 0x154f95c7143ba1c1ull,
                              0xf0ae6acdf3d0e747ull, 0xedce6ecc21dbf440ull, 0x120177419e0bfb75ull};
-static const u64 G1_GY[6] = {0xbaac93d50ce72271ull, 0x8c22631a7918fd8eull, 0xdd595f13570725ceull,
+static const u64 G1_GY[FPL] = {0xbaac93d50ce72271ull, 0x8c22631a7918fd8eull, 0xdd595f13570725ceull,
                              0x51ac582950405194ull, 0x0e1c8c3fad0059c0ull, 0x0bbc3efc5008a26aull};
-static const u64 G1_B[6] = {0xaa270000000cfff3ull, 0x53cc0032fc34000aull, 0x478fe97a6b0a807full,
+static const u64 G1_B[FPL] = {0xaa270000000cfff3ull, 0x53cc0032fc34000aull, 0x478fe97a6b0a807full,
                             0xb1d37ebee6ba24d7ull, 0x8ec9733bbf78ab2full, 0x09d645513d83de7eull};
+
+#endif
 
 /* ------------------------------------------------------------------------------------------ */
 /* generic n-limb Montgomery arithmetic (semantics of include/field/mont_t.cuh: canonical       */
@@ -169,14 +194,14 @@ static void fr_from_i64(u64 *r, int64_t x) {
     if (x < 0) fr_neg(r, r);
 }
 /* ---- Fp ---- */
-static inline void fp_add(u64 *r, const u64 *a, const u64 *b) { mod_add(r, a, b, FP_MOD, 6); }
-static inline void fp_sub(u64 *r, const u64 *a, const u64 *b) { mod_sub(r, a, b, FP_MOD, 6); }
-static inline void fp_mul(u64 *r, const u64 *a, const u64 *b) { mont_mul_n(r, a, b, FP_MOD, FP_M0, 6); }
-static inline void fp_sqr(u64 *r, const u64 *a) { mont_mul_n(r, a, a, FP_MOD, FP_M0, 6); }
-static inline void fp_neg(u64 *r, const u64 *a) { mod_neg(r, a, FP_MOD, 6); }
-static inline void fp_inv(u64 *r, const u64 *a) { mont_inv_n(r, a, FP_MOD, FP_M0, FP_ONE, FP_PM2, 6); }
-static inline void fp_cpy(u64 *r, const u64 *a) { memcpy(r, a, 48); }
-static inline int fp_is_zero(const u64 *a) { return is_zero_n(a, 6); }
+static inline void fp_add(u64 *r, const u64 *a, const u64 *b) { mod_add(r, a, b, FP_MOD, FPL); }
+static inline void fp_sub(u64 *r, const u64 *a, const u64 *b) { mod_sub(r, a, b, FP_MOD, FPL); }
+static inline void fp_mul(u64 *r, const u64 *a, const u64 *b) { mont_mul_n(r, a, b, FP_MOD, FP_M0, FPL); }
+static inline void fp_sqr(u64 *r, const u64 *a) { mont_mul_n(r, a, a, FP_MOD, FP_M0, FPL); }
+static inline void fp_neg(u64 *r, const u64 *a) { mod_neg(r, a, FP_MOD, FPL); }
+static inline void fp_inv(u64 *r, const u64 *a) { mont_inv_n(r, a, FP_MOD, FP_M0, FP_ONE, FP_PM2, FPL); }
+static inline void fp_cpy(u64 *r, const u64 *a) { memcpy(r, a, 8 * FPL); }
+static inline int fp_is_zero(const u64 *a) { return is_zero_n(a, FPL); }
 
 int orc_num_threads(void) {
 #ifdef _OPENMP
@@ -216,7 +241,7 @@ void orc_fp_neg(u64 *r, const u64 *a) { fp_neg(r, a); }
 void orc_fp_inv(u64 *r, const u64 *a) { fp_inv(r, a); }
 void orc_fp_to_mont(u64 *r, const u64 *a) { fp_mul(r, a, FP_RR); }
 void orc_fp_from_mont(u64 *r, const u64 *a) {
-    u64 one[6] = {1, 0, 0, 0, 0, 0};
+    u64 one[FPL] = {1};
     fp_mul(r, a, one);
 }
 
@@ -364,8 +389,8 @@ void orc_fr_mle_eval(u64 *out, u64 *t, uint64_t size, const u64 *u, uint32_t nu)
 /* ------------------------------------------------------------------------------------------ */
 /* G1: include/curve/{affine_t,jacobian_t,xyzz_t}.cuh                                           */
 /* ------------------------------------------------------------------------------------------ */
-typedef struct { u64 x[6], y[6]; } aff_t;
-typedef struct { u64 x[6], y[6], zz[6], zzz[6]; } xyzz_t;
+typedef struct { u64 x[FPL], y[FPL]; } aff_t;
+typedef struct { u64 x[FPL], y[FPL], zz[FPL], zzz[FPL]; } xyzz_t;
 
 static inline int aff_is_inf(const aff_t *p) { return fp_is_zero(p->x) && fp_is_zero(p->y); }
 static inline int xyzz_is_inf(const xyzz_t *p) { return fp_is_zero(p->zz); }
@@ -374,7 +399,7 @@ static inline void xyzz_set_inf(xyzz_t *p) { memset(p, 0, sizeof *p); }
 /* acc += +-p: xyzz_t::add(affine, subtract) xyzz_t.cuh:363-441 */
 static void xyzz_madd(xyzz_t *acc, const aff_t *p, int subtract) {
     if (aff_is_inf(p)) return;
-    u64 py[6];
+    u64 py[FPL];
     if (subtract) fp_neg(py, p->y);
     else fp_cpy(py, p->y);
     if (xyzz_is_inf(acc)) {
@@ -384,7 +409,7 @@ static void xyzz_madd(xyzz_t *acc, const aff_t *p, int subtract) {
         fp_cpy(acc->zzz, FP_ONE);
         return;
     }
-    u64 P[6], R[6], PP[6], PPP[6], Q[6], X3[6], t[6];
+    u64 P[FPL], R[FPL], PP[FPL], PPP[FPL], Q[FPL], X3[FPL], t[FPL];
     fp_mul(P, p->x, acc->zz);
     fp_sub(P, P, acc->x);
     fp_mul(R, py, acc->zzz);
@@ -405,7 +430,7 @@ static void xyzz_madd(xyzz_t *acc, const aff_t *p, int subtract) {
         fp_mul(acc->zz, acc->zz, PP);
         fp_mul(acc->zzz, acc->zzz, PPP);
     } else if (fp_is_zero(R)) {
-        u64 U[6], V[6], W[6], S[6], M[6];
+        u64 U[FPL], V[FPL], W[FPL], S[FPL], M[FPL];
         fp_add(U, py, py);
         fp_sqr(V, U);
         fp_mul(W, U, V);
@@ -430,7 +455,7 @@ static void xyzz_madd(xyzz_t *acc, const aff_t *p, int subtract) {
 /* acc = 2*acc (dbl-2008-s-1 as in xyzz_t.cuh:170-200) */
 static void xyzz_dbl(xyzz_t *acc) {
     if (xyzz_is_inf(acc)) return;
-    u64 U[6], V[6], W[6], S[6], M[6], X3[6], t[6];
+    u64 U[FPL], V[FPL], W[FPL], S[FPL], M[FPL], X3[FPL], t[FPL];
     fp_add(U, acc->y, acc->y);
     fp_sqr(V, U);
     fp_mul(W, U, V);
@@ -456,7 +481,7 @@ static void xyzz_add(xyzz_t *acc, const xyzz_t *q) {
         *acc = *q;
         return;
     }
-    u64 U1[6], S1[6], P[6], R[6], PP[6], PPP[6], Q[6], X3[6], t[6];
+    u64 U1[FPL], S1[FPL], P[FPL], R[FPL], PP[FPL], PPP[FPL], Q[FPL], X3[FPL], t[FPL];
     fp_mul(U1, acc->x, q->zz);
     fp_mul(S1, acc->y, q->zzz);
     fp_mul(P, q->x, acc->zz);
@@ -492,7 +517,7 @@ static void xyzz_to_affine(aff_t *r, const xyzz_t *p) {
         memset(r, 0, sizeof *r);
         return;
     }
-    u64 zi[6], zzi[6];
+    u64 zi[FPL], zzi[FPL];
     fp_inv(zi, p->zzz);       /* 1/ZZZ */
     fp_mul(r->y, p->y, zi);
     fp_mul(zzi, zi, p->zz);   /* 1/Z */
@@ -515,18 +540,18 @@ static void g1_scalar_mul(aff_t *out, const aff_t *p, const u64 *k) {
 }
 
 void orc_g1_generator(u64 *out) {
-    memcpy(out, G1_GX, 48);
-    memcpy(out + 6, G1_GY, 48);
+    memcpy(out, G1_GX, 8 * FPL);
+    memcpy(out + FPL, G1_GY, 8 * FPL);
 }
 int orc_g1_on_curve(const u64 *p) {
     const aff_t *a = (const aff_t *)p;
     if (aff_is_inf(a)) return 1;
-    u64 l[6], r[6];
+    u64 l[FPL], r[FPL];
     fp_sqr(l, a->y);
     fp_sqr(r, a->x);
     fp_mul(r, r, a->x);
     fp_add(r, r, G1_B);
-    return memcmp(l, r, 48) == 0;
+    return memcmp(l, r, 8 * FPL) == 0;
 }
 void orc_g1_add_affine(u64 *out, const u64 *a, const u64 *b) {
     xyzz_t acc;
@@ -541,19 +566,19 @@ void orc_g1_make_generators(u64 *out, const u64 *k, uint64_t n) {
     aff_t g;
     orc_g1_generator((u64 *)&g);
 #pragma omp parallel for schedule(dynamic, 4)
-    for (int64_t i = 0; i < (int64_t)n; i++) g1_scalar_mul((aff_t *)(out + 12 * i), &g, k + 4 * i);
+    for (int64_t i = 0; i < (int64_t)n; i++) g1_scalar_mul((aff_t *)(out + 2 * FPL * i), &g, k + 4 * i);
 }
 /* jacobian_t -> affine, jacobian_t.cuh:33-41 */
 void orc_g1_jac_to_affine(u64 *out, const u64 *in, uint64_t n) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < (int64_t)n; i++) {
-        const u64 *X = in + 18 * i, *Y = X + 6, *Z = X + 12;
-        aff_t *r = (aff_t *)(out + 12 * i);
+        const u64 *X = in + 3 * FPL * i, *Y = X + FPL, *Z = X + 2 * FPL;
+        aff_t *r = (aff_t *)(out + 2 * FPL * i);
         if (fp_is_zero(Z)) {
             memset(r, 0, sizeof *r);
             continue;
         }
-        u64 zi[6], zi2[6], zi3[6];
+        u64 zi[FPL], zi2[FPL], zi3[FPL];
         fp_inv(zi, Z);
         fp_sqr(zi2, zi);
         fp_mul(zi3, zi2, zi);
@@ -565,11 +590,11 @@ void orc_g1_jac_to_affine(u64 *out, const u64 *in, uint64_t n) {
 void orc_g1_table(u64 *table, const u64 *gens, uint64_t N, uint32_t W) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < (int64_t)N; i++) {
-        const aff_t *g = (const aff_t *)(gens + 12 * i);
+        const aff_t *g = (const aff_t *)(gens + 2 * FPL * i);
         xyzz_t res;
         xyzz_set_inf(&res);
         for (uint32_t w = 0; w < W; w++) {
-            xyzz_to_affine((aff_t *)(table + 12 * ((uint64_t)w * N + i)), &res);
+            xyzz_to_affine((aff_t *)(table + 2 * FPL * ((uint64_t)w * N + i)), &res);
             xyzz_madd(&res, g, 0);
         }
     }
@@ -599,7 +624,7 @@ void orc_commit_i32(u64 *out, const int32_t *scalars, const u64 *table, uint64_t
             for (int d = 0; d < 8; d++) xyzz_dbl(&total);
             xyzz_add(&total, &sum);
         }
-        xyzz_to_affine((aff_t *)(out + 12 * r), &total);
+        xyzz_to_affine((aff_t *)(out + 2 * FPL * r), &total);
     }
 }
 /*
@@ -626,7 +651,7 @@ void orc_commit_fr(u64 *out, const u64 *scalars, const u64 *table, uint64_t size
             for (int d = 0; d < 8; d++) xyzz_dbl(&total);
             xyzz_add(&total, &sum);
         }
-        xyzz_to_affine((aff_t *)(out + 12 * r), &total);
+        xyzz_to_affine((aff_t *)(out + 2 * FPL * r), &total);
     }
 }
 /* brute force sum_i s_i*G_i by double-and-add (the check commented out at test/HyraxTest.cu:146-178) */
@@ -637,7 +662,7 @@ void orc_msm_naive_i64(u64 *out, const int64_t *scalars, const u64 *gens, uint64
         int64_t s = scalars[i];
         u64 k[4] = {s < 0 ? (u64)0 - (u64)s : (u64)s, 0, 0, 0};
         aff_t t;
-        g1_scalar_mul(&t, (const aff_t *)(gens + 12 * i), k);
+        g1_scalar_mul(&t, (const aff_t *)(gens + 2 * FPL * i), k);
         xyzz_madd(&total, &t, s < 0);
     }
     xyzz_to_affine((aff_t *)out, &total);

@@ -9,6 +9,9 @@
  * Memory formats are the reference's: an Fr element is 4 x u64 little-endian limbs holding the
  * canonical Montgomery residue x*2^256 mod r; an Fp element is 6 x u64 (x*2^384 mod p); an affine
  * G1 point is (x, y) = 12 x u64 with infinity = all zero; a Jacobian point is 18 x u64.
+ * Compiled with -DORC_BN254 the same code is the BN254 instantiation (the reference's
+ * include/field/alt_bn128.cuh): Fp is 4 x u64 (x*2^256 mod p), an affine point 8 x u64, a
+ * Jacobian point 12 x u64, the curve y^2 = x^3 + 3 with generator (1, 2).
  *
  * How each function is pinned (what independent check guards it) is listed in grape_oracle.c.
  */
@@ -20,7 +23,11 @@ extern "C" {
 #endif
 
 typedef uint64_t orc_fr[4];
+#if defined(ORC_BN254)
+typedef uint64_t orc_fp[4];
+#else
 typedef uint64_t orc_fp[6];
+#endif
 
 int orc_num_threads(void);
 uint32_t orc_log2(uint32_t n);

@@ -5,14 +5,30 @@ Nothing here shares code with the oracle or the HIP library: field operations ar
 rule, multilinear extensions are evaluated by brute force from their definition.  The tests
 compare the oracle (64-bit limbs, Montgomery form) with these closed forms.
 """
+import os
 import numpy as np
 
-R_MOD = 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001
-P_MOD = 0x1a0111ea397fe69a4b1ba7b6434bacd764774b84f38512bf6730d2a0f6b0f6241eabfffeb153ffffb9feffffffffaaab
-FR_R = 1 << 256   # Montgomery radix of Fr
-FP_R = 1 << 384   # Montgomery radix of Fp
-G1_X = 0x17f1d3a73197d7942695638c4fa9ac0fc3688c4f9774b905a14e3a3f171bac586c55e83ff97a1aeffb3af00adb22c6bb
-G1_Y = 0x08b3f481e3aaa0f1a09e30ed741d8ae4fcf5e095d5d00af600db18cb2c04b3edd03cc744a2888ae40caa232946c5e7e1
+# The curve is chosen by the environment variable GRAPE_CURVE: "bls12_381" (default, the curve of
+# the benchmark configurations) or "bn254" (the reference's active curve).
+CURVE = os.environ.get("GRAPE_CURVE", "bls12_381")
+if CURVE == "bn254":
+    R_MOD = 21888242871839275222246405745257275088548364400416034343698204186575808495617
+    P_MOD = 21888242871839275222246405745257275088696311157297823662689037894645226208583
+    FP_LIMBS = 4      # 64-bit limbs of a base-field element
+    CURVE_B = 3
+    G1_X, G1_Y = 1, 2
+elif CURVE == "bls12_381":
+    R_MOD = 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001
+    P_MOD = 0x1a0111ea397fe69a4b1ba7b6434bacd764774b84f38512bf6730d2a0f6b0f6241eabfffeb153ffffb9feffffffffaaab
+    FP_LIMBS = 6
+    CURVE_B = 4
+    G1_X = 0x17f1d3a73197d7942695638c4fa9ac0fc3688c4f9774b905a14e3a3f171bac586c55e83ff97a1aeffb3af00adb22c6bb
+    G1_Y = 0x08b3f481e3aaa0f1a09e30ed741d8ae4fcf5e095d5d00af600db18cb2c04b3edd03cc744a2888ae40caa232946c5e7e1
+else:
+    raise ValueError("GRAPE_CURVE must be bls12_381 or bn254, not %r" % CURVE)
+FR_R = 1 << 256                  # Montgomery radix of Fr
+FP_R = 1 << (64 * FP_LIMBS)      # Montgomery radix of Fp
+G1_WORDS = 2 * FP_LIMBS          # 64-bit words of an affine point
 G1 = (G1_X, G1_Y)
 
 
@@ -44,28 +60,28 @@ def fr_unpack(arr):
 
 
 def fp_pack(vals):
-    return ints_to_limbs([(v % P_MOD) * FP_R % P_MOD for v in vals], 6)
+    return ints_to_limbs([(v % P_MOD) * FP_R % P_MOD for v in vals], FP_LIMBS)
 
 
 def fp_unpack(arr):
     rinv = pow(FP_R, -1, P_MOD)
-    return [x * rinv % P_MOD for x in limbs_to_ints(np.asarray(arr).reshape(-1, 6))]
+    return [x * rinv % P_MOD for x in limbs_to_ints(np.asarray(arr).reshape(-1, FP_LIMBS))]
 
 
 def g1_pack(points):
-    """list of affine points (x,y) or None (infinity) -> (n,12) uint64 Montgomery."""
+    """list of affine points (x,y) or None (infinity) -> (n, G1_WORDS) uint64 Montgomery."""
     flat = []
     for pt in points:
         if pt is None:
             flat += [0, 0]
         else:
             flat += [pt[0], pt[1]]
-    return fp_pack(flat).reshape(len(points), 12)
+    return fp_pack(flat).reshape(len(points), G1_WORDS)
 
 
 def g1_unpack(arr):
-    arr = np.asarray(arr, dtype=np.uint64).reshape(-1, 12)
-    coords = fp_unpack(arr.reshape(-1, 6))
+    arr = np.asarray(arr, dtype=np.uint64).reshape(-1, G1_WORDS)
+    coords = fp_unpack(arr.reshape(-1, FP_LIMBS))
     out = []
     for i in range(arr.shape[0]):
         x, y = coords[2 * i], coords[2 * i + 1]
@@ -78,7 +94,7 @@ def g1_on_curve(pt):
     if pt is None:
         return True
     x, y = pt
-    return (y * y - x * x * x - 4) % P_MOD == 0
+    return (y * y - x * x * x - CURVE_B) % P_MOD == 0
 
 
 def g1_neg(pt):

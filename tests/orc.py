@@ -5,6 +5,8 @@ import os
 import subprocess
 import numpy as np
 
+from bigref import FP_LIMBS as FPL, G1_WORDS as G1W
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _ORACLE_DIR = os.path.join(os.path.dirname(_HERE), "oracle")
 _LIB = None
@@ -18,7 +20,9 @@ i64p = ctypes.POINTER(ctypes.c_int64)
 def lib():
     global _LIB
     if _LIB is None:
-        path = os.path.join(_ORACLE_DIR, "libgrape_oracle.so")
+        import bigref
+        name = "libgrape_oracle_bn254.so" if bigref.CURVE == "bn254" else "libgrape_oracle.so"
+        path = os.path.join(_ORACLE_DIR, name)
         if not os.path.exists(path):
             subprocess.check_call(["make", "-C", _ORACLE_DIR, "-s"])
         _LIB = ctypes.CDLL(path)
@@ -71,11 +75,11 @@ def fr_sub(a, b): return _bin("orc_fr_sub", a, b)
 def fr_mul(a, b): return _bin("orc_fr_mul", a, b)
 def fr_neg(a): return _un("orc_fr_neg", a)
 def fr_inv(a): return _un("orc_fr_inv", a)
-def fp_add(a, b): return _bin("orc_fp_add", a, b, 6)
-def fp_sub(a, b): return _bin("orc_fp_sub", a, b, 6)
-def fp_mul(a, b): return _bin("orc_fp_mul", a, b, 6)
-def fp_neg(a): return _un("orc_fp_neg", a, 6)
-def fp_inv(a): return _un("orc_fp_inv", a, 6)
+def fp_add(a, b): return _bin("orc_fp_add", a, b, FPL)
+def fp_sub(a, b): return _bin("orc_fp_sub", a, b, FPL)
+def fp_mul(a, b): return _bin("orc_fp_mul", a, b, FPL)
+def fp_neg(a): return _un("orc_fp_neg", a, FPL)
+def fp_inv(a): return _un("orc_fp_inv", a, FPL)
 
 
 def vec2(name, a, b):
@@ -139,22 +143,22 @@ def mle_eval(t, u):
 
 
 def g1_generator():
-    r = np.zeros(12, dtype=np.uint64)
+    r = np.zeros(G1W, dtype=np.uint64)
     lib().orc_g1_generator(P(r))
     return r
 
 
 def g1_make_generators(k_plain):
     k = np.ascontiguousarray(k_plain, dtype=np.uint64).reshape(-1, 4)
-    r = np.zeros((k.shape[0], 12), dtype=np.uint64)
+    r = np.zeros((k.shape[0], G1W), dtype=np.uint64)
     lib().orc_g1_make_generators(P(r), P(k), c64(k.shape[0]))
     return r
 
 
 def g1_table(gens, W):
-    gens = np.ascontiguousarray(gens, dtype=np.uint64).reshape(-1, 12)
+    gens = np.ascontiguousarray(gens, dtype=np.uint64).reshape(-1, G1W)
     n = gens.shape[0]
-    r = np.zeros((W * n, 12), dtype=np.uint64)
+    r = np.zeros((W * n, G1W), dtype=np.uint64)
     lib().orc_g1_table(P(r), P(gens), c64(n), c32(W))
     return r
 
@@ -163,7 +167,7 @@ def commit_i32(scalars, table, rowlen, npoints):
     s = np.ascontiguousarray(scalars, dtype=np.int32).reshape(-1)
     table = np.ascontiguousarray(table, dtype=np.uint64)
     rows = s.shape[0] // rowlen
-    r = np.zeros((rows, 12), dtype=np.uint64)
+    r = np.zeros((rows, G1W), dtype=np.uint64)
     lib().orc_commit_i32(P(r), P(s, i32p), P(table), c64(s.shape[0]), c32(rowlen), c64(npoints))
     return r
 
@@ -172,15 +176,15 @@ def commit_fr(scalars_mont, table, rowlen, npoints):
     s = np.ascontiguousarray(scalars_mont, dtype=np.uint64).reshape(-1, 4)
     table = np.ascontiguousarray(table, dtype=np.uint64)
     rows = s.shape[0] // rowlen
-    r = np.zeros((rows, 12), dtype=np.uint64)
+    r = np.zeros((rows, G1W), dtype=np.uint64)
     lib().orc_commit_fr(P(r), P(s), P(table), c64(s.shape[0]), c32(rowlen), c64(npoints))
     return r
 
 
 def msm_naive_i64(scalars, gens):
     s = np.ascontiguousarray(scalars, dtype=np.int64).reshape(-1)
-    gens = np.ascontiguousarray(gens, dtype=np.uint64).reshape(-1, 12)
-    r = np.zeros(12, dtype=np.uint64)
+    gens = np.ascontiguousarray(gens, dtype=np.uint64).reshape(-1, G1W)
+    r = np.zeros(G1W, dtype=np.uint64)
     lib().orc_msm_naive_i64(P(r), P(s, i64p), P(gens), c64(s.shape[0]))
     return r
 

@@ -177,7 +177,7 @@ def test_jacobian_conversions(ops, gens64):
     jac = ops.g1_affine_to_jacobian(dev)
     back = ops.g1_jacobian_to_affine(jac)
     assert_same(ops.g1_to_host(back), host, "affine -> jacobian -> affine")
-    hj = jac.cpu().numpy().view(np.uint64).reshape(-1, 18)
-    want = np.zeros((64, 12), dtype=np.uint64)
+    hj = jac.cpu().numpy().view(np.uint64).reshape(-1, 3 * br.FP_LIMBS)
+    want = np.zeros((64, br.G1_WORDS), dtype=np.uint64)
     orc.lib().orc_g1_jac_to_affine(orc.P(want), orc.P(np.ascontiguousarray(hj)), orc.c64(64))
     assert_same(want, host, "oracle jacobian -> affine")

@@ -323,8 +323,8 @@ def test_file_helpers_and_on_disk_formats(ops, host, gens, tmp_path):
     ops.sync()
     f_pts = str(tmp_path / "points.bin")
     host.savebin(f_pts, table.data_ptr(), table.numel() * 4)
-    assert host.findsize(f_pts) == 256 * npoints * 96
-    assert np.array_equal(np.fromfile(f_pts, dtype=np.uint64).reshape(-1, 12), orc.g1_table(hg, 256))
+    assert host.findsize(f_pts) == 256 * npoints * 8 * br.G1_WORDS
+    assert np.array_equal(np.fromfile(f_pts, dtype=np.uint64).reshape(-1, br.G1_WORDS), orc.g1_table(hg, 256))
     table2 = torch.zeros_like(table)
     host.loadbin(f_pts, table2.data_ptr(), table2.numel() * 4)
     assert torch.equal(table, table2)

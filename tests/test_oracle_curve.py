@@ -16,7 +16,7 @@ def test_generator_and_order():
     g = br.g1_unpack(orc.g1_generator())[0]
     assert g == br.G1 and br.g1_on_curve(g)
     assert br.g1_mul(br.R_MOD, br.G1) is None            # the group has order r
-    out = np.zeros(12, dtype=np.uint64)
+    out = np.zeros(br.G1_WORDS, dtype=np.uint64)
     orc.lib().orc_g1_scalar_mul(orc.P(out), orc.P(orc.g1_generator()), orc.P(br.ints_to_limbs([br.R_MOD], 4)))
     assert br.g1_unpack(out)[0] is None
 
@@ -36,7 +36,7 @@ def test_add_special_cases():
     b = br.g1_mul(7, br.G1)
     cases = [(a, b), (a, a), (a, br.g1_neg(a)), (None, a), (a, None), (None, None)]
     for x, y in cases:
-        out = np.zeros(12, dtype=np.uint64)
+        out = np.zeros(br.G1_WORDS, dtype=np.uint64)
         orc.lib().orc_g1_add_affine(orc.P(out), orc.P(br.g1_pack([x])[0]), orc.P(br.g1_pack([y])[0]))
         assert br.g1_unpack(out)[0] == br.g1_add(x, y)
 
