@@ -7,7 +7,13 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libgrape_hip.so")
+# One curve per process, fixed when the library is compiled: GRAPE_CURVE = bls12_381 (default) or
+# bn254 picks which build is loaded.
+CURVE = os.environ.get("GRAPE_CURVE", "bls12_381")
+if CURVE not in ("bls12_381", "bn254"):
+    raise ValueError("GRAPE_CURVE must be bls12_381 or bn254, not %r" % CURVE)
+LIB_PATH = os.path.join(_HERE, "libgrape_hip_bn254.so" if CURVE == "bn254" else "libgrape_hip.so")
+FP_WORDS = 8 if CURVE == "bn254" else 12      # 32-bit words of an Fp element in memory
 
 c_void_p = ctypes.c_void_p
 c_size_t = ctypes.c_size_t
@@ -91,7 +97,7 @@ class GrapeError(RuntimeError):
 
 
 def load():
-    """Load libgrape_hip.so and declare every entry point; raises if the library is missing."""
+    """Load the kernel library of the chosen curve and declare every entry point; raises if the library is missing."""
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):

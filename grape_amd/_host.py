@@ -4,7 +4,9 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "host", "libgrape_host.so")
+from ._capi import CURVE, FP_WORDS
+LIB_PATH = os.path.join(_HERE, "host", "libgrape_host_bn254.so" if CURVE == "bn254" else "libgrape_host.so")
+G1W = FP_WORDS              # u64 words of an affine point (2 coordinates of FP_WORDS / 2)
 _lib = None
 
 NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
@@ -124,7 +126,7 @@ def mle_eval(dT, size, u):
 def hyrax_commit_i32(d_scalars, size, N, d_table, npoints, com_scale=16, layer_num=1):
     lib = load()
     rows = size // (N * com_scale)
-    out = np.zeros((rows, 12), dtype=np.uint64)
+    out = np.zeros((rows, G1W), dtype=np.uint64)
     _check(lib.grape_host_hyrax_commit_i32(_dp(d_scalars), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(out)))
     return out
 
@@ -132,7 +134,7 @@ def hyrax_commit_i32(d_scalars, size, N, d_table, npoints, com_scale=16, layer_n
 def hyrax_commit_fr(d_scalars, size, N, d_table, npoints, com_scale=16, layer_num=1):
     lib = load()
     rows = size // (N * com_scale)
-    out = np.zeros((rows, 12), dtype=np.uint64)
+    out = np.zeros((rows, G1W), dtype=np.uint64)
     _check(lib.grape_host_hyrax_commit_fr(_dp(d_scalars), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(out)))
     return out
 
@@ -157,10 +159,10 @@ def tlookup_range_prove(dS, D, low, length, alpha, u, v, d_table, npoints, com_s
     nr = ctypes.c_uint32(0)
     sc = np.zeros(4, dtype=np.uint64)
     Dp = 1 << max(0, (D - 1).bit_length())
-    comA = np.zeros((Dp // (msm_size * com_scale), 12), dtype=np.uint64) if want_commitments else None
+    comA = np.zeros((Dp // (msm_size * com_scale), G1W), dtype=np.uint64) if want_commitments else None
     logn = (size - 1).bit_length()
     mN = 1 << (logn // 2)
-    comm = np.zeros((size // (mN * com_scale), 12), dtype=np.uint64) if want_commitments else None
+    comm = np.zeros((size // (mN * com_scale), G1W), dtype=np.uint64) if want_commitments else None
     ct = ctypes.c_double(0)
     _check(lib.grape_host_tlookup_range_prove(_dp(dS), D, low, length, _hp(alpha), _hp(u), _hp(v), u.shape[0], _dp(d_table),
                                               npoints, com_scale, msm_size, _hp(m), _hp(tr), ctypes.byref(nr), _hp(sc),
@@ -193,7 +195,7 @@ def fr_op(op, a, b=None):
 def g1_mul_generator(k_mont):
     lib = load()
     k = _fr(k_mont, 1)
-    out = np.zeros(12, dtype=np.uint64)
+    out = np.zeros(G1W, dtype=np.uint64)
     _check(lib.grape_host_g1_mul_generator(_hp(k), _hp(out)))
     return out
 
@@ -225,6 +227,6 @@ def generate_data(size):
 
 
 def single_commit(d_scalars, N, d_table, npoints):
-    out = np.zeros(12, dtype=np.uint64)
+    out = np.zeros(G1W, dtype=np.uint64)
     _check(load().grape_host_single_commit(_dp(d_scalars), N, _dp(d_table), npoints, _hp(out)))
     return out

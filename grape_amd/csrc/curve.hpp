@@ -1,4 +1,5 @@
-// BLS12-381 G1 (y^2 = x^3 + 4 over Fp) group law on Montgomery-form coordinates.
+// G1 group law (short Weierstrass, a = 0: BLS12-381 y^2 = x^3 + 4, BN254 y^2 = x^3 + 3) on
+// Montgomery-form coordinates; the formulas never use b, so one body serves both curves.
 //
 // Point encodings follow the reference: affine infinity is (0,0) (include/curve/affine_t.cuh:28-39),
 // a Jacobian point is at infinity when Z = 0 (include/curve/jacobian_t.cuh), an extended-Jacobian
@@ -33,9 +34,9 @@ GRAPE_HD Fp fp_inverse(const Fp& a) {
     for (int i = 2; i < 16; i++) tbl[i] = fmul(tbl[i - 1], a);
     Fp acc = Fp::one();
     bool started = false;
-    for (int limb = 11; limb >= 0; limb--) {
+    for (int limb = FpParams::N - 1; limb >= 0; limb--) {
         uint32_t e = 0;
-        for (int k = 0; k < 12; k++) e = (k == limb) ? FpParams::pm2(k) : e;
+        for (int k = 0; k < FpParams::N; k++) e = (k == limb) ? FpParams::pm2(k) : e;
         for (int nib = 7; nib >= 0; nib--) {
             if (started) {
                 acc = fsqr(acc);
@@ -51,6 +52,29 @@ GRAPE_HD Fp fp_inverse(const Fp& a) {
         }
     }
     return acc;
+}
+
+// Affine coordinates of the standard generator in memory (Montgomery) form: the usual BLS12-381
+// G1 generator resp. BN254's (1, 2) - what the reference's host group type calls one().
+GRAPE_HD uint32_t g1_gen_x(int i) {
+#if defined(GRAPE_CURVE_BN254)
+    constexpr uint32_t t[8] = {0xc58f0d9du, 0xd35d438du, 0xf5c70b3du, 0x0a78eb28u,
+                               0x7879462cu, 0x666ea36fu, 0x9a07df2fu, 0x0e0a77c1u};
+#else
+    constexpr uint32_t t[12] = {0xfd530c16u, 0x5cb38790u, 0x9976fff5u, 0x7817fc67u, 0x143ba1c1u, 0x154f95c7u,
+                                0xf3d0e747u, 0xf0ae6acdu, 0x21dbf440u, 0xedce6eccu, 0x9e0bfb75u, 0x12017741u};
+#endif
+    return t[i];
+}
+GRAPE_HD uint32_t g1_gen_y(int i) {
+#if defined(GRAPE_CURVE_BN254)
+    constexpr uint32_t t[8] = {0x8b1e1b3au, 0xa6ba871bu, 0xeb8e167bu, 0x14f1d651u,
+                               0xf0f28c58u, 0xccdd46deu, 0x340fbe5eu, 0x1c14ef83u};
+#else
+    constexpr uint32_t t[12] = {0x0ce72271u, 0xbaac93d5u, 0x7918fd8eu, 0x8c22631au, 0x570725ceu, 0xdd595f13u,
+                                0x50405194u, 0x51ac5829u, 0xad0059c0u, 0x0e1c8c3fu, 0x5008a26au, 0x0bbc3efcu};
+#endif
+    return t[i];
 }
 
 struct alignas(16) G1Affine {

@@ -25,6 +25,60 @@ namespace grape {
 // Parameter packs. Limb accessors are functions with local constexpr tables so that, after
 // unrolling, every modulus limb becomes a scalar literal on the device (no VGPRs, no loads).
 // ---------------------------------------------------------------------------------------------
+// The curve is chosen when the library is compiled: BLS12-381 (include/field/bls12-381.cuh) by
+// default, BN254 (include/field/alt_bn128.cuh) with -DGRAPE_CURVE_BN254.
+#if defined(GRAPE_CURVE_BN254)
+struct FrParams {   // BN254 scalar field (include/field/alt_bn128.cuh: ALT_BN128_r, rRR, rone, m0)
+    static constexpr int N = 8;
+    static constexpr uint32_t M0 = 0xefffffffu;  // -r^-1 mod 2^32
+    static GRAPE_HD uint32_t mod(int i) {
+        constexpr uint32_t t[8] = {0xf0000001u, 0x43e1f593u, 0x79b97091u, 0x2833e848u,
+                                   0x8181585du, 0xb85045b6u, 0xe131a029u, 0x30644e72u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t one(int i) {  // 2^256 mod r
+        constexpr uint32_t t[8] = {0x4ffffffbu, 0xac96341cu, 0x9f60cd29u, 0x36fc7695u,
+                                   0x7879462eu, 0x666ea36fu, 0x9a07df2fu, 0x0e0a77c1u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t rr(int i) {  // 2^512 mod r
+        constexpr uint32_t t[8] = {0xae216da7u, 0x1bb8e645u, 0xe35c59e3u, 0x53fe3ab1u,
+                                   0x53bb8085u, 0x8c49833du, 0x7f4e44a5u, 0x0216d0b1u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t pm2(int i) {  // r - 2 (Fermat exponent)
+        constexpr uint32_t t[8] = {0xefffffffu, 0x43e1f593u, 0x79b97091u, 0x2833e848u,
+                                   0x8181585du, 0xb85045b6u, 0xe131a029u, 0x30644e72u};
+        return t[i];
+    }
+};
+
+struct FpParams {   // BN254 base field (include/field/alt_bn128.cuh: ALT_BN128_P, RR, one, M0)
+    static constexpr int N = 8;
+    static constexpr uint32_t M0 = 0xe4866389u;  // -p^-1 mod 2^32
+    static GRAPE_HD uint32_t mod(int i) {
+        constexpr uint32_t t[8] = {0xd87cfd47u, 0x3c208c16u, 0x6871ca8du, 0x97816a91u,
+                                   0x8181585du, 0xb85045b6u, 0xe131a029u, 0x30644e72u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t one(int i) {  // 2^256 mod p
+        constexpr uint32_t t[8] = {0xc58f0d9du, 0xd35d438du, 0xf5c70b3du, 0x0a78eb28u,
+                                   0x7879462cu, 0x666ea36fu, 0x9a07df2fu, 0x0e0a77c1u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t rr(int i) {  // 2^512 mod p
+        constexpr uint32_t t[8] = {0x538afa89u, 0xf32cfc5bu, 0xd44501fbu, 0xb5e71911u,
+                                   0x0a417ff6u, 0x47ab1effu, 0xcab8351fu, 0x06d89f71u};
+        return t[i];
+    }
+    static GRAPE_HD uint32_t pm2(int i) {  // p - 2
+        constexpr uint32_t t[8] = {0xd87cfd45u, 0x3c208c16u, 0x6871ca8du, 0x97816a91u,
+                                   0x8181585du, 0xb85045b6u, 0xe131a029u, 0x30644e72u};
+        return t[i];
+    }
+};
+
+#else
 struct FrParams {
     static constexpr int N = 8;
     static constexpr uint32_t M0 = 0xffffffffu;  // -r^-1 mod 2^32
@@ -78,6 +132,8 @@ struct FpParams {
         return t[i];
     }
 };
+
+#endif
 
 // ---------------------------------------------------------------------------------------------
 // Field element

@@ -1,5 +1,5 @@
-// BLS12-381 Fp on 14 signed limbs of 28 bits with lazy reduction - the working form of the
-// commitment kernels.
+// Fp on signed limbs of 28 bits with lazy reduction - the working form of the commitment kernels
+// (14 limbs, radix 2^392, for BLS12-381; 10 limbs, radix 2^280, for BN254).
 //
 // Why: on gfx950 a 32x32+64 multiply-add (v_mad_i64_i32 / v_mad_u64_u32) issues at the same rate
 // as an addition, so the cost of a field product is its instruction count, and with saturated
@@ -9,19 +9,61 @@
 // borrow chain and no bias.
 //
 // Representation: x = sum_i v[i] * 2^(28 i), v[i] signed 32-bit.  "Normalised" means
-// 0 <= v[i] < 2^28 for i < 13 (the top limb carries the sign and the overflow).  A value stands
-// for its residue mod p; arithmetic is Montgomery with radix R' = 2^392.  The canonical memory
-// form elsewhere in the library is the reference's: 12 x 32-bit limbs, radix 2^384
-// (include/field/mont_t.cuh, include/field/bls12-381.cuh:7-23); conversion is exact both ways.
+// 0 <= v[i] < 2^28 for i < N-1 (the top limb carries the sign and the overflow).  A value stands
+// for its residue mod p; arithmetic is Montgomery with radix R' = 2^(28 N).  The canonical memory
+// form elsewhere in the library is the reference's: 32-bit limbs, radix 2^384 resp. 2^256
+// (include/field/mont_t.cuh, include/field/bls12-381.cuh:7-23, include/field/alt_bn128.cuh);
+// conversion is exact both ways.
 //
 // Bounds (checked by the callers' comments): mul28(a, b) needs |a| < alpha*p, |b| < beta*p with
 // alpha*beta <= 2^11 and limb magnitudes with 14 * 2^(la+lb) < 2^62, i.e. la + lb <= 58; its
-// result is normalised and lies in (0, 3p).
+// result is normalised and lies in (0, 3p).  The figures are those of BLS12-381, the tighter
+// case: BN254 leaves R'/p = 2^26 of head-room instead of 2^11 and sums 10 limb products.
 #pragma once
 #include "curve.hpp"
 
 namespace grape {
 
+#if defined(GRAPE_CURVE_BN254)
+struct Fp28 {
+    int32_t v[10];
+};
+
+namespace fp28 {
+
+constexpr int N = 10;
+constexpr int W = 28;
+constexpr uint32_t MASK = (1u << W) - 1;
+constexpr uint32_t PINV = 0x4866389u;   // -p^-1 mod 2^28
+
+GRAPE_HD int32_t P(int i) {
+    constexpr int32_t t[10] = {0x87cfd47, 0x208c16d, 0x1ca8d3c, 0x6a91687, 0x85d9781,
+                               0xb681815, 0x9b85045, 0xe131a02, 0x0644e72, 0x0000003};
+    return t[i];
+}
+GRAPE_HD int32_t P2(int i) {   // 2p
+    constexpr int32_t t[10] = {0x0f9fa8e, 0x41182db, 0x3951a78, 0xd522d0e, 0x0bb2f02,
+                               0x6d0302b, 0x370a08b, 0xc263405, 0x0c89ce5, 0x0000006};
+    return t[i];
+}
+GRAPE_HD int32_t ONE(int i) {   // 2^280 mod p
+    constexpr int32_t t[10] = {0xa0e0d96, 0x6a56a28, 0x56d8f97, 0x1e6c92b, 0xee608fc,
+                               0x10581c8, 0x89f6e5c, 0x8c59c9e, 0x7359fa8, 0x0000000};
+    return t[i];
+}
+GRAPE_HD int32_t CMEM(int i) {   // 2^256 mod p: mul28(x*2^280, CMEM) = x*2^256
+    constexpr int32_t t[10] = {0x58f0d9d, 0x5d438dc, 0x70b3dd3, 0xeb28f5c, 0x62c0a78,
+                               0x6f78794, 0xf666ea3, 0x9a07df2, 0xe0a77c1, 0x0000000};
+    return t[i];
+}
+// Montgomery (radix 2^256) form of 2^24, 32-bit limbs: mul(x*2^256, MCONV) = x*2^280 mod p
+GRAPE_HD uint32_t MCONV(int i) {
+    constexpr uint32_t t[8] = {0x8a0e0d96u, 0x976a56a2u, 0x92b56d8fu, 0x08fc1e6cu,
+                               0x581c8ee6u, 0x9f6e5c10u, 0x8c59c9e8u, 0x07359fa8u};
+    return t[i];
+}
+
+#else
 struct Fp28 {
     int32_t v[14];
 };
@@ -48,17 +90,19 @@ GRAPE_HD int32_t ONE(int i) {   // 2^392 mod p
                                0xda0f73e, 0x9b09b42, 0x1297bb0, 0x515d98f, 0x012ca7c, 0x659fcfa, 0x000577a};
     return t[i];
 }
-GRAPE_HD int32_t C384(int i) {   // 2^384 mod p: mul28(x*2^392, C384) = x*2^384
+GRAPE_HD int32_t CMEM(int i) {   // 2^384 mod p: mul28(x*2^392, CMEM) = x*2^384
     constexpr int32_t t[14] = {0x002fffd, 0x0900000, 0xc000276, 0x000bc40, 0x8baebf4, 0x5753c75, 0x55f4898,
                                0x7052574, 0x7ce5853, 0x56ec6d7, 0x71a97a2, 0xe4935c0, 0xec3fa80, 0x0015f65};
     return t[i];
 }
-// Montgomery (radix 2^384) form of 2^8, 32-bit limbs: mul(x*2^384, M256) = x*2^392 mod p
-GRAPE_HD uint32_t M256(int i) {
+// Montgomery (radix 2^384) form of 2^8, 32-bit limbs: mul(x*2^384, MCONV) = x*2^392 mod p
+GRAPE_HD uint32_t MCONV(int i) {
     constexpr uint32_t t[12] = {0x0347fcb8u, 0x19d80000u, 0x6d2002b1u, 0x12e00cdeu, 0xa2090c72u, 0x37669f83u,
                                 0xda0f73e0u, 0x09b09b42u, 0x8f1297bbu, 0xa7c515d9u, 0xfcfa012cu, 0x0577a659u};
     return t[i];
 }
+
+#endif
 
 GRAPE_HD Fp28 one() {
     Fp28 r;
@@ -99,7 +143,7 @@ GRAPE_HD Fp28 cneg(const Fp28& a, bool flag) {
     return r;
 }
 
-// signed carry propagation: same value, limbs 0..12 in [0, 2^28)
+// signed carry propagation: same value, limbs 0..N-2 in [0, 2^28)
 GRAPE_HD Fp28 normalize(const Fp28& a) {
     Fp28 r;
     int32_t c = 0;
@@ -113,7 +157,7 @@ GRAPE_HD Fp28 normalize(const Fp28& a) {
     return r;
 }
 
-// Montgomery product a*b/2^392 (mod p), result normalised in (0, 3p).
+// Montgomery product a*b/R' (mod p), result normalised in (0, 3p).
 GRAPE_HD Fp28 mul(const Fp28& a, const Fp28& b) {
     int64_t C[2 * N];
 #pragma unroll
@@ -140,7 +184,6 @@ GRAPE_HD Fp28 mul(const Fp28& a, const Fp28& b) {
     return r;
 }
 
-// a^2/2^392: the off-diagonal limb products are taken once with a doubled operand.
 // a*b - c*d with one Montgomery reduction: both products accumulate in the same columns.
 // Needs 14*(2^(la+lb) + 2^(lc+ld)) + 14*2^56 < 2^63 for the limb bounds and |ab| + |cd| <= 2^11 p^2
 // for the values; the result is normalised in (0, 3p) like a product.
@@ -174,6 +217,7 @@ GRAPE_HD Fp28 mul_sub(const Fp28& a, const Fp28& b, const Fp28& c, const Fp28& d
     return r;
 }
 
+// a^2/R': the off-diagonal limb products are taken once with a doubled operand.
 GRAPE_HD Fp28 sqr(const Fp28& a) {
     int64_t C[2 * N];
 #pragma unroll
@@ -218,23 +262,24 @@ GRAPE_HD bool is_zero_mod_p(const Fp28& a) {
     return (z0 == 0) | (z1 == 0) | (z2 == 0);
 }
 
-// ---- conversions with the canonical 12 x 32-bit, radix-2^384 Montgomery form ----
-// pure re-limbing of a 384-bit non-negative integer
+// ---- conversions with the canonical 32-bit-limb Montgomery form (radix 2^384 resp. 2^256) ----
+constexpr int FW = FpParams::N;   // 32-bit words of the canonical form
+// pure re-limbing of a non-negative integer of FW words
 GRAPE_HD Fp28 pack(const Fp& x) {
     Fp28 r;
 #pragma unroll
     for (int k = 0; k < N; k++) {
         const int bit = W * k, q = bit >> 5, s = bit & 31;
-        uint64_t two = (uint64_t)x.v[q] | ((q + 1 < 12) ? ((uint64_t)x.v[q + 1] << 32) : 0);
+        uint64_t two = (uint64_t)x.v[q] | ((q + 1 < FW) ? ((uint64_t)x.v[q + 1] << 32) : 0);
         r.v[k] = (int32_t)((uint32_t)(two >> s) & MASK);
     }
     return r;
 }
-// inverse of pack for a normalised, non-negative value below 2^384
+// inverse of pack for a normalised, non-negative value below 2^(32 FW)
 GRAPE_HD Fp unpack(const Fp28& a) {
     Fp r;
 #pragma unroll
-    for (int q = 0; q < 12; q++) {
+    for (int q = 0; q < FW; q++) {
         // word q covers bits [32q, 32q+32): limbs k0 = floor(32q/28) .. up to two more
         const int k0 = (32 * q) / W;
         uint64_t acc = 0;
@@ -254,19 +299,19 @@ GRAPE_HD Fp unpack(const Fp28& a) {
     }
     return r;
 }
-// canonical x*2^384 (32-bit limbs) -> x*2^392 (28-bit limbs), canonical and normalised
+// canonical memory form (32-bit limbs) -> working form (28-bit limbs), canonical and normalised
 GRAPE_HD Fp28 from_canonical(const Fp& x) {
     Fp m;
 #pragma unroll
-    for (int i = 0; i < 12; i++) m.v[i] = M256(i);
+    for (int i = 0; i < FW; i++) m.v[i] = MCONV(i);
     return pack(fmul(x, m));
 }
-// value in (-9p, 3p), any limb form -> canonical x*2^384, 32-bit limbs
+// value in (-9p, 3p), any limb form -> canonical memory form, 32-bit limbs
 GRAPE_HD Fp to_canonical(const Fp28& a) {
     Fp28 c;
 #pragma unroll
-    for (int i = 0; i < N; i++) c.v[i] = C384(i);
-    Fp28 t = mul(normalize(a), c);   // in (0, 3p), now with radix 2^384
+    for (int i = 0; i < N; i++) c.v[i] = CMEM(i);
+    Fp28 t = mul(normalize(a), c);   // in (0, 3p), now with the radix of the memory form
     // subtract p while the result stays non-negative (at most twice)
 #pragma unroll
     for (int rep = 0; rep < 2; rep++) {
@@ -290,9 +335,9 @@ GRAPE_HD Fp28 inverse(const Fp28& a) {
     for (int i = 2; i < 16; i++) tbl[i] = mul(tbl[i - 1], tbl[1]);
     Fp28 acc = one();
     bool started = false;
-    for (int limb = 11; limb >= 0; limb--) {
+    for (int limb = FW - 1; limb >= 0; limb--) {
         uint32_t e = 0;
-        for (int k = 0; k < 12; k++) e = (k == limb) ? FpParams::pm2(k) : e;
+        for (int k = 0; k < FW; k++) e = (k == limb) ? FpParams::pm2(k) : e;
         for (int nib = 7; nib >= 0; nib--) {
             if (started) {
                 acc = sqr(acc);
@@ -320,15 +365,27 @@ GRAPE_HD Fp28 inverse(const Fp28& a) {
 // ------------------------------------------------------------------------------------------------
 namespace by {
 
+#if defined(GRAPE_CURVE_BN254)
+constexpr int L = 9;                        // 9 x 30 = 270 bits
+constexpr uint32_t PINV30 = 0x1b799c77u;    // p^-1 mod 2^30
+GRAPE_HD int32_t P30(int i) {
+    constexpr int32_t t[9] = {0x187cfd47, 0x3082305b, 0x071ca8d3, 0x205aa45a, 0x01585d97,
+                              0x0116da06, 0x1a029b85, 0x139cb84c, 0x00003064};
+    return t[i];
+}
+#else
 constexpr int L = 13;                       // 13 x 30 = 390 bits
-constexpr int32_t M30 = (1 << 30) - 1;
 constexpr uint32_t PINV30 = 0x00030003u;    // p^-1 mod 2^30
-
 GRAPE_HD int32_t P30(int i) {
     constexpr int32_t t[13] = {0x3fffaaab, 0x27fbffff, 0x153ffffb, 0x2affffac, 0x30f6241e, 0x034a83da, 0x112bf673,
                                0x12e13ce1, 0x2cd76477, 0x1ed90d2e, 0x29a4b1ba, 0x3a8e5ff9, 0x001a0111};
     return t[i];
 }
+#endif
+constexpr int32_t M30 = (1 << 30) - 1;
+// floor((49 d + 57) / 17) divsteps always suffice for d-bit inputs (Bernstein-Yang, d >= 46):
+// 1110 for 384 bits, 741 for 256 bits; taken 30 at a time
+constexpr int kBatches = ((49 * 32 * FpParams::N + 57) / 17 + 29) / 30;
 
 struct Mat { int32_t u, v, q, r; };
 
@@ -410,12 +467,17 @@ GRAPE_HD void update_de(int32_t* d, int32_t* e, const Mat& t) {
 
 // R'^3 mod p: turns the plain inverse of a Montgomery-form value back into Montgomery form
 GRAPE_HD int32_t R3(int i) {
+#if defined(GRAPE_CURVE_BN254)
+    constexpr int32_t t[10] = {0xfdd47fe, 0xb246b8d, 0x1ffde25, 0xb55ed86, 0x14bbcde,
+                               0xad156f8, 0x483330b, 0x59ae72c, 0x1df6aee, 0x0000000};
+#else
     constexpr int32_t t[14] = {0x1f7b890, 0x294cc4d, 0x9f3af22, 0xb5ba56c, 0xcb5c0cc, 0xc0d975c, 0xc89a8c5,
                                0x6c968b4, 0x22672ea, 0x91de8c9, 0x35652a6, 0x84977c8, 0x424bbb9, 0x00141ab};
+#endif
     return t[i];
 }
 
-// 1/a in Montgomery form (radix 2^392) for a in (-9p, 3p), a != 0 mod p; result normalised in (0, 3p).
+// 1/a in Montgomery form (radix R') for a in (-9p, 3p), a != 0 mod p; result normalised in (0, 3p).
 GRAPE_HD Fp28 inverse_by(const Fp28& a) {
     using namespace by;
     // canonical integer of a (still carrying the Montgomery factor) in [0, p)
@@ -430,7 +492,7 @@ GRAPE_HD Fp28 inverse_by(const Fp28& a) {
 #pragma unroll
         for (int i = 0; i < N; i++) t.v[i] = ok ? dd.v[i] : t.v[i];
     }
-    // re-limb 14 x 28 -> 13 x 30
+    // re-limb N x 28 -> L x 30
     int32_t f[L], g[L], d[L], e[L];
 #pragma unroll
     for (int k = 0; k < L; k++) {
@@ -445,8 +507,7 @@ GRAPE_HD Fp28 inverse_by(const Fp28& a) {
     }
     e[0] = 1;
     int32_t delta = 1;
-    // at most floor((49*384+57)/17) = 1110 divsteps are ever needed for 384-bit inputs
-    for (int batch = 0; batch < 37; batch++) {
+    for (int batch = 0; batch < kBatches; batch++) {
         uint32_t gz = 0;
 #pragma unroll
         for (int k = 0; k < L; k++) gz |= (uint32_t)g[k];
@@ -470,7 +531,7 @@ GRAPE_HD Fp28 inverse_by(const Fp28& a) {
         c = s >> 30;
     }
     x[L - 1] = (int32_t)((int64_t)x[L - 1] + 2 * (int64_t)P30(L - 1) + c);
-    // re-limb 13 x 30 -> 14 x 28 (value in (0, 4p), below 2^384)
+    // re-limb L x 30 -> N x 28 (value in (0, 4p), below 2^(32 FW))
     Fp28 r;
 #pragma unroll
     for (int k = 0; k < N; k++) {

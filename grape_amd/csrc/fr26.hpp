@@ -1,4 +1,4 @@
-// BLS12-381 Fr on 10 signed limbs of 26 bits with lazy accumulation - the working form of the
+// Fr (BLS12-381 or BN254, both r = 1 mod 2^26) on 10 signed limbs of 26 bits with lazy accumulation - the working form of the
 // streaming Fr kernels (fold, sumcheck rounds, logUp rounds, element-wise products).
 //
 // Tensors stay in memory in the reference's format (8 x 32-bit limbs, canonical Montgomery
@@ -30,6 +30,26 @@ struct Acc {            // columns of a double-width sum of limb products
     int64_t c[2 * N];
 };
 
+// The bounds quoted below (r/2^260 = 1/35.3) are those of BLS12-381; BN254's r is smaller
+// (r/2^260 = 1/84.6), so every bound holds there with more room.
+#if defined(GRAPE_CURVE_BN254)
+GRAPE_HD int32_t R(int i) {   // the modulus r; R(0) = 1 and -r^-1 mod 2^26 = -1
+    constexpr int32_t t[10] = {0x0000001, 0x07d64fc, 0x309143e, 0x121e6e5, 0x12833e8,
+                               0x0605617, 0x1045b68, 0x280a6e1, 0x272e131, 0x00c1913};
+    return t[i];
+}
+GRAPE_HD int32_t X16(int i) {   // 16 * 2^260 mod r: reduce(t * X16) = 16 t
+    constexpr int32_t t[10] = {0x3fffab6, 0x0c7e327, 0x1faef6e, 0x2b0c4ca, 0x15d7570,
+                               0x278a8d2, 0x2f48b70, 0x38d5c9d, 0x064ef86, 0x0035e45};
+    return t[i];
+}
+GRAPE_HD int32_t C516(int i) {   // 2^516 mod r: reduce(x * C516) = x * 2^256 (into memory form)
+    constexpr int32_t t[10] = {0x216da70, 0x39916b8, 0x1e31bb8, 0x078d716, 0x13fe3ab,
+                               0x2ee0215, 0x1833d53, 0x1296312, 0x317f4e4, 0x0085b42};
+    return t[i];
+}
+
+#else
 GRAPE_HD int32_t R(int i) {   // the modulus r; R(0) = 1 and -r^-1 mod 2^26 = -1
     constexpr int32_t t[10] = {0x0000001, 0x3ffffc0, 0x1bfefff, 0x00bfff9, 0x153bda4,
                                0x2687601, 0x39d8080, 0x1f520cc, 0x353299d, 0x01cfb69};
@@ -45,6 +65,8 @@ GRAPE_HD int32_t C516(int i) {   // 2^516 mod r: reduce(x * C516) = x * 2^256 (i
                                0x2e8703b, 0x37715f1, 0x1cf20a7, 0x246cc02, 0x00027fd};
     return t[i];
 }
+
+#endif
 
 // 8 x 32-bit canonical -> 10 x 26-bit, non-negative
 GRAPE_HD Limbs pack(const Fr& x) {

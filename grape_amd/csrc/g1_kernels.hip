@@ -19,44 +19,50 @@ namespace grape {
 __device__ __noinline__ Fp fp_mul_outline(Fp a, Fp b) { return mul(a, b); }
 __device__ __noinline__ Fp fp_sqr_outline(Fp a) { return sqr(a); }
 
+// Memory images in 32-bit words: an Fp element is FW words (12 for BLS12-381, 8 for BN254), an
+// affine point 2 FW, a Jacobian point 3 FW, an XYZZ point 4 FW; L28 is the limb count of the
+// 28-bit working form.
+constexpr int FW = FpParams::N;
+constexpr int L28 = fp28::N;
+
 __device__ __forceinline__ Fp ld_fp(const uint32_t* p) {
     const uint4* q = reinterpret_cast<const uint4*>(p);
-    uint4 a = q[0], b = q[1], c = q[2];
     Fp r;
-    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
-    r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
-    r.v[8] = c.x; r.v[9] = c.y; r.v[10] = c.z; r.v[11] = c.w;
+#pragma unroll
+    for (int i = 0; i < FW / 4; i++) {
+        const uint4 a = q[i];
+        r.v[4 * i] = a.x; r.v[4 * i + 1] = a.y; r.v[4 * i + 2] = a.z; r.v[4 * i + 3] = a.w;
+    }
     return r;
 }
 __device__ __forceinline__ void st_fp(uint32_t* p, const Fp& a) {
     uint4* q = reinterpret_cast<uint4*>(p);
-    q[0] = make_uint4(a.v[0], a.v[1], a.v[2], a.v[3]);
-    q[1] = make_uint4(a.v[4], a.v[5], a.v[6], a.v[7]);
-    q[2] = make_uint4(a.v[8], a.v[9], a.v[10], a.v[11]);
+#pragma unroll
+    for (int i = 0; i < FW / 4; i++) q[i] = make_uint4(a.v[4 * i], a.v[4 * i + 1], a.v[4 * i + 2], a.v[4 * i + 3]);
 }
 __device__ __forceinline__ G1Affine ld_affine(const uint32_t* base, size_t i) {
     G1Affine r;
-    r.x = ld_fp(base + 24 * i);
-    r.y = ld_fp(base + 24 * i + 12);
+    r.x = ld_fp(base + 2 * FW * i);
+    r.y = ld_fp(base + 2 * FW * i + FW);
     return r;
 }
 __device__ __forceinline__ void st_affine(uint32_t* base, size_t i, const G1Affine& p) {
-    st_fp(base + 24 * i, p.x);
-    st_fp(base + 24 * i + 12, p.y);
+    st_fp(base + 2 * FW * i, p.x);
+    st_fp(base + 2 * FW * i + FW, p.y);
 }
 __device__ __forceinline__ G1Xyzz ld_xyzz(const uint32_t* base, size_t i) {
     G1Xyzz r;
-    r.x = ld_fp(base + 48 * i);
-    r.y = ld_fp(base + 48 * i + 12);
-    r.zz = ld_fp(base + 48 * i + 24);
-    r.zzz = ld_fp(base + 48 * i + 36);
+    r.x = ld_fp(base + 4 * FW * i);
+    r.y = ld_fp(base + 4 * FW * i + FW);
+    r.zz = ld_fp(base + 4 * FW * i + 2 * FW);
+    r.zzz = ld_fp(base + 4 * FW * i + 3 * FW);
     return r;
 }
 __device__ __forceinline__ void st_xyzz(uint32_t* base, size_t i, const G1Xyzz& p) {
-    st_fp(base + 48 * i, p.x);
-    st_fp(base + 48 * i + 12, p.y);
-    st_fp(base + 48 * i + 24, p.zz);
-    st_fp(base + 48 * i + 36, p.zzz);
+    st_fp(base + 4 * FW * i, p.x);
+    st_fp(base + 4 * FW * i + FW, p.y);
+    st_fp(base + 4 * FW * i + 2 * FW, p.zz);
+    st_fp(base + 4 * FW * i + 3 * FW, p.zzz);
 }
 __device__ __forceinline__ Fr ld_fr8(const uint32_t* base, size_t i) {
     const uint4* p = reinterpret_cast<const uint4*>(base) + 2 * i;
@@ -67,20 +73,20 @@ __device__ __forceinline__ Fr ld_fr8(const uint32_t* base, size_t i) {
     return r;
 }
 
-// Wide-table entry: an affine point in the 28-bit working form, x[14] then y[14] as 32-bit
-// words plus 16 bytes of padding = 128 bytes, so that every gather is exactly one cache line.
+// Wide-table entry: an affine point in the 28-bit working form, x[L28] then y[L28] as 32-bit
+// words, padded to 128 bytes, so that every gather is exactly one cache line.
 constexpr int kWideEntryWords = 32;
 __device__ __forceinline__ Affine28 ld_entry28(const uint32_t* table, size_t e) {
     const uint4* q = reinterpret_cast<const uint4*>(table + (size_t)kWideEntryWords * e);
-    uint4 w[7];
+    uint4 w[L28 / 2];
 #pragma unroll
-    for (int i = 0; i < 7; i++) w[i] = q[i];
+    for (int i = 0; i < L28 / 2; i++) w[i] = q[i];
     const uint32_t* f = reinterpret_cast<const uint32_t*>(w);
     Affine28 r;
 #pragma unroll
-    for (int i = 0; i < 14; i++) {
+    for (int i = 0; i < L28; i++) {
         r.x.v[i] = (int32_t)f[i];
-        r.y.v[i] = (int32_t)f[14 + i];
+        r.y.v[i] = (int32_t)f[L28 + i];
     }
     return r;
 }
@@ -88,11 +94,12 @@ __device__ __forceinline__ void st_entry28(uint32_t* table, size_t e, const G1Af
     Fp28 x = fp28::from_canonical(a.x), y = fp28::from_canonical(a.y);
     uint32_t f[32];
 #pragma unroll
-    for (int i = 0; i < 14; i++) {
+    for (int i = 0; i < L28; i++) {
         f[i] = (uint32_t)x.v[i];
-        f[14 + i] = (uint32_t)y.v[i];
+        f[L28 + i] = (uint32_t)y.v[i];
     }
-    f[28] = f[29] = f[30] = f[31] = 0;
+#pragma unroll
+    for (int i = 2 * L28; i < 32; i++) f[i] = 0;
     uint4* q = reinterpret_cast<uint4*>(table + (size_t)kWideEntryWords * e);
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
@@ -100,49 +107,49 @@ __device__ __forceinline__ void st_entry28(uint32_t* table, size_t e, const G1Af
 __device__ __forceinline__ bool entry_is_inf(const Affine28& a) {
     uint32_t z = 0;
 #pragma unroll
-    for (int i = 0; i < 14; i++) z |= (uint32_t)a.x.v[i] | (uint32_t)a.y.v[i];
+    for (int i = 0; i < L28; i++) z |= (uint32_t)a.x.v[i] | (uint32_t)a.y.v[i];
     return z == 0;
 }
-// Per-lane partial accumulator in memory: x, y, zz, zzz (14 words each), the identity flag and
+// Per-lane partial accumulator in memory: x, y, zz, zzz (L28 words each), the identity flag and
 // padding = 64 words (256 bytes).
 constexpr int kPartialWords = 64;
 __device__ __forceinline__ void st_partial28(uint32_t* base, size_t i, const Xyzz28& a) {
     uint32_t f[64];
 #pragma unroll
-    for (int k = 0; k < 14; k++) {
+    for (int k = 0; k < L28; k++) {
         f[k] = (uint32_t)a.x.v[k];
-        f[14 + k] = (uint32_t)a.y.v[k];
-        f[28 + k] = (uint32_t)a.zz.v[k];
-        f[42 + k] = (uint32_t)a.zzz.v[k];
+        f[L28 + k] = (uint32_t)a.y.v[k];
+        f[2 * L28 + k] = (uint32_t)a.zz.v[k];
+        f[3 * L28 + k] = (uint32_t)a.zzz.v[k];
     }
-    f[56] = a.inf ? 1u : 0u;
+    f[4 * L28] = a.inf ? 1u : 0u;
 #pragma unroll
-    for (int k = 57; k < 64; k++) f[k] = 0;
+    for (int k = 4 * L28 + 1; k < 64; k++) f[k] = 0;
     uint4* q = reinterpret_cast<uint4*>(base + (size_t)kPartialWords * i);
 #pragma unroll
     for (int k = 0; k < 16; k++) q[k] = make_uint4(f[4 * k], f[4 * k + 1], f[4 * k + 2], f[4 * k + 3]);
 }
 __device__ __forceinline__ Xyzz28 ld_partial28(const uint32_t* base, size_t i) {
     const uint4* q = reinterpret_cast<const uint4*>(base + (size_t)kPartialWords * i);
-    uint4 w[15];
+    uint4 w[L28 + 1];
 #pragma unroll
-    for (int k = 0; k < 15; k++) w[k] = q[k];
+    for (int k = 0; k < L28 + 1; k++) w[k] = q[k];
     const uint32_t* f = reinterpret_cast<const uint32_t*>(w);
     Xyzz28 a;
 #pragma unroll
-    for (int k = 0; k < 14; k++) {
+    for (int k = 0; k < L28; k++) {
         a.x.v[k] = (int32_t)f[k];
-        a.y.v[k] = (int32_t)f[14 + k];
-        a.zz.v[k] = (int32_t)f[28 + k];
-        a.zzz.v[k] = (int32_t)f[42 + k];
+        a.y.v[k] = (int32_t)f[L28 + k];
+        a.zz.v[k] = (int32_t)f[2 * L28 + k];
+        a.zzz.v[k] = (int32_t)f[3 * L28 + k];
     }
-    a.inf = f[56] != 0;
+    a.inf = f[4 * L28] != 0;
     return a;
 }
 __device__ __forceinline__ Xyzz28 shfl_down_xyzz28(const Xyzz28& a, int off) {
     Xyzz28 r;
 #pragma unroll
-    for (int k = 0; k < 14; k++) {
+    for (int k = 0; k < L28; k++) {
         r.x.v[k] = __shfl_down(a.x.v[k], off, 64);
         r.y.v[k] = __shfl_down(a.y.v[k], off, 64);
         r.zz.v[k] = __shfl_down(a.zz.v[k], off, 64);
@@ -231,7 +238,7 @@ __device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k, const u
 __device__ __forceinline__ G1Xyzz shfl_down_xyzz(const G1Xyzz& a, int off) {
     G1Xyzz r;
 #pragma unroll
-    for (int i = 0; i < 12; i++) {
+    for (int i = 0; i < FW; i++) {
         r.x.v[i] = __shfl_down(a.x.v[i], off, 64);
         r.y.v[i] = __shfl_down(a.y.v[i], off, 64);
         r.zz.v[i] = __shfl_down(a.zz.v[i], off, 64);
@@ -335,7 +342,7 @@ __global__ void __launch_bounds__(64) wide_normalize_kernel(uint32_t* table, con
         size_t e = t0 + (size_t)k * nthreads;
         pre[k] = acc;
         if (e < n_entries) {
-            Fp zzz = ld_fp(tmp + 48 * e + 36);
+            Fp zzz = ld_fp(tmp + 4 * FW * e + 3 * FW);
             if (!zzz.is_zero()) acc = fmul(acc, zzz);
         }
     }
@@ -467,7 +474,7 @@ __global__ void __launch_bounds__(64) scaled_normalize_kernel(uint32_t* out, con
         size_t e = t0 + (size_t)k * nthreads;
         pre[k] = acc;
         if (e < n_entries) {
-            Fp zzz = ld_fp(tmp + 48 * e + 36);
+            Fp zzz = ld_fp(tmp + 4 * FW * e + 3 * FW);
             if (!zzz.is_zero()) acc = fmul(acc, zzz);
         }
     }
@@ -563,17 +570,17 @@ __global__ void __launch_bounds__(64) affine_to_jac_kernel(uint32_t* out, const 
     if (i >= n) return;
     G1Affine a = ld_affine(in, i);
     bool inf = a.is_inf();
-    st_fp(out + 36 * i, a.x);
-    st_fp(out + 36 * i + 12, a.y);
-    st_fp(out + 36 * i + 24, inf ? Fp::zero() : Fp::one());
+    st_fp(out + 3 * FW * i, a.x);
+    st_fp(out + 3 * FW * i + FW, a.y);
+    st_fp(out + 3 * FW * i + 2 * FW, inf ? Fp::zero() : Fp::one());
 }
 __global__ void __launch_bounds__(64) jac_to_affine_kernel(uint32_t* out, const uint32_t* in, size_t n) {
     size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
     if (i >= n) return;
     G1Jac p;
-    p.x = ld_fp(in + 36 * i);
-    p.y = ld_fp(in + 36 * i + 12);
-    p.z = ld_fp(in + 36 * i + 24);
+    p.x = ld_fp(in + 3 * FW * i);
+    p.y = ld_fp(in + 3 * FW * i + FW);
+    p.z = ld_fp(in + 3 * FW * i + 2 * FW);
     st_affine(out, i, jac_to_affine(p));
 }
 
@@ -582,11 +589,6 @@ __global__ void __launch_bounds__(64) jac_to_affine_kernel(uint32_t* out, const 
 using namespace grape;
 
 #define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")
-
-static const uint32_t kGenX[12] = {0xfd530c16u, 0x5cb38790u, 0x9976fff5u, 0x7817fc67u, 0x143ba1c1u, 0x154f95c7u,
-                                   0xf3d0e747u, 0xf0ae6acdu, 0x21dbf440u, 0xedce6eccu, 0x9e0bfb75u, 0x12017741u};
-static const uint32_t kGenY[12] = {0x0ce72271u, 0xbaac93d5u, 0x7918fd8eu, 0x8c22631au, 0x570725ceu, 0xdd595f13u,
-                                   0x50405194u, 0x51ac5829u, 0xad0059c0u, 0x0e1c8c3fu, 0x5008a26au, 0x0bbc3efcu};
 
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
@@ -634,9 +636,9 @@ extern "C" {
 
 int grape_g1_generator(uint32_t* out) {
     GRAPE_REQUIRE(out != nullptr, "null output");
-    for (int i = 0; i < 12; i++) {
-        out[i] = kGenX[i];
-        out[12 + i] = kGenY[i];
+    for (int i = 0; i < FW; i++) {
+        out[i] = g1_gen_x(i);
+        out[FW + i] = g1_gen_y(i);
     }
     return GRAPE_OK;
 }
@@ -670,12 +672,12 @@ int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uin
     if (K < CH) CH = K;
     const uint32_t nchunks = (K + CH - 1) / CH;
     // slab the chunk index so that the XYZZ staging buffer stays below ~1.5 GiB
-    size_t slab_chunks = ((size_t)3 << 29) / (per_chunk * CH * 192);
+    size_t slab_chunks = ((size_t)3 << 29) / (per_chunk * CH * (16 * FW));
     if (slab_chunks < 1) slab_chunks = 1;
     if (slab_chunks > nchunks) slab_chunks = nchunks;
     void* ws;
-    const size_t bases_bytes = per_chunk * 96;
-    const size_t tmp_bytes = slab_chunks * CH * per_chunk * 192;
+    const size_t bases_bytes = per_chunk * (8 * FW);
+    const size_t tmp_bytes = slab_chunks * CH * per_chunk * (16 * FW);
     int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes, &ws);
     if (rc) return rc;
     uint32_t* bases = (uint32_t*)ws;
@@ -702,13 +704,13 @@ int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len
     GRAPE_REQUIRE(c >= 2 && c <= 16 && (uint64_t)nw * c >= 256 && K >= (1u << (c - 1)), "need a full-width wide table");
     hipStream_t s = as_stream(st);
     // slabs of scalars so that the XYZZ staging buffer stays near 1.5 GiB
-    size_t slab = ((size_t)3 << 29) / (ncols * 192);
+    size_t slab = ((size_t)3 << 29) / (ncols * (16 * FW));
     if (slab < 1) slab = 1;
     if (slab > len) slab = len;
     void* ws;
-    int rc = scratch_get(kSlotMsm, slab * ncols * 192 + 64, &ws);
+    int rc = scratch_get(kSlotMsm, slab * ncols * (16 * FW) + 64, &ws);
     if (rc) return rc;
-    int* err = (int*)((char*)ws + slab * ncols * 192);
+    int* err = (int*)((char*)ws + slab * ncols * (16 * FW));
     GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
     for (size_t t0 = 0; t0 < len; t0 += slab) {
         size_t nt = len - t0 < slab ? len - t0 : slab;

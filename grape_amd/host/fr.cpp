@@ -78,11 +78,6 @@ std::ostream& operator<<(std::ostream& os, const Fr& x) {
 }
 
 // ------------------------------------------------------------------ G1
-static const uint32_t kGenX[12] = {0xfd530c16u, 0x5cb38790u, 0x9976fff5u, 0x7817fc67u, 0x143ba1c1u, 0x154f95c7u,
-                                   0xf3d0e747u, 0xf0ae6acdu, 0x21dbf440u, 0xedce6eccu, 0x9e0bfb75u, 0x12017741u};
-static const uint32_t kGenY[12] = {0x0ce72271u, 0xbaac93d5u, 0x7918fd8eu, 0x8c22631au, 0x570725ceu, 0xdd595f13u,
-                                   0x50405194u, 0x51ac5829u, 0xad0059c0u, 0x0e1c8c3fu, 0x5008a26au, 0x0bbc3efcu};
-
 G1::G1(const affine_t& a) {
     if (a.is_inf()) {
         p = grape::G1Jac::inf();
@@ -95,9 +90,9 @@ G1::G1(const affine_t& a) {
 
 G1 G1::one() {
     affine_t a;
-    for (int i = 0; i < 12; i++) {
-        a.x.v[i] = kGenX[i];
-        a.y.v[i] = kGenY[i];
+    for (int i = 0; i < grape::FpParams::N; i++) {
+        a.x.v[i] = grape::g1_gen_x(i);
+        a.y.v[i] = grape::g1_gen_y(i);
     }
     return G1(a);
 }

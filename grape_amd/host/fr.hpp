@@ -75,7 +75,7 @@ public:
     bool operator==(const G1& o) const;
     bool operator!=(const G1& o) const { return !(*this == o); }
 };
-static_assert(sizeof(G1) == 144, "G1 must have the jacob_t memory image");
+static_assert(sizeof(G1) == 3 * 4 * grape::FpParams::N, "G1 must have the jacob_t memory image (144 bytes for BLS12-381, 96 for BN254)");
 G1 operator*(const Fr& k, const G1& pt);
 
 typedef G1 bn128;   // the reference's name for its host group type

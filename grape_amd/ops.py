@@ -1,8 +1,9 @@
 """Thin Python helpers over the C ABI for tests and benchmarks.
 
 Device memory comes from torch (plumbing only): an Fr tensor of n elements is a CUDA int32
-tensor of shape (n, 8) whose bytes are the fr_t array; affine G1 points are (n, 24), XYZZ
-(n, 48).  Host-side values travel as numpy uint64 arrays of shape (n, 4) / (n, 12).
+tensor of shape (n, 8) whose bytes are the fr_t array; affine G1 points are (n, 24) for
+BLS12-381 and (n, 16) for BN254.  Host-side values travel as numpy uint64 arrays of shape
+(n, 4) / (n, 12 or 8).
 Every helper enqueues on torch's current stream.
 """
 import ctypes
@@ -57,7 +58,7 @@ def fr_to_host(t):
 
 
 def g1_to_host(t):
-    return t.detach().cpu().contiguous().numpy().view(np.uint64).reshape(-1, 12)
+    return t.detach().cpu().contiguous().numpy().view(np.uint64).reshape(-1, _capi.FP_WORDS)
 
 
 def fr_empty(n):
@@ -65,7 +66,7 @@ def fr_empty(n):
 
 
 def g1_empty(n):
-    return torch.empty((int(n), 24), dtype=torch.int32, device="cuda")
+    return torch.empty((int(n), 2 * _capi.FP_WORDS), dtype=torch.int32, device="cuda")
 
 
 # ------------------------------------------------------------------ Fr tensors
@@ -280,7 +281,7 @@ def fr_fold_msb_multi(tensors, n_out, v):
 # ------------------------------------------------------------------ G1
 def g1_generator():
     lib = init()
-    out = np.zeros(12, dtype=np.uint64)
+    out = np.zeros(_capi.FP_WORDS, dtype=np.uint64)
     _capi.check(lib.grape_g1_generator(out.ctypes.data_as(ctypes.c_void_p)))
     return out
 
@@ -289,7 +290,7 @@ def g1_make_generators(k_plain):
     """k_plain: numpy uint64 (n,4) canonical scalars -> device affine points (n,24)."""
     lib = init()
     k = to_dev(np.ascontiguousarray(k_plain, dtype=np.uint64).reshape(-1, 4))
-    base = to_dev(g1_generator().reshape(1, 12))
+    base = to_dev(g1_generator().reshape(1, _capi.FP_WORDS))
     out = g1_empty(k.shape[0])
     _capi.check(lib.grape_g1_scalar_mul_base(_p(out), _p(k), _p(base), k.shape[0], _s()))
     return out
@@ -315,13 +316,16 @@ def g1_wide_table_gen(gens, c, nw, K):
 def wide_table_entries_to_host(table, idx):
     """decode entries of a wide table into affine points (x, y) as Python integers
     (None for the identity); for tests."""
-    P = 0x1a0111ea397fe69a4b1ba7b6434bacd764774b84f38512bf6730d2a0f6b0f6241eabfffeb153ffffb9feffffffffaaab
-    rinv = pow(1 << 392, -1, P)
+    if _capi.CURVE == "bn254":
+        P, L = 21888242871839275222246405745257275088696311157297823662689037894645226208583, 10
+    else:
+        P, L = 0x1a0111ea397fe69a4b1ba7b6434bacd764774b84f38512bf6730d2a0f6b0f6241eabfffeb153ffffb9feffffffffaaab, 14
+    rinv = pow(1 << (28 * L), -1, P)
     rows = table[idx].cpu().numpy()
     out = []
     for r in rows:
-        x = sum(int(r[i]) << (28 * i) for i in range(14))
-        y = sum(int(r[14 + i]) << (28 * i) for i in range(14))
+        x = sum(int(r[i]) << (28 * i) for i in range(L))
+        y = sum(int(r[L + i]) << (28 * i) for i in range(L))
         out.append(None if (x == 0 and y == 0) else (x * rinv % P, y * rinv % P))
     return out
 
@@ -360,7 +364,7 @@ def commit_fr_ref_table(scalars, rowlen, table, npoints):
 
 def g1_affine_to_jacobian(a):
     lib = init()
-    out = torch.empty((a.shape[0], 36), dtype=torch.int32, device="cuda")
+    out = torch.empty((a.shape[0], 3 * _capi.FP_WORDS), dtype=torch.int32, device="cuda")
     _capi.check(lib.grape_g1_affine_to_jacobian(_p(out), _p(a), a.shape[0], _s()))
     return out
 

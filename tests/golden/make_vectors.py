@@ -1,5 +1,6 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/vectors.json: small known-answer vectors for the proving hot path.
+"""Writes tests/golden/vectors.json (BLS12-381) or, under GRAPE_CURVE=bn254,
+tests/golden/vectors_bn254.json: small known-answer vectors for the proving hot path.
 
 The reference ships no vectors for this path, so these are computed here from the definitions
 with Python integers only (tests/bigref.py: `%` arithmetic, textbook affine chord-and-tangent
@@ -106,7 +107,7 @@ def main():
                       "T": [hx((low + t) % R) for t in range(length)],
                       "B": [hx(pow((low + t + beta) % R, -1, R)) for t in range(length)]}
 
-    with open(os.path.join(HERE, "vectors.json"), "w") as f:
+    with open(os.path.join(HERE, "vectors_bn254.json" if br.CURVE == "bn254" else "vectors.json"), "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)
         f.write("\n")
 

@@ -3,54 +3,56 @@
 #include <cstring>
 #include "../../grape_amd/csrc/fp28.hpp"
 using namespace grape;
+static constexpr int FW = FpParams::N;     // 32-bit words of an Fp element in memory
+static constexpr size_t FB = 4 * FW;       // bytes
 
 extern "C" {
-// canonical (12 x u32, radix 2^384) in, canonical out, through the 28-bit domain
+// canonical memory form (FW x u32) in, canonical out, through the 28-bit domain
 void t28_mul(const uint32_t* a, const uint32_t* b, uint32_t* out) {
     Fp x, y;
-    memcpy(&x, a, 48);
-    memcpy(&y, b, 48);
+    memcpy(&x, a, FB);
+    memcpy(&y, b, FB);
     Fp r = fp28::to_canonical(fp28::mul(fp28::from_canonical(x), fp28::from_canonical(y)));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 void t28_sqr(const uint32_t* a, uint32_t* out) {
     Fp x;
-    memcpy(&x, a, 48);
+    memcpy(&x, a, FB);
     Fp r = fp28::to_canonical(fp28::sqr(fp28::from_canonical(x)));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 void t28_roundtrip(const uint32_t* a, uint32_t* out) {
     Fp x;
-    memcpy(&x, a, 48);
+    memcpy(&x, a, FB);
     Fp r = fp28::to_canonical(fp28::from_canonical(x));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 // (a - b - 2c) * d with lazy subtraction, the pattern of the mixed addition
 void t28_lazy(const uint32_t* a, const uint32_t* b, const uint32_t* c, const uint32_t* d, uint32_t* out) {
     Fp xa, xb, xc, xd;
-    memcpy(&xa, a, 48); memcpy(&xb, b, 48); memcpy(&xc, c, 48); memcpy(&xd, d, 48);
+    memcpy(&xa, a, FB); memcpy(&xb, b, FB); memcpy(&xc, c, FB); memcpy(&xd, d, FB);
     Fp28 A = fp28::from_canonical(xa), B = fp28::from_canonical(xb), C = fp28::from_canonical(xc), D = fp28::from_canonical(xd);
     Fp28 t;
-    for (int i = 0; i < 14; i++) t.v[i] = A.v[i] - B.v[i] - 2 * C.v[i];
+    for (int i = 0; i < fp28::N; i++) t.v[i] = A.v[i] - B.v[i] - 2 * C.v[i];
     Fp r = fp28::to_canonical(fp28::mul(fp28::normalize(t), D));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 int t28_is_zero(const uint32_t* a, int times_p) {
     // a canonical; checks is_zero_mod_p on (a + times_p * p) normalised
     Fp x;
-    memcpy(&x, a, 48);
+    memcpy(&x, a, FB);
     Fp28 v = fp28::pack(x);
-    for (int i = 0; i < 14; i++) v.v[i] += times_p * fp28::P(i);
+    for (int i = 0; i < fp28::N; i++) v.v[i] += times_p * fp28::P(i);
     return fp28::is_zero_mod_p(fp28::normalize(v)) ? 1 : 0;
 }
-// sum_i (+-) points[i] through the 28-bit mixed addition; affine points canonical 24 x u32;
+// sum_i (+-) points[i] through the 28-bit mixed addition; affine points canonical 2 FW x u32;
 // returns the number of exceptional steps that had to take the exact path
 int t28_sum(const uint32_t* points, const int* negate, int n, uint32_t* out_xyzz) {
     Xyzz28 acc = xyzz28_inf();
     int slow = 0;
     for (int i = 0; i < n; i++) {
         G1Affine p;
-        memcpy(&p, points + 24 * i, 96);
+        memcpy(&p, points + 2 * FW * i, 2 * FB);
         if (p.is_inf()) continue;
         Affine28 q;
         q.x = fp28::from_canonical(p.x);
@@ -63,7 +65,7 @@ int t28_sum(const uint32_t* points, const int* negate, int n, uint32_t* out_xyzz
         }
     }
     G1Xyzz r = xyzz28_to_canonical(acc);
-    memcpy(out_xyzz, &r, 192);
+    memcpy(out_xyzz, &r, 4 * FB);
     return slow;
 }
 // tree-style sum: partial sums of two halves combined with the accumulator+accumulator addition,
@@ -73,7 +75,7 @@ int t28_sum_tree(const uint32_t* points, const int* negate, int n, uint32_t* out
     int slow = 0;
     for (int i = 0; i < n; i++) {
         G1Affine p;
-        memcpy(&p, points + 24 * i, 96);
+        memcpy(&p, points + 2 * FW * i, 2 * FB);
         if (p.is_inf()) continue;
         Affine28 q;
         q.x = fp28::from_canonical(p.x);
@@ -93,25 +95,25 @@ int t28_sum_tree(const uint32_t* points, const int* negate, int n, uint32_t* out
         slow++;
     }
     G1Affine r = xyzz28_to_affine(part[0]);
-    memcpy(out_affine, &r, 96);
+    memcpy(out_affine, &r, 2 * FB);
     return slow;
 }
 void t28_inverse(const uint32_t* a, uint32_t* out) {
     Fp x;
-    memcpy(&x, a, 48);
+    memcpy(&x, a, FB);
     Fp r = fp28::to_canonical(fp28::inverse(fp28::from_canonical(x)));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 void t28_inverse_by(const uint32_t* a, uint32_t* out) {
     Fp x;
-    memcpy(&x, a, 48);
+    memcpy(&x, a, FB);
     Fp r = fp28::to_canonical(fp28::inverse_by(fp28::from_canonical(x)));
-    memcpy(out, &r, 48);
+    memcpy(out, &r, FB);
 }
 void t28_xyzz_to_affine(const uint32_t* xyzz, uint32_t* out) {
     G1Xyzz a;
-    memcpy(&a, xyzz, 192);
+    memcpy(&a, xyzz, 4 * FB);
     G1Affine r = xyzz_to_affine(a);
-    memcpy(out, &r, 96);
+    memcpy(out, &r, 2 * FB);
 }
 }

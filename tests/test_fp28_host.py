@@ -12,21 +12,25 @@ import bigref as br
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "native", "fp28_host.cpp")
-LIB = os.path.join(HERE, "native", "libfp28_host.so")
+BN = br.CURVE == "bn254"
+LIB = os.path.join(HERE, "native", "libfp28_host_bn254.so" if BN else "libfp28_host.so")
 P = br.P_MOD
+FW = 2 * br.FP_LIMBS          # 32-bit words of an Fp element in memory
+PB = P.bit_length()
 
 
 @pytest.fixture(scope="module")
 def lib():
     deps = [SRC] + [os.path.join(HERE, "..", "grape_amd", "csrc", f) for f in ("fp28.hpp", "curve.hpp", "field.hpp")]
     if not os.path.exists(LIB) or any(os.path.getmtime(d) > os.path.getmtime(LIB) for d in deps):
-        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas", "-o", LIB, SRC])
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas"]
+                              + (["-DGRAPE_CURVE_BN254"] if BN else []) + ["-o", LIB, SRC])
     return ctypes.CDLL(LIB)
 
 
 def _p32(vals):
-    """canonical values -> (n, 12) uint32 Montgomery (radix 2^384) limbs"""
-    return np.ascontiguousarray(br.fp_pack(vals).view(np.uint32).reshape(len(vals), 12))
+    """canonical values -> (n, FW) uint32 Montgomery (memory form) limbs"""
+    return np.ascontiguousarray(br.fp_pack(vals).view(np.uint32).reshape(len(vals), FW))
 
 
 def _u32(a):
@@ -34,16 +38,16 @@ def _u32(a):
 
 
 def _val(a):
-    return br.fp_unpack(np.ascontiguousarray(a).view(np.uint64).reshape(1, 6))[0]
+    return br.fp_unpack(np.ascontiguousarray(a).view(np.uint64).reshape(1, br.FP_LIMBS))[0]
 
 
-EDGE = [0, 1, 2, P - 1, P - 2, (1 << 380), (1 << 381) % P, (1 << 28) - 1, 1 << 28, (1 << 364) - 1, P >> 1]
+EDGE = [0, 1, 2, P - 1, P - 2, 1 << (PB - 1), (1 << PB) % P, (1 << 28) - 1, 1 << 28, (1 << (PB - 17)) - 1, P >> 1]
 
 
 def test_mul_sqr_roundtrip(lib):
     rng = random.Random(1)
     vals = EDGE + [rng.randrange(P) for _ in range(60)]
-    out = np.zeros(12, dtype=np.uint32)
+    out = np.zeros(FW, dtype=np.uint32)
     for a in vals:
         pa = _p32([a])[0]
         lib.t28_roundtrip(_u32(pa), _u32(out))
@@ -58,7 +62,7 @@ def test_mul_sqr_roundtrip(lib):
 
 def test_lazy_expression(lib):
     rng = random.Random(2)
-    out = np.zeros(12, dtype=np.uint32)
+    out = np.zeros(FW, dtype=np.uint32)
     for _ in range(200):
         a, b, c, d = (rng.choice(EDGE) if rng.random() < 0.3 else rng.randrange(P) for _ in range(4))
         pa, pb, pc, pd = (_p32([x])[0] for x in (a, b, c, d))
@@ -67,7 +71,7 @@ def test_lazy_expression(lib):
 
 
 def test_zero_detection(lib):
-    plain = lambda v: np.ascontiguousarray(br.ints_to_limbs([v], 6).view(np.uint32).reshape(12))
+    plain = lambda v: np.ascontiguousarray(br.ints_to_limbs([v], br.FP_LIMBS).view(np.uint32).reshape(FW))
     for k in (0, 1, 2):
         assert lib.t28_is_zero(_u32(plain(0)), k) == 1
         assert lib.t28_is_zero(_u32(plain(1)), k) == 0
@@ -79,13 +83,13 @@ def _points(ks):
 
 
 def _sum28(lib, pts, negs):
-    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 24))
+    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 2 * FW))
     neg = np.array(negs, dtype=np.int32)
-    xyzz = np.zeros(48, dtype=np.uint32)
+    xyzz = np.zeros(4 * FW, dtype=np.uint32)
     slow = lib.t28_sum(_u32(arr), neg.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), len(pts), _u32(xyzz))
-    aff = np.zeros(24, dtype=np.uint32)
+    aff = np.zeros(2 * FW, dtype=np.uint32)
     lib.t28_xyzz_to_affine(_u32(xyzz), _u32(aff))
-    return br.g1_unpack(aff.view(np.uint64).reshape(1, 12))[0], slow
+    return br.g1_unpack(aff.view(np.uint64).reshape(1, br.G1_WORDS))[0], slow
 
 
 def test_point_sums_vs_textbook(lib):
@@ -120,16 +124,16 @@ def test_exceptional_cases_take_the_exact_path(lib):
 
 def test_inverse(lib):
     rng = random.Random(4)
-    out = np.zeros(12, dtype=np.uint32)
-    for a in [1, 2, P - 1, (1 << 380)] + [rng.randrange(1, P) for _ in range(10)]:
+    out = np.zeros(FW, dtype=np.uint32)
+    for a in [1, 2, P - 1, 1 << (PB - 1)] + [rng.randrange(1, P) for _ in range(10)]:
         lib.t28_inverse(_u32(_p32([a])[0]), _u32(out))
         assert _val(out) == pow(a, -1, P)
 
 
 def test_inverse_by_divsteps(lib):
     rng = random.Random(6)
-    out = np.zeros(12, dtype=np.uint32)
-    vals = [1, 2, 3, P - 1, P - 2, (1 << 380), (1 << 381) % P, (P + 1) // 2, 0xffffffff, 1 << 64]
+    out = np.zeros(FW, dtype=np.uint32)
+    vals = [1, 2, 3, P - 1, P - 2, 1 << (PB - 1), (1 << PB) % P, (P + 1) // 2, 0xffffffff, 1 << 64]
     vals += [rng.randrange(1, P) for _ in range(300)]
     for a in vals:
         lib.t28_inverse_by(_u32(_p32([a])[0]), _u32(out))
@@ -137,11 +141,11 @@ def test_inverse_by_divsteps(lib):
 
 
 def _sum_tree(lib, pts, negs):
-    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 24))
+    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 2 * FW))
     neg = np.array(negs, dtype=np.int32)
-    aff = np.zeros(24, dtype=np.uint32)
+    aff = np.zeros(2 * FW, dtype=np.uint32)
     slow = lib.t28_sum_tree(_u32(arr), neg.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), len(pts), _u32(aff))
-    return br.g1_unpack(aff.view(np.uint64).reshape(1, 12))[0], slow
+    return br.g1_unpack(aff.view(np.uint64).reshape(1, br.G1_WORDS))[0], slow
 
 
 def test_accumulator_plus_accumulator(lib):

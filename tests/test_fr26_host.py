@@ -11,7 +11,8 @@ import bigref as br
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "native", "fr26_host.cpp")
-LIB = os.path.join(HERE, "native", "libfr26_host.so")
+BN = br.CURVE == "bn254"
+LIB = os.path.join(HERE, "native", "libfr26_host_bn254.so" if BN else "libfr26_host.so")
 R = br.R_MOD
 
 
@@ -19,7 +20,8 @@ R = br.R_MOD
 def lib():
     deps = [SRC] + [os.path.join(HERE, "..", "grape_amd", "csrc", f) for f in ("fr26.hpp", "field.hpp")]
     if not os.path.exists(LIB) or any(os.path.getmtime(d) > os.path.getmtime(LIB) for d in deps):
-        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas", "-o", LIB, SRC])
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas"]
+                              + (["-DGRAPE_CURVE_BN254"] if BN else []) + ["-o", LIB, SRC])
     return ctypes.CDLL(LIB)
 
 
@@ -35,7 +37,7 @@ def _val(a):
     return br.fr_unpack(np.ascontiguousarray(a).view(np.uint64).reshape(1, 4))[0]
 
 
-EDGE = [0, 1, 2, R - 1, R - 2, (1 << 254), (1 << 255) % R, (1 << 26) - 1, 1 << 26, (1 << 234) - 1, R >> 1, 2**64 - 1]
+EDGE = [0, 1, 2, R - 1, R - 2, (1 << 254) % R, (1 << 255) % R, (1 << 26) - 1, 1 << 26, (1 << 234) - 1, R >> 1, 2**64 - 1]
 
 
 def test_mulc_and_montgomery(lib):

@@ -10,7 +10,8 @@ import orc
 from gpuutil import rand_fr
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-with open(os.path.join(HERE, "golden", "vectors.json")) as f:
+VECTORS = "vectors_bn254.json" if br.CURVE == "bn254" else "vectors.json"
+with open(os.path.join(HERE, "golden", VECTORS)) as f:
     V = json.load(f)
 R = br.R_MOD
 
@@ -40,7 +41,7 @@ def test_fixture_is_reproducible(tmp_path):
     for name in ("bigref.py", "gpuutil.py"):
         shutil.copy(os.path.join(HERE, name), tmp_path / name)
     subprocess.check_call([sys.executable, str(work / "make_vectors.py")])
-    with open(work / "vectors.json") as f:
+    with open(work / VECTORS) as f:
         assert json.load(f) == V
 
 
