@@ -31,14 +31,19 @@ SEED_G = 20240002
 RADIX_BITS = 16        # one signed 16-bit digit per scalar
 K_DIGIT = 32768
 
+# The curve is BLS12-381 (what the benchmark configurations name) unless GRAPE_CURVE=bn254 selects
+# the BN254 build of the libraries and of the oracle.
+CURVE = os.environ.get("GRAPE_CURVE", "bls12_381")
+FP_WORDS, FP_LIMBS28 = (8, 10) if CURVE == "bn254" else (12, 14)
 # Algorithmic work per committed point, the reference's algorithm (two non-zero byte windows of an
-# int16 scalar, each a mixed XYZZ addition of 8M+2S, 300 32x32 multiplies per 12-limb Montgomery
-# product): 2 * 10 * 300.
-ALG_MULS_PER_POINT = 6000
-# What the fast path executes: ONE mixed addition per point on 14 limbs of 28 bits:
-# 6 products of 14*14 + 14*14 + 14 multiply-adds, one fused difference of two products
-# (2*14*14 + 14*14 + 14) and 2 squares of 105 + 14*14 + 14.
-EXEC_MULS_PER_POINT = 6 * (196 + 196 + 14) + (3 * 196 + 14) + 2 * (105 + 196 + 14)
+# int16 scalar, each a mixed XYZZ addition of 8M+2S, 2n^2+n 32x32 multiplies per n-limb Montgomery
+# product: 300 for the 12 limbs of BLS12-381, 136 for the 8 of BN254): 2 * 10 * 300 = 6000.
+ALG_MULS_PER_POINT = 2 * 10 * (2 * FP_WORDS * FP_WORDS + FP_WORDS)
+# What the fast path executes: ONE mixed addition per point on L limbs of 28 bits (L = 14 resp.
+# 10): 6 products of L*L + L*L + L multiply-adds, one fused difference of two products
+# (2*L*L + L*L + L) and 2 squares of L(L+1)/2 + L*L + L: 3668 for L = 14, 1900 for L = 10.
+_L = FP_LIMBS28
+EXEC_MULS_PER_POINT = 6 * (2 * _L * _L + _L) + (3 * _L * _L + _L) + 2 * (_L * (_L + 1) // 2 + _L * _L + _L)
 # lane-level 32x32 multiplies per second if every SIMD issued one v_mad_u64_u32 per cycle:
 # 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz
 PEAK_MULS_NOMINAL = 256 * 64 * 2.4e9
@@ -343,7 +348,8 @@ def lookup_workload(args):
 
 def _fr_const(x):
     """Montgomery limbs of a small constant, as a (1, 4) uint64 array"""
-    r = 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001
+    r = (21888242871839275222246405745257275088548364400416034343698204186575808495617 if CURVE == "bn254"
+         else 0x73eda753299d7d483339d80809a1d80553bda402fffe5bfeffffffff00000001)
     v = (x << 256) % r
     return np.array([[(v >> (64 * i)) & ((1 << 64) - 1) for i in range(4)]], dtype=np.uint64)
 
@@ -423,11 +429,12 @@ def main():
         "peak": peak_measured / 1e12,
         "unit": "Tmul/s",
         "frac": achieved_alg / peak_measured,
-        "traffic": COMMIT_KERNEL_TRAFFIC_BYTES,
+        "traffic": COMMIT_KERNEL_TRAFFIC_BYTES if CURVE == "bls12_381" else None,
         "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the 1 GiB copy kernel "
                           "(FETCH_SIZE unit 2 KiB, WRITE_SIZE unit 1 KiB); algorithmic bytes 2.28e9",
-        "note": "achieved counts the reference algorithm's 6000 multiplies per point; the kernel executes 3668 "
-                "(one addition per point instead of two), so frac can exceed 1 - frac_executed is the issue-rate view",
+        "note": "achieved counts the reference algorithm's %d multiplies per point; the kernel executes %d "
+                "(one addition per point instead of two), so frac can exceed 1 - frac_executed is the issue-rate view"
+                % (ALG_MULS_PER_POINT, EXEC_MULS_PER_POINT),
         "achieved_executed": achieved_exec / 1e12,
         "frac_executed": achieved_exec / peak_measured,
         "peak_nominal": PEAK_MULS_NOMINAL / 1e12,
@@ -487,7 +494,7 @@ def main():
         "config": {"workload": "configs[1]: Hyrax commit of a 4096x4096 int16-range matrix "
                                "(Gaussian sigma=2^10, clipped), 4096 seeded G1 generators, "
                                "small-scalar path, 4096 affine outputs",
-                   "rows": ROWS, "cols": COLS, "radix_bits": RADIX_BITS,
+                   "curve": CURVE, "rows": ROWS, "cols": COLS, "radix_bits": RADIX_BITS,
                    "table_bytes": int(table.numel()) * 4, "table_gen_s": table_gen_s},
         "roofline": roofline,
         "roofline_streaming": roofline_streaming,
