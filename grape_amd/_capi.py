@@ -77,6 +77,15 @@ SIGNATURES = {
     "grape_commit_fr_ref_table": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_void_p],
     "grape_g1_affine_to_jacobian": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_g1_jacobian_to_affine": [c_void_p, c_void_p, c_size_t, c_void_p],
+    "grape_wit_matmul_rescale": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_u32, c_u32, ctypes.c_int64, c_int, c_void_p],
+    "grape_wit_elemul_rescale": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, ctypes.c_int64, c_void_p],
+    "grape_wit_table_lookup": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p, c_void_p],
+    "grape_wit_add_i32": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    "grape_wit_softmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_u32, c_u32,
+                          ctypes.c_int64, c_void_p],
+    "grape_wit_row_sumsq": [c_void_p, c_void_p, c_u32, c_u32, c_void_p],
+    "grape_wit_rmsnorm_apply": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, ctypes.c_int64, c_void_p],
+    "grape_wit_status": [ctypes.POINTER(c_u32), c_void_p],
     "grape_bench_copy": [c_void_p, c_void_p, c_size_t, c_int, ctypes.POINTER(ctypes.c_float), c_void_p],
     "grape_bench_copy_fr": [c_void_p, c_void_p, c_size_t, c_int, ctypes.POINTER(ctypes.c_float), c_void_p],
     "grape_bench_mad_u64_u32": [c_int, c_int, c_int, ctypes.POINTER(ctypes.c_double), c_void_p],

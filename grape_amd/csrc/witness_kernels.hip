@@ -1,0 +1,478 @@
+// Quantised-layer witness generation on the GPU: the fixed-point rules of the reference's Python
+// generator (zzllama/llama/model.py) as integer kernels.  Every product is exact (64-bit
+// accumulation of 32 x 32-bit products: v_mad_i64_i32 issues at the rate of an addition on gfx950),
+// every rescaling is q = floor((y + S/2) / S), r = y - q*S (model.py:489-491), and the epilogue of
+// a matrix product writes quotient and remainder directly, so the 64-bit products never reach
+// memory.
+//
+// Conditions the reference asserts (table indices in range, model.py:86-87) or silently assumes
+// (quotients fit 32 bits) are recorded in a sticky device-side status word, read and cleared by
+// grape_wit_status().
+#include "common.hpp"
+
+namespace grape {
+
+enum WitFlag : uint32_t { kWitQuotient = 1, kWitIndex = 2, kWitSum = 4, kWitSquares = 8 };
+
+// floor((y + s/2) / s) and the centred remainder; s > 0, sh = log2(s) or -1 when s is no power of 2
+__device__ __forceinline__ void rescale64(int64_t y, int64_t s, int sh, int32_t& q, int32_t& r, uint32_t& bad) {
+    const int64_t t = y + (s >> 1);
+    int64_t qq;
+    if (sh >= 0) {
+        qq = t >> sh;                         // arithmetic shift floors
+    } else {
+        qq = t / s;
+        if ((t % s != 0) && (t < 0)) qq -= 1;  // C division truncates; floor wanted
+    }
+    bad |= (qq != (int64_t)(int32_t)qq) ? (uint32_t)kWitQuotient : 0u;
+    q = (int32_t)qq;
+    r = (int32_t)(y - qq * s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Y[l][n][m] = sum_k A[l][n][k] * B[l][m][k], rescaled.  Tile 128 x 128 x 32 per workgroup of 256
+// threads; each thread owns the 8 x 8 outputs (ty + 16 i, tx + 16 j).  Tiles sit in LDS row-major
+// with a row stride of 36 words, which makes the 16-byte fragment reads of 16 consecutive rows hit
+// 16 disjoint groups of 4 banks.  The next tile travels from memory into registers while the
+// current one is multiplied.
+// ------------------------------------------------------------------------------------------------
+constexpr int kTM = 128, kTK = 32, kLd = 36;
+
+struct MatmulArgs {
+    int32_t* q;
+    int32_t* r;          // may be null
+    const int32_t* a;
+    const int32_t* b;
+    uint32_t N, M, K;
+    int64_t scale;
+    int shift;           // log2(scale) or -1
+    int transpose_out;   // write [m][n] instead of [n][m]
+    uint32_t tiles_n, tiles_m;
+    uint32_t* status;
+};
+
+__global__ void __launch_bounds__(256, 2) wit_matmul_tiled_kernel(MatmulArgs p) {
+    __shared__ __attribute__((aligned(16))) int32_t As[kTM * kLd];
+    __shared__ __attribute__((aligned(16))) int32_t Bs[kTM * kLd];
+    // consecutive workgroups go to different XCDs; give each XCD a contiguous run of tiles so
+    // that the tiles sharing rows of A and of B meet in the same L2
+    uint32_t bid = blockIdx.x;
+    const uint32_t nb = gridDim.x;
+    if ((nb & 7u) == 0) bid = (bid & 7u) * (nb >> 3) + (bid >> 3);
+    const uint32_t tn = bid / p.tiles_m, tm = bid - tn * p.tiles_m;
+    const uint32_t l = blockIdx.y;
+    const int32_t* A = p.a + (size_t)l * p.N * p.K;
+    const int32_t* B = p.b + (size_t)l * p.M * p.K;
+    const uint32_t n0 = tn * kTM, m0 = tm * kTM;
+    const uint32_t t = threadIdx.x, tx = t & 15u, ty = t >> 4;
+
+    // staging: 4 + 4 vectors of 4 words per thread; vector v = t + 256 p covers row v / 8, words 4 (v % 8)
+    uint4 sa[4], sb[4];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) {
+            const uint32_t v = t + 256u * pp, row = v >> 3, kk = k0 + 4u * (v & 7u);
+            const bool ka = kk < p.K;     // K is a multiple of 4: a vector is inside or outside as a whole
+            const uint32_t ra = n0 + row < p.N ? n0 + row : p.N - 1, rb = m0 + row < p.M ? m0 + row : p.M - 1;
+            const uint32_t kc = ka ? kk : 0;
+            uint4 va = *reinterpret_cast<const uint4*>(A + (size_t)ra * p.K + kc);
+            uint4 vb = *reinterpret_cast<const uint4*>(B + (size_t)rb * p.K + kc);
+            const bool oka = ka && (n0 + row < p.N), okb = ka && (m0 + row < p.M);
+            sa[pp] = oka ? va : make_uint4(0, 0, 0, 0);
+            sb[pp] = okb ? vb : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) {
+            const uint32_t v = t + 256u * pp, row = v >> 3, c = 4u * (v & 7u);
+            *reinterpret_cast<uint4*>(&As[row * kLd + c]) = sa[pp];
+            *reinterpret_cast<uint4*>(&Bs[row * kLd + c]) = sb[pp];
+        }
+    };
+
+    int64_t acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[i][j] = 0;
+
+    fetch(0);
+    for (uint32_t k0 = 0; k0 < p.K; k0 += kTK) {
+        __syncthreads();                 // everyone is done with the previous tile
+        stage();
+        __syncthreads();
+        if (k0 + kTK < p.K) fetch(k0 + kTK);
+#pragma unroll 1
+        for (int kk = 0; kk < kTK; kk += 4) {
+            int4 fa[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) fa[i] = *reinterpret_cast<const int4*>(&As[(ty + 16 * i) * kLd + kk]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int4 fb = *reinterpret_cast<const int4*>(&Bs[(tx + 16 * j) * kLd + kk]);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    acc[i][j] += (int64_t)fa[i].x * (int64_t)fb.x;
+                    acc[i][j] += (int64_t)fa[i].y * (int64_t)fb.y;
+                    acc[i][j] += (int64_t)fa[i].z * (int64_t)fb.z;
+                    acc[i][j] += (int64_t)fa[i].w * (int64_t)fb.w;
+                }
+            }
+        }
+    }
+
+    uint32_t bad = 0;
+    int32_t* Q = p.q + (size_t)l * p.N * p.M;
+    int32_t* R = p.r ? p.r + (size_t)l * p.N * p.M : nullptr;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t n = n0 + ty + 16 * i;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t m = m0 + tx + 16 * j;
+            if (n < p.N && m < p.M) {
+                int32_t q, r;
+                rescale64(acc[i][j], p.scale, p.shift, q, r, bad);
+                const size_t o = p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m;
+                Q[o] = q;
+                if (R) R[o] = r;
+            }
+        }
+    }
+    if (bad) atomicOr(p.status, bad);
+}
+
+// any shape: one thread per output, used when K is no multiple of 4 or a row is not 16-byte aligned
+__global__ void __launch_bounds__(kBlock) wit_matmul_simple_kernel(MatmulArgs p, uint32_t L) {
+    const size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t per = (size_t)p.N * p.M;
+    if (idx >= per * L) return;
+    const uint32_t l = (uint32_t)(idx / per);
+    const size_t nm = idx - (size_t)l * per;
+    const uint32_t n = (uint32_t)(nm / p.M), m = (uint32_t)(nm - (size_t)n * p.M);
+    const int32_t* a = p.a + ((size_t)l * p.N + n) * p.K;
+    const int32_t* b = p.b + ((size_t)l * p.M + m) * p.K;
+    int64_t acc = 0;
+    for (uint32_t k = 0; k < p.K; k++) acc += (int64_t)a[k] * (int64_t)b[k];
+    uint32_t bad = 0;
+    int32_t q, r;
+    rescale64(acc, p.scale, p.shift, q, r, bad);
+    const size_t o = (size_t)l * per + (p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m);
+    p.q[o] = q;
+    if (p.r) p.r[o] = r;
+    if (bad) atomicOr(p.status, bad);
+}
+
+__global__ void __launch_bounds__(kBlock) wit_elemul_rescale_kernel(int32_t* q, int32_t* r, const int32_t* a, const int32_t* b, size_t n,
+                                                                    int64_t scale, int shift, uint32_t* status) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    uint32_t bad = 0;
+    int32_t qq, rr;
+    rescale64((int64_t)a[i] * (int64_t)b[i], scale, shift, qq, rr, bad);
+    q[i] = qq;
+    if (r) r[i] = rr;
+    if (bad) atomicOr(status, bad);
+}
+
+__global__ void __launch_bounds__(kBlock) wit_lookup_kernel(int32_t* out, const int32_t* in, size_t n, int32_t low, uint32_t len,
+                                                            const int32_t* table, uint32_t* status) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t idx = (int64_t)in[i] - (int64_t)low;
+    const bool ok = idx >= 0 && idx < (int64_t)len;
+    out[i] = table[ok ? idx : 0];
+    if (!ok) atomicOr(status, (uint32_t)kWitIndex);
+}
+
+__global__ void __launch_bounds__(kBlock) wit_add_kernel(int32_t* out, const int32_t* a, const int32_t* b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = (int32_t)((uint32_t)a[i] + (uint32_t)b[i]);
+}
+
+// block-wide reductions over 256 threads (4 waves)
+__device__ __forceinline__ int32_t block_max_i32(int32_t v, int32_t* sh) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const int32_t o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    int32_t m = sh[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / 64; w++) m = sh[w] > m ? sh[w] : m;
+    __syncthreads();
+    return m;
+}
+__device__ __forceinline__ uint64_t block_sum_u64(uint64_t v, uint64_t* sh) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor((unsigned long long)v, off, 64);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    uint64_t s = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) s += sh[w];
+    __syncthreads();
+    return s;
+}
+
+// One workgroup per row of the scores (model.py:76-116).
+__global__ void __launch_bounds__(kBlock) wit_softmax_kernel(int32_t* out_max, int32_t* out_shift, int32_t* out_exp, int32_t* out_sum,
+                                                             int32_t* out_prob, int32_t* out_query, const int32_t* scores, uint32_t cols,
+                                                             const int32_t* table, uint32_t offset, uint32_t len, int64_t scale,
+                                                             uint32_t* status) {
+    __shared__ int32_t sh_i[kBlock / 64];
+    __shared__ uint64_t sh_u[kBlock / 64];
+    const size_t row = blockIdx.x;
+    const int32_t* x = scores + row * cols;
+    int32_t mx = INT32_MIN;
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) mx = x[c] > mx ? x[c] : mx;
+    mx = block_max_i32(mx, sh_i);
+    uint64_t sum = 0;
+    uint32_t bad = 0;
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) {
+        const int64_t d = (int64_t)x[c] - (int64_t)mx;               // <= 0
+        const int64_t idx = d + (int64_t)offset;
+        const bool ok = idx >= 0 && idx < (int64_t)len;
+        const int32_t e = table[ok ? idx : 0];
+        bad |= ok ? 0u : (uint32_t)kWitIndex;
+        bad |= e < 0 ? (uint32_t)kWitSum : 0u;
+        out_shift[row * cols + c] = (int32_t)d;
+        out_exp[row * cols + c] = e;
+        sum += (uint64_t)(uint32_t)(e < 0 ? 0 : e);
+    }
+    sum = block_sum_u64(sum, sh_u);
+    if (sum == 0) {
+        bad |= (uint32_t)kWitSum;
+        sum = 1;
+    }
+    if (threadIdx.x == 0) {
+        out_max[row] = mx;
+        out_sum[row] = (int32_t)sum;            // the reference stores the 64-bit sum as int32 (model.py:103)
+    }
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) {
+        const uint64_t e = (uint64_t)(uint32_t)out_exp[row * cols + c];   // this thread's own earlier store
+        const uint64_t o = (e * (uint64_t)scale + (sum >> 1)) / sum;
+        out_prob[row * cols + c] = (int32_t)o;
+        out_query[row * cols + c] = (int32_t)((int64_t)(e * 2u * (uint64_t)scale) - (int64_t)sum * (2 * (int64_t)o - 1));
+    }
+    if (bad) atomicOr(status, bad);
+}
+
+// per row: exact sum of squares as a 64-bit integer (status flag when it leaves 64 bits)
+__global__ void __launch_bounds__(kBlock) wit_row_sumsq_kernel(uint64_t* out, const int32_t* x, uint32_t cols, uint32_t* status) {
+    __shared__ uint64_t sh_u[kBlock / 64];
+    const size_t row = blockIdx.x;
+    uint64_t lo = 0, hi = 0;
+    for (uint32_t c = threadIdx.x; c < cols; c += kBlock) {
+        const int64_t v = x[row * cols + c];
+        const uint64_t sq = (uint64_t)(v * v);
+        lo += sq;
+        hi += lo < sq ? 1u : 0u;
+    }
+    // the high parts and the low parts are summed separately; low parts are split so that their
+    // block sum cannot wrap (256 values below 2^56 each)
+    const uint64_t lo_lo = lo & 0x00ffffffffffffffull, lo_hi = lo >> 56;
+    const uint64_t s_lo = block_sum_u64(lo_lo, sh_u);
+    const uint64_t s_hi = block_sum_u64(lo_hi + (hi << 8), sh_u);     // units of 2^56
+    if (threadIdx.x == 0) {
+        const uint64_t top = s_hi + (s_lo >> 56);                      // total = top * 2^56 + (s_lo mod 2^56)
+        if (top >> 8) atomicOr(status, (uint32_t)kWitSquares);
+        out[row] = (top << 56) | (s_lo & 0x00ffffffffffffffull);
+    }
+}
+
+// model.py:228-234: rms_w = rescale(rms[row] * w[col]); out = rescale(rms_w.q * x)
+__global__ void __launch_bounds__(kBlock) wit_rmsnorm_apply_kernel(int32_t* q_rmsw, int32_t* r_rmsw, int32_t* q_out, int32_t* r_out,
+                                                                   const int32_t* x, const int32_t* rms, const int32_t* w, size_t n,
+                                                                   uint32_t cols, int64_t scale, int shift, uint32_t* status) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const size_t row = i / cols;
+    const uint32_t col = (uint32_t)(i - row * cols);
+    uint32_t bad = 0;
+    int32_t q1, r1, q2, r2;
+    rescale64((int64_t)rms[row] * (int64_t)w[col], scale, shift, q1, r1, bad);
+    rescale64((int64_t)q1 * (int64_t)x[i], scale, shift, q2, r2, bad);
+    q_rmsw[i] = q1;
+    r_rmsw[i] = r1;
+    q_out[i] = q2;
+    r_out[i] = r2;
+    if (bad) atomicOr(status, bad);
+}
+
+__global__ void wit_status_clear_kernel(uint32_t* status) { *status = 0; }
+
+static uint32_t* g_status[16] = {nullptr};
+
+static int status_word(uint32_t** out, hipStream_t s) {
+    int dev = 0;
+    GRAPE_HIP_CHECK(hipGetDevice(&dev));
+    GRAPE_REQUIRE(dev >= 0 && dev < 16, "device index out of range");
+    if (!g_status[dev]) {
+        GRAPE_HIP_CHECK(hipMalloc((void**)&g_status[dev], 256));
+        wit_status_clear_kernel<<<1, 1, 0, s>>>(g_status[dev]);
+        GRAPE_LAUNCH_CHECK();
+        GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    }
+    *out = g_status[dev];
+    return GRAPE_OK;
+}
+
+static int log2_exact(int64_t s) {
+    if (s <= 0 || (s & (s - 1)) != 0) return -1;
+    int sh = 0;
+    while ((((int64_t)1) << sh) != s) sh++;
+    return sh;
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+#define CHECK_PTR(p) GRAPE_REQUIRE((p) != nullptr, #p " is null")
+
+extern "C" {
+
+int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, const int32_t* d_b, uint32_t L, uint32_t N, uint32_t M,
+                             uint32_t K, int64_t scale, int transpose_out, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    GRAPE_REQUIRE(scale >= 1 && scale <= ((int64_t)1 << 31), "scale must be in 1..2^31 (the remainder is stored as int32)");
+    if (L == 0 || N == 0 || M == 0) return GRAPE_OK;
+    CHECK_PTR(d_q); CHECK_PTR(d_a); CHECK_PTR(d_b);
+    GRAPE_REQUIRE(K >= 1, "empty inner dimension");
+    GRAPE_REQUIRE((uint64_t)L * N * M < ((uint64_t)1 << 40) && (uint64_t)N * K < ((uint64_t)1 << 40) && (uint64_t)M * K < ((uint64_t)1 << 40),
+                  "tensor too large");
+    hipStream_t s = as_stream(st);
+    MatmulArgs p;
+    p.q = d_q; p.r = d_r; p.a = d_a; p.b = d_b;
+    p.N = N; p.M = M; p.K = K;
+    p.scale = scale;
+    p.shift = log2_exact(scale);
+    p.transpose_out = transpose_out ? 1 : 0;
+    p.tiles_n = (N + kTM - 1) / kTM;
+    p.tiles_m = (M + kTM - 1) / kTM;
+    int rc = status_word(&p.status, s);
+    if (rc) return rc;
+    const bool aligned = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_a) | reinterpret_cast<uintptr_t>(d_b)) & 15) == 0;
+    if (profiling()) {
+        profile_begin();
+        profile_mark(s);
+    }
+    if (aligned && L <= 65535) {
+        dim3 grid(p.tiles_n * p.tiles_m, L);
+        wit_matmul_tiled_kernel<<<grid, 256, 0, s>>>(p);
+    } else {
+        wit_matmul_simple_kernel<<<blocks_for((size_t)L * N * M), kBlock, 0, s>>>(p, L);
+    }
+    GRAPE_LAUNCH_CHECK();
+    if (profiling()) profile_mark(s);
+    return GRAPE_OK;
+}
+
+int grape_wit_elemul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, const int32_t* d_b, size_t n, int64_t scale, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    GRAPE_REQUIRE(scale >= 1 && scale <= ((int64_t)1 << 31), "scale must be in 1..2^31 (the remainder is stored as int32)");
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR(d_q); CHECK_PTR(d_a); CHECK_PTR(d_b);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    wit_elemul_rescale_kernel<<<blocks_for(n), kBlock, 0, s>>>(d_q, d_r, d_a, d_b, n, scale, log2_exact(scale), status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_table_lookup(int32_t* d_out, const int32_t* d_in, size_t n, int32_t low, uint32_t len, const int32_t* d_table, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    GRAPE_REQUIRE(len >= 1, "empty table");
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR(d_out); CHECK_PTR(d_in); CHECK_PTR(d_table);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    wit_lookup_kernel<<<blocks_for(n), kBlock, 0, s>>>(d_out, d_in, n, low, len, d_table, status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_add_i32(int32_t* d_out, const int32_t* d_a, const int32_t* d_b, size_t n, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR(d_out); CHECK_PTR(d_a); CHECK_PTR(d_b);
+    wit_add_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(d_out, d_a, d_b, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_softmax(int32_t* d_max, int32_t* d_shifted, int32_t* d_exp, int32_t* d_sum, int32_t* d_prob, int32_t* d_query,
+                      const int32_t* d_scores, uint32_t rows, uint32_t cols, const int32_t* d_table, uint32_t bit_shift,
+                      uint32_t index_bits, int64_t scale, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    GRAPE_REQUIRE(bit_shift >= 1 && bit_shift <= 30 && index_bits >= 1 && index_bits <= 30, "bit_shift and index_bits must be in 1..30");
+    GRAPE_REQUIRE(scale >= 1 && scale <= ((int64_t)1 << 30), "scale must be in 1..2^30");
+    if (rows == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(cols >= 1, "empty rows");
+    CHECK_PTR(d_max); CHECK_PTR(d_shifted); CHECK_PTR(d_exp); CHECK_PTR(d_sum); CHECK_PTR(d_prob); CHECK_PTR(d_query);
+    CHECK_PTR(d_scores); CHECK_PTR(d_table);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    wit_softmax_kernel<<<rows, kBlock, 0, s>>>(d_max, d_shifted, d_exp, d_sum, d_prob, d_query, d_scores, cols, d_table,
+                                               (1u << bit_shift) - 1u, 1u << index_bits, scale, status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_row_sumsq(uint64_t* d_out, const int32_t* d_x, uint32_t rows, uint32_t cols, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    if (rows == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(cols >= 1, "empty rows");
+    CHECK_PTR(d_out); CHECK_PTR(d_x);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    wit_row_sumsq_kernel<<<rows, kBlock, 0, s>>>(d_out, d_x, cols, status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_rmsnorm_apply(int32_t* d_q_rmsw, int32_t* d_r_rmsw, int32_t* d_q_out, int32_t* d_r_out, const int32_t* d_x,
+                            const int32_t* d_rms, const int32_t* d_w, uint32_t rows, uint32_t cols, int64_t scale, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    GRAPE_REQUIRE(scale >= 1 && scale <= ((int64_t)1 << 31), "scale must be in 1..2^31 (the remainder is stored as int32)");
+    if (rows == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(cols >= 1, "empty rows");
+    CHECK_PTR(d_q_rmsw); CHECK_PTR(d_r_rmsw); CHECK_PTR(d_q_out); CHECK_PTR(d_r_out); CHECK_PTR(d_x); CHECK_PTR(d_rms); CHECK_PTR(d_w);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    const size_t n = (size_t)rows * cols;
+    wit_rmsnorm_apply_kernel<<<blocks_for(n), kBlock, 0, s>>>(d_q_rmsw, d_r_rmsw, d_q_out, d_r_out, d_x, d_rms, d_w, n, cols, scale,
+                                                              log2_exact(scale), status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wit_status(uint32_t* flags, grape_stream_t st) {
+    GRAPE_REQUIRE(initialised(), "grape_init has not been called");
+    CHECK_PTR(flags);
+    hipStream_t s = as_stream(st);
+    uint32_t* status;
+    int rc = status_word(&status, s);
+    if (rc) return rc;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(flags, status, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    wit_status_clear_kernel<<<1, 1, 0, s>>>(status);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+}  // extern "C"

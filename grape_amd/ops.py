@@ -376,6 +376,84 @@ def g1_jacobian_to_affine(a):
     return out
 
 
+# ------------------------------------------------------------------ witness generation
+def _i32(*shape):
+    return torch.empty(shape, dtype=torch.int32, device="cuda")
+
+
+def wit_matmul_rescale(a, b, scale, want_r=True, transpose_out=False):
+    """a: (L, N, K) or (N, K) int32, b: (L, M, K) or (M, K) -> quotient, remainder of a . b^T"""
+    lib = init()
+    batched = a.dim() == 3
+    L = a.shape[0] if batched else 1
+    N, K = a.shape[-2], a.shape[-1]
+    M = b.shape[-2]
+    assert b.shape[-1] == K and (not batched or b.shape[0] == L)
+    shape = ((L,) if batched else ()) + ((M, N) if transpose_out else (N, M))
+    q = _i32(*shape)
+    r = _i32(*shape) if want_r else None
+    _capi.check(lib.grape_wit_matmul_rescale(_p(q), _p(r), _p(a), _p(b), L, N, M, K, int(scale), 1 if transpose_out else 0, _s()))
+    return q, r
+
+
+def wit_elemul_rescale(a, b, scale):
+    lib = init()
+    q, r = torch.empty_like(a), torch.empty_like(a)
+    _capi.check(lib.grape_wit_elemul_rescale(_p(q), _p(r), _p(a), _p(b), a.numel(), int(scale), _s()))
+    return q, r
+
+
+def wit_table_lookup(x, low, table):
+    lib = init()
+    out = torch.empty_like(x)
+    _capi.check(lib.grape_wit_table_lookup(_p(out), _p(x), x.numel(), int(low), table.numel(), _p(table), _s()))
+    return out
+
+
+def wit_add(a, b):
+    lib = init()
+    out = torch.empty_like(a)
+    _capi.check(lib.grape_wit_add_i32(_p(out), _p(a), _p(b), a.numel(), _s()))
+    return out
+
+
+def wit_softmax(scores, table, bit_shift=20, index_bits=20, scale=1 << 16):
+    """scores (rows, cols) int32 -> dict of the tensors the reference saves for its table softmax"""
+    lib = init()
+    rows, cols = scores.shape
+    out = {"max": _i32(rows, 1), "exp_input": _i32(rows, cols), "exp_output": _i32(rows, cols), "exp_sum": _i32(rows, 1),
+           "softmax_output": _i32(rows, cols), "softmax_lookup_query": _i32(rows, cols)}
+    _capi.check(lib.grape_wit_softmax(_p(out["max"]), _p(out["exp_input"]), _p(out["exp_output"]), _p(out["exp_sum"]),
+                                      _p(out["softmax_output"]), _p(out["softmax_lookup_query"]), _p(scores), rows, cols,
+                                      _p(table), bit_shift, index_bits, int(scale), _s()))
+    return out
+
+
+def wit_row_sumsq(x):
+    lib = init()
+    rows, cols = x.shape
+    out = torch.empty(rows, dtype=torch.int64, device="cuda")
+    _capi.check(lib.grape_wit_row_sumsq(_p(out), _p(x), rows, cols, _s()))
+    return out
+
+
+def wit_rmsnorm_apply(x, rms, w, scale=1 << 16):
+    lib = init()
+    rows, cols = x.shape
+    outs = [_i32(rows, cols) for _ in range(4)]
+    _capi.check(lib.grape_wit_rmsnorm_apply(_p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), _p(x), _p(rms), _p(w), rows, cols,
+                                            int(scale), _s()))
+    return outs
+
+
+def wit_status():
+    """status bits set since the last call (synchronises and clears them)"""
+    lib = init()
+    f = ctypes.c_uint32(0)
+    _capi.check(lib.grape_wit_status(ctypes.byref(f), _s()))
+    return f.value
+
+
 # ------------------------------------------------------------------ measurement
 def bench_copy(nbytes, iters=10):
     lib = init()

@@ -12,7 +12,9 @@
  *     src/fr-tensor.cu:214,352,437;
  *   - an Fp element is 12 x u32 (x*2^384 mod p); an affine G1 point is {x,y} = 96 bytes with
  *     infinity = all zero (include/curve/affine_t.cuh:28-39); a Jacobian point is {X,Y,Z} = 144
- *     bytes with Z = 0 for infinity; an XYZZ accumulator is {X,Y,ZZ,ZZZ} = 192 bytes;
+ *     bytes with Z = 0 for infinity; an XYZZ accumulator is {X,Y,ZZ,ZZZ} = 192 bytes.  These are
+ *     the sizes of the BLS12-381 library; the BN254 build of the same sources (libgrape_hip_bn254.so,
+ *     include/field/alt_bn128.cuh) has Fp = 8 x u32 (x*2^256 mod p) and points of 64 / 96 / 128 bytes;
  *   - every function returns 0 on success and a negative GRAPE_E* code otherwise;
  *     grape_last_error() gives the message.  Nothing is printed, nothing throws;
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Kernels are only
@@ -236,6 +238,49 @@ int grape_commit_fr_ref_table(uint32_t *d_out_affine, const uint32_t *d_scalars_
 /* Format conversions for callers that keep the reference's jacob_t arrays. */
 int grape_g1_affine_to_jacobian(uint32_t *d_out_jac, const uint32_t *d_in_affine, size_t n, grape_stream_t stream);
 int grape_g1_jacobian_to_affine(uint32_t *d_out_affine, const uint32_t *d_in_jac, size_t n, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ witness generation ------- */
+/* The fixed-point rules of the reference's witness generator (zzllama/llama/model.py) on int32
+ * device tensors.  Conditions the reference asserts or assumes (table index in range, quotient
+ * fits int32, row sum positive, sum of squares below 2^64) do not fail the call: they set bits of a
+ * sticky per-device status word, see grape_wit_status.
+ *
+ * Y[l][n][m] = sum_k a[l][n][k] * b[l][m][k] exactly (64-bit), then q = floor((Y + scale/2) / scale)
+ * and r = Y - q*scale (1 <= scale <= 2^31); d_r may be NULL; transpose_out writes [l][m][n].  The matrix products and
+ * rescalings of model.py:485-491, :547-550, :574-583, :646-658, :683-686. */
+int grape_wit_matmul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, const int32_t *d_b, uint32_t L, uint32_t N,
+                             uint32_t M, uint32_t K, int64_t scale, int transpose_out, grape_stream_t stream);
+/* q, r of a[i] * b[i] (d_r may be NULL).  model.py:673-675. */
+int grape_wit_elemul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, const int32_t *d_b, size_t n, int64_t scale,
+                             grape_stream_t stream);
+/* out[i] = table[in[i] - low] for in[i] in [low, low + len).  my_silu, model.py:118-149 (low = -2^18, len = 2^19). */
+int grape_wit_table_lookup(int32_t *d_out, const int32_t *d_in, size_t n, int32_t low, uint32_t len, const int32_t *d_table,
+                           grape_stream_t stream);
+/* out[i] = a[i] + b[i] (the two skip connections, model.py:764-771). */
+int grape_wit_add_i32(int32_t *d_out, const int32_t *d_a, const int32_t *d_b, size_t n, grape_stream_t stream);
+/* Row-wise table softmax, my_softmax, model.py:76-116: max[rows], shifted = x - max, exp =
+ * table[shifted + 2^bit_shift - 1] (table of 2^index_bits entries), sum[rows] (low 32 bits, as the
+ * reference stores it), prob = floor((exp*scale + floor(sum/2)) / sum), query = 2*scale*exp -
+ * sum*(2*prob - 1); all outputs rows x cols int32 except max and sum. */
+int grape_wit_softmax(int32_t *d_max, int32_t *d_shifted, int32_t *d_exp, int32_t *d_sum, int32_t *d_prob, int32_t *d_query,
+                      const int32_t *d_scores, uint32_t rows, uint32_t cols, const int32_t *d_table, uint32_t bit_shift,
+                      uint32_t index_bits, int64_t scale, grape_stream_t stream);
+/* out[row] = sum of x[row][c]^2 as an exact 64-bit integer: the integer part of RMSNorm's mean
+ * square (model.py:193); the float16 reciprocal root is taken on the host from this sum. */
+int grape_wit_row_sumsq(uint64_t *d_out, const int32_t *d_x, uint32_t rows, uint32_t cols, grape_stream_t stream);
+/* RMSNorm.forward, model.py:228-234, given rms_int per row: (q,r)_rmsw = rescale(rms[row] * w[col]),
+ * (q,r)_out = rescale(q_rmsw * x). */
+int grape_wit_rmsnorm_apply(int32_t *d_q_rmsw, int32_t *d_r_rmsw, int32_t *d_q_out, int32_t *d_r_out, const int32_t *d_x,
+                            const int32_t *d_rms, const int32_t *d_w, uint32_t rows, uint32_t cols, int64_t scale,
+                            grape_stream_t stream);
+/* Synchronises, returns the status bits set since the last call and clears them: 1 = a quotient left
+ * int32, 2 = a table index out of range (the reference's assertions, model.py:86-87, :137-138),
+ * 4 = a softmax row summed to zero or met a negative table entry, 8 = a sum of squares left 64 bits. */
+#define GRAPE_WIT_QUOTIENT 1u
+#define GRAPE_WIT_INDEX 2u
+#define GRAPE_WIT_SUM 4u
+#define GRAPE_WIT_SQUARES 8u
+int grape_wit_status(uint32_t *flags, grape_stream_t stream);
 
 /* ------------------------------------------------------------------ measurement -------------- */
 /* Device-to-device copy of `bytes` with the library's own streaming kernel, `iters` times;
