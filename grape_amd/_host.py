@@ -13,7 +13,9 @@ NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seco
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
          "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
          "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
-         "grape_host_generate_data", "grape_host_single_commit"]
+         "grape_host_generate_data", "grape_host_single_commit", "grape_host_layer_witness_new", "grape_host_layer_witness_generate",
+         "grape_host_layer_witness_names", "grape_host_layer_witness_tensor", "grape_host_layer_witness_save",
+         "grape_host_layer_witness_free", "grape_host_witness_tables", "grape_host_to_float16"]
 
 
 class HostError(RuntimeError):
@@ -35,6 +37,8 @@ def load():
         lib.grape_host_last_prove_seconds.restype = ctypes.c_double
         lib.grape_host_last_commit_seconds.restype = ctypes.c_double
         lib.grape_host_findsize.restype = ctypes.c_ulong
+        lib.grape_host_to_float16.restype = ctypes.c_double
+        lib.grape_host_to_float16.argtypes = [ctypes.c_double]
         lib.grape_host_findsize.argtypes = [ctypes.c_char_p]
         lib.grape_host_bin_io.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
         lib.grape_host_load_data.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_uint32)]
@@ -230,3 +234,70 @@ def single_commit(d_scalars, N, d_table, npoints):
     out = np.zeros(G1W, dtype=np.uint64)
     _check(load().grape_host_single_commit(_dp(d_scalars), N, _dp(d_table), npoints, _hp(out)))
     return out
+
+
+# ------------------------------------------------------------------ witness generator
+WEIGHT_ORDER = ("Q", "K", "V", "O", "gate", "up", "down", "NormFirst", "NormSecond")
+
+
+def witness_tables():
+    """(exp table, SiLU table) as numpy int32 arrays, from the C++ generator"""
+    e = np.zeros(1 << 20, dtype=np.int32)
+    s = np.zeros(1 << 19, dtype=np.int32)
+    _check(load().grape_host_witness_tables(_hp(e), _hp(s)))
+    return e, s
+
+
+def to_float16(x):
+    return load().grape_host_to_float16(float(x))
+
+
+class LayerWitness:
+    """handle on the C++ LayerWitness; tensors come back as torch int32 views of device memory that
+    stay valid while this object lives"""
+
+    def __init__(self, seq_len, dim, hidden):
+        self._h = ctypes.c_void_p()
+        self.shape = (seq_len, dim, hidden)
+        _check(load().grape_host_layer_witness_new(ctypes.byref(self._h), ctypes.c_uint32(seq_len), ctypes.c_uint32(dim), ctypes.c_uint32(hidden)))
+
+    def generate(self, x, weights, exp_table, silu_table, eps=1e-5):
+        """x, weights[name], tables: contiguous CUDA int32 tensors"""
+        self._keep = (x, dict(weights), exp_table, silu_table)
+        ptrs = (ctypes.c_void_p * 9)(*[weights[k].data_ptr() for k in WEIGHT_ORDER])
+        _check(load().grape_host_layer_witness_generate(self._h, _dp(x), ptrs, _dp(exp_table), _dp(silu_table), ctypes.c_double(eps)))
+
+    def names(self):
+        buf = ctypes.create_string_buffer(1 << 14)
+        _check(load().grape_host_layer_witness_names(self._h, buf, ctypes.c_size_t(len(buf))))
+        return [n for n in buf.value.decode().split("\n") if n]
+
+    def tensor(self, name):
+        """host copy (numpy int32, flat)"""
+        p = ctypes.c_void_p()
+        n = ctypes.c_size_t(0)
+        _check(load().grape_host_layer_witness_tensor(self._h, name.encode(), ctypes.byref(p), ctypes.byref(n)))
+        out = np.zeros(n.value, dtype=np.int32)
+        from . import _capi
+        _capi.check(_capi.load().grape_memcpy_d2h(_hp(out), p, n.value * 4, None))
+        return out
+
+    def device_ptr(self, name):
+        p = ctypes.c_void_p()
+        n = ctypes.c_size_t(0)
+        _check(load().grape_host_layer_witness_tensor(self._h, name.encode(), ctypes.byref(p), ctypes.byref(n)))
+        return p.value, n.value
+
+    def save(self, data_dir, group):
+        _check(load().grape_host_layer_witness_save(self._h, data_dir.encode(), ctypes.c_uint32(group)))
+
+    def close(self):
+        if self._h:
+            _check(load().grape_host_layer_witness_free(self._h))
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libgrape_host.so")
-SOURCES = ["fr.cpp", "polynomial.cpp", "fr_tensor.cpp", "ec_operation.cpp", "hyrax.cpp", "prove.cpp", "tlookup.cpp", "ioutils.cpp", "timer.cpp", "host_capi.cpp"]
+SOURCES = ["fr.cpp", "polynomial.cpp", "fr_tensor.cpp", "ec_operation.cpp", "hyrax.cpp", "prove.cpp", "tlookup.cpp", "ioutils.cpp", "timer.cpp", "witness.cpp", "host_capi.cpp"]
 
 
 # flavour -> (library, extra compiler flags, kernel library to link)

@@ -8,6 +8,7 @@
 #include "hyrax.hpp"
 #include "prove.hpp"
 #include "tlookup.hpp"
+#include "witness.hpp"
 
 static thread_local std::string g_err;
 static double g_last_prove_s = 0;
@@ -318,5 +319,59 @@ int grape_host_generate_data(int32_t** d_out, uint32_t size) {
     *d_out = p;
     GUARD_END
 }
+
+
+int grape_host_layer_witness_new(void** handle, uint32_t seq_len, uint32_t dim, uint32_t hidden) {
+    GUARD_BEGIN
+    *handle = new LayerWitness(seq_len, dim, hidden);
+    GUARD_END
+}
+int grape_host_layer_witness_generate(void* handle, const int32_t* d_x, const int32_t* const* w, const int32_t* d_exp,
+                                      const int32_t* d_silu, double eps) {
+    GUARD_BEGIN
+    LayerWitness::Weights ws{w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8]};
+    LayerWitness::Tables tb{d_exp, d_silu};
+    ProveTimer timer;
+    static_cast<LayerWitness*>(handle)->generate(d_x, ws, tb, eps);
+    GUARD_END
+}
+int grape_host_layer_witness_names(void* handle, char* buf, size_t cap) {
+    GUARD_BEGIN
+    std::string all;
+    for (const auto& n : static_cast<LayerWitness*>(handle)->names()) all += n + "\n";
+    if (all.size() + 1 > cap) throw std::length_error("name buffer too small");
+    std::memcpy(buf, all.c_str(), all.size() + 1);
+    GUARD_END
+}
+int grape_host_layer_witness_tensor(void* handle, const char* name, const int32_t** d_ptr, size_t* size) {
+    GUARD_BEGIN
+    const LayerWitness* lw = static_cast<LayerWitness*>(handle);
+    *d_ptr = lw->tensor(name);
+    *size = lw->tensor_size(name);
+    GUARD_END
+}
+int grape_host_layer_witness_save(void* handle, const char* dir, uint32_t group) {
+    GUARD_BEGIN
+    static_cast<LayerWitness*>(handle)->save(dir, group);
+    GUARD_END
+}
+int grape_host_layer_witness_free(void* handle) {
+    GUARD_BEGIN
+    delete static_cast<LayerWitness*>(handle);
+    GUARD_END
+}
+int grape_host_witness_tables(int32_t* exp_out, int32_t* silu_out) {
+    GUARD_BEGIN
+    if (exp_out) {
+        std::vector<int> t = LayerWitness::make_exp_table();
+        std::memcpy(exp_out, t.data(), sizeof(int) * t.size());
+    }
+    if (silu_out) {
+        std::vector<int> t = LayerWitness::make_silu_table();
+        std::memcpy(silu_out, t.data(), sizeof(int) * t.size());
+    }
+    GUARD_END
+}
+double grape_host_to_float16(double x) { return LayerWitness::to_float16(x); }
 
 }  // extern "C"

@@ -84,6 +84,21 @@ unsigned long grape_host_findsize(const char *filename);
 int grape_host_load_data(const char *filename, int32_t **d_out, uint32_t *n);
 int grape_host_generate_data(int32_t **d_out, uint32_t size);
 
+/* Quantised-layer witness generator (witness.hpp; zzllama/llama/model.py).  d_weights9: device int32
+ * pointers in the order Q, K, V, O, gate, up, down, NormFirst, NormSecond.  _names writes the tensor
+ * names separated by '\n' into buf (NUL-terminated); _tensor returns the device pointer and element
+ * count of one tensor; _save appends all tensors to <dir>/<W|Q|R>/<name>-<group>.bin. */
+int grape_host_layer_witness_new(void **handle, uint32_t seq_len, uint32_t dim, uint32_t hidden);
+int grape_host_layer_witness_generate(void *handle, const int32_t *d_x, const int32_t *const *d_weights9, const int32_t *d_exp,
+                                      const int32_t *d_silu, double eps);
+int grape_host_layer_witness_names(void *handle, char *buf, size_t cap);
+int grape_host_layer_witness_tensor(void *handle, const char *name, const int32_t **d_ptr, size_t *size);
+int grape_host_layer_witness_save(void *handle, const char *dir, uint32_t group);
+int grape_host_layer_witness_free(void *handle);
+/* The exp (2^20 entries) and SiLU (2^19 entries) tables into host arrays; round-to-nearest-even float16. */
+int grape_host_witness_tables(int32_t *exp_out, int32_t *silu_out);
+double grape_host_to_float16(double x);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,9 +2,11 @@
 // little-endian dumps of device or host buffers.  The formats are the reference's own:
 //   * int tensors  (data/{W,Q,R}/*.bin): int32, row-major;
 //   * Fr tensors:  fr_t[n], 32 bytes each, Montgomery form;
-//   * points.bin:  affine_t[256 * npoints], entry w * npoints + i = w * G_i, 96 bytes each;
-//   * commitments: jacob_t[rows], 144 bytes each.
-// (Files written for BN254 by the reference are not interchangeable with this BLS12-381 build.)
+//   * points.bin:  affine_t[256 * npoints], entry w * npoints + i = w * G_i, 96 bytes each
+//                  (64 in the BN254 build);
+//   * commitments: jacob_t[rows], 144 bytes each (96 in the BN254 build).
+// Point files are specific to the curve the library was built for; the BN254 build
+// (-DGRAPE_CURVE_BN254) reads and writes the layout of the reference's own BN254 build.
 #pragma once
 #include <string>
 

@@ -146,3 +146,49 @@ def test_full_size_matmul_properties(ops):
     y = torch.matmul(x[rows].double(), w.double().t()).to(torch.int64)
     assert torch.equal(q[rows].to(torch.int64) * S + r[rows].to(torch.int64), y)
     assert ops.wit_status() == 0
+
+
+# ------------------------------------------------------------------ the C++ LayerWitness class
+def _run_layer(T, D, F, seed):
+    from grape_amd import _host as host
+    x, weights = witutil.layer_inputs(T, D, F, seed)
+    e, s = wo.exp_table(), wo.silu_table()
+    lw = host.LayerWitness(T, D, F)
+    lw.generate(dev(x), {k: dev(v) for k, v in weights.items()}, dev(e), dev(s))
+    want = wo.layer(x, weights, {"exp": e, "silu": s})
+    return lw, want
+
+
+@pytest.mark.parametrize("T,D,F,seed", [(8, 64, 176, 6), (5, 36, 50, 7), (64, 256, 688, 8)])
+def test_layer_witness_matches_the_oracle_tensor_by_tensor(ops, T, D, F, seed):
+    lw, want = _run_layer(T, D, F, seed)
+    assert sorted(lw.names()) == sorted(witutil.TENSOR_NAMES)
+    for name in witutil.TENSOR_NAMES:
+        got = lw.tensor(name)
+        assert got.size == want[name].size, name
+        assert np.array_equal(got, want[name].reshape(-1)), name
+    lw.close()
+
+
+def test_layer_witness_files_follow_the_reference_layout(ops, tmp_path):
+    """save() appends raw int32 to <dir>/<W|Q|R>/<name>-<group>.bin, one layer after the other"""
+    for d in ("W", "Q", "R"):
+        (tmp_path / d).mkdir()
+    lw, want = _run_layer(8, 64, 176, 6)
+    lw.save(str(tmp_path), 3)
+    lw.save(str(tmp_path), 3)                       # a second layer of the same group is appended
+    for name in witutil.TENSOR_NAMES:
+        data = np.fromfile(tmp_path / (name + "-3.bin"), dtype=np.int32)
+        flat = want[name].reshape(-1)
+        assert data.size == 2 * flat.size and np.array_equal(data[:flat.size], flat) and np.array_equal(data[flat.size:], flat), name
+    lw.close()
+
+
+def test_layer_witness_raises_where_the_reference_asserts(ops):
+    from grape_amd import _host as host
+    x, weights = witutil.layer_inputs(8, 64, 176, 9)
+    weights["gate"] = weights["gate"] * 4096          # gate pre-activations far beyond the SiLU table
+    lw = host.LayerWitness(8, 64, 176)
+    with pytest.raises(host.HostError, match="table index"):
+        lw.generate(dev(x), {k: dev(v) for k, v in weights.items()}, dev(wo.exp_table()), dev(wo.silu_table()))
+    lw.close()

@@ -58,3 +58,19 @@ def test_cpp_driver_compiles_against_the_host_headers():
     exe = driver_build.build()
     import os
     assert os.path.exists(exe)
+
+
+def test_witness_tables_and_float16_match_the_oracle():
+    """the C++ table generators and float16 rounding against the numpy oracle (no GPU involved)"""
+    import numpy as np
+    from oracle import witness_oracle as wo
+    from grape_amd import _host as host
+    e, s = host.witness_tables()
+    assert np.array_equal(e, wo.exp_table()) and np.array_equal(s, wo.silu_table())
+    rng = np.random.default_rng(11)
+    xs = np.concatenate([rng.uniform(0, 400, 2000), rng.uniform(0, 1e-3, 500), rng.uniform(0, 1e-7, 200),
+                         np.array([0.0, 1.0, 65504.0, 2.0 ** -14, 2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -25, 1.00048828125, 1.00146484375])])
+    want = wo.to_float16(xs)
+    for x, w in zip(xs.tolist(), want.tolist()):
+        assert host.to_float16(x) == w, x
+        assert host.to_float16(-x) == -w
