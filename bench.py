@@ -96,9 +96,10 @@ def layer_workload(args):
     FFN 11008, seq_len 2048 by default) proved on one GPU with seeded synthetic int16 weights and
     activations: Hyrax commitments of the 7 weight matrices, matmul sumchecks for Q/K/V/O/gate/up/
     down and per-head QK^T / AV, range lookups on every rescaling remainder, mapping lookups for the
-    softmax exponential and SiLU.  Witnesses (exact integer products, quotients, remainders) are
-    produced with torch, as the reference produces its own with a Python model; all proving goes
-    through the C++ host classes.  One step = one whole layer; prints one JSON line."""
+    softmax exponential and SiLU.  Witnesses (exact integer products, quotients, remainders) come
+    from the library's integer kernels (--witness native, default) or from torch (--witness torch),
+    as the reference produces its own with a Python model; all proving goes through the C++ host
+    classes.  One step = one whole layer; prints one JSON line."""
     import torch
     from grape_amd import ops, _host as host
     from gpuutil import rand_fr
@@ -187,6 +188,14 @@ def layer_workload(args):
     def mm(a, b):      # exact: every product sum stays below 2^53
         return torch.matmul(a.to(torch.float64), b.to(torch.float64).transpose(-1, -2)).to(torch.int64)
 
+    native = args.witness == "native"
+
+    def mmr(a, b):
+        """quotient and remainder of a . b^T at scale 2^16: the library's integer kernel, or torch"""
+        if native:
+            return ops.wit_matmul_rescale(a.contiguous(), b.contiguous(), 1 << SH)
+        return rescale(mm(a, b))
+
     # synthetic tables for the two mapping lookups (the reference's own table files are not in its tree)
     exp_low, exp_len = -(1 << 19), 1 << 20
     xs = torch.arange(exp_len, dtype=torch.float64) + exp_low
@@ -206,16 +215,13 @@ def layer_workload(args):
         # attention projections
         proj = {}
         for name in ("q", "k", "v"):
-            y = mm(x, weights[name])
-            proj[name], rem = rescale(y)
+            proj[name], rem = mmr(x, weights[name])
             matmul_proof(x, weights[name], 1, T, D, D, proj[name], rem)
             range_lookup(rem)
         qh = proj["q"].view(T, H, HD).permute(1, 0, 2).contiguous()
         kh = proj["k"].view(T, H, HD).permute(1, 0, 2).contiguous()
         vh = proj["v"].view(T, H, HD).permute(1, 2, 0).contiguous()       # [H][HD][T]
-        sc = mm(qh, kh)                                                    # [H][T][T]
-        sc_q, sc_r = rescale(sc)
-        del sc
+        sc_q, sc_r = mmr(qh, kh)                                           # [H][T][T]
         matmul_proof(qh, kh, H, T, T, HD, sc_q, sc_r)
         range_lookup(sc_r)
         del sc_r
@@ -223,29 +229,27 @@ def layer_workload(args):
         e_out = d_exp_map[(e_in - exp_low).long()]
         mapping_lookup(e_in, e_out, exp_low, exp_len, exp_map)
         del sc_q, e_in
-        av = mm(e_out, vh)                                                 # [H][T][HD]
-        av_q, av_r = rescale(av)
+        av_q, av_r = mmr(e_out, vh)                                        # [H][T][HD]
         matmul_proof(e_out, vh, H, T, HD, T, av_q, av_r)
         range_lookup(av_r)
         del e_out
         attn = av_q.permute(1, 0, 2).contiguous().view(T, D)
-        y = mm(attn, weights["o"])
-        o_q, o_r = rescale(y)
+        o_q, o_r = mmr(attn, weights["o"])
         matmul_proof(attn, weights["o"], 1, T, D, D, o_q, o_r)
         range_lookup(o_r)
         # feed-forward
         x2 = o_q
-        gq, gr = rescale(mm(x2, weights["gate"]))
+        gq, gr = mmr(x2, weights["gate"])
         matmul_proof(x2, weights["gate"], 1, T, F, D, gq, gr)
         range_lookup(gr)
-        uq, ur = rescale(mm(x2, weights["up"]))
+        uq, ur = mmr(x2, weights["up"])
         matmul_proof(x2, weights["up"], 1, T, F, D, uq, ur)
         range_lookup(ur)
         s_in = gq.clamp(silu_low, silu_low + silu_len - 1)
         s_out = d_silu_map[(s_in - silu_low).long()]
         mapping_lookup(s_in, s_out, silu_low, silu_len, silu_map)
         hq, _ = rescale(s_out.to(torch.int64) * uq.to(torch.int64))
-        dq, dr = rescale(mm(hq, weights["down"]))
+        dq, dr = mmr(hq, weights["down"])
         matmul_proof(hq, weights["down"], 1, T, D, F, dq, dr)
         range_lookup(dr)
         return times["commit_weights"] + times["matmul"] + times["lookup"]
@@ -266,8 +270,9 @@ def layer_workload(args):
                    "breakdown_s": {k: float(v) for k, v in times.items()},
                    "n_matmul_sumchecks": counts["matmul"], "n_lookups": counts["lookup"],
                    "weight_points": weight_points,
+                   "witness": "the library's integer kernels (grape_wit_matmul_rescale)" if native else "torch (float64 products, exact below 2^53)",
                    "note": "time inside the provers (commitments, sumchecks, lookups incl. their commitments of A and m); "
-                           "witness generation with torch is outside"}}))
+                           "witness generation is outside"}}))
     return 0
 
 
@@ -346,6 +351,104 @@ def lookup_workload(args):
     return 0
 
 
+def witness_workload(args):
+    """Witness generation for one LLaMA-2-7B-shape transformer block (d_model 4096, FFN 11008, one
+    attention head as the reference's generator forces, seq_len 2048 by default): the C++
+    LayerWitness class over the integer kernels.  One step = every tensor of the layer (quotients,
+    remainders, softmax and SiLU table rows, RMSNorm parts).  Checks the proved relations on sampled
+    entries, reports the matrix-product kernel against the measured multiply-add issue peak and the
+    numpy oracle's exact integer product on a bounded sample of rows."""
+    import torch
+    from grape_amd import ops, _host as host
+    ops.init(0)
+    host.load()
+    T, D, F = args.seq, 4096, 11008
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4242)
+
+    def gauss(shape, sigma, clip=None):
+        x = (torch.randn(*shape, generator=g, device="cuda", dtype=torch.float32) * sigma).round()
+        if clip:
+            x = x.clamp_(-clip, clip - 1)
+        return x.to(torch.int32)
+
+    x = gauss((T, D), 65536.0)
+    weights = {k: gauss(shape, SIGMA, 32768) for k, shape in (("Q", (D, D)), ("K", (D, D)), ("V", (D, D)), ("O", (D, D)),
+                                                                ("gate", (F, D)), ("up", (F, D)), ("down", (D, F)))}
+    weights["NormFirst"] = torch.full((D,), 65536, dtype=torch.int32, device="cuda")
+    weights["NormSecond"] = torch.full((D,), 65536, dtype=torch.int32, device="cuda")
+    e_np, s_np = host.witness_tables()
+    d_exp, d_silu = torch.from_numpy(e_np).cuda(), torch.from_numpy(s_np).cuda()
+    lw = host.LayerWitness(T, D, F)
+    secs = []
+    for i in range(args.warmup + args.steps):
+        lw.generate(x, weights, d_exp, d_silu)
+        if i >= args.warmup:
+            secs.append(host.last_prove_seconds())
+    t = float(np.mean(secs))
+
+    # the relations the proofs rely on, on sampled entries of the full-size tensors
+    rng = np.random.default_rng(3)
+    S = 1 << 16
+    n1 = lw.tensor("Q/normOutSecond").reshape(T, D).astype(np.int64)
+    gate_w = weights["gate"].cpu().numpy().astype(np.int64)
+    q, r = lw.tensor("Q/gate_out").reshape(T, F).astype(np.int64), lw.tensor("R/gate_out").reshape(T, F).astype(np.int64)
+    for n, m in zip(rng.integers(0, T, 64).tolist(), rng.integers(0, F, 64).tolist()):
+        if q[n, m] * (1 << 20) + r[n, m] != int(np.dot(n1[n], gate_w[m])):
+            print("bench.py: gate projection witness is inconsistent", file=sys.stderr)
+            return 1
+    if r.min() < -(1 << 19) or r.max() >= (1 << 19):
+        print("bench.py: remainder outside its range", file=sys.stderr)
+        return 1
+    out = lw.tensor("Q/output").astype(np.int64)
+    if not np.array_equal(out, lw.tensor("Q/skip").astype(np.int64) + lw.tensor("Q/down_out").astype(np.int64)):
+        print("bench.py: skip connection is inconsistent", file=sys.stderr)
+        return 1
+    del q, r, n1, out
+
+    # dominant kernel: the gate/up projection's matrix product (T x 11008 x 4096), HIP events inside the library
+    h2 = torch.from_numpy(lw.tensor("Q/normOutSecond").reshape(T, D)).cuda()
+    ops.profile_enable(True)
+    ms = []
+    for _ in range(6):
+        ops.wit_matmul_rescale(h2, weights["gate"], 1 << 20)
+        ms.append(ops.profile_last()[0])
+    ops.profile_enable(False)
+    kern_ms = float(np.median(ms[1:]))
+    mads = float(T) * D * F
+    peak = ops.bench_mad(16384, 512, 5)
+    layer_mads = float(T) * D * (4 * D + 3 * F) + 2.0 * T * T * D
+    roofline = {"bound": "valu_int32_mul", "kernel": "wit_matmul_tiled_kernel (%d x %d x %d)" % (T, F, D),
+                "achieved": mads / (kern_ms * 1e-3) / 1e12, "peak": peak / 1e12, "unit": "Tmul/s",
+                "frac": mads / (kern_ms * 1e-3) / peak, "traffic": None, "kernel_ms": kern_ms,
+                "peak_source": "v_mad_u64_u32 issue-rate microbenchmark measured in this run",
+                "layer_multiplies": layer_mads, "layer_frac": layer_mads / t / peak}
+    result = {
+        "metric": "layer_witness_time", "value": t, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int64",
+        "data": "synthetic",
+        "config": {"workload": "witness of one transformer block in the reference generator's fixed-point rules: seq_len %d, "
+                               "d_model 4096, FFN 11008, one head; %d named int32 tensors" % (T, len(lw.names())),
+                   "tensors": len(lw.names())},
+        "roofline": roofline}
+    if not args.no_cpu_baseline:
+        from oracle import witness_oracle as wo
+        rows = 512
+        a = lw.tensor("Q/normOutSecond").reshape(T, D)[:rows]
+        t0 = time.perf_counter()
+        wq, wr = wo.rescale(wo.matmul_t(a, gate_w), 1 << 20)
+        dt = time.perf_counter() - t0
+        if not np.array_equal(wq, lw.tensor("Q/gate_out").reshape(T, F)[:rows]):
+            print("bench.py: GPU and oracle quotients differ", file=sys.stderr)
+            return 1
+        result["cpu_baseline"] = {"value": rows * D * F / dt / 1e9, "unit": "Gmul/s", "cores": 1, "kind": "port",
+                                  "sample": "first %d of %d rows of the gate projection (exact int64 numpy product), %.1f s" % (rows, T, dt),
+                                  "gpu_same_unit": mads / (kern_ms * 1e-3) / 1e9}
+    lw.close()
+    print(json.dumps(result))
+    return 0
+
+
 def _fr_const(x):
     """Montgomery limbs of a small constant, as a (1, 4) uint64 array"""
     r = (21888242871839275222246405745257275088548364400416034343698204186575808495617 if CURVE == "bn254"
@@ -360,15 +463,21 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup"], default="commit",
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "witness"], default="commit",
                     help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
-                         "lookup: configs[3]; layer: configs[4]")
-    ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer workload")
+                         "lookup: configs[3]; layer: configs[4]; witness: the layer's witness generator")
+    ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer and witness workloads")
+    ap.add_argument("--witness", choices=["torch", "native"], default="native",
+                    help="layer workload: who computes quotients and remainders of the matrix products")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
         return 2
+    if args.workload == "witness":
+        args.steps = 3 if args.steps is None else args.steps
+        args.warmup = 1 if args.warmup is None else args.warmup
+        return witness_workload(args)
     if args.workload in ("matmul", "lookup"):
         args.steps = 5 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup

@@ -105,19 +105,20 @@ __global__ void __launch_bounds__(256, 2) wit_matmul_tiled_kernel(MatmulArgs p) 
         if (k0 + kTK < p.K) fetch(k0 + kTK);
 #pragma unroll 1
         for (int kk = 0; kk < kTK; kk += 4) {
-            int4 fa[8];
+            int32_t fa[8][4];
 #pragma unroll
-            for (int i = 0; i < 8; i++) fa[i] = *reinterpret_cast<const int4*>(&As[(ty + 16 * i) * kLd + kk]);
+            for (int i = 0; i < 8; i++) {
+                const int4 v = *reinterpret_cast<const int4*>(&As[(ty + 16 * i) * kLd + kk]);
+                fa[i][0] = v.x; fa[i][1] = v.y; fa[i][2] = v.z; fa[i][3] = v.w;
+            }
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const int4 fb = *reinterpret_cast<const int4*>(&Bs[(tx + 16 * j) * kLd + kk]);
+                const int4 v = *reinterpret_cast<const int4*>(&Bs[(tx + 16 * j) * kLd + kk]);
+                const int32_t fb[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    acc[i][j] += (int64_t)fa[i].x * (int64_t)fb.x;
-                    acc[i][j] += (int64_t)fa[i].y * (int64_t)fb.y;
-                    acc[i][j] += (int64_t)fa[i].z * (int64_t)fb.z;
-                    acc[i][j] += (int64_t)fa[i].w * (int64_t)fb.w;
-                }
+                for (int c = 0; c < 4; c++)
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[i][j] += (int64_t)fa[i][c] * (int64_t)fb[c];
             }
         }
     }
