@@ -78,6 +78,7 @@ SIGNATURES = {
     "grape_g1_affine_to_jacobian": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_g1_jacobian_to_affine": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_wit_matmul_rescale": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_u32, c_u32, ctypes.c_int64, c_int, c_void_p],
+    "grape_wit_set_matmul_method": [c_int],
     "grape_wit_elemul_rescale": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, ctypes.c_int64, c_void_p],
     "grape_wit_table_lookup": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p, c_void_p],
     "grape_wit_add_i32": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],

@@ -43,7 +43,7 @@ static inline unsigned blocks_for(size_t n, int per_block = kBlock) {
 
 // Scratch pool: one growing device allocation per slot, reused across calls so the hot path
 // never allocates.  Slots are independent buffers (a call may use several at once).
-enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kNumSlots = 8 };
+enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kSlotWitA = 8, kSlotWitB = 9, kNumSlots = 10 };
 int scratch_get(ScratchSlot slot, size_t bytes, void** out);
 bool initialised();
 

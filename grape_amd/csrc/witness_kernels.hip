@@ -165,6 +165,193 @@ __global__ void __launch_bounds__(kBlock) wit_matmul_simple_kernel(MatmulArgs p,
     if (bad) atomicOr(p.status, bad);
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same product on the matrix cores.  An int32 operand is split into P planes of signed bytes
+// (balanced radix-256 digits, x = sum_p d_p 256^p, d_p in [-128, 127]); the product is the sum over
+// plane pairs of int8 x int8 -> int32 matrix products (v_mfma_i32_32x32x32_i8), and pairs with the
+// same p + q share an accumulator.  All of it is exact: a digit product is at most 2^14 and a
+// group absorbs at most min(PA, PB) * K of them, kept below 2^31 by the host.  The groups are
+// recombined as 64-bit integers in the epilogue and rescaled like in the kernel above.
+//
+// Workgroup tile 64 (rows of a) x 128 (rows of b), K step 64 bytes; four waves, each 32 x 64 (two
+// MFMA tiles); LDS rows are padded to 80 bytes so that 16 consecutive rows' 16-byte fragments
+// fall in disjoint banks; the next K step travels through registers while this one multiplies.
+// ------------------------------------------------------------------------------------------------
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+constexpr int kMfTN = 64, kMfTM = 128, kMfK = 64, kMfLd = 80;
+
+__global__ void __launch_bounds__(kBlock) wit_maxabs_kernel(uint32_t* out, const int32_t* x, size_t n) {
+    uint32_t m = 0;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const int32_t v = x[i];
+        const uint32_t a = v < 0 ? 0u - (uint32_t)v : (uint32_t)v;
+        m = a > m ? a : m;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t o = __shfl_xor(m, off, 64);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
+}
+
+// planes[p][row][k] for k < Kp (zero beyond K); one thread per 4 consecutive k
+__global__ void __launch_bounds__(kBlock) wit_split_kernel(int8_t* planes, const int32_t* x, uint32_t R, uint32_t K, uint32_t Kp, int P) {
+    const size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t per_row = Kp / 4;
+    if (idx >= (size_t)R * per_row) return;
+    const uint32_t row = (uint32_t)(idx / per_row), k = 4u * (uint32_t)(idx - (size_t)row * per_row);
+    int32_t v[4] = {0, 0, 0, 0};
+    if (k < K) {      // K is a multiple of 4
+        const int4 t = *reinterpret_cast<const int4*>(x + (size_t)row * K + k);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    for (int p = 0; p < P; p++) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int32_t d = (int32_t)(int8_t)(v[j] & 0xff);
+            // (v - d) is a multiple of 256; the subtraction cannot wrap (|d| <= 128 towards zero)
+            v[j] = (int32_t)(((int64_t)v[j] - d) >> 8);
+            w |= ((uint32_t)d & 0xffu) << (8 * j);
+        }
+        *reinterpret_cast<uint32_t*>(planes + ((size_t)p * R + row) * Kp + k) = w;
+    }
+}
+
+struct MfmaArgs {
+    int32_t* q;
+    int32_t* r;
+    const int8_t* a;     // [PA][N][Kp]
+    const int8_t* b;     // [PB][M][Kp]
+    uint32_t N, M, Kp;
+    int64_t scale;
+    int shift, transpose_out;
+    uint32_t tiles_m;
+    uint32_t* status;
+};
+
+template <int PA, int PB>
+__global__ void __launch_bounds__(256, 2) wit_matmul_mfma_kernel(MfmaArgs p) {
+    constexpr int G = PA + PB - 1;
+    __shared__ __attribute__((aligned(16))) int8_t As[PA * kMfTN * kMfLd];
+    __shared__ __attribute__((aligned(16))) int8_t Bs[PB * kMfTM * kMfLd];
+    uint32_t bid = blockIdx.x;
+    const uint32_t nb = gridDim.x;
+    if ((nb & 7u) == 0) bid = (bid & 7u) * (nb >> 3) + (bid >> 3);
+    const uint32_t tn = bid / p.tiles_m, tm = bid - tn * p.tiles_m;
+    const uint32_t n0 = tn * kMfTN, m0 = tm * kMfTM;
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+    const uint32_t wn = (wave & 1u) * 32u, wm = (wave >> 1) * 64u;
+
+    // staging: 16-byte chunks; a: row t/4, chunk t%4 of every plane; b: rows (t + 256 h)/4, h = 0, 1
+    // named registers (planes beyond PA / PB are never touched)
+    uint4 sa0, sa1, sa2 = make_uint4(0, 0, 0, 0), sb00, sb01, sb10, sb11, sb20 = make_uint4(0, 0, 0, 0), sb21 = make_uint4(0, 0, 0, 0);
+    const uint32_t ra = (n0 + (t >> 2) < p.N) ? n0 + (t >> 2) : p.N - 1;
+    const uint32_t rb0 = (m0 + (t >> 2) < p.M) ? m0 + (t >> 2) : p.M - 1;
+    const uint32_t rb1 = (m0 + 64u + (t >> 2) < p.M) ? m0 + 64u + (t >> 2) : p.M - 1;
+    const uint32_t ck = 16u * (t & 3u);
+    const int8_t* ga = p.a + (size_t)ra * p.Kp + ck;
+    const int8_t* gb0 = p.b + (size_t)rb0 * p.Kp + ck;
+    const int8_t* gb1 = p.b + (size_t)rb1 * p.Kp + ck;
+    const size_t pla = (size_t)p.N * p.Kp, plb = (size_t)p.M * p.Kp;     // plane strides
+    v16i_t acc[G][2];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[g][tt][i] = 0;
+
+    const uint32_t frow = lane & 31u, fk = 16u * (lane >> 5);
+#define WIT_LD16(ptr) (*reinterpret_cast<const uint4*>(ptr))
+#define WIT_ST16(arr, row, v) (*reinterpret_cast<uint4*>(&arr[(row) * kMfLd + ck]) = (v))
+    sa0 = WIT_LD16(ga);
+    sa1 = WIT_LD16(ga + pla);
+    if (PA > 2) sa2 = WIT_LD16(ga + 2 * pla);
+    sb00 = WIT_LD16(gb0);
+    sb01 = WIT_LD16(gb1);
+    sb10 = WIT_LD16(gb0 + plb);
+    sb11 = WIT_LD16(gb1 + plb);
+    if (PB > 2) {
+        sb20 = WIT_LD16(gb0 + 2 * plb);
+        sb21 = WIT_LD16(gb1 + 2 * plb);
+    }
+    const uint32_t lr = t >> 2;
+    for (uint32_t k0 = 0; k0 < p.Kp; k0 += kMfK) {
+        __syncthreads();
+        WIT_ST16(As, lr, sa0);
+        WIT_ST16(As, kMfTN + lr, sa1);
+        if (PA > 2) WIT_ST16(As, 2 * kMfTN + lr, sa2);
+        WIT_ST16(Bs, lr, sb00);
+        WIT_ST16(Bs, 64 + lr, sb01);
+        WIT_ST16(Bs, kMfTM + lr, sb10);
+        WIT_ST16(Bs, kMfTM + 64 + lr, sb11);
+        if (PB > 2) {
+            WIT_ST16(Bs, 2 * kMfTM + lr, sb20);
+            WIT_ST16(Bs, 2 * kMfTM + 64 + lr, sb21);
+        }
+        __syncthreads();
+        if (k0 + kMfK < p.Kp) {
+            const uint32_t kn = k0 + kMfK;
+            sa0 = WIT_LD16(ga + kn);
+            sa1 = WIT_LD16(ga + pla + kn);
+            if (PA > 2) sa2 = WIT_LD16(ga + 2 * pla + kn);
+            sb00 = WIT_LD16(gb0 + kn);
+            sb01 = WIT_LD16(gb1 + kn);
+            sb10 = WIT_LD16(gb0 + plb + kn);
+            sb11 = WIT_LD16(gb1 + plb + kn);
+            if (PB > 2) {
+                sb20 = WIT_LD16(gb0 + 2 * plb + kn);
+                sb21 = WIT_LD16(gb1 + 2 * plb + kn);
+            }
+        }
+#pragma unroll
+        for (int kk = 0; kk < kMfK; kk += 32) {
+            v4i_t fa[PA], fb[PB][2];
+#pragma unroll
+            for (int pa = 0; pa < PA; pa++) fa[pa] = *reinterpret_cast<const v4i_t*>(&As[(pa * kMfTN + wn + frow) * kMfLd + kk + fk]);
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+                    fb[pb][tt] = *reinterpret_cast<const v4i_t*>(&Bs[(pb * kMfTM + wm + 32 * tt + frow) * kMfLd + kk + fk]);
+#pragma unroll
+            for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                    for (int tt = 0; tt < 2; tt++)
+                        acc[pa + pb][tt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[pa], fb[pb][tt], acc[pa + pb][tt], 0, 0, 0);
+        }
+    }
+
+#undef WIT_LD16
+#undef WIT_ST16
+    // accumulator register i of lane l holds row 8 (i / 4) + 4 (l / 32) + i % 4, column l % 32
+    uint32_t bad = 0;
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) {
+        const uint32_t m = m0 + wm + 32 * tt + (lane & 31u);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t n = n0 + wn + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
+            int64_t y = 0;
+#pragma unroll
+            for (int g = G - 1; g >= 0; g--) y = y * 256 + (int64_t)acc[g][tt][i];
+            if (n < p.N && m < p.M) {
+                int32_t q, r;
+                rescale64(y, p.scale, p.shift, q, r, bad);
+                const size_t o = p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m;
+                p.q[o] = q;
+                if (p.r) p.r[o] = r;
+            }
+        }
+    }
+    if (bad) atomicOr(p.status, bad);
+}
+
 __global__ void __launch_bounds__(kBlock) wit_elemul_rescale_kernel(int32_t* q, int32_t* r, const int32_t* a, const int32_t* b, size_t n,
                                                                     int64_t scale, int shift, uint32_t* status) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -322,6 +509,17 @@ static int status_word(uint32_t** out, hipStream_t s) {
     return GRAPE_OK;
 }
 
+static int g_matmul_method = 0;   // 0 = choose, 1 = multiply-add kernels only, 2 = matrix cores or fail
+
+// signed byte planes needed for magnitudes up to maxabs (one spare bit keeps the top digit small)
+static int planes_for(uint32_t maxabs) {
+    if (maxabs < (1u << 6)) return 1;
+    if (maxabs < (1u << 14)) return 2;
+    if (maxabs < (1u << 22)) return 3;
+    if (maxabs < (1u << 30)) return 4;
+    return 5;
+}
+
 static int log2_exact(int64_t s) {
     if (s <= 0 || (s & (s - 1)) != 0) return -1;
     int sh = 0;
@@ -358,11 +556,58 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
     int rc = status_word(&p.status, s);
     if (rc) return rc;
     const bool aligned = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_a) | reinterpret_cast<uintptr_t>(d_b)) & 15) == 0;
+    // matrix-core path: one batch, aligned rows, operands of at most three byte planes each
+    bool use_mfma = false;
+    int PA = 0, PB = 0;
+    const uint32_t Kp = (K + kMfK - 1) / kMfK * kMfK;
+    if (g_matmul_method != 1 && L == 1 && aligned && (g_matmul_method == 2 || (uint64_t)N * M * K >= ((uint64_t)1 << 26))) {
+        void* mx;
+        rc = scratch_get(kSlotMisc, 64, &mx);
+        if (rc) return rc;
+        uint32_t* d_mx = (uint32_t*)mx;
+        wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx);
+        wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx + 1);
+        const size_t na = (size_t)N * K, nbb = (size_t)M * K;
+        wit_maxabs_kernel<<<(unsigned)((na + kBlock * 16 - 1) / (kBlock * 16) < 2048 ? (na + kBlock * 16 - 1) / (kBlock * 16) : 2048), kBlock, 0, s>>>(d_mx, d_a, na);
+        wit_maxabs_kernel<<<(unsigned)((nbb + kBlock * 16 - 1) / (kBlock * 16) < 2048 ? (nbb + kBlock * 16 - 1) / (kBlock * 16) : 2048), kBlock, 0, s>>>(d_mx + 1, d_b, nbb);
+        GRAPE_LAUNCH_CHECK();
+        uint32_t h_mx[2] = {0, 0};
+        GRAPE_HIP_CHECK(hipMemcpyAsync(h_mx, d_mx, sizeof(h_mx), hipMemcpyDeviceToHost, s));
+        GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+        PA = planes_for(h_mx[0]);
+        PB = planes_for(h_mx[1]);
+        if (PA < 2) PA = 2;
+        if (PB < 2) PB = 2;
+        const int pmin = PA < PB ? PA : PB;
+        use_mfma = PA <= 3 && PB <= 3 && (uint64_t)Kp * pmin < 131072;   // a group stays below 2^31
+    }
+    GRAPE_REQUIRE(!(g_matmul_method == 2 && !use_mfma), "the matrix-core path needs one batch, K a multiple of 4, 16-byte aligned rows and operands below 2^22");
     if (profiling()) {
         profile_begin();
         profile_mark(s);
     }
-    if (aligned && L <= 65535) {
+    if (use_mfma) {
+        void *pa, *pb;
+        rc = scratch_get(kSlotWitA, (size_t)PA * N * Kp, &pa);
+        if (rc) return rc;
+        rc = scratch_get(kSlotWitB, (size_t)PB * M * Kp, &pb);
+        if (rc) return rc;
+        wit_split_kernel<<<blocks_for((size_t)N * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pa, d_a, N, K, Kp, PA);
+        wit_split_kernel<<<blocks_for((size_t)M * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pb, d_b, M, K, Kp, PB);
+        GRAPE_LAUNCH_CHECK();
+        if (profiling()) profile_mark(s);
+        MfmaArgs m;
+        m.q = d_q; m.r = d_r; m.a = (const int8_t*)pa; m.b = (const int8_t*)pb;
+        m.N = N; m.M = M; m.Kp = Kp;
+        m.scale = scale; m.shift = p.shift; m.transpose_out = p.transpose_out;
+        m.tiles_m = (M + kMfTM - 1) / kMfTM;
+        m.status = p.status;
+        const unsigned grid = ((N + kMfTN - 1) / kMfTN) * m.tiles_m;
+        if (PA == 2 && PB == 2) wit_matmul_mfma_kernel<2, 2><<<grid, 256, 0, s>>>(m);
+        else if (PA == 3 && PB == 2) wit_matmul_mfma_kernel<3, 2><<<grid, 256, 0, s>>>(m);
+        else if (PA == 2 && PB == 3) wit_matmul_mfma_kernel<2, 3><<<grid, 256, 0, s>>>(m);
+        else wit_matmul_mfma_kernel<3, 3><<<grid, 256, 0, s>>>(m);
+    } else if (aligned && L <= 65535) {
         dim3 grid(p.tiles_n * p.tiles_m, L);
         wit_matmul_tiled_kernel<<<grid, 256, 0, s>>>(p);
     } else {
@@ -370,6 +615,12 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
     }
     GRAPE_LAUNCH_CHECK();
     if (profiling()) profile_mark(s);
+    return GRAPE_OK;
+}
+
+int grape_wit_set_matmul_method(int method) {
+    GRAPE_REQUIRE(method >= 0 && method <= 2, "method must be 0 (choose), 1 (multiply-add kernels) or 2 (matrix cores)");
+    g_matmul_method = method;
     return GRAPE_OK;
 }
 

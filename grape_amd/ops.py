@@ -396,6 +396,11 @@ def wit_matmul_rescale(a, b, scale, want_r=True, transpose_out=False):
     return q, r
 
 
+def wit_set_matmul_method(method):
+    """0 = choose, 1 = multiply-add kernels only, 2 = matrix cores (error when not applicable)"""
+    _capi.check(init().grape_wit_set_matmul_method(int(method)))
+
+
 def wit_elemul_rescale(a, b, scale):
     lib = init()
     q, r = torch.empty_like(a), torch.empty_like(a)

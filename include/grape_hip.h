@@ -250,6 +250,13 @@ int grape_g1_jacobian_to_affine(uint32_t *d_out_affine, const uint32_t *d_in_jac
  * rescalings of model.py:485-491, :547-550, :574-583, :646-658, :683-686. */
 int grape_wit_matmul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, const int32_t *d_b, uint32_t L, uint32_t N,
                              uint32_t M, uint32_t K, int64_t scale, int transpose_out, grape_stream_t stream);
+/* Two implementations give the same (exact) result: 64-bit multiply-add kernels for any shape, and,
+ * for one batch of 16-byte aligned operands with K a multiple of 4 and magnitudes below 2^22, int8
+ * matrix-core products of signed byte planes (this path reads the operands' ranges back and so
+ * synchronises the stream).  method 0 = choose (matrix cores from 2^26 multiply-adds), 1 = multiply-add
+ * kernels only, 2 = matrix cores or GRAPE_EINVAL.  With grape_profile_enable, grape_profile_last()
+ * gives [0] the product kernel, or [0] the plane split and [1] the product kernel on the matrix cores. */
+int grape_wit_set_matmul_method(int method);
 /* q, r of a[i] * b[i] (d_r may be NULL).  model.py:673-675. */
 int grape_wit_elemul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, const int32_t *d_b, size_t n, int64_t scale,
                              grape_stream_t stream);

@@ -25,24 +25,72 @@ def host(t):
     return t.cpu().numpy()
 
 
-@pytest.mark.parametrize("L,N,M,K,scale,tr", [
+SHAPES = [
     (1, 8, 64, 64, 1 << 16, False), (1, 8, 176, 64, 1 << 20, False), (1, 8, 64, 176, 1 << 16, False),
     (1, 8, 8, 64, 1 << 22, False), (1, 8, 64, 8, 1 << 16, True), (1, 130, 257, 100, 1 << 16, False),
     (3, 129, 40, 36, 1 << 16, True), (1, 5, 7, 13, 1 << 16, False), (2, 3, 9, 6, 1000, True),
-    (1, 256, 384, 512, 1 << 16, False), (1, 1, 1, 4, 1 << 16, False), (1, 300, 128, 68, 12345, False)])
-def test_matmul_rescale_matches_the_oracle(ops, L, N, M, K, scale, tr):
+    (1, 256, 384, 512, 1 << 16, False), (1, 1, 1, 4, 1 << 16, False), (1, 300, 128, 68, 12345, False)]
+
+
+@pytest.mark.parametrize("method", [1, 2])
+@pytest.mark.parametrize("L,N,M,K,scale,tr", SHAPES)
+def test_matmul_rescale_matches_the_oracle(ops, L, N, M, K, scale, tr, method):
+    """method 1: 64-bit multiply-add kernels; method 2: int8 matrix-core products of byte planes"""
+    if method == 2 and (L != 1 or K % 4):
+        pytest.skip("the matrix-core path takes one batch with K a multiple of 4")
     rng = np.random.default_rng(L * 1000 + N + M + K)
     a = rng.integers(-(1 << 20), 1 << 20, (L, N, K)).astype(np.int32)
     b = rng.integers(-(1 << 17), 1 << 17, (L, M, K)).astype(np.int32)
-    q, r = ops.wit_matmul_rescale(dev(a), dev(b), scale, transpose_out=tr)
+    ops.wit_set_matmul_method(method)
+    try:
+        q, r = ops.wit_matmul_rescale(dev(a), dev(b), scale, transpose_out=tr)
+        q2, r2 = ops.wit_matmul_rescale(dev(a), dev(b), scale, want_r=False, transpose_out=tr)
+    finally:
+        ops.wit_set_matmul_method(0)
     for l in range(L):
         wq, wr = wo.rescale(wo.matmul_t(a[l], b[l]), scale)
         if tr:
             wq, wr = wq.T, wr.T
         assert np.array_equal(host(q)[l], wq) and np.array_equal(host(r)[l], wr)
-    q2, r2 = ops.wit_matmul_rescale(dev(a), dev(b), scale, want_r=False, transpose_out=tr)
     assert r2 is None and torch.equal(q2, q)
     assert ops.wit_status() == 0
+
+
+@pytest.mark.parametrize("amax,bmax", [(50, 50), (1 << 13, 60), (60, 1 << 13), ((1 << 22) - 1, (1 << 14) - 1), ((1 << 14) - 1, (1 << 22) - 1),
+                                       ((1 << 22) - 1, (1 << 22) - 1)])
+def test_matrix_core_path_over_every_plane_count(ops, amax, bmax):
+    """operands at the edges of the 1-, 2- and 3-plane ranges, including the extreme values themselves"""
+    rng = np.random.default_rng(amax % 1000 + bmax % 777)
+    N, M, K = 70, 130, 200
+    a = rng.integers(-amax, amax + 1, (N, K)).astype(np.int32)
+    b = rng.integers(-bmax, bmax + 1, (M, K)).astype(np.int32)
+    a[0, :4] = (amax, -amax, amax, -amax)
+    b[0, :4] = (bmax, -bmax, -bmax, bmax)
+    a[1, :] = amax
+    b[1, :] = -bmax
+    ops.wit_set_matmul_method(2)
+    try:
+        q, r = ops.wit_matmul_rescale(dev(a), dev(b), 1 << 31)
+    finally:
+        ops.wit_set_matmul_method(0)
+    wq, wr = wo.rescale(wo.matmul_t(a, b), 1 << 31)
+    assert np.array_equal(host(q), wq) and np.array_equal(host(r), wr)
+    assert ops.wit_status() == 0
+
+
+def test_matrix_core_path_refuses_what_it_cannot_do(ops):
+    from grape_amd import _capi
+    a = np.full((8, 64), 1 << 22, dtype=np.int32)      # four byte planes
+    b = np.ones((8, 64), dtype=np.int32)
+    ops.wit_set_matmul_method(2)
+    try:
+        with pytest.raises(_capi.GrapeError):
+            ops.wit_matmul_rescale(dev(a), dev(b), 1 << 16)
+    finally:
+        ops.wit_set_matmul_method(0)
+    q, r = ops.wit_matmul_rescale(dev(a), dev(b), 1 << 16)      # the chooser falls back to the multiply-add kernel
+    assert np.array_equal(host(q).astype(np.int64) * 65536 + host(r), wo.matmul_t(a, b))
+    ops.wit_status()
 
 
 def test_matmul_extreme_entries_stay_exact(ops):
