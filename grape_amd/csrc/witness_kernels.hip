@@ -181,19 +181,40 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
 constexpr int kMfTN = 64, kMfTM = 128, kMfK = 64, kMfLd = 80;
 
+// largest magnitude of n values (n a multiple of 4, 16-byte aligned), folded into *out with an atomic maximum
 __global__ void __launch_bounds__(kBlock) wit_maxabs_kernel(uint32_t* out, const int32_t* x, size_t n) {
+    const int4* x4 = reinterpret_cast<const int4*>(x);
+    const size_t n4 = n / 4;
+    const size_t stride = (size_t)gridDim.x * kBlock;
     uint32_t m = 0;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        const int32_t v = x[i];
-        const uint32_t a = v < 0 ? 0u - (uint32_t)v : (uint32_t)v;
-        m = a > m ? a : m;
+    auto fold = [&](const int4& v) {
+        const int32_t e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t a = e[j] < 0 ? 0u - (uint32_t)e[j] : (uint32_t)e[j];
+            m = a > m ? a : m;
+        }
+    };
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {      // four loads in flight
+        const int4 v0 = x4[i], v1 = x4[i + stride], v2 = x4[i + 2 * stride], v3 = x4[i + 3 * stride];
+        fold(v0); fold(v1); fold(v2); fold(v3);
     }
+    for (; i < n4; i += stride) fold(x4[i]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
         const uint32_t o = __shfl_xor(m, off, 64);
         m = o > m ? o : m;
     }
-    if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
+    // one atomic per workgroup: atomics on one address are served one after the other
+    __shared__ uint32_t sh[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kBlock / 64; w++) m = sh[w] > m ? sh[w] : m;
+        if (m) atomicMax(out, m);
+    }
 }
 
 // planes[p][row][k] for k < Kp (zero beyond K); one thread per 4 consecutive k
@@ -568,8 +589,10 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
         wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx);
         wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx + 1);
         const size_t na = (size_t)N * K, nbb = (size_t)M * K;
-        wit_maxabs_kernel<<<(unsigned)((na + kBlock * 16 - 1) / (kBlock * 16) < 2048 ? (na + kBlock * 16 - 1) / (kBlock * 16) : 2048), kBlock, 0, s>>>(d_mx, d_a, na);
-        wit_maxabs_kernel<<<(unsigned)((nbb + kBlock * 16 - 1) / (kBlock * 16) < 2048 ? (nbb + kBlock * 16 - 1) / (kBlock * 16) : 2048), kBlock, 0, s>>>(d_mx + 1, d_b, nbb);
+        // K is a multiple of 4, so both element counts are; at least 8 vectors of 4 per thread, at most 1024 workgroups
+        const size_t ga_ = (na / 4 + kBlock * 8 - 1) / (kBlock * 8), gb_ = (nbb / 4 + kBlock * 8 - 1) / (kBlock * 8);
+        wit_maxabs_kernel<<<(unsigned)(ga_ < 1024 ? ga_ : 1024), kBlock, 0, s>>>(d_mx, d_a, na);
+        wit_maxabs_kernel<<<(unsigned)(gb_ < 1024 ? gb_ : 1024), kBlock, 0, s>>>(d_mx + 1, d_b, nbb);
         GRAPE_LAUNCH_CHECK();
         uint32_t h_mx[2] = {0, 0};
         GRAPE_HIP_CHECK(hipMemcpyAsync(h_mx, d_mx, sizeof(h_mx), hipMemcpyDeviceToHost, s));
