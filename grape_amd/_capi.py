@@ -113,6 +113,12 @@ def load():
         if not os.path.exists(LIB_PATH):
             raise GrapeError("%s not found: build it with `python -m grape_amd.build` "
                              "(there is no CPU fallback)" % LIB_PATH)
+        # torch ships its own HIP runtime; when both live in one process the kernel library must
+        # bind to the one torch has loaded, or the two runtimes fight over the device
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = ctypes.CDLL(LIB_PATH)
         for name, args in SIGNATURES.items():
             fn = getattr(lib, name)     # AttributeError if a declared symbol is not exported
