@@ -367,3 +367,19 @@ def test_cpp_driver_runs(ops, tmp_path):
     res = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=280)
     assert res.returncode == 0, res.stderr
     assert "driver_flow OK" in res.stdout
+
+
+def test_cpp_layer_driver_runs(ops, tmp_path):
+    """one transformer block (1024 tokens, d_model 4096, FFN 11008) proved in the order of the
+    reference's layer driver (test/llm.cu:73-611) by a C++ program against the host classes, on the
+    witness of the library's own generator: 37 chained steps (openings, range and mapping lookups,
+    matmul / element-product sumchecks, combine_claims), every one of the reference's assertions
+    kept; runs in a child process because it holds tens of GB of tables"""
+    import subprocess
+    import torch
+    import driver_build
+    exe = driver_build.build(None, "layer_flow")
+    torch.cuda.empty_cache()
+    res = subprocess.run([exe, "1024", str(tmp_path)], capture_output=True, text=True, timeout=280)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    assert "layer_flow OK: 37 steps" in res.stdout

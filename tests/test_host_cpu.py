@@ -54,9 +54,10 @@ def test_file_helpers_on_host_memory(tmp_path):
 def test_cpp_driver_compiles_against_the_host_headers():
     """a driver in the reference's style builds with g++ against the host classes alone (no HIP
     headers, no kernels); the GPU suite runs it"""
-    import driver_build
-    exe = driver_build.build()
     import os
+    import driver_build
+    assert os.path.exists(driver_build.build(None, "layer_flow"))
+    exe = driver_build.build()
     assert os.path.exists(exe)
 
 
