@@ -62,6 +62,11 @@ GRAPE_HD uint32_t MCONV(int i) {
                                0x581c8ee6u, 0x9f6e5c10u, 0x8c59c9e8u, 0x07359fa8u};
     return t[i];
 }
+GRAPE_HD int32_t CIN(int i) {   // 2^304 mod p: mul28(pack(x*2^256), CIN) = x*2^280
+    constexpr int32_t t[10] = {0x8b6fea0, 0xa73d9f9, 0x09603cf, 0xb860a8d, 0x8b33888,
+                               0x9628387, 0xb8b8d5d, 0x9a84442, 0xe142fd5, 0x0000000};
+    return t[i];
+}
 
 #else
 struct Fp28 {
@@ -99,6 +104,11 @@ GRAPE_HD int32_t CMEM(int i) {   // 2^384 mod p: mul28(x*2^392, CMEM) = x*2^384
 GRAPE_HD uint32_t MCONV(int i) {
     constexpr uint32_t t[12] = {0x0347fcb8u, 0x19d80000u, 0x6d2002b1u, 0x12e00cdeu, 0xa2090c72u, 0x37669f83u,
                                 0xda0f73e0u, 0x09b09b42u, 0x8f1297bbu, 0xa7c515d9u, 0xfcfa012cu, 0x0577a659u};
+    return t[i];
+}
+GRAPE_HD int32_t CIN(int i) {   // 2^400 mod p: mul28(pack(x*2^384), CIN) = x*2^392
+    constexpr int32_t t[14] = {0x80e6299, 0x3500034, 0xeb12856, 0xdeb2699, 0xc988670, 0x4ef6697, 0x70983e8,
+                               0xa4e6fe9, 0x3e8a053, 0xecf271e, 0xc20d323, 0x6eb6385, 0x47f1286, 0x00156da};
     return t[i];
 }
 
@@ -305,6 +315,14 @@ GRAPE_HD Fp28 from_canonical(const Fp& x) {
 #pragma unroll
     for (int i = 0; i < FW; i++) m.v[i] = MCONV(i);
     return pack(fmul(x, m));
+}
+// the same conversion with the 28-bit multiplier only (a third of the instructions): the result is
+// normalised in (0, 3p) instead of canonical, which every consumer of a product accepts
+GRAPE_HD Fp28 from_canonical_lazy(const Fp& x) {
+    Fp28 c;
+#pragma unroll
+    for (int i = 0; i < N; i++) c.v[i] = CIN(i);
+    return mul(pack(x), c);
 }
 // value in (-9p, 3p), any limb form -> canonical memory form, 32-bit limbs
 GRAPE_HD Fp to_canonical(const Fp28& a) {

@@ -11,6 +11,7 @@
 #define GRAPE_FP_MUL_OUTLINE 1
 #include "common.hpp"
 #include "fp28.hpp"
+#include "fr26.hpp"
 
 namespace grape {
 
@@ -523,46 +524,70 @@ __global__ void __launch_bounds__(64) commit_reduce_kernel(uint32_t* out, const 
 }
 
 // ------------------------------------------------------------------------------------------------
-// commitment through the reference-format table (k*G_i, k < 256): one wave per row, byte windows
-// from the top, 8 doublings between windows.  Compatibility path, not tuned.
+// commitment through the reference-format table (entry k * npoints + i = k * G_i, k < 256, canonical
+// affine points): the reference's algorithm (byte windows, 8 doublings between windows,
+// src/Hyrax.cu:46-167) re-ordered so that it fills the chip whatever the number of rows - one wave
+// per (row, window, column segment) sums its table entries in the 28-bit form, the row-reduction
+// kernel folds the lanes and segments of every (row, window), and a last kernel runs the Horner
+// chain over a row's windows.  A table entry is converted on the fly (one 28-bit product per
+// coordinate); no wide table has to be built, which is what single rows (Hyrax::open's blinding
+// row, single_commit) and rows too long for a wide table need.
 // ------------------------------------------------------------------------------------------------
 template <bool FR>
-__global__ void __launch_bounds__(64) commit_ref_kernel(uint32_t* out, const void* scalars, uint32_t rowlen, size_t rows,
-                                                        const uint32_t* table, size_t npoints) {
-    const int lane = threadIdx.x;
-    const size_t row = blockIdx.x;
-    if (row >= rows) return;
-    const int nwin = FR ? 32 : 4;
-    G1Xyzz total = G1Xyzz::inf();
-    for (int w = nwin - 1; w >= 0; w--) {
-        G1Xyzz acc = G1Xyzz::inf();
-        for (uint32_t col = lane; col < rowlen; col += 64) {
-            uint32_t idx;
-            bool neg = false;
-            if (FR) {
-                const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
-                uint32_t limb = 0;
+__global__ void __launch_bounds__(kBlock, 2) commit_ref28_kernel(uint32_t* partial, const void* scalars, uint32_t rowlen, size_t rows,
+                                                                 uint32_t seg, uint32_t nseg, const uint32_t* table, size_t npoints) {
+    constexpr uint32_t nwin = FR ? 32 : 4;
+    const size_t unit = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;      // one wave per unit
+    const uint32_t lane = threadIdx.x & 63;
+    if (unit >= rows * nwin * nseg) return;
+    const uint32_t sg = (uint32_t)(unit % nseg);
+    const size_t rw = unit / nseg;
+    const uint32_t w = (uint32_t)(rw % nwin);
+    const size_t row = rw / nwin;
+    const uint32_t col_end = (sg + 1) * seg < rowlen ? (sg + 1) * seg : rowlen;
+    Xyzz28 acc = xyzz28_inf();
+    for (uint32_t col = sg * seg + lane; col < col_end; col += 64) {
+        uint32_t idx;
+        bool neg = false;
+        if (FR) {
+            const Fr k = fr26::from_montc(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
+            uint32_t limb = 0;
 #pragma unroll
-                for (int q = 0; q < 8; q++) limb = (q == (w >> 2)) ? k.v[q] : limb;
-                idx = (limb >> (8 * (w & 3))) & 255u;
-            } else {
-                int32_t sv = ((const int32_t*)scalars)[row * rowlen + col];
-                neg = sv < 0;
-                uint32_t a = neg ? (uint32_t)0 - (uint32_t)sv : (uint32_t)sv;
-                idx = (a >> (8 * w)) & 255u;
+            for (int q = 0; q < 8; q++) limb = (q == (int)(w >> 2)) ? k.v[q] : limb;
+            idx = (limb >> (8 * (w & 3))) & 255u;
+        } else {
+            const int32_t sv = ((const int32_t*)scalars)[row * rowlen + col];
+            neg = sv < 0;
+            const uint32_t a = neg ? (uint32_t)0 - (uint32_t)sv : (uint32_t)sv;
+            idx = (a >> (8 * w)) & 255u;
+        }
+        if (idx) {
+            const G1Affine a = ld_affine(table, (size_t)idx * npoints + col);
+            if (!a.is_inf()) {
+                Affine28 e;
+                e.x = fp28::from_canonical_lazy(a.x);      // in (0, 3p): fine for every product it enters
+                e.y = fp28::from_canonical_lazy(a.y);
+                if (!xyzz28_madd(acc, e, neg)) {           // entry = +-accumulator: exact canonical-form addition
+                    G1Xyzz c = xyzz28_to_canonical(acc);
+                    xyzz_add_affine(c, a, neg);
+                    acc = xyzz28_from_canonical(c);
+                }
             }
-            if (idx) madd(acc, ld_affine(table, (size_t)idx * npoints + col), neg);
         }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            G1Xyzz o = shfl_down_xyzz(acc, off);
-            if (lane + off < 64) padd(acc, o);
-        }
-        // lane 0 carries the running Horner value; other lanes follow along harmlessly
-        for (int d = 0; d < 8; d++) pdbl(total);
-        padd(total, acc);
     }
-    if (lane == 0) st_affine(out, row, to_affine(total));
+    st_partial28(partial, unit * 64 + lane, acc);
+}
+
+// total = sum_w 2^(8 w) * sums[row * nwin + w]: one thread per row
+__global__ void __launch_bounds__(64) commit_ref_horner_kernel(uint32_t* out, const uint32_t* sums, size_t rows, uint32_t nwin) {
+    const size_t row = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (row >= rows) return;
+    G1Xyzz total = G1Xyzz::inf();
+    for (int w = (int)nwin - 1; w >= 0; w--) {
+        for (int d = 0; d < 8; d++) pdbl(total);
+        madd(total, ld_affine(sums, row * nwin + w), false);
+    }
+    st_affine(out, row, to_affine(total));
 }
 
 __global__ void __launch_bounds__(64) affine_to_jac_kernel(uint32_t* out, const uint32_t* in, size_t n) {
@@ -629,6 +654,43 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
         set_error("commit: a scalar does not fit the table's digit range (c=%u, nw=%u, K=%u)", c, nw, K);
         return GRAPE_EINVAL;
     }
+    return GRAPE_OK;
+}
+
+template <bool FR>
+static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t npoints,
+                           grape_stream_t st) {
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
+    const size_t rows = size / rowlen;
+    if (rows == 0) return GRAPE_OK;
+    hipStream_t s = as_stream(st);
+    const uint32_t nwin = FR ? 32 : 4;
+    // column segments: enough waves to fill the chip, at least one 64-column sweep each
+    uint32_t nseg = 1;
+    while (rows * nwin * nseg < 8192 && rowlen / (nseg * 2) >= 64) nseg *= 2;
+    const uint32_t seg = (rowlen + nseg - 1) / nseg;
+    // rows go through in slabs so that the per-lane partial sums stay within 512 MiB
+    size_t slab = 32768 / ((size_t)nwin * nseg);
+    if (slab < 1) slab = 1;
+    if (slab > rows) slab = rows;
+    const size_t partial_bytes = slab * nwin * nseg * 64 * (size_t)(4 * kPartialWords);
+    void* ws;
+    int rc = scratch_get(kSlotMsm, partial_bytes + slab * nwin * (size_t)(8 * FW) + 64, &ws);
+    if (rc) return rc;
+    uint32_t* sums = (uint32_t*)((char*)ws + partial_bytes);
+    const size_t elem_words = FR ? 8 : 1;
+    for (size_t r0 = 0; r0 < rows; r0 += slab) {
+        const size_t nr = rows - r0 < slab ? rows - r0 : slab;
+        const size_t units = nr * nwin * nseg;
+        const uint32_t* sc = (const uint32_t*)scalars + r0 * rowlen * elem_words;
+        commit_ref28_kernel<FR><<<blocks_for(units * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, npoints);
+        const uint32_t lg_lpr = 3;
+        const size_t per_wave = (size_t)64 >> lg_lpr, rw = nr * nwin;
+        commit_reduce_kernel<<<(unsigned)((rw + per_wave - 1) / per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rw, nseg * 64, lg_lpr);
+        commit_ref_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, nwin);
+    }
+    GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
 
@@ -741,23 +803,11 @@ int grape_commit_fr(uint32_t* out, const uint32_t* scalars, size_t size, uint32_
 
 int grape_commit_i32_ref_table(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table,
                                size_t npoints, grape_stream_t st) {
-    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
-    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
-    size_t rows = size / rowlen;
-    if (rows == 0) return GRAPE_OK;
-    commit_ref_kernel<false><<<(unsigned)rows, 64, 0, as_stream(st)>>>(out, scalars, rowlen, rows, table, npoints);
-    GRAPE_LAUNCH_CHECK();
-    return GRAPE_OK;
+    return commit_ref_impl<false>(out, scalars, size, rowlen, table, npoints, st);
 }
 int grape_commit_fr_ref_table(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table,
                               size_t npoints, grape_stream_t st) {
-    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
-    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
-    size_t rows = size / rowlen;
-    if (rows == 0) return GRAPE_OK;
-    commit_ref_kernel<true><<<(unsigned)rows, 64, 0, as_stream(st)>>>(out, scalars, rowlen, rows, table, npoints);
-    GRAPE_LAUNCH_CHECK();
-    return GRAPE_OK;
+    return commit_ref_impl<true>(out, scalars, size, rowlen, table, npoints, st);
 }
 
 int grape_g1_affine_to_jacobian(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st) {

@@ -91,17 +91,21 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
 }
 
 // Full-width scalars cost ceil(256/c) additions each, so the widest radix whose table fits the
-// budget is used.  For 4096 generators: c = 14 is 19 additions per element (82 GB, what the
+// budget is used (from c = 10 up).  For 4096 generators: c = 14 is 19 additions per element (82 GB, what the
 // default budget allows next to the other tables), c = 13 is 20 (43 GB), c = 15 is 17.5 on average
 // (155 GB; measured no faster than c = 14, its gathers miss more), against 32 plus a doubling
 // chain for the reference's byte windows.
-bool Hyrax::ensure_fr_table(uint rowlen) {
+bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
+    if (!build) return false;
     size_t used = 0;
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
     if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
-    // ceil(256 / c) windows: the top signed digit of a 255-bit scalar may carry into one more
-    for (uint c = 15; c >= 8; c--) {
+    // ceil(256 / c) windows: the top signed digit of a 255-bit scalar may carry into one more.
+    // Below c = 10 a wide table (32 additions per element at c = 8) saves nothing over the
+    // reference-format table, whose path needs no build, so very long rows (the reference's
+    // com_scale = 16 shapes: 65536 to 262144 columns) stay on that path.
+    for (uint c = 15; c >= 10; c--) {
         uint nw = (256 + c - 1) / c, K = 1u << (c - 1);
         if (used + grape_g1_wide_table_bytes(rowlen, nw, K) <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }
@@ -198,7 +202,8 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185)
     affine_t* com_d_dev = nullptr;
     check(grape_malloc((void**)&com_d_dev, sizeof(affine_t)), "grape_malloc");
-    if (ensure_fr_table(new_N)) {
+    // one row only: a table that is already there is used, none is built for it
+    if (ensure_fr_table(new_N, false)) {
         check(grape_commit_fr(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
                               fr_table_.K, nullptr),
               "grape_commit_fr");

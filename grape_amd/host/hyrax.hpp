@@ -68,7 +68,7 @@ private:
         uint ngen = 0, c = 0, nw = 0, K = 0;
     };
     bool ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K);
-    bool ensure_fr_table(uint rowlen);
+    bool ensure_fr_table(uint rowlen, bool build = true);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;

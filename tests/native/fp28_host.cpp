@@ -21,6 +21,12 @@ void t28_sqr(const uint32_t* a, uint32_t* out) {
     Fp r = fp28::to_canonical(fp28::sqr(fp28::from_canonical(x)));
     memcpy(out, &r, FB);
 }
+void t28_roundtrip_lazy(const uint32_t* a, uint32_t* out) {
+    Fp x;
+    memcpy(&x, a, FB);
+    Fp r = fp28::to_canonical(fp28::from_canonical_lazy(x));
+    memcpy(out, &r, FB);
+}
 void t28_roundtrip(const uint32_t* a, uint32_t* out) {
     Fp x;
     memcpy(&x, a, FB);

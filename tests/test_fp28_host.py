@@ -52,6 +52,8 @@ def test_mul_sqr_roundtrip(lib):
         pa = _p32([a])[0]
         lib.t28_roundtrip(_u32(pa), _u32(out))
         assert _val(out) == a
+        lib.t28_roundtrip_lazy(_u32(pa), _u32(out))
+        assert _val(out) == a
         lib.t28_sqr(_u32(pa), _u32(out))
         assert _val(out) == a * a % P
         for b in vals[:14] + vals[-4:]:

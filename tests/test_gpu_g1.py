@@ -181,3 +181,36 @@ def test_jacobian_conversions(ops, gens64):
     want = np.zeros((64, br.G1_WORDS), dtype=np.uint64)
     orc.lib().orc_g1_jac_to_affine(orc.P(want), orc.P(np.ascontiguousarray(hj)), orc.c64(64))
     assert_same(want, host, "oracle jacobian -> affine")
+
+
+def test_reference_table_path_in_every_launch_shape(ops):
+    """commitments through the reference-format table agree with the wide-table path when a row
+    spans several column segments, when rows are many enough for several slabs, on ragged row
+    lengths, on edge scalars, and with repeated generators (the exceptional additions)"""
+    import torch
+    k = _scalars(512, 303)
+    k[5] = k[4]                                  # two equal generators: entry = accumulator can occur
+    dev = ops.g1_make_generators(k)
+    dtab = ops.g1_table_gen(dev, 256)
+    wide = ops.g1_wide_table_gen(dev, 8, 32, 128)
+    # one long row (segments), a few rows of ragged length, many short rows (slabs)
+    for rows, rowlen in ((1, 512), (3, 200), (1100, 8)):
+        s = rand_fr(rows * rowlen, rows + rowlen)
+        s[0] = 0
+        s[1] = br.fr_pack([br.R_MOD - 1])[0]
+        s[2] = br.fr_pack([1])[0]
+        if rowlen > 5:
+            s[4] = s[5] = br.fr_pack([7])[0]     # 7*G + 7*G on the two equal generators
+        d = ops.to_dev(s)
+        got = ops.g1_to_host(ops.commit_fr_ref_table(d, rowlen, dtab, 512))
+        want = ops.g1_to_host(ops.commit_fr(d, rowlen, wide, 512, 8, 32, 128))
+        assert_same(got, want, "fr ref table %dx%d" % (rows, rowlen))
+    wide_i = ops.g1_wide_table_gen(dev, 8, 5, 128)
+    for rows, rowlen in ((1, 512), (2, 300), (9000, 4)):
+        rng = np.random.default_rng(rows)
+        v = rng.integers(-2**31, 2**31, size=(rows, rowlen), dtype=np.int64).astype(np.int32)
+        v[0, :4] = [-2**31, 2**31 - 1, 0, -1]
+        d = torch.from_numpy(v).cuda()
+        got = ops.g1_to_host(ops.commit_i32_ref_table(d, rowlen, dtab, 512))
+        want = ops.g1_to_host(ops.commit_i32(d, rowlen, wide_i, 512, 8, 5, 128))
+        assert_same(got, want, "i32 ref table %dx%d" % (rows, rowlen))
