@@ -615,6 +615,17 @@ using namespace grape;
 
 #define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")
 
+// Lanes that share a row in the row-reduction kernel: 8 when rows alone fill the chip (measured best
+// for 4096 rows of 64 partials: 4 lanes +6 %, 16 +33 %, 32 +65 % - idle lanes of the tree steps cost
+// more than shorter chains save), up to a whole wave when rows are few and the chain per lane is
+// what takes the time (one row of 32768 partials: 150 ms with 8 lanes).
+static uint32_t reduce_lanes_log2(size_t rows) {
+    if (rows >= 2048) return 3;
+    if (rows >= 1024) return 4;
+    if (rows >= 512) return 5;
+    return 6;
+}
+
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                             uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
@@ -626,9 +637,11 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     const size_t rows = size / rowlen;
     if (rows == 0) return GRAPE_OK;
     hipStream_t s = as_stream(st);
-    // segments: enough waves to fill the chip (>= 4 per SIMD) but at least 64 columns per lane-sweep
+    // segments: enough waves to fill the chip (>= 4 per SIMD) but at least 64 columns per lane-sweep,
+    // and no more than leaves each reducing lane a chain of 128 partial sums
+    const uint32_t lg_lpr = reduce_lanes_log2(rows);
     uint32_t nseg = 1;
-    while (rows * nseg < 4096 && rowlen / (nseg * 2) >= 64) nseg *= 2;
+    while (rows * nseg < 4096 && rowlen / (nseg * 2) >= 64 && nseg * 2 <= (2u << lg_lpr)) nseg *= 2;
     const uint32_t seg = (rowlen + nseg - 1) / nseg;
     const size_t nwaves = rows * nseg;
     void* ws;
@@ -640,9 +653,6 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     profile_mark(s);
     commit_wide_kernel<FR><<<blocks_for(nwaves * 64), kBlock, 0, s>>>((uint32_t*)ws, scalars, rowlen, rows, seg, nseg, table, N, c, nw, K, err);
     profile_mark(s);
-    // 8 lanes per row: measured best for 4096 rows of 64 partials (4 lanes: +6 %, 16: +33 %,
-    // 32: +65 % - the idle lanes of the tree steps cost more than the shorter chains save)
-    const uint32_t lg_lpr = 3;
     const size_t rows_per_wave = (size_t)64 >> lg_lpr;
     commit_reduce_kernel<<<(unsigned)((rows + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out, (const uint32_t*)ws, rows, nseg * 64, lg_lpr);
     profile_mark(s);
@@ -666,9 +676,11 @@ static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint
     if (rows == 0) return GRAPE_OK;
     hipStream_t s = as_stream(st);
     const uint32_t nwin = FR ? 32 : 4;
-    // column segments: enough waves to fill the chip, at least one 64-column sweep each
+    // column segments: enough waves to fill the chip, at least one 64-column sweep each, and chains
+    // of at most 128 partial sums per reducing lane
+    const uint32_t lg_lpr = reduce_lanes_log2(rows * nwin);
     uint32_t nseg = 1;
-    while (rows * nwin * nseg < 8192 && rowlen / (nseg * 2) >= 64) nseg *= 2;
+    while (rows * nwin * nseg < 8192 && rowlen / (nseg * 2) >= 64 && nseg * 2 <= (2u << lg_lpr)) nseg *= 2;
     const uint32_t seg = (rowlen + nseg - 1) / nseg;
     // rows go through in slabs so that the per-lane partial sums stay within 512 MiB
     size_t slab = 32768 / ((size_t)nwin * nseg);
@@ -685,7 +697,6 @@ static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint
         const size_t units = nr * nwin * nseg;
         const uint32_t* sc = (const uint32_t*)scalars + r0 * rowlen * elem_words;
         commit_ref28_kernel<FR><<<blocks_for(units * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, npoints);
-        const uint32_t lg_lpr = 3;
         const size_t per_wave = (size_t)64 >> lg_lpr, rw = nr * nwin;
         commit_reduce_kernel<<<(unsigned)((rw + per_wave - 1) / per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rw, nseg * 64, lg_lpr);
         commit_ref_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, nwin);
