@@ -41,6 +41,7 @@ Hyrax::Hyrax(uint layer_num_, uint npoints_, affine_t* g, bn128& G_, uint com_sc
 }
 Hyrax::~Hyrax() {
     grape_free(int16_table_.d);
+    grape_free(int16x2_table_.d);
     grape_free(int32_table_.d);
     grape_free(fr_table_.d);
 }
@@ -75,12 +76,19 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
     const uint rows = size / rowlen;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
-    // small-scalar fast path: one signed 16-bit digit per scalar, one mixed addition per element
-    if (int16_ok_ && ensure_table(int16_table_, rowlen, 16, 1, 32768)) {
-        int rc = grape_commit_i32(W(out), tensor, size, rowlen, W(int16_table_.d), int16_table_.ngen, 16, 1, 32768, nullptr);
-        if (rc == GRAPE_OK) return out;
-        if (rc != GRAPE_EINVAL) check(rc, "grape_commit_i32");
-        int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
+    // small-scalar fast paths: one signed 16-bit digit per scalar (one mixed addition per element)
+    // when that table fits the budget, else two signed 9-bit digits (two additions; 17 GB instead of
+    // 275 GB for the 262144-column rows of the reference's com_scale = 16 shapes)
+    if (int16_ok_) {
+        WideTable* t = nullptr;
+        if (ensure_table(int16_table_, rowlen, 16, 1, 32768)) t = &int16_table_;
+        else if (ensure_table(int16x2_table_, rowlen, 9, 2, 256)) t = &int16x2_table_;
+        if (t) {
+            int rc = grape_commit_i32(W(out), tensor, size, rowlen, W(t->d), t->ngen, t->c, t->nw, t->K, nullptr);
+            if (rc == GRAPE_OK) return out;
+            if (rc != GRAPE_EINVAL) check(rc, "grape_commit_i32");
+            int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
+        }
     }
     if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
         check(grape_commit_i32(W(out), tensor, size, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr), "grape_commit_i32");
@@ -100,6 +108,7 @@ bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (!build) return false;
     size_t used = 0;
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
+    if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);
     if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
     // ceil(256 / c) windows: the top signed digit of a 255-bit scalar may carry into one more.
     // Below c = 10 a wide table (32 additions per element at c = 8) saves nothing over the
@@ -134,6 +143,7 @@ affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
     size_t bytes = (size_t)scalars.size * ncols * 128;
     size_t used = scaled_bytes_ + grape_g1_wide_table_bytes(fr_table_.ngen, fr_table_.nw, fr_table_.K);
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
+    if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);
     if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
     if (used + bytes > table_budget_) return nullptr;
     affine_t* out = nullptr;

@@ -70,7 +70,7 @@ private:
     bool ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K);
     bool ensure_fr_table(uint rowlen, bool build = true);
     void check_shape(uint size, uint N) const;
-    WideTable int16_table_, int32_table_, fr_table_;
+    WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;
     size_t scaled_bytes_ = 0;
     size_t table_budget_ = (size_t)128 << 30;

@@ -50,6 +50,29 @@ int main(int argc, char** argv) {
         require(grape_memcpy_d2h(h_fr.data(), com_fr, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
         for (uint i = 0; i < rows; i++) require(h_int[i] == h_fr[i], "int path and Fr path commit to different points");
 
+        // ---- the same under a table budget that leaves only the small tables: int16 values go through
+        // the two-digit table, field elements through the reference-format table; same commitments
+        {
+            std::vector<int> small(size);
+            for (uint i = 0; i < size; i++) small[i] = (int)((i * 2654435761u) >> 16) % 65536 - 32768;
+            small[0] = -32768; small[1] = 32767; small[2] = 0;
+            int* d_small = nullptr;
+            require(grape_malloc((void**)&d_small, sizeof(int) * size) == 0, "grape_malloc");
+            require(grape_memcpy_h2d(d_small, small.data(), sizeof(int) * size, nullptr) == 0, "h2d");
+            Hyrax tight(layer_num, npoints / com_scale, points, cpu_points[0]);
+            tight.set_table_budget((size_t)8 << 20);        // 8 MiB: 2 * 256 * 64 entries of 128 bytes fit, 32768 * 64 do not
+            FrTensor fr_small(size, d_small);
+            jacob_t* c1 = tight.commit(d_small, size, N);
+            jacob_t* c2 = tight.commit(fr_small, size, N);
+            jacob_t* c3 = hyrax.commit(d_small, size, N);
+            std::vector<bn128> h1(rows), h2(rows), h3(rows);
+            require(grape_memcpy_d2h(h1.data(), c1, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
+            require(grape_memcpy_d2h(h2.data(), c2, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
+            require(grape_memcpy_d2h(h3.data(), c3, sizeof(jacob_t) * rows, nullptr) == 0, "d2h");
+            for (uint i = 0; i < rows; i++) require(h1[i] == h2[i] && h1[i] == h3[i], "commitments differ between table choices");
+            grape_free(c1); grape_free(c2); grape_free(c3); grape_free(d_small);
+        }
+
         // ---- open at a random point, verify, and compare with the multilinear extension (test/HyraxTest.cu:76-125)
         std::vector<Fr> eval_point = random_vec(Log2(size));
         Fr c = Fr::random_element();
