@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Benchmark of the headline metric: Hyrax row commitment of a quantised weight matrix
-(BASELINE.json configs[1]) on one MI355X.
+(benchmark configuration configs[1]) on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
@@ -92,7 +92,7 @@ def cpu_baseline(W, gens_dev, ops, budget_s=15.0):
 
 
 def layer_workload(args):
-    """BASELINE.json configs[4]: one LLaMA-2-7B-shape decoder layer (d_model 4096, 32 heads of 128,
+    """Benchmark configuration configs[4]: one LLaMA-2-7B-shape decoder layer (d_model 4096, 32 heads of 128,
     FFN 11008, seq_len 2048 by default) proved on one GPU with seeded synthetic int16 weights and
     activations: Hyrax commitments of the 7 weight matrices, matmul sumchecks for Q/K/V/O/gate/up/
     down and per-head QK^T / AV, range lookups on every rescaling remainder, mapping lookups for the
@@ -277,7 +277,7 @@ def layer_workload(args):
 
 
 def matmul_workload(args):
-    """BASELINE.json configs[2]: prove_matmul of a 2048 x 4096 activation by a 4096 x 4096 weight
+    """Benchmark configuration configs[2]: prove_matmul of a 2048 x 4096 activation by a 4096 x 4096 weight
     (both int16-range, seeded), 12 sumcheck rounds over k after folding the row variables of both
     operands.  One step = one proof; the claim and the final evaluations are checked against
     independent multilinear evaluations on the GPU."""
@@ -317,7 +317,7 @@ def matmul_workload(args):
 
 
 def lookup_workload(args):
-    """BASELINE.json configs[3]: tLookupRange proof of 2^24 values in a 2^16-entry range with its
+    """Benchmark configuration configs[3]: tLookupRange proof of 2^24 values in a 2^16-entry range with its
     commitments of A and m (4096 generators).  One step = one proof."""
     import torch
     from grape_amd import ops, _host as host
