@@ -45,6 +45,9 @@ static inline unsigned blocks_for(size_t n, int per_block = kBlock) {
 // never allocates.  Slots are independent buffers (a call may use several at once).
 enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kSlotWitA = 8, kSlotWitB = 9, kNumSlots = 10 };
 int scratch_get(ScratchSlot slot, size_t bytes, void** out);
+// Zeroes device memory with a small fill kernel (word-sized regions) so that a caller who captures
+// the stream into a graph records a kernel node, not a memset node.
+int zero_fill(void* d_ptr, size_t bytes, hipStream_t s);
 bool initialised();
 
 // Optional per-kernel event timing (see grape_profile_enable).

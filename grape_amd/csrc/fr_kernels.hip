@@ -473,8 +473,7 @@ int grape_fr_sum(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st)
     CHECK_PTR16(out);
     hipStream_t s = as_stream(st);
     if (n == 0) {
-        GRAPE_HIP_CHECK(hipMemsetAsync(out, 0, 32, s));
-        return GRAPE_OK;
+        return zero_fill(out, 32, s);
     }
     CHECK_PTR16(in);
     unsigned nb = blocks_for(n);

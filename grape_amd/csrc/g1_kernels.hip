@@ -662,7 +662,8 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     int rc = scratch_get(kSlotMsm, nwaves * 64 * (size_t)(4 * kPartialWords) + 64, &ws);
     if (rc) return rc;
     int* err = (int*)((char*)ws + nwaves * 64 * (size_t)(4 * kPartialWords));
-    GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
+    rc = zero_fill(err, sizeof(int), s);
+    if (rc) return rc;
     profile_begin();
     profile_mark(s);
     commit_wide_kernel<FR><<<blocks_for(nwaves * 64), kBlock, 0, s>>>((uint32_t*)ws, scalars, rowlen, rows, seg, nseg, table, N, c, nw, K, err);
@@ -798,7 +799,8 @@ int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len
     int rc = scratch_get(kSlotMsm, slab * ncols * (16 * FW) + 64, &ws);
     if (rc) return rc;
     int* err = (int*)((char*)ws + slab * ncols * (16 * FW));
-    GRAPE_HIP_CHECK(hipMemsetAsync(err, 0, sizeof(int), s));
+    rc = zero_fill(err, sizeof(int), s);
+    if (rc) return rc;
     for (size_t t0 = 0; t0 < len; t0 += slab) {
         size_t nt = len - t0 < slab ? len - t0 : slab;
         size_t n_entries = nt * ncols;

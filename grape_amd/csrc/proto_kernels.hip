@@ -544,7 +544,8 @@ int grape_tlookup_inverse_by_table(uint32_t* A, const uint32_t* S, const int32_t
     void* cnt;
     int rc = scratch_get(kSlotMisc, 64, &cnt);
     if (rc) return rc;
-    GRAPE_HIP_CHECK(hipMemsetAsync(cnt, 0, sizeof(unsigned int), s));
+    rc = zero_fill(cnt, sizeof(unsigned int), s);
+    if (rc) return rc;
     inverse_by_table_kernel<<<blocks_for(n), kBlock, 0, s>>>(A, S, idx1, T, B, n, len, (unsigned int*)cnt);
     GRAPE_LAUNCH_CHECK();
     unsigned int h = 0;
