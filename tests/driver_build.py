@@ -1,4 +1,4 @@
-"""Builds the C++ drivers of the test-suite (tests/native/driver_flow.cpp, layer_flow.cpp: programs
+"""Builds the C++ drivers of the test-suite (tests/native/driver_flow.cpp, layer_flow.cpp, commit_flow.cpp: programs
 in the reference's style against the host classes) with g++, for the curve GRAPE_CURVE names
 (<name> for BLS12-381, <name>_bn254 for BN254)."""
 import os
@@ -6,7 +6,7 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-DRIVERS = ("driver_flow", "layer_flow")
+DRIVERS = ("driver_flow", "layer_flow", "commit_flow")
 
 
 def exe_path(curve, name="driver_flow"):

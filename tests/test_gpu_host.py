@@ -383,3 +383,18 @@ def test_cpp_layer_driver_runs(ops, tmp_path):
     res = subprocess.run([exe, "1024", str(tmp_path)], capture_output=True, text=True, timeout=280)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
     assert "layer_flow OK: 37 steps" in res.stdout
+
+
+def test_cpp_commit_driver_runs(ops, tmp_path):
+    """the reference's artefact pipeline (test/ppgen.cu, the witness files of zzllama/llama/model.py,
+    test/commit.cu:37-183) by a C++ program against the host classes, at 1/16 of the model's widths:
+    points.bin / cpu_points.bin written and read back, 32 witness files committed from disk into
+    com{W,Q,R}, and the stored commitments verify openings of the stored tensors (a changed
+    commitment does not)"""
+    import subprocess
+    import driver_build
+    exe = driver_build.build(None, "commit_flow")
+    res = subprocess.run([exe, str(tmp_path / "artefacts"), "64"], capture_output=True, text=True, timeout=280)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    assert "commit_flow OK" in res.stdout
+    assert (tmp_path / "artefacts" / "comW" / "down-0.bin").stat().st_size > 0

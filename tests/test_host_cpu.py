@@ -57,6 +57,7 @@ def test_cpp_driver_compiles_against_the_host_headers():
     import os
     import driver_build
     assert os.path.exists(driver_build.build(None, "layer_flow"))
+    assert os.path.exists(driver_build.build(None, "commit_flow"))
     exe = driver_build.build()
     assert os.path.exists(exe)
 
