@@ -1,12 +1,12 @@
-"""Builds the C++ drivers of the test-suite (tests/native/driver_flow.cpp, layer_flow.cpp, commit_flow.cpp: programs
-in the reference's style against the host classes) with g++, for the curve GRAPE_CURVE names
+"""Builds the C++ drivers of the test-suite (tests/native/driver_flow.cpp, layer_flow.cpp, commit_flow.cpp,
+programs_flow.cpp: programs in the reference's style against the host classes) with g++, for the curve GRAPE_CURVE names
 (<name> for BLS12-381, <name>_bn254 for BN254)."""
 import os
 import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-DRIVERS = ("driver_flow", "layer_flow", "commit_flow")
+DRIVERS = ("driver_flow", "layer_flow", "commit_flow", "programs_flow")
 
 
 def exe_path(curve, name="driver_flow"):
@@ -24,7 +24,7 @@ def build(curve=None, name="driver_flow"):
     src = os.path.join(HERE, "native", name + ".cpp")
     host = os.path.join(ROOT, "grape_amd", "host")
     pkg = os.path.join(ROOT, "grape_amd")
-    deps = [src, os.path.join(host, "libgrape_host%s.so" % suffix), os.path.join(pkg, "libgrape_hip%s.so" % suffix)]
+    deps = [src, os.path.join(HERE, "native", "artefacts.hpp"), os.path.join(host, "libgrape_host%s.so" % suffix), os.path.join(pkg, "libgrape_hip%s.so" % suffix)]
     if os.path.exists(exe) and all(os.path.getmtime(d) <= os.path.getmtime(exe) for d in deps):
         return exe
     subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-Wno-unknown-pragmas", "-Wno-class-memaccess"]

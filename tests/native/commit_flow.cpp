@@ -16,49 +16,12 @@
 #include <stdexcept>
 #include <string>
 #include <vector>
-#include "../../include/grape_hip.h"
-#include "../../grape_amd/host/ec_operation.hpp"
+#include "artefacts.hpp"
 #include "../../grape_amd/host/fr_tensor.hpp"
 #include "../../grape_amd/host/hyrax.hpp"
-#include "../../grape_amd/host/ioutils.hpp"
-#include "../../grape_amd/host/witness.hpp"
 
 static void require(bool ok, const std::string& what) {
     if (!ok) throw std::runtime_error("commit_flow: " + what);
-}
-
-struct Rng {
-    unsigned long long s;
-    explicit Rng(unsigned long long seed) : s(seed * 0x9e3779b97f4a7c15ull + 1) {}
-    unsigned next() {
-        s ^= s << 13; s ^= s >> 7; s ^= s << 17;
-        return (unsigned)(s >> 32);
-    }
-    int gauss(double sigma) {
-        double u = 0;
-        for (int i = 0; i < 4; i++) u += (double)next() / 4294967296.0;
-        return (int)((u - 2.0) * 1.7320508 * sigma);
-    }
-};
-
-static int* device_ints(size_t n, Rng& rng, double sigma, int clip, int offset = 0) {
-    std::vector<int> h(n);
-    for (size_t i = 0; i < n; i++) {
-        int v = rng.gauss(sigma);
-        if (clip) v = v < -clip ? -clip : (v > clip - 1 ? clip - 1 : v);
-        h[i] = v + offset;
-    }
-    int* d = nullptr;
-    require(grape_malloc((void**)&d, sizeof(int) * n) == 0, "grape_malloc");
-    require(grape_memcpy_h2d(d, h.data(), sizeof(int) * n, nullptr) == 0, "h2d");
-    return d;
-}
-
-static int* upload(const std::vector<int>& h) {
-    int* d = nullptr;
-    require(grape_malloc((void**)&d, sizeof(int) * h.size()) == 0, "grape_malloc");
-    require(grape_memcpy_h2d(d, h.data(), sizeof(int) * h.size(), nullptr) == 0, "h2d");
-    return d;
 }
 
 struct FileInfo {
@@ -75,21 +38,13 @@ int main(int argc, char** argv) {
     try {
         require(input_tokens >= 16 && input_tokens % 16 == 0, "input_tokens must be a multiple of 16");
         auto t0 = std::chrono::steady_clock::now();
-        for (const char* sub : {"", "/W", "/Q", "/R", "/comW", "/comQ", "/comR"}) mkdir((dir + sub).c_str(), 0755);
         Fr::seed(99);
+        const artefacts::Shape shape = {input_tokens, dim, max_embed_dim, npoints, com_scale};
 
         // ---- test/ppgen.cu: generators, the reference-format table, both files; read back as test/commit.cu:28-32 does
         const size_t ngen = (size_t)npoints * com_scale;
-        affine_t* points = nullptr;
-        require(grape_malloc((void**)&points, sizeof(affine_t) * 256 * ngen) == 0, "grape_malloc");
-        {
-            std::vector<bn128> gens = precompute_generators((uint)ngen, 256, points);
-            savebin(dir + "/points.bin", points, sizeof(affine_t) * 256 * ngen);
-            savebin(dir + "/cpu_points.bin", gens.data(), gens.size() * sizeof(bn128), false);
-            require(findsize(dir + "/points.bin") == sizeof(affine_t) * 256 * ngen, "points.bin size");
-            require(findsize(dir + "/cpu_points.bin") == sizeof(bn128) * ngen, "cpu_points.bin size");
-            require(grape_memset_zero(points, sizeof(affine_t) * 256 * ngen, nullptr) == 0, "memset");
-        }
+        affine_t* points = artefacts::write_parameters(dir, shape);
+        require(grape_memset_zero(points, sizeof(affine_t) * 256 * ngen, nullptr) == 0, "memset");
         loadbin(dir + "/points.bin", points, sizeof(affine_t) * 256 * ngen);
         std::vector<bn128> cpu_points(ngen);
         loadbin(dir + "/cpu_points.bin", cpu_points.data(), ngen * sizeof(bn128), false);
@@ -97,23 +52,8 @@ int main(int argc, char** argv) {
         Hyrax hyrax(layer_num, npoints, points, cpu_points[0]);
 
         // ---- the witness files of one block
-        Rng rng(5);
-        const size_t DD = (size_t)dim * dim, FD = (size_t)max_embed_dim * dim;
-        LayerWitness::Weights w;
-        w.Q = device_ints(DD, rng, 4096, 32768);
-        w.K = device_ints(DD, rng, 4096, 32768);
-        w.V = device_ints(DD, rng, 4096, 32768);
-        w.O = device_ints(DD, rng, 4096, 32768);
-        w.gate = device_ints(FD, rng, 4096, 32768);
-        w.up = device_ints(FD, rng, 4096, 32768);
-        w.down = device_ints(FD, rng, 4096, 32768);
-        w.norm_first = device_ints(dim, rng, 500, 0, 65536);
-        w.norm_second = device_ints(dim, rng, 500, 0, 65536);
-        int* x = device_ints((size_t)input_tokens * dim, rng, 65536, 0);
-        LayerWitness::Tables tables{upload(LayerWitness::make_exp_table()), upload(LayerWitness::make_silu_table())};
-        LayerWitness lw(input_tokens, dim, max_embed_dim);
-        lw.generate(x, w, tables);
-        lw.save(dir, 0);
+        artefacts::write_witness(dir, shape, 5);
+        for (const char* sub : {"/comW", "/comQ", "/comR"}) mkdir((dir + sub).c_str(), 0755);
         std::printf("parameters and witness files written after %.1f s\n", std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count());
         std::fflush(stdout);
 

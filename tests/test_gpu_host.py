@@ -398,3 +398,17 @@ def test_cpp_commit_driver_runs(ops, tmp_path):
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
     assert "commit_flow OK" in res.stdout
     assert (tmp_path / "artefacts" / "comW" / "down-0.bin").stat().st_size > 0
+
+
+def test_cpp_reference_programs_run(ops, tmp_path):
+    """the reference's five single-protocol programs (test/matmul.cu, eleWiseMul.cu, combine_value.cu,
+    tlookupTest.cu, tlookupMapTest.cu) as functions of a C++ program that keep their call
+    sequences and read points.bin / cpu_points.bin / table/*.bin / {W,Q,R}/*.bin with loadbin and
+    load_data; each result is also checked against a direct evaluation, and the two lookups refuse
+    a witness that is off the table"""
+    import subprocess
+    import driver_build
+    exe = driver_build.build(None, "programs_flow")
+    res = subprocess.run([exe, str(tmp_path / "artefacts")], capture_output=True, text=True, timeout=280)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    assert "programs_flow OK" in res.stdout

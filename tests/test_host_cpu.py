@@ -58,6 +58,7 @@ def test_cpp_driver_compiles_against_the_host_headers():
     import driver_build
     assert os.path.exists(driver_build.build(None, "layer_flow"))
     assert os.path.exists(driver_build.build(None, "commit_flow"))
+    assert os.path.exists(driver_build.build(None, "programs_flow"))
     exe = driver_build.build()
     assert os.path.exists(exe)
 
