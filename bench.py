@@ -268,6 +268,8 @@ def layer_workload(args):
         "config": {"workload": "configs[4]: LLaMA-2-7B-shape decoder layer proof, seq_len %d, d_model 4096, 32 heads x 128, "
                                "FFN 11008, int16 weights/activations" % T,
                    "breakdown_s": {k: float(v) for k, v in times.items()},
+                   "step_s": [float(t) for t in totals],
+                   "hbm_free_gib_at_end": torch.cuda.mem_get_info()[0] / 2**30,
                    "n_matmul_sumchecks": counts["matmul"], "n_lookups": counts["lookup"],
                    "weight_points": weight_points,
                    "witness": "the library's integer kernels (grape_wit_matmul_rescale)" if native else "torch (float64 products, exact below 2^53)",

@@ -207,8 +207,21 @@ __device__ __forceinline__ uint32_t fr_digit(const Fr& k, uint32_t w, uint32_t c
 // acc += k * G_col through the wide table: one gather and one mixed addition per non-zero digit.
 // While the addition of digit w runs, the table line of digit w+1 is already on its way (one
 // word of it is touched right after the entry of digit w has been requested).
-__device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k, const uint32_t* table, size_t N, uint32_t col,
+__device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k_in, const uint32_t* table, size_t N, uint32_t col,
                                                uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
+    // The scalar is taken as +-|k| with |k| <= (r-1)/2 < 2^254 (r - k and the negated point when k is
+    // in the upper half): the top window then never carries out, and nw = ceil(255/c) windows are
+    // enough - one addition fewer per scalar at c = 15.
+    Fr k = k_in;
+    uint32_t borrow = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t half_i = (FrParams::mod(i) >> 1) | (i + 1 < 8 ? FrParams::mod(i + 1) << 31 : 0u);
+        const uint64_t t = (uint64_t)half_i - (uint64_t)k.v[i] - (uint64_t)borrow;
+        borrow = (uint32_t)(t >> 63);
+    }
+    const bool flip = borrow != 0;                        // k > (r-1)/2
+    k = cneg(k, flip);
     uint32_t nwin = nw;
     while (nwin > 0 && (nwin - 1) * c >= 256) nwin--;     // windows that start inside the scalar
     uint32_t carry = 0;
@@ -226,14 +239,14 @@ __device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k, const u
                 // unconditional, so that the compiler counts the outstanding loads exactly
                 const size_t nxt = (mag_n != 0 && mag_n <= K) ? ((size_t)(w + 1) * K + (mag_n - 1)) * N + col : (size_t)col;
                 touch = table[(size_t)kWideEntryWords * nxt];
-                madd28(acc, e, neg);
+                madd28(acc, e, neg != flip);
             }
         }
         mag = mag_n;
         neg = neg_n;
     }
     asm volatile("" ::"v"(touch));      // keeps the last touch alive until here
-    if (carry) *err_flag = 1;   // cannot happen for canonical 255-bit scalars when nw*c >= 256
+    if (carry) *err_flag = 1;   // cannot happen for canonical scalars when nw*c >= 255
 }
 
 __device__ __forceinline__ G1Xyzz shfl_down_xyzz(const G1Xyzz& a, int off) {
@@ -647,7 +660,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
     GRAPE_REQUIRE(c >= 2 && c <= (FR ? 16u : 24u) && nw >= 1 && K >= (1u << (c - 1)), "need 2 <= c <= 16 (24 for int32) and K >= 2^(c-1)");
-    if (FR) GRAPE_REQUIRE((uint64_t)nw * c >= 256, "Fr scalars need nw*c >= 256");
+    if (FR) GRAPE_REQUIRE((uint64_t)nw * c >= 255, "Fr scalars need nw*c >= 255");
     const size_t rows = size / rowlen;
     if (rows == 0) return GRAPE_OK;
     hipStream_t s = as_stream(st);
@@ -789,7 +802,7 @@ int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len
                               uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(len >= 1 && ncols >= 1 && ncols <= N, "bad shape");
-    GRAPE_REQUIRE(c >= 2 && c <= 16 && (uint64_t)nw * c >= 256 && K >= (1u << (c - 1)), "need a full-width wide table");
+    GRAPE_REQUIRE(c >= 2 && c <= 16 && (uint64_t)nw * c >= 255 && K >= (1u << (c - 1)), "need a full-width wide table");
     hipStream_t s = as_stream(st);
     // slabs of scalars so that the XYZZ staging buffer stays near 1.5 GiB
     size_t slab = ((size_t)3 << 29) / (ncols * (16 * FW));

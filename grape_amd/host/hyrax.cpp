@@ -1,6 +1,8 @@
 #include "hyrax.hpp"
 #include <cstdlib>
 #include <cassert>
+#include <map>
+#include <utility>
 #include "../../include/grape_hip.h"
 
 using grape_host::check;
@@ -39,7 +41,16 @@ Hyrax::Hyrax(uint layer_num_, uint npoints_, affine_t* g, bn128& G_, uint com_sc
         if (end != e) table_budget_ = (size_t)gib << 30;
     }
 }
+// scaled tables handed out: table -> (the Hyrax object whose budget holds it, bytes).  Never
+// destroyed: lookup objects with static lifetime release their tables while the process exits.
+static std::map<const void*, std::pair<Hyrax*, size_t>>& scaled_registry() {
+    static auto* r = new std::map<const void*, std::pair<Hyrax*, size_t>>();
+    return *r;
+}
+
 Hyrax::~Hyrax() {
+    for (auto& e : scaled_registry())
+        if (e.second.first == this) e.second.first = nullptr;
     grape_free(int16_table_.d);
     grape_free(int16x2_table_.d);
     grape_free(int32_table_.d);
@@ -110,12 +121,13 @@ bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
     if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);
     if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
-    // ceil(256 / c) windows: the top signed digit of a 255-bit scalar may carry into one more.
+    // ceil(255 / c) windows: the kernel takes a scalar of the upper half as -(r - k), so magnitudes
+    // stay below 2^254 and the top signed digit never carries out (c = 15: 17 windows, not 18).
     // Below c = 10 a wide table (32 additions per element at c = 8) saves nothing over the
     // reference-format table, whose path needs no build, so very long rows (the reference's
     // com_scale = 16 shapes: 65536 to 262144 columns) stay on that path.
     for (uint c = 15; c >= 10; c--) {
-        uint nw = (256 + c - 1) / c, K = 1u << (c - 1);
+        uint nw = (255 + c - 1) / c, K = 1u << (c - 1);
         if (used + grape_g1_wide_table_bytes(rowlen, nw, K) <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }
     return false;
@@ -152,7 +164,18 @@ affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
                                     fr_table_.nw, fr_table_.K, nullptr),
           "grape_g1_scaled_table_gen");
     scaled_bytes_ += bytes;
+    scaled_registry()[out] = std::make_pair(this, bytes);
     return out;
+}
+
+void Hyrax::release_scaled_table(affine_t* table) {
+    if (!table) return;
+    auto it = scaled_registry().find(table);
+    if (it != scaled_registry().end()) {
+        if (it->second.first) it->second.first->scaled_bytes_ -= it->second.second;
+        scaled_registry().erase(it);
+    }
+    grape_free(table);
 }
 
 affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len) {

@@ -55,6 +55,9 @@ public:
     // owned by the caller, freed with grape_free); nullptr when it would not fit the budget.
     // With it, a tensor whose elements are scalars[idx] commits at one addition per element:
     affine_t* build_scaled_table(const FrTensor& scalars, uint ncols);
+    // frees a table that build_scaled_table returned and gives its bytes back to the budget of the
+    // Hyrax object that built it, if that object still exists
+    static void release_scaled_table(affine_t* table);
     // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
     affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len);
 

@@ -13,7 +13,7 @@ tLookup::tLookup(const uint size) : alpha(Fr::random_element()), beta(Fr((long)s
 tLookup::~tLookup() {
     grape_free(com_A);
     grape_free(com_m);
-    grape_free(scaled_table_);
+    Hyrax::release_scaled_table(scaled_table_);
     grape_free(d_idx_);
 }
 
@@ -122,7 +122,7 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         grape_free(com_m);
         const uint rowlen = msm_size * hyrax.com_scale;
         if (indexed_commit_ && index_known_ && (scaled_for_ != &hyrax || scaled_cols_ < rowlen)) {
-            grape_free(scaled_table_);
+            Hyrax::release_scaled_table(scaled_table_);
             scaled_table_ = hyrax.build_scaled_table(B, rowlen);   // nullptr when over budget
             scaled_cols_ = scaled_table_ ? rowlen : 0;
             scaled_for_ = &hyrax;

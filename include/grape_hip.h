@@ -225,7 +225,9 @@ int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t si
                      const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
 /* Same for full-width Fr scalars (Montgomery form in, left untouched — the reference's
  * tensor.from()/to() round trip of src/Hyrax.cu:347,356 is not needed).
- * Hyrax::commit(FrTensor&, size, N), src/Hyrax.cu:335-359. Requires nw*c >= 256. */
+ * Hyrax::commit(FrTensor&, size, N), src/Hyrax.cu:335-359. Requires nw*c >= 255: a scalar in the
+ * upper half of the field is taken as -(r - k), so magnitudes stay below 2^254 and the top window
+ * never carries out. */
 int grape_commit_fr(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
                     const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
 /* Commitments through the reference-format table (k*G_i, k < 256, byte windows of |s| resp. of

@@ -152,6 +152,37 @@ def test_commit_fr_edge_scalars_and_int_path_agreement(ops, gens64):
     assert_same(a, b, "int path == Fr path")
 
 
+def test_commit_fr_half_range_recoding(ops, gens64):
+    """windows that cover only 255 bits (nw * c = 255): a scalar above (r-1)/2 is committed as
+    -(r - k), so the top window never carries out; scalars at and around r/2, at the ends of the
+    field and with long carry chains against the big-integer sum"""
+    k, host, dev = gens64
+    n = 16
+    r = br.R_MOD
+    top = 1 << (r.bit_length() - 1)
+    vals = [(r - 1) // 2, (r + 1) // 2, (r - 1) // 2 - 1, (r + 1) // 2 + 1, r - 1, r - 2, 1, 0,
+            top - 1, top, (1 << 240) - 1, r - (1 << 240), 0x7fff7fff7fff7fff7fff, (1 << 254) % r, r // 3, 2 * r // 3]
+    s = br.fr_pack(vals)
+    want = br.g1_msm(vals, br.g1_unpack(host[:n]))
+    for c, nw in ((15, 17), (5, 51), (16, 16)):
+        wide = ops.g1_wide_table_gen(dev[:n].contiguous(), c, nw, 1 << (c - 1))
+        got = br.g1_unpack(ops.g1_to_host(ops.commit_fr(ops.to_dev(s), n, wide, n, c, nw, 1 << (c - 1))))[0]
+        assert got == want, (c, nw)
+        # each scalar alone, so that no cancellation can hide a wrong digit
+        rows = np.zeros((n, n, 4), dtype=np.uint64)
+        for i in range(n):
+            rows[i, i] = s[i]
+        got = br.g1_unpack(ops.g1_to_host(ops.commit_fr(ops.to_dev(rows.reshape(n * n, 4)), n, wide, n, c, nw, 1 << (c - 1))))
+        pts = br.g1_unpack(host[:n])
+        for i in range(n):
+            assert got[i] == br.g1_msm([vals[i]], [pts[i]]), (c, nw, i)
+        del wide
+    from grape_amd import GrapeError
+    wide = ops.g1_wide_table_gen(dev[:n].contiguous(), 15, 16, 1 << 14)
+    with pytest.raises(GrapeError):
+        ops.commit_fr(ops.to_dev(s), n, wide, n, 15, 16, 1 << 14)       # 240 bits of windows: refused
+
+
 def test_commit_linearity_medium(ops):
     # size-independent property on a larger shape: com(a + b) = com(a) + com(b)
     import torch
