@@ -523,6 +523,7 @@ int grape_i32_pad_fill(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad
 }
 
 int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
+    if (N == 0) return GRAPE_OK;
     CHECK_PTR16(t); CHECK_PTR16(x);
     GRAPE_REQUIRE(c >= 1 && gap >= 1 && N >= (size_t)c * gap && N % ((size_t)c * gap) == 0, "N must be a multiple of c*gap");
     hipStream_t s = as_stream(st);

@@ -656,6 +656,7 @@ static uint32_t reduce_lanes_log2(size_t rows) {
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                             uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
@@ -698,6 +699,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
 template <bool FR>
 static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t npoints,
                            grape_stream_t st) {
+    if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
     const size_t rows = size / rowlen;

@@ -1,0 +1,90 @@
+"""Empty inputs: every entry point that takes an element count accepts zero, launches nothing and
+leaves its outputs alone (the reference's kernels are launched with (n + 255) / 256 blocks, i.e.
+none; here a zero-sized launch would be an error, so each entry point returns early)."""
+import numpy as np
+import pytest
+
+import bigref as br
+from gpuutil import rand_fr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from grape_amd import ops as o
+    o.init(0)
+    return o
+
+
+def test_field_entry_points_accept_zero_elements(ops):
+    import torch
+    e = ops.fr_empty(0)
+    x = ops.to_dev(rand_fr(1, 1))
+    assert ops.fr_add(e, e).shape[0] == 0
+    assert ops.fr_sub(e, e).shape[0] == 0
+    assert ops.fr_mul(e, e).shape[0] == 0
+    assert ops.fr_bcast_add(e, x).shape[0] == 0
+    assert ops.fr_bcast_mul(e, x).shape[0] == 0
+    assert ops.fr_from_i32(torch.empty(0, dtype=torch.int32, device="cuda")).shape[0] == 0
+    assert ops.fr_to_mont(e).shape[0] == 0
+    assert ops.fr_from_mont(e).shape[0] == 0
+    assert ops.fr_batch_inverse(e).shape[0] == 0
+    assert ops.fr_shift_inverse(e, x).shape[0] == 0
+    assert not np.any(ops.fr_to_host(ops.fr_sum(e, 0)))
+
+
+def test_protocol_entry_points_accept_zero_elements(ops):
+    import torch
+    e = ops.fr_empty(0)
+    x = ops.to_dev(rand_fr(1, 2))
+    hist = ops.tlookup_hist(e, -8, 16)
+    assert hist.cpu().numpy().sum() == 0
+    assert ops.tlookup_index(e, -8, 16).shape[0] == 0
+    ops.fr_fold_msb_multi([ops.fr_empty(0)], 0, x)
+    assert ops.fr_pad(e, 3, 4, 0, x).shape[0] == 0
+    assert ops.i32_pad(torch.empty(0, dtype=torch.int32, device="cuda"), 3, 4, 0).shape[0] == 0
+    ops.fr_fold(e, 0, x, 1, 0, 1)
+    assert ops.fr_sum_by_dim(e, 0, 4).shape[0] == 0
+    # a protocol round over no indices has no meaning: refused, not silently "proved"
+    from grape_amd import GrapeError
+    for call in (lambda: ops.sumcheck_round2(e, e, 0, 0, x), lambda: ops.tlookup_round_sums(e, e, x, e, 0),
+                 lambda: ops.tlookup_mb_sums(e, e, 0)):
+        with pytest.raises(GrapeError):
+            call()
+
+
+def test_commitment_of_no_rows(ops):
+    import torch
+    k = [3, 5, 7, 11]
+    dev = ops.g1_make_generators(k)
+    wide = ops.g1_wide_table_gen(dev, 8, 5, 128)
+    out = ops.commit_i32(torch.empty(0, dtype=torch.int32, device="cuda"), 4, wide, 4, 8, 5, 128)
+    assert out.shape[0] == 0
+    wide_fr = ops.g1_wide_table_gen(dev, 8, 32, 128)
+    assert ops.commit_fr(ops.fr_empty(0), 4, wide_fr, 4, 8, 32, 128).shape[0] == 0
+    tab = ops.g1_table_gen(dev, 256)
+    assert ops.commit_i32_ref_table(torch.empty(0, dtype=torch.int32, device="cuda"), 4, tab, 4).shape[0] == 0
+    assert ops.commit_fr_ref_table(ops.fr_empty(0), 4, tab, 4).shape[0] == 0
+    assert ops.g1_affine_to_jacobian(ops.g1_empty(0)).shape[0] == 0
+
+
+def test_witness_entry_points_accept_zero_rows(ops):
+    import torch
+    z = torch.empty((0, 8), dtype=torch.int32, device="cuda")
+    w = torch.ones((4, 8), dtype=torch.int32, device="cuda")
+    q, r = ops.wit_matmul_rescale(z, w, 1 << 16)
+    assert q.shape[0] == 0 and r.shape[0] == 0
+    q, r = ops.wit_elemul_rescale(z, z, 1 << 16)
+    assert q.numel() == 0
+    assert ops.wit_add(z, z).numel() == 0
+    table = torch.arange(16, dtype=torch.int32, device="cuda")
+    assert ops.wit_table_lookup(z, 0, table).numel() == 0
+    assert ops.wit_row_sumsq(z).numel() == 0
+    big = torch.zeros(1 << 20, dtype=torch.int32, device="cuda")
+    assert ops.wit_softmax(z, big)["softmax_output"].numel() == 0
+    assert ops.wit_rmsnorm_apply(z, torch.empty(0, dtype=torch.int32, device="cuda"), torch.ones(8, dtype=torch.int32, device="cuda"))[0].numel() == 0
+    assert ops.wit_status() == 0
