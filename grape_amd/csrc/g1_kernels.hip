@@ -657,6 +657,7 @@ template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                             uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
+    GRAPE_REQUIRE(size <= 0xffffffffull, "size must fit the reference's 32-bit element count");
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
@@ -671,20 +672,30 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     uint32_t nseg = 1;
     while (rows * nseg < 4096 && rowlen / (nseg * 2) >= 64 && nseg * 2 <= (2u << lg_lpr)) nseg *= 2;
     const uint32_t seg = (rowlen + nseg - 1) / nseg;
-    const size_t nwaves = rows * nseg;
+    // rows go through in slabs so that the per-lane partial sums stay within 512 MiB whatever the
+    // number of rows (a row segment leaves 64 partial sums of 256 bytes)
+    size_t slab = 32768 / (size_t)nseg;
+    if (slab > rows) slab = rows;
+    const size_t partial_bytes = slab * nseg * 64 * (size_t)(4 * kPartialWords);
     void* ws;
-    int rc = scratch_get(kSlotMsm, nwaves * 64 * (size_t)(4 * kPartialWords) + 64, &ws);
+    int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws);
     if (rc) return rc;
-    int* err = (int*)((char*)ws + nwaves * 64 * (size_t)(4 * kPartialWords));
+    int* err = (int*)((char*)ws + partial_bytes);
     rc = zero_fill(err, sizeof(int), s);
     if (rc) return rc;
-    profile_begin();
-    profile_mark(s);
-    commit_wide_kernel<FR><<<blocks_for(nwaves * 64), kBlock, 0, s>>>((uint32_t*)ws, scalars, rowlen, rows, seg, nseg, table, N, c, nw, K, err);
-    profile_mark(s);
+    const size_t elem_words = FR ? 8 : 1;
     const size_t rows_per_wave = (size_t)64 >> lg_lpr;
-    commit_reduce_kernel<<<(unsigned)((rows + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out, (const uint32_t*)ws, rows, nseg * 64, lg_lpr);
-    profile_mark(s);
+    profile_begin();
+    for (size_t r0 = 0; r0 < rows; r0 += slab) {
+        const size_t nr = rows - r0 < slab ? rows - r0 : slab;
+        const uint32_t* sc = (const uint32_t*)scalars + r0 * rowlen * elem_words;
+        profile_mark(s);
+        commit_wide_kernel<FR><<<blocks_for(nr * nseg * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, N, c, nw, K, err);
+        profile_mark(s);
+        commit_reduce_kernel<<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), (const uint32_t*)ws, nr,
+                                                                                                 nseg * 64, lg_lpr);
+        profile_mark(s);
+    }
     GRAPE_LAUNCH_CHECK();
     int h_err = 0;
     GRAPE_HIP_CHECK(hipMemcpyAsync(&h_err, err, sizeof(int), hipMemcpyDeviceToHost, s));
@@ -700,6 +711,7 @@ template <bool FR>
 static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t npoints,
                            grape_stream_t st) {
     if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
+    GRAPE_REQUIRE(size <= 0xffffffffull, "size must fit the reference's 32-bit element count");
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
     const size_t rows = size / rowlen;
