@@ -160,6 +160,8 @@ def layer_workload(args):
         times["lookup"] += host.last_prove_seconds()
         times["lookup_commits"] += res["commit_s"]
         counts["lookup"] += 1
+        if os.environ.get("GRAPE_BENCH_VERBOSE"):
+            print("  range lookup n=%d: %.4f s (commitments %.4f)" % (n, host.last_prove_seconds(), res["commit_s"]), file=sys.stderr)
 
     def mapping_lookup(x_in, x_out, low, length, fmap):
         a, b = x_in.contiguous().view(-1), x_out.contiguous().view(-1)
@@ -169,6 +171,9 @@ def layer_workload(args):
         times["lookup"] += host.last_prove_seconds()
         times["lookup_commits"] += host.last_commit_seconds()
         counts["lookup"] += 1
+        if os.environ.get("GRAPE_BENCH_VERBOSE"):
+            print("  mapping lookup n=%d len=%d: %.4f s (commitments %.4f)" % (n, length, host.last_prove_seconds(),
+                                                                             host.last_commit_seconds()), file=sys.stderr)
 
     def matmul_proof(a_int, b_int, L, N, M, K, q, r):
         """sumcheck for Y[l][n][m] = sum_k A[l][n][k] B[l][m][k] with claim Y(u), Y = q*2^16 + r"""

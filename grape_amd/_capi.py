@@ -28,6 +28,7 @@ SIGNATURES = {
     "grape_stream_sync": [c_void_p],
     "grape_malloc": [ctypes.POINTER(c_void_p), c_size_t],
     "grape_free": [c_void_p],
+    "grape_alloc_cache_release": [c_void_p],
     "grape_memcpy_h2d": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_memcpy_d2h": [c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_memcpy_d2d": [c_void_p, c_void_p, c_size_t, c_void_p],

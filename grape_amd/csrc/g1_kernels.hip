@@ -75,8 +75,12 @@ __device__ __forceinline__ Fr ld_fr8(const uint32_t* base, size_t i) {
 }
 
 // Wide-table entry: an affine point in the 28-bit working form, x[L28] then y[L28] as 32-bit
-// words, padded to 128 bytes, so that every gather is exactly one cache line.
-constexpr int kWideEntryWords = 32;
+// words.  BLS12-381's 112 bytes are padded to 128, so that every gather is exactly one cache line;
+// BN254's 80 bytes are stored dense (a multiple of 16 bytes: the loads stay aligned, half of the
+// entries straddle two lines) - the table is 37.5 % smaller, which is what lets 15-bit windows fit
+// the table budget there.
+constexpr int kWideEntryWords = (2 * L28 <= 20) ? 2 * L28 : 32;
+static_assert(kWideEntryWords % 4 == 0 && kWideEntryWords >= 2 * L28, "entry layout");
 __device__ __forceinline__ Affine28 ld_entry28(const uint32_t* table, size_t e) {
     const uint4* q = reinterpret_cast<const uint4*>(table + (size_t)kWideEntryWords * e);
     uint4 w[L28 / 2];
@@ -93,17 +97,17 @@ __device__ __forceinline__ Affine28 ld_entry28(const uint32_t* table, size_t e) 
 }
 __device__ __forceinline__ void st_entry28(uint32_t* table, size_t e, const G1Affine& a) {
     Fp28 x = fp28::from_canonical(a.x), y = fp28::from_canonical(a.y);
-    uint32_t f[32];
+    uint32_t f[kWideEntryWords];
 #pragma unroll
     for (int i = 0; i < L28; i++) {
         f[i] = (uint32_t)x.v[i];
         f[L28 + i] = (uint32_t)y.v[i];
     }
 #pragma unroll
-    for (int i = 2 * L28; i < 32; i++) f[i] = 0;
+    for (int i = 2 * L28; i < kWideEntryWords; i++) f[i] = 0;
     uint4* q = reinterpret_cast<uint4*>(table + (size_t)kWideEntryWords * e);
 #pragma unroll
-    for (int i = 0; i < 8; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+    for (int i = 0; i < kWideEntryWords / 4; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
 }
 __device__ __forceinline__ bool entry_is_inf(const Affine28& a) {
     uint32_t z = 0;
@@ -239,6 +243,7 @@ __device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k_in, cons
                 // unconditional, so that the compiler counts the outstanding loads exactly
                 const size_t nxt = (mag_n != 0 && mag_n <= K) ? ((size_t)(w + 1) * K + (mag_n - 1)) * N + col : (size_t)col;
                 touch = table[(size_t)kWideEntryWords * nxt];
+                if (kWideEntryWords % 32 != 0) touch |= table[(size_t)kWideEntryWords * nxt + kWideEntryWords - 1];   // dense entries: both lines
                 madd28(acc, e, neg != flip);
             }
         }
@@ -460,6 +465,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                     if (mag > K) { *err_flag = 1; continue; }
                     const Affine28 e = ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col);
                     touch = *touch_ptr;
+                    if (kWideEntryWords % 32 != 0) touch |= touch_ptr[kWideEntryWords - 1];   // dense entries: both lines
                     madd28(acc, e, neg);
                 }
             }

@@ -1,7 +1,10 @@
 // Runtime part of the C ABI: device selection, error text, memory helpers, the scratch pool and
 // the two roofline micro-benchmarks (stream copy, v_mad_u64_u32 issue rate).
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
+#include <map>
+#include <mutex>
 #include "common.hpp"
 
 namespace grape {
@@ -52,6 +55,8 @@ int zero_fill(void* d_ptr, size_t bytes, hipStream_t s) {
     return GRAPE_OK;
 }
 
+size_t alloc_cache_release();   // gives the blocks kept by grape_free back to the driver
+
 int scratch_get(ScratchSlot slot, size_t bytes, void** out) {
     if (bytes > g_scratch_bytes[slot]) {
         if (g_scratch[slot]) {
@@ -62,6 +67,10 @@ int scratch_get(ScratchSlot slot, size_t bytes, void** out) {
         }
         size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
         hipError_t e = hipMalloc(&g_scratch[slot], want);
+        if (e != hipSuccess && alloc_cache_release() > 0) {
+            (void)hipGetLastError();
+            e = hipMalloc(&g_scratch[slot], want);
+        }
         if (e != hipSuccess) {
             set_error("scratch allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
             return GRAPE_ENOMEM;
@@ -99,6 +108,51 @@ __global__ void __launch_bounds__(256) mad_kernel(uint64_t* out, int inner, uint
     if (r == 0x123456789abcdefull) out[0] = r;   // practically never; keeps the chains alive
 }
 
+// Block cache of grape_malloc / grape_free.  The host classes allocate and free a tensor per
+// call as the reference does (cudaMalloc / cudaFree, src/fr-tensor.cu:371-374, :235-241); hipMalloc
+// and hipFree of multi-GiB blocks take from a millisecond to hundreds of them, so a freed block of
+// 1 MiB or more is kept (up to a total that GRAPE_ALLOC_CACHE_GIB sets, 32 GiB by default, 0 = off)
+// and handed out again to a request of exactly its size.  hipFree waits for the device; a caller
+// may rely on that and free a buffer that queued kernels still use, so the wait happens when a
+// cached block is handed out again instead.
+static std::mutex g_alloc_mu;
+static std::map<void*, size_t>* g_live = nullptr;              // blocks handed out by grape_malloc
+static std::multimap<size_t, void*>* g_cached = nullptr;       // freed blocks kept for reuse
+static size_t g_cached_bytes = 0;
+static size_t alloc_cache_cap() {
+    static size_t cap = [] {
+        size_t gib = 32;
+        if (const char* e = getenv("GRAPE_ALLOC_CACHE_GIB")) {
+            char* end = nullptr;
+            unsigned long long v = strtoull(e, &end, 10);
+            if (end != e) gib = (size_t)v;
+        }
+        return gib << 30;
+    }();
+    return cap;
+}
+static void alloc_tables() {
+    if (!g_live) {
+        g_live = new std::map<void*, size_t>();
+        g_cached = new std::multimap<size_t, void*>();
+    }
+}
+// gives every cached block back to the driver; returns the bytes released
+static size_t alloc_cache_release_locked() {
+    size_t n = g_cached_bytes;
+    if (g_cached) {
+        for (auto& e : *g_cached) (void)hipFree(e.second);
+        g_cached->clear();
+    }
+    g_cached_bytes = 0;
+    return n;
+}
+
+size_t alloc_cache_release() {
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    return alloc_cache_release_locked();
+}
+
 }  // namespace grape
 
 using namespace grape;
@@ -123,15 +177,55 @@ int grape_stream_sync(grape_stream_t s) {
 }
 int grape_malloc(void** p, size_t bytes) {
     GRAPE_REQUIRE(p != nullptr, "null output pointer");
-    hipError_t e = hipMalloc(p, bytes ? bytes : 1);
+    if (bytes == 0) bytes = 1;
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    alloc_tables();
+    auto it = g_cached->find(bytes);
+    if (it != g_cached->end()) {
+        void* q = it->second;
+        g_cached->erase(it);
+        g_cached_bytes -= bytes;
+        GRAPE_HIP_CHECK(hipDeviceSynchronize());          // what hipFree would have waited for
+        (*g_live)[q] = bytes;
+        *p = q;
+        return GRAPE_OK;
+    }
+    hipError_t e = hipMalloc(p, bytes);
+    if (e != hipSuccess && alloc_cache_release_locked() > 0) {
+        (void)hipGetLastError();
+        e = hipMalloc(p, bytes);                          // once more with the cache given back
+    }
     if (e != hipSuccess) {
+        (void)hipGetLastError();
         set_error("hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
         return GRAPE_ENOMEM;
     }
+    (*g_live)[*p] = bytes;
     return GRAPE_OK;
 }
 int grape_free(void* p) {
-    if (p) GRAPE_HIP_CHECK(hipFree(p));
+    if (!p) return GRAPE_OK;
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    alloc_tables();
+    auto it = g_live->find(p);
+    if (it != g_live->end()) {
+        const size_t bytes = it->second;
+        g_live->erase(it);
+        if (bytes >= ((size_t)1 << 20) && g_cached_bytes + bytes <= alloc_cache_cap()) {
+            g_cached->emplace(bytes, p);
+            g_cached_bytes += bytes;
+            return GRAPE_OK;
+        }
+    }
+    GRAPE_HIP_CHECK(hipFree(p));
+    return GRAPE_OK;
+}
+int grape_alloc_cache_release(size_t* bytes_released) {
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    alloc_tables();
+    GRAPE_HIP_CHECK(hipDeviceSynchronize());
+    const size_t n = alloc_cache_release_locked();
+    if (bytes_released) *bytes_released = n;
     return GRAPE_OK;
 }
 int grape_memcpy_h2d(void* d, const void* s, size_t bytes, grape_stream_t st) {

@@ -152,7 +152,7 @@ affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
 affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
     if (ncols > npoints) throw std::runtime_error("row longer than the generator set");
     if (!ensure_fr_table(ncols)) return nullptr;
-    size_t bytes = (size_t)scalars.size * ncols * 128;
+    size_t bytes = grape_g1_wide_table_bytes(ncols, 1, scalars.size);   // one entry per (scalar, column)
     size_t used = scaled_bytes_ + grape_g1_wide_table_bytes(fr_table_.ngen, fr_table_.nw, fr_table_.K);
     if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
     if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);

@@ -304,11 +304,17 @@ def g1_table_gen(gens, W):
     return out
 
 
+# 32-bit words of a wide-table entry: 2 x 14 limbs padded to 32 (one cache line) on BLS12-381,
+# 2 x 10 limbs stored dense on BN254
+WIDE_ENTRY_WORDS = 20 if _capi.CURVE == "bn254" else 32
+
+
 def g1_wide_table_gen(gens, c, nw, K):
     lib = init()
     n = gens.shape[0]
     nbytes = lib.grape_g1_wide_table_bytes(n, nw, K)
-    out = torch.empty((nbytes // 128, 32), dtype=torch.int32, device="cuda")
+    words = WIDE_ENTRY_WORDS
+    out = torch.empty((nbytes // (4 * words), words), dtype=torch.int32, device="cuda")
     _capi.check(lib.grape_g1_wide_table_gen(_p(out), _p(gens), n, c, nw, K, _s()))
     return out
 

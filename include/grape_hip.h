@@ -48,6 +48,12 @@ int grape_stream_sync(grape_stream_t stream);
  * direct cudaMalloc / cudaMemcpy / cudaFree calls, e.g. src/fr-tensor.cu:371-374,322-328). */
 int grape_malloc(void **d_ptr, size_t bytes);
 int grape_free(void *d_ptr);
+/* grape_free keeps blocks of 1 MiB and more for grape_malloc to hand out again (to a request of
+ * exactly the same size; up to GRAPE_ALLOC_CACHE_GIB in total, default 32, 0 switches it off): the
+ * host classes allocate and free a tensor per call as the reference does, and the driver's
+ * allocation calls cost milliseconds at these sizes.  This gives every kept block back to the
+ * driver (it also happens by itself when an allocation fails).  No counterpart in the reference. */
+int grape_alloc_cache_release(size_t *bytes_released);
 int grape_memcpy_h2d(void *d_dst, const void *src, size_t bytes, grape_stream_t stream);
 int grape_memcpy_d2h(void *dst, const void *d_src, size_t bytes, grape_stream_t stream); /* syncs */
 int grape_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, grape_stream_t stream);
@@ -193,9 +199,10 @@ int grape_g1_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, 
  * With c = 16, nw = 1, K = 32768 a signed 16-bit scalar is ONE mixed addition; with c = 8,
  * nw = 32, K = 128 a 255-bit scalar is 32 signed-digit additions into a single accumulator.
  * The table is private to this library (only the commitment entry points read it): each entry
- * is 128 bytes - the affine coordinates as 14 limbs of 28 bits each, Montgomery radix 2^392,
- * the working form of the commitment kernels - so a gather is exactly one cache line.
- * Size: grape_g1_wide_table_bytes(N, nw, K) = nw*K*N*128 bytes.
+ * holds the affine coordinates in the working form of the commitment kernels - on BLS12-381
+ * 2 x 14 limbs of 28 bits (Montgomery radix 2^392) padded to 128 bytes, so a gather is exactly one
+ * cache line; on BN254 2 x 10 limbs (radix 2^280) stored dense in 80 bytes.
+ * Size: grape_g1_wide_table_bytes(N, nw, K) = nw*K*N entries of 128 bytes (80 in the BN254 build).
  */
 int grape_g1_wide_table_gen(uint32_t *d_table_affine, const uint32_t *d_gens_affine, size_t N, uint32_t c, uint32_t nw,
                             uint32_t K, grape_stream_t stream);
@@ -203,11 +210,11 @@ size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K);
 /*
  * Scaled table out[t*ncols + i] = s_t * G_i for `len` scalars s_t (device, Montgomery Fr) and the
  * first ncols generators, computed through a full-width wide table (c, nw, K as built above).
- * Same 128-byte entry format, so grape_commit_i32(out, idx, size, rowlen, table = this, N = ncols,
+ * Same entry format, so grape_commit_i32(out, idx, size, rowlen, table = this, N = ncols,
  * c = log2(len)+1, nw = 1, K = len) with idx = t+1 gives sum_i s_{t_i} * G_i at ONE addition per
  * element.  Used for the logUp commitment of A = 1/(S+beta): its elements take only `len`
  * distinct values B[t] (the reference commits A as a full-width tensor, src/tlookup.cu:320).
- * No counterpart in the reference.  Size: len*ncols*128 bytes.
+ * No counterpart in the reference.  Size: grape_g1_wide_table_bytes(ncols, 1, len) bytes.
  */
 int grape_g1_scaled_table_gen(uint32_t *d_out, const uint32_t *d_scalars_mont, size_t len, size_t ncols,
                               const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);

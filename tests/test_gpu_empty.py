@@ -88,3 +88,29 @@ def test_witness_entry_points_accept_zero_rows(ops):
     assert ops.wit_softmax(z, big)["softmax_output"].numel() == 0
     assert ops.wit_rmsnorm_apply(z, torch.empty(0, dtype=torch.int32, device="cuda"), torch.ones(8, dtype=torch.int32, device="cuda"))[0].numel() == 0
     assert ops.wit_status() == 0
+
+
+def test_freed_blocks_are_handed_out_again_and_released(ops):
+    """grape_free keeps large blocks, grape_malloc hands a kept block to a request of exactly its
+    size, grape_alloc_cache_release gives them back; small blocks are never kept"""
+    import ctypes
+    from grape_amd import _capi
+    lib = _capi.load()
+    lib.grape_alloc_cache_release(None)
+    n = 64 << 20
+    p, q, r = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    _capi.check(lib.grape_malloc(ctypes.byref(p), n))
+    first = p.value
+    _capi.check(lib.grape_free(p))
+    _capi.check(lib.grape_malloc(ctypes.byref(q), n + 16))       # another size: a fresh block
+    _capi.check(lib.grape_malloc(ctypes.byref(r), n))            # the same size: the kept block
+    assert r.value == first and q.value != first
+    _capi.check(lib.grape_free(q))
+    _capi.check(lib.grape_free(r))
+    released = ctypes.c_size_t(0)
+    _capi.check(lib.grape_alloc_cache_release(ctypes.byref(released)))
+    assert released.value == 2 * n + 16
+    _capi.check(lib.grape_malloc(ctypes.byref(p), 4096))
+    _capi.check(lib.grape_free(p))
+    _capi.check(lib.grape_alloc_cache_release(ctypes.byref(released)))
+    assert released.value == 0

@@ -56,7 +56,7 @@ def test_wide_table_entries(ops, gens64):
     k, host, dev = gens64
     n, c, nw, K = 8, 8, 3, 128
     table = ops.g1_wide_table_gen(dev[:n].contiguous(), c, nw, K)
-    assert table.numel() * 4 == nw * K * n * 128
+    assert table.numel() * 4 == nw * K * n * 4 * ops.WIDE_ENTRY_WORDS
     pts = br.g1_unpack(host[:n])
     cases = [(0, 1, 0), (0, 128, 7), (1, 1, 3), (1, 77, 2), (2, 128, 5), (2, 2, 0), (0, 65, 1), (1, 64, 6)]
     idx = [(w * K + (kk - 1)) * n + i for (w, kk, i) in cases]
