@@ -110,9 +110,9 @@ __global__ void __launch_bounds__(256) mad_kernel(uint64_t* out, int inner, uint
 
 // Block cache of grape_malloc / grape_free.  The host classes allocate and free a tensor per
 // call as the reference does (cudaMalloc / cudaFree, src/fr-tensor.cu:371-374, :235-241); hipMalloc
-// and hipFree of multi-GiB blocks take from a millisecond to hundreds of them, so a freed block of
-// 1 MiB or more is kept (up to a total that GRAPE_ALLOC_CACHE_GIB sets, 32 GiB by default, 0 = off)
-// and handed out again to a request of exactly its size.  hipFree waits for the device; a caller
+// and hipFree take tens of microseconds for small blocks and from a millisecond to hundreds of them
+// for multi-GiB ones, so a freed block is kept (up to a total that GRAPE_ALLOC_CACHE_GIB sets,
+// 32 GiB by default, 0 = off) and handed out again to a request of exactly its size.  hipFree waits for the device; a caller
 // may rely on that and free a buffer that queued kernels still use, so the wait happens when a
 // cached block is handed out again instead.
 static std::mutex g_alloc_mu;
@@ -211,7 +211,7 @@ int grape_free(void* p) {
     if (it != g_live->end()) {
         const size_t bytes = it->second;
         g_live->erase(it);
-        if (bytes >= ((size_t)1 << 20) && g_cached_bytes + bytes <= alloc_cache_cap()) {
+        if (g_cached_bytes + bytes <= alloc_cache_cap()) {
             g_cached->emplace(bytes, p);
             g_cached_bytes += bytes;
             return GRAPE_OK;

@@ -48,10 +48,10 @@ int grape_stream_sync(grape_stream_t stream);
  * direct cudaMalloc / cudaMemcpy / cudaFree calls, e.g. src/fr-tensor.cu:371-374,322-328). */
 int grape_malloc(void **d_ptr, size_t bytes);
 int grape_free(void *d_ptr);
-/* grape_free keeps blocks of 1 MiB and more for grape_malloc to hand out again (to a request of
- * exactly the same size; up to GRAPE_ALLOC_CACHE_GIB in total, default 32, 0 switches it off): the
- * host classes allocate and free a tensor per call as the reference does, and the driver's
- * allocation calls cost milliseconds at these sizes.  This gives every kept block back to the
+/* grape_free keeps the block for grape_malloc to hand out again (to a request of exactly the same
+ * size; up to GRAPE_ALLOC_CACHE_GIB in total, default 32, 0 switches it off): the host classes
+ * allocate and free a tensor per call as the reference does, and the driver's allocation calls
+ * cost tens of microseconds for small blocks and milliseconds and more for multi-GiB ones.  This gives every kept block back to the
  * driver (it also happens by itself when an allocation fails).  No counterpart in the reference. */
 int grape_alloc_cache_release(size_t *bytes_released);
 int grape_memcpy_h2d(void *d_dst, const void *src, size_t bytes, grape_stream_t stream);
