@@ -123,3 +123,7 @@ void generate_data(int** out_ptr, uint size) {
     check(grape_malloc((void**)out_ptr, sizeof(int) * (size_t)(size ? size : 1)), "grape_malloc");
     if (size) check(grape_memcpy_h2d(*out_ptr, host.data(), sizeof(int) * (size_t)size, nullptr), "grape_memcpy_h2d");
 }
+
+const char* grape_host::device_checkpoint() {
+    return grape_stream_sync(nullptr) == 0 ? "no error" : grape_last_error();
+}

@@ -8,6 +8,8 @@
 // Point files are specific to the curve the library was built for; the BN254 build
 // (-DGRAPE_CURVE_BN254) reads and writes the layout of the reference's own BN254 build.
 #pragma once
+#include <chrono>
+#include <cstdio>
 #include <string>
 
 typedef unsigned int uint;
@@ -26,3 +28,25 @@ uint load_data(const std::string& filename, int** gpu_ptr);
 uint load_data(const std::string& filename, int** gpu_ptr, int** cpu_ptr);
 // `size` uniformly distributed int32 from std::mt19937(123456) into a fresh device buffer
 void generate_data(int** out_ptr, uint size);
+
+// The drivers' timing and checkpoint macros (include/ioutils.cuh:20-48), same names and output
+// lines.  The reference times device work with events on stream 0; every public call of this build
+// has finished its device work when it returns, so here both timer kinds read the host clock after
+// waiting for the device.
+namespace grape_host {
+struct StopWatch {
+    std::chrono::high_resolution_clock::time_point t0 = std::chrono::high_resolution_clock::now();
+    double ms() const { return std::chrono::duration<double, std::milli>(std::chrono::high_resolution_clock::now() - t0).count(); }
+};
+// waits for the device and returns the text of its last error ("no error" when there is none)
+const char* device_checkpoint();
+}  // namespace grape_host
+#define CUDA_DEBUG std::printf("%d %s\n", __LINE__, grape_host::device_checkpoint());
+#define CUDA_TIMER_START(timer_name) \
+    grape_host::device_checkpoint(); \
+    grape_host::StopWatch timer_name##_watch;
+#define CUDA_TIMER_STOP(timer_name)  \
+    grape_host::device_checkpoint(); \
+    std::printf("%s elapsed: %f ms\n", #timer_name, timer_name##_watch.ms());
+#define CPU_TIMER_START(timer_name) grape_host::StopWatch timer_name##_watch;
+#define CPU_TIMER_STOP(timer_name) std::printf("%s elapsed: %f ms\n", #timer_name, timer_name##_watch.ms())

@@ -6,7 +6,8 @@
 // `size /= (4 / layer_num)` becomes layer_num = 1 on a one-block file), the direct launches of the
 // reference's int_to_fr kernel are FrTensor::get_data (the same conversion), and the widths are a
 // small model's (dim 256, feed-forward 1024, 1024 tokens, 1024 x 16 generators; powers of two,
-// because the reference hard-codes its 11008 -> 16384 padding).  Where a reference program ends
+// because the reference hard-codes its 11008 -> 16384 padding).  The programs' CPU_TIMER_* /
+// CUDA_TIMER_* / CUDA_DEBUG macros come from ioutils.hpp.  Where a reference program ends
 // without looking at its result, the function checks the result against a direct evaluation.
 //
 // Arguments: working directory (default /tmp/grape_programs_flow).  Prints "programs_flow OK" when
@@ -122,7 +123,10 @@ static void program_eleWiseMul(const std::string& data, uint layer_num, uint tok
     upSilu.partial_eval(upSilu_size, U, upSilu_size / second_size, Log2(second_size), second_size);
     upSilu.partial_eval(second_size, U, second_size, 0, 1);
     Fr claim = first_element(upSilu);
+    CPU_TIMER_START(prove_eleMul);
     std::pair<Fr, Fr> pr = prove_eleMul(up_out, silu_out, layer_num, tokens, second_size, u, v, claim);
+    CUDA_DEBUG;
+    CPU_TIMER_STOP(prove_eleMul);
 
     // not in the reference program: the returned values are the two factors at v
     require(up_out_kept(v) == pr.first, "eleWiseMul: first factor");
@@ -143,7 +147,10 @@ static void program_combine_value(const std::string& data) {
     Fr claim2 = X(u2);
     X.get_data(size, tensor);
     auto v1 = random_vec(Log2(size));
+    CPU_TIMER_START(combine);
     const Fr merged = combine_claims(X, {claim1, claim2}, {u1, u2}, v1, size);
+    CUDA_DEBUG;
+    CPU_TIMER_STOP(combine);
     // not in the reference program: the merged claim is the tensor at v1
     X.get_data(size, tensor);
     require(X(v1) == merged, "combine_value: merged claim");
@@ -165,7 +172,9 @@ static void program_tlookupTest(const std::string& data, uint layer_num, const a
     x_tensor.get_data(x_size, x_data);
     FrTensor kept(x_tensor);
     auto v = random_vec(Log2(x_size));
+    CUDA_TIMER_START(test);
     const Fr value = rs.prove(x_tensor, tlookup_A, v, hyrax, sh.hidden, com_time);
+    CUDA_TIMER_STOP(test);
     // not in the reference program: the returned value is the witness at v
     require(kept(v) == value, "tlookupTest: returned value");
 
