@@ -319,3 +319,111 @@ Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, cons
     drop_index();
     return ret;
 }
+
+// ------------------------------------------------------------------ round-by-round form
+namespace {
+// coefficient arrays of (X0 + t X1)(Y0 + shift + t Y1) over the two halves of X and Y
+// (tLookup_poly_kernel, src/tlookup.cu:64-81), each evaluated at the remaining variables
+struct PolyArrays {
+    FrTensor c0, c1, c2;
+    explicit PolyArrays(uint n) : c0(n ? n : 1), c1(n ? n : 1), c2(n ? n : 1) {
+        c0.set_size(n);
+        c1.set_size(n);
+        c2.set_size(n);
+    }
+    void products(const FrTensor& X, const FrTensor& Y, const Fr* shift, uint n) {
+        const uint32_t* d_shift = shift ? W(grape_host::device_scalar(*shift)) : nullptr;
+        check(grape_tlookup_poly(W(X.gpu_data), W(Y.gpu_data), d_shift, W(c0.gpu_data), W(c1.gpu_data), W(c2.gpu_data), n, nullptr),
+              "grape_tlookup_poly");
+    }
+    void halves(const FrTensor& X, uint n) {     // c0 = X0, c1 = X1 - X0 (tLookup_poly_sum_kernel, :83-91)
+        check(grape_tlookup_poly_sum(W(X.gpu_data), W(c0.gpu_data), W(c1.gpu_data), n, nullptr), "grape_tlookup_poly_sum");
+    }
+};
+std::vector<Fr> without_last(const std::vector<Fr>& x) { return std::vector<Fr>(x.begin(), x.end() - (x.empty() ? 0 : 1)); }
+}  // namespace
+
+Polynomial tLookup_phase1_step_poly(const Fr& claim, const FrTensor& A, const FrTensor& S, const Fr& alpha, const Fr& beta, const Fr& C,
+                                    const std::vector<Fr>& u) {
+    (void)claim;
+    if (A.size != S.size) throw std::runtime_error("A.size != S.size");
+    if (u.empty()) throw std::runtime_error("tLookup_phase1_step_poly: no variable left");
+    const uint half = A.size >> 1;
+    const std::vector<Fr> rest = without_last(u);
+    PolyArrays w(half);
+    w.products(A, S, &beta, half);
+    Polynomial weighted({w.c0(rest), w.c1(rest), w.c2(rest)});      // the evaluations consume the arrays
+    weighted = weighted * alpha;
+    weighted *= Polynomial::eq(u.back());
+    w.halves(A, half);
+    Polynomial plain({w.c0.sum(half), w.c1.sum(half)});
+    return weighted + plain + Polynomial(C * Fr(2).invert());
+}
+
+Polynomial tLookup_phase2_step_poly(const FrTensor& A, const FrTensor& S, const FrTensor& B, const FrTensor& T, const FrTensor& m,
+                                    const Fr& alpha_, const Fr& beta, const Fr& inv_size_ratio, const Fr& alpha_sq,
+                                    const std::vector<Fr>& u) {
+    if (u.empty()) throw std::runtime_error("tLookup_phase2_step_poly: no variable left");
+    const uint half = m.size >> 1;
+    const std::vector<Fr> rest = without_last(u);
+    PolyArrays w(half);
+    w.products(A, S, &beta, half);
+    Polynomial weighted({w.c0(rest), w.c1(rest), w.c2(rest)});
+    weighted = weighted * alpha_;
+    const Fr coef = inv_size_ratio * alpha_sq;
+    w.products(B, T, &beta, half);
+    weighted += Polynomial({w.c0(rest) * coef, w.c1(rest) * coef, w.c2(rest) * coef});
+    w.halves(A, half);
+    Polynomial plain({w.c0.sum(half), w.c1.sum(half)});
+    w.products(m, B, nullptr, half);
+    Polynomial mb({w.c0.sum(half), w.c1.sum(half), w.c2.sum(half)});
+    return Polynomial::eq(u.back()) * weighted + plain - mb * inv_size_ratio;
+}
+
+Fr tLookup_phase2(const Fr& claim, const FrTensor& A, const FrTensor& S, const FrTensor& B, const FrTensor& T, const FrTensor& m,
+                  const Fr& alpha_, const Fr& beta, const Fr& inv_size_ratio, const Fr& alpha_sq, const std::vector<Fr>& u,
+                  const std::vector<Fr>& v2) {
+    // the reference recurses on fresh half-size tensors; here one set of working copies is bound in place
+    FrTensor a(A), s(S), b(B), t(T), mm(m);
+    Fr running = claim, weight = alpha_, weight_sq = alpha_sq;
+    std::vector<Fr> uu(u), vv(v2);
+    while (!vv.empty()) {
+        const Polynomial p = tLookup_phase2_step_poly(a, s, b, t, mm, weight, beta, inv_size_ratio, weight_sq, uu);
+        if (running != p(0) + p(1)) throw std::runtime_error("tLookup_phase2: claim != p(0) + p(1)");
+        const uint half = a.size >> 1;
+        uint32_t* ptrs[5] = {W(a.gpu_data), W(s.gpu_data), W(b.gpu_data), W(t.gpu_data), W(mm.gpu_data)};
+        check(grape_fr_fold_msb_multi(ptrs, 5, half, W(grape_host::device_scalar(vv.back())), nullptr), "grape_fr_fold_msb_multi");
+        check(grape_stream_sync(nullptr), "sync");
+        for (FrTensor* x : {&a, &s, &b, &t, &mm}) x->set_size(half);
+        running = p(vv.back());
+        const Fr e = Polynomial::eq(uu.back(), vv.back());
+        weight *= e;
+        weight_sq *= e;
+        uu.pop_back();
+        vv.pop_back();
+    }
+    return s(0u);
+}
+
+Fr tLookup_phase1(const Fr& claim, FrTensor& A, FrTensor& S, const FrTensor& B, const FrTensor& T, FrTensor& m, const Fr& alpha,
+                  const Fr& beta, const Fr& C, const Fr& inv_size_ratio, const Fr& alpha_sq, const std::vector<Fr>& u,
+                  const std::vector<Fr>& v1, const std::vector<Fr>& v2) {
+    Fr running = claim, weight = alpha, constant = C;
+    std::vector<Fr> uu(u), vv(v1);
+    const Fr two_inv = Fr(2).invert();
+    while (!vv.empty()) {
+        const Polynomial p = tLookup_phase1_step_poly(running, A, S, weight, beta, constant, uu);
+        if (running != p(0) + p(1)) throw std::runtime_error("tLookup_phase1: claim != p(0) + p(1)");
+        fr_t* d_v = grape_host::device_scalar(vv.back());
+        A.partial_eval(A.size, d_v, 2, 0, A.size >> 1);
+        A.set_size(A.size >> 1);
+        S.partial_eval(S.size, d_v, 2, 0, S.size >> 1);
+        S.set_size(S.size >> 1);
+        running = p(vv.back());
+        weight *= Polynomial::eq(uu.back(), vv.back());
+        constant *= two_inv;
+        uu.pop_back();
+        vv.pop_back();
+    }
+    return tLookup_phase2(running, A, S, B, T, m, weight, beta, inv_size_ratio, alpha_sq, uu, v2);
+}

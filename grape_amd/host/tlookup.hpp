@@ -84,3 +84,21 @@ public:
 private:
     void init_from_host(const int* host_table, uint len);
 };
+
+// The round-by-round form of the logUp sumcheck, as the reference exposes it
+// (include/tlookup.cuh:22-34, src/tlookup.cu:117-244): one round polynomial per call from the
+// coefficient arrays of (A0 + tA1)(S0 + beta + tS1), three multilinear evaluations and two sums;
+// phase 1 binds the variables of D/N with v1 (from the back), phase 2 those of the table with v2.
+// prove() does not go through these (its rounds are fused and queued); they give a caller the
+// reference's own entry points and the tests an unfused restatement to compare with.
+Polynomial tLookup_phase1_step_poly(const Fr& claim, const FrTensor& A, const FrTensor& S, const Fr& alpha, const Fr& beta, const Fr& C,
+                                    const std::vector<Fr>& u);
+Polynomial tLookup_phase2_step_poly(const FrTensor& A, const FrTensor& S, const FrTensor& B, const FrTensor& T, const FrTensor& m,
+                                    const Fr& alpha_, const Fr& beta, const Fr& inv_size_ratio, const Fr& alpha_sq,
+                                    const std::vector<Fr>& u);
+Fr tLookup_phase2(const Fr& claim, const FrTensor& A, const FrTensor& S, const FrTensor& B, const FrTensor& T, const FrTensor& m,
+                  const Fr& alpha_, const Fr& beta, const Fr& inv_size_ratio, const Fr& alpha_sq, const std::vector<Fr>& u,
+                  const std::vector<Fr>& v2);
+Fr tLookup_phase1(const Fr& claim, FrTensor& A, FrTensor& S, const FrTensor& B, const FrTensor& T, FrTensor& m, const Fr& alpha,
+                  const Fr& beta, const Fr& C, const Fr& inv_size_ratio, const Fr& alpha_sq, const std::vector<Fr>& u,
+                  const std::vector<Fr>& v1, const std::vector<Fr>& v2);

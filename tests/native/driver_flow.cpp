@@ -112,6 +112,33 @@ int main(int argc, char** argv) {
         double commit_time = 0.0;
         Fr lookup_value = rs.prove(S, Aux, v2, hyrax, N, commit_time);
         require(lookup_value == S_keep(v2), "lookup value differs from S(v)");
+        // ---- the reference's round-by-round entry points (src/tlookup.cu:117-244) on the same witness,
+        // point and challenges: the same round polynomials and the same returned value as prove()
+        {
+            const uint Nt = rs.T.size;
+            std::vector<Fr> u = random_vec(Log2(D));
+            rs.set_u(u);
+            FrTensor S1(D, d_s), A1(D);
+            const Fr fused_value = rs.prove(S1, A1, v2, hyrax, N, commit_time);
+            const SumcheckTranscript fused = rs.last_transcript;
+            require(fused.rounds.size() == Log2(D), "lookup round count");
+            FrTensor S2(D, d_s), A2(D);
+            A2 = S2;
+            A2 += (int)Nt;                      // beta is the table size (src/tlookup.cu:247)
+            A2.inverse();
+            FrTensor Bm(rs.B);
+            Bm *= rs.m;
+            const Fr alpha_sq = rs.alpha * rs.alpha;
+            const Fr C = alpha_sq - Bm.sum(Nt);
+            const Fr first_claim = rs.alpha + alpha_sq;
+            const Fr N_div_D = Fr((long)Nt) * Fr((long)D).invert();
+            const std::vector<Fr> v_hi(v2.begin() + Log2(Nt), v2.end()), v_lo(v2.begin(), v2.begin() + Log2(Nt));
+            const Polynomial first = tLookup_phase1_step_poly(first_claim, A2, S2, rs.alpha, rs.beta, C, u);
+            require(first.coefficients() == fused.rounds[0].coefficients(), "first round polynomial of the unfused form differs");
+            const Fr unfused_value = tLookup_phase1(first_claim, A2, S2, rs.B, rs.T, rs.m, rs.alpha, rs.beta, C, N_div_D, alpha_sq, u, v_hi, v_lo);
+            require(unfused_value == fused_value, "round-by-round lookup value differs from prove()");
+        }
+
         // a witness with one value outside the range is rejected by the prover's own check
         h_s[5] = 600;
         require(grape_memcpy_h2d(d_s, h_s.data(), sizeof(int) * D, nullptr) == 0, "h2d");
