@@ -195,3 +195,17 @@ std::vector<Fr> FrTensor::to_host() const {
     check(grape_memcpy_d2h(v.data(), gpu_data, sizeof(fr_t) * (size_t)size, nullptr), "grape_memcpy_d2h");
     return v;
 }
+
+void Fr_partial_me(uint N, FrTensor& t, fr_t* x, uint id, uint cur_dim, uint window_size) {
+    if (cur_dim <= 1 || N == 0) return;
+    const size_t dim = (size_t)cur_dim * window_size;
+    if (N % dim != 0) throw std::runtime_error("Fr_partial_me: N is not a multiple of cur_dim * window_size");
+    const uint outer = (uint)(N / dim);
+    FrTensor folded(N);
+    check(grape_memcpy_d2d(folded.gpu_data, t.gpu_data, sizeof(fr_t) * (size_t)N, nullptr), "grape_memcpy_d2d");
+    check(grape_fr_fold(W(folded.gpu_data), N, W(x), cur_dim, id, window_size, nullptr), "grape_fr_fold");
+    for (uint o = 0; o < outer; o++)
+        check(grape_memcpy_d2d(t.gpu_data + (size_t)o * dim, folded.gpu_data + (size_t)o * window_size, sizeof(fr_t) * (size_t)window_size, nullptr),
+              "grape_memcpy_d2d");
+    check(grape_stream_sync(nullptr), "sync");
+}

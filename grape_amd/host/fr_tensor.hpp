@@ -70,3 +70,10 @@ public:
 private:
     uint capacity_;
 };
+
+// The fold WITHOUT the compaction that FrTensor::partial_eval adds (src/fr-tensor.cu:168-188): the
+// first N elements of t are read as [outer][cur_dim][window_size]; the cur_dim axis is bound with
+// x[id], x[id+1], ... and the value of outer index o, inner index g is left at
+// t[o * cur_dim * window_size + g], where the reference's in-place rounds leave it.  The other
+// positions of the tensor, which hold intermediate values in the reference, keep their contents here.
+void Fr_partial_me(uint N, FrTensor& t, fr_t* x, uint id, uint cur_dim, uint window_size);

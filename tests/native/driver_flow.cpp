@@ -151,6 +151,20 @@ int main(int argc, char** argv) {
         }
         require(rejected, "out-of-range witness was not rejected");
 
+        // ---- Fr_partial_me: the fold without compaction leaves value (o, g) at o * c * w + g
+        {
+            const uint c = 6, w = 5, outer = 3, n = outer * c * w;     // an odd tail in the second round
+            FrTensor t = FrTensor::random(n), t2(t);
+            std::vector<Fr> x = random_vec(Log2(c));
+            fr_t* dx = grape_host::upload(x);
+            t2.partial_eval(n, dx, c, 0, w);
+            Fr_partial_me(n, t, dx, 0, c, w);
+            const std::vector<Fr> strided = t.to_host(), compact = t2.to_host();
+            for (uint o = 0; o < outer; o++)
+                for (uint g = 0; g < w; g++) require(strided[o * c * w + g] == compact[o * w + g], "Fr_partial_me position");
+            grape_free(dx);
+        }
+
         grape_free(d_s);
         grape_free(com_int);
         grape_free(com_fr);
