@@ -1,5 +1,5 @@
-// The reference's five single-protocol test programs (test/matmul.cu, test/eleWiseMul.cu,
-// test/combine_value.cu, test/tlookupTest.cu, test/tlookupMapTest.cu), each as one function that keeps
+// The reference's six single-protocol test programs (test/matmul.cu, test/eleWiseMul.cu,
+// test/combine_value.cu, test/tlookupTest.cu, test/tlookupMapTest.cu, test/HyraxTest.cu), each as one function that keeps
 // the program's sequence of calls, run on files in the reference's layouts: the functions read
 // points.bin / cpu_points.bin, table/*.bin and {W,Q,R}/<name>-0.bin with loadbin / load_data as the
 // programs do.  Differences, all forced: the files hold one block instead of four (the programs'
@@ -234,6 +234,67 @@ static void program_tlookupMapTest(const std::string& data, uint layer_num, cons
     grape_free(pp.points);
 }
 
+// test/HyraxTest.cu:16-131, with the verifier's two equations checked on the host exactly as there
+// (host_partial_me over the row commitments, a host-side sum of z_j * G_j, the three-term check
+// on the evaluation) instead of through Hyrax::verify
+static void program_HyraxTest(const std::string& data, uint layer_num, const artefacts::Shape& sh) {
+    const uint N = 64;                                   // 4096 in the reference; rows of N * com_scale
+    const uint com_scale = sh.com_scale;
+    Parameters pp = load_parameters(data, sh.npoints, com_scale);
+    std::vector<bn128>& cpu_points = pp.cpu_points;
+    int* tensor = nullptr;
+    uint size = N * N * 64;
+    generate_data(&tensor, size);
+    Hyrax hyrax(layer_num, sh.npoints, pp.points, cpu_points[0]);
+    FrTensor fr_tensor(size, tensor);
+    FrTensor t1 = FrTensor::random((size / N) * (1 << Log2(N)));
+    CPU_TIMER_START(commit);
+    pad_int(&tensor, N, 1 << Log2(N), (size / N) * (1 << Log2(N)));
+    jacob_t* commitment = hyrax.commit(tensor, (size / N) * (1 << Log2(N)), 1 << Log2(N));
+    CUDA_DEBUG;
+    CPU_TIMER_STOP(commit);
+    CPU_TIMER_START(commit_fr);
+    jacob_t* commitment1 = hyrax.commit(t1, (size / N) * (1 << Log2(N)), 1 << Log2(N));
+    CUDA_DEBUG;
+    CPU_TIMER_STOP(commit_fr);
+
+    std::vector<Fr> eval_point(Log2(size));
+    for (uint i = 0; i < Log2(size); i++) eval_point[i] = Fr::random_element();
+    Fr c = Fr::random_element();
+    CPU_TIMER_START(open);
+    auto proof = hyrax.open(fr_tensor, eval_point, c, size, N);
+    CUDA_DEBUG;
+    CPU_TIMER_STOP(open);
+
+    CPU_TIMER_START(verify);
+    std::vector<bn128> host_commitment(size / N / com_scale);
+    require(grape_memcpy_d2h(host_commitment.data(), commitment, sizeof(jacob_t) * (size / N / com_scale), nullptr) == 0, "d2h");
+    uint start_x = Log2(N * com_scale);
+    std::vector<bn128> layer_C_(layer_num);
+    for (uint i = 0; i < layer_num; i++) {
+        layer_C_[i] = host_partial_me<bn128>(host_commitment.data() + i * (size / com_scale / N / layer_num), size / N / com_scale / layer_num,
+                                             eval_point.begin() + start_x, eval_point.end() - Log2(layer_num));
+    }
+    bn128 C_ = host_partial_me<bn128>(layer_C_.data(), layer_num, eval_point.begin() + Log2(size / layer_num), eval_point.end());
+    bn128 commit_z = bn128::zero();
+    for (uint j = 0; j < (1u << Log2(N)) * com_scale; j++) commit_z = commit_z + proof.z[j] * cpu_points[j];
+    C_ = c * C_;
+    C_ = C_ + proof.commit_d;
+    require(C_ == commit_z, "HyraxTest: c * C + com(d) != com(z)");
+    Fr az = host_partial_me<Fr>(proof.z, (1 << Log2(N)) * com_scale, eval_point.begin(), eval_point.begin() + start_x);
+    bn128 left = (c * proof.result) * cpu_points[0] + proof.commit_ad;
+    bn128 right = az * cpu_points[0];
+    require(left == right, "HyraxTest: c * y * G + com(<a, d>) != <a, z> * G");
+    CPU_TIMER_STOP(verify);
+    // not in the reference program: the opened value is the tensor at the point
+    FrTensor again(size, tensor);
+    require(again(eval_point) == proof.result, "HyraxTest: opened value");
+    grape_free(tensor);
+    grape_free(pp.points);
+    grape_free(commitment);
+    grape_free(commitment1);
+}
+
 int main(int argc, char** argv) {
     const std::string dir = argc > 1 ? argv[1] : "/tmp/grape_programs_flow";
     try {
@@ -256,6 +317,8 @@ int main(int argc, char** argv) {
         lap("tlookupTest");
         program_tlookupMapTest(dir, 1, kShape);
         lap("tlookupMapTest");
+        program_HyraxTest(dir, 1, kShape);
+        lap("HyraxTest");
         std::printf("programs_flow OK: %.1f s\n", std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count());
         return 0;
     } catch (const std::exception& e) {

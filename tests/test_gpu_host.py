@@ -401,8 +401,8 @@ def test_cpp_commit_driver_runs(ops, tmp_path):
 
 
 def test_cpp_reference_programs_run(ops, tmp_path):
-    """the reference's five single-protocol programs (test/matmul.cu, eleWiseMul.cu, combine_value.cu,
-    tlookupTest.cu, tlookupMapTest.cu) as functions of a C++ program that keep their call
+    """the reference's six single-protocol programs (test/matmul.cu, eleWiseMul.cu, combine_value.cu,
+    tlookupTest.cu, tlookupMapTest.cu, HyraxTest.cu) as functions of a C++ program that keep their call
     sequences and read points.bin / cpu_points.bin / table/*.bin / {W,Q,R}/*.bin with loadbin and
     load_data; each result is also checked against a direct evaluation, and the two lookups refuse
     a witness that is off the table"""
