@@ -42,6 +42,10 @@ __global__ void __launch_bounds__(kBlock) zero_words_kernel(uint32_t* p, size_t 
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < words; i += (size_t)gridDim.x * kBlock) p[i] = 0;
 }
 
+__global__ void __launch_bounds__(kBlock) zero_bytes_kernel(uint8_t* p, size_t bytes) {
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < bytes; i += (size_t)gridDim.x * kBlock) p[i] = 0;
+}
+
 int zero_fill(void* d_ptr, size_t bytes, hipStream_t s) {
     if (bytes == 0) return GRAPE_OK;
     if ((bytes & 3) == 0 && (reinterpret_cast<uintptr_t>(d_ptr) & 3) == 0) {
@@ -51,7 +55,10 @@ int zero_fill(void* d_ptr, size_t bytes, hipStream_t s) {
         GRAPE_LAUNCH_CHECK();
         return GRAPE_OK;
     }
-    GRAPE_HIP_CHECK(hipMemsetAsync(d_ptr, 0, bytes, s));   // odd sizes: no caller inside this library
+    // sizes or addresses that are no multiple of 4 (no caller inside this library): byte by byte
+    const size_t want = (bytes + kBlock - 1) / kBlock;
+    zero_bytes_kernel<<<(unsigned)(want < 4096 ? want : 4096), kBlock, 0, s>>>((uint8_t*)d_ptr, bytes);
+    GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
 

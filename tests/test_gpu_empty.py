@@ -112,3 +112,19 @@ def test_freed_blocks_are_handed_out_again_and_released(ops):
     assert released.value == 2 * n + 16
     _capi.check(lib.grape_alloc_cache_release(ctypes.byref(released)))
     assert released.value == 0
+
+
+def test_memset_zero_of_any_size_and_alignment(ops):
+    """grape_memset_zero clears exactly the bytes asked for, also when size or address is no
+    multiple of four (a fill kernel in every case: nothing a captured stream could not replay)"""
+    import ctypes
+    import torch
+    from grape_amd import _capi
+    lib = _capi.load()
+    buf = torch.full((4096,), 0x5a, dtype=torch.uint8, device="cuda")
+    for off, n in ((0, 1024), (1, 7), (3, 1001), (16, 0), (2000, 2096)):
+        buf.fill_(0x5a)
+        _capi.check(lib.grape_memset_zero(ctypes.c_void_p(buf.data_ptr() + off), n, None))
+        torch.cuda.synchronize()
+        h = buf.cpu().numpy()
+        assert not h[off:off + n].any() and (h[:off] == 0x5a).all() and (h[off + n:] == 0x5a).all(), (off, n)
