@@ -84,3 +84,27 @@ def test_commitment_in_several_slabs_and_the_32_bit_size_bound(ops):
         with pytest.raises(GrapeError):
             _capi.check(lib.grape_commit_fr(ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(dW.data_ptr()), size, rowlen,
                                             ctypes.c_void_p(wide_fr.data_ptr()), rowlen, 8, 32, 128, None))
+
+
+def test_commitment_of_2_pow_28_scalars_in_two_full_slabs(ops):
+    """65536 rows of 4096 int16-range scalars (1 GiB of int32, two launches of 32768 rows): rows at
+    the slab boundary and at both ends equal the same rows committed alone, and one of them the
+    big-integer sum"""
+    import torch
+    rowlen, rows = 4096, 65536
+    k = rand_fr(rowlen, 21)
+    dev = ops.g1_make_generators(k)
+    wide = ops.g1_wide_table_gen(dev, 16, 1, 32768)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    W = torch.randint(-32768, 32768, (rows, rowlen), dtype=torch.int32, device="cuda", generator=g)
+    out = ops.commit_i32(W.view(-1), rowlen, wide, rowlen, 16, 1, 32768)
+    assert out.shape[0] == rows
+    for r in (0, 32767, 32768, rows - 1):
+        one = ops.commit_i32(W[r].contiguous(), rowlen, wide, rowlen, 16, 1, 32768)
+        assert torch.equal(one[0], out[r]), r
+    r = 32768
+    want = br.g1_msm([int(v) for v in W[r].cpu().numpy()], br.g1_unpack(ops.g1_to_host(dev)))
+    assert br.g1_unpack(ops.g1_to_host(out[r:r + 1].contiguous()))[0] == want
+    del W, out, wide
+    torch.cuda.empty_cache()
