@@ -259,8 +259,13 @@ def layer_workload(args):
         range_lookup(dr)
         return times["commit_weights"] + times["matmul"] + times["lookup"]
 
-    for _ in range(args.warmup):
-        one_layer()
+    # the first layer of a process also builds the tables tied to the Hyrax object and to every
+    # lookup object (wide fixed-base tables, B[t] * G_i); it is reported as the cold figure
+    cold_s, cold_breakdown = None, None
+    for i in range(args.warmup):
+        t = one_layer()
+        if i == 0:
+            cold_s, cold_breakdown = float(t), {k: float(v) for k, v in times.items()}
     totals = []
     for _ in range(args.steps):
         totals.append(one_layer())
@@ -274,6 +279,7 @@ def layer_workload(args):
                                "FFN 11008, int16 weights/activations" % T,
                    "breakdown_s": {k: float(v) for k, v in times.items()},
                    "step_s": [float(t) for t in totals],
+                   "cold_s": cold_s, "cold_breakdown_s": cold_breakdown,
                    "hbm_free_gib_at_end": torch.cuda.mem_get_info()[0] / 2**30,
                    "n_matmul_sumchecks": counts["matmul"], "n_lookups": counts["lookup"],
                    "weight_points": weight_points,
@@ -562,18 +568,23 @@ def main():
     roofline = {
         "bound": "valu_int32_mul",
         "kernel": "commit_wide_kernel<int32>",
-        "achieved": achieved_alg / 1e12,
+        # multiply-adds the kernel executes (one mixed addition per point), against the issue rate
+        # of that instruction measured in this run
+        "achieved": achieved_exec / 1e12,
         "peak": peak_measured / 1e12,
         "unit": "Tmul/s",
-        "frac": achieved_alg / peak_measured,
+        "frac": achieved_exec / peak_measured,
+        "mads_per_point": EXEC_MULS_PER_POINT,
+        "points_per_launch": points,
         "traffic": COMMIT_KERNEL_TRAFFIC_BYTES if CURVE == "bls12_381" else None,
-        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the 1 GiB copy kernel "
-                          "(FETCH_SIZE unit 2 KiB, WRITE_SIZE unit 1 KiB); algorithmic bytes 2.28e9",
-        "note": "achieved counts the reference algorithm's %d multiplies per point; the kernel executes %d "
-                "(one addition per point instead of two), so frac can exceed 1 - frac_executed is the issue-rate view"
-                % (ALG_MULS_PER_POINT, EXEC_MULS_PER_POINT),
-        "achieved_executed": achieved_exec / 1e12,
-        "frac_executed": achieved_exec / peak_measured,
+        "traffic_source": "recorded, not measured in this run: profiles/commit_wide_kernel_configs1_pmc_traffic.txt "
+                          "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by the 1 GiB copy kernel; "
+                          "FETCH_SIZE unit 2 KiB, WRITE_SIZE unit 1 KiB); algorithmic bytes 2.28e9",
+        # the same launch priced as the reference's algorithm (two byte-window additions per int16
+        # scalar): above the peak because the kernel does one addition per point, not two
+        "reference_algorithm_equiv": {"muls_per_point": ALG_MULS_PER_POINT, "Tmul_per_s": achieved_alg / 1e12,
+                                      "over_peak": achieved_alg / peak_measured},
+        "frac_of_nominal_peak": achieved_exec / PEAK_MULS_NOMINAL,
         "peak_nominal": PEAK_MULS_NOMINAL / 1e12,
         "peak_source": "v_mad_u64_u32 issue-rate microbenchmark measured in this run "
                        "(no published integer-multiply peak exists for MI355X)",
@@ -667,7 +678,10 @@ def layer_in_child():
             return {"value": None, "unit": "s", "error": (res.stderr or res.stdout)[-300:]}
         d = json.loads(lines[-1])
         return {"value": d["value"], "unit": "s", "steps": d["steps"], "warmup": d["warmup"], "workload": d["config"]["workload"],
-                "breakdown_s": d["config"]["breakdown_s"], "step_s": d["config"]["step_s"]}
+                "breakdown_s": d["config"]["breakdown_s"], "step_s": d["config"]["step_s"],
+                "cold_s": d["config"]["cold_s"], "cold_breakdown_s": d["config"]["cold_breakdown_s"],
+                "note": "value = a layer with the one-off tables in place; cold_s = the first layer of the process, "
+                        "which also builds them"}
     except Exception as e:      # a time-out or a missing interpreter: report, do not fail the headline
         return {"value": None, "unit": "s", "error": str(e)[-300:]}
 

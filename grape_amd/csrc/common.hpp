@@ -41,10 +41,11 @@ static inline unsigned blocks_for(size_t n, int per_block = kBlock) {
     return (unsigned)((n + per_block - 1) / per_block);
 }
 
-// Scratch pool: one growing device allocation per slot, reused across calls so the hot path
-// never allocates.  Slots are independent buffers (a call may use several at once).
+// Scratch pool: one growing device allocation per (stream, slot), reused across calls so the hot
+// path never allocates once warm.  Slots are independent buffers (a call may use several at once);
+// the buffer belongs to `stream`: only kernels launched on that stream may touch it.
 enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kSlotWitA = 8, kSlotWitB = 9, kNumSlots = 10 };
-int scratch_get(ScratchSlot slot, size_t bytes, void** out);
+int scratch_get(ScratchSlot slot, size_t bytes, void** out, hipStream_t stream);
 // Zeroes device memory with a small fill kernel (word-sized regions) so that a caller who captures
 // the stream into a graph records a kernel node, not a memset node.
 int zero_fill(void* d_ptr, size_t bytes, hipStream_t s);

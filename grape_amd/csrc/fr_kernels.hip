@@ -375,7 +375,7 @@ static int batch_inverse_impl(uint32_t* out, const uint32_t* in, const uint32_t*
         total += cur;
     }
     void* ws;
-    int rc = scratch_get(kSlotInv, total * 32, &ws);
+    int rc = scratch_get(kSlotInv, total * 32, &ws, s);
     if (rc) return rc;
     uint32_t* lvl[16];
     {
@@ -482,7 +482,7 @@ int grape_fr_sum(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st)
         sum_kernel<<<1, kBlock, 0, s>>>(out, in, n);
     } else {
         void* ws;
-        int rc = scratch_get(kSlotReduce, (size_t)nb * 32, &ws);
+        int rc = scratch_get(kSlotReduce, (size_t)nb * 32, &ws, s);
         if (rc) return rc;
         sum_kernel<<<nb, kBlock, 0, s>>>((uint32_t*)ws, in, n);
         final_sum_kernel<1><<<1, kBlock, 0, s>>>(out, (const uint32_t*)ws, nb);
@@ -588,7 +588,7 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
     const int32_t* wts = nullptr;
     if (plan.npass) {
         void* p;
-        int rc = scratch_get(kSlotFoldW, ((size_t)kFoldMaxPasses * (1u << kFoldMaxBits) + 64) * fr26::N * 4, &p);
+        int rc = scratch_get(kSlotFoldW, ((size_t)kFoldMaxPasses * (1u << kFoldMaxBits) + 64) * fr26::N * 4, &p, s);
         if (rc) return rc;
         profile_begin();
         profile_mark(s);
@@ -604,7 +604,7 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
             if (outer > 1 && src == t) {
                 // reading slabs o*cur_c*gap while writing o*gap would race across workgroups
                 void* p;
-                int rc = scratch_get(kSlotFold, outer * gap * 32 * 2 + 64, &p);
+                int rc = scratch_get(kSlotFold, outer * gap * 32 * 2 + 64, &p, s);
                 if (rc) return rc;
                 dst = (uint32_t*)p;
             }
@@ -625,7 +625,7 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
                 void* p;
                 // two buffers, each large enough for the first pass output
                 size_t each = outer * c_out * gap * 32;
-                int rc = scratch_get(kSlotFold, 2 * each + 64, &p);
+                int rc = scratch_get(kSlotFold, 2 * each + 64, &p, s);
                 if (rc) return rc;
                 ws[0] = (uint32_t*)p;
                 ws[1] = (uint32_t*)((char*)p + each);

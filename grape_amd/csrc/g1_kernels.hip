@@ -684,7 +684,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     if (slab > rows) slab = rows;
     const size_t partial_bytes = slab * nseg * 64 * (size_t)(4 * kPartialWords);
     void* ws;
-    int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws);
+    int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws, s);
     if (rc) return rc;
     int* err = (int*)((char*)ws + partial_bytes);
     rc = zero_fill(err, sizeof(int), s);
@@ -736,7 +736,7 @@ static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint
     if (slab > rows) slab = rows;
     const size_t partial_bytes = slab * nwin * nseg * 64 * (size_t)(4 * kPartialWords);
     void* ws;
-    int rc = scratch_get(kSlotMsm, partial_bytes + slab * nwin * (size_t)(8 * FW) + 64, &ws);
+    int rc = scratch_get(kSlotMsm, partial_bytes + slab * nwin * (size_t)(8 * FW) + 64, &ws, s);
     if (rc) return rc;
     uint32_t* sums = (uint32_t*)((char*)ws + partial_bytes);
     const size_t elem_words = FR ? 8 : 1;
@@ -799,7 +799,7 @@ int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uin
     void* ws;
     const size_t bases_bytes = per_chunk * (8 * FW);
     const size_t tmp_bytes = slab_chunks * CH * per_chunk * (16 * FW);
-    int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes, &ws);
+    int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes, &ws, s);
     if (rc) return rc;
     uint32_t* bases = (uint32_t*)ws;
     uint32_t* tmp = (uint32_t*)((char*)ws + bases_bytes);
@@ -829,7 +829,7 @@ int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len
     if (slab < 1) slab = 1;
     if (slab > len) slab = len;
     void* ws;
-    int rc = scratch_get(kSlotMsm, slab * ncols * (16 * FW) + 64, &ws);
+    int rc = scratch_get(kSlotMsm, slab * ncols * (16 * FW) + 64, &ws, s);
     if (rc) return rc;
     int* err = (int*)((char*)ws + slab * ncols * (16 * FW));
     rc = zero_fill(err, sizeof(int), s);

@@ -426,7 +426,7 @@ static int sumcheck2_impl(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, ui
     if (sums) {
         CHECK_PTR16(sums);
         void* ws;
-        int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws);
+        int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws, s);
         if (rc) return rc;
         partial = (uint32_t*)ws;
     }
@@ -490,7 +490,7 @@ static int hist_lds_from_index(uint32_t* hist, const int32_t* idx, size_t n, uin
     size_t per_chunk = (n + chunks - 1) / chunks;
     per_chunk = (per_chunk + 3) & ~(size_t)3;
     void* partial;
-    int rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial);
+    int rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial, s);
     if (rc) return rc;
     const dim3 grid((unsigned)chunks, ranges);
     if (bins == 32768)
@@ -514,7 +514,7 @@ int grape_tlookup_hist(uint32_t* hist, const uint32_t* vals, size_t n, int32_t l
         return GRAPE_OK;
     }
     void* idx;
-    int rc = scratch_get(kSlotHistIdx, n * 4, &idx);
+    int rc = scratch_get(kSlotHistIdx, n * 4, &idx, s);
     if (rc) return rc;
     index_kernel<<<blocks_for(n), kBlock, 0, s>>>((int32_t*)idx, vals, n, low, len);
     GRAPE_LAUNCH_CHECK();
@@ -542,7 +542,7 @@ int grape_tlookup_inverse_by_table(uint32_t* A, const uint32_t* S, const int32_t
     CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(T); CHECK_PTR16(B);
     hipStream_t s = as_stream(st);
     void* cnt;
-    int rc = scratch_get(kSlotMisc, 64, &cnt);
+    int rc = scratch_get(kSlotMisc, 64, &cnt, s);
     if (rc) return rc;
     rc = zero_fill(cnt, sizeof(unsigned int), s);
     if (rc) return rc;
@@ -597,7 +597,7 @@ int grape_tlookup_round_sums(const uint32_t* A, const uint32_t* S, const uint32_
     hipStream_t s = as_stream(st);
     unsigned nb = reduce_grid(n_out);
     void* ws;
-    int rc = scratch_get(kSlotReduce, (size_t)nb * 5 * 32, &ws);
+    int rc = scratch_get(kSlotReduce, (size_t)nb * 5 * 32, &ws, s);
     if (rc) return rc;
     tl_round_kernel<<<nb, kBlock, 0, s>>>(A, S, beta, eq, n_out, (uint32_t*)ws);
     final_sum_kernel<5><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
@@ -610,7 +610,7 @@ int grape_tlookup_mb_sums(const uint32_t* m, const uint32_t* B, size_t n_out, ui
     hipStream_t s = as_stream(st);
     unsigned nb = reduce_grid(n_out);
     void* ws;
-    int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws);
+    int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws, s);
     if (rc) return rc;
     tl_mb_kernel<<<nb, kBlock, 0, s>>>(m, B, n_out, (uint32_t*)ws);
     final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);

@@ -11,8 +11,6 @@ namespace grape {
 
 static thread_local char g_err[512] = "";
 static bool g_init = false;
-static void* g_scratch[kNumSlots] = {nullptr};
-static size_t g_scratch_bytes[kNumSlots] = {0};
 
 void set_error(const char* fmt, ...) {
     va_list ap;
@@ -64,27 +62,44 @@ int zero_fill(void* d_ptr, size_t bytes, hipStream_t s) {
 
 size_t alloc_cache_release();   // gives the blocks kept by grape_free back to the driver
 
-int scratch_get(ScratchSlot slot, size_t bytes, void** out) {
-    if (bytes > g_scratch_bytes[slot]) {
-        if (g_scratch[slot]) {
-            GRAPE_HIP_CHECK(hipDeviceSynchronize());
-            GRAPE_HIP_CHECK(hipFree(g_scratch[slot]));
-            g_scratch[slot] = nullptr;
-            g_scratch_bytes[slot] = 0;
+// One pool per stream: a buffer is only ever used by kernels of the stream it was handed out for,
+// so calls on different streams (from one host thread or from several) never share scratch
+// memory, and growing a buffer only has to wait for its own stream.  The bookkeeping is behind a
+// mutex; one host thread per stream stays the rule (two threads that interleave calls on the SAME
+// stream would still share its buffers).
+struct StreamPool {
+    void* ptr[kNumSlots] = {nullptr};
+    size_t bytes[kNumSlots] = {0};
+};
+static std::mutex g_scratch_mu;
+static std::map<hipStream_t, StreamPool>* g_pools = nullptr;
+
+int scratch_get(ScratchSlot slot, size_t bytes, void** out, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_pools) g_pools = new std::map<hipStream_t, StreamPool>();
+    StreamPool& pool = (*g_pools)[stream];
+    if (bytes > pool.bytes[slot]) {
+        if (pool.ptr[slot]) {
+            GRAPE_HIP_CHECK(hipStreamSynchronize(stream));
+            GRAPE_HIP_CHECK(hipFree(pool.ptr[slot]));
+            pool.ptr[slot] = nullptr;
+            pool.bytes[slot] = 0;
         }
         size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
-        hipError_t e = hipMalloc(&g_scratch[slot], want);
+        hipError_t e = hipMalloc(&pool.ptr[slot], want);
         if (e != hipSuccess && alloc_cache_release() > 0) {
             (void)hipGetLastError();
-            e = hipMalloc(&g_scratch[slot], want);
+            e = hipMalloc(&pool.ptr[slot], want);
         }
         if (e != hipSuccess) {
+            (void)hipGetLastError();
+            pool.ptr[slot] = nullptr;
             set_error("scratch allocation of %zu bytes failed: %s", want, hipGetErrorString(e));
             return GRAPE_ENOMEM;
         }
-        g_scratch_bytes[slot] = want;
+        pool.bytes[slot] = want;
     }
-    *out = g_scratch[slot];
+    *out = pool.ptr[slot];
     return GRAPE_OK;
 }
 
@@ -317,7 +332,7 @@ int grape_bench_copy(void* d_dst, const void* d_src, size_t bytes, int iters, fl
 int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double* mads_per_s, grape_stream_t st) {
     GRAPE_REQUIRE(blocks > 0 && inner > 0 && iters > 0 && mads_per_s, "bad arguments");
     void* out;
-    int rc = scratch_get(kSlotMisc, 64, &out);
+    int rc = scratch_get(kSlotMisc, 64, &out, as_stream(st));
     if (rc) return rc;
     hipEvent_t e0, e1;
     GRAPE_HIP_CHECK(hipEventCreate(&e0));

@@ -583,7 +583,7 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
     const uint32_t Kp = (K + kMfK - 1) / kMfK * kMfK;
     if (g_matmul_method != 1 && L == 1 && aligned && (g_matmul_method == 2 || (uint64_t)N * M * K >= ((uint64_t)1 << 26))) {
         void* mx;
-        rc = scratch_get(kSlotMisc, 64, &mx);
+        rc = scratch_get(kSlotMisc, 64, &mx, s);
         if (rc) return rc;
         uint32_t* d_mx = (uint32_t*)mx;
         wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx);
@@ -611,9 +611,9 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
     }
     if (use_mfma) {
         void *pa, *pb;
-        rc = scratch_get(kSlotWitA, (size_t)PA * N * Kp, &pa);
+        rc = scratch_get(kSlotWitA, (size_t)PA * N * Kp, &pa, s);
         if (rc) return rc;
-        rc = scratch_get(kSlotWitB, (size_t)PB * M * Kp, &pb);
+        rc = scratch_get(kSlotWitB, (size_t)PB * M * Kp, &pb, s);
         if (rc) return rc;
         wit_split_kernel<<<blocks_for((size_t)N * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pa, d_a, N, K, Kp, PA);
         wit_split_kernel<<<blocks_for((size_t)M * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pb, d_b, M, K, Kp, PB);

@@ -6,7 +6,8 @@ using grape_host::check;
 
 std::vector<bn128> precompute_generators(uint N, uint W, affine_t* out) {
     grape_host::ensure_init();
-    // scalars on the host (seeded), points on the device
+    // scalars on the host, points on the device; the scalars (the generators' discrete logarithms,
+    // which would break the binding of every commitment) are wiped on both sides once used
     std::vector<uint32_t> k(8 * (size_t)N);
     for (uint i = 0; i < N; i++) Fr::random_element().to_plain(&k[8 * (size_t)i]);
     uint32_t* d_k = nullptr;
@@ -23,6 +24,12 @@ std::vector<bn128> precompute_generators(uint N, uint W, affine_t* out) {
     check(grape_g1_table_gen(reinterpret_cast<uint32_t*>(out), reinterpret_cast<uint32_t*>(d_gens), N, W, nullptr), "grape_g1_table_gen");
     std::vector<affine_t> host(N);
     check(grape_memcpy_d2h(host.data(), d_gens, sizeof(affine_t) * (size_t)N, nullptr), "d2h");
+    check(grape_memset_zero(d_k, 32 * (size_t)N, nullptr), "grape_memset_zero");
+    check(grape_stream_sync(nullptr), "sync");
+    {
+        volatile uint32_t* w = k.data();
+        for (size_t i = 0; i < k.size(); i++) w[i] = 0;
+    }
     grape_free(d_k);
     grape_free(d_base);
     grape_free(d_gens);

@@ -5,7 +5,8 @@
 #include "fr.hpp"
 #include "fr_tensor.hpp"
 
-// N seeded generators (random scalars times the standard generator, derived on the GPU) and the
+// N generators (scalars from Fr::random_element times the standard generator, derived on the GPU;
+// the scalars are wiped afterwards) and the
 // reference-format table out[w*N + i] = w*G_i, w < W, on the device
 // (precompute_generators + naive_msm, src/ec_operation.cu:15-49).  `out` is device memory for
 // W*N affine points.

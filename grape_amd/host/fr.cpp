@@ -1,8 +1,13 @@
 #include "fr.hpp"
-#include <ostream>
+#include <errno.h>
+#include <sys/random.h>
 #include <iomanip>
+#include <mutex>
+#include <ostream>
+#include <stdexcept>
 
 namespace {
+// Deterministic generator of the opt-in seeded mode (tests, benchmarks): xoshiro256**.
 struct Xoshiro {
     uint64_t s[4];
     static uint64_t splitmix(uint64_t& x) {
@@ -19,9 +24,43 @@ struct Xoshiro {
         return r;
     }
 };
-Xoshiro& rng() {
-    static Xoshiro g = [] { Xoshiro x; x.seed(0x47524150452d4d49ull); return x; }();
-    return g;
+// The random source of Fr::random_element.  By default every draw comes from the operating
+// system's generator (getrandom(2), the source behind libff's std::random_device draws,
+// src/ec_operation.cu:35,55): blinding rows, challenges and generator scalars are unpredictable and
+// never repeat between processes.  Fr::seed(s) switches the whole process to a reproducible stream
+// (one generator behind a mutex, so OpenMP callers stay safe, though their interleaving is not
+// reproducible); Fr::seed_from_os() switches back.
+std::mutex g_rng_mu;
+bool g_seeded = false;
+Xoshiro g_xo;
+
+// 64 random bits from the OS, buffered per thread
+uint64_t os_random64() {
+    thread_local uint64_t buf[64];
+    thread_local size_t have = 0;
+    if (have == 0) {
+        size_t got = 0;
+        unsigned char* p = reinterpret_cast<unsigned char*>(buf);
+        while (got < sizeof buf) {
+            ssize_t n = getrandom(p + got, sizeof buf - got, 0);
+            if (n < 0) {
+                if (errno == EINTR) continue;
+                throw std::runtime_error("Fr::random_element: getrandom failed");
+            }
+            got += (size_t)n;
+        }
+        have = 64;
+    }
+    const uint64_t w = buf[--have];
+    buf[have] = 0;                       // a word is handed out once and not kept
+    return w;
+}
+uint64_t next64() {
+    {
+        std::lock_guard<std::mutex> lock(g_rng_mu);
+        if (g_seeded) return g_xo.next();
+    }
+    return os_random64();
 }
 bool below_modulus(const uint32_t* a) {
     for (int i = 7; i >= 0; i--) {
@@ -42,13 +81,25 @@ Fr::Fr(long x) {
     if (x < 0) v = grape::neg(v);
 }
 
-void Fr::seed(uint64_t s) { rng().seed(s); }
+void Fr::seed(uint64_t s) {
+    std::lock_guard<std::mutex> lock(g_rng_mu);
+    g_xo.seed(s);
+    g_seeded = true;
+}
+void Fr::seed_from_os() {
+    std::lock_guard<std::mutex> lock(g_rng_mu);
+    g_seeded = false;
+}
+bool Fr::seeded() {
+    std::lock_guard<std::mutex> lock(g_rng_mu);
+    return g_seeded;
+}
 
 Fr Fr::random_element() {
     for (;;) {
         fr_t raw;
         for (int i = 0; i < 4; i++) {
-            uint64_t w = rng().next();
+            uint64_t w = next64();
             raw.v[2 * i] = (uint32_t)w;
             raw.v[2 * i + 1] = (uint32_t)(w >> 32);
         }

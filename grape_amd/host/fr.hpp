@@ -27,10 +27,16 @@ public:
 
     static Fr zero() { return Fr(); }
     static Fr one() { return Fr(grape::Fr::one()); }
-    // Seeded replacement of libff's unseeded random_element (src/ec_operation.cu:55):
-    // xoshiro256** streams, rejection-sampled 255-bit draws.
+    // Uniform element by rejection sampling of 255-bit draws.  The bits come from the operating
+    // system's generator (getrandom), as libff's random_element draws from std::random_device
+    // (src/ec_operation.cu:35,55), unless seed() has put the process into its reproducible mode
+    // (a xoshiro256** stream behind a mutex) - for tests and benchmarks only: with a known seed the
+    // blinding row of Hyrax::open, the lookups' alpha and r and the generator scalars are all
+    // predictable.  seed_from_os() returns to the default.  Safe to call from several threads.
     static Fr random_element();
     static void seed(uint64_t s);
+    static void seed_from_os();
+    static bool seeded();
 
     bool is_zero() const { return v.is_zero(); }
     Fr& invert();                       // in place, 1/0 = 0; returns *this like libff
@@ -64,7 +70,7 @@ public:
 
     static G1 zero() { return G1(); }
     static G1 one();                     // the standard generator
-    static G1 random_element();          // random scalar times the generator (seeded, see Fr::seed)
+    static G1 random_element();          // random scalar times the generator (see Fr::random_element)
 
     bool is_zero() const { return p.is_inf(); }
     affine_t to_affine() const;

@@ -19,8 +19,10 @@ void ensure_init() {
 
 static constexpr int kSlots = 64;
 fr_t* device_scalar(const Fr& x) {
-    static fr_t* ring = nullptr;
-    static int next = 0;
+    // one ring per host thread: a slot is rewritten after kSlots further calls of the same thread,
+    // never by another thread
+    thread_local fr_t* ring = nullptr;
+    thread_local int next = 0;
     ensure_init();
     if (!ring) check(grape_malloc((void**)&ring, sizeof(fr_t) * kSlots), "grape_malloc");
     fr_t* slot = ring + next;

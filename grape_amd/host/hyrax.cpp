@@ -226,6 +226,7 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     uint pad_N = 1u << Log2(N);
     uint new_N = pad_N * com_scale;
     assert(eval_point_.size() == Log2(size));
+    last_open_point_ = eval_point_;
     fr_t* eval_point = grape_host::upload(eval_point_);
 
     std::vector<Fr> host_d(new_N);
@@ -302,4 +303,9 @@ bool Hyrax::verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr
     std::vector<Fr> inner_point(eval_point.begin(), eval_point.begin() + inner);
     Fr az = z(inner_point);
     return (c * proof.result) * G + proof.commit_ad == az * G;
+}
+
+void Hyrax::verify(Hyrax_proof& proof, jacob_t* commitment, Fr c, uint size, uint N) {
+    if (last_open_point_.size() != Log2(size)) throw std::runtime_error("Hyrax::verify: no opening of this size was made by this object");
+    if (!verify(proof, commitment, last_open_point_, c, size, N)) throw std::runtime_error("Hyrax::verify: the opening does not match the commitment");
 }

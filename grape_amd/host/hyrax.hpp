@@ -50,6 +50,11 @@ public:
     // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
     // the reference's own verify is an empty stub (src/Hyrax.cu:307-310).
     bool verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
+    // The reference's signature (include/Hyrax.cuh:85), so that its call sites compile unchanged.  It
+    // carries no evaluation point: the point of this object's most recent open() is used, and a
+    // failed check (or a call before any open) throws std::runtime_error where the reference's
+    // empty body returns silently.
+    void verify(Hyrax_proof& proof, jacob_t* commitment, Fr c, uint size, uint N);
 
     // Scaled table out[t*ncols + i] = scalars[t] * G_i over the first ncols generators (device,
     // owned by the caller, freed with grape_free); nullptr when it would not fit the budget.
@@ -76,5 +81,6 @@ private:
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
     bool int16_ok_ = true;
     size_t scaled_bytes_ = 0;
+    std::vector<Fr> last_open_point_;
     size_t table_budget_ = (size_t)128 << 30;
 };

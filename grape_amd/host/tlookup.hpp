@@ -18,7 +18,7 @@ public:
     tLookup(const uint size);
 
     // The reference draws the prover's point u inside prove() from an unseeded generator
-    // (src/tlookup.cu:293); by default it comes from the seeded generator of Fr::random_element,
+    // (src/tlookup.cu:293); by default it comes from Fr::random_element (the OS generator unless seeded),
     // and a caller that needs a reproducible transcript can fix it here (consumed by the next prove).
     void set_u(const std::vector<Fr>& u) { forced_u_ = u; }
     // Round polynomials of the most recent prove (the reference keeps none).

@@ -20,8 +20,14 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Kernels are only
  *     enqueued; results are ready after grape_stream_sync(stream).  Functions that return a value
  *     to the host say so and synchronise the stream themselves;
- *   - one host thread per stream; calls on the same device share an internal scratch pool, so
- *     calls issued from different host threads must not overlap.
+ *   - one host thread per stream.  Internal scratch memory (partial sums, fold buffers, MSM
+ *     partials) is pooled per stream, so calls on DIFFERENT streams - from one host thread or from
+ *     several - never share it and may overlap; calls on the same stream are ordered by the
+ *     stream.  A buffer of the pool grows on demand (hipMalloc after waiting for its stream), so a
+ *     caller who captures a stream into a graph runs each shape once before capturing;
+ *   - grape_free does NOT wait for the device the way cudaFree / hipFree do: it only hands the block
+ *     to the allocation cache described below, and the wait happens when that block is handed out
+ *     again.  A caller that relied on cudaFree as a synchronisation point calls grape_stream_sync.
  */
 #ifndef GRAPE_HIP_H
 #define GRAPE_HIP_H

@@ -79,6 +79,18 @@ int main(int argc, char** argv) {
         FrTensor copy1(fr_tensor), copy2(fr_tensor);
         Hyrax_proof proof = hyrax.open(copy1, eval_point, c, size, N);
         require(hyrax.verify(proof, com_fr, eval_point, c, size, N), "opening does not verify");
+        hyrax.verify(proof, com_fr, c, size, N);          // the reference's signature (include/Hyrax.cuh:85): throws on a mismatch
+        {
+            Hyrax_proof forged(proof);
+            forged.result += Fr::one();
+            bool refused = false;
+            try {
+                hyrax.verify(forged, com_fr, c, size, N);
+            } catch (const std::runtime_error&) {
+                refused = true;
+            }
+            require(refused, "a forged opening passed the reference-signature verify");
+        }
         require(proof.result == copy2(eval_point), "opened value differs from the multilinear extension");
 
         // ---- matmul sumcheck (the pattern of test/llm.cu): Y[n][m] = sum_k A[n][k] B[m][k]

@@ -102,8 +102,6 @@ def test_mle_eval_operator(ops, host):
 @pytest.mark.parametrize("logD,logN,low", [(4, 2, -2), (5, 3, -4), (3, 3, 0), (12, 6, -32), (14, 8, -128), (16, 16, -32768)])
 def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed):
     import torch
-    if logN == 16 and indexed:
-        pytest.skip("the 2^16-entry scaled table is exercised by the full-size run")
     host.set_indexed_commit(indexed)
     hg, dg = gens
     D, N = 1 << logD, 1 << logN
@@ -119,19 +117,24 @@ def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed
     table = ops.g1_table_gen(dg, 256)               # 256 generators: com(m) uses rows of 2^(logN/2)
     dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
     msm = min(D, 16)
-    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 256, 1, msm, want_commitments=(logD <= 5))
+    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 256, 1, msm, want_commitments=True)
     assert_same(res["m"], m, "multiplicities")
     assert_same(res["transcript"], wtr, "transcript")
     assert_same(res["S_claim"], wsc, "S(v)")
     assert br.fr_unpack(res["m"]) == [int(x) for x in np.bincount(S.astype(np.int64) - low, minlength=N)]
     host.set_indexed_commit(True)
-    if logD <= 5:
-        # the commitments of A = 1/(S+beta) and of m made inside prove
-        Ainv = orc.vec1("orc_fr_vec_inv", orc.vec_bcast("orc_fr_vec_bcast_add", Sp, beta))
-        tab = orc.g1_table(hg, 256)
-        assert_same(res["com_A"], orc.commit_fr(Ainv, tab, msm, 256), "com(A)")
-        mN = 1 << (logN // 2)
-        assert_same(res["com_m"], orc.commit_fr(m, tab, mN, 256), "com(m)")
+    # the commitments of A = 1/(S+beta) and of m made inside prove (through the scaled table
+    # B[t] * G_i and the indexed commitment when `indexed`): every row up to 64 rows, else the two
+    # ends, the middle and a seeded sample
+    Ainv = orc.vec1("orc_fr_vec_inv", orc.vec_bcast("orc_fr_vec_bcast_add", Sp, beta))
+    tab = orc.g1_table(hg, 256)
+    nrows = D // msm
+    assert res["com_A"].shape[0] == nrows
+    rows = list(range(nrows)) if nrows <= 64 else sorted({0, 1, nrows // 2, nrows - 2, nrows - 1} | set(rng.integers(0, nrows, 24).tolist()))
+    for r in rows:
+        assert_same(res["com_A"][r:r + 1], orc.commit_fr(Ainv[r * msm:(r + 1) * msm], tab, msm, 256), "com(A) row %d" % r)
+    mN = 1 << (logN // 2)
+    assert_same(res["com_m"], orc.commit_fr(m, tab, mN, 256), "com(m)")
 
 
 def test_tlookup_range_rejects_out_of_range(ops, host, gens):
@@ -369,8 +372,9 @@ def test_cpp_driver_runs(ops, tmp_path):
     assert "driver_flow OK" in res.stdout
 
 
-def test_cpp_layer_driver_runs(ops, tmp_path):
-    """one transformer block (1024 tokens, d_model 4096, FFN 11008) proved in the order of the
+@pytest.mark.parametrize("tokens", ["2048"])
+def test_cpp_layer_driver_runs(ops, tmp_path, tokens):
+    """one transformer block (2048 tokens, d_model 4096, FFN 11008) proved in the order of the
     reference's layer driver (test/llm.cu:73-611) by a C++ program against the host classes, on the
     witness of the library's own generator: 37 chained steps (openings, range and mapping lookups,
     matmul / element-product sumchecks, combine_claims), every one of the reference's assertions
@@ -380,7 +384,7 @@ def test_cpp_layer_driver_runs(ops, tmp_path):
     import driver_build
     exe = driver_build.build(None, "layer_flow")
     torch.cuda.empty_cache()
-    res = subprocess.run([exe, "1024", str(tmp_path)], capture_output=True, text=True, timeout=280)
+    res = subprocess.run([exe, tokens, str(tmp_path)], capture_output=True, text=True, timeout=280)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
     assert "layer_flow OK: 37 steps" in res.stdout
 
