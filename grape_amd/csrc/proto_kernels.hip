@@ -1,6 +1,7 @@
 // Protocol kernels: fused sumcheck rounds (prove.cu) and the logUp / tlookup kernels (tlookup.cu).
 // Every round kernel streams its operands once and leaves per-workgroup partial sums that a
 // one-block kernel finishes; nothing here allocates.
+#include <mutex>
 #include "fr_device.hpp"
 
 namespace grape {
@@ -408,6 +409,42 @@ static unsigned reduce_grid(size_t n) {
     return need > cap ? need : cap;
 }
 
+// ---------------------------------------------------------------- entry point that allocates nothing
+// Partial sums of grape_sumcheck_round2_noalloc: a fixed array in the code object instead of a
+// pool buffer, sized for the largest round that entry point accepts (kNoAllocMaxOut output indices
+// -> at most kNoAllocMaxBlocks workgroups leaving three 32-byte sums each: 1.5 MiB per GPU, held
+// until the process ends).  Host code never uses this name as an address: it asks the runtime for
+// the array's device address once per device (noalloc_scratch) and passes that to the kernels.
+constexpr uint32_t kNoAllocMaxOut = 1u << 26;
+constexpr unsigned kNoAllocMaxBlocks = kNoAllocMaxOut / (kBlock * kRoundIters);
+static __device__ __align__(256) uint32_t scratch[(size_t)kNoAllocMaxBlocks * 3 * 8];
+
+constexpr int kMaxDevices = 64;
+static uint32_t* g_noalloc_ptr[kMaxDevices] = {nullptr};
+static std::mutex g_noalloc_mu;
+
+// device address of `scratch` on the current device (looked up once per device)
+static int noalloc_scratch(uint32_t** out) {
+    int dev = -1;
+    GRAPE_HIP_CHECK(hipGetDevice(&dev));
+    GRAPE_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_noalloc_mu);
+    if (!g_noalloc_ptr[dev]) {
+        void* p = nullptr;
+        GRAPE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        GRAPE_REQUIRE(p != nullptr, "no device address for the static scratch array");
+        g_noalloc_ptr[dev] = (uint32_t*)p;
+    }
+    *out = g_noalloc_ptr[dev];
+    return GRAPE_OK;
+}
+// called by grape_init with its device current, so that the entry point's first call finds the
+// address already there
+int noalloc_setup() {
+    uint32_t* p;
+    return noalloc_scratch(&p);
+}
+
 }  // namespace grape
 
 using namespace grape;
@@ -454,6 +491,28 @@ int grape_sumcheck_round2_tail(uint32_t* A, uint32_t* B, uint32_t in_size, uint3
 int grape_sumcheck_round2(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {
     GRAPE_REQUIRE(sums != nullptr, "d_sums is required");
     return sumcheck2_impl<false>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, sums, st);
+}
+int grape_sumcheck_round2_noalloc(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums,
+                                  grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(B); CHECK_PTR16(v); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * out_size, "need out_size <= in_size <= 2*out_size");
+    if (out_size > kNoAllocMaxOut) {
+        set_error("grape_sumcheck_round2_noalloc: out_size %u exceeds the limit of %u output indices of the static scratch array "
+                  "(use grape_sumcheck_round2)", out_size, kNoAllocMaxOut);
+        return GRAPE_EINVAL;
+    }
+    uint32_t* partial = nullptr;
+    int rc = noalloc_scratch(&partial);
+    if (rc) return rc;
+    hipStream_t s = as_stream(st);
+    const unsigned nb = reduce_grid(out_size);            // <= kNoAllocMaxBlocks for out_size <= kNoAllocMaxOut
+    GRAPE_REQUIRE(nb <= kNoAllocMaxBlocks, "grid exceeds the static scratch array");
+    // every workgroup writes its three partial sums and the finishing kernel reads exactly those, so
+    // nothing of the previous call's contents is read and nothing has to be cleared
+    sumcheck2_kernel<false><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, partial);
+    final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
 }
 int grape_sumcheck_round2_coeffs(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, uint32_t* c, uint32_t in_size,
                                  uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {

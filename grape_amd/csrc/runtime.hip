@@ -61,6 +61,7 @@ int zero_fill(void* d_ptr, size_t bytes, hipStream_t s) {
 }
 
 size_t alloc_cache_release();   // gives the blocks kept by grape_free back to the driver
+int noalloc_setup();            // proto_kernels.hip: looks up the static scratch array of the current device
 
 // One pool per stream: a buffer is only ever used by kernels of the stream it was handed out for,
 // so calls on different streams (from one host thread or from several) never share scratch
@@ -190,7 +191,7 @@ int grape_init(int device) {
         return GRAPE_EINVAL;
     }
     g_init = true;
-    return GRAPE_OK;
+    return noalloc_setup();
 }
 const char* grape_last_error(void) { return g_err; }
 int grape_stream_sync(grape_stream_t s) {

@@ -119,6 +119,16 @@ int grape_fr_fold(uint32_t *d_t, size_t N, const uint32_t *d_x, uint32_t c, uint
  */
 int grape_sumcheck_round2(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size,
                           const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
+/* The same round for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * results as grape_sumcheck_round2, but the per-workgroup partial sums go to a fixed 1.5 MiB array
+ * inside the library's code object instead of the growing scratch pool, so the call never calls
+ * hipMalloc / hipFree; out_size is limited to 2^26 indices (GRAPE_EINVAL beyond).  grape_init looks the
+ * array's address up for its device (a call on a device grape_init has not seen does so itself on
+ * first use).  Every call on one GPU shares that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe. */
+int grape_sumcheck_round2_noalloc(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size,
+                                  const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
 /* The last rounds of the same sumcheck in one launch (one workgroup, a barrier between rounds):
  * `rounds` successive rounds starting from in_size <= 512 elements, out_size = 2^(ceil(log2 in_size) - 1)
  * and halving from there; round i takes its challenge from d_v_end[-(i+1)] (the reference walks
