@@ -55,6 +55,11 @@ SIGNATURES = {
     "grape_sumcheck_round2_tail": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_coeffs": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round1": [c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p],
+    "grape_eq_pyramid_elems": [c_u32],
+    "grape_eq_pyramid": [c_void_p, c_void_p, c_u32, c_void_p],
+    "grape_wround2": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_u32, c_u32, c_void_p, c_int, c_void_p, c_void_p],
+    "grape_sumcheck_round2_seg": [c_void_p, c_void_p, c_u32, c_u32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
+    "grape_wsum1_multi": [c_void_p, ctypes.POINTER(c_void_p), c_u32, c_u32, c_u32, c_void_p, c_void_p],
     "grape_tlookup_hist": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
     "grape_tlookup_index": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
     "grape_tlookup_hist_index": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p],
@@ -99,7 +104,7 @@ SIGNATURES = {
     "grape_event_record": [c_void_p, c_void_p],
     "grape_event_elapsed_ms": [ctypes.POINTER(ctypes.c_float), c_void_p, c_void_p],
 }
-_RESTYPES = {"grape_last_error": ctypes.c_char_p, "grape_g1_wide_table_bytes": c_size_t}
+_RESTYPES = {"grape_last_error": ctypes.c_char_p, "grape_g1_wide_table_bytes": c_size_t, "grape_eq_pyramid_elems": c_size_t}
 
 _lib = None
 

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgrape_hip.so")
-SOURCES = ["runtime.hip", "fr_kernels.hip", "proto_kernels.hip", "g1_kernels.hip", "witness_kernels.hip"]
+SOURCES = ["runtime.hip", "fr_kernels.hip", "proto_kernels.hip", "round_kernels.hip", "g1_kernels.hip", "witness_kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-std=c++17", "-O3", "--offload-arch=gfx950", "-fPIC",
          # packed-FP32 instruction forms are kept out of every device code object

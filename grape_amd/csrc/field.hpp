@@ -185,18 +185,42 @@ struct alignas(16) Mont {
 
 namespace detail {
 
+// One word of a carry / borrow chain (carry and borrow are 0 or 1).  With clang the builtins become
+// one add-with-carry / subtract-with-borrow instruction per word on the device (64-bit emulation of
+// the chain costs three to four times as many instructions there); other compilers spell it out.
+GRAPE_HD uint32_t adc32(uint32_t a, uint32_t b, uint32_t& carry) {
+#if defined(__clang__)
+    unsigned int out;
+    const uint32_t r = __builtin_addc(a, b, carry, &out);
+    carry = out;
+    return r;
+#else
+    const uint64_t t = (uint64_t)a + b + carry;
+    carry = (uint32_t)(t >> 32);
+    return (uint32_t)t;
+#endif
+}
+GRAPE_HD uint32_t sbb32(uint32_t a, uint32_t b, uint32_t& borrow) {
+#if defined(__clang__)
+    unsigned int out;
+    const uint32_t r = __builtin_subc(a, b, borrow, &out);
+    borrow = out;
+    return r;
+#else
+    const uint64_t t = (uint64_t)a - b - borrow;
+    borrow = (uint32_t)(t >> 32) & 1u;
+    return (uint32_t)t;
+#endif
+}
+
 // r = a - mod if a >= mod else a (a < 2*mod assumed, carry_in is the bit above limb N-1).
 template <class P>
 GRAPE_HD void final_sub(uint32_t* r, const uint32_t* a, uint32_t carry_in) {
     constexpr int N = P::N;
     uint32_t d[N];
-    uint64_t borrow = 0;
+    uint32_t borrow = 0;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-        uint64_t s = (uint64_t)a[i] - P::mod(i) - borrow;
-        d[i] = (uint32_t)s;
-        borrow = (s >> 32) & 1u;
-    }
+    for (int i = 0; i < N; i++) d[i] = sbb32(a[i], P::mod(i), borrow);
     // a >= mod  <=>  no final borrow, or the overflow bit was set
     bool ge = (borrow == 0) | (carry_in != 0);
 #pragma unroll
@@ -209,15 +233,11 @@ template <class P>
 GRAPE_HD Mont<P> add(const Mont<P>& a, const Mont<P>& b) {
     constexpr int N = P::N;
     uint32_t s[N];
-    uint64_t c = 0;
+    uint32_t c = 0;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-        uint64_t t = (uint64_t)a.v[i] + b.v[i] + c;
-        s[i] = (uint32_t)t;
-        c = t >> 32;
-    }
+    for (int i = 0; i < N; i++) s[i] = detail::adc32(a.v[i], b.v[i], c);
     Mont<P> r;
-    detail::final_sub<P>(r.v, s, (uint32_t)c);
+    detail::final_sub<P>(r.v, s, c);
     return r;
 }
 
@@ -225,23 +245,15 @@ template <class P>
 GRAPE_HD Mont<P> sub(const Mont<P>& a, const Mont<P>& b) {
     constexpr int N = P::N;
     uint32_t d[N];
-    uint64_t borrow = 0;
+    uint32_t borrow = 0;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-        uint64_t t = (uint64_t)a.v[i] - b.v[i] - borrow;
-        d[i] = (uint32_t)t;
-        borrow = (t >> 32) & 1u;
-    }
+    for (int i = 0; i < N; i++) d[i] = detail::sbb32(a.v[i], b.v[i], borrow);
     // add the modulus back when the subtraction wrapped
-    uint32_t mask = (uint32_t)0 - (uint32_t)borrow;
+    const uint32_t mask = (uint32_t)0 - borrow;
     Mont<P> r;
-    uint64_t c = 0;
+    uint32_t c = 0;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-        uint64_t t = (uint64_t)d[i] + (P::mod(i) & mask) + c;
-        r.v[i] = (uint32_t)t;
-        c = t >> 32;
-    }
+    for (int i = 0; i < N; i++) r.v[i] = detail::adc32(d[i], P::mod(i) & mask, c);
     return r;
 }
 
@@ -254,12 +266,11 @@ GRAPE_HD Mont<P> cneg(const Mont<P>& a, bool flag) {
     for (int i = 0; i < N; i++) nz |= a.v[i];
     bool doit = flag & (nz != 0);
     Mont<P> r;
-    uint64_t borrow = 0;
+    uint32_t borrow = 0;
 #pragma unroll
     for (int i = 0; i < N; i++) {
-        uint64_t t = (uint64_t)P::mod(i) - a.v[i] - borrow;
-        r.v[i] = doit ? (uint32_t)t : a.v[i];
-        borrow = (t >> 32) & 1u;
+        const uint32_t t = detail::sbb32(P::mod(i), a.v[i], borrow);
+        r.v[i] = doit ? t : a.v[i];
     }
     return r;
 }

@@ -286,5 +286,50 @@ GRAPE_HD Limbs weight16(const Fr& w) {
     return pack(t);
 }
 
+// Working limbs of a value in [0, 4r) (limbs 0..8 normalised, top limb non-negative) -> canonical
+// memory form: nine 32-bit words, then a conditional subtraction of 2r and one of r on borrow chains
+// (one instruction per word; the same step on 26-bit limbs costs three times as much).
+GRAPE_HD Fr canon4_unpack(const Limbs& t) {
+    uint32_t w[9];
+    const Fr lo = unpack(t);                       // bits 0..255
+#pragma unroll
+    for (int i = 0; i < 8; i++) w[i] = lo.v[i];
+    w[8] = (uint32_t)t.v[N - 1] >> (256 - W * (N - 1));   // bits 256 and up
+#pragma unroll
+    for (int rep = 0; rep < 2; rep++) {
+        // rep 0 subtracts 2r (its ninth word is the bit shifted out of the top word of r), rep 1 subtracts r
+        uint32_t d[9];
+        uint32_t borrow = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t m = rep == 0 ? ((FrParams::mod(i) << 1) | (i ? FrParams::mod(i - 1) >> 31 : 0u)) : FrParams::mod(i);
+            d[i] = detail::sbb32(w[i], m, borrow);
+        }
+        d[8] = detail::sbb32(w[8], rep == 0 ? FrParams::mod(7) >> 31 : 0u, borrow);
+        const bool below = borrow != 0;            // w < 2r resp. r: keep w
+#pragma unroll
+        for (int i = 0; i < 9; i++) w[i] = below ? w[i] : d[i];
+    }
+    Fr r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.v[i] = w[i];
+    return r;
+}
+
+// lo + v * (hi - lo) in canonical memory form with w1 = weight16(v) and d = hi - lo as signed
+// limbs: ONE limb product.  lo enters the accumulator as lo * 2^260 (its limbs are the starting
+// values of columns N..2N-1), so the reduction returns v*d + lo directly: |w1 * d| < r^2 and
+// 0 <= lo < r put the result, with one r added, in (0.97 r, 3.03 r).
+GRAPE_HD Fr fold1(const Limbs& w1, const Limbs& lo, const Limbs& d) {
+    Acc F;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        F.c[i] = 0;
+        F.c[N + i] = (int64_t)(uint32_t)lo.v[i];
+    }
+    mac(F, w1, d);
+    return canon4_unpack(reduce(F, 1));
+}
+
 }  // namespace fr26
 }  // namespace grape

@@ -23,14 +23,16 @@ __device__ __forceinline__ void st_fr(uint32_t* base, size_t i, const Fr& a) {
 // element as 26-bit working limbs straight from memory
 __device__ __forceinline__ fr26::Limbs ld_l26(const uint32_t* base, size_t i) { return fr26::pack(ld_fr(base, i)); }
 
-// (1-v)*lo + v*hi in canonical memory form, with w0 = weight16(1-v), w1 = weight16(v):
-// the sum of two products is below 2 r^2, so one conditional subtraction finishes it.
-__device__ __forceinline__ Fr fold2(const fr26::Limbs& w0, const fr26::Limbs& w1, const fr26::Limbs& lo, const fr26::Limbs& hi) {
-    fr26::Acc F;
-    fr26::acc_zero(F);
-    fr26::mac(F, w0, lo);
-    fr26::mac(F, w1, hi);
-    return fr26::unpack(fr26::canon(fr26::reduce(F, 0), 1));
+using fr26::fold1;
+
+// hi operand of the MSB split: X[g + h] or zero when that index is past the live extent
+__device__ __forceinline__ Fr ld_hi(const uint32_t* X, size_t g, size_t h, size_t in_size) {
+    return (g + h < in_size) ? ld_fr(X, g + h) : Fr::zero();
+}
+
+// hi operand as working limbs (zero past the live extent)
+__device__ __forceinline__ fr26::Limbs ld_hi26(const uint32_t* X, size_t g, size_t h, size_t in_size) {
+    return fr26::pack(ld_hi(X, g, h, in_size));
 }
 
 __device__ __forceinline__ Fr shfl_down_fr(const Fr& a, int off) {

@@ -6,29 +6,21 @@
 
 namespace grape {
 
-// hi operand of the MSB split: X[g + h] or zero when that index is past the live extent
-__device__ __forceinline__ Fr ld_hi(const uint32_t* X, size_t g, size_t h, size_t in_size) {
-    return (g + h < in_size) ? ld_fr(X, g + h) : Fr::zero();
-}
-
-// hi operand as working limbs (zero past the live extent)
-__device__ __forceinline__ fr26::Limbs ld_hi26(const uint32_t* X, size_t g, size_t h, size_t in_size) {
-    return fr26::pack(ld_hi(X, g, h, in_size));
-}
-
-// Iterations per thread of the round kernels: the three coefficient sums are kept as
-// double-width column accumulators across the grid-stride loop and reduced once per thread,
-// which bounds how many products a column may absorb (16 iterations x 2 products x 10 limb
-// products x 2^52 < 2^61).
-constexpr int kRoundIters = 16;
+// Iterations per thread of the round kernels: the coefficient sums are kept as double-width column
+// accumulators across the grid-stride loop and reduced once per thread, which bounds how many
+// products an accumulator may absorb: a column takes ten limb products below 2^52 per operand
+// pair (2^55.4), so 64 pairs stay below 2^61.4, and |sum| < 64 r^2 leaves the reduction within
+// (-1.82 r, 2.82 r) of its offset - inside the windows finish_sum is called with below.  The
+// reduction and the workgroup tree that follow cost about five thousand instructions per thread:
+// with 16 pairs per thread that was a quarter of the kernel, with 64 it is a fifteenth.
+constexpr int kRoundIters = 64;
 
 template <bool COEFFS>
 __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
                                                            uint32_t in_size, uint32_t out_size, const uint32_t* v,
                                                            uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
-    const Fr vv = ld_fr(v, 0);
-    const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
     fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
     fr26::acc_zero(Q);
@@ -37,9 +29,9 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t
     for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < out_size; g += stride) {
         const fr26::Limbs a0 = ld_l26(A, g), b0 = ld_l26(B, g);
         const fr26::Limbs a1 = ld_hi26(A, g, out_size, in_size), b1 = ld_hi26(B, g, out_size, in_size);
-        st_fr(A, g, fold2(w0, w1, a0, a1));
-        st_fr(B, g, fold2(w0, w1, b0, b1));
         const fr26::Limbs da = fr26::sub(a1, a0), db = fr26::sub(b1, b0);   // signed, |limb| < 2^26
+        st_fr(A, g, fold1(w1, a0, da));
+        st_fr(B, g, fold1(w1, b0, db));
         if (COEFFS) {
             // materialised coefficient arrays (phase 1 folds them further)
             fr26::Acc T;
@@ -89,14 +81,15 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_tail_kernel(uint32_t* A, uin
         Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
         if (g < out) {
             const Fr vv = ld_fr(v_end - 8 * (size_t)(i + 1), 0);
-            const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
+            const fr26::Limbs w1 = fr26::weight16(vv);
             const Fr a0c = ld_fr(A, g), b0c = ld_fr(B, g);
             const Fr a1c = ld_hi(A, g, out, in), b1c = ld_hi(B, g, out, in);
             acc[0] = fr26::mulc(a0c, b0c);
             acc[2] = fr26::mulc(sub(a1c, a0c), sub(b1c, b0c));
             acc[1] = sub(sub(fr26::mulc(a1c, b1c), acc[0]), acc[2]);
-            st_fr(A, g, fold2(w0, w1, fr26::pack(a0c), fr26::pack(a1c)));
-            st_fr(B, g, fold2(w0, w1, fr26::pack(b0c), fr26::pack(b1c)));
+            const fr26::Limbs a0 = fr26::pack(a0c), b0 = fr26::pack(b0c);
+            st_fr(A, g, fold1(w1, a0, fr26::sub(fr26::pack(a1c), a0)));
+            st_fr(B, g, fold1(w1, b0, fr26::sub(fr26::pack(b1c), b0)));
         }
         block_sum<3>(acc, lds);
         if (threadIdx.x == 0) {
@@ -113,10 +106,10 @@ __global__ void __launch_bounds__(kBlock) sumcheck1_kernel(uint32_t* X, uint32_t
                                                            uint32_t out_size, const uint32_t* v) {
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (g >= out_size) return;
-    const Fr vv = ld_fr(v, 0);
     const Fr Xb = ld_fr(X, g);
     const Fr Xh = ld_hi(X, g, out_size, in_size);
-    st_fr(X, g, fold2(fr26::weight16(sub(Fr::one(), vv)), fr26::weight16(vv), fr26::pack(Xb), fr26::pack(Xh)));
+    const fr26::Limbs lo = fr26::pack(Xb);
+    st_fr(X, g, fold1(fr26::weight16(ld_fr(v, 0)), lo, fr26::sub(fr26::pack(Xh), lo)));
     st_fr(b, g, Xb);
     st_fr(a, g, sub(Xh, Xb));
 }
@@ -391,28 +384,30 @@ struct PtrPack { uint32_t* p[8]; };
 __global__ void __launch_bounds__(kBlock) fold_msb_multi_kernel(PtrPack pk, uint32_t k, size_t n_out, const uint32_t* v) {
     size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (g >= n_out) return;
-    const Fr vv = ld_fr(v, 0);
-    const fr26::Limbs w1 = fr26::weight16(vv), w0 = fr26::weight16(sub(Fr::one(), vv));
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
     for (uint32_t j = 0; j < k; j++) {
         uint32_t* X = pk.p[j];
-        st_fr(X, g, fold2(w0, w1, ld_l26(X, g), ld_l26(X, g + n_out)));
+        const fr26::Limbs lo = ld_l26(X, g);
+        st_fr(X, g, fold1(w1, lo, fr26::sub(ld_l26(X, g + n_out), lo)));
     }
 }
 
-// enough workgroups that no thread runs more than kRoundIters iterations, at most one element
-// per thread below that
-static unsigned reduce_grid(size_t n) {
+// enough workgroups that no thread runs more than `iters` iterations, at most one element per
+// thread while that still leaves every CU a few workgroups
+static unsigned reduce_grid(size_t n, int iters = kRoundIters) {
     unsigned nb = blocks_for(n);
-    unsigned cap = kNumCU * 8;
+    unsigned cap = kNumCU * 4;
     if (nb <= cap) return nb;
-    unsigned need = blocks_for(n, kBlock * kRoundIters);
+    unsigned need = blocks_for(n, kBlock * iters);
     return need > cap ? need : cap;
 }
+// the logUp round sums grow faster per iteration (see tl_round_kernel)
+constexpr int kLogUpIters = 16;
 
 // ---------------------------------------------------------------- entry point that allocates nothing
 // Partial sums of grape_sumcheck_round2_noalloc: a fixed array in the code object instead of a
 // pool buffer, sized for the largest round that entry point accepts (kNoAllocMaxOut output indices
-// -> at most kNoAllocMaxBlocks workgroups leaving three 32-byte sums each: 1.5 MiB per GPU, held
+// -> at most kNoAllocMaxBlocks workgroups leaving three 32-byte sums each: 384 KiB per GPU, held
 // until the process ends).  Host code never uses this name as an address: it asks the runtime for
 // the array's device address once per device (noalloc_scratch) and passes that to the kernels.
 constexpr uint32_t kNoAllocMaxOut = 1u << 26;
@@ -654,7 +649,7 @@ int grape_tlookup_round_sums(const uint32_t* A, const uint32_t* S, const uint32_
     CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(eq); CHECK_PTR16(sums);
     GRAPE_REQUIRE(n_out >= 1, "empty round");
     hipStream_t s = as_stream(st);
-    unsigned nb = reduce_grid(n_out);
+    unsigned nb = reduce_grid(n_out, kLogUpIters);
     void* ws;
     int rc = scratch_get(kSlotReduce, (size_t)nb * 5 * 32, &ws, s);
     if (rc) return rc;

@@ -1,0 +1,360 @@
+// Sumcheck rounds whose terms carry an eq(u, x) weight: the element-product sumcheck (src/prove.cu:
+// 119-172), phase 1 of the matmul sumcheck (:49-85), the claim-merging sumcheck (:245-300) and the
+// logUp rounds of tLookup (src/tlookup.cu:117-244).  The reference materialises coefficient arrays
+// and folds each of them over the remaining variables of u in every round; here a round is ONE
+// pass over the operands: the weights come from a pyramid of eq tables built once per proof (no
+// per-round halving), the operands are folded in place by the same pass, and the weighted sums
+// leave the kernel as per-workgroup partial sums that a one-block kernel finishes.  Challenges are
+// known before the first round, so the host queues all rounds and reads the sums once.
+#include "fr_device.hpp"
+
+namespace grape {
+
+// ---------------------------------------------------------------- eq pyramid
+// Level j (2^j entries) sits at element offset 2^j - 1; level j holds eq(u[0..j-1], i), bit b of i
+// paired with u[b].  Level j+1 from level j: hi = lo * u[j], lo' = lo - hi.
+constexpr uint32_t kPyrHeadLevels = 9;   // levels 0..9 built by one workgroup (512 threads' worth at the top)
+
+__global__ void __launch_bounds__(kBlock) eq_pyramid_head_kernel(uint32_t* pyr, const uint32_t* u, uint32_t levels) {
+    if (threadIdx.x == 0) st_fr(pyr, 0, Fr::one());
+    __syncthreads();
+    for (uint32_t j = 0; j < levels; j++) {
+        const size_t half = (size_t)1 << j, src = half - 1, dst = 2 * half - 1;
+        const Fr uj = ld_fr(u, j);
+        for (size_t i = threadIdx.x; i < half; i += kBlock) {
+            const Fr lo = ld_fr(pyr, src + i);
+            const Fr hi = fr26::mulc(lo, uj);
+            st_fr(pyr, dst + i + half, hi);
+            st_fr(pyr, dst + i, sub(lo, hi));
+        }
+        __threadfence_block();
+        __syncthreads();
+    }
+}
+__global__ void __launch_bounds__(kBlock) eq_pyramid_level_kernel(uint32_t* pyr, const uint32_t* u, uint32_t j) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t half = (size_t)1 << j;
+    if (i >= half) return;
+    const Fr lo = ld_fr(pyr, half - 1 + i);
+    const Fr hi = fr26::mulc(lo, ld_fr(u, j));
+    st_fr(pyr, 2 * half - 1 + i + half, hi);
+    st_fr(pyr, 2 * half - 1 + i, sub(lo, hi));
+}
+
+// ---------------------------------------------------------------- weighted two-tensor round
+// One thread runs at most kWIters indices; the three weighted sums are double-width column
+// accumulators reduced once per thread.  Per index (e = weight, x0/x1 = halves of the MSB split,
+// d = x1 - x0, S' = S + beta):
+//   ea0 = e*a0 in (0, 1.46 r), ead = e*da in (0.54 r, 2.46 r)        (limbs normalised, below 2^26)
+//   W0 += ea0 * s0'        < 2.92 r^2         s0' < 2r, limbs < 2^27
+//   W2 += ead * ds         < 2.46 r^2         |ds| < r, |limb| < 2^26
+//   WQ += (ea0+ead) * s1'  < 7.84 r^2         s1' < 2r, limbs < 2^27 -> a column grows by < 2^57.4
+// so 24 indices keep a column below 2^62 and the sums within +-5.4 r of their offsets.  The sums
+// leave the thread WITHOUT the radix factor 16 (value / 2^260, canonical); the finishing kernel
+// applies it once.  The middle coefficient is WQ - W0 - W2 (one product instead of two).
+constexpr int kWIters = 24;
+
+// a finished column sum -> canonical element of value V / 2^260 + (a multiple of r)
+__device__ __forceinline__ Fr reduce_to_fr(fr26::Acc& C, int lo_r) {
+    return fr26::unpack(fr26::canon_wide(fr26::reduce(C, lo_r)));
+}
+
+template <bool BETA, bool PLAIN>
+__global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E,
+                                                         uint32_t in_size, uint32_t n_out, uint32_t rowlen, uint32_t rowpad,
+                                                         const uint32_t* v, uint32_t* partial) {
+    constexpr int NV = PLAIN ? 5 : 3;
+    __shared__ Fr lds[NV * (kBlock / 64)];
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    fr26::Limbs bt;
+    if (BETA) bt = fr26::pack(ld_fr(beta, 0));
+    fr26::Acc W0, WQ, W2;
+    fr26::acc_zero(W0);
+    fr26::acc_zero(WQ);
+    fr26::acc_zero(W2);
+    fr26::Limbs sa0, sa1;                       // plain limb-wise sums of A's halves (24 terms below 2^26)
+#pragma unroll
+    for (int k = 0; k < fr26::N; k++) sa0.v[k] = sa1.v[k] = 0;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < n_out; g += stride) {
+        // weights live on rows of `rowpad` entries when the tensors' rows hold `rowlen` < rowpad
+        const size_t ei = rowlen == rowpad ? g : g + (size_t)((uint32_t)g / rowlen) * (rowpad - rowlen);
+        const fr26::Limbs e16 = fr26::pack16(ld_fr(E, ei));
+        const fr26::Limbs a0 = ld_l26(A, g);
+        const fr26::Limbs a1 = ld_hi26(A, g, n_out, in_size);
+        const fr26::Limbs da = fr26::sub(a1, a0);
+        st_fr(A, g, fold1(w1, a0, da));
+        fr26::Acc T;
+        fr26::acc_zero(T);
+        fr26::mac(T, e16, a0);
+        const fr26::Limbs ea0 = fr26::reduce(T, 0);
+        fr26::acc_zero(T);
+        fr26::mac(T, e16, da);
+        const fr26::Limbs ead = fr26::reduce(T, 1);
+        if (PLAIN) {
+            sa0 = fr26::add(sa0, a0);
+            sa1 = fr26::add(sa1, a1);
+        }
+        const fr26::Limbs s0r = ld_l26(S, g);
+        const fr26::Limbs s1r = ld_hi26(S, g, n_out, in_size);
+        const fr26::Limbs ds = fr26::sub(s1r, s0r);
+        st_fr(S, g, fold1(w1, s0r, ds));
+        fr26::mac(W2, ead, ds);
+        if (BETA) {
+            fr26::mac(W0, ea0, fr26::add(s0r, bt));
+            fr26::mac(WQ, fr26::add(ea0, ead), fr26::add(s1r, bt));
+        } else {
+            fr26::mac(W0, ea0, s0r);
+            fr26::mac(WQ, fr26::add(ea0, ead), s1r);
+        }
+    }
+    // offsets: |W0| < 71 r^2 -> within 2 r, |W2| < 60 r^2 -> within 1.7 r, |WQ| < 189 r^2 -> within 5.4 r
+    Fr acc[NV];
+    acc[0] = reduce_to_fr(W0, 3);
+    acc[1] = reduce_to_fr(WQ, 6);
+    acc[2] = reduce_to_fr(W2, 3);
+    if (PLAIN) {
+        acc[3] = fr26::limb_sum_to_fr(sa0, 0);      // below 24 r
+        acc[4] = fr26::limb_sum_to_fr(sa1, 0);
+    }
+    block_sum<NV>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) st_fr(partial, (size_t)blockIdx.x * NV + k, acc[k]);
+    }
+}
+
+// sums[0..2] = 16 * (W0, WQ - W0 - W2, W2); with PLAIN sums[3] = sum A0, sums[4] = sum A1 - sum A0
+template <bool PLAIN>
+__global__ void __launch_bounds__(kBlock) wround2_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
+    constexpr int NV = PLAIN ? 5 : 3;
+    __shared__ Fr lds[NV * (kBlock / 64)];
+    Fr acc[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) acc[k] = Fr::zero();
+    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) acc[k] = add(acc[k], ld_fr(partial, (size_t)b * NV + k));
+    }
+    block_sum<NV>(acc, lds);
+    if (threadIdx.x == 0) {
+        Fr w[3] = {acc[0], sub(sub(acc[1], acc[0]), acc[2]), acc[2]};
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            Fr t = w[k];
+#pragma unroll
+            for (int d = 0; d < 4; d++) t = add(t, t);
+            st_fr(out, k, t);
+        }
+        if (PLAIN) {
+            st_fr(out, 3, acc[3]);
+            st_fr(out, 4, sub(acc[4], acc[3]));
+        }
+    }
+}
+
+// ---------------------------------------------------------------- matmul phase 1: weights per segment
+// Indices g = seg * seglen + k; every index of a segment shares the weight e[seg], so the three
+// sums are taken per (segment, chunk) without weights and the finishing kernel applies e[seg].
+__global__ void __launch_bounds__(kBlock) sumcheck2_seg_kernel(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size,
+                                                               uint32_t seglen, const uint32_t* v, uint32_t* partial) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    fr26::Acc C0, Q, C2;
+    fr26::acc_zero(C0);
+    fr26::acc_zero(Q);
+    fr26::acc_zero(C2);
+    const uint32_t seg = blockIdx.y;
+    const uint32_t stride = gridDim.x * kBlock;      // the host keeps seglen / stride <= 64
+    for (uint32_t k = blockIdx.x * kBlock + threadIdx.x; k < seglen; k += stride) {
+        const size_t g = (size_t)seg * seglen + k;
+        if (g >= out_size) break;
+        const fr26::Limbs a0 = ld_l26(A, g), b0 = ld_l26(B, g);
+        const fr26::Limbs a1 = ld_hi26(A, g, out_size, in_size), b1 = ld_hi26(B, g, out_size, in_size);
+        const fr26::Limbs da = fr26::sub(a1, a0), db = fr26::sub(b1, b0);
+        st_fr(A, g, fold1(w1, a0, da));
+        st_fr(B, g, fold1(w1, b0, db));
+        fr26::mac(C0, a0, b0);
+        fr26::mac(Q, a1, b1);
+        fr26::mac(C2, da, db);
+    }
+    const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2), q1 = fr26::finish_sum(Q, 2);
+    Fr acc[3] = {c0, sub(sub(q1, c0), c2), c2};
+    block_sum<3>(acc, lds);
+    if (threadIdx.x == 0) {
+        const size_t slot = (size_t)seg * gridDim.x + blockIdx.x;
+#pragma unroll
+        for (int t = 0; t < 3; t++) st_fr(partial, slot * 3 + t, acc[t]);
+    }
+}
+// sums[t] = sum_seg e[seg] * sum_chunk partial[seg][chunk][t]
+__global__ void __launch_bounds__(kBlock) seg_final_kernel(uint32_t* out, const uint32_t* partial, const uint32_t* e, uint32_t nseg,
+                                                           uint32_t nchunk) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    for (uint32_t s = threadIdx.x; s < nseg; s += kBlock) {
+        Fr t[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+        for (uint32_t c = 0; c < nchunk; c++) {
+#pragma unroll
+            for (int k = 0; k < 3; k++) t[k] = add(t[k], ld_fr(partial, ((size_t)s * nchunk + c) * 3 + k));
+        }
+        const Fr w = ld_fr(e, s);
+#pragma unroll
+        for (int k = 0; k < 3; k++) acc[k] = add(acc[k], fr26::mulc(w, t[k]));
+    }
+    block_sum<3>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 3; k++) st_fr(out, k, acc[k]);
+    }
+}
+
+// ---------------------------------------------------------------- claim merging: one tensor, several weight tables
+// For claim j (blockIdx.y) with weights e_j: sums[2j] = sum_x e_j[x] X0[x], sums[2j+1] = sum_x e_j[x] (X1[x] - X0[x]).
+// Nothing is modified (the fold is a separate launch: every claim reads the unfolded tensor).
+struct PyrPack { const uint32_t* p[16]; };
+__global__ void __launch_bounds__(kBlock) wsum1_kernel(const uint32_t* X, PyrPack E, uint32_t in_size, uint32_t n_out, uint32_t* partial) {
+    __shared__ Fr lds[2 * (kBlock / 64)];
+    const uint32_t* e = E.p[blockIdx.y];
+    fr26::Acc C0, C1;
+    fr26::acc_zero(C0);
+    fr26::acc_zero(C1);
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    // 64 indices per thread at most: e, x0 below 2^26 per limb -> a column grows by < 2^55.4 per index
+    for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < n_out; g += stride) {
+        const fr26::Limbs w = ld_l26(e, g);
+        const fr26::Limbs x0 = ld_l26(X, g);
+        const fr26::Limbs x1 = ld_hi26(X, g, n_out, in_size);
+        fr26::mac(C0, w, x0);
+        fr26::mac(C1, w, fr26::sub(x1, x0));
+    }
+    // |sum| < 64 r^2 -> within 1.82 r of the offset; the factor 16 is applied by the finishing kernel
+    Fr acc[2] = {reduce_to_fr(C0, 2), reduce_to_fr(C1, 2)};
+    block_sum<2>(acc, lds);
+    if (threadIdx.x == 0) {
+        const size_t slot = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+        st_fr(partial, slot * 2, acc[0]);
+        st_fr(partial, slot * 2 + 1, acc[1]);
+    }
+}
+__global__ void __launch_bounds__(kBlock) wsum1_final_kernel(uint32_t* out, const uint32_t* partial, uint32_t nblocks) {
+    __shared__ Fr lds[2 * (kBlock / 64)];
+    const uint32_t j = blockIdx.x;
+    Fr acc[2] = {Fr::zero(), Fr::zero()};
+    for (uint32_t b = threadIdx.x; b < nblocks; b += kBlock) {
+        acc[0] = add(acc[0], ld_fr(partial, ((size_t)j * nblocks + b) * 2));
+        acc[1] = add(acc[1], ld_fr(partial, ((size_t)j * nblocks + b) * 2 + 1));
+    }
+    block_sum<2>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            Fr t = acc[k];
+#pragma unroll
+            for (int d = 0; d < 4; d++) t = add(t, t);
+            st_fr(out, 2 * (size_t)j + k, t);
+        }
+    }
+}
+
+}  // namespace grape
+
+using namespace grape;
+
+extern "C" {
+
+size_t grape_eq_pyramid_elems(uint32_t nu) { return ((size_t)2 << nu) - 1; }
+
+int grape_eq_pyramid(uint32_t* pyr, const uint32_t* u, uint32_t nu, grape_stream_t st) {
+    CHECK_PTR16(pyr);
+    GRAPE_REQUIRE(nu <= 30, "too many variables");
+    if (nu) CHECK_PTR16(u);
+    hipStream_t s = as_stream(st);
+    const uint32_t head = nu < kPyrHeadLevels ? nu : kPyrHeadLevels;
+    eq_pyramid_head_kernel<<<1, kBlock, 0, s>>>(pyr, u, head);
+    for (uint32_t j = head; j < nu; j++) eq_pyramid_level_kernel<<<blocks_for((size_t)1 << j), kBlock, 0, s>>>(pyr, u, j);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E, uint32_t in_size, uint32_t n_out,
+                  uint32_t rowlen, uint32_t rowpad, const uint32_t* v, int plain_sums, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(E); CHECK_PTR16(v); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(n_out >= 1 && in_size >= n_out && in_size <= 2 * (uint64_t)n_out, "need n_out <= in_size <= 2*n_out");
+    GRAPE_REQUIRE(rowlen >= 1 && rowlen <= rowpad, "need 1 <= rowlen <= rowpad");
+    if (beta) CHECK_PTR16(beta);
+    hipStream_t s = as_stream(st);
+    unsigned nb = blocks_for(n_out);
+    if (nb > (unsigned)kNumCU * 4) {
+        const unsigned need = blocks_for(n_out, kBlock * kWIters);
+        nb = need > (unsigned)kNumCU * 4 ? need : (unsigned)kNumCU * 4;
+    }
+    const int nv = plain_sums ? 5 : 3;
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nb * nv * 32, &ws, s);
+    if (rc) return rc;
+    uint32_t* partial = (uint32_t*)ws;
+    if (beta && plain_sums) {
+        wround2_kernel<true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        wround2_final_kernel<true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    } else if (beta) {
+        wround2_kernel<true, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        wround2_final_kernel<false><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    } else if (plain_sums) {
+        wround2_kernel<false, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        wround2_final_kernel<true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    } else {
+        wround2_kernel<false, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        wround2_final_kernel<false><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    }
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_sumcheck_round2_seg(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, uint32_t seglen, const uint32_t* e,
+                              const uint32_t* v, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(B); CHECK_PTR16(e); CHECK_PTR16(v); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * (uint64_t)out_size, "need out_size <= in_size <= 2*out_size");
+    GRAPE_REQUIRE(seglen >= 1 && out_size % seglen == 0, "out_size must be a whole number of segments");
+    const uint32_t nseg = out_size / seglen;
+    GRAPE_REQUIRE(nseg <= 65535, "too many segments");
+    hipStream_t s = as_stream(st);
+    // chunks per segment: one index per thread until the grid is large, never more than 64 per thread
+    uint32_t nchunk = blocks_for(seglen);
+    const uint32_t cap = nseg >= 2048 ? 1 : 2048 / nseg;
+    if (nchunk > cap) nchunk = cap;
+    const uint32_t need = blocks_for(seglen, kBlock * 64);
+    if (nchunk < need) nchunk = need;
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nseg * nchunk * 3 * 32, &ws, s);
+    if (rc) return rc;
+    sumcheck2_seg_kernel<<<dim3(nchunk, nseg), kBlock, 0, s>>>(A, B, in_size, out_size, seglen, v, (uint32_t*)ws);
+    seg_final_kernel<<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, e, nseg, nchunk);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wsum1_multi(const uint32_t* X, const uint32_t* const* e_tables, uint32_t num, uint32_t in_size, uint32_t n_out,
+                      uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(X); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(e_tables != nullptr && num >= 1 && num <= 16, "1..16 weight tables");
+    GRAPE_REQUIRE(n_out >= 1 && in_size >= n_out && in_size <= 2 * (uint64_t)n_out, "need n_out <= in_size <= 2*n_out");
+    PyrPack pk;
+    for (uint32_t j = 0; j < 16; j++) pk.p[j] = j < num ? e_tables[j] : nullptr;
+    for (uint32_t j = 0; j < num; j++) CHECK_PTR16(pk.p[j]);
+    hipStream_t s = as_stream(st);
+    unsigned nb = blocks_for(n_out);
+    if (nb > (unsigned)kNumCU * 4) {
+        const unsigned need = blocks_for(n_out, kBlock * 64);
+        nb = need > (unsigned)kNumCU * 4 ? need : (unsigned)kNumCU * 4;
+    }
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nb * num * 2 * 32, &ws, s);
+    if (rc) return rc;
+    wsum1_kernel<<<dim3(nb, num), kBlock, 0, s>>>(X, pk, in_size, n_out, (uint32_t*)ws);
+    wsum1_final_kernel<<<num, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+}  // extern "C"

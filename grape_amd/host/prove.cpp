@@ -1,5 +1,6 @@
 #include "prove.hpp"
 #include <cassert>
+#include <memory>
 #include "../../include/grape_hip.h"
 
 using grape_host::check;
@@ -15,30 +16,66 @@ static void read3(fr_t* d_sums, Fr out[3]) {
     check(grape_memcpy_d2h(out, d_sums, 3 * sizeof(fr_t), nullptr), "grape_memcpy_d2h");
 }
 
-// src/prove.cu:49-85
+namespace {
+// device buffer released on scope exit
+struct DeviceBuf {
+    void* p = nullptr;
+    explicit DeviceBuf(size_t bytes) { check(grape_malloc(&p, bytes ? bytes : 1), "grape_malloc"); }
+    ~DeviceBuf() { grape_free(p); }
+    DeviceBuf(const DeviceBuf&) = delete;
+    DeviceBuf& operator=(const DeviceBuf&) = delete;
+    fr_t* fr() const { return static_cast<fr_t*>(p); }
+};
+// eq tables of every prefix of `nvars` device challenges starting at d_u (level j at offset 2^j - 1)
+struct EqPyramid {
+    DeviceBuf buf;
+    EqPyramid(const fr_t* d_u, uint nvars) : buf(sizeof(fr_t) * grape_eq_pyramid_elems(nvars)) {
+        check(grape_eq_pyramid(W(buf.fr()), reinterpret_cast<const uint32_t*>(d_u), nvars, nullptr), "grape_eq_pyramid");
+    }
+    fr_t* level(uint j) const { return buf.fr() + (((size_t)1 << j) - 1); }
+};
+std::vector<Fr> download_vec(const fr_t* d, size_t n) {
+    std::vector<Fr> out(n);
+    if (n) check(grape_memcpy_d2h(out.data(), d, sizeof(fr_t) * n, nullptr), "grape_memcpy_d2h");
+    return out;
+}
+}  // namespace
+
+// Phase 1 of the matmul sumcheck (src/prove.cu:49-85) binds the batch variables l of
+// sum_l eq(u_l, l) sum_k A[l][k] B[l][k].  The reference writes three coefficient arrays per round,
+// folds each over the remaining l-bits of u and sums the K survivors; here every round is one
+// launch that folds A and B and takes the three sums per batch row, weighted by that row's
+// eq(u_low, l') from a table built once.  The rounds are queued back to back (the challenges
+// are known up front) and their sums read with one copy.
 Fr matmul_sumcheck_phase1(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* u, fr_t* v, uint K, uint size,
                           Fr& claim, SumcheckTranscript* transcript) {
-    uint rounds = Log2(size / K);
-    uint inputsize = size;
-    uint outputsize = inputsize / 2;
+    (void)a;
+    (void)b;
+    (void)c;
+    const uint rounds = Log2(size / K);
     Fr eq_accumulate = Fr::one();
+    if (rounds == 0) return eq_accumulate;
+    if (size != (K << rounds)) throw std::runtime_error("matmul_phase1: the batch extent must be a power of two");
+    const std::vector<Fr> us = download_vec(u - rounds, rounds), vs = download_vec(v - rounds, rounds);
+    EqPyramid eq(u - rounds, rounds - 1);
+    FrTensor sums(3 * rounds);
+    uint in = size;
     for (uint i = 0; i < rounds; i++) {
-        check(grape_sumcheck_round2_coeffs(W(A.gpu_data), W(B.gpu_data), W(a.gpu_data), W(b.gpu_data), W(c.gpu_data), inputsize,
-                                           outputsize, W(v - i - 1), nullptr, nullptr),
-              "grape_sumcheck_round2_coeffs");
-        a.partial_eval(outputsize, u - rounds, outputsize / K, 0, K);
-        b.partial_eval(outputsize, u - rounds, outputsize / K, 0, K);
-        c.partial_eval(outputsize, u - rounds, outputsize / K, 0, K);
-        Polynomial p({c.sum(K), b.sum(K), a.sum(K)});
-        Fr u_now = grape_host::download(u - i - 1);
+        const uint out = in / 2;
+        check(grape_sumcheck_round2_seg(W(A.gpu_data), W(B.gpu_data), in, out, K, W(eq.level(rounds - 1 - i)), W(v - i - 1),
+                                        W(sums.gpu_data + 3 * i), nullptr),
+              "grape_sumcheck_round2_seg");
+        in = out;
+    }
+    const std::vector<Fr> s = download_vec(sums.gpu_data, 3 * (size_t)rounds);
+    for (uint i = 0; i < rounds; i++) {
+        const Fr &u_now = us[rounds - 1 - i], &v_now = vs[rounds - 1 - i];
+        Polynomial p({s[3 * i], s[3 * i + 1], s[3 * i + 2]});
         p *= (Polynomial::eq(u_now) * eq_accumulate);
         if (p(0) + p(1) != claim) throw std::runtime_error("matmul_phase1: claim != p(0) + p(1)");
-        Fr v_now = grape_host::download(v - i - 1);
         claim = p(v_now);
         record(transcript, p, claim);
-        inputsize = outputsize;
-        outputsize = outputsize / 2;
-        eq_accumulate *= (Fr::one() - v_now) * (Fr::one() - u_now) + v_now * u_now;
+        eq_accumulate *= Polynomial::eq(u_now, v_now);
     }
     return eq_accumulate;
 }
@@ -92,8 +129,7 @@ std::pair<Fr, Fr> prove_matmul(FrTensor& A, FrTensor& B, int L, int N, int M, in
     try {
         A.partial_eval(A.size, U, N, Log2(M), K);
         B.partial_eval(B.size, U, M, 0, K);
-        uint LK = (uint)L * (uint)K;
-        FrTensor a(LK < 3 ? 3 : LK), b(LK), c(LK);
+        FrTensor a(1), b(1), c(1);      // the reference's coefficient arrays (src/prove.cu:190-192): not used by the fused rounds
         Fr eq_accumulate = matmul_sumcheck_phase1(A, B, a, b, c, U + Log2(L * N * M), V + Log2(L * K), K, K * L, claim, transcript);
         matmul_sumcheck_phase2(A, B, a, b, c, V + Log2(K), K, claim, eq_accumulate, transcript);
         Fr A_claim = grape_host::download(A.gpu_data);
@@ -110,37 +146,47 @@ std::pair<Fr, Fr> prove_matmul(FrTensor& A, FrTensor& B, int L, int N, int M, in
     return ret;
 }
 
-// src/prove.cu:119-172
+// The element-product sumcheck (src/prove.cu:119-172) proves sum_x eq(u, x) A(x) B(x) over tensors
+// of first_size rows of second_size = size / first_size elements, the row index bound first
+// (rows are not padded; a last row extent that is no power of two reads as zero-extended).  The
+// reference writes three coefficient arrays per round and folds each over the remaining variables
+// of u; here a round is one launch that folds A and B and takes the three sums weighted by
+// eq(u_low, x) from a pyramid of tables built once - on rows padded to a power of two, which is
+// where the variables of u live.
 Fr eleMul_sumcheck(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* u, fr_t* v, uint first_size, uint size,
                    Fr& claim, SumcheckTranscript* transcript) {
+    (void)a;
+    (void)b;
+    (void)c;
     if ((1u << Log2(first_size)) != first_size) throw std::runtime_error("eleMul_sumcheck: first_size is illegal");
-    uint second_size = size / first_size;
-    uint rounds = Log2(size);
-    uint inputsize = size;
-    uint outputsize = size / 2;
+    const uint second_size = size / first_size;
+    const uint rounds = Log2(size);
     Fr eq_accumulate = Fr::one();
+    if (rounds == 0) return eq_accumulate;
+    const uint row_pad = 1u << Log2(second_size);
+    const std::vector<Fr> us = download_vec(u - rounds, rounds), vs = download_vec(v - rounds, rounds);
+    EqPyramid eq(u - rounds, rounds - 1);
+    FrTensor sums(3 * rounds);
+    uint in = size, out = size / 2;
     for (uint i = 0; i < rounds; i++) {
-        check(grape_sumcheck_round2_coeffs(W(A.gpu_data), W(B.gpu_data), W(a.gpu_data), W(b.gpu_data), W(c.gpu_data), inputsize,
-                                           outputsize, W(v - i - 1), nullptr, nullptr),
-              "grape_sumcheck_round2_coeffs");
-        if (inputsize > second_size) {
-            for (FrTensor* t : {&a, &b, &c}) {
-                t->partial_eval(outputsize, u - Log2(first_size), outputsize / second_size, 0, second_size);
-                t->partial_eval(second_size, u - Log2(size), second_size, 0, 1);
-            }
-        } else {
-            for (FrTensor* t : {&a, &b, &c}) t->partial_eval(outputsize, u - Log2(size), outputsize, 0, 1);
-        }
-        Polynomial p({c(0u), b(0u), a(0u)});
-        Fr u_now = grape_host::download(u - i - 1);
+        // while whole rows are paired the weights are addressed on padded rows
+        const bool rows = in > second_size && second_size != row_pad;
+        check(grape_wround2(W(A.gpu_data), W(B.gpu_data), nullptr, W(eq.level(rounds - 1 - i)), in, out, rows ? second_size : 1,
+                            rows ? row_pad : 1, W(v - i - 1), 0, W(sums.gpu_data + 3 * i), nullptr),
+              "grape_wround2");
+        in = out;
+        out = out == second_size ? (1u << (Log2(out) - 1)) : out / 2;
+        if (out == 0) out = 1;
+    }
+    const std::vector<Fr> s = download_vec(sums.gpu_data, 3 * (size_t)rounds);
+    for (uint i = 0; i < rounds; i++) {
+        const Fr &u_now = us[rounds - 1 - i], &v_now = vs[rounds - 1 - i];
+        Polynomial p({s[3 * i], s[3 * i + 1], s[3 * i + 2]});
         p *= (Polynomial::eq(u_now) * eq_accumulate);
         if (p(0) + p(1) != claim) throw std::runtime_error("ele_Mul: claim != p(0) + p(1)");
-        Fr v_now = grape_host::download(v - i - 1);
         claim = p(v_now);
         record(transcript, p, claim);
-        inputsize = outputsize;
-        outputsize = outputsize == second_size ? (1u << (Log2(outputsize) - 1)) : outputsize / 2;
-        eq_accumulate *= ((Fr::one() - v_now) * (Fr::one() - u_now) + v_now * u_now);
+        eq_accumulate *= Polynomial::eq(u_now, v_now);
     }
     return eq_accumulate;
 }
@@ -152,8 +198,7 @@ std::pair<Fr, Fr> prove_eleMul(FrTensor& A, FrTensor& B, int L, int M, int N, co
     fr_t* V = grape_host::upload(v);
     std::pair<Fr, Fr> ret;
     try {
-        uint half = (uint)(L * M * N / 2);
-        FrTensor a(half ? half : 1), b(half ? half : 1), c(half ? half : 1);
+        FrTensor a(1), b(1), c(1);      // the reference's coefficient arrays (src/prove.cu:224-226): not used by the fused rounds
         Fr eq_accumulate = eleMul_sumcheck(A, B, a, b, c, U + Log2(L * N * M), V + Log2(L * M * N), L * M, L * M * N, claim, transcript);
         Fr A_claim = grape_host::download(A.gpu_data);
         Fr B_claim = grape_host::download(B.gpu_data);
@@ -169,49 +214,71 @@ std::pair<Fr, Fr> prove_eleMul(FrTensor& A, FrTensor& B, int L, int M, int N, co
     return ret;
 }
 
-// src/prove.cu:245-300: several claims X(u_j) = claim_j about one tensor reduced to one claim X(v)
+// combine_claims (src/prove.cu:245-300) merges several claims X(u_j) = claim_j about one tensor into
+// one claim X(v) by a sumcheck over sum_j sum_x eq(u_j, x) X(x).  Per round the reference copies
+// the two coefficient arrays once per claim and evaluates each copy at the remaining variables of
+// u_j; here the weights of every claim come from its own eq pyramid (built once), one launch takes
+// all 2*num weighted sums of the round from a single read of X per claim, a second folds X, and
+// the rounds are queued without copies in between.
 Fr combine_claims(FrTensor& X, const std::vector<Fr>& claims, const std::vector<std::vector<Fr>>& u, const std::vector<Fr>& v,
                   const uint size, SumcheckTranscript* transcript) {
     if (size != (1u << Log2(size))) throw std::runtime_error("combine_claims: size must be a power of two");
-    uint num = (uint)claims.size();
+    const uint num = (uint)claims.size();
     for (uint i = 0; i < num; i++)
         if (u[i].size() != v.size()) throw std::runtime_error("combine_claims: point sizes differ");
     if ((1u << v.size()) != size) throw std::runtime_error("combine_claims: 2^|v| != size");
     Fr claim = Fr::zero();
     for (uint i = 0; i < num; i++) claim += claims[i];
-    uint rounds = (uint)v.size();
-    uint half = size / 2 ? size / 2 : 1;
-    FrTensor a(half), b(half), tmp_a(half), tmp_b(half);
-    uint input_size = size, output_size = size / 2;
-    std::vector<std::vector<Fr>> new_u = u;
-    std::vector<Fr> new_v = v;
+    const uint rounds = (uint)v.size();
     std::vector<Fr> eq_accumulate(num, Fr::one());
-    for (uint i = 0; i < rounds; i++) {
-        a.set_size(output_size);
-        b.set_size(output_size);
-        tmp_a.set_size(output_size);
-        tmp_b.set_size(output_size);
-        fr_t* d_v = grape_host::device_scalar(new_v.back());
-        check(grape_sumcheck_round1(W(X.gpu_data), W(a.gpu_data), W(b.gpu_data), input_size, output_size, W(d_v), nullptr),
-              "grape_sumcheck_round1");
-        Polynomial p(2);
-        for (uint j = 0; j < num; j++) {
-            Fr now_u = new_u[j].back();
-            new_u[j].pop_back();
-            tmp_a = a;
-            tmp_b = b;
-            Polynomial p1({tmp_b(new_u[j]), tmp_a(new_u[j])});
-            p1 *= Polynomial::eq(now_u);
-            p1 *= eq_accumulate[j];
-            p += p1;
-            eq_accumulate[j] *= Polynomial::eq(now_u, new_v.back());
+    if (rounds > 0 && num > 0) {
+        if (num > 16) throw std::runtime_error("combine_claims: at most 16 claims");
+        fr_t* d_v = grape_host::upload(v);
+        std::vector<std::unique_ptr<EqPyramid>> eq;
+        std::vector<fr_t*> d_u(num, nullptr);
+        FrTensor sums(2 * num * rounds);
+        try {
+            for (uint j = 0; j < num; j++) {
+                d_u[j] = grape_host::upload(u[j]);
+                eq.emplace_back(new EqPyramid(d_u[j], rounds - 1));
+            }
+            uint in = size;
+            for (uint i = 0; i < rounds; i++) {
+                const uint out = in / 2;
+                const uint32_t* tables[16];
+                for (uint j = 0; j < num; j++) tables[j] = W(eq[j]->level(rounds - 1 - i));
+                check(grape_wsum1_multi(W(X.gpu_data), tables, num, in, out, W(sums.gpu_data + 2 * (size_t)num * i), nullptr),
+                      "grape_wsum1_multi");
+                uint32_t* ptrs[1] = {W(X.gpu_data)};
+                check(grape_fr_fold_msb_multi(ptrs, 1, out, W(d_v + (rounds - 1 - i)), nullptr), "grape_fr_fold_msb_multi");
+                in = out;
+            }
+            const std::vector<Fr> s = download_vec(sums.gpu_data, 2 * (size_t)num * rounds);
+            for (uint i = 0; i < rounds; i++) {
+                const Fr& v_now = v[rounds - 1 - i];
+                Polynomial p(2);
+                for (uint j = 0; j < num; j++) {
+                    const Fr& now_u = u[j][rounds - 1 - i];
+                    const Fr* sj = &s[2 * ((size_t)num * i + j)];
+                    Polynomial p1({sj[0], sj[1]});
+                    p1 *= Polynomial::eq(now_u);
+                    p1 *= eq_accumulate[j];
+                    p += p1;
+                    eq_accumulate[j] *= Polynomial::eq(now_u, v_now);
+                }
+                if (p(0) + p(1) != claim) throw std::runtime_error("combine_claims: claim != p(0) + p(1)");
+                claim = p(v_now);
+                record(transcript, p, claim);
+            }
+        } catch (...) {
+            check(grape_stream_sync(nullptr), "sync");
+            for (fr_t* d : d_u) grape_free(d);
+            grape_free(d_v);
+            throw;
         }
-        if (p(0) + p(1) != claim) throw std::runtime_error("combine_claims: claim != p(0) + p(1)");
-        claim = p(new_v.back());
-        record(transcript, p, claim);
-        new_v.pop_back();
-        input_size = output_size;
-        output_size = output_size / 2;
+        check(grape_stream_sync(nullptr), "sync");
+        for (fr_t* d : d_u) grape_free(d);
+        grape_free(d_v);
     }
     Fr ret = X(0u);
     Fr sum = Fr::zero();

@@ -156,12 +156,13 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     const Fr two_inv = Fr(2).invert();
     const uint logN = Log2(N);
 
-    // eq(u[0 .. nu-2], x) for x < D/2
+    // eq tables of every prefix of u[0 .. nu-2]: round k (which binds variable nu-1-k) weights its
+    // D / 2^(k+1) index pairs with level nu-1-k; nothing is halved between rounds
     const uint nu = (uint)u.size();
-    FrTensor E(D / 2 ? D / 2 : 1);
+    FrTensor E((uint)grape_eq_pyramid_elems(nu ? nu - 1 : 0));
     {
         fr_t* d_u = grape_host::upload(u);
-        check(grape_eq_table(W(E.gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_table");
+        check(grape_eq_pyramid(W(E.gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_pyramid");
         check(grape_stream_sync(nullptr), "sync");
         grape_free(d_u);
     }
@@ -179,23 +180,20 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
             const uint half = cur / 2;
             fr_t* slot = sums.gpu_data + 13 * (size_t)k;
-            check(grape_tlookup_round_sums(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(E.gpu_data), half, W(slot), nullptr),
-                  "grape_tlookup_round_sums");
-            if (vi >= (int)logN) {
-                // phase 1: D -> N
-                uint32_t* ptrs[2] = {W(A.gpu_data), W(S.gpu_data)};
-                check(grape_fr_fold_msb_multi(ptrs, 2, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
-            } else {
+            const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
+            // A and S: five sums and the fold of both tensors in one pass
+            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), nullptr),
+                  "grape_wround2");
+            if (vi < (int)logN) {
                 // phase 2: the table variables
-                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(E.gpu_data), half, W(slot + 5), nullptr),
+                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(e), half, W(slot + 5), nullptr),
                       "grape_tlookup_round_sums");
                 check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(slot + 10), nullptr), "grape_tlookup_mb_sums");
-                uint32_t* ptrs[5] = {W(A.gpu_data), W(S.gpu_data), W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
-                check(grape_fr_fold_msb_multi(ptrs, 5, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
+                uint32_t* ptrs[3] = {W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
+                check(grape_fr_fold_msb_multi(ptrs, 3, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
             }
             A.set_size(half);
             S.set_size(half);
-            if (half >= 2) check(grape_eq_table_halve(W(E.gpu_data), half / 2, nullptr), "grape_eq_table_halve");
             cur = half;
         }
         std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1));

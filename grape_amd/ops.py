@@ -272,6 +272,38 @@ def eq_table_halve(e, n_out):
     _capi.check(lib.grape_eq_table_halve(_p(e), n_out, _s()))
 
 
+def eq_pyramid(u, nu=None):
+    """all levels of eq(u[0..j-1], .) in one tensor; level j = out[2^j - 1 : 2^(j+1) - 1]"""
+    lib = init()
+    nu = u.shape[0] if nu is None else nu
+    pyr = fr_empty(lib.grape_eq_pyramid_elems(nu))
+    _capi.check(lib.grape_eq_pyramid(_p(pyr), _p(u) if nu else None, nu, _s()))
+    return pyr
+
+
+def wround2(A, S, beta, e, in_size, n_out, v, plain_sums=False, rowlen=1, rowpad=1):
+    lib = init()
+    sums = fr_empty(5 if plain_sums else 3)
+    _capi.check(lib.grape_wround2(_p(A), _p(S), _p(beta), _p(e), in_size, n_out, rowlen, rowpad, _p(v), 1 if plain_sums else 0,
+                                  _p(sums), _s()))
+    return sums
+
+
+def sumcheck_round2_seg(A, B, in_size, out_size, seglen, e, v):
+    lib = init()
+    sums = fr_empty(3)
+    _capi.check(lib.grape_sumcheck_round2_seg(_p(A), _p(B), in_size, out_size, seglen, _p(e), _p(v), _p(sums), _s()))
+    return sums
+
+
+def wsum1_multi(X, tables, in_size, n_out):
+    lib = init()
+    sums = fr_empty(2 * len(tables))
+    arr = (ctypes.c_void_p * len(tables))(*[t.data_ptr() for t in tables])
+    _capi.check(lib.grape_wsum1_multi(_p(X), arr, len(tables), in_size, n_out, _p(sums), _s()))
+    return sums
+
+
 def fr_fold_msb_multi(tensors, n_out, v):
     lib = init()
     arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])

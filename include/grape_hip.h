@@ -121,7 +121,7 @@ int grape_sumcheck_round2(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32
                           const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
 /* The same round for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
- * results as grape_sumcheck_round2, but the per-workgroup partial sums go to a fixed 1.5 MiB array
+ * results as grape_sumcheck_round2, but the per-workgroup partial sums go to a fixed 384 KiB array
  * inside the library's code object instead of the growing scratch pool, so the call never calls
  * hipMalloc / hipFree; out_size is limited to 2^26 indices (GRAPE_EINVAL beyond).  grape_init looks the
  * array's address up for its device (a call on a device grape_init has not seen does so itself on
@@ -144,6 +144,51 @@ int grape_sumcheck_round2_coeffs(uint32_t *d_A, uint32_t *d_B, uint32_t *d_a, ui
 /* Single-tensor round (sumcheck_kernel, src/prove.cu:14-27): X[g] = Xa*v + Xb, a[g] = Xa, b[g] = Xb. */
 int grape_sumcheck_round1(uint32_t *d_X, uint32_t *d_a, uint32_t *d_b, uint32_t in_size, uint32_t out_size,
                           const uint32_t *d_v, grape_stream_t stream);
+
+/* ------------------------------------------------------------------ eq-weighted rounds -------- */
+/*
+ * Pyramid of eq tables for nu challenges u (device array): level j (2^j elements) starts at element
+ * offset 2^j - 1 and holds eq(u[0..j-1], i) = prod_{b<j} (u_b if bit_b(i) else 1 - u_b), for
+ * j = 0..nu; grape_eq_pyramid_elems(nu) = 2^(nu+1) - 1 elements in all.  A sumcheck that binds the
+ * top variable first uses level nu-1 in its first round, nu-2 in the second, ...: no table is
+ * recomputed or halved between rounds (the reference folds its coefficient arrays over the
+ * remaining variables of u in every round instead: src/prove.cu:64-66,142-154, src/tlookup.cu:129-138).
+ */
+size_t grape_eq_pyramid_elems(uint32_t nu);
+int grape_eq_pyramid(uint32_t *d_pyr, const uint32_t *d_u, uint32_t nu, grape_stream_t stream);
+/*
+ * One round of a sumcheck over sum_x e[x] * A(x) * (S(x) + beta), fused with the fold of both
+ * tensors: for g < n_out, with X0 = X[g], X1 = X[g + n_out] (zero when g + n_out >= in_size),
+ *   d_sums[0..2] = sum_g e[g'] * coefficients (low to high) of (A0 + t(A1-A0)) * (S0 + beta + t(S1-S0))
+ *   d_sums[3], d_sums[4] = sum_g A0, sum_g (A1 - A0)                    (only when plain_sums != 0)
+ *   A[g] = A0 + v(A1 - A0), S[g] = S0 + v(S1 - S0)                      (in place)
+ * d_beta may be NULL (beta = 0).  d_e is the weight table of this round (a level of the pyramid above).
+ * When the tensors' rows hold rowlen elements but the weights live on rows padded to rowpad entries
+ * (rows of 11008 with weights over 16384), g' = g + (g / rowlen) * (rowpad - rowlen); otherwise pass
+ * rowlen = rowpad and g' = g.  d_sums holds 3 (5 with plain_sums) elements.
+ * One pass replaces sumcheck_kernel + three folds of coefficient arrays per round in eleMul_sumcheck
+ * (src/prove.cu:119-172) and tLookup_poly_kernel + three multilinear evaluations +
+ * tLookup_poly_sum_kernel + two sums + the reduce kernel in tLookup_phase1 (src/tlookup.cu:117-151,216-244).
+ */
+int grape_wround2(uint32_t *d_A, uint32_t *d_S, const uint32_t *d_beta, const uint32_t *d_e, uint32_t in_size, uint32_t n_out,
+                  uint32_t rowlen, uint32_t rowpad, const uint32_t *d_v, int plain_sums, uint32_t *d_sums, grape_stream_t stream);
+/*
+ * One round of matmul_sumcheck_phase1 (src/prove.cu:49-85): grape_sumcheck_round2 on indices
+ * g = seg * seglen + k where every index of a segment carries the weight d_e[seg]
+ * (out_size / seglen segments): d_sums[t] = sum_seg d_e[seg] * sum_k coefficient_t(seg, k); A and B
+ * are folded in place.
+ */
+int grape_sumcheck_round2_seg(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size, uint32_t seglen,
+                              const uint32_t *d_e, const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
+/*
+ * Weighted sums of one tensor against several weight tables at once (combine_claims,
+ * src/prove.cu:245-300, evaluates the two coefficient arrays at the remaining variables of every
+ * claim's point): for j < num (at most 16),
+ *   d_sums[2j] = sum_g e_j[g] * X0,  d_sums[2j+1] = sum_g e_j[g] * (X1 - X0),   g < n_out.
+ * e_tables is a host array of num device pointers.  X is not modified.
+ */
+int grape_wsum1_multi(const uint32_t *d_X, const uint32_t *const *e_tables, uint32_t num, uint32_t in_size, uint32_t n_out,
+                      uint32_t *d_sums, grape_stream_t stream);
 
 /* ------------------------------------------------------------------ tlookup / logUp ---------- */
 /* hist[(v - low) as integer] += 1 for n values (Montgomery Fr); hist has `len` u32 counters and

@@ -51,4 +51,15 @@ void t26_canon_wide(const uint32_t* a, const uint32_t* b, int k, uint32_t* out) 
     for (int i = 0; i < fr26::N; i++) r.v[i] = k * A.v[i] + B.v[i];
     st(out, fr26::unpack(fr26::canon_wide(fr26::normalize(r))));
 }
+// lo + v * (hi - lo) through the single-product fold (v, lo, hi canonical; hi may be absent = zero)
+void t26_fold1(const uint32_t* v, const uint32_t* lo, const uint32_t* hi, uint32_t* out) {
+    const fr26::Limbs l = fr26::pack(ld(lo));
+    st(out, fr26::fold1(fr26::weight16(ld(v)), l, fr26::sub(fr26::pack(ld(hi)), l)));
+}
+// k * a + b for canonical a, b and 0 <= k <= 3 with k*a + b < 4r, through canon4_unpack
+void t26_canon4(const uint32_t* a, const uint32_t* b, int k, uint32_t* out) {
+    fr26::Limbs A = fr26::pack(ld(a)), B = fr26::pack(ld(b)), r;
+    for (int i = 0; i < fr26::N; i++) r.v[i] = k * A.v[i] + B.v[i];
+    st(out, fr26::canon4_unpack(fr26::normalize(r)));
+}
 }

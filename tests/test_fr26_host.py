@@ -104,3 +104,26 @@ def test_split_weighted_sum_and_wide_canon(lib):
             for b in (0, 1, R - 1, rng.randrange(R)):
                 lib.t26_canon_wide(_u32(_p([a % R])[0]), _u32(_p([b])[0]), k, _u32(out))
                 assert _val(out) == (k * (a % R) + b) % R
+
+
+def test_single_product_fold_and_canon4(lib):
+    """lo + v*(hi - lo) with one limb product and lo added into the upper accumulator columns: every
+    pairing of the edge values (differences of either sign, v = 0, 1, r-1) and random triples; the
+    nine-word canonicalisation on multiples k*a + b up to just below 4r"""
+    rng = random.Random(5)
+    out = np.zeros(8, dtype=np.uint32)
+    vals = EDGE + [rng.randrange(R) for _ in range(12)]
+    for v in [0, 1, R - 1, R >> 1] + [rng.randrange(R) for _ in range(6)]:
+        pv = _p([v])[0]
+        for lo in vals:
+            plo = _p([lo])[0]
+            for hi in vals:
+                lib.t26_fold1(_u32(pv), _u32(plo), _u32(_p([hi])[0]), _u32(out))
+                assert _val(out) == (lo + v * (hi - lo)) % R, (v, lo, hi)
+    for k in (0, 1, 2, 3):
+        for a in EDGE + [rng.randrange(R) for _ in range(10)]:
+            for b in (0, 1, R - 1, R - 2, rng.randrange(R)):
+                if k * (a % R) + b >= 4 * R:
+                    continue
+                lib.t26_canon4(_u32(_p([a % R])[0]), _u32(_p([b])[0]), k, _u32(out))
+                assert _val(out) == (k * (a % R) + b) % R
