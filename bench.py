@@ -479,6 +479,68 @@ def witness_workload(args):
     return 0
 
 
+def rounds_workload(args):
+    """The streaming kernels of the sumcheck and logUp rounds at 2^24 index pairs (tensors of 2^25
+    elements, 1 GiB each, four times the Infinity Cache): the two-tensor round (src/prove.cu:29-46
+    with its three reductions), the eq-weighted round with the fold fused in (element-product sumcheck
+    and logUp rounds), the logUp sums alone, the MSB fold of two tensors and the element-wise product.
+    Each is timed with events on the launch stream over `steps` launches; algorithmic bytes per index
+    are the operands read once and the folded tensors written once.  One JSON line."""
+    import torch
+    from grape_amd import ops
+    from gpuutil import rand_fr
+    ops.init(0)
+    lg = args.log_elems
+    n, h = 1 << lg, 1 << (lg - 1)
+    seeds = rand_fr(4, 77)
+    v, beta = ops.to_dev(seeds[0:1]), ops.to_dev(seeds[1:2])
+    A = ops.fr_from_i32(torch.arange(n, dtype=torch.int32, device="cuda"))
+    B = ops.fr_from_i32(torch.arange(n, dtype=torch.int32, device="cuda") * 3 + 1)
+    ops.fr_bcast_mul(A, ops.to_dev(seeds[2:3]), out=A)          # full-width values
+    ops.fr_bcast_mul(B, ops.to_dev(seeds[3:4]), out=B)
+    pyr = ops.eq_pyramid(ops.to_dev(rand_fr(lg - 1, 78)))
+    e = pyr[h - 1: 2 * h - 1]
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    cases = [
+        ("sumcheck2_kernel<false> + final_sum (grape_sumcheck_round2)", 192, h, lambda: ops.sumcheck_round2(A, B, n, h, v)),
+        ("wround2_kernel<beta, plain sums> + final (grape_wround2, logUp round)", 224, h,
+         lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True)),
+        ("wround2_kernel<no beta> + final (grape_wround2, element-product round)", 224, h,
+         lambda: ops.wround2(A, B, None, e, n, h, v)),
+        ("tl_round_kernel + final_sum (grape_tlookup_round_sums, read only)", 160, h, lambda: ops.tlookup_round_sums(A, B, beta, e, h)),
+        ("fold_msb_multi_kernel, two tensors", 192, h, lambda: ops.fr_fold_msb_multi([A, B], h, v)),
+        ("ew_kernel<mul> (grape_fr_mul)", 96, n, lambda: ops.fr_mul(A, B, out=A)),
+    ]
+    out = []
+    for name, bytes_per, units, fn in cases:
+        ms = timed(fn)
+        gbps = bytes_per * units / (ms * 1e-3) / 1e9
+        out.append({"kernel": name, "bytes_per_unit": bytes_per, "units": units, "ms": ms, "GBps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS})
+    copy_ms = ops.bench_copy(1 << 30, 5)
+    head = out[0]
+    print(json.dumps({
+        "metric": "round_kernel_bandwidth", "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "sumcheck / logUp round kernels at 2^%d index pairs (tensors of 2^%d Fr elements)" % (lg - 1, lg)},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["frac_of_hbm_peak"],
+                     "traffic": None, "kernel": head["kernel"]},
+        "kernels": out,
+        "hbm_copy": {"kernel": "copy_kernel", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "GBps": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9}}))
+    return 0
+
+
 def _fr_const(x):
     """Montgomery limbs of a small constant, as a (1, 4) uint64 array"""
     r = (21888242871839275222246405745257275088548364400416034343698204186575808495617 if CURVE == "bn254"
@@ -495,9 +557,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
-    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "witness"], default="commit",
+    ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "witness", "rounds"], default="commit",
                     help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
-                         "lookup: configs[3]; layer: configs[4]; witness: the layer's witness generator")
+                         "lookup: configs[3]; layer: configs[4]; witness: the layer's witness generator; "
+                         "rounds: the streaming kernels of the sumcheck / logUp rounds")
     ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer and witness workloads")
     ap.add_argument("--matmul", choices=["auto", "valu", "mfma"], default="auto",
                     help="witness workload: integer matrix products on the matrix cores (auto, mfma) or with 64-bit multiply-adds (valu)")
@@ -508,6 +572,10 @@ def main():
         print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
         return 2
+    if args.workload == "rounds":
+        args.steps = 10 if args.steps is None else args.steps
+        args.warmup = 2 if args.warmup is None else args.warmup
+        return rounds_workload(args)
     if args.workload == "witness":
         args.steps = 3 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
