@@ -644,6 +644,36 @@ GRAPE_HD bool xyzz28_madd(Xyzz28& acc, const Affine28& p, bool negate) {
     return true;
 }
 
+// acc <- 2 * acc in the 28-bit form (curve with a = 0, 6M + 3S: U = 2Y, V = U^2, W = U V, S = X V,
+// M = 3 X^2, X3 = M^2 - 2S, Y3 = M (S - X3) - W Y, ZZ3 = V ZZ, ZZZ3 = W ZZZ).  No exceptional case on
+// a group of odd prime order; the identity stays the identity.
+GRAPE_HD void xyzz28_dbl(Xyzz28& acc) {
+    using namespace fp28;
+    if (acc.inf) return;
+    Fp28 U;
+#pragma unroll
+    for (int i = 0; i < N; i++) U.v[i] = 2 * acc.y.v[i];            // (-6p, 6p), |limb| < 2^29
+    const Fp28 V = sqr(U);                                          // 36
+    const Fp28 Wd = mul(U, V);                                      // 6 * 3
+    const Fp28 S = mul(acc.x, V);                                   // 9 * 3
+    const Fp28 X2 = sqr(acc.x);                                     // 81
+    Fp28 M;
+#pragma unroll
+    for (int i = 0; i < N; i++) M.v[i] = 3 * X2.v[i];               // (0, 9p)
+    M = normalize(M);
+    const Fp28 MM = sqr(M);                                         // 81
+    Fp28 X3;
+#pragma unroll
+    for (int i = 0; i < N; i++) X3.v[i] = MM.v[i] - 2 * S.v[i];     // (-6p, 3p)
+    X3 = normalize(X3);
+    const Fp28 T = sub(S, X3);                                      // (-3p, 9p), |limb| < 2^29
+    const Fp28 Y3 = mul_sub(M, T, Wd, acc.y);                       // 81 + 9; limbs 28+29, 28+28
+    acc.zz = mul(V, acc.zz);                                        // 9
+    acc.zzz = mul(Wd, acc.zzz);                                     // 9
+    acc.x = X3;
+    acc.y = Y3;
+}
+
 // acc += q, both accumulators in the 28-bit form (12M + 2S).  Returns false, leaving acc
 // untouched, in the exceptional cases q = +-acc; identities are handled here.
 GRAPE_HD bool xyzz28_add(Xyzz28& acc, const Xyzz28& q) {

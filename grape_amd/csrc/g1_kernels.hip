@@ -10,6 +10,7 @@
 // result to affine coordinates.
 #define GRAPE_FP_MUL_OUTLINE 1
 #include "common.hpp"
+#include "commit_geometry.hpp"
 #include "fp28.hpp"
 #include "fr26.hpp"
 
@@ -117,7 +118,7 @@ __device__ __forceinline__ bool entry_is_inf(const Affine28& a) {
 }
 // Per-lane partial accumulator in memory: x, y, zz, zzz (L28 words each), the identity flag and
 // padding = 64 words (256 bytes).
-constexpr int kPartialWords = 64;
+using geom::kPartialWords;
 __device__ __forceinline__ void st_partial28(uint32_t* base, size_t i, const Xyzz28& a) {
     uint32_t f[64];
 #pragma unroll
@@ -130,12 +131,12 @@ __device__ __forceinline__ void st_partial28(uint32_t* base, size_t i, const Xyz
     f[4 * L28] = a.inf ? 1u : 0u;
 #pragma unroll
     for (int k = 4 * L28 + 1; k < 64; k++) f[k] = 0;
-    uint4* q = reinterpret_cast<uint4*>(base + (size_t)kPartialWords * i);
+    uint4* q = reinterpret_cast<uint4*>(base + geom::partial_word(i));
 #pragma unroll
     for (int k = 0; k < 16; k++) q[k] = make_uint4(f[4 * k], f[4 * k + 1], f[4 * k + 2], f[4 * k + 3]);
 }
 __device__ __forceinline__ Xyzz28 ld_partial28(const uint32_t* base, size_t i) {
-    const uint4* q = reinterpret_cast<const uint4*>(base + (size_t)kPartialWords * i);
+    const uint4* q = reinterpret_cast<const uint4*>(base + geom::partial_word(i));
     uint4 w[L28 + 1];
 #pragma unroll
     for (int k = 0; k < L28 + 1; k++) w[k] = q[k];
@@ -239,9 +240,9 @@ __device__ __forceinline__ void madd_scalar_fr(Xyzz28& acc, const Fr& k_in, cons
             if (mag > K) {
                 *err_flag = 1;
             } else {
-                const Affine28 e = ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col);
+                const Affine28 e = ld_entry28(table, geom::table_entry(w, K, mag, N, col));
                 // unconditional, so that the compiler counts the outstanding loads exactly
-                const size_t nxt = (mag_n != 0 && mag_n <= K) ? ((size_t)(w + 1) * K + (mag_n - 1)) * N + col : (size_t)col;
+                const size_t nxt = (mag_n != 0 && mag_n <= K) ? geom::table_entry(w + 1, K, mag_n, N, col) : (size_t)col;
                 touch = table[(size_t)kWideEntryWords * nxt];
                 if (kWideEntryWords % 32 != 0) touch |= table[(size_t)kWideEntryWords * nxt + kWideEntryWords - 1];   // dense entries: both lines
                 madd28(acc, e, neg != flip);
@@ -407,9 +408,9 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
     const int lane = threadIdx.x & 63;
     const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
     if (wave >= rows * nseg) return;
-    const size_t row = wave / nseg;
-    const uint32_t s = (uint32_t)(wave - row * nseg);
-    const uint32_t col_end = (s + 1) * seg < rowlen ? (s + 1) * seg : rowlen;
+    const geom::WaveSpan span = geom::wave_span(wave, nseg, seg, rowlen);
+    const size_t row = span.row;
+    const uint32_t s = span.s, col_end = span.col_end;
     const uint32_t half = 1u << (c - 1), mask = (c == 32) ? 0xffffffffu : ((1u << c) - 1u);
     Xyzz28 acc = xyzz28_inf();
     // int path: the scalars of the next two columns are kept in flight (the next one addresses
@@ -417,20 +418,20 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
     int32_t sc1 = 0, sc2 = 0;
     if (!FR) {
         const uint32_t c0 = s * seg + lane;
-        if (c0 + 64 < col_end) sc1 = ((const int32_t*)scalars)[row * rowlen + c0 + 64];
-        if (c0 + 128 < col_end) sc2 = ((const int32_t*)scalars)[row * rowlen + c0 + 128];
+        if (c0 + 64 < col_end) sc1 = ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, c0 + 64)];
+        if (c0 + 128 < col_end) sc2 = ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, c0 + 128)];
     }
-    int32_t sc0 = (!FR && s * seg + lane < col_end) ? ((const int32_t*)scalars)[row * rowlen + s * seg + lane] : 0;
+    int32_t sc0 = (!FR && s * seg + lane < col_end) ? ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, s * seg + lane)] : 0;
     for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
         if (FR) {
-            const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, row * rowlen + col));
+            const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, geom::scalar_index(row, rowlen, col)));
             madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
         } else {
             int64_t v = sc0;
             const int64_t v_next = sc1;
             sc0 = sc1;
             sc1 = sc2;
-            sc2 = (col + 192 < col_end) ? ((const int32_t*)scalars)[row * rowlen + col + 192] : 0;
+            sc2 = (col + 192 < col_end) ? ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, col + 192)] : 0;
             // The table line of the NEXT column's first digit is touched (one word) right after
             // this column's own entry is requested, so that it is in cache when its turn comes:
             // with two waves per SIMD an exposed HBM round trip per addition costs issue slots.
@@ -446,7 +447,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 if (dn > (int64_t)half || (dn == (int64_t)half && vn < 0)) dn -= (int64_t)mask + 1;
                 const uint32_t magn = (uint32_t)(dn < 0 ? -dn : dn);
                 have_next = magn != 0 && magn <= K;
-                if (have_next) next_entry = ((size_t)(magn - 1)) * N + col + 64;
+                if (have_next) next_entry = geom::table_entry(0, K, magn, N, col + 64);
             }
             const uint32_t* touch_ptr = table + (size_t)kWideEntryWords * next_entry;
             uint32_t touch = 0;
@@ -463,7 +464,7 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 const uint32_t mag = (uint32_t)(neg ? -d : d);
                 if (mag != 0) {
                     if (mag > K) { *err_flag = 1; continue; }
-                    const Affine28 e = ld_entry28(table, ((size_t)w * K + (mag - 1)) * N + col);
+                    const Affine28 e = ld_entry28(table, geom::table_entry(w, K, mag, N, col));
                     touch = *touch_ptr;
                     if (kWideEntryWords % 32 != 0) touch |= touch_ptr[kWideEntryWords - 1];   // dense entries: both lines
                     madd28(acc, e, neg);
@@ -522,14 +523,125 @@ __global__ void __launch_bounds__(64) scaled_normalize_kernel(uint32_t* out, con
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// commitment, strided table (full-width scalars)
+// ------------------------------------------------------------------------------------------------
+// A per-window table spends its bytes on ceil(255/c) sets of 2^(c-1) multiples.  Keeping only every
+// J-th set - entries k * 2^(c J q) * G_i for q < nsets = ceil(nw / J) - leaves room for wider windows
+// within the same bytes: window w = q J + j is looked up in set q, and the J residues j get their own
+// sums A_j, combined per row as sum_j 2^(c j) A_j by a Horner chain of (J - 1) c doublings.  With
+// 4096 generators c = 16, J = 4 is 16 additions per scalar from 68 GB where the per-window table
+// gives 19 from 82 GB; with 262144 generators c = 12, J = 22 (one set, 68 GB) is 22 additions where
+// no per-window table above c = 8 fits.
+//
+// Digits are taken carry-free: with H = sum_w 2^(c w + c - 1), digit_w = ((k + H) >> c w mod 2^c) - 2^(c-1)
+// lies in [-2^(c-1), 2^(c-1)) and sum_w digit_w 2^(c w) = k, so any window can be read on its own.
+// One wave per (row, residue, column segment); lanes own columns.
+__device__ __forceinline__ uint32_t window_bits(const Fr& k, uint32_t w, uint32_t c) {
+    const uint32_t bit = w * c, limb = bit >> 5, sh = bit & 31;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        lo = (q == (int)limb) ? k.v[q] : lo;
+        hi = (q == (int)limb + 1) ? k.v[q] : hi;
+    }
+    const uint64_t both = ((uint64_t)hi << 32) | lo;
+    return (uint32_t)(both >> sh) & ((1u << c) - 1u);
+}
+// The bias H restricted to the bits a 256-bit word can hold: bit (c w + c - 1) for every window whose
+// top bit lies below 256 (a window that reaches past bit 255 keeps its digit unsigned: see digit_of).
+__device__ __forceinline__ Fr window_bias(uint32_t c, uint32_t nw) {
+    Fr h = Fr::zero();
+    for (uint32_t w = 0; w < nw; w++) {
+        const uint32_t pos = w * c + c - 1;
+#pragma unroll
+        for (int i = 0; i < 8; i++) h.v[i] |= ((pos >> 5) == (uint32_t)i) ? (1u << (pos & 31)) : 0u;
+    }
+    return h;
+}
+// |k| + H for the half-range representative of a Montgomery-form scalar; flip = the scalar was negated.
+// |k| <= (r-1)/2 < 0.91 * 2^254 and H < 1.01 * 2^255, so the sum stays below 2^256.
+__device__ __forceinline__ Fr biased_half_range(const Fr& k_mont, const Fr& H, bool& flip) {
+    Fr k = fr26::from_montc(k_mont);
+    uint32_t borrow = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t half_i = (FrParams::mod(i) >> 1) | (i + 1 < 8 ? FrParams::mod(i + 1) << 31 : 0u);
+        (void)detail::sbb32(half_i, k.v[i], borrow);
+    }
+    flip = borrow != 0;                                   // k > (r-1)/2
+    k = cneg(k, flip);
+    uint32_t carry = 0;
+    Fr out;
+#pragma unroll
+    for (int i = 0; i < 8; i++) out.v[i] = detail::adc32(k.v[i], H.v[i], carry);
+    return out;
+}
+// signed digit of window w of a biased scalar: in [-2^(c-1), 2^(c-1)) (unsigned, below 2^(256 - c w), for
+// a top window whose bias bit does not exist)
+__device__ __forceinline__ int32_t digit_of(const Fr& kb, uint32_t w, uint32_t c) {
+    const int32_t bits = (int32_t)window_bits(kb, w, c);
+    return (w * c + c - 1 < 256) ? bits - (int32_t)(1u << (c - 1)) : bits;
+}
+
+__global__ void __launch_bounds__(kBlock) commit_strided_kernel(uint32_t* partial, const uint32_t* scalars, uint32_t rowlen, size_t rows,
+                                                                uint32_t seg, uint32_t nseg, const uint32_t* table, size_t N,
+                                                                uint32_t c, uint32_t nw, uint32_t K, uint32_t J, uint32_t nsets) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+    if (wave >= rows * J * nseg) return;
+    const geom::WaveSpan span = geom::wave_span(wave, nseg, seg, rowlen);   // "row" here is (row, residue)
+    const size_t row = span.row / J;
+    const uint32_t j = (uint32_t)(span.row - row * J);
+    const Fr H = window_bias(c, nw);                      // wave-uniform
+    Xyzz28 acc = xyzz28_inf();
+    for (uint32_t col = span.s * seg + lane; col < span.col_end; col += 64) {
+        bool flip;
+        const Fr kb = biased_half_range(ld_fr8(scalars, geom::scalar_index(row, rowlen, col)), H, flip);
+        // digit of set 0 now, the next set's one addition ahead (its table line is touched early)
+        int32_t d = j < nw ? digit_of(kb, j, c) : 0;
+        uint32_t touch = 0;
+        for (uint32_t q = 0; q < nsets; q++) {
+            const uint32_t wn = (q + 1) * J + j;
+            const int32_t d_n = (q + 1 < nsets && wn < nw) ? digit_of(kb, wn, c) : 0;
+            if (d != 0) {
+                const bool neg = d < 0;
+                const uint32_t mag = (uint32_t)(neg ? -d : d);
+                const Affine28 e = ld_entry28(table, geom::table_entry(q, K, mag, N, col));
+                const uint32_t mag_n = (uint32_t)(d_n < 0 ? -d_n : d_n);
+                const size_t nxt = mag_n != 0 ? geom::table_entry(q + 1, K, mag_n, N, col) : (size_t)col;
+                touch = table[(size_t)kWideEntryWords * nxt];
+                if (kWideEntryWords % 32 != 0) touch |= table[(size_t)kWideEntryWords * nxt + kWideEntryWords - 1];
+                madd28(acc, e, neg != flip);
+            }
+            d = d_n;
+        }
+        asm volatile("" ::"v"(touch));
+    }
+    st_partial28(partial, wave * 64 + lane, acc);
+}
+
+// total_row = sum_j 2^(c j) A[row * J + j] by Horner from the top residue down, then affine
+__global__ void __launch_bounds__(64) strided_horner_kernel(uint32_t* out, const uint32_t* sums, size_t rows, uint32_t J, uint32_t c) {
+    const size_t row = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (row >= rows) return;
+    Xyzz28 total = ld_partial28(sums, row * J + (J - 1));
+    for (int j = (int)J - 2; j >= 0; j--) {
+        for (uint32_t d = 0; d < c; d++) xyzz28_dbl(total);
+        padd28(total, ld_partial28(sums, row * J + j));
+    }
+    st_affine(out, row, xyzz28_to_affine(total));
+}
+
 // Row epilogue: 2^lg_lpr lanes per row, each sums its share of the partials serially, then a
 // tree over those lanes; the leader maps the row sum to affine coordinates.  All in the 28-bit form.
+template <bool AFFINE>
 __global__ void __launch_bounds__(64) commit_reduce_kernel(uint32_t* out, const uint32_t* partial, size_t rows, uint32_t nparts,
                                                            uint32_t lg_lpr) {
     const int lane = threadIdx.x & 63;
     const int lpr = 1 << lg_lpr;                       // lanes per row: 8, 16, 32 or 64
     const int sub = lane & (lpr - 1);
-    const size_t row = (size_t)blockIdx.x * (64 >> lg_lpr) + (lane >> lg_lpr);
+    const size_t row = geom::reduce_row(blockIdx.x, lane, lg_lpr);
     Xyzz28 acc = xyzz28_inf();
     // one addition site serves both the serial part and the tree steps (code size)
     const uint32_t nserial = (nparts + lpr - 1) >> lg_lpr;
@@ -547,7 +659,10 @@ __global__ void __launch_bounds__(64) commit_reduce_kernel(uint32_t* out, const 
         }
         if (doit) padd28(acc, q);
     }
-    if (row < rows && sub == 0) st_affine(out, row, xyzz28_to_affine(acc));
+    if (row < rows && sub == 0) {
+        if (AFFINE) st_affine(out, row, xyzz28_to_affine(acc));
+        else st_partial28(out, row, acc);        // left as an accumulator (256 bytes) for a later combination
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -648,22 +763,16 @@ using namespace grape;
 
 #define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")
 
-// Lanes that share a row in the row-reduction kernel: 8 when rows alone fill the chip (measured best
-// for 4096 rows of 64 partials: 4 lanes +6 %, 16 +33 %, 32 +65 % - idle lanes of the tree steps cost
-// more than shorter chains save), up to a whole wave when rows are few and the chain per lane is
-// what takes the time (one row of 32768 partials: 150 ms with 8 lanes).
-static uint32_t reduce_lanes_log2(size_t rows) {
-    if (rows >= 2048) return 3;
-    if (rows >= 1024) return 4;
-    if (rows >= 512) return 5;
-    return 6;
-}
+using geom::reduce_lanes_log2;
+// Largest commitment one call accepts: 2^28 scalars (1 GiB of int32, 8 GiB of field elements), the
+// largest size the GPU tests run; the host classes split longer tensors by rows.
+constexpr size_t kMaxCommitScalars = (size_t)1 << 28;
 
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                             uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
-    GRAPE_REQUIRE(size <= 0xffffffffull, "size must fit the reference's 32-bit element count");
+    GRAPE_REQUIRE(size <= kMaxCommitScalars, "more than 2^28 scalars in one call: commit the rows in several calls");
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
@@ -672,17 +781,11 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     const size_t rows = size / rowlen;
     if (rows == 0) return GRAPE_OK;
     hipStream_t s = as_stream(st);
-    // segments: enough waves to fill the chip (>= 4 per SIMD) but at least 64 columns per lane-sweep,
-    // and no more than leaves each reducing lane a chain of 128 partial sums
-    const uint32_t lg_lpr = reduce_lanes_log2(rows);
-    uint32_t nseg = 1;
-    while (rows * nseg < 4096 && rowlen / (nseg * 2) >= 64 && nseg * 2 <= (2u << lg_lpr)) nseg *= 2;
-    const uint32_t seg = (rowlen + nseg - 1) / nseg;
     // rows go through in slabs so that the per-lane partial sums stay within 512 MiB whatever the
     // number of rows (a row segment leaves 64 partial sums of 256 bytes)
-    size_t slab = 32768 / (size_t)nseg;
-    if (slab > rows) slab = rows;
-    const size_t partial_bytes = slab * nseg * 64 * (size_t)(4 * kPartialWords);
+    const geom::WidePlan plan = geom::wide_plan(size, rowlen, geom::kSlabSegments);
+    const uint32_t lg_lpr = plan.lg_lpr, nseg = plan.nseg, seg = plan.seg;
+    const size_t slab = plan.slab, partial_bytes = plan.partial_bytes;
     void* ws;
     int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws, s);
     if (rc) return rc;
@@ -698,7 +801,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
         profile_mark(s);
         commit_wide_kernel<FR><<<blocks_for(nr * nseg * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, N, c, nw, K, err);
         profile_mark(s);
-        commit_reduce_kernel<<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), (const uint32_t*)ws, nr,
+        commit_reduce_kernel<true><<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), (const uint32_t*)ws, nr,
                                                                                                  nseg * 64, lg_lpr);
         profile_mark(s);
     }
@@ -717,7 +820,7 @@ template <bool FR>
 static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t npoints,
                            grape_stream_t st) {
     if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
-    GRAPE_REQUIRE(size <= 0xffffffffull, "size must fit the reference's 32-bit element count");
+    GRAPE_REQUIRE(size <= kMaxCommitScalars, "more than 2^28 scalars in one call: commit the rows in several calls");
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0 && rowlen <= npoints, "bad shape");
     const size_t rows = size / rowlen;
@@ -746,7 +849,7 @@ static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint
         const uint32_t* sc = (const uint32_t*)scalars + r0 * rowlen * elem_words;
         commit_ref28_kernel<FR><<<blocks_for(units * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, npoints);
         const size_t per_wave = (size_t)64 >> lg_lpr, rw = nr * nwin;
-        commit_reduce_kernel<<<(unsigned)((rw + per_wave - 1) / per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rw, nseg * 64, lg_lpr);
+        commit_reduce_kernel<true><<<(unsigned)((rw + per_wave - 1) / per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rw, nseg * 64, lg_lpr);
         commit_ref_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, nwin);
     }
     GRAPE_LAUNCH_CHECK();
@@ -782,9 +885,8 @@ int grape_g1_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t
 
 size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K) { return (size_t)nw * K * N * 4 * kWideEntryWords; }
 
-int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
-    CHECK_PTR16(table); CHECK_PTR16(gens);
-    GRAPE_REQUIRE(N >= 1 && c >= 1 && c <= 16 && nw >= 1 && K >= 1 && K <= (1u << 16), "bad table shape");
+// table[(w*K + k-1)*N + i] = k * 2^(spacing*w) * G_i for k = 1..K, w < nw
+static int wide_table_gen_impl(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     hipStream_t s = as_stream(st);
     const size_t per_chunk = (size_t)nw * N;
     // chunk length: long enough to amortise the start-up scalar multiplication, short enough
@@ -815,6 +917,61 @@ int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uin
         wide_normalize_kernel<<<blocks_for(nthr2, 64), 64, 0, s>>>(table, tmp, N, nw, K, CH, j0, n_entries);
         GRAPE_LAUNCH_CHECK();
     }
+    return GRAPE_OK;
+}
+
+int grape_g1_wide_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    CHECK_PTR16(table); CHECK_PTR16(gens);
+    GRAPE_REQUIRE(N >= 1 && c >= 1 && c <= 16 && nw >= 1 && K >= 1 && K <= (1u << 16), "bad table shape");
+    return wide_table_gen_impl(table, gens, N, c, nw, K, st);
+}
+
+int grape_g1_strided_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t J, uint32_t nsets, grape_stream_t st) {
+    CHECK_PTR16(table); CHECK_PTR16(gens);
+    GRAPE_REQUIRE(N >= 1 && c >= 2 && c <= 18 && J >= 1 && nsets >= 1 && (uint64_t)c * J * (nsets - 1) < 256, "bad table shape");
+    return wide_table_gen_impl(table, gens, N, c * J, nsets, 1u << (c - 1), st);
+}
+
+// Full-width scalars through a strided table (see commit_strided_kernel): nw = ceil(255 / c) windows,
+// J residues, nsets = ceil(nw / J) table sets of K = 2^(c-1) multiples.
+int grape_commit_fr_strided(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                            uint32_t c, uint32_t J, uint32_t nsets, grape_stream_t st) {
+    if (size == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(size <= kMaxCommitScalars, "more than 2^28 scalars in one call: commit the rows in several calls");
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
+    GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
+    GRAPE_REQUIRE(c >= 2 && c <= 18 && J >= 1, "need 2 <= c <= 18 and J >= 1");
+    const uint32_t nw = (255 + c - 1) / c, K = 1u << (c - 1);
+    GRAPE_REQUIRE(J <= nw && (uint64_t)nsets * J >= nw, "nsets * J must cover ceil(255 / c) windows");
+    const size_t rows = size / rowlen;
+    hipStream_t s = as_stream(st);
+    // (row, residue) pairs are the rows of the accumulation and reduction launches
+    const geom::WidePlan plan = geom::wide_plan(rows * J * (size_t)rowlen, rowlen, geom::kSlabSegments);
+    const uint32_t lg_lpr = plan.lg_lpr, nseg = plan.nseg, seg = plan.seg;
+    size_t slab = plan.slab / J;                              // whole rows per launch
+    if (slab < 1) slab = 1;
+    if (slab > rows) slab = rows;
+    const size_t partial_bytes = slab * J * nseg * 64 * (size_t)(4 * kPartialWords);
+    const size_t sums_bytes = slab * J * (size_t)(4 * kPartialWords);
+    void* ws;
+    int rc = scratch_get(kSlotMsm, partial_bytes + sums_bytes, &ws, s);
+    if (rc) return rc;
+    uint32_t* sums = (uint32_t*)((char*)ws + partial_bytes);
+    const size_t rows_per_wave = (size_t)64 >> lg_lpr;
+    profile_begin();
+    for (size_t r0 = 0; r0 < rows; r0 += slab) {
+        const size_t nr = rows - r0 < slab ? rows - r0 : slab;
+        const uint32_t* sc = scalars + r0 * rowlen * 8;
+        profile_mark(s);
+        commit_strided_kernel<<<blocks_for(nr * J * nseg * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, N, c, nw, K, J, nsets);
+        profile_mark(s);
+        const size_t rj = nr * J;
+        commit_reduce_kernel<false><<<(unsigned)((rj + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rj, nseg * 64, lg_lpr);
+        strided_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, J, c);
+        profile_mark(s);
+    }
+    GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
 

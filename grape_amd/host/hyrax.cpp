@@ -55,6 +55,7 @@ Hyrax::~Hyrax() {
     grape_free(int16x2_table_.d);
     grape_free(int32_table_.d);
     grape_free(fr_table_.d);
+    grape_free(fr_strided_.d);
 }
 
 // src/Hyrax.cu:314-315 / :337-338
@@ -81,6 +82,25 @@ bool Hyrax::ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K) {
     return true;
 }
 
+namespace {
+// One C-ABI commitment call takes at most 2^28 scalars (the largest single call that is tested on the
+// GPU); longer tensors go through in whole rows, each call writing its own rows of the output.
+constexpr size_t kMaxScalarsPerCall = (size_t)1 << 28;
+// fn(first_element, elements, first_row) -> status; stops at the first non-zero status
+template <class F>
+int for_row_chunks(size_t size, uint rowlen, F fn) {
+    size_t rows_per_call = kMaxScalarsPerCall / rowlen;
+    if (rows_per_call < 1) rows_per_call = 1;
+    const size_t rows = size / rowlen;
+    for (size_t r0 = 0; r0 < rows; r0 += rows_per_call) {
+        const size_t nr = rows - r0 < rows_per_call ? rows - r0 : rows_per_call;
+        int rc = fn(r0 * rowlen, nr * rowlen, r0);
+        if (rc != GRAPE_OK) return rc;
+    }
+    return GRAPE_OK;
+}
+}  // namespace
+
 affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;
@@ -95,42 +115,117 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
         if (ensure_table(int16_table_, rowlen, 16, 1, 32768)) t = &int16_table_;
         else if (ensure_table(int16x2_table_, rowlen, 9, 2, 256)) t = &int16x2_table_;
         if (t) {
-            int rc = grape_commit_i32(W(out), tensor, size, rowlen, W(t->d), t->ngen, t->c, t->nw, t->K, nullptr);
+            int rc = for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                return grape_commit_i32(W(out + r0), tensor + e0, n, rowlen, W(t->d), t->ngen, t->c, t->nw, t->K, nullptr);
+            });
             if (rc == GRAPE_OK) return out;
             if (rc != GRAPE_EINVAL) check(rc, "grape_commit_i32");
             int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
         }
     }
     if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
-        check(grape_commit_i32(W(out), tensor, size, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr), "grape_commit_i32");
+        check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  return grape_commit_i32(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr);
+              }),
+              "grape_commit_i32");
     } else {
-        check(grape_commit_i32_ref_table(W(out), tensor, size, rowlen, W(g_affine), npoints, nullptr), "grape_commit_i32_ref_table");
+        check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  return grape_commit_i32_ref_table(W(out + r0), tensor + e0, n, rowlen, W(g_affine), npoints, nullptr);
+              }),
+              "grape_commit_i32_ref_table");
     }
     return out;
 }
 
-// Full-width scalars cost ceil(256/c) additions each, so the widest radix whose table fits the
-// budget is used (from c = 10 up).  For 4096 generators: c = 14 is 19 additions per element (82 GB, what the
-// default budget allows next to the other tables), c = 13 is 20 (43 GB), c = 15 is 17.5 on average
-// (155 GB; measured no faster than c = 14, its gathers miss more), against 32 plus a doubling
-// chain for the reference's byte windows.
+size_t Hyrax::table_bytes_in_use() const {
+    size_t used = scaled_bytes_;
+    for (const WideTable* t : {&int16_table_, &int16x2_table_, &int32_table_, &fr_table_})
+        if (t->d) used += grape_g1_wide_table_bytes(t->ngen, t->nw, t->K);
+    if (fr_strided_.d) used += grape_g1_wide_table_bytes(fr_strided_.ngen, fr_strided_.nsets, 1u << (fr_strided_.c - 1));
+    return used;
+}
+
+// A small per-window table for full-width scalars (every window has its own set of multiples, so a
+// scalar multiple needs additions only): what the scaled table B[t] * G_i of a lookup object is built
+// through, one-off, at 24 additions per entry (c = 11: 13 GB for 4096 generators).  Commitments do
+// not use it when a strided table exists.
 bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
     if (!build) return false;
-    size_t used = 0;
-    if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
-    if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);
-    if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
-    // ceil(255 / c) windows: the kernel takes a scalar of the upper half as -(r - k), so magnitudes
-    // stay below 2^254 and the top signed digit never carries out (c = 15: 17 windows, not 18).
-    // Below c = 10 a wide table (32 additions per element at c = 8) saves nothing over the
-    // reference-format table, whose path needs no build, so very long rows (the reference's
-    // com_scale = 16 shapes: 65536 to 262144 columns) stay on that path.
-    for (uint c = 15; c >= 10; c--) {
-        uint nw = (255 + c - 1) / c, K = 1u << (c - 1);
-        if (used + grape_g1_wide_table_bytes(rowlen, nw, K) <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
+    const size_t used = table_bytes_in_use();
+    for (uint c = 11; c >= 8; c--) {
+        const uint nw = (255 + c - 1) / c, K = 1u << (c - 1);
+        const size_t bytes = grape_g1_wide_table_bytes(rowlen, nw, K);
+        if (bytes <= ((size_t)16 << 30) && used + bytes <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }
     return false;
+}
+
+// Full-width scalars cost one addition per c-bit window, so the table that leaves the fewest
+// additions per scalar within its share of the budget is built: windows of c bits, every J-th
+// window set kept, the J residue sums combined by (J-1)*c doublings per row.  Measured cost per
+// scalar, in additions: ceil(255/c) + 0.3 J (each residue recodes the scalar again).  Half of the
+// budget at most goes to this table - the rest is for the int16 table and the lookups' scaled
+// tables.  4096 generators: c = 16, J = 4, 4 sets, 69 GB, 16 additions (a per-window table of the
+// same bytes has c = 14 and 19); 65536 generators: c = 13, J = 10; 262144: c = 11, J = 12, against
+// 32 additions plus a doubling chain per row for the reference's byte windows.
+bool Hyrax::ensure_strided_table(uint rowlen, bool build) {
+    if (fr_strided_.d && fr_strided_.ngen >= rowlen) return true;
+    if (!build) return false;
+    if (rowlen > npoints) throw std::runtime_error("row longer than the generator set");
+    const size_t used = table_bytes_in_use() - (fr_strided_.d ? grape_g1_wide_table_bytes(fr_strided_.ngen, fr_strided_.nsets, 1u << (fr_strided_.c - 1)) : 0);
+    size_t cap = table_budget_ / 2;
+    if (used + cap > table_budget_) cap = table_budget_ > used ? table_budget_ - used : 0;
+    double best = 30.0;                   // a table that does not beat this is not worth building
+    uint bc = 0, bj = 0, bs = 0;
+    for (uint c = 8; c <= 17; c++) {
+        const uint nw = (255 + c - 1) / c;
+        for (uint J = 1; J <= nw; J++) {
+            const uint nsets = (nw + J - 1) / J;
+            if ((nsets - 1) * J * c >= 256) continue;
+            const size_t bytes = grape_g1_wide_table_bytes(rowlen, nsets, 1u << (c - 1));
+            if (bytes > cap) continue;
+            const double cost = nw + 0.3 * J + (double)bytes / 1e12;
+            if (cost < best) {
+                best = cost;
+                bc = c;
+                bj = J;
+                bs = nsets;
+            }
+        }
+    }
+    if (bc == 0) return false;
+    grape_free(fr_strided_.d);
+    fr_strided_ = StridedTable();
+    check(grape_malloc((void**)&fr_strided_.d, grape_g1_wide_table_bytes(rowlen, bs, 1u << (bc - 1))), "grape_malloc");
+    check(grape_g1_strided_table_gen(W(fr_strided_.d), W(g_affine + npoints), rowlen, bc, bj, bs, nullptr), "grape_g1_strided_table_gen");
+    fr_strided_.ngen = rowlen;
+    fr_strided_.c = bc;
+    fr_strided_.J = bj;
+    fr_strided_.nsets = bs;
+    return true;
+}
+
+void Hyrax::commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build) {
+    // one row only (an opening's blinding row): a table that is already there is used, none is built for it
+    if (ensure_strided_table(rowlen, may_build)) {
+        const StridedTable& t = fr_strided_;
+        check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  return grape_commit_fr_strided(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.J, t.nsets, nullptr);
+              }),
+              "grape_commit_fr_strided");
+    } else if (ensure_fr_table(rowlen, false)) {
+        const WideTable& t = fr_table_;
+        check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  return grape_commit_fr(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, nullptr);
+              }),
+              "grape_commit_fr");
+    } else {
+        check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  return grape_commit_fr_ref_table(W(out + r0), W(scalars + e0), n, rowlen, W(g_affine), npoints, nullptr);
+              }),
+              "grape_commit_fr_ref_table");
+    }
 }
 
 affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
@@ -139,13 +234,7 @@ affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
     const uint rows = size / rowlen;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
-    if (ensure_fr_table(rowlen)) {
-        check(grape_commit_fr(W(out), W(tensor.gpu_data), size, rowlen, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
-                              fr_table_.K, nullptr),
-              "grape_commit_fr");
-    } else {
-        check(grape_commit_fr_ref_table(W(out), W(tensor.gpu_data), size, rowlen, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
-    }
+    commit_fr_rows(out, tensor.gpu_data, size, rowlen, rows > 1);
     return out;
 }
 
@@ -153,11 +242,7 @@ affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
     if (ncols > npoints) throw std::runtime_error("row longer than the generator set");
     if (!ensure_fr_table(ncols)) return nullptr;
     size_t bytes = grape_g1_wide_table_bytes(ncols, 1, scalars.size);   // one entry per (scalar, column)
-    size_t used = scaled_bytes_ + grape_g1_wide_table_bytes(fr_table_.ngen, fr_table_.nw, fr_table_.K);
-    if (int16_table_.d) used += grape_g1_wide_table_bytes(int16_table_.ngen, int16_table_.nw, int16_table_.K);
-    if (int16x2_table_.d) used += grape_g1_wide_table_bytes(int16x2_table_.ngen, int16x2_table_.nw, int16x2_table_.K);
-    if (int32_table_.d) used += grape_g1_wide_table_bytes(int32_table_.ngen, int32_table_.nw, int32_table_.K);
-    if (used + bytes > table_budget_) return nullptr;
+    if (table_bytes_in_use() + bytes > table_budget_) return nullptr;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, bytes), "grape_malloc");
     check(grape_g1_scaled_table_gen(W(out), W(scalars.gpu_data), scalars.size, ncols, W(fr_table_.d), fr_table_.ngen, fr_table_.c,
@@ -187,7 +272,10 @@ affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
     // one unsigned "digit" idx+1 in [1, len]: radix 2^(log2(len)+1) keeps it below the sign threshold
     const uint c = Log2(len) + 1;
-    check(grape_commit_i32(W(out), idx_plus1, size, rowlen, W(scaled_table), ncols, c, 1, len, nullptr), "grape_commit_i32 (indexed)");
+    check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+              return grape_commit_i32(W(out + r0), idx_plus1 + e0, n, rowlen, W(scaled_table), ncols, c, 1, len, nullptr);
+          }),
+          "grape_commit_i32 (indexed)");
     return out;
 }
 
@@ -236,14 +324,7 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185)
     affine_t* com_d_dev = nullptr;
     check(grape_malloc((void**)&com_d_dev, sizeof(affine_t)), "grape_malloc");
-    // one row only: a table that is already there is used, none is built for it
-    if (ensure_fr_table(new_N, false)) {
-        check(grape_commit_fr(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
-                              fr_table_.K, nullptr),
-              "grape_commit_fr");
-    } else {
-        check(grape_commit_fr_ref_table(W(com_d_dev), W(d.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
-    }
+    commit_fr_rows(com_d_dev, d.gpu_data, new_N, new_N, false);
 
     FrTensor x(new_N);
     tensor.partial_eval(size, eval_point, (size / layer_num) / (N * com_scale), Log2(N * com_scale), N * com_scale);
@@ -289,13 +370,7 @@ bool Hyrax::verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr
     FrTensor z = FrTensor::from_host(zv);
     affine_t* com_z_dev = nullptr;
     check(grape_malloc((void**)&com_z_dev, sizeof(affine_t)), "grape_malloc");
-    if (ensure_fr_table(new_N)) {
-        check(grape_commit_fr(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(fr_table_.d), fr_table_.ngen, fr_table_.c, fr_table_.nw,
-                              fr_table_.K, nullptr),
-              "grape_commit_fr");
-    } else {
-        check(grape_commit_fr_ref_table(W(com_z_dev), W(z.gpu_data), new_N, new_N, W(g_affine), npoints, nullptr), "grape_commit_fr_ref_table");
-    }
+    commit_fr_rows(com_z_dev, z.gpu_data, new_N, new_N, false);
     affine_t com_z;
     check(grape_memcpy_d2h(&com_z, com_z_dev, sizeof(affine_t), nullptr), "d2h");
     grape_free(com_z_dev);

@@ -75,10 +75,20 @@ private:
         affine_t* d = nullptr;
         uint ngen = 0, c = 0, nw = 0, K = 0;
     };
+    // every J-th window set of a full-width table: window w = q*J + j is looked up in set q
+    struct StridedTable {
+        affine_t* d = nullptr;
+        uint ngen = 0, c = 0, J = 0, nsets = 0;
+    };
     bool ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K);
-    bool ensure_fr_table(uint rowlen, bool build = true);
+    bool ensure_fr_table(uint rowlen, bool build = true);       // small per-window table (scaled-table builds)
+    bool ensure_strided_table(uint rowlen, bool build = true);  // the table full-width commitments go through
+    size_t table_bytes_in_use() const;
+    // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
+    void commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
+    StridedTable fr_strided_;
     bool int16_ok_ = true;
     size_t scaled_bytes_ = 0;
     std::vector<Fr> last_open_point_;

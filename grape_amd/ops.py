@@ -384,6 +384,23 @@ def commit_fr(scalars, rowlen, table, N, c, nw, K, out=None):
     return out
 
 
+def g1_strided_table_gen(gens, c, J, nsets):
+    lib = init()
+    N = gens.shape[0]
+    nbytes = lib.grape_g1_wide_table_bytes(N, nsets, 1 << (c - 1))
+    table = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_g1_strided_table_gen(_p(table), _p(gens), N, c, J, nsets, _s()))
+    return table
+
+
+def commit_fr_strided(scalars, rowlen, table, N, c, J, nsets, out=None):
+    lib = init()
+    size = scalars.shape[0]
+    out = g1_empty(size // rowlen) if out is None else out
+    _capi.check(lib.grape_commit_fr_strided(_p(out), _p(scalars), size, rowlen, _p(table), N, c, J, nsets, _s()))
+    return out
+
+
 def commit_i32_ref_table(scalars, rowlen, table, npoints):
     lib = init()
     size = scalars.numel()

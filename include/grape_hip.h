@@ -287,7 +287,9 @@ int grape_g1_scaled_table_gen(uint32_t *d_out, const uint32_t *d_scalars_mont, s
  * N >= rowlen generators with radix 2^c, nw windows and K >= 2^(c-1); scalars are recoded into
  * signed radix-2^c digits (2 <= c <= 24 here), so any int32 is accepted when nw*c >= 33, and the
  * int16 fast path (c = 16, nw = 1) requires -32768 <= s <= 32767 (checked on device: returns
- * GRAPE_EINVAL after synchronising if violated).
+ * GRAPE_EINVAL after synchronising if violated).  One call takes at most 2^28 scalars (GRAPE_EINVAL
+ * beyond; every commitment entry point has this bound): rows are independent, so a longer tensor is
+ * committed in several calls, as the host class Hyrax does.
  */
 int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
                      const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
@@ -298,6 +300,21 @@ int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t si
  * never carries out. */
 int grape_commit_fr(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
                     const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/*
+ * Strided fixed-base table: table[(q*K + (k-1))*N + i] = k * 2^(c*J*q) * G_i, k = 1..K = 2^(c-1), q < nsets
+ * (the same entry format as the wide table; size grape_g1_wide_table_bytes(N, nsets, K)), and the
+ * commitment of full-width scalars through it: window w = q*J + j of a scalar is looked up in set q,
+ * the J residues j are summed apart and combined per row as sum_j 2^(c*j) * A_j by (J-1)*c doublings.
+ * For the same bytes as a per-window table this affords wider windows: 16 additions per scalar
+ * (c = 16, J = 4, 68 GB for 4096 generators) against 19 (c = 14, 82 GB), and it reaches generator sets
+ * no per-window table fits (262144 generators: c = 12, J = 22, one set, 68 GB, 22 additions against
+ * the 32 of the reference's byte windows).  Requires nsets * J >= ceil(255 / c), 2 <= c <= 18.
+ * Same results as grape_commit_fr.  Hyrax::commit(FrTensor&, size, N), src/Hyrax.cu:335-359.
+ */
+int grape_g1_strided_table_gen(uint32_t *d_table, const uint32_t *d_gens_affine, size_t N, uint32_t c, uint32_t J, uint32_t nsets,
+                               grape_stream_t stream);
+int grape_commit_fr_strided(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
+                            const uint32_t *d_table, size_t N, uint32_t c, uint32_t J, uint32_t nsets, grape_stream_t stream);
 /* Commitments through the reference-format table (k*G_i, k < 256, byte windows of |s| resp. of
  * the canonical scalar) — the reference's own algorithm, kept for tables loaded from its
  * points.bin.  Output affine. */

@@ -122,4 +122,28 @@ void t28_xyzz_to_affine(const uint32_t* xyzz, uint32_t* out) {
     G1Affine r = xyzz_to_affine(a);
     memcpy(out, &r, 2 * FB);
 }
+// Horner pattern of the strided-table commitment: acc = points[0]; then for each further point
+// `dbl` doublings of the accumulator and one accumulator+accumulator addition; affine result
+void t28_horner(const uint32_t* points, int n, int dbl, uint32_t* out_affine) {
+    Xyzz28 acc = xyzz28_inf();
+    for (int i = 0; i < n; i++) {
+        for (int d = 0; d < dbl && i > 0; d++) xyzz28_dbl(acc);
+        G1Affine p;
+        memcpy(&p, points + 2 * FW * i, 2 * FB);
+        Xyzz28 q = xyzz28_inf();
+        if (!p.is_inf()) {
+            Affine28 a;
+            a.x = fp28::from_canonical(p.x);
+            a.y = fp28::from_canonical(p.y);
+            xyzz28_madd(q, a, false);
+        }
+        if (!xyzz28_add(acc, q)) {
+            G1Xyzz c = xyzz28_to_canonical(acc);
+            xyzz_add(c, xyzz28_to_canonical(q));
+            acc = xyzz28_from_canonical(c);
+        }
+    }
+    G1Affine r = xyzz28_to_affine(acc);
+    memcpy(out_affine, &r, 2 * FB);
+}
 }

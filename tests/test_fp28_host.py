@@ -165,3 +165,23 @@ def test_accumulator_plus_accumulator(lib):
     assert _sum_tree(lib, [a, a], [False, True]) == (None, 1)
     assert _sum_tree(lib, [a], [False]) == (a, 0)
     assert _sum_tree(lib, [a, b, b, a], [False, False, True, True])[0] is None
+
+
+def test_doubling_chain_horner(lib):
+    """sum_j 2^(d j) P_j by Horner with the 28-bit doubling (from the top point down): against the
+    textbook group law for several chain lengths, with identities among the points and after them"""
+    rng = random.Random(6)
+    for n, d in ((1, 3), (2, 1), (3, 16), (5, 7), (4, 17)):
+        ks = [rng.randrange(1, br.R_MOD) for _ in range(n)]
+        pts = _points(ks)
+        if n >= 3:
+            pts[1] = None
+        arr = br.g1_pack(pts).view(np.uint32).reshape(-1)
+        aff = np.zeros(2 * FW, dtype=np.uint32)
+        lib.t28_horner(_u32(np.ascontiguousarray(arr)), n, d, _u32(aff))
+        got = br.g1_unpack(aff.view(np.uint64).reshape(1, br.G1_WORDS))[0]
+        want = None
+        for p in pts:                      # first point is the most significant
+            want = br.g1_mul(1 << d, want) if want is not None else None
+            want = br.g1_add(want, p)
+        assert got == want, (n, d)

@@ -183,6 +183,63 @@ def test_commit_fr_half_range_recoding(ops, gens64):
         ops.commit_fr(ops.to_dev(s), n, wide, n, 15, 16, 1 << 14)       # 240 bits of windows: refused
 
 
+@pytest.mark.parametrize("c,J", [(16, 4), (17, 8), (15, 2), (12, 22), (14, 1), (5, 7), (18, 15), (16, 16), (13, 3)])
+def test_commit_fr_strided_table(ops, gens64, c, J):
+    """full-width scalars through the strided table (every J-th window set, J residue sums combined by
+    doublings, carry-free signed digits): edge scalars one by one and together against the big-integer
+    sum, random rows against the per-window path and the oracle"""
+    k, host, dev = gens64
+    n = 16
+    r = br.R_MOD
+    nw = (255 + c - 1) // c
+    nsets = (nw + J - 1) // J
+    top = 1 << (r.bit_length() - 1)
+    vals = [(r - 1) // 2, (r + 1) // 2, (r - 1) // 2 - 1, (r + 1) // 2 + 1, r - 1, r - 2, 1, 0,
+            top - 1, top, (1 << 240) - 1, r - (1 << 240), 0x7fff7fff7fff7fff7fff, (1 << (c - 1)), (1 << (c - 1)) + 1, 2 * r // 3]
+    s = br.fr_pack(vals)
+    pts = br.g1_unpack(host[:n])
+    table = ops.g1_strided_table_gen(dev[:n].contiguous(), c, J, nsets)
+    got = br.g1_unpack(ops.g1_to_host(ops.commit_fr_strided(ops.to_dev(s), n, table, n, c, J, nsets)))[0]
+    assert got == br.g1_msm(vals, pts)
+    rows = np.zeros((n, n, 4), dtype=np.uint64)
+    for i in range(n):
+        rows[i, i] = s[i]
+    got = br.g1_unpack(ops.g1_to_host(ops.commit_fr_strided(ops.to_dev(rows.reshape(n * n, 4)), n, table, n, c, J, nsets)))
+    for i in range(n):
+        assert got[i] == br.g1_msm([vals[i]], [pts[i]]), (c, J, i)
+    del table
+    # 24 random rows of 64 against the oracle's byte-window commitment (and 3 ragged rows of 40)
+    table = ops.g1_strided_table_gen(dev, c, J, nsets)
+    x = rand_fr(24 * 64, 300 + c)
+    got = ops.g1_to_host(ops.commit_fr_strided(ops.to_dev(x), 64, table, 64, c, J, nsets))
+    assert_same(got, orc.commit_fr(x, orc.g1_table(host, 256), 64, 64), "strided vs oracle")
+    y = rand_fr(3 * 40, 400 + c)
+    got = ops.g1_to_host(ops.commit_fr_strided(ops.to_dev(y), 40, table, 64, c, J, nsets))
+    assert_same(got, orc.commit_fr(y, orc.g1_table(host, 256), 40, 64), "strided, short rows")
+
+
+def test_commit_fr_strided_many_rows_and_long_rows(ops):
+    """more (row, residue) units than one launch takes, and one long row cut into column segments:
+    equal to the per-window path on the same scalars"""
+    k = _scalars(2048, 811)
+    dev = ops.g1_make_generators(k)
+    # 20000 rows of 8 with J = 4: 80000 units, three launches
+    small = dev[:8].contiguous()
+    t1, w1 = ops.g1_strided_table_gen(small, 16, 4, 4), ops.g1_wide_table_gen(small, 8, 32, 128)
+    x = ops.to_dev(rand_fr(20000 * 8, 812))
+    a = ops.commit_fr_strided(x, 8, t1, 8, 16, 4, 4)
+    b = ops.commit_fr(x, 8, w1, 8, 8, 32, 128)
+    import torch
+    assert torch.equal(a, b)
+    # 3 rows of 2048 columns: 32 segments per (row, residue)
+    t2, w2 = ops.g1_strided_table_gen(dev, 12, 22, 1), ops.g1_wide_table_gen(dev, 8, 32, 128)
+    y = ops.to_dev(rand_fr(3 * 2048, 813))
+    assert torch.equal(ops.commit_fr_strided(y, 2048, t2, 2048, 12, 22, 1), ops.commit_fr(y, 2048, w2, 2048, 8, 32, 128))
+    from grape_amd import GrapeError
+    with pytest.raises(GrapeError):
+        ops.commit_fr_strided(y, 2048, t2, 2048, 12, 21, 1)        # 21 residues x 1 set < 22 windows
+
+
 def test_commit_linearity_medium(ops):
     # size-independent property on a larger shape: com(a + b) = com(a) + com(b)
     import torch

@@ -47,8 +47,7 @@ def test_field_tensor_of_more_than_2_pow_31_elements(ops):
 def test_commitment_in_several_slabs_and_the_32_bit_size_bound(ops):
     """more rows than one launch takes (the partial sums of 32768 row segments fill the 512 MiB
     work buffer): rows on both sides of the slab boundary against the oracle and against the same
-    rows committed alone; element counts that do not fit the reference's 32-bit `uint size` are
-    refused before anything is launched"""
+    rows committed alone; more than 2^28 scalars in one call are refused before anything is launched"""
     import ctypes
     import torch
     import orc
@@ -75,12 +74,12 @@ def test_commitment_in_several_slabs_and_the_32_bit_size_bound(ops):
     out_fr = ops.g1_to_host(ops.commit_fr(ops.to_dev(s), rowlen, wide_fr, rowlen, 8, 32, 128))
     sub = np.ascontiguousarray(s.reshape(rows, rowlen, 4)[[32767, 32768, rows - 1]].reshape(-1, 4))
     assert np.array_equal(out_fr[[32767, 32768, rows - 1]], orc.commit_fr(sub, orc.g1_table(host, 256), rowlen, rowlen))
-    # 2^32 elements and more: refused (nothing is read - the pointers are those of the small tensors)
+    # more than 2^28 scalars in one call: refused (nothing is read - the pointers are those of the small tensors)
     lib = _capi.load()
-    for size in ((1 << 32), (1 << 32) + 8 * rowlen):
+    for size in ((1 << 28) + rowlen, (1 << 32), (1 << 32) + 8 * rowlen):
         rc = lib.grape_commit_i32(ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(dW.data_ptr()), size, rowlen,
                                   ctypes.c_void_p(wide.data_ptr()), rowlen, 16, 1, 32768, None)
-        assert rc != 0 and b"32-bit" in lib.grape_last_error()
+        assert rc != 0 and b"2^28" in lib.grape_last_error()
         with pytest.raises(GrapeError):
             _capi.check(lib.grape_commit_fr(ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(dW.data_ptr()), size, rowlen,
                                             ctypes.c_void_p(wide_fr.data_ptr()), rowlen, 8, 32, 128, None))
