@@ -176,30 +176,42 @@ bool Hyrax::ensure_strided_table(uint rowlen, bool build) {
     const size_t used = table_bytes_in_use() - (fr_strided_.d ? grape_g1_wide_table_bytes(fr_strided_.ngen, fr_strided_.nsets, 1u << (fr_strided_.c - 1)) : 0);
     size_t cap = table_budget_ / 2;
     if (used + cap > table_budget_) cap = table_budget_ > used ? table_budget_ - used : 0;
-    double best = 30.0;                   // a table that does not beat this is not worth building
-    uint bc = 0, bj = 0, bs = 0;
-    for (uint c = 8; c <= 17; c++) {
-        const uint nw = (255 + c - 1) / c;
-        for (uint J = 1; J <= nw; J++) {
-            const uint nsets = (nw + J - 1) / J;
-            if ((nsets - 1) * J * c >= 256) continue;
-            const size_t bytes = grape_g1_wide_table_bytes(rowlen, nsets, 1u << (c - 1));
-            if (bytes > cap) continue;
-            const double cost = nw + 0.3 * J + (double)bytes / 1e12;
-            if (cost < best) {
-                best = cost;
-                bc = c;
-                bj = J;
-                bs = nsets;
+    // the cheapest table over `ngen` generators within the cap: cost per scalar, c, J, number of sets
+    struct Choice { double cost; uint c, J, nsets; };
+    auto choose = [&](uint ngen) {
+        Choice best{30.0, 0, 0, 0};       // a table that does not beat 30 additions per scalar is not worth building
+        for (uint c = 8; c <= 17; c++) {
+            const uint nw = (255 + c - 1) / c;
+            for (uint J = 1; J <= nw; J++) {
+                const uint nsets = (nw + J - 1) / J;
+                if ((nsets - 1) * J * c >= 256) continue;
+                const size_t bytes = grape_g1_wide_table_bytes(ngen, nsets, 1u << (c - 1));
+                if (bytes > cap) continue;
+                const double cost = nw + 0.3 * J + (double)bytes / 1e12;
+                if (cost < best.cost) best = Choice{cost, c, J, nsets};
             }
         }
+        return best;
+    };
+    // one table over every generator serves all row lengths; it is preferred to a table over the
+    // first `rowlen` generators (which a longer row would have to replace, at half a second per
+    // build) unless that costs over a quarter more additions per scalar
+    Choice pick = choose(rowlen);
+    uint ngen = rowlen;
+    if (npoints > rowlen) {
+        const Choice all = choose(npoints);
+        if (all.c != 0 && (pick.c == 0 || all.cost <= 1.25 * pick.cost)) {
+            pick = all;
+            ngen = npoints;
+        }
     }
+    const uint bc = pick.c, bj = pick.J, bs = pick.nsets;
     if (bc == 0) return false;
     grape_free(fr_strided_.d);
     fr_strided_ = StridedTable();
-    check(grape_malloc((void**)&fr_strided_.d, grape_g1_wide_table_bytes(rowlen, bs, 1u << (bc - 1))), "grape_malloc");
-    check(grape_g1_strided_table_gen(W(fr_strided_.d), W(g_affine + npoints), rowlen, bc, bj, bs, nullptr), "grape_g1_strided_table_gen");
-    fr_strided_.ngen = rowlen;
+    check(grape_malloc((void**)&fr_strided_.d, grape_g1_wide_table_bytes(ngen, bs, 1u << (bc - 1))), "grape_malloc");
+    check(grape_g1_strided_table_gen(W(fr_strided_.d), W(g_affine + npoints), ngen, bc, bj, bs, nullptr), "grape_g1_strided_table_gen");
+    fr_strided_.ngen = ngen;
     fr_strided_.c = bc;
     fr_strided_.J = bj;
     fr_strided_.nsets = bs;

@@ -270,3 +270,104 @@ def test_fold_msb_multi(ops):
     for t, dt in zip(ts, dts):
         want = orc.partial_eval(t, 2 * n_out, v, 2, 0, n_out)[:n_out]
         assert_same(ops.fr_to_host(dt)[:n_out], want, "msb fold")
+
+
+def test_eq_pyramid_levels(ops):
+    """every level j of the pyramid is eq(u[0..j-1], .): against the product definition, the level's
+    sum (1) and the older doubling table"""
+    u = rand_fr(13, 171)
+    ui = br.fr_unpack(u)
+    pyr = ops.fr_to_host(ops.eq_pyramid(ops.to_dev(u)))
+    assert pyr.shape[0] == (2 << 13) - 1
+    for j in (0, 1, 2, 5, 9, 10, 11, 13):          # 9/10 straddle the one-workgroup head and the per-level launches
+        lvl = br.fr_unpack(pyr[(1 << j) - 1:(2 << j) - 1])
+        assert sum(lvl) % R == 1
+        for i in {0, 1 % (1 << j), (1 << j) - 1, (1 << j) // 3, 77 % (1 << j)}:
+            assert lvl[i] == br.eq_weight(i, ui[:j]), (j, i)
+    assert_same(pyr[(1 << 13) - 1:], ops.fr_to_host(ops.eq_table(ops.to_dev(u))), "top level = eq table")
+    assert br.fr_unpack(ops.fr_to_host(ops.eq_pyramid(ops.to_dev(u), 0))) == [1]
+
+
+@pytest.mark.parametrize("in_size,n_out,beta,plain", [(2, 1, True, True), (8192, 4096, True, True), (8192, 4096, False, False),
+                                                      (6001, 4096, False, False), (1 << 18, 1 << 17, True, True), (70000, 65536, True, False)])
+def test_weighted_round_with_fused_fold(ops, in_size, n_out, beta, plain):
+    """grape_wround2 against the unfused steps: coefficient arrays of the reference's kernel evaluated at
+    the remaining variables (oracle), plain sums, and the MSB fold of both tensors (ragged upper halves
+    read as zero)"""
+    logh = br.log2ceil(n_out)
+    A, S = rand_fr(in_size, 181 + in_size), rand_fr(in_size, 182 + in_size)
+    bt, v, u = rand_fr(1, 183), rand_fr(1, 184), rand_fr(max(logh, 1), 185)
+    Ap, Sp = np.zeros((2 * n_out, 4), dtype=np.uint64), np.zeros((2 * n_out, 4), dtype=np.uint64)
+    Ap[:in_size], Sp[:in_size] = A, S
+    dA, dS = ops.to_dev(A), ops.to_dev(S)
+    e = ops.eq_pyramid(ops.to_dev(u), logh)[n_out - 1:2 * n_out - 1].contiguous()
+    sums = ops.fr_to_host(ops.wround2(dA, dS, ops.to_dev(bt) if beta else None, e, in_size, n_out, ops.to_dev(v), plain_sums=plain))
+    o = [ops.fr_to_host(t) for t in ops.tlookup_poly(ops.to_dev(Ap), ops.to_dev(Sp), ops.to_dev(bt) if beta else None, n_out)]
+    for k in range(3):
+        assert_same(sums[k], orc.mle_eval(o[k], u[:logh]), "weighted coefficient %d" % k)
+    if plain:
+        assert_same(sums[3], orc.fr_sum(Ap[:n_out]), "sum A0")
+        assert_same(sums[4], orc.fr_sub(orc.fr_sum(Ap[n_out:]), orc.fr_sum(Ap[:n_out])), "sum A1 - A0")
+    assert_same(ops.fr_to_host(dA)[:n_out], orc.partial_eval(Ap, 2 * n_out, v, 2, 0, n_out)[:n_out], "folded A")
+    assert_same(ops.fr_to_host(dS)[:n_out], orc.partial_eval(Sp, 2 * n_out, v, 2, 0, n_out)[:n_out], "folded S")
+
+
+def test_weighted_round_on_padded_rows(ops):
+    """rows of 11 elements whose weights live on rows padded to 16: row f, column j takes e[16 f + j]"""
+    rows, rl, rp = 64, 11, 16
+    n_out = rows * rl
+    A, S = rand_fr(2 * n_out, 191), rand_fr(2 * n_out, 192)
+    v, u = rand_fr(1, 193), rand_fr(10, 194)
+    e = ops.eq_pyramid(ops.to_dev(u))[(1 << 10) - 1:].contiguous()        # 64 x 16 weights
+    dA, dS = ops.to_dev(A), ops.to_dev(S)
+    sums = br.fr_unpack(ops.fr_to_host(ops.wround2(dA, dS, None, e, 2 * n_out, n_out, ops.to_dev(v), rowlen=rl, rowpad=rp)))
+    Ai, Si, ui = br.fr_unpack(A), br.fr_unpack(S), br.fr_unpack(u)
+    want = [0, 0, 0]
+    for f in range(rows):
+        for j in range(rl):
+            g = f * rl + j
+            w = br.eq_weight(f * rp + j, ui)
+            a0, a1, s0, s1 = Ai[g], Ai[g + n_out] - Ai[g], Si[g], Si[g + n_out] - Si[g]
+            want[0] += w * a0 * s0
+            want[1] += w * (a0 * s1 + a1 * s0)
+            want[2] += w * a1 * s1
+    assert sums == [x % R for x in want]
+
+
+@pytest.mark.parametrize("nseg,seglen,ragged", [(1, 8, 0), (4, 96, 0), (32, 128, 0), (2, 20000, 0), (8, 300, 1000)])
+def test_segment_weighted_round(ops, nseg, seglen, ragged):
+    """grape_sumcheck_round2_seg: the three sums of every segment of seglen indices times that segment's
+    weight, and the folds - against the plain round kernel run per segment"""
+    out = nseg * seglen
+    in_size = 2 * out - ragged
+    A, B = rand_fr(in_size, 201 + nseg), rand_fr(in_size, 202 + nseg)
+    v, w = rand_fr(1, 203), rand_fr(nseg, 204)
+    dA, dB = ops.to_dev(A), ops.to_dev(B)
+    got = ops.fr_to_host(ops.sumcheck_round2_seg(dA, dB, in_size, out, seglen, ops.to_dev(w), ops.to_dev(v)))
+    wA, wB, wa, wb, wc = _oracle_round2(A, B, in_size, out, v)
+    want = [np.zeros(4, dtype=np.uint64)] * 3
+    for s_ in range(nseg):
+        sl = slice(s_ * seglen, (s_ + 1) * seglen)
+        for k, arr in enumerate((wc, wb, wa)):
+            want[k] = orc.fr_add(want[k], orc.fr_mul(w[s_], orc.fr_sum(arr[sl])))
+    for k in range(3):
+        assert_same(got[k], want[k], "coefficient %d" % k)
+    assert_same(ops.fr_to_host(dA)[:out], wA[:out], "folded A")
+    assert_same(ops.fr_to_host(dB)[:out], wB[:out], "folded B")
+
+
+def test_weighted_sums_of_one_tensor_against_several_tables(ops):
+    n_out, logh, num = 1 << 13, 13, 5
+    for in_size in (2 * n_out, 2 * n_out - 1000):
+        X = rand_fr(in_size, 211)
+        Xp = np.zeros((2 * n_out, 4), dtype=np.uint64)
+        Xp[:in_size] = X
+        us = [rand_fr(logh, 212 + j) for j in range(num)]
+        tabs = [ops.eq_pyramid(ops.to_dev(uj))[n_out - 1:].contiguous() for uj in us]
+        dX = ops.to_dev(X)
+        got = ops.fr_to_host(ops.wsum1_multi(dX, tabs, in_size, n_out))
+        assert_same(ops.fr_to_host(dX), X, "tensor untouched")
+        d = orc.vec2("orc_fr_vec_sub", Xp[n_out:], Xp[:n_out])
+        for j in range(num):
+            assert_same(got[2 * j], orc.mle_eval(Xp[:n_out], us[j]), "claim %d, X0" % j)
+            assert_same(got[2 * j + 1], orc.mle_eval(d, us[j]), "claim %d, X1 - X0" % j)
