@@ -166,14 +166,15 @@ def layer_workload(args):
     def mapping_lookup(x_in, x_out, low, length, fmap):
         a, b = x_in.contiguous().view(-1), x_out.contiguous().view(-1)
         n = a.numel()
-        host.tlookup_mapping_prove(ops.fr_from_i32(a), ops.fr_from_i32(b), n, low, length, fmap, chal(1), chal(1),
-                                   chal(log2c(n)), chal(log2c(n)), table, NPTS, 1, 4096)
+        res = host.tlookup_mapping_prove_ex(ops.fr_from_i32(a), ops.fr_from_i32(b), n, low, length, fmap, chal(1), chal(1),
+                                            chal(log2c(n)), chal(log2c(n)), table, NPTS, 1, 4096)
         times["lookup"] += host.last_prove_seconds()
         times["lookup_commits"] += host.last_commit_seconds()
         counts["lookup"] += 1
         if os.environ.get("GRAPE_BENCH_VERBOSE"):
-            print("  mapping lookup n=%d len=%d: %.4f s (commitments %.4f)" % (n, length, host.last_prove_seconds(),
-                                                                             host.last_commit_seconds()), file=sys.stderr)
+            print("  mapping lookup n=%d len=%d: %.4f s (commitments %.4f; %d table entries with a row of B[t]*G_i, %d elements "
+                  "as full-width scalars)" % (n, length, host.last_prove_seconds(), host.last_commit_seconds(), res[3], res[4]),
+                  file=sys.stderr)
 
     def matmul_proof(a_int, b_int, L, N, M, K, q, r):
         """sumcheck for Y[l][n][m] = sum_k A[l][n][k] B[l][m][k] with claim Y(u), Y = q*2^16 + r"""

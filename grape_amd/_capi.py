@@ -64,6 +64,12 @@ SIGNATURES = {
     "grape_tlookup_index": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
     "grape_tlookup_hist_index": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p],
     "grape_tlookup_inverse_by_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_u32, ctypes.POINTER(c_size_t), c_void_p],
+    "grape_tlookup_hot_select": [c_void_p, c_u32, c_u32, c_u32, c_void_p, c_void_p, ctypes.POINTER(ctypes.c_uint64), c_void_p],
+    "grape_tlookup_hot_index": [c_void_p, c_void_p, c_size_t, c_void_p, c_u32, c_void_p],
+    "grape_fr_mask_cold": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    "grape_fr_gather": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    "grape_commit_fr_sparse": [c_void_p, c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
+    "grape_g1_affine_add": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_init": [c_void_p, c_void_p, c_i32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_tlookup_poly": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_poly_sum": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],

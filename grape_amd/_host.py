@@ -11,7 +11,7 @@ _lib = None
 
 NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
-         "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove",
+         "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove", "grape_host_tlookup_mapping_prove_ex",
          "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
          "grape_host_generate_data", "grape_host_single_commit", "grape_host_layer_witness_new", "grape_host_layer_witness_generate",
          "grape_host_layer_witness_names", "grape_host_layer_witness_tensor", "grape_host_layer_witness_save",
@@ -185,6 +185,24 @@ def tlookup_mapping_prove(dS_in, dS_out, D, low, length, table, alpha, r, u, v, 
                                                 _hp(u), _hp(v), u.shape[0], _dp(d_table), npoints, com_scale, msm_size,
                                                 _hp(tr), ctypes.byref(nr), _hp(sc)))
     return tr[: nr.value].copy(), sc
+
+
+def tlookup_mapping_prove_ex(dS_in, dS_out, D, low, length, table, alpha, r, u, v, d_table, npoints, com_scale, msm_size,
+                             hot_min_count=0):
+    """returns (transcript, S(v), com_A, entries with a table row, elements committed as full-width scalars)"""
+    lib = load()
+    alpha, r, u, v = _fr(alpha, 1), _fr(r, 1), _fr(u), _fr(v)
+    table = np.ascontiguousarray(table, dtype=np.int32)
+    tr = np.zeros((64, 4, 4), dtype=np.uint64)
+    nr = ctypes.c_uint32(0)
+    sc = np.zeros(4, dtype=np.uint64)
+    Dp = 1 << max(0, (D - 1).bit_length())
+    com_a = np.zeros((Dp // (msm_size * com_scale), G1W), dtype=np.uint64)
+    stats = (ctypes.c_uint64 * 2)()
+    _check(lib.grape_host_tlookup_mapping_prove_ex(_dp(dS_in), _dp(dS_out), D, low, length, _hp(table), _hp(alpha), _hp(r),
+                                                   _hp(u), _hp(v), u.shape[0], _dp(d_table), npoints, com_scale, msm_size,
+                                                   _hp(tr), ctypes.byref(nr), _hp(sc), hot_min_count, _hp(com_a), stats))
+    return tr[: nr.value].copy(), sc, com_a, int(stats[0]), int(stats[1])
 
 
 def fr_op(op, a, b=None):

@@ -633,6 +633,53 @@ __global__ void __launch_bounds__(64) strided_horner_kernel(uint32_t* out, const
     st_affine(out, row, xyzz28_to_affine(total));
 }
 
+// ------------------------------------------------------------------------------------------------
+// commitment of the few elements of a tensor that a flag array lets through (full-width scalars)
+// ------------------------------------------------------------------------------------------------
+// One wave per row.  The wave sweeps the row's flags 64 columns at a time and queues the columns
+// whose flag is zero in LDS; whenever 64 are queued (and once more at the end of the row) every lane
+// takes one queued column, loads its scalar and adds scalar * G_col through the per-window table.
+// Lanes therefore work on dense batches however thinly the live elements are spread: sweeping the
+// whole tensor with the dense kernel costs a recoding per element and an addition slot per WAVE
+// that holds one live element - 80 ms for 2^27 elements of which 0.7 % are live, against 3 ms here.
+__global__ void __launch_bounds__(64) commit_sparse_fr_kernel(uint32_t* partial, const uint32_t* scalars, const int32_t* __restrict__ skip,
+                                                              uint32_t rowlen, size_t rows, const uint32_t* table, size_t N,
+                                                              uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
+    __shared__ uint32_t queue[128];
+    const int lane = threadIdx.x;
+    const size_t row = blockIdx.x;
+    if (row >= rows) return;
+    Xyzz28 acc = xyzz28_inf();
+    uint32_t qn = 0;                                     // queued columns (wave-uniform)
+    for (uint32_t base = 0;; base += 64) {
+        const bool last = base >= rowlen;
+        if (!last) {
+            const uint32_t col = base + lane;
+            const bool take = col < rowlen && skip[geom::scalar_index(row, rowlen, col)] == 0;
+            const unsigned long long m = __ballot(take);
+            if (take) queue[qn + __popcll(m & ((1ull << lane) - 1ull))] = col;
+            qn += (uint32_t)__popcll(m);
+            __syncthreads();
+        }
+        if (qn >= 64 || (last && qn > 0)) {
+            const uint32_t n = qn < 64 ? qn : 64;
+            if ((uint32_t)lane < n) {
+                const uint32_t col = queue[lane];
+                const Fr k = from_mont(ld_fr8(scalars, geom::scalar_index(row, rowlen, col)));
+                madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
+            }
+            __syncthreads();
+            const uint32_t moved = (uint32_t)lane + 64 < qn ? queue[lane + 64] : 0u;
+            __syncthreads();
+            if ((uint32_t)lane + 64 < qn) queue[lane] = moved;
+            qn -= n;
+            __syncthreads();
+        }
+        if (last) break;
+    }
+    st_partial28(partial, row * 64 + lane, acc);
+}
+
 // Row epilogue: 2^lg_lpr lanes per row, each sums its share of the partials serially, then a
 // tree over those lanes; the leader maps the row sum to affine coordinates.  All in the 28-bit form.
 template <bool AFFINE>
@@ -757,6 +804,16 @@ __global__ void __launch_bounds__(64) jac_to_affine_kernel(uint32_t* out, const 
     st_affine(out, i, a);
 }
 
+// out[i] = a[i] + b[i] for affine points (either may be the point at infinity, or both equal or opposite)
+__global__ void __launch_bounds__(64) affine_add_kernel(uint32_t* out, const uint32_t* a, const uint32_t* b, size_t n) {
+    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n) return;
+    G1Xyzz acc = G1Xyzz::inf();
+    madd(acc, ld_affine(a, i), false);
+    madd(acc, ld_affine(b, i), false);
+    st_affine(out, i, to_affine(acc));
+}
+
 }  // namespace grape
 
 using namespace grape;
@@ -776,7 +833,10 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
     GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
     GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
-    GRAPE_REQUIRE(c >= 2 && c <= (FR ? 16u : 24u) && nw >= 1 && K >= (1u << (c - 1)), "need 2 <= c <= 16 (24 for int32) and K >= 2^(c-1)");
+    // a single-window table may hold fewer than 2^(c-1) multiples (the indexed commitments: K table
+    // rows, digits 1..K); a digit above K is caught on the device
+    GRAPE_REQUIRE(c >= 2 && c <= (FR ? 16u : 24u) && nw >= 1 && K >= 1 && (K >= (1u << (c - 1)) || (!FR && nw == 1)),
+                  "need 2 <= c <= 16 (24 for int32) and K >= 2^(c-1) (any K >= 1 with one window of int32 digits)");
     if (FR) GRAPE_REQUIRE((uint64_t)nw * c >= 255, "Fr scalars need nw*c >= 255");
     const size_t rows = size / rowlen;
     if (rows == 0) return GRAPE_OK;
@@ -1009,6 +1069,45 @@ int grape_g1_scaled_table_gen(uint32_t* out, const uint32_t* scalars, size_t len
     return GRAPE_OK;
 }
 
+int grape_commit_fr_sparse(uint32_t* out, const uint32_t* scalars, const int32_t* skip, size_t size, uint32_t rowlen,
+                           const uint32_t* table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+    if (size == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(size <= kMaxCommitScalars, "more than 2^28 scalars in one call: commit the rows in several calls");
+    CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
+    GRAPE_REQUIRE(skip != nullptr, "no flag array");
+    GRAPE_REQUIRE(rowlen >= 1 && size % rowlen == 0, "size must be a multiple of rowlen");
+    GRAPE_REQUIRE(rowlen <= N, "row longer than the generator set");
+    GRAPE_REQUIRE(c >= 2 && c <= 16 && (uint64_t)nw * c >= 255 && K >= (1u << (c - 1)), "need a full-width wide table");
+    const size_t rows = size / rowlen;
+    hipStream_t s = as_stream(st);
+    const size_t slab = rows < geom::kSlabSegments ? rows : geom::kSlabSegments;
+    const size_t partial_bytes = slab * geom::kWaveLanes * (size_t)(4 * geom::kPartialWords);
+    void* ws;
+    int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws, s);
+    if (rc) return rc;
+    int* err = (int*)((char*)ws + partial_bytes);
+    rc = zero_fill(err, sizeof(int), s);
+    if (rc) return rc;
+    for (size_t r0 = 0; r0 < rows; r0 += slab) {
+        const size_t nr = rows - r0 < slab ? rows - r0 : slab;
+        const uint32_t lg_lpr = reduce_lanes_log2(nr);
+        const size_t rows_per_wave = (size_t)64 >> lg_lpr;
+        commit_sparse_fr_kernel<<<(unsigned)nr, 64, 0, s>>>((uint32_t*)ws, scalars + r0 * rowlen * 8, skip + r0 * rowlen, rowlen, nr, table, N,
+                                                           c, nw, K, err);
+        commit_reduce_kernel<true><<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW),
+                                                                                                  (const uint32_t*)ws, nr, 64, lg_lpr);
+    }
+    GRAPE_LAUNCH_CHECK();
+    int h_err = 0;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(&h_err, err, sizeof(int), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    if (h_err) {
+        set_error("sparse commit: a scalar digit exceeds the wide table's range");
+        return GRAPE_EINVAL;
+    }
+    return GRAPE_OK;
+}
+
 int grape_commit_i32(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                      uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     return commit_wide_impl<false>(out, scalars, size, rowlen, table, N, c, nw, K, st);
@@ -1038,6 +1137,14 @@ int grape_g1_jacobian_to_affine(uint32_t* out, const uint32_t* in, size_t n, gra
     if (n == 0) return GRAPE_OK;
     CHECK_PTR16(out); CHECK_PTR16(in);
     jac_to_affine_kernel<<<blocks_for(n, 64), 64, 0, as_stream(st)>>>(out, in, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_g1_affine_add(uint32_t* out, const uint32_t* a, const uint32_t* b, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(a); CHECK_PTR16(b);
+    affine_add_kernel<<<blocks_for(n, 64), 64, 0, as_stream(st)>>>(out, a, b, n);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

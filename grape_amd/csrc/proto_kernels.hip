@@ -245,6 +245,71 @@ __global__ void __launch_bounds__(kBlock) inverse_by_table_kernel(uint32_t* A, c
     if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
 }
 
+// ---- occupied-entry ("hot") selection for the commitment of A = B[index]
+// A logUp tensor A takes only the values B[t] of the entries that occur in the witness.  Entries
+// that occur at least min_count times get a slot (in table order, at most max_hot of them): the
+// committer builds B[t]*G_i for those entries only and adds one table point per element; the rest
+// of the elements ("cold") keep their full-width scalars.  One workgroup: every thread counts the
+// hot entries of its contiguous share, an exclusive scan over the threads gives its first slot.
+constexpr int kHotThreads = 1024;
+__global__ void __launch_bounds__(kHotThreads) hot_select_kernel(const uint32_t* __restrict__ hist, uint32_t len, uint32_t min_count,
+                                                                 uint32_t max_hot, int32_t* __restrict__ slot1,
+                                                                 uint32_t* __restrict__ hot_list, unsigned long long* info) {
+    __shared__ uint32_t cnt[kHotThreads];
+    __shared__ unsigned long long cold[kHotThreads];
+    const uint32_t per = (len + kHotThreads - 1) / kHotThreads;
+    const uint32_t t0 = threadIdx.x * per, t1 = t0 + per < len ? t0 + per : len;
+    uint32_t mine = 0;
+    for (uint32_t t = t0; t < t1; t++) mine += hist[t] >= min_count ? 1u : 0u;
+    cnt[threadIdx.x] = mine;
+    __syncthreads();
+    // inclusive scan (Hillis-Steele) over 1024 counters
+    for (int off = 1; off < kHotThreads; off <<= 1) {
+        const uint32_t add = (int)threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
+        __syncthreads();
+        cnt[threadIdx.x] += add;
+        __syncthreads();
+    }
+    uint32_t slot = cnt[threadIdx.x] - mine;          // exclusive prefix
+    unsigned long long cold_mine = 0;
+    for (uint32_t t = t0; t < t1; t++) {
+        const uint32_t h = hist[t];
+        const bool hot = h >= min_count && slot < max_hot;
+        slot1[t] = hot ? (int32_t)(slot + 1) : 0;
+        if (hot) hot_list[slot] = t;
+        if (h >= min_count) slot++;
+        if (!hot) cold_mine += h;
+    }
+    cold[threadIdx.x] = cold_mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long c = 0;
+        for (int i = 0; i < kHotThreads; i++) c += cold[i];
+        const uint32_t total = cnt[kHotThreads - 1];
+        info[0] = total < max_hot ? total : max_hot;
+        info[1] = c;
+    }
+}
+// out[i] = slot + 1 of the element's entry (0: cold entry or outside the table)
+__global__ void __launch_bounds__(kBlock) hot_index_kernel(int32_t* __restrict__ out, const int32_t* __restrict__ idx1, size_t n,
+                                                           const int32_t* __restrict__ slot1, uint32_t len) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t j = (uint32_t)idx1[i];
+    out[i] = (j >= 1 && j <= len) ? slot1[j - 1] : 0;
+}
+// out[i] = X[i] where hot1[i] == 0, zero elsewhere
+__global__ void __launch_bounds__(kBlock) mask_cold_kernel(uint32_t* out, const uint32_t* X, const int32_t* __restrict__ hot1, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, hot1[i] == 0 ? ld_fr(X, i) : Fr::zero());
+}
+__global__ void __launch_bounds__(kBlock) gather_fr_kernel(uint32_t* out, const uint32_t* src, const uint32_t* __restrict__ list, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, ld_fr(src, list[i]));
+}
+
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -614,6 +679,47 @@ int grape_tlookup_index(int32_t* out, const uint32_t* vals, size_t n, int32_t lo
     GRAPE_REQUIRE(out != nullptr && len > 0, "bad arguments");
     CHECK_PTR16(vals);
     index_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, vals, n, low, len);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_hot_select(const uint32_t* hist, uint32_t len, uint32_t min_count, uint32_t max_hot, int32_t* slot1,
+                             uint32_t* hot_list, uint64_t* info, grape_stream_t st) {
+    GRAPE_REQUIRE(hist != nullptr && slot1 != nullptr && hot_list != nullptr && info != nullptr && len > 0, "bad arguments");
+    GRAPE_REQUIRE(min_count >= 1, "min_count must be at least 1");
+    hipStream_t s = as_stream(st);
+    void* d_info;
+    int rc = scratch_get(kSlotMisc, 64, &d_info, s);
+    if (rc) return rc;
+    hot_select_kernel<<<1, kHotThreads, 0, s>>>(hist, len, min_count, max_hot, slot1, hot_list, (unsigned long long*)d_info);
+    GRAPE_LAUNCH_CHECK();
+    GRAPE_HIP_CHECK(hipMemcpyAsync(info, d_info, 2 * sizeof(uint64_t), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    return GRAPE_OK;
+}
+
+int grape_tlookup_hot_index(int32_t* out, const int32_t* idx1, size_t n, const int32_t* slot1, uint32_t len, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    GRAPE_REQUIRE(out != nullptr && idx1 != nullptr && slot1 != nullptr && len > 0, "bad arguments");
+    hot_index_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, idx1, n, slot1, len);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_mask_cold(uint32_t* out, const uint32_t* X, const int32_t* hot1, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(X);
+    GRAPE_REQUIRE(hot1 != nullptr, "bad arguments");
+    mask_cold_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, X, hot1, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_fr_gather(uint32_t* out, const uint32_t* src, const uint32_t* list, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(src);
+    GRAPE_REQUIRE(list != nullptr, "bad arguments");
+    gather_fr_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, src, list, n);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

@@ -229,11 +229,11 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
     GUARD_END
 }
 
-int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S_out, uint32_t D, int32_t low, uint32_t len,
-                                     const int32_t* map, const uint32_t* alpha, const uint32_t* r, const uint32_t* u,
-                                     const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints, uint32_t com_scale,
-                                     uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim) {
-    GUARD_BEGIN
+static void mapping_prove_impl(const uint32_t* d_S_in, const uint32_t* d_S_out, uint32_t D, int32_t low, uint32_t len,
+                               const int32_t* map, const uint32_t* alpha, const uint32_t* r, const uint32_t* u,
+                               const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints, uint32_t com_scale,
+                               uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim,
+                               uint32_t hot_min_count, uint32_t* com_A_out, uint64_t* hot_stats) {
     Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
     // r is drawn in the constructor; to pin it, seed-independent, rebuild the table with the given r
     struct Pinned : tLookupRangeMapping {
@@ -245,6 +245,8 @@ int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S
                               "grape_tlookup_init");
         }
     } lk(low, len, map, fr_from(r));
+    lk.set_indexed_commit(g_indexed_commit);
+    lk.set_hot_min_count(hot_min_count);
     lk.alpha = fr_from(alpha);
     lk.set_u(vec_from(u, nuv));
     uint32_t Dp = 1u << Log2(D);
@@ -260,6 +262,31 @@ int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S
     g_last_commit_s = ct;
     fr_to(S_claim, sc);
     put_transcript(lk.last_transcript, transcript, n_rounds);
+    if (com_A_out) grape_host::check(grape_memcpy_d2h(com_A_out, lk.com_A, sizeof(affine_t) * (size_t)lk.com_A_rows, nullptr), "d2h");
+    if (hot_stats) {
+        hot_stats[0] = lk.hot_entries();
+        hot_stats[1] = lk.cold_elements();
+    }
+}
+
+int grape_host_tlookup_mapping_prove(const uint32_t* d_S_in, const uint32_t* d_S_out, uint32_t D, int32_t low, uint32_t len,
+                                     const int32_t* map, const uint32_t* alpha, const uint32_t* r, const uint32_t* u,
+                                     const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints, uint32_t com_scale,
+                                     uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim) {
+    GUARD_BEGIN
+    mapping_prove_impl(d_S_in, d_S_out, D, low, len, map, alpha, r, u, v, nuv, d_table, npoints, com_scale, msm_size, transcript,
+                       n_rounds, S_claim, 0, nullptr, nullptr);
+    GUARD_END
+}
+
+int grape_host_tlookup_mapping_prove_ex(const uint32_t* d_S_in, const uint32_t* d_S_out, uint32_t D, int32_t low, uint32_t len,
+                                        const int32_t* map, const uint32_t* alpha, const uint32_t* r, const uint32_t* u,
+                                        const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints,
+                                        uint32_t com_scale, uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds,
+                                        uint32_t* S_claim, uint32_t hot_min_count, uint32_t* com_A_out, uint64_t* hot_stats) {
+    GUARD_BEGIN
+    mapping_prove_impl(d_S_in, d_S_out, D, low, len, map, alpha, r, u, v, nuv, d_table, npoints, com_scale, msm_size, transcript,
+                       n_rounds, S_claim, hot_min_count, com_A_out, hot_stats);
     GUARD_END
 }
 

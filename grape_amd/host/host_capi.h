@@ -67,6 +67,16 @@ int grape_host_tlookup_mapping_prove(const uint32_t *d_S_in, const uint32_t *d_S
                                      const uint32_t *u, const uint32_t *v, uint32_t nuv, const uint32_t *d_table,
                                      uint32_t npoints, uint32_t com_scale, uint32_t msm_size, uint32_t *transcript,
                                      uint32_t *n_rounds, uint32_t *S_claim);
+/* The same, with the count from which a table entry gets a row of the per-proof table B[t]*G_i
+ * (0 = the break-even count), the commitment of A (affine, D / (msm_size*com_scale) points) and
+ * hot_stats[0] = entries that got a row, hot_stats[1] = elements committed as full-width scalars
+ * (both zero when the plain path was taken). */
+int grape_host_tlookup_mapping_prove_ex(const uint32_t *d_S_in, const uint32_t *d_S_out, uint32_t D, int32_t low,
+                                        uint32_t len, const int32_t *map, const uint32_t *alpha, const uint32_t *r,
+                                        const uint32_t *u, const uint32_t *v, uint32_t nuv, const uint32_t *d_table,
+                                        uint32_t npoints, uint32_t com_scale, uint32_t msm_size, uint32_t *transcript,
+                                        uint32_t *n_rounds, uint32_t *S_claim, uint32_t hot_min_count, uint32_t *com_A_out,
+                                        uint64_t *hot_stats);
 /* Host-side scalar arithmetic checks: out = a op b with op in {0:+, 1:-, 2:*, 3: a^-1}. */
 int grape_host_fr_op(int op, const uint32_t *a, const uint32_t *b, uint32_t *out);
 /* k * G as a host computation (affine out) */

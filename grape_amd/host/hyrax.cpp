@@ -283,11 +283,26 @@ affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
     // one unsigned "digit" idx+1 in [1, len]: radix 2^(log2(len)+1) keeps it below the sign threshold
-    const uint c = Log2(len) + 1;
+    const uint c = Log2(len) + 1 < 2 ? 2 : Log2(len) + 1;
     check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
               return grape_commit_i32(W(out + r0), idx_plus1 + e0, n, rowlen, W(scaled_table), ncols, c, 1, len, nullptr);
           }),
           "grape_commit_i32 (indexed)");
+    return out;
+}
+
+affine_t* Hyrax::commit_sparse_affine(FrTensor& tensor, int* skip, uint size, uint N) {
+    check_shape(size, N);
+    const uint rowlen = N * com_scale;
+    if (!ensure_fr_table(rowlen, false)) return nullptr;
+    const WideTable& t = fr_table_;
+    const uint rows = size / rowlen;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)rows), "grape_malloc");
+    check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+              return grape_commit_fr_sparse(W(out + r0), W(tensor.gpu_data + e0), skip + e0, n, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, nullptr);
+          }),
+          "grape_commit_fr_sparse");
     return out;
 }
 

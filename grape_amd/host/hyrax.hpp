@@ -66,9 +66,18 @@ public:
     // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
     affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len);
 
+    // Row commitments of the elements whose flag skip[j] is zero, the others left out; through the
+    // per-window table that scaled tables are built with.  nullptr when that table does not exist.
+    affine_t* commit_sparse_affine(FrTensor& tensor, int* skip, uint size, uint N);
+
     // Upper bound for the wide fixed-base tables this object may build (default 128 GiB of the 288 GB; GRAPE_TABLE_BUDGET_GIB overrides).  When a
     // table would not fit, commitments go through the reference-format table instead.
     void set_table_budget(size_t bytes) { table_budget_ = bytes; }
+    // bytes of that budget not taken by tables that exist now
+    size_t table_bytes_free() const {
+        const size_t used = table_bytes_in_use();
+        return used < table_budget_ ? table_budget_ - used : 0;
+    }
 
 private:
     struct WideTable {

@@ -32,10 +32,12 @@ void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
     d_idx_ = padded;
 }
 void tLookup::drop_index() {
-    if (d_idx_) {
+    if (d_idx_ || d_hist_) {
         check(grape_stream_sync(nullptr), "sync");
         grape_free(d_idx_);
+        grape_free(d_hist_);
         d_idx_ = nullptr;
+        d_hist_ = nullptr;
     }
 }
 // multiplicities from the indices (get_histogram_kernel, src/tlookup.cu:5-14, with the padding
@@ -53,7 +55,73 @@ void tLookup::index_to_m(uint witness_size, int low_) {
     }
     m.get_data(m.size, hist);
     check(grape_stream_sync(nullptr), "sync");
-    grape_free(hist);
+    grape_free(d_hist_);
+    d_hist_ = hist;                           // kept for the proof in flight: the commitment of A picks its table entries by count
+}
+
+// com(A) through the entries that occur often.  A[i] = B[index_i]; an entry t that occurs n_t times
+// costs n_t full-width scalars (16 additions each with the strided table) on the plain path, or one
+// row B[t]*G_i of the scaled table (rowlen entries at about 27 additions each, built for this proof
+// only) plus n_t single additions.  So an entry is worth a row when n_t > 1.8 rowlen; with the
+// activations of a transformer layer nearly all elements sit on such entries.  Elements of the
+// other entries keep their scalars and are committed on the plain path; the two sums are added.
+// Returns false (nothing committed) when no entry qualifies or the table does not fit.
+bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& hyrax) {
+    const uint N = T.size;
+    const uint rowlen = msm_size * hyrax.com_scale;
+    const uint rows = D / rowlen;
+    const uint min_count = hot_min_count_ ? hot_min_count_ : (uint)(1.8 * rowlen) + 1;
+    const size_t row_bytes = grape_g1_wide_table_bytes(rowlen, 1, 1);
+    const size_t free_bytes = hyrax.table_bytes_free();
+    size_t max_hot = free_bytes / row_bytes;
+    if (max_hot > N) max_hot = N;
+    if (max_hot == 0) return false;
+    int* d_slot1 = nullptr;
+    uint32_t* d_list = nullptr;
+    int* d_hot = nullptr;
+    affine_t* table = nullptr;
+    affine_t* com_cold = nullptr;
+    bool done = false;
+    try {
+        check(grape_malloc((void**)&d_slot1, sizeof(int) * (size_t)N), "grape_malloc");
+        check(grape_malloc((void**)&d_list, sizeof(uint32_t) * (size_t)N), "grape_malloc");
+        uint64_t info[2] = {0, 0};
+        check(grape_tlookup_hot_select(d_hist_, N, min_count, (uint32_t)max_hot, d_slot1, d_list, info, nullptr), "grape_tlookup_hot_select");
+        const uint n_hot = (uint)info[0];
+        if (n_hot != 0) {
+            FrTensor Bhot(n_hot);
+            check(grape_fr_gather(W(Bhot.gpu_data), W(B.gpu_data), d_list, n_hot, nullptr), "grape_fr_gather");
+            table = hyrax.build_scaled_table(Bhot, rowlen);
+        }
+        if (table) {
+            check(grape_malloc((void**)&d_hot, sizeof(int) * (size_t)D), "grape_malloc");
+            check(grape_tlookup_hot_index(d_hot, d_idx_, D, d_slot1, N, nullptr), "grape_tlookup_hot_index");
+            com_A = hyrax.commit_indexed_affine(d_hot, D, msm_size, table, rowlen, n_hot);
+            if (info[1] != 0) {
+                // the elements without a table row: queued per row and committed as full-width scalars
+                com_cold = hyrax.commit_sparse_affine(A, d_hot, D, msm_size);
+                if (!com_cold) {
+                    FrTensor Acold(D);
+                    check(grape_fr_mask_cold(W(Acold.gpu_data), W(A.gpu_data), d_hot, D, nullptr), "grape_fr_mask_cold");
+                    com_cold = hyrax.commit_affine(Acold, D, msm_size);
+                }
+                check(grape_g1_affine_add((uint32_t*)com_A, (const uint32_t*)com_A, (const uint32_t*)com_cold, rows, nullptr),
+                      "grape_g1_affine_add");
+            }
+            hot_entries_ = n_hot;
+            cold_elements_ = info[1];
+            done = true;
+        }
+        check(grape_stream_sync(nullptr), "sync");
+    } catch (...) {
+        grape_stream_sync(nullptr);
+        grape_free(d_slot1); grape_free(d_list); grape_free(d_hot); grape_free(com_cold);
+        Hyrax::release_scaled_table(table);
+        throw;
+    }
+    grape_free(d_slot1); grape_free(d_list); grape_free(d_hot); grape_free(com_cold);
+    Hyrax::release_scaled_table(table);
+    return done;
 }
 
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
@@ -136,6 +204,8 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             com_A = hyrax.commit_indexed_affine(d_idx, D, msm_size, scaled_table_, scaled_cols_, N);
             check(grape_stream_sync(nullptr), "sync");
             if (d_idx != d_idx_) grape_free(d_idx);
+        } else if (indexed_commit_ && from_table && d_idx_ && d_hist_ && D / rowlen > 1 && commit_A_by_occupancy(A, D, msm_size, hyrax)) {
+            // committed through a table of the entries that occur often
         } else {
             com_A = hyrax.commit_affine(A, D, msm_size);
         }

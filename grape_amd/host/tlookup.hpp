@@ -34,6 +34,12 @@ public:
     // B[t]*G_i built once per object - one addition per element instead of one per scalar digit.
     // The commitment is the same group element either way.
     void set_indexed_commit(bool on) { indexed_commit_ = on; }
+    // Where no table over every entry fits (mapping lookups), A is committed through a table of
+    // the entries that occur at least `n` times in the witness, built for that proof (0 = the
+    // break-even count, 1.8 times the row length).  What the last prove() did is reported below.
+    void set_hot_min_count(uint n) { hot_min_count_ = n; }
+    uint hot_entries() const { return hot_entries_; }
+    uint64_t cold_elements() const { return cold_elements_; }
 
 protected:
     Fr run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
@@ -49,6 +55,11 @@ protected:
     void drop_index();
     void pad_index(uint N, uint pad_N, uint pad_size, int fill);   // rows of N indices -> rows of pad_N
     void index_to_m(uint witness_size, int low_);
+    uint32_t* d_hist_ = nullptr;        // counts per table entry of the proof in flight (made by index_to_m)
+    uint hot_min_count_ = 0;
+    uint hot_entries_ = 0;
+    uint64_t cold_elements_ = 0;
+    bool commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& hyrax);
     affine_t* scaled_table_ = nullptr;  // B[t]*G_i, built on first use
     uint scaled_cols_ = 0;
     Hyrax* scaled_for_ = nullptr;

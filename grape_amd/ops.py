@@ -215,6 +215,53 @@ def tlookup_hist_index(idx1, length, hist=None):
     return hist
 
 
+def tlookup_hot_select(hist, min_count, max_hot):
+    """returns (slot1, hot_list[:n_hot], n_hot, cold_elements)"""
+    lib = init()
+    length = hist.shape[0]
+    slot1 = torch.empty(length, dtype=torch.int32, device="cuda")
+    hot = torch.empty(length, dtype=torch.int32, device="cuda")
+    info = (ctypes.c_uint64 * 2)()
+    _capi.check(lib.grape_tlookup_hot_select(_p(hist), length, min_count, max_hot, _p(slot1), _p(hot), info, _s()))
+    return slot1, hot[:int(info[0])], int(info[0]), int(info[1])
+
+
+def tlookup_hot_index(idx1, slot1):
+    lib = init()
+    out = torch.empty_like(idx1)
+    _capi.check(lib.grape_tlookup_hot_index(_p(out), _p(idx1), idx1.shape[0], _p(slot1), slot1.shape[0], _s()))
+    return out
+
+
+def fr_mask_cold(X, hot1):
+    lib = init()
+    out = fr_empty(X.shape[0])
+    _capi.check(lib.grape_fr_mask_cold(_p(out), _p(X), _p(hot1), X.shape[0], _s()))
+    return out
+
+
+def fr_gather(src, index_list):
+    lib = init()
+    out = fr_empty(index_list.shape[0])
+    _capi.check(lib.grape_fr_gather(_p(out), _p(src), _p(index_list), index_list.shape[0], _s()))
+    return out
+
+
+def commit_fr_sparse(scalars, skip, rowlen, table, N, c, nw, K):
+    lib = init()
+    size = scalars.shape[0]
+    out = g1_empty(size // rowlen)
+    _capi.check(lib.grape_commit_fr_sparse(_p(out), _p(scalars), _p(skip), size, rowlen, _p(table), N, c, nw, K, _s()))
+    return out
+
+
+def g1_affine_add(a, b):
+    lib = init()
+    out = g1_empty(a.shape[0])
+    _capi.check(lib.grape_g1_affine_add(_p(out), _p(a), _p(b), a.shape[0], _s()))
+    return out
+
+
 def tlookup_inverse_by_table(S, idx1, T, B, A=None):
     """returns (A, mismatches)"""
     lib = init()

@@ -211,6 +211,29 @@ int grape_tlookup_hist_index(uint32_t *d_hist, const int32_t *d_idx1, size_t n, 
  * grape_fr_shift_inverse instead. */
 int grape_tlookup_inverse_by_table(uint32_t *d_A, const uint32_t *d_S, const int32_t *d_idx1, const uint32_t *d_T,
                                    const uint32_t *d_B, size_t n, uint32_t len, size_t *mismatches, grape_stream_t stream);
+/*
+ * Occupied-entry selection for the commitment of a logUp tensor A = B[index] whose table is too
+ * large for a table of B[t]*G_i over every entry t (the mapping lookups' 2^19..2^20 entries): the
+ * elements of A take only the values of the entries that occur in the witness, and activations
+ * concentrate on few of them.  Entries with d_hist[t] >= min_count get a slot, in table order, at
+ * most max_hot of them: d_slot1[t] = slot + 1 (0 for the others), d_hot_list[slot] = t.
+ * info (HOST, two words; the call synchronises): info[0] = number of slots given, info[1] =
+ * number of witness elements whose entry got none.  The committer then builds the scaled table of
+ * B[d_hot_list[.]] (grape_fr_gather + grape_g1_scaled_table_gen), commits the slotted elements at
+ * one addition each (grape_tlookup_hot_index + grape_commit_i32) and the others as full-width
+ * scalars (grape_fr_mask_cold + grape_commit_fr*), and adds the two (grape_g1_affine_add).  The
+ * reference commits A as a full-width tensor (src/tlookup.cu:320, :433); the group elements are
+ * the same.  No counterpart in the reference.
+ */
+int grape_tlookup_hot_select(const uint32_t *d_hist, uint32_t len, uint32_t min_count, uint32_t max_hot, int32_t *d_slot1,
+                             uint32_t *d_hot_list, uint64_t *info, grape_stream_t stream);
+/* out[i] = d_slot1[d_idx1[i] - 1] (0 when d_idx1[i] is 0 or above len). */
+int grape_tlookup_hot_index(int32_t *d_out, const int32_t *d_idx1, size_t n, const int32_t *d_slot1, uint32_t len,
+                            grape_stream_t stream);
+/* out[i] = X[i] where d_hot1[i] == 0, zero elsewhere (n field elements). */
+int grape_fr_mask_cold(uint32_t *d_out, const uint32_t *d_X, const int32_t *d_hot1, size_t n, grape_stream_t stream);
+/* out[i] = src[d_list[i]] (n field elements). */
+int grape_fr_gather(uint32_t *d_out, const uint32_t *d_src, const uint32_t *d_list, size_t n, grape_stream_t stream);
 /* T[i] = low + i (+ r*map[i] when d_map != NULL), B[i] = 1/(T[i] + beta).
  * tlookuprange_init_kernel / tLookupRangeMapping_init_kernel, src/tlookup.cu:16-50. */
 int grape_tlookup_init(uint32_t *d_T, uint32_t *d_B, int32_t low, uint32_t len, const uint32_t *d_beta,
@@ -284,7 +307,8 @@ int grape_g1_scaled_table_gen(uint32_t *d_out, const uint32_t *d_scalars_mont, s
  * C_row = sum_i s[row*rowlen + i] * G_i, i < rowlen, written as AFFINE points (96 bytes each).
  * Hyrax::commit(int*, size, N), src/Hyrax.cu:312-333 (int_windows_sum :46-65, int_windows_reduce
  * :67-87); rowlen is the reference's N*com_scale.  The wide table must have been built for
- * N >= rowlen generators with radix 2^c, nw windows and K >= 2^(c-1); scalars are recoded into
+ * N >= rowlen generators with radix 2^c, nw windows and K >= 2^(c-1) (with nw = 1 any K >= 1: the
+ * indexed commitments pass digits 1..K, and a larger digit returns GRAPE_EINVAL); scalars are recoded into
  * signed radix-2^c digits (2 <= c <= 24 here), so any int32 is accepted when nw*c >= 33, and the
  * int16 fast path (c = 16, nw = 1) requires -32768 <= s <= 32767 (checked on device: returns
  * GRAPE_EINVAL after synchronising if violated).  One call takes at most 2^28 scalars (GRAPE_EINVAL
@@ -323,6 +347,19 @@ int grape_commit_i32_ref_table(uint32_t *d_out_affine, const int32_t *d_scalars,
 int grape_commit_fr_ref_table(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
                               const uint32_t *d_table_affine, size_t npoints, grape_stream_t stream);
 /* Format conversions for callers that keep the reference's jacob_t arrays. */
+/* Row commitments of the elements of a full-width tensor whose flag is zero (d_skip[i] != 0 leaves
+ * element i out): C_row = sum_{i : d_skip[row*rowlen+i] == 0} s[row*rowlen+i] * G_i, through a
+ * per-window full-width table (grape_g1_wide_table_gen with nw*c >= 255).  Made for tensors of
+ * which a small share is live (the elements of a logUp tensor that the occupied-entry table of
+ * grape_tlookup_hot_select does not cover): live columns are queued per row and worked on in dense
+ * batches.  No counterpart in the reference (it commits the whole tensor, src/tlookup.cu:320). */
+int grape_commit_fr_sparse(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, const int32_t *d_skip, size_t size,
+                           uint32_t rowlen, const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K,
+                           grape_stream_t stream);
+/* out[i] = a[i] + b[i] for n affine points (infinity, equal and opposite operands included); the
+ * group law of include/curve/xyzz_t.cuh.  Combines two partial row commitments. */
+int grape_g1_affine_add(uint32_t *d_out_affine, const uint32_t *d_a_affine, const uint32_t *d_b_affine, size_t n,
+                        grape_stream_t stream);
 int grape_g1_affine_to_jacobian(uint32_t *d_out_jac, const uint32_t *d_in_affine, size_t n, grape_stream_t stream);
 int grape_g1_jacobian_to_affine(uint32_t *d_out_affine, const uint32_t *d_in_jac, size_t n, grape_stream_t stream);
 

@@ -302,3 +302,30 @@ def test_reference_table_path_in_every_launch_shape(ops):
         got = ops.g1_to_host(ops.commit_i32_ref_table(d, rowlen, dtab, 512))
         want = ops.g1_to_host(ops.commit_i32(d, rowlen, wide_i, 512, 8, 5, 128))
         assert_same(got, want, "i32 ref table %dx%d" % (rows, rowlen))
+
+
+@pytest.mark.parametrize("rowlen,rows,live", [(16, 5, 0.3), (200, 7, 0.02), (200, 7, 0.9), (64, 3, 0.0), (1000, 4, 0.07)])
+def test_commit_fr_sparse_against_dense_commitment_of_masked_tensor(ops, rowlen, rows, live):
+    """the commitment of the flagged-in elements only (queued per row, dense batches of 64, a last
+    partial batch, rows with none) equals the dense commitment of the tensor with the others zeroed,
+    and the oracle's on a few rows"""
+    import torch
+    k = _scalars(rowlen, 131)
+    dev = ops.g1_make_generators(k)
+    rng = np.random.default_rng(rowlen + rows)
+    s = rand_fr(rows * rowlen, 132)
+    skip = (rng.random(rows * rowlen) >= live).astype(np.int32) * rng.integers(1, 9, size=rows * rowlen).astype(np.int32)
+    if live > 0:
+        skip[rowlen: 2 * rowlen] = 1                                   # one row with nothing live
+    c, nw, K = 11, 24, 1024
+    wide = ops.g1_wide_table_gen(dev, c, nw, K)
+    got = ops.g1_to_host(ops.commit_fr_sparse(ops.to_dev(s), torch.from_numpy(skip).cuda(), rowlen, wide, rowlen, c, nw, K))
+    masked = s.copy()
+    masked[skip != 0] = 0
+    want = ops.g1_to_host(ops.commit_fr(ops.to_dev(masked), rowlen, wide, rowlen, c, nw, K))
+    assert_same(got, want, "sparse == dense of the masked tensor")
+    if live > 0:
+        assert not got[1].any()                                        # the empty row commits to infinity
+    if rowlen <= 200:
+        tab = orc.g1_table(orc.g1_make_generators(k), 256)
+        assert_same(got[:1], orc.commit_fr(masked[:rowlen], tab, rowlen, rowlen), "oracle, first row")

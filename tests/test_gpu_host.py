@@ -416,3 +416,111 @@ def test_cpp_reference_programs_run(ops, tmp_path):
     res = subprocess.run([exe, str(tmp_path / "artefacts")], capture_output=True, text=True, timeout=280)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
     assert "programs_flow OK" in res.stdout
+
+
+@pytest.mark.parametrize("hot_min_count,pad", [(0, False), (1, False), (40, False), (300, False), (40, True)])
+def test_tlookup_mapping_commits_A_through_occupied_entries(ops, host, gens, hot_min_count, pad):
+    """com(A) of a mapping lookup through a per-proof table of the entries that occur often: the
+    witness sits on a few entries of a 4096-entry table (activations do), the rest of it is spread.
+    Whatever the split between table rows and full-width scalars (none with the break-even count of
+    this tiny shape, every occupied entry with 1, a mix with 40 or 300), the commitment is the
+    oracle's commitment of A = 1/(S + beta), and the transcript does not change."""
+    import torch
+    hg, dg = gens
+    logN, low = 12, -2048
+    N = 1 << logN
+    D = 2 * 11008 if pad else 1 << 13
+    rng = np.random.default_rng(71 + hot_min_count)
+    fmap = rng.integers(-1000, 1000, size=N).astype(np.int32)
+    S_in = np.clip(np.rint(rng.normal(0.0, 6.0, size=D)), low, low + N - 1).astype(np.int32)
+    spread = rng.random(D) < 0.1
+    S_in[spread] = rng.integers(low, low + N, size=int(spread.sum()))
+    S_out = fmap[S_in - low]
+    logDp = 15 if pad else 13
+    alpha, r, u, v = rand_fr(1, 72), rand_fr(1, 73), rand_fr(logDp, 74), rand_fr(logDp, 75)
+    beta = br.fr_pack([N])[0]
+    T, B = orc.tlookup_init(low, N, beta, orc.from_i32(fmap), r[0])
+    m = orc.tlookup_prep(orc.from_i32(S_in), low, N)
+    S = orc.vec2("orc_fr_vec_add", orc.vec_bcast("orc_fr_vec_bcast_mul", orc.from_i32(S_out), r[0]), orc.from_i32(S_in))
+    if pad:
+        pad_val = orc.fr_mul(orc.from_i32(fmap[-low: -low + 1])[0], r[0])
+        Spad = np.zeros((32768, 4), dtype=np.uint64)
+        orc.lib().orc_fr_pad(orc.P(Spad), orc.P(S), orc.c32(11008), orc.c32(16384), orc.c64(32768), orc.P(pad_val))
+        S = Spad
+    st, wtr, wsc = orc.tlookup_prove(S, T, B, m, alpha[0], beta, u, v)
+    assert st == 0
+    msm = 64
+    table = ops.g1_table_gen(dg[:msm].contiguous(), 256)
+    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
+    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
+    tr, sc, com_a, n_hot, n_cold = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, msm, 1, msm,
+                                                                 hot_min_count=hot_min_count)
+    assert_same(tr, wtr, "transcript")
+    assert_same(sc, wsc, "S(v)")
+    counts = np.bincount(S_in.astype(np.int64) - low, minlength=N)
+    if pad:
+        counts[-low] += 32768 - D
+    thr = hot_min_count if hot_min_count else int(1.8 * msm) + 1
+    assert n_hot == int((counts >= thr).sum())
+    assert n_cold == int(counts[counts < thr].sum())
+    if hot_min_count == 1:
+        assert n_cold == 0
+    if hot_min_count in (40, 300):
+        assert n_hot > 0 and n_cold > 0
+    Ainv = orc.vec1("orc_fr_vec_inv", orc.vec_bcast("orc_fr_vec_bcast_add", S, beta))
+    tab = orc.g1_table(hg[:msm], 256)
+    nrows = S.shape[0] // msm
+    assert com_a.shape[0] == nrows
+    rows = sorted({0, 1, nrows // 2, nrows - 2, nrows - 1} | set(rng.integers(0, nrows, 16).tolist()))
+    for rr in rows:
+        assert_same(com_a[rr:rr + 1], orc.commit_fr(Ainv[rr * msm:(rr + 1) * msm], tab, msm, msm), "com(A) row %d" % rr)
+
+
+def test_occupied_entry_selection_kernels(ops):
+    """the device steps of the occupancy commitment against numpy: slots in table order for entries at
+    or above the count, the cap on the number of slots, the cold element count, the remapped
+    indices, the masked tensor, the gathered scalars; and the affine sum of two commitments
+    (equal, opposite and infinite operands included) against the oracle's group law"""
+    import torch
+    rng = np.random.default_rng(81)
+    N, n = 5000, 100000
+    idx1 = rng.integers(0, N + 1, size=n).astype(np.int32)          # 0 = outside the table
+    idx1[: n // 2] = rng.integers(1, 40, size=n // 2)
+    hist = np.bincount(idx1[idx1 > 0].astype(np.int64) - 1, minlength=N).astype(np.int32)
+    for min_count, max_hot in [(1, N), (50, N), (50, 7), (10 ** 6, N)]:
+        slot1, hot, n_hot, n_cold = ops.tlookup_hot_select(torch.from_numpy(hist).cuda(), min_count, max_hot)
+        want_hot = np.nonzero(hist >= min_count)[0][:max_hot]
+        assert n_hot == len(want_hot) and np.array_equal(hot.cpu().numpy(), want_hot)
+        want_slot = np.zeros(N, dtype=np.int32)
+        want_slot[want_hot] = np.arange(1, len(want_hot) + 1)
+        assert np.array_equal(slot1.cpu().numpy(), want_slot)
+        assert n_cold == int(hist.sum()) - int(hist[want_hot].sum())
+        d_idx = torch.from_numpy(idx1).cuda()
+        h1 = ops.tlookup_hot_index(d_idx, slot1).cpu().numpy()
+        assert np.array_equal(h1, np.where(idx1 > 0, want_slot[np.maximum(idx1, 1) - 1], 0))
+    X = rand_fr(3000, 82)
+    h = rng.integers(0, 3, size=3000).astype(np.int32)
+    got = ops.fr_to_host(ops.fr_mask_cold(ops.to_dev(X), torch.from_numpy(h).cuda()))
+    want = X.copy()
+    want[h != 0] = 0
+    assert_same(got, want, "masked")
+    lst = rng.integers(0, 3000, size=777).astype(np.int32)
+    assert_same(ops.fr_to_host(ops.fr_gather(ops.to_dev(X), torch.from_numpy(lst).cuda())), X[lst], "gathered")
+    # affine sums
+    k = rand_fr(40, 83)
+    hp = orc.g1_make_generators(k)
+    a, b = hp[:20].copy(), hp[20:].copy()
+    b[0] = a[0]                                   # doubling
+    half = a.shape[1] // 2
+    b[1, :half] = a[1, :half]
+    b[1, half:] = orc.fp_neg(a[1, half:])         # opposite -> infinity
+    a[2] = 0                                      # infinity + Q
+    b[3] = 0                                      # P + infinity
+    a[4] = 0
+    b[4] = 0
+    got = ops.g1_to_host(ops.g1_affine_add(ops.to_dev(a), ops.to_dev(b)))
+    want = np.zeros_like(a)
+    for i in range(a.shape[0]):
+        orc.lib().orc_g1_add_affine(orc.P(want[i]), orc.P(a[i]), orc.P(b[i]))
+    assert not want[1].any() and not want[4].any() and np.array_equal(want[2], b[2]) and np.array_equal(want[3], a[3])
+    assert_same(got, want, "affine sums")
