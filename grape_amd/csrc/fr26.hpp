@@ -331,5 +331,67 @@ GRAPE_HD Fr fold1(const Limbs& w1, const Limbs& lo, const Limbs& d) {
     return canon4_unpack(reduce(F, 1));
 }
 
+
+// ---- fold by a challenge that every lane shares: multiplication and reduction in one table
+// lo + v * d needs a product by the SAME v for every element of a round, so the reduction can be
+// folded into the multiplier: with W_j = v * 2^(26 j + 52) mod r (ten canonical constants per
+// challenge, made once by fold_table), sum_j d_j W_j = v * d * 2^52 (mod r) is a 10 x 10 limb
+// product whose value stays below 10 * 2^26 r, and TWO Montgomery steps (dividing by 2^52) bring it
+// to within 2^-22 r of [0, r) - against ten steps for a general product.  118 multiply-adds per
+// fold instead of 190, and a third of the carry handling.
+constexpr int kFoldTableWords = N * N;
+// tab[j * N + k] = limb k of v * 2^(26 j + 52) mod r for the memory-form challenge v_mem
+GRAPE_HD void fold_table(int32_t* tab, const Fr& v_mem) {
+    Fr p52 = Fr::zero(), p26 = Fr::zero();
+    p52.v[1] = 1u << 20;                      // the integer 2^52
+    p26.v[0] = 1u << 26;                      // the integer 2^26
+    const Fr step = to_montc(p26);            // mulc(x, step) = x * 2^26
+    Fr w = mulc(v_mem, p52);                  // v_mem * 2^52 / 2^256 = v * 2^52
+    for (int j = 0; j < N; j++) {
+        const Limbs l = pack(w);
+#pragma unroll
+        for (int k = 0; k < N; k++) tab[j * N + k] = l.v[k];
+        w = mulc(w, step);
+    }
+}
+// Two Montgomery steps and the carry chain that finish a table fold: c holds lo * 2^52 + sum_j d_j W_j
+// in twelve columns; returns lo + v * d in canonical memory form (the value before the last step lies
+// in (0.99 r, 3.01 r)).
+GRAPE_HD Fr foldt_finish(int64_t* c) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int32_t m = (int32_t)((0u - (uint32_t)c[i]) & MASK);
+        c[i] += (int64_t)m;
+#pragma unroll
+        for (int j = 1; j < N; j++) c[i + j] += (int64_t)m * (int64_t)R(j);
+        c[i + 1] += c[i] >> W;
+    }
+    Limbs r;
+    int64_t carry = 0;
+#pragma unroll
+    for (int k = 0; k < N - 1; k++) {
+        const int64_t t = c[2 + k] + (int64_t)R(k) + carry;                 // + one r
+        r.v[k] = (int32_t)((uint32_t)t & MASK);
+        carry = t >> W;
+    }
+    r.v[N - 1] = (int32_t)(c[N + 1] + (int64_t)R(N - 1) + carry);
+    return canon4_unpack(r);
+}
+// lo + v * d in canonical memory form for canonical lo (limbs from pack) and signed limbs d = hi - lo
+// (|limb| < 2^26), through the table of v's multiples.
+template <class TabPtr>
+GRAPE_HD Fr foldt(TabPtr tab, const Limbs& lo, const Limbs& d) {
+    int64_t c[N + 2];
+    c[0] = c[1] = 0;
+#pragma unroll
+    for (int k = 0; k < N; k++) c[k + 2] = (int64_t)(uint32_t)lo.v[k];      // lo * 2^52
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+#pragma unroll
+        for (int k = 0; k < N; k++) c[k] += (int64_t)d.v[j] * (int64_t)tab[j * N + k];
+    }
+    return foldt_finish(c);
+}
+
 }  // namespace fr26
 }  // namespace grape

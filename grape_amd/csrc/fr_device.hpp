@@ -25,6 +25,52 @@ __device__ __forceinline__ fr26::Limbs ld_l26(const uint32_t* base, size_t i) { 
 
 using fr26::fold1;
 
+// Table folds of TWO elements by the same challenge, row by row of the table: the ten words of a row
+// arrive through one scalar load and serve both elements, and the row pointer is re-derived from a
+// value the previous row produced, so that the compiler keeps one or two rows in scalar registers
+// instead of loading (and then spilling) all hundred words ahead of the loop.
+typedef const __attribute__((address_space(4))) int32_t* FoldTabPtr;
+__device__ __forceinline__ void foldt2(const int32_t* tab, const fr26::Limbs& lo_a, const fr26::Limbs& d_a, const fr26::Limbs& lo_b,
+                                       const fr26::Limbs& d_b, Fr& out_a, Fr& out_b) {
+    constexpr int N = fr26::N;
+    int64_t ca[N + 2], cb[N + 2];
+    ca[0] = ca[1] = cb[0] = cb[1] = 0;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        ca[k + 2] = (int64_t)(uint32_t)lo_a.v[k];
+        cb[k + 2] = (int64_t)(uint32_t)lo_b.v[k];
+    }
+    // rows j and j + 1 are addressable from the start; the pointer of row j + 2 is released by a value
+    // that row j has produced, so its scalar load is in flight while row j + 1 is multiplied
+    FoldTabPtr row[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) row[j] = (FoldTabPtr)(uintptr_t)(tab + j * N);
+    asm volatile("" : "+s"(row[0]), "+s"(row[1]));
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+#pragma unroll
+        for (int k = 0; k < N; k++) {
+            const int32_t w = row[j][k];
+            ca[k] += (int64_t)d_a.v[j] * (int64_t)w;
+            cb[k] += (int64_t)d_b.v[j] * (int64_t)w;
+        }
+        if (j + 2 < N) asm volatile("" : "+s"(row[j + 2]) : "v"((uint32_t)ca[0]));
+    }
+    out_a = fr26::foldt_finish(ca);
+    out_b = fr26::foldt_finish(cb);
+}
+
+// The ten multiples of a round's challenge that the table fold multiplies by (fr26::fold_table), for
+// `count` <= 64 challenges: thread t writes the table of v[t] at tabs + 100 t.  (static: every
+// source file that launches it gets its own copy)
+static __global__ void __launch_bounds__(64) fold_tables_kernel(int32_t* tabs, const uint32_t* v, uint32_t count) {
+    if (threadIdx.x < count) fr26::fold_table(tabs + (size_t)fr26::kFoldTableWords * threadIdx.x, ld_fr(v, threadIdx.x));
+}
+// Rounds of at least this many output indices fold through the table of the challenge's multiples
+// (one more small launch per round); shorter rounds are launch-bound and keep the single product.
+constexpr uint32_t kTableFoldMinOut = 1u << 16;
+constexpr size_t kFoldTableBytes = 512;                  // 100 words, padded
+
 // hi operand of the MSB split: X[g + h] or zero when that index is past the live extent
 __device__ __forceinline__ Fr ld_hi(const uint32_t* X, size_t g, size_t h, size_t in_size) {
     return (g + h < in_size) ? ld_fr(X, g + h) : Fr::zero();

@@ -15,12 +15,13 @@ namespace grape {
 // with 16 pairs per thread that was a quarter of the kernel, with 64 it is a fifteenth.
 constexpr int kRoundIters = 64;
 
-template <bool COEFFS>
-__global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
+template <bool COEFFS, bool TAB>
+__global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
                                                            uint32_t in_size, uint32_t out_size, const uint32_t* v,
-                                                           uint32_t* partial) {
+                                                           const int32_t* __restrict__ tab, uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
-    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    fr26::Limbs w1;
+    if (!TAB) w1 = fr26::weight16(ld_fr(v, 0));
     fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
     fr26::acc_zero(Q);
@@ -30,8 +31,17 @@ __global__ void __launch_bounds__(kBlock) sumcheck2_kernel(uint32_t* A, uint32_t
         const fr26::Limbs a0 = ld_l26(A, g), b0 = ld_l26(B, g);
         const fr26::Limbs a1 = ld_hi26(A, g, out_size, in_size), b1 = ld_hi26(B, g, out_size, in_size);
         const fr26::Limbs da = fr26::sub(a1, a0), db = fr26::sub(b1, b0);   // signed, |limb| < 2^26
-        st_fr(A, g, fold1(w1, a0, da));
-        st_fr(B, g, fold1(w1, b0, db));
+        // long rounds fold through the table of the challenge's multiples (no full reduction), short
+        // ones through one limb product (no table to prepare)
+        if (TAB) {
+            Fr fa, fb;
+            foldt2(tab, a0, da, b0, db, fa, fb);
+            st_fr(A, g, fa);
+            st_fr(B, g, fb);
+        } else {
+            st_fr(A, g, fold1(w1, a0, da));
+            st_fr(B, g, fold1(w1, b0, db));
+        }
         if (COEFFS) {
             // materialised coefficient arrays (phase 1 folds them further)
             fr26::Acc T;
@@ -477,7 +487,7 @@ constexpr int kLogUpIters = 16;
 // the array's device address once per device (noalloc_scratch) and passes that to the kernels.
 constexpr uint32_t kNoAllocMaxOut = 1u << 26;
 constexpr unsigned kNoAllocMaxBlocks = kNoAllocMaxOut / (kBlock * kRoundIters);
-static __device__ __align__(256) uint32_t scratch[(size_t)kNoAllocMaxBlocks * 3 * 8];
+static __device__ __align__(256) uint32_t scratch[(size_t)kNoAllocMaxBlocks * 3 * 8 + kFoldTableBytes / 4];
 
 constexpr int kMaxDevices = 64;
 static uint32_t* g_noalloc_ptr[kMaxDevices] = {nullptr};
@@ -520,14 +530,20 @@ static int sumcheck2_impl(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, ui
     hipStream_t s = as_stream(st);
     unsigned nb = reduce_grid(out_size);
     uint32_t* partial = nullptr;
-    if (sums) {
-        CHECK_PTR16(sums);
-        void* ws;
-        int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws, s);
-        if (rc) return rc;
-        partial = (uint32_t*)ws;
+    if (sums) CHECK_PTR16(sums);
+    // the partial sums, then the table of the challenge's multiples
+    const size_t partial_bytes = (size_t)nb * 3 * 32;
+    void* ws;
+    int rc = scratch_get(kSlotReduce, partial_bytes + kFoldTableBytes, &ws, s);
+    if (rc) return rc;
+    if (sums) partial = (uint32_t*)ws;
+    if (out_size >= kTableFoldMinOut) {
+        int32_t* tab = (int32_t*)((char*)ws + partial_bytes);
+        fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+        sumcheck2_kernel<COEFFS, true><<<nb, kBlock, 0, s>>>(A, B, a, b, c, in_size, out_size, v, tab, partial);
+    } else {
+        sumcheck2_kernel<COEFFS, false><<<nb, kBlock, 0, s>>>(A, B, a, b, c, in_size, out_size, v, nullptr, partial);
     }
-    sumcheck2_kernel<COEFFS><<<nb, kBlock, 0, s>>>(A, B, a, b, c, in_size, out_size, v, partial);
     if (sums) final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
@@ -569,7 +585,13 @@ int grape_sumcheck_round2_noalloc(uint32_t* A, uint32_t* B, uint32_t in_size, ui
     GRAPE_REQUIRE(nb <= kNoAllocMaxBlocks, "grid exceeds the static scratch array");
     // every workgroup writes its three partial sums and the finishing kernel reads exactly those, so
     // nothing of the previous call's contents is read and nothing has to be cleared
-    sumcheck2_kernel<false><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, partial);
+    if (out_size >= kTableFoldMinOut) {
+        int32_t* tab = (int32_t*)(partial + (size_t)kNoAllocMaxBlocks * 3 * 8);   // behind the partial sums, rewritten by every call
+        fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+        sumcheck2_kernel<false, true><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, tab, partial);
+    } else {
+        sumcheck2_kernel<false, false><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, nullptr, partial);
+    }
     final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;

@@ -123,6 +123,13 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
             int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
         }
     }
+    commit_i32_rows(out, tensor, size, rowlen);
+    return out;
+}
+
+// any int32 scalars: five signed 8-bit digits per scalar through a small table, or the reference's
+// byte windows when even that table is over budget
+void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen) {
     if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
                   return grape_commit_i32(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr);
@@ -134,6 +141,14 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
               }),
               "grape_commit_i32_ref_table");
     }
+}
+
+affine_t* Hyrax::commit_affine_i32(int* tensor, uint size, uint N) {
+    check_shape(size, N);
+    const uint rowlen = N * com_scale;
+    affine_t* out = nullptr;
+    check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)(size / rowlen)), "grape_malloc");
+    commit_i32_rows(out, tensor, size, rowlen);
     return out;
 }
 

@@ -45,6 +45,9 @@ public:
     // The same commitments as affine points (what the kernels produce).
     affine_t* commit_affine(int* tensor, uint size, uint N);
     affine_t* commit_affine(FrTensor& tensor, uint size, uint N);
+    // Integers of any int32 magnitude, without trying the int16 table first (and without giving that
+    // table up for this object when a value does not fit it): lookup multiplicities.
+    affine_t* commit_affine_i32(int* tensor, uint size, uint N);
 
     Hyrax_proof open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
     // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
@@ -95,6 +98,7 @@ private:
     size_t table_bytes_in_use() const;
     // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
     void commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build);
+    void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
     StridedTable fr_strided_;

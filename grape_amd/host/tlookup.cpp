@@ -211,7 +211,10 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         }
         com_A_rows = D / (msm_size * hyrax.com_scale);
         uint m_N = 1u << (Log2(N) / 2);
-        com_m = hyrax.commit_affine(m, N, m_N);
+        // the multiplicities are small integers: committed from the counters they were made from
+        // (five 8-bit digits each) where those are at hand, as field elements otherwise
+        if (d_hist_ && D < (1u << 31)) com_m = hyrax.commit_affine_i32(reinterpret_cast<int*>(d_hist_), N, m_N);
+        else com_m = hyrax.commit_affine(m, N, m_N);
         com_m_rows = N / (m_N * hyrax.com_scale);
         check(grape_stream_sync(nullptr), "sync");
         commit_time += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();

@@ -56,6 +56,12 @@ void t26_fold1(const uint32_t* v, const uint32_t* lo, const uint32_t* hi, uint32
     const fr26::Limbs l = fr26::pack(ld(lo));
     st(out, fr26::fold1(fr26::weight16(ld(v)), l, fr26::sub(fr26::pack(ld(hi)), l)));
 }
+// the ten constants of the table fold for a challenge v, and lo + v * (hi - lo) through them
+void t26_fold_table(const uint32_t* v, int32_t* tab) { fr26::fold_table(tab, ld(v)); }
+void t26_foldt(const int32_t* tab, const uint32_t* lo, const uint32_t* hi, uint32_t* out) {
+    const fr26::Limbs l = fr26::pack(ld(lo));
+    st(out, fr26::foldt(tab, l, fr26::sub(fr26::pack(ld(hi)), l)));
+}
 // k * a + b for canonical a, b and 0 <= k <= 3 with k*a + b < 4r, through canon4_unpack
 void t26_canon4(const uint32_t* a, const uint32_t* b, int k, uint32_t* out) {
     fr26::Limbs A = fr26::pack(ld(a)), B = fr26::pack(ld(b)), r;

@@ -127,3 +127,24 @@ def test_single_product_fold_and_canon4(lib):
                     continue
                 lib.t26_canon4(_u32(_p([a % R])[0]), _u32(_p([b])[0]), k, _u32(out))
                 assert _val(out) == (k * (a % R) + b) % R
+
+
+def test_table_fold(lib):
+    """the fold through ten precomputed multiples of the challenge: row j of the table is the integer
+    v * 2^(26 j + 52) mod r in 26-bit limbs, and lo + v*(hi - lo) comes out canonical for every pairing
+    of the edge values (differences of either sign, an absent hi) and v = 0, 1, r-1, r/2"""
+    rng = random.Random(6)
+    out = np.zeros(8, dtype=np.uint32)
+    tab = np.zeros(100, dtype=np.int32)
+    vals = EDGE + [rng.randrange(R) for _ in range(12)]
+    for v in [0, 1, R - 1, R >> 1, R - 2] + [rng.randrange(R) for _ in range(6)]:
+        lib.t26_fold_table(_u32(_p([v])[0]), tab.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+        for j in range(10):
+            row = sum(int(tab[10 * j + k]) << (26 * k) for k in range(10))
+            assert all(0 <= int(tab[10 * j + k]) < (1 << 26) for k in range(10))
+            assert row == (v << (26 * j + 52)) % R, (v, j)
+        for lo in vals:
+            plo = _p([lo])[0]
+            for hi in vals:
+                lib.t26_foldt(tab.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), _u32(plo), _u32(_p([hi])[0]), _u32(out))
+                assert _val(out) == (lo + v * (hi - lo)) % R, (v, lo, hi)
