@@ -259,45 +259,95 @@ __global__ void __launch_bounds__(kBlock) inverse_by_table_kernel(uint32_t* A, c
 // A logUp tensor A takes only the values B[t] of the entries that occur in the witness.  Entries
 // that occur at least min_count times get a slot (in table order, at most max_hot of them): the
 // committer builds B[t]*G_i for those entries only and adds one table point per element; the rest
-// of the elements ("cold") keep their full-width scalars.  One workgroup: every thread counts the
-// hot entries of its contiguous share, an exclusive scan over the threads gives its first slot.
-constexpr int kHotThreads = 1024;
-__global__ void __launch_bounds__(kHotThreads) hot_select_kernel(const uint32_t* __restrict__ hist, uint32_t len, uint32_t min_count,
-                                                                 uint32_t max_hot, int32_t* __restrict__ slot1,
-                                                                 uint32_t* __restrict__ hot_list, unsigned long long* info) {
-    __shared__ uint32_t cnt[kHotThreads];
-    __shared__ unsigned long long cold[kHotThreads];
-    const uint32_t per = (len + kHotThreads - 1) / kHotThreads;
-    const uint32_t t0 = threadIdx.x * per, t1 = t0 + per < len ? t0 + per : len;
+// of the elements ("cold") keep their full-width scalars.  Three small launches: hot entries per tile
+// of 1024, an exclusive scan of the tile counts, slots within every tile.
+constexpr int kHotTile = 1024;          // entries per workgroup: 4 per thread
+// pass 1: hot entries per tile
+__global__ void __launch_bounds__(kBlock) hot_count_kernel(const uint32_t* __restrict__ hist, uint32_t len, uint32_t min_count,
+                                                           uint32_t* __restrict__ tile_count) {
+    __shared__ uint32_t wsum[kBlock / 64];
+    const uint32_t base = blockIdx.x * kHotTile + threadIdx.x * 4;
     uint32_t mine = 0;
-    for (uint32_t t = t0; t < t1; t++) mine += hist[t] >= min_count ? 1u : 0u;
-    cnt[threadIdx.x] = mine;
+#pragma unroll
+    for (int k = 0; k < 4; k++) mine += (base + k < len && hist[base + k] >= min_count) ? 1u : 0u;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mine += __shfl_down(mine, off, 64);
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = mine;
     __syncthreads();
-    // inclusive scan (Hillis-Steele) over 1024 counters
-    for (int off = 1; off < kHotThreads; off <<= 1) {
-        const uint32_t add = (int)threadIdx.x >= off ? cnt[threadIdx.x - off] : 0u;
+    if (threadIdx.x == 0) tile_count[blockIdx.x] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+}
+// pass 2 (one workgroup): tile_count -> exclusive prefix, in place; info[0] = slots given
+__global__ void __launch_bounds__(kBlock) hot_scan_kernel(uint32_t* tile_count, uint32_t ntiles, uint32_t max_hot, unsigned long long* info) {
+    __shared__ uint32_t part[kBlock];
+    const uint32_t per = (ntiles + kBlock - 1) / kBlock;
+    const uint32_t t0 = threadIdx.x * per, t1 = t0 + per < ntiles ? t0 + per : ntiles;
+    uint32_t mine = 0;
+    for (uint32_t t = t0; t < t1; t++) mine += tile_count[t];
+    part[threadIdx.x] = mine;
+    __syncthreads();
+    for (int off = 1; off < kBlock; off <<= 1) {
+        const uint32_t add = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0u;
         __syncthreads();
-        cnt[threadIdx.x] += add;
+        part[threadIdx.x] += add;
         __syncthreads();
     }
-    uint32_t slot = cnt[threadIdx.x] - mine;          // exclusive prefix
-    unsigned long long cold_mine = 0;
+    uint32_t run = part[threadIdx.x] - mine;
     for (uint32_t t = t0; t < t1; t++) {
-        const uint32_t h = hist[t];
-        const bool hot = h >= min_count && slot < max_hot;
-        slot1[t] = hot ? (int32_t)(slot + 1) : 0;
-        if (hot) hot_list[slot] = t;
-        if (h >= min_count) slot++;
-        if (!hot) cold_mine += h;
+        const uint32_t c = tile_count[t];
+        tile_count[t] = run;
+        run += c;
     }
-    cold[threadIdx.x] = cold_mine;
+    if (threadIdx.x == kBlock - 1) {
+        const uint32_t total = part[kBlock - 1];
+        info[0] = total < max_hot ? total : max_hot;
+        info[1] = 0;
+    }
+}
+// pass 3: slots in table order; info[1] += witness elements whose entry got none
+__global__ void __launch_bounds__(kBlock) hot_assign_kernel(const uint32_t* __restrict__ hist, uint32_t len, uint32_t min_count,
+                                                            uint32_t max_hot, const uint32_t* __restrict__ tile_base,
+                                                            int32_t* __restrict__ slot1, uint32_t* __restrict__ hot_list,
+                                                            unsigned long long* info) {
+    __shared__ uint32_t wsum[kBlock / 64];
+    __shared__ unsigned long long wcold[kBlock / 64];
+    const uint32_t base = blockIdx.x * kHotTile + threadIdx.x * 4;
+    uint32_t h[4];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        h[k] = base + k < len ? hist[base + k] : 0u;
+        mine += (base + k < len && h[k] >= min_count) ? 1u : 0u;
+    }
+    // exclusive prefix of `mine` over the workgroup: inclusive scan within the wave, then the waves before
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    uint32_t slot = tile_base[blockIdx.x] + incl - mine;
+    for (int w = 0; w < wave; w++) slot += wsum[w];
+    unsigned long long cold = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (base + k >= len) break;
+        const bool cand = h[k] >= min_count;
+        const bool hot = cand && slot < max_hot;
+        slot1[base + k] = hot ? (int32_t)(slot + 1) : 0;
+        if (hot) hot_list[slot] = base + k;
+        if (cand) slot++;
+        if (!hot) cold += h[k];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) cold += __shfl_down(cold, off, 64);
+    if (lane == 0) wcold[wave] = cold;
     __syncthreads();
     if (threadIdx.x == 0) {
-        unsigned long long c = 0;
-        for (int i = 0; i < kHotThreads; i++) c += cold[i];
-        const uint32_t total = cnt[kHotThreads - 1];
-        info[0] = total < max_hot ? total : max_hot;
-        info[1] = c;
+        const unsigned long long c = wcold[0] + wcold[1] + wcold[2] + wcold[3];
+        if (c) atomicAdd(&info[1], c);
     }
 }
 // out[i] = slot + 1 of the element's entry (0: cold entry or outside the table)
@@ -710,10 +760,15 @@ int grape_tlookup_hot_select(const uint32_t* hist, uint32_t len, uint32_t min_co
     GRAPE_REQUIRE(hist != nullptr && slot1 != nullptr && hot_list != nullptr && info != nullptr && len > 0, "bad arguments");
     GRAPE_REQUIRE(min_count >= 1, "min_count must be at least 1");
     hipStream_t s = as_stream(st);
-    void* d_info;
-    int rc = scratch_get(kSlotMisc, 64, &d_info, s);
+    const uint32_t ntiles = (len + kHotTile - 1) / kHotTile;
+    void* ws;
+    int rc = scratch_get(kSlotMisc, 64 + sizeof(uint32_t) * (size_t)ntiles, &ws, s);
     if (rc) return rc;
-    hot_select_kernel<<<1, kHotThreads, 0, s>>>(hist, len, min_count, max_hot, slot1, hot_list, (unsigned long long*)d_info);
+    unsigned long long* d_info = (unsigned long long*)ws;
+    uint32_t* tiles = (uint32_t*)((char*)ws + 64);
+    hot_count_kernel<<<ntiles, kBlock, 0, s>>>(hist, len, min_count, tiles);
+    hot_scan_kernel<<<1, kBlock, 0, s>>>(tiles, ntiles, max_hot, d_info);
+    hot_assign_kernel<<<ntiles, kBlock, 0, s>>>(hist, len, min_count, max_hot, tiles, slot1, hot_list, d_info);
     GRAPE_LAUNCH_CHECK();
     GRAPE_HIP_CHECK(hipMemcpyAsync(info, d_info, 2 * sizeof(uint64_t), hipMemcpyDeviceToHost, s));
     GRAPE_HIP_CHECK(hipStreamSynchronize(s));
