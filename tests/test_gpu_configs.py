@@ -198,3 +198,53 @@ def test_configs4_lookups_on_padded_ffn_rows(ops, host, gens4096):
                                         D, lowm, Nm, silu, alpha, r, u, v, table, NGEN, 1, 4096)
     assert_same(tr, wtr, "mapping lookup transcript")
     assert_same(sc, wsc, "S(v)")
+
+
+def test_configs4_softmax_mapping_lookup_through_occupied_entries(ops, host, gens4096):
+    """the layer's exponential lookup at its table size (2^20 entries, low = -2^19) and row length (4096
+    generators) on 2^24 scores distributed like the layer's (Gaussian, sigma 181, plus 0.5 % spread over
+    the whole table): the default path commits A through a per-proof table of the entries that reach
+    the break-even count and the rest as full-width scalars.  Transcript and S(v) against the oracle,
+    com(A) on sampled rows against the oracle's full-width commitment of 1/(S + beta), the split
+    against numpy; the same witness through the plain path (no table) gives the same commitment."""
+    import torch
+    hg, dg, htab = gens4096
+    table = ops.g1_table_gen(dg, 256)
+    exp_map, _ = host.witness_tables()
+    low, N = -(1 << 19), 1 << 20
+    logD = 24
+    D = 1 << logD
+    rng = np.random.default_rng(91)
+    S_in = np.clip(np.rint(rng.normal(0.0, 181.0, size=D)), low, low + N - 1).astype(np.int32)
+    spread = rng.random(D) < 0.005
+    S_in[spread] = rng.integers(low, low + N, size=int(spread.sum()))
+    S_out = np.ascontiguousarray(exp_map[S_in - low])
+    alpha, r, u, v = rand_fr(1, 92), rand_fr(1, 93), rand_fr(logD, 94), rand_fr(logD, 95)
+    beta = br.fr_pack([N])[0]
+    host.set_indexed_commit(True)
+    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
+    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
+    tr, sc, com_a, n_hot, n_cold = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    counts = np.bincount(S_in.astype(np.int64) - low, minlength=N)
+    thr = int(1.8 * 4096) + 1
+    assert n_hot == int((counts >= thr).sum()) and n_hot > 100
+    assert n_cold == int(counts[counts < thr].sum()) and 0 < n_cold < D // 5
+    # the plain path on the same witness
+    host.set_indexed_commit(False)
+    tr2, sc2, com_a2, h2, c2 = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    host.set_indexed_commit(True)
+    assert h2 == 0 and c2 == 0
+    assert_same(com_a, com_a2, "com(A): occupied-entry table == full-width commitment")
+    assert_same(tr, tr2, "transcripts")
+    del dSi, dSo, table
+    torch.cuda.empty_cache()
+    T, B = orc.tlookup_init(low, N, beta, orc.from_i32(exp_map), r[0])
+    m = orc.tlookup_prep(orc.from_i32(S_in), low, N)
+    S = orc.vec2("orc_fr_vec_add", orc.vec_bcast("orc_fr_vec_bcast_mul", orc.from_i32(S_out), r[0]), orc.from_i32(S_in))
+    for rr in (0, 517, D // 4096 - 1):
+        Ainv = orc.vec1("orc_fr_vec_inv", orc.vec_bcast("orc_fr_vec_bcast_add", S[rr * 4096:(rr + 1) * 4096], beta))
+        assert_same(com_a[rr:rr + 1], orc.commit_fr(Ainv, htab, 4096, NGEN), "com(A) row %d" % rr)
+    st, wtr, wsc = orc.tlookup_prove(S, T, B, m, alpha[0], beta, u, v)
+    assert st == 0 and wtr.shape[0] == logD
+    assert_same(tr, wtr, "transcript")
+    assert_same(sc, wsc, "S(v)")
