@@ -41,6 +41,14 @@ __global__ void __launch_bounds__(kBlock) bcast_kernel(uint32_t* out, const uint
     st_fr(out, i, apply<OP>(ld_fr(a, i), ld_fr(x, 0)));
 }
 
+// out = x + r * y with one scalar r (the combined witness of a mapping lookup, S_in + r * S_out,
+// src/tlookup.cu:407-410, in one pass instead of a copy, a scalar product and a sum)
+__global__ void __launch_bounds__(kBlock) axpy_kernel(uint32_t* out, const uint32_t* x, const uint32_t* r, const uint32_t* y, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    st_fr(out, i, add(ld_fr(x, i), fr26::mulc(ld_fr(y, i), ld_fr(r, 0))));
+}
+
 __global__ void __launch_bounds__(kBlock) from_i32_kernel(uint32_t* out, const int32_t* in, size_t n) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
@@ -428,6 +436,13 @@ int grape_bench_copy_fr(uint32_t* out, const uint32_t* in, size_t n, int iters, 
     return GRAPE_OK;
 }
 
+int grape_fr_axpy(uint32_t* out, const uint32_t* x, const uint32_t* r, const uint32_t* y, size_t n, grape_stream_t st) {
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(out); CHECK_PTR16(x); CHECK_PTR16(r); CHECK_PTR16(y);
+    axpy_kernel<<<blocks_for(n), kBlock, 0, as_stream(st)>>>(out, x, r, y, n);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
 int grape_fr_from_i32(uint32_t* out, const int32_t* in, size_t n, grape_stream_t st) {
     if (n == 0) return GRAPE_OK;
     CHECK_PTR16(out);

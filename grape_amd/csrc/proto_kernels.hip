@@ -370,6 +370,34 @@ __global__ void __launch_bounds__(kBlock) gather_fr_kernel(uint32_t* out, const 
     st_fr(out, i, ld_fr(src, list[i]));
 }
 
+// Index and logUp tensor in one pass: idx1[i] = (key_i - low) + 1 for a key inside the table (0
+// otherwise) and A[i] = B[index].  With `cmp` (mapping lookups) the element's second component must
+// equal the table's (cmp[i] == cmp_table[index], i.e. S_out = f(S_in)); an element outside the table
+// or with a wrong second component is counted in *mismatches and its A left unwritten.
+__global__ void __launch_bounds__(kBlock) index_inverse_kernel(int32_t* idx1, uint32_t* A, const uint32_t* key, size_t n, int32_t low,
+                                                                uint32_t len, const uint32_t* B, const uint32_t* cmp,
+                                                                const uint32_t* cmp_table, unsigned int* mismatches) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    bool bad = false;
+    if (i < n) {
+        const Fr d = fr26::from_montc(sub(ld_fr(key, i), fr26::from_i32c(low)));
+        const uint32_t hi = d.v[1] | d.v[2] | d.v[3] | d.v[4] | d.v[5] | d.v[6] | d.v[7];
+        const bool inside = hi == 0 && d.v[0] < len;
+        idx1[i] = inside ? (int32_t)(d.v[0] + 1) : 0;
+        bad = !inside;
+        if (inside && cmp) {
+            const Fr a = ld_fr(cmp, i), b = ld_fr(cmp_table, d.v[0]);
+            uint32_t diff = 0;
+#pragma unroll
+            for (int k = 0; k < 8; k++) diff |= a.v[k] ^ b.v[k];
+            bad = diff != 0;
+        }
+        if (!bad) st_fr(A, i, ld_fr(B, d.v[0]));
+    }
+    const unsigned long long b = __ballot(bad);
+    if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
+}
+
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -738,6 +766,30 @@ int grape_tlookup_inverse_by_table(uint32_t* A, const uint32_t* S, const int32_t
     rc = zero_fill(cnt, sizeof(unsigned int), s);
     if (rc) return rc;
     inverse_by_table_kernel<<<blocks_for(n), kBlock, 0, s>>>(A, S, idx1, T, B, n, len, (unsigned int*)cnt);
+    GRAPE_LAUNCH_CHECK();
+    unsigned int h = 0;
+    GRAPE_HIP_CHECK(hipMemcpyAsync(&h, cnt, sizeof h, hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    *mismatches = h;
+    return GRAPE_OK;
+}
+
+int grape_tlookup_index_inverse(int32_t* idx1, uint32_t* A, const uint32_t* key, size_t n, int32_t low, uint32_t len,
+                                const uint32_t* B, const uint32_t* cmp, const uint32_t* cmp_table, size_t* mismatches,
+                                grape_stream_t st) {
+    GRAPE_REQUIRE(mismatches != nullptr && idx1 != nullptr && len > 0, "bad arguments");
+    *mismatches = 0;
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(A); CHECK_PTR16(key); CHECK_PTR16(B);
+    GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr), "cmp and cmp_table go together");
+    if (cmp) { CHECK_PTR16(cmp); CHECK_PTR16(cmp_table); }
+    hipStream_t s = as_stream(st);
+    void* cnt;
+    int rc = scratch_get(kSlotMisc, 64, &cnt, s);
+    if (rc) return rc;
+    rc = zero_fill(cnt, sizeof(unsigned int), s);
+    if (rc) return rc;
+    index_inverse_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, key, n, low, len, B, cmp, cmp_table, (unsigned int*)cnt);
     GRAPE_LAUNCH_CHECK();
     unsigned int h = 0;
     GRAPE_HIP_CHECK(hipMemcpyAsync(&h, cnt, sizeof h, hipMemcpyDeviceToHost, s));

@@ -22,6 +22,17 @@ void tLookup::make_index(const FrTensor& vals, int low_) {
     check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(vals.size ? vals.size : 1)), "grape_malloc");
     check(grape_tlookup_index(d_idx_, W(vals.gpu_data), vals.size, low_, T.size, nullptr), "grape_tlookup_index");
 }
+void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table) {
+    drop_index();
+    a_ready_ = false;
+    check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(key.size ? key.size : 1)), "grape_malloc");
+    size_t mismatches = 0;
+    check(grape_tlookup_index_inverse(d_idx_, W(A.gpu_data), W(key.gpu_data), key.size, low_, T.size, W(B.gpu_data),
+                                      cmp ? W(cmp->gpu_data) : nullptr, cmp_table ? W(cmp_table->gpu_data) : nullptr, &mismatches,
+                                      nullptr),
+          "grape_tlookup_index_inverse");
+    a_ready_ = mismatches == 0;
+}
 void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
     if (!d_idx_ || N == pad_N) return;
     int* padded = nullptr;
@@ -174,8 +185,9 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     // A = 1/(S + beta): read from B where the witness matches its table entry (every element of
     // a valid witness does), computed by batched inversion otherwise (tlookup_inv_kernel,
     // src/tlookup.cu:52-62, inverts per element)
-    bool from_table = false;
-    if (d_idx_) {
+    bool from_table = a_ready_;
+    a_ready_ = false;
+    if (!from_table && d_idx_) {
         size_t mismatches = 0;
         check(grape_tlookup_inverse_by_table(W(A.gpu_data), W(S.gpu_data), d_idx_, W(T.gpu_data), W(B.gpu_data), D, N, &mismatches, nullptr),
               "grape_tlookup_inverse_by_table");
@@ -313,7 +325,9 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
 
 Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
     uint D = S.size;
-    make_index(S, low);
+    a_ready_ = false;
+    if (D == (1u << Log2(D)) && A.size >= D) make_index_and_A(S, low, A, nullptr, nullptr);   // no padding: index and A = B[index] together
+    else make_index(S, low);
     index_to_m(D, low);                       // what prep(S) computes, from the shared indices
     if (D != (1u << Log2(D))) {
         // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
@@ -368,13 +382,15 @@ void tLookupRangeMapping::prep(const FrTensor& vals) { histogram_to_m(m, vals, l
 Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax,
                               uint msm_size, double& commit_time) {
     uint D = S_in.size;
-    make_index(S_in, low);
+    a_ready_ = false;
+    if (S_out.size != D) throw std::runtime_error("tLookupRangeMapping: S_in.size != S_out.size");
+    // no padding: index, the check S_out = f(S_in) and A = B[index] in one pass
+    if (D == (1u << Log2(D)) && A.size >= D) make_index_and_A(S_in, low, A, &S_out, &mapped_vals);
+    else make_index(S_in, low);
     index_to_m(D, low);                       // what prep(S_in) computes, from the shared indices
     FrTensor S(1u << Log2(D));
     S.set_size(D);
-    S = S_out;
-    S *= r;
-    S.add_with_size(D, S_in);
+    check(grape_fr_axpy(W(S.gpu_data), W(S_in.gpu_data), W(grape_host::device_scalar(r)), W(S_out.gpu_data), D, nullptr), "grape_fr_axpy");
     if (D != (1u << Log2(D))) {
         Fr pad_value = mapped_vals((uint)(-low)) * r;
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);

@@ -52,6 +52,10 @@ protected:
     // nullptr when the witness is padded (its indices then do not line up with the padded tensor).
     int* d_idx_ = nullptr;
     void make_index(const FrTensor& vals, int low_);
+    // index and A = B[index] in one pass over a witness that needs no padding; cmp / cmp_table: the
+    // second component of a mapping lookup and the table's.  Sets a_ready_ when every element matched.
+    void make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table);
+    bool a_ready_ = false;              // A of the proof in flight already holds B[index]
     void drop_index();
     void pad_index(uint N, uint pad_N, uint pad_size, int fill);   // rows of N indices -> rows of pad_N
     void index_to_m(uint witness_size, int low_);

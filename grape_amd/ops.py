@@ -215,6 +215,26 @@ def tlookup_hist_index(idx1, length, hist=None):
     return hist
 
 
+def tlookup_index_inverse(key, low, B, cmp=None, cmp_table=None):
+    """returns (idx1, A, mismatches)"""
+    lib = init()
+    n = key.shape[0]
+    idx1 = torch.empty(n, dtype=torch.int32, device="cuda")
+    A = fr_empty(n)
+    mm = ctypes.c_size_t(0)
+    _capi.check(lib.grape_tlookup_index_inverse(_p(idx1), _p(A), _p(key), n, low, B.shape[0], _p(B),
+                                                _p(cmp) if cmp is not None else None, _p(cmp_table) if cmp_table is not None else None,
+                                                ctypes.byref(mm), _s()))
+    return idx1, A, mm.value
+
+
+def fr_axpy(x, r, y, out=None):
+    lib = init()
+    out = fr_empty(x.shape[0]) if out is None else out
+    _capi.check(lib.grape_fr_axpy(_p(out), _p(x), _p(r), _p(y), x.shape[0], _s()))
+    return out
+
+
 def tlookup_hot_select(hist, min_count, max_hot):
     """returns (slot1, hot_list[:n_hot], n_hot, cold_elements)"""
     lib = init()

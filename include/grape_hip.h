@@ -74,6 +74,9 @@ int grape_fr_mul(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_b, size
 /* out[i] = a[i] (+,*) x[0], x one device element.  Fr_broadcast_add/mul, src/fr-tensor.cu:88-108. */
 int grape_fr_bcast_add(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_x, size_t n, grape_stream_t stream);
 int grape_fr_bcast_mul(uint32_t *d_out, const uint32_t *d_a, const uint32_t *d_x, size_t n, grape_stream_t stream);
+/* out[i] = x[i] + r * y[i] with one device scalar r (out may alias x or y): the combined witness
+ * S_in + r*S_out of a mapping lookup in one pass (src/tlookup.cu:407-410 takes three). */
+int grape_fr_axpy(uint32_t *d_out, const uint32_t *d_x, const uint32_t *d_r, const uint32_t *d_y, size_t n, grape_stream_t stream);
 /* Integer embedding, negatives as r-|v|.  int_to_fr / uint_to_fr, src/fr-tensor.cu:30-46. */
 int grape_fr_from_i32(uint32_t *d_out, const int32_t *d_in, size_t n, grape_stream_t stream);
 int grape_fr_from_u32(uint32_t *d_out, const uint32_t *d_in, size_t n, grape_stream_t stream);
@@ -200,6 +203,17 @@ int grape_tlookup_hist(uint32_t *d_hist, const uint32_t *d_vals, size_t n, int32
  * reference derives inside get_histogram_kernel, src/tlookup.cu:9-12).  Feeds the indexed
  * commitment of A = 1/(S+beta) below. */
 int grape_tlookup_index(int32_t *d_out, const uint32_t *d_vals, size_t n, int32_t low, uint32_t len, grape_stream_t stream);
+/* Index and logUp tensor in one pass over the witness: d_idx1 as grape_tlookup_index makes it from
+ * d_key (the witness of a range lookup, the input component of a mapping lookup), and
+ * d_A[i] = d_B[index] = 1/(T[index] + beta) where the element matches its table entry: for a range
+ * lookup (d_cmp = d_cmp_table = NULL) every key inside the table does; for a mapping lookup the
+ * output component must equal the table's, d_cmp[i] == d_cmp_table[index].  Other elements are
+ * left unwritten and counted in *mismatches (host; the call synchronises), as
+ * grape_tlookup_inverse_by_table does.  Replaces grape_tlookup_index + that call (src/tlookup.cu:9-12
+ * and :52-62) where the witness needs no padding. */
+int grape_tlookup_index_inverse(int32_t *d_idx1, uint32_t *d_A, const uint32_t *d_key, size_t n, int32_t low, uint32_t len,
+                                const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table, size_t *mismatches,
+                                grape_stream_t stream);
 /* The same histogram from indices already made by grape_tlookup_index (d_idx1[i] = index + 1,
  * 0 = outside the table): hist[d_idx1[i] - 1] += 1. */
 int grape_tlookup_hist_index(uint32_t *d_hist, const int32_t *d_idx1, size_t n, uint32_t len, grape_stream_t stream);

@@ -524,3 +524,45 @@ def test_occupied_entry_selection_kernels(ops):
         orc.lib().orc_g1_add_affine(orc.P(want[i]), orc.P(a[i]), orc.P(b[i]))
     assert not want[1].any() and not want[4].any() and np.array_equal(want[2], b[2]) and np.array_equal(want[3], a[3])
     assert_same(got, want, "affine sums")
+
+
+def test_index_and_inverse_in_one_pass_and_axpy(ops):
+    """grape_tlookup_index_inverse against the two calls it replaces (index, then A = B[index] with
+    the entry check), for a range witness and for a mapping witness with wrong outputs and keys
+    outside the table; grape_fr_axpy against the oracle's scalar product and sum"""
+    import torch
+    rng = np.random.default_rng(101)
+    low, N, n = -50, 128, 5000
+    beta, r = br.fr_pack([N])[0], rand_fr(1, 102)
+    fmap = rng.integers(-999, 999, size=N).astype(np.int32)
+    keys = rng.integers(low, low + N, size=n).astype(np.int32)
+    # range: every key inside
+    T, B = orc.tlookup_init(low, N, beta)
+    dK = ops.fr_from_i32(torch.from_numpy(keys).cuda())
+    idx1, A, mm = ops.tlookup_index_inverse(dK, low, ops.to_dev(B))
+    assert mm == 0
+    assert np.array_equal(idx1.cpu().numpy(), keys - low + 1)
+    assert_same(ops.fr_to_host(A), B[keys - low], "A = B[index]")
+    # mapping: 7 wrong outputs and 5 keys outside the table are counted and left alone
+    outs = fmap[keys - low].copy()
+    wrong = rng.choice(n, 7, replace=False)
+    outs[wrong] += 1
+    keys2 = keys.copy()
+    outside = np.setdiff1d(rng.choice(n, 20, replace=False), wrong)[:5]
+    keys2[outside] = low + N + 3
+    dK2 = ops.fr_from_i32(torch.from_numpy(keys2).cuda())
+    dO = ops.fr_from_i32(torch.from_numpy(outs).cuda())
+    Tm, Bm = orc.tlookup_init(low, N, beta, orc.from_i32(fmap), r[0])
+    idx1, A, mm = ops.tlookup_index_inverse(dK2, low, ops.to_dev(Bm), cmp=dO, cmp_table=ops.fr_from_i32(torch.from_numpy(fmap).cuda()))
+    assert mm == 12
+    want_idx = keys2 - low + 1
+    want_idx[outside] = 0
+    assert np.array_equal(idx1.cpu().numpy(), want_idx)
+    good = np.ones(n, dtype=bool)
+    good[wrong] = False
+    good[outside] = False
+    assert_same(ops.fr_to_host(A)[good], Bm[(keys2 - low)[good]], "A where the element matches its entry")
+    # x + r*y
+    x, y = rand_fr(777, 103), rand_fr(777, 104)
+    want = orc.vec2("orc_fr_vec_add", x, orc.vec_bcast("orc_fr_vec_bcast_mul", y, r[0]))
+    assert_same(ops.fr_to_host(ops.fr_axpy(ops.to_dev(x), ops.to_dev(r), ops.to_dev(y))), want, "x + r*y")
