@@ -365,6 +365,48 @@ def lookup_workload(args):
     return 0
 
 
+def mapping_workload(args):
+    """The layer's largest single proof on its own: the softmax exponential's mapping lookup, 2^27 scores
+    (32 heads x 2048 x 2048) into the 2^20-entry table, 4096 generators, scores distributed as the layer's
+    are (Gaussian, sigma 181).  One step = one tLookupRangeMapping proof with its commitments of A and m;
+    A goes through the per-proof table of the occupied entries, or as full-width scalars with
+    --plain-commit."""
+    import torch
+    from grape_amd import ops, _host as host
+    from gpuutil import rand_fr
+    ops.init(0)
+    host.load()
+    host.set_indexed_commit(not args.plain_commit)
+    lg = args.log_elems if args.log_elems != 25 else 27
+    D, N, low = 1 << lg, 1 << 20, -(1 << 19)
+    exp_map, _ = host.witness_tables()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    x = (torch.randn(D, generator=g, device="cuda") * 181.0).round().to(torch.int32).clamp_(low, low + N - 1)
+    y = torch.from_numpy(exp_map).cuda()[(x - low).long()]
+    gens = ops.g1_make_generators(rand_fr(4096, 42))
+    table = ops.g1_table_gen(gens, 256)
+    alpha, r, u, v = rand_fr(1, 43), rand_fr(1, 46), rand_fr(lg, 44), rand_fr(lg, 45)
+    secs, commits = [], []
+    for i in range(args.warmup + args.steps):
+        res = host.tlookup_mapping_prove_ex(ops.fr_from_i32(x), ops.fr_from_i32(y), D, low, N, exp_map, alpha, r, u, v, table,
+                                            4096, 1, 4096)
+        if i >= args.warmup:
+            secs.append(host.last_prove_seconds())
+            commits.append(host.last_commit_seconds())
+    t = float(np.mean(secs))
+    print(json.dumps({
+        "metric": "mapping_lookup_prove_time", "value": t, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "tLookupRangeMapping, 2^%d lookups into the 2^20-entry exponential table, 4096 generators "
+                               "(the softmax lookup of configs[4])" % lg,
+                   "commit_s": float(np.mean(commits)),
+                   "table_entries_with_a_row": res[3], "elements_as_full_width_scalars": res[4],
+                   "commit_of_A": "full-width scalars" if args.plain_commit else "per-proof table of the occupied entries"}}))
+    return 0
+
+
 def witness_workload(args):
     """Witness generation for one LLaMA-2-7B-shape transformer block (d_model 4096, FFN 11008, one
     attention head as the reference's generator forces, seq_len 2048 by default): the C++
@@ -559,10 +601,13 @@ def main():
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
     ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")
-    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "witness", "rounds"], default="commit",
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "mapping", "witness", "rounds"], default="commit",
                     help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
-                         "lookup: configs[3]; layer: configs[4]; witness: the layer's witness generator; "
+                         "lookup: configs[3]; layer: configs[4]; mapping: the layer's softmax lookup on its own; "
+                         "witness: the layer's witness generator; "
                          "rounds: the streaming kernels of the sumcheck / logUp rounds")
+    ap.add_argument("--plain-commit", action="store_true",
+                    help="mapping workload: commit A as full-width scalars instead of through its occupied entries")
     ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer and witness workloads")
     ap.add_argument("--matmul", choices=["auto", "valu", "mfma"], default="auto",
                     help="witness workload: integer matrix products on the matrix cores (auto, mfma) or with 64-bit multiply-adds (valu)")
@@ -581,6 +626,10 @@ def main():
         args.steps = 3 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
         return witness_workload(args)
+    if args.workload == "mapping":
+        args.steps = 3 if args.steps is None else args.steps
+        args.warmup = 1 if args.warmup is None else args.warmup
+        return mapping_workload(args)
     if args.workload in ("matmul", "lookup"):
         args.steps = 5 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
