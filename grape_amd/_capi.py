@@ -109,6 +109,9 @@ SIGNATURES = {
     "grape_bench_mad_u64_u32": [c_int, c_int, c_int, ctypes.POINTER(ctypes.c_double), c_void_p],
     "grape_profile_enable": [c_int],
     "grape_profile_last": [ctypes.POINTER(ctypes.c_float), c_int, ctypes.POINTER(c_int)],
+    "grape_stream_create": [ctypes.POINTER(c_void_p)],
+    "grape_stream_destroy": [c_void_p],
+    "grape_stream_wait_event": [c_void_p, c_void_p],
     "grape_event_create": [ctypes.POINTER(c_void_p)],
     "grape_event_destroy": [c_void_p],
     "grape_event_record": [c_void_p, c_void_p],

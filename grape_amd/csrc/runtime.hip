@@ -289,6 +289,39 @@ int grape_profile_last(float* ms, int cap, int* n) {
     return GRAPE_OK;
 }
 
+// A stream of the default priority that does not synchronise with the legacy default stream; its
+// scratch pool is dropped with it.
+int grape_stream_create(grape_stream_t* out) {
+    GRAPE_REQUIRE(out != nullptr, "null output");
+    hipStream_t s;
+    GRAPE_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = reinterpret_cast<grape_stream_t>(s);
+    return GRAPE_OK;
+}
+int grape_stream_destroy(grape_stream_t st) {
+    hipStream_t s = as_stream(st);
+    GRAPE_REQUIRE(s != nullptr, "the default stream cannot be destroyed");
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        if (g_pools) {
+            auto it = g_pools->find(s);
+            if (it != g_pools->end()) {
+                for (int k = 0; k < kNumSlots; k++)
+                    if (it->second.ptr[k]) (void)hipFree(it->second.ptr[k]);
+                g_pools->erase(it);
+            }
+        }
+    }
+    GRAPE_HIP_CHECK(hipStreamDestroy(s));
+    return GRAPE_OK;
+}
+int grape_stream_wait_event(grape_stream_t st, void* ev) {
+    GRAPE_REQUIRE(ev != nullptr, "null event");
+    GRAPE_HIP_CHECK(hipStreamWaitEvent(as_stream(st), (hipEvent_t)ev, 0));
+    return GRAPE_OK;
+}
+
 int grape_event_create(void** ev) {
     hipEvent_t e;
     GRAPE_HIP_CHECK(hipEventCreate(&e));

@@ -135,6 +135,45 @@ bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& h
     return done;
 }
 
+namespace {
+// A second stream (one per process, created on first use) and the two events that order it against
+// the default stream: begin() makes it wait for what the default stream has queued, end() makes the
+// default stream wait for it.  If the scope is left by an exception the destructor waits for the
+// stream, so nothing it still reads is freed under it.
+struct SideChain {
+    grape_stream_t stream = nullptr;
+    bool open = false;
+    SideChain() {
+        static grape_stream_t s = nullptr;
+        static void* e0 = nullptr;
+        static void* e1 = nullptr;
+        if (!s) {
+            check(grape_stream_create(&s), "grape_stream_create");
+            check(grape_event_create(&e0), "grape_event_create");
+            check(grape_event_create(&e1), "grape_event_create");
+        }
+        stream = s;
+        ev_begin = e0;
+        ev_end = e1;
+    }
+    void begin() {
+        check(grape_event_record(ev_begin, nullptr), "grape_event_record");
+        check(grape_stream_wait_event(stream, ev_begin), "grape_stream_wait_event");
+        open = true;
+    }
+    void end() {
+        check(grape_event_record(ev_end, stream), "grape_event_record");
+        check(grape_stream_wait_event(nullptr, ev_end), "grape_stream_wait_event");
+        open = false;
+    }
+    ~SideChain() {
+        if (open) grape_stream_sync(stream);
+    }
+    void* ev_begin = nullptr;
+    void* ev_end = nullptr;
+};
+}  // namespace
+
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
     uint32_t* hist = nullptr;
     check(grape_malloc((void**)&hist, sizeof(uint32_t) * (size_t)m.size), "grape_malloc");
@@ -179,6 +218,7 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     if (u.size() != v.size()) throw std::runtime_error("u.size() != v.size()");
     if (v.size() != Log2(D)) throw std::runtime_error("u.size() != ceilLog2(D)");
     if (D % msm_size != 0) throw std::runtime_error("D % msm_size != 0");
+    if (N > D) throw std::runtime_error("tLookup: the table is longer than the witness");   // phase 2 binds log2(N) of the log2(D) variables
     last_transcript = SumcheckTranscript();
 
     fr_t* d_beta = grape_host::device_scalar(beta);
@@ -260,6 +300,27 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     fr_t* d_v = grape_host::upload(v);
     FrTensor Bw(B), Tw(T), mw(m);          // phase 2 binds copies; T, B, m of this object stay intact
     try {
+        // The table side of phase 2 (B, T, m: sums and folds of the last log2(N) rounds) depends on
+        // nothing the witness side produces, so it runs as a chain of its own on a second stream,
+        // beside the rounds over A and S (the short rounds are launch- and latency-bound: five
+        // small kernels per round on the table side, two on the witness side).
+        SideChain side;
+        side.begin();                       // the second stream waits for everything queued so far
+        {
+            uint cur_t = N;
+            for (int vi = (int)logN - 1; vi >= 0 && vi < (int)rounds; vi--) {
+                const uint k = rounds - 1 - (uint)vi;
+                const uint half = cur_t / 2;
+                fr_t* slot = sums.gpu_data + 13 * (size_t)k;
+                const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
+                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(e), half, W(slot + 5), side.stream),
+                      "grape_tlookup_round_sums");
+                check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(slot + 10), side.stream), "grape_tlookup_mb_sums");
+                uint32_t* ptrs[3] = {W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
+                check(grape_fr_fold_msb_multi(ptrs, 3, half, W(d_v + vi), side.stream), "grape_fr_fold_msb_multi");
+                cur_t = half;
+            }
+        }
         uint cur = D;
         uint k = 0;
         for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
@@ -269,18 +330,11 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             // A and S: five sums and the fold of both tensors in one pass
             check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), nullptr),
                   "grape_wround2");
-            if (vi < (int)logN) {
-                // phase 2: the table variables
-                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(e), half, W(slot + 5), nullptr),
-                      "grape_tlookup_round_sums");
-                check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(slot + 10), nullptr), "grape_tlookup_mb_sums");
-                uint32_t* ptrs[3] = {W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
-                check(grape_fr_fold_msb_multi(ptrs, 3, half, W(d_v + vi), nullptr), "grape_fr_fold_msb_multi");
-            }
             A.set_size(half);
             S.set_size(half);
             cur = half;
         }
+        side.end();                         // the default stream waits for the table side
         std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1));
         check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * 13 * (size_t)rounds, nullptr), "d2h");
         grape_free(d_v);

@@ -444,7 +444,16 @@ int grape_bench_mad_u64_u32(int blocks, int inner, int iters, double *mads_per_s
  * one entry per pass); *n receives how many were written. */
 int grape_profile_enable(int on);
 int grape_profile_last(float *ms, int cap, int *n);
-/* Event timing helpers on a stream (HIP events), for benchmarks that live above this ABI. */
+/* A second stream for work that is independent of the caller's (the host classes run the table side
+ * of a lookup's rounds on one, beside the witness side): default priority, no implicit
+ * synchronisation with the default stream; order across streams with grape_event_record +
+ * grape_stream_wait_event.  Scratch memory is per stream, so calls on different streams never share
+ * any; grape_stream_destroy waits for the stream and frees its scratch. */
+int grape_stream_create(grape_stream_t *out);
+int grape_stream_destroy(grape_stream_t stream);
+int grape_stream_wait_event(grape_stream_t stream, void *ev);
+/* Event helpers on a stream (HIP events): ordering between streams, and timing for benchmarks that
+ * live above this ABI. */
 int grape_event_create(void **ev);
 int grape_event_destroy(void *ev);
 int grape_event_record(void *ev, grape_stream_t stream);
