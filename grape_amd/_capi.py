@@ -87,6 +87,7 @@ SIGNATURES = {
     "grape_g1_wide_table_bytes": [c_size_t, c_u32, c_u32],
     "grape_g1_scaled_table_gen": [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_i32": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
+    "grape_commit_i32_nowait": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p, c_void_p],
     "grape_commit_fr": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_g1_strided_table_gen": [c_void_p, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_fr_strided": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],

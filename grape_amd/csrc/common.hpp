@@ -33,7 +33,15 @@ void set_error(const char* fmt, ...);
 
 #define GRAPE_LAUNCH_CHECK() GRAPE_HIP_CHECK(hipGetLastError())
 
-static inline hipStream_t as_stream(grape_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+// Tells the block cache of grape_malloc / grape_free which streams carry this library's work (see
+// runtime.hip): the default stream and the streams made by grape_stream_create are known to it, any
+// other stream makes it wait for the whole device again before a kept block is reused.
+void note_stream(hipStream_t s);
+static inline hipStream_t as_stream(grape_stream_t s) {
+    hipStream_t h = reinterpret_cast<hipStream_t>(s);
+    if (h) note_stream(h);
+    return h;
+}
 
 constexpr int kBlock = 256;          // 4 wave64 per workgroup
 constexpr int kNumCU = 256;          // MI355X

@@ -827,7 +827,7 @@ constexpr size_t kMaxCommitScalars = (size_t)1 << 28;
 
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
-                            uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
+                            uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st, int* caller_flag = nullptr) {
     if (size == 0) return GRAPE_OK;                      // no rows: nothing is read or written
     GRAPE_REQUIRE(size <= kMaxCommitScalars, "more than 2^28 scalars in one call: commit the rows in several calls");
     CHECK_PTR16(out); CHECK_PTR16(scalars); CHECK_PTR16(table);
@@ -849,9 +849,13 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     void* ws;
     int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws, s);
     if (rc) return rc;
-    int* err = (int*)((char*)ws + partial_bytes);
-    rc = zero_fill(err, sizeof(int), s);
-    if (rc) return rc;
+    // the digit-range flag: the call's own (cleared here, read back at the end), or one the caller
+    // owns, has cleared and reads when it likes - then nothing here waits for the stream
+    int* err = caller_flag ? caller_flag : (int*)((char*)ws + partial_bytes);
+    if (!caller_flag) {
+        rc = zero_fill(err, sizeof(int), s);
+        if (rc) return rc;
+    }
     const size_t elem_words = FR ? 8 : 1;
     const size_t rows_per_wave = (size_t)64 >> lg_lpr;
     profile_begin();
@@ -866,6 +870,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
         profile_mark(s);
     }
     GRAPE_LAUNCH_CHECK();
+    if (caller_flag) return GRAPE_OK;
     int h_err = 0;
     GRAPE_HIP_CHECK(hipMemcpyAsync(&h_err, err, sizeof(int), hipMemcpyDeviceToHost, s));
     GRAPE_HIP_CHECK(hipStreamSynchronize(s));
@@ -1111,6 +1116,11 @@ int grape_commit_fr_sparse(uint32_t* out, const uint32_t* scalars, const int32_t
 int grape_commit_i32(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                      uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     return commit_wide_impl<false>(out, scalars, size, rowlen, table, N, c, nw, K, st);
+}
+int grape_commit_i32_nowait(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                            uint32_t c, uint32_t nw, uint32_t K, int32_t* d_flag, grape_stream_t st) {
+    GRAPE_REQUIRE(d_flag != nullptr, "the caller's flag is required");
+    return commit_wide_impl<false>(out, scalars, size, rowlen, table, N, c, nw, K, st, d_flag);
 }
 int grape_commit_fr(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                     uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {

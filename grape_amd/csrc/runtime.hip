@@ -3,8 +3,10 @@
 #include <stdarg.h>
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
 #include <map>
 #include <mutex>
+#include <vector>
 #include "common.hpp"
 
 namespace grape {
@@ -139,9 +141,28 @@ __global__ void __launch_bounds__(256) mad_kernel(uint64_t* out, int inner, uint
 // may rely on that and free a buffer that queued kernels still use, so the wait happens when a
 // cached block is handed out again instead.
 static std::mutex g_alloc_mu;
-static std::map<void*, size_t>* g_live = nullptr;              // blocks handed out by grape_malloc
-static std::multimap<size_t, void*>* g_cached = nullptr;       // freed blocks kept for reuse
+// A kept block may only be handed out again once the work that was queued when it was freed has
+// finished - what hipFree would have waited for.  Waiting for the whole device at that point
+// (hipDeviceSynchronize) would also wait for work queued LATER on other streams, e.g. for the rounds
+// a lookup has queued on its side streams while its commitments allocate on the default stream; so
+// the free records an event on every stream the library knows (the default stream and the streams
+// of grape_stream_create) and the reuse waits for those events only.  Once a caller has brought a
+// stream of its own the cache cannot know what that stream still runs and goes back to waiting for
+// the device.
+constexpr int kMaxLibStreams = 16;
+struct CachedBlock {
+    void* p = nullptr;
+    hipEvent_t ev[1 + kMaxLibStreams];
+    int nev = 0;
+    bool whole_device = false;
+};
+static std::map<void*, size_t>* g_live = nullptr;                    // blocks handed out by grape_malloc
+static std::multimap<size_t, CachedBlock>* g_cached = nullptr;       // freed blocks kept for reuse
 static size_t g_cached_bytes = 0;
+static std::vector<hipEvent_t>* g_event_pool = nullptr;
+static hipStream_t g_lib_streams[kMaxLibStreams];
+static std::atomic<int> g_n_lib_streams{0};
+static std::atomic<bool> g_foreign_stream{false};
 static size_t alloc_cache_cap() {
     static size_t cap = [] {
         size_t gib = 32;
@@ -157,18 +178,67 @@ static size_t alloc_cache_cap() {
 static void alloc_tables() {
     if (!g_live) {
         g_live = new std::map<void*, size_t>();
-        g_cached = new std::multimap<size_t, void*>();
+        g_cached = new std::multimap<size_t, CachedBlock>();
+        g_event_pool = new std::vector<hipEvent_t>();
     }
+}
+static bool take_event(hipEvent_t* out) {
+    if (!g_event_pool->empty()) {
+        *out = g_event_pool->back();
+        g_event_pool->pop_back();
+        return true;
+    }
+    if (hipEventCreateWithFlags(out, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return true;
+}
+// marks the point up to which the block may still be in use: an event on every known stream
+static void stamp_block(CachedBlock& b) {
+    b.nev = 0;
+    b.whole_device = g_foreign_stream.load();
+    if (b.whole_device) return;
+    const int n = g_n_lib_streams.load();
+    for (int i = -1; i < n; i++) {
+        hipEvent_t e;
+        if (!take_event(&e) || hipEventRecord(e, i < 0 ? (hipStream_t) nullptr : g_lib_streams[i]) != hipSuccess) {
+            (void)hipGetLastError();
+            b.whole_device = true;
+            break;
+        }
+        b.ev[b.nev++] = e;
+    }
+}
+static int wait_block(CachedBlock& b) {
+    if (b.whole_device) GRAPE_HIP_CHECK(hipDeviceSynchronize());
+    for (int i = 0; i < b.nev; i++) {
+        if (!b.whole_device) GRAPE_HIP_CHECK(hipEventSynchronize(b.ev[i]));
+        g_event_pool->push_back(b.ev[i]);
+    }
+    b.nev = 0;
+    return GRAPE_OK;
 }
 // gives every cached block back to the driver; returns the bytes released
 static size_t alloc_cache_release_locked() {
     size_t n = g_cached_bytes;
     if (g_cached) {
-        for (auto& e : *g_cached) (void)hipFree(e.second);
+        for (auto& e : *g_cached) {
+            (void)hipFree(e.second.p);                    // waits for the device
+            for (int i = 0; i < e.second.nev; i++) g_event_pool->push_back(e.second.ev[i]);
+        }
         g_cached->clear();
     }
     g_cached_bytes = 0;
     return n;
+}
+
+void note_stream(hipStream_t s) {
+    if (g_foreign_stream.load(std::memory_order_relaxed)) return;
+    const int n = g_n_lib_streams.load(std::memory_order_acquire);
+    for (int i = 0; i < n; i++)
+        if (g_lib_streams[i] == s) return;
+    g_foreign_stream.store(true);
 }
 
 size_t alloc_cache_release() {
@@ -205,13 +275,13 @@ int grape_malloc(void** p, size_t bytes) {
     alloc_tables();
     auto it = g_cached->find(bytes);
     if (it != g_cached->end()) {
-        void* q = it->second;
+        CachedBlock b = it->second;
         g_cached->erase(it);
         g_cached_bytes -= bytes;
-        GRAPE_HIP_CHECK(hipDeviceSynchronize());          // what hipFree would have waited for
-        (*g_live)[q] = bytes;
-        *p = q;
-        return GRAPE_OK;
+        int rc = wait_block(b);                           // what hipFree would have waited for
+        (*g_live)[b.p] = bytes;
+        *p = b.p;
+        return rc;
     }
     hipError_t e = hipMalloc(p, bytes);
     if (e != hipSuccess && alloc_cache_release_locked() > 0) {
@@ -235,7 +305,10 @@ int grape_free(void* p) {
         const size_t bytes = it->second;
         g_live->erase(it);
         if (g_cached_bytes + bytes <= alloc_cache_cap()) {
-            g_cached->emplace(bytes, p);
+            CachedBlock b;
+            b.p = p;
+            stamp_block(b);
+            g_cached->emplace(bytes, b);
             g_cached_bytes += bytes;
             return GRAPE_OK;
         }
@@ -294,7 +367,12 @@ int grape_profile_last(float* ms, int cap, int* n) {
 int grape_stream_create(grape_stream_t* out) {
     GRAPE_REQUIRE(out != nullptr, "null output");
     hipStream_t s;
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    const int n = g_n_lib_streams.load();
+    GRAPE_REQUIRE(n < kMaxLibStreams, "too many streams");
     GRAPE_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    g_lib_streams[n] = s;
+    g_n_lib_streams.store(n + 1, std::memory_order_release);
     *out = reinterpret_cast<grape_stream_t>(s);
     return GRAPE_OK;
 }
@@ -310,6 +388,20 @@ int grape_stream_destroy(grape_stream_t st) {
                 for (int k = 0; k < kNumSlots; k++)
                     if (it->second.ptr[k]) (void)hipFree(it->second.ptr[k]);
                 g_pools->erase(it);
+            }
+        }
+    }
+    {
+        // the blocks freed while this stream existed carry events recorded on it: wait for the device
+        // once, so that those events count as reached, and forget the stream
+        std::lock_guard<std::mutex> lock(g_alloc_mu);
+        GRAPE_HIP_CHECK(hipDeviceSynchronize());
+        const int n = g_n_lib_streams.load();
+        for (int i = 0; i < n; i++) {
+            if (g_lib_streams[i] == s) {
+                g_lib_streams[i] = g_lib_streams[n - 1];
+                g_n_lib_streams.store(n - 1, std::memory_order_release);
+                break;
             }
         }
     }

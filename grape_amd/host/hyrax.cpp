@@ -123,15 +123,18 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
             int16_ok_ = false;   // a scalar outside int16: use the general tables from now on
         }
     }
-    commit_i32_rows(out, tensor, size, rowlen);
+    commit_i32_rows(out, tensor, size, rowlen, nullptr);
     return out;
 }
 
 // any int32 scalars: five signed 8-bit digits per scalar through a small table, or the reference's
 // byte windows when even that table is over budget
-void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen) {
+void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag) {
     if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+                  if (d_flag)
+                      return grape_commit_i32_nowait(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128,
+                                                     d_flag, nullptr);
                   return grape_commit_i32(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr);
               }),
               "grape_commit_i32");
@@ -143,12 +146,12 @@ void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen
     }
 }
 
-affine_t* Hyrax::commit_affine_i32(int* tensor, uint size, uint N) {
+affine_t* Hyrax::commit_affine_i32(int* tensor, uint size, uint N, int* d_flag) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)(size / rowlen)), "grape_malloc");
-    commit_i32_rows(out, tensor, size, rowlen);
+    commit_i32_rows(out, tensor, size, rowlen, d_flag);
     return out;
 }
 
@@ -290,7 +293,7 @@ void Hyrax::release_scaled_table(affine_t* table) {
     grape_free(table);
 }
 
-affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len) {
+affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len, int* d_flag) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;
     if (rowlen > ncols) throw std::runtime_error("row longer than the scaled table");
@@ -300,6 +303,7 @@ affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine
     // one unsigned "digit" idx+1 in [1, len]: radix 2^(log2(len)+1) keeps it below the sign threshold
     const uint c = Log2(len) + 1 < 2 ? 2 : Log2(len) + 1;
     check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
+              if (d_flag) return grape_commit_i32_nowait(W(out + r0), idx_plus1 + e0, n, rowlen, W(scaled_table), ncols, c, 1, len, d_flag, nullptr);
               return grape_commit_i32(W(out + r0), idx_plus1 + e0, n, rowlen, W(scaled_table), ncols, c, 1, len, nullptr);
           }),
           "grape_commit_i32 (indexed)");

@@ -47,7 +47,9 @@ public:
     affine_t* commit_affine(FrTensor& tensor, uint size, uint N);
     // Integers of any int32 magnitude, without trying the int16 table first (and without giving that
     // table up for this object when a value does not fit it): lookup multiplicities.
-    affine_t* commit_affine_i32(int* tensor, uint size, uint N);
+    // With d_flag (a device int the caller owns and has cleared) the call queues its kernels and returns
+    // without waiting; the flag is 1 afterwards if a scalar did not fit the table's digits.
+    affine_t* commit_affine_i32(int* tensor, uint size, uint N, int* d_flag = nullptr);
 
     Hyrax_proof open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
     // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
@@ -67,7 +69,7 @@ public:
     // Hyrax object that built it, if that object still exists
     static void release_scaled_table(affine_t* table);
     // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
-    affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len);
+    affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len, int* d_flag = nullptr);
 
     // Row commitments of the elements whose flag skip[j] is zero, the others left out; through the
     // per-window table that scaled tables are built with.  nullptr when that table does not exist.
@@ -98,7 +100,7 @@ private:
     size_t table_bytes_in_use() const;
     // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
     void commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build);
-    void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen);
+    void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
     StridedTable fr_strided_;

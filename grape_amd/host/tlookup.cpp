@@ -2,6 +2,7 @@
 #include <cassert>
 #include <chrono>
 #include <cstdio>
+#include <functional>
 #include "../../include/grape_hip.h"
 
 using grape_host::check;
@@ -136,25 +137,25 @@ bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& h
 }
 
 namespace {
-// A second stream (one per process, created on first use) and the two events that order it against
+// A stream beside the default one (two per process, created on first use) and the two events that order it against
 // the default stream: begin() makes it wait for what the default stream has queued, end() makes the
 // default stream wait for it.  If the scope is left by an exception the destructor waits for the
 // stream, so nothing it still reads is freed under it.
 struct SideChain {
     grape_stream_t stream = nullptr;
     bool open = false;
-    SideChain() {
-        static grape_stream_t s = nullptr;
-        static void* e0 = nullptr;
-        static void* e1 = nullptr;
-        if (!s) {
-            check(grape_stream_create(&s), "grape_stream_create");
-            check(grape_event_create(&e0), "grape_event_create");
-            check(grape_event_create(&e1), "grape_event_create");
+    explicit SideChain(int which) {
+        static grape_stream_t s[2] = {nullptr, nullptr};
+        static void* e0[2] = {nullptr, nullptr};
+        static void* e1[2] = {nullptr, nullptr};
+        if (!s[which]) {
+            check(grape_stream_create(&s[which]), "grape_stream_create");
+            check(grape_event_create(&e0[which]), "grape_event_create");
+            check(grape_event_create(&e1[which]), "grape_event_create");
         }
-        stream = s;
-        ev_begin = e0;
-        ev_end = e1;
+        stream = s[which];
+        ev_begin = e0[which];
+        ev_end = e1[which];
     }
     void begin() {
         check(grape_event_record(ev_begin, nullptr), "grape_event_record");
@@ -172,6 +173,16 @@ struct SideChain {
     void* ev_begin = nullptr;
     void* ev_end = nullptr;
 };
+// the two events that bracket the commitments queued beside the rounds
+std::pair<void*, void*> commit_events() {
+    static void* a = nullptr;
+    static void* b = nullptr;
+    if (!a) {
+        check(grape_event_create(&a), "grape_event_create");
+        check(grape_event_create(&b), "grape_event_create");
+    }
+    return {a, b};
+}
 }  // namespace
 
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
@@ -236,18 +247,32 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     if (!from_table) check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
     A.set_size(D);
 
-    {   // commitments of A and m (kept, not dropped)
+    // Commitments of A and m (kept, not dropped).  With the scaled table of a range lookup the
+    // commitment of A reads only the indices, so it does not have to finish before the rounds start
+    // folding A: the rounds are then queued first, on streams of their own, and the commitments run
+    // beside them (the short rounds and the row reductions of the commitments are latency chains
+    // that leave most of the chip idle on their own).  Otherwise the commitments come first.
+    const uint rowlen = msm_size * hyrax.com_scale;
+    auto timed = [&](const std::function<void()>& fn) {
         auto t0 = std::chrono::steady_clock::now();
-        grape_free(com_A);
-        grape_free(com_m);
-        const uint rowlen = msm_size * hyrax.com_scale;
+        fn();
+        commit_time += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    };
+    timed([&] {
         if (indexed_commit_ && index_known_ && (scaled_for_ != &hyrax || scaled_cols_ < rowlen)) {
             Hyrax::release_scaled_table(scaled_table_);
             scaled_table_ = hyrax.build_scaled_table(B, rowlen);   // nullptr when over budget
             scaled_cols_ = scaled_table_ ? rowlen : 0;
             scaled_for_ = &hyrax;
         }
-        if (indexed_commit_ && index_known_ && scaled_table_) {
+    });
+    const bool indexed = indexed_commit_ && index_known_ && scaled_table_;
+    const bool overlap = indexed && d_idx_ != nullptr;
+    auto commit_all = [&] {
+        grape_free(com_A);
+        grape_free(com_m);
+        com_A = com_m = nullptr;
+        if (indexed) {
             int* d_idx = d_idx_;
             if (!d_idx) {
                 check(grape_malloc((void**)&d_idx, sizeof(int) * (size_t)D), "grape_malloc");
@@ -269,8 +294,8 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         else com_m = hyrax.commit_affine(m, N, m_N);
         com_m_rows = N / (m_N * hyrax.com_scale);
         check(grape_stream_sync(nullptr), "sync");
-        commit_time += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-    }
+    };
+    if (!overlap) timed(commit_all);
 
     FrTensor Bm(B);
     Bm *= m;
@@ -298,14 +323,57 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     const uint rounds = (uint)v.size();
     FrTensor sums(13 * (rounds ? rounds : 1));
     fr_t* d_v = grape_host::upload(v);
+    int* d_flags = nullptr;
     FrTensor Bw(B), Tw(T), mw(m);          // phase 2 binds copies; T, B, m of this object stay intact
     try {
         // The table side of phase 2 (B, T, m: sums and folds of the last log2(N) rounds) depends on
         // nothing the witness side produces, so it runs as a chain of its own on a second stream,
         // beside the rounds over A and S (the short rounds are launch- and latency-bound: five
         // small kernels per round on the table side, two on the witness side).
-        SideChain side;
+        SideChain side(0), witness(1);
         side.begin();                       // the second stream waits for everything queued so far
+        grape_stream_t ws = nullptr;        // where the witness side runs: the default stream, or one of its own beside the commitments
+        if (overlap) {
+            witness.begin();                // both streams wait for what is queued so far - not for the commitments, queued next
+            ws = witness.stream;
+        }
+        // overlap: the commitments are queued now, without waiting (their digit-range flags are read
+        // after the rounds have been queued too), so the chip works on them while the host issues
+        // the rounds' launches; everything that needs the host to wait on the default stream (the
+        // sums above) is behind us
+        if (overlap) {
+            check(grape_malloc((void**)&d_flags, 2 * sizeof(int)), "grape_malloc");
+            check(grape_memset_zero(d_flags, 2 * sizeof(int), nullptr), "grape_memset_zero");
+            // commit_time of this mode: what the commitment kernels take on the default stream, between two events
+            check(grape_event_record(commit_events().first, nullptr), "grape_event_record");
+            timed([&] {
+                grape_free(com_A);
+                grape_free(com_m);
+                com_A = com_m = nullptr;
+                com_A = hyrax.commit_indexed_affine(d_idx_, D, msm_size, scaled_table_, scaled_cols_, N, d_flags);
+                com_A_rows = D / (msm_size * hyrax.com_scale);
+                uint m_N = 1u << (Log2(N) / 2);
+                if (d_hist_ && D < (1u << 31)) com_m = hyrax.commit_affine_i32(reinterpret_cast<int*>(d_hist_), N, m_N, d_flags + 1);
+                else com_m = hyrax.commit_affine(m, N, m_N);
+                com_m_rows = N / (m_N * hyrax.com_scale);
+            });
+            check(grape_event_record(commit_events().second, nullptr), "grape_event_record");
+        }
+        uint cur = D;
+        uint k = 0;
+        for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
+            const uint half = cur / 2;
+            fr_t* slot = sums.gpu_data + 13 * (size_t)k;
+            const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
+            // A and S: five sums and the fold of both tensors in one pass
+            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), ws),
+                  "grape_wround2");
+            A.set_size(half);
+            S.set_size(half);
+            cur = half;
+        }
+        // the table side is queued second: its many small launches reach the chip while it works on the
+        // first, long rounds of the witness side
         {
             uint cur_t = N;
             for (int vi = (int)logN - 1; vi >= 0 && vi < (int)rounds; vi--) {
@@ -321,20 +389,18 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
                 cur_t = half;
             }
         }
-        uint cur = D;
-        uint k = 0;
-        for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
-            const uint half = cur / 2;
-            fr_t* slot = sums.gpu_data + 13 * (size_t)k;
-            const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
-            // A and S: five sums and the fold of both tensors in one pass
-            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), nullptr),
-                  "grape_wround2");
-            A.set_size(half);
-            S.set_size(half);
-            cur = half;
-        }
+        if (overlap) witness.end();
         side.end();                         // the default stream waits for the table side
+        if (overlap) {
+            int flags[2] = {0, 0};
+            check(grape_memcpy_d2h(flags, d_flags, sizeof flags, nullptr), "d2h");
+            grape_free(d_flags);
+            d_flags = nullptr;
+            if (flags[0] || flags[1]) throw std::runtime_error("tLookup: a commitment inside the proof met a scalar outside its table's digits");
+            float ms = 0;
+            check(grape_event_elapsed_ms(&ms, commit_events().first, commit_events().second), "grape_event_elapsed_ms");
+            commit_time += ms * 1e-3;
+        }
         std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1));
         check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * 13 * (size_t)rounds, nullptr), "d2h");
         grape_free(d_v);
@@ -372,6 +438,7 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         }
     } catch (...) {
         grape_free(d_v);
+        grape_free(d_flags);
         throw;
     }
     return S(0u);

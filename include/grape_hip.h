@@ -331,6 +331,14 @@ int grape_g1_scaled_table_gen(uint32_t *d_out, const uint32_t *d_scalars_mont, s
  */
 int grape_commit_i32(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
                      const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/* grape_commit_i32 without the wait at its end: the kernels are queued and the call returns.  The
+ * digit-range check lands in *d_flag (device int32 the caller owns and has cleared: set to 1 when a
+ * scalar did not fit, in which case the outputs are meaningless); the caller reads it after
+ * synchronising the stream.  For callers that queue other work while the commitment runs (the
+ * lookups' rounds on streams of their own). */
+int grape_commit_i32_nowait(uint32_t *d_out_affine, const int32_t *d_scalars, size_t size, uint32_t rowlen,
+                            const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, int32_t *d_flag,
+                            grape_stream_t stream);
 /* Same for full-width Fr scalars (Montgomery form in, left untouched — the reference's
  * tensor.from()/to() round trip of src/Hyrax.cu:347,356 is not needed).
  * Hyrax::commit(FrTensor&, size, N), src/Hyrax.cu:335-359. Requires nw*c >= 255: a scalar in the
