@@ -6,6 +6,7 @@
 #include <atomic>
 #include <map>
 #include <mutex>
+#include <thread>
 #include <vector>
 #include "common.hpp"
 
@@ -163,6 +164,28 @@ static std::vector<hipEvent_t>* g_event_pool = nullptr;
 static hipStream_t g_lib_streams[kMaxLibStreams];
 static std::atomic<int> g_n_lib_streams{0};
 static std::atomic<bool> g_foreign_stream{false};
+// Blocks are also freed while the process exits (destructors of static objects that own tensors).
+// By then layers under this one may be half torn down - a profiler's per-thread stream bookkeeping
+// is gone once the main thread's thread-local objects have been destroyed, and a stream call then
+// aborts - so from that point on a free records nothing.  The point is marked by the destructor of a
+// thread-local object of the thread that initialised the library: thread-local objects of the
+// exiting thread are destroyed before any static object.
+static std::atomic<bool> g_exit_started{false};
+static std::atomic<bool> g_first_thread_set{false};
+static std::thread::id g_first_thread;
+struct ExitSentinel {
+    ~ExitSentinel() {
+        if (g_first_thread_set.load() && std::this_thread::get_id() == g_first_thread) g_exit_started.store(true);
+    }
+};
+static void touch_exit_sentinel() {
+    thread_local ExitSentinel sentinel;
+    (void)&sentinel;
+    if (!g_first_thread_set.load()) {
+        g_first_thread = std::this_thread::get_id();
+        g_first_thread_set.store(true);
+    }
+}
 static size_t alloc_cache_cap() {
     static size_t cap = [] {
         size_t gib = 32;
@@ -197,9 +220,11 @@ static bool take_event(hipEvent_t* out) {
 // marks the point up to which the block may still be in use: an event on every known stream
 static void stamp_block(CachedBlock& b) {
     b.nev = 0;
-    b.whole_device = g_foreign_stream.load();
-    if (b.whole_device) return;
     const int n = g_n_lib_streams.load();
+    // with the default stream alone there is nothing a wait for the device would wait for needlessly,
+    // and it costs less than an event per free
+    b.whole_device = n == 0 || g_foreign_stream.load() || g_exit_started.load();
+    if (b.whole_device) return;
     for (int i = -1; i < n; i++) {
         hipEvent_t e;
         if (!take_event(&e) || hipEventRecord(e, i < 0 ? (hipStream_t) nullptr : g_lib_streams[i]) != hipSuccess) {
@@ -261,6 +286,7 @@ int grape_init(int device) {
         return GRAPE_EINVAL;
     }
     g_init = true;
+    touch_exit_sentinel();
     return noalloc_setup();
 }
 const char* grape_last_error(void) { return g_err; }
@@ -299,6 +325,7 @@ int grape_malloc(void** p, size_t bytes) {
 int grape_free(void* p) {
     if (!p) return GRAPE_OK;
     std::lock_guard<std::mutex> lock(g_alloc_mu);
+    touch_exit_sentinel();
     alloc_tables();
     auto it = g_live->find(p);
     if (it != g_live->end()) {

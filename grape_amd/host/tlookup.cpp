@@ -141,21 +141,22 @@ namespace {
 // the default stream: begin() makes it wait for what the default stream has queued, end() makes the
 // default stream wait for it.  If the scope is left by an exception the destructor waits for the
 // stream, so nothing it still reads is freed under it.
+grape_stream_t g_side_stream[2] = {nullptr, nullptr};
+void* g_side_event[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+void* g_commit_event[2] = {nullptr, nullptr};
+// (never destroyed: they live as long as the process, like the HIP runtime's own default stream)
 struct SideChain {
     grape_stream_t stream = nullptr;
     bool open = false;
     explicit SideChain(int which) {
-        static grape_stream_t s[2] = {nullptr, nullptr};
-        static void* e0[2] = {nullptr, nullptr};
-        static void* e1[2] = {nullptr, nullptr};
-        if (!s[which]) {
-            check(grape_stream_create(&s[which]), "grape_stream_create");
-            check(grape_event_create(&e0[which]), "grape_event_create");
-            check(grape_event_create(&e1[which]), "grape_event_create");
+        if (!g_side_stream[which]) {
+            check(grape_stream_create(&g_side_stream[which]), "grape_stream_create");
+            check(grape_event_create(&g_side_event[which][0]), "grape_event_create");
+            check(grape_event_create(&g_side_event[which][1]), "grape_event_create");
         }
-        stream = s[which];
-        ev_begin = e0[which];
-        ev_end = e1[which];
+        stream = g_side_stream[which];
+        ev_begin = g_side_event[which][0];
+        ev_end = g_side_event[which][1];
     }
     void begin() {
         check(grape_event_record(ev_begin, nullptr), "grape_event_record");
@@ -175,13 +176,11 @@ struct SideChain {
 };
 // the two events that bracket the commitments queued beside the rounds
 std::pair<void*, void*> commit_events() {
-    static void* a = nullptr;
-    static void* b = nullptr;
-    if (!a) {
-        check(grape_event_create(&a), "grape_event_create");
-        check(grape_event_create(&b), "grape_event_create");
+    if (!g_commit_event[0]) {
+        check(grape_event_create(&g_commit_event[0]), "grape_event_create");
+        check(grape_event_create(&g_commit_event[1]), "grape_event_create");
     }
-    return {a, b};
+    return {g_commit_event[0], g_commit_event[1]};
 }
 }  // namespace
 
