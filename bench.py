@@ -556,8 +556,11 @@ def rounds_workload(args):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / args.steps
 
+    claim = ops.to_dev(rand_fr(1, 79))
     cases = [
-        ("sumcheck2_kernel<false> + final_sum (grape_sumcheck_round2)", 192, h, lambda: ops.sumcheck_round2(A, B, n, h, v)),
+        ("sumcheck2_kernel<two sums> + claim_final (grape_sumcheck_round2_claim, as prove_matmul's long rounds run)", 192, h,
+         lambda: ops.sumcheck_round2_claim(A, B, n, h, v, claim)),
+        ("sumcheck2_kernel<three sums> + final_sum (grape_sumcheck_round2)", 192, h, lambda: ops.sumcheck_round2(A, B, n, h, v)),
         ("wround2_kernel<beta, plain sums> + final (grape_wround2, logUp round)", 224, h,
          lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True)),
         ("wround2_kernel<no beta> + final (grape_wround2, element-product round)", 224, h,

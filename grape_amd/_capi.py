@@ -51,6 +51,7 @@ SIGNATURES = {
     "grape_i32_pad_fill": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_i32, c_void_p],
     "grape_fr_fold": [c_void_p, c_size_t, c_void_p, c_u32, c_u32, c_u32, c_void_p],
     "grape_sumcheck_round2": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
+    "grape_sumcheck_round2_claim": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_noalloc": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_tail": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_coeffs": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],

@@ -21,6 +21,11 @@ __device__ __forceinline__ void st_fr(uint32_t* base, size_t i, const Fr& a) {
 }
 
 // element as 26-bit working limbs straight from memory
+// Marks an element as used at this point of the program, so that the wait for the loads that
+// produce it is placed here.
+__device__ __forceinline__ void arrived(Fr& a) {
+    asm volatile("" : "+v"(a.v[0]), "+v"(a.v[1]), "+v"(a.v[2]), "+v"(a.v[3]), "+v"(a.v[4]), "+v"(a.v[5]), "+v"(a.v[6]), "+v"(a.v[7]));
+}
 __device__ __forceinline__ fr26::Limbs ld_l26(const uint32_t* base, size_t i) { return fr26::pack(ld_fr(base, i)); }
 
 using fr26::fold1;

@@ -15,7 +15,10 @@ namespace grape {
 // with 16 pairs per thread that was a quarter of the kernel, with 64 it is a fifteenth.
 constexpr int kRoundIters = 64;
 
-template <bool COEFFS, bool TAB>
+// CLAIM: the sum of the round polynomial over {0, 1} is known (it is the value the previous round's
+// polynomial took at its challenge), so the value at t = 1 is not accumulated: the kernel leaves
+// c0 and c2 and the finishing kernel takes c1 = claim - 2 c0 - c2.
+template <bool COEFFS, bool TAB, bool CLAIM = false, bool PREFETCH = CLAIM>
 __global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint32_t* B, uint32_t* ca, uint32_t* cb, uint32_t* cc,
                                                            uint32_t in_size, uint32_t out_size, const uint32_t* v,
                                                            const int32_t* __restrict__ tab, uint32_t* partial) {
@@ -27,20 +30,22 @@ __global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint3
     fr26::acc_zero(Q);
     fr26::acc_zero(C2);
     const size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x; g < out_size; g += stride) {
-        const fr26::Limbs a0 = ld_l26(A, g), b0 = ld_l26(B, g);
-        const fr26::Limbs a1 = ld_hi26(A, g, out_size, in_size), b1 = ld_hi26(B, g, out_size, in_size);
+    size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    // one index: fold both tensors in place and add the index's products to the coefficient sums
+    auto step = [&](size_t i, const Fr& ra0, const Fr& rb0, const Fr& ra1, const Fr& rb1) __attribute__((always_inline)) {
+        const fr26::Limbs a0 = fr26::pack(ra0), b0 = fr26::pack(rb0);
+        const fr26::Limbs a1 = fr26::pack(ra1), b1 = fr26::pack(rb1);
         const fr26::Limbs da = fr26::sub(a1, a0), db = fr26::sub(b1, b0);   // signed, |limb| < 2^26
         // long rounds fold through the table of the challenge's multiples (no full reduction), short
         // ones through one limb product (no table to prepare)
         if (TAB) {
             Fr fa, fb;
             foldt2(tab, a0, da, b0, db, fa, fb);
-            st_fr(A, g, fa);
-            st_fr(B, g, fb);
+            st_fr(A, i, fa);
+            st_fr(B, i, fb);
         } else {
-            st_fr(A, g, fold1(w1, a0, da));
-            st_fr(B, g, fold1(w1, b0, db));
+            st_fr(A, i, fold1(w1, a0, da));
+            st_fr(B, i, fold1(w1, b0, db));
         }
         if (COEFFS) {
             // materialised coefficient arrays (phase 1 folds them further)
@@ -53,26 +58,90 @@ __global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint3
             const Fr a_ = fr26::finish_sum(T, 1);
             fr26::acc_zero(T);
             fr26::mac(T, a1, b1);
-            st_fr(cc, g, c_);
-            st_fr(cb, g, sub(sub(fr26::finish_sum(T, 0), c_), a_));
-            st_fr(ca, g, a_);
+            st_fr(cc, i, c_);
+            st_fr(cb, i, sub(sub(fr26::finish_sum(T, 0), c_), a_));
+            st_fr(ca, i, a_);
         }
         // middle coefficient by Karatsuba: da*b0 + a0*db = a1*b1 - a0*b0 - da*db, so the value at
         // t = 1 is accumulated with one product instead of two
         fr26::mac(C0, a0, b0);
-        fr26::mac(Q, a1, b1);
+        if (!CLAIM) fr26::mac(Q, a1, b1);
         fr26::mac(C2, da, db);
+    };
+    if (!PREFETCH) {
+        for (; g < out_size; g += stride)
+            step(g, ld_fr(A, g), ld_fr(B, g), ld_hi(A, g, out_size, in_size), ld_hi(B, g, out_size, in_size));
+    } else if (g < out_size) {
+        // The next index's four operands are requested before this index's arithmetic starts, so a
+        // wave's memory latency passes under its own ~3000 cycles of multiplies instead of under the
+        // one other wave that the register budget leaves on the SIMD.  Two register sets take turns
+        // (one is loaded while the other is worked on), so no copies stand between the loads and their
+        // use.  All loads are unconditional, for the same reason: past the thread's last index they
+        // repeat the current index (values unused), and an upper operand past the live extent is read
+        // from the lower operand's address and replaced by zero when it is used.
+        struct Set { Fr a0, b0, a1, b1; uint32_t hi_mask; };
+        auto request = [&](Set& s, size_t i) __attribute__((always_inline)) {
+            const bool hi_live = i + out_size < in_size;
+            s.hi_mask = hi_live ? 0xffffffffu : 0u;
+            const size_t ih = hi_live ? i + out_size : i;
+            s.a0 = ld_fr(A, i), s.b0 = ld_fr(B, i), s.a1 = ld_fr(A, ih), s.b1 = ld_fr(B, ih);
+        };
+        auto work = [&](size_t i, const Set& s) __attribute__((always_inline)) {
+            Fr a1 = s.a1, b1 = s.b1;
+#pragma unroll
+            for (int k = 0; k < 8; k++) a1.v[k] &= s.hi_mask, b1.v[k] &= s.hi_mask;
+            step(i, s.a0, s.b0, a1, b1);
+        };
+        Set x, y;
+        request(x, g);
+        // the first operands are waited for here: a wait at the loop's head would also hold up every
+        // later pass, whose operands arrived during the pass before
+        arrived(x.a0), arrived(x.b0), arrived(x.a1), arrived(x.b1);
+        for (;;) {
+            size_t gn = g + stride;
+            request(y, gn < out_size ? gn : g);
+            work(g, x);
+            if (gn >= out_size) break;
+            g = gn, gn = g + stride;
+            request(x, gn < out_size ? gn : g);
+            work(g, y);
+            if (gn >= out_size) break;
+            g = gn;
+        }
     }
     if (partial) {
         // |sum| < 16 r^2 -> within (-0.46 r, 1.46 r) after reduction
-        const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2), q1 = fr26::finish_sum(Q, 2);
-        Fr acc[3] = {c0, sub(sub(q1, c0), c2), c2};
+        const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2);
+        Fr acc[3] = {c0, Fr::zero(), c2};
+        if (!CLAIM) acc[1] = sub(sub(fr26::finish_sum(Q, 2), c0), c2);
         block_sum<3>(acc, lds);
         if (threadIdx.x == 0) {
             st_fr(partial, (size_t)blockIdx.x * 3 + 0, acc[0]);
             st_fr(partial, (size_t)blockIdx.x * 3 + 1, acc[1]);
             st_fr(partial, (size_t)blockIdx.x * 3 + 2, acc[2]);
         }
+    }
+}
+
+// Finishes a round that was summed without its middle coefficient: out = (c0, claim - 2 c0 - c2, c2),
+// and the claim of the next round, the polynomial's value at the challenge v, replaces *claim.
+__global__ void __launch_bounds__(kBlock) sumcheck2_claim_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks,
+                                                                       uint32_t* claim, const uint32_t* v) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
+    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
+        acc[0] = add(acc[0], ld_fr(partial, (size_t)b * 3));
+        acc[2] = add(acc[2], ld_fr(partial, (size_t)b * 3 + 2));
+    }
+    block_sum<3>(acc, lds);
+    if (threadIdx.x == 0) {
+        const Fr c0 = acc[0], c2 = acc[2];
+        const Fr c1 = sub(sub(sub(ld_fr(claim, 0), c0), c0), c2);
+        const Fr vv = ld_fr(v, 0);
+        st_fr(out, 0, c0);
+        st_fr(out, 1, c1);
+        st_fr(out, 2, c2);
+        st_fr(claim, 0, add(c0, fr26::mulc(vv, add(c1, fr26::mulc(vv, c2)))));
     }
 }
 
@@ -645,6 +714,28 @@ int grape_sumcheck_round2_tail(uint32_t* A, uint32_t* B, uint32_t in_size, uint3
 int grape_sumcheck_round2(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums, grape_stream_t st) {
     GRAPE_REQUIRE(sums != nullptr, "d_sums is required");
     return sumcheck2_impl<false>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, sums, st);
+}
+int grape_sumcheck_round2_claim(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* claim,
+                                uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(B); CHECK_PTR16(v); CHECK_PTR16(claim); CHECK_PTR16(sums);
+    GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * out_size, "need out_size <= in_size <= 2*out_size");
+    hipStream_t s = as_stream(st);
+    const unsigned nb = reduce_grid(out_size);
+    const size_t partial_bytes = (size_t)nb * 3 * 32;
+    void* ws;
+    int rc = scratch_get(kSlotReduce, partial_bytes + kFoldTableBytes, &ws, s);
+    if (rc) return rc;
+    uint32_t* partial = (uint32_t*)ws;
+    if (out_size >= kTableFoldMinOut) {
+        int32_t* tab = (int32_t*)((char*)ws + partial_bytes);
+        fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+        sumcheck2_kernel<false, true, true><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, tab, partial);
+    } else {
+        sumcheck2_kernel<false, false, true><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, nullptr, partial);
+    }
+    sumcheck2_claim_final_kernel<<<1, kBlock, 0, s>>>(sums, partial, nb, claim, v);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
 }
 int grape_sumcheck_round2_noalloc(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, const uint32_t* v, uint32_t* sums,
                                   grape_stream_t st) {

@@ -80,6 +80,9 @@ Fr matmul_sumcheck_phase1(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, Fr
     return eq_accumulate;
 }
 
+// rounds of at least this many index pairs take their middle coefficient from the running claim
+static constexpr uint kClaimRoundMinOut = 1u << 16;
+
 // src/prove.cu:87-117, with the three reductions fused into the round kernel
 void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor& c, fr_t* v, uint K, Fr& claim,
                             Fr& eq_accumulate, SumcheckTranscript* transcript) {
@@ -97,7 +100,26 @@ void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, 
     // each leaving its three sums in its own slot, and read with one copy at the end (the
     // reference copies and synchronises after every round).
     FrTensor sums(3 * rounds);
+    // Long rounds (2^16 index pairs and more) are bound by their limb products, and one of the three
+    // per pair can go when the round is given the running claim: p(0) + p(1) = claim fixes the middle
+    // coefficient.  The claim the kernels chain is the one of the bare sums (without eq_accumulate).
+    fr_t* d_claim = nullptr;
+    if (outputsize >= kClaimRoundMinOut && !(eq_accumulate == Fr::zero())) {
+        d_claim = grape_host::upload(std::vector<Fr>{claim * eq_accumulate.inverse()});
+    }
+    struct Release {
+        fr_t*& p;
+        ~Release() { grape_free(p); }
+    } release{d_claim};
     for (uint i = 0; i < rounds; i++) {
+        if (d_claim && outputsize >= kClaimRoundMinOut) {
+            check(grape_sumcheck_round2_claim(W(A.gpu_data), W(B.gpu_data), inputsize, outputsize, W(v - i - 1), W(d_claim),
+                                              W(sums.gpu_data + 3 * i), nullptr),
+                  "grape_sumcheck_round2_claim");
+            inputsize = outputsize;
+            outputsize = outputsize / 2;
+            continue;
+        }
         if (inputsize <= 512) {
             // short tensors: all remaining rounds in one launch
             check(grape_sumcheck_round2_tail(W(A.gpu_data), W(B.gpu_data), inputsize, rounds - i, W(v - i), W(sums.gpu_data + 3 * i), nullptr),

@@ -163,6 +163,14 @@ def fr_fold(t, N, x, c, idx, gap):
 
 
 # ------------------------------------------------------------------ sumcheck / tlookup
+def sumcheck_round2_claim(A, B, in_size, out_size, v, claim):
+    """claim (device, one element) is replaced by the next round's claim; returns the three sums"""
+    lib = init()
+    sums = fr_empty(3)
+    _capi.check(lib.grape_sumcheck_round2_claim(_p(A), _p(B), in_size, out_size, _p(v), _p(claim), _p(sums), _s()))
+    return sums
+
+
 def sumcheck_round2(A, B, in_size, out_size, v):
     lib = init()
     sums = fr_empty(3)

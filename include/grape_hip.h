@@ -122,6 +122,16 @@ int grape_fr_fold(uint32_t *d_t, size_t N, const uint32_t *d_x, uint32_t c, uint
  */
 int grape_sumcheck_round2(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size,
                           const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
+/* The same round when the caller holds the running claim: the sum of a round's polynomial over
+ * {0, 1} equals the value the previous round's polynomial took at its challenge (the check
+ * src/prove.cu:107 makes), so with that value in *d_claim (device, one element) the kernel sums only
+ * c0 and c2 and takes c1 = claim - 2 c0 - c2 - one limb product per index pair fewer, which is what a
+ * long round is bound by.  d_sums receives (c0, c1, c2) as above and *d_claim the next round's claim
+ * c0 + c1 v + c2 v^2, so a chain of rounds needs the claim only once.  A caller that uses it gives up
+ * the per-round check of the sums against the claim; the check of the final claim against the folded
+ * values (src/prove.cu:204) still covers the whole chain. */
+int grape_sumcheck_round2_claim(uint32_t *d_A, uint32_t *d_B, uint32_t in_size, uint32_t out_size, const uint32_t *d_v,
+                                uint32_t *d_claim, uint32_t *d_sums, grape_stream_t stream);
 /* The same round for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
  * results as grape_sumcheck_round2, but the per-workgroup partial sums go to a fixed 384 KiB array

@@ -42,7 +42,8 @@ def _int_tensor(shape, seed):
 
 
 @pytest.mark.parametrize("L,N,M,K", [(1, 4, 8, 16), (2, 4, 4, 8), (4, 2, 4, 4), (1, 3, 5, 6), (1, 8, 4, 1),
-                                     (1, 64, 128, 512), (2, 16, 32, 256), (1, 172, 64, 96)])
+                                     (1, 64, 128, 512), (2, 16, 32, 256), (1, 172, 64, 96),
+                                     (1, 2, 2, 1 << 18)])        # long rounds: middle coefficient from the running claim
 def test_prove_matmul_vs_oracle(ops, host, L, N, M, K):
     import torch
     A = _int_tensor(L * N * K, 1 + N)
@@ -79,13 +80,14 @@ def test_prove_matmul_vs_oracle(ops, host, L, N, M, K):
     assert_same(bc, wbc, "B(v)")
 
 
-def test_prove_matmul_rejects_wrong_claim(ops, host):
+@pytest.mark.parametrize("K", [4, 1 << 17])      # the long case starts with a round that takes its middle coefficient from the claim
+def test_prove_matmul_rejects_wrong_claim(ops, host, K):
     import torch
-    A, B = _int_tensor(2 * 4, 5), _int_tensor(2 * 4, 6)
+    A, B = _int_tensor(2 * K, 5), _int_tensor(2 * K, 6)
     dA = ops.fr_from_i32(torch.from_numpy(A).cuda())
     dB = ops.fr_from_i32(torch.from_numpy(B).cuda())
     with pytest.raises(host.HostError, match="matmul_phase2"):
-        host.prove_matmul(dA, dB, 1, 2, 2, 4, rand_fr(2, 7), rand_fr(2, 8), br.fr_pack([12345])[0])
+        host.prove_matmul(dA, dB, 1, 2, 2, K, rand_fr(2, 7), rand_fr(br.log2ceil(K), 8), br.fr_pack([12345])[0])
 
 
 def test_mle_eval_operator(ops, host):

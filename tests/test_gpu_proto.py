@@ -371,3 +371,33 @@ def test_weighted_sums_of_one_tensor_against_several_tables(ops):
         for j in range(num):
             assert_same(got[2 * j], orc.mle_eval(Xp[:n_out], us[j]), "claim %d, X0" % j)
             assert_same(got[2 * j + 1], orc.mle_eval(d, us[j]), "claim %d, X1 - X0" % j)
+
+
+@pytest.mark.parametrize("in_size", [1 << 18, (1 << 18) - 3000, 5000])
+def test_sumcheck_rounds_chained_through_their_claim(ops, in_size):
+    """grape_sumcheck_round2_claim over four rounds in a row against grape_sumcheck_round2: the same
+    three sums and folded tensors in every round (the middle coefficient comes from the claim), and the
+    claim it leaves is the round polynomial's value at the challenge; sizes on both sides of the
+    table-fold threshold, ragged included"""
+    A, B = rand_fr(in_size, 401), rand_fr(in_size, 402)
+    v = rand_fr(4, 403)
+    dA, dB = ops.to_dev(A), ops.to_dev(B)
+    cA, cB = ops.to_dev(A), ops.to_dev(B)
+    Ai, Bi = br.fr_unpack(A), br.fr_unpack(B)
+    claim = sum(x * y for x, y in zip(Ai, Bi)) % R
+    d_claim = ops.to_dev(br.fr_pack([claim]))
+    n_in = in_size
+    n_out = 1 << (br.log2ceil(in_size) - 1)
+    for k in range(4):
+        dv = ops.to_dev(v[k:k + 1])
+        want = ops.fr_to_host(ops.sumcheck_round2(dA, dB, n_in, n_out, dv))
+        got = ops.fr_to_host(ops.sumcheck_round2_claim(cA, cB, n_in, n_out, dv, d_claim))
+        assert_same(got, want, "sums of round %d" % k)
+        assert_same(ops.fr_to_host(cA)[:n_out], ops.fr_to_host(dA)[:n_out], "folded A, round %d" % k)
+        assert_same(ops.fr_to_host(cB)[:n_out], ops.fr_to_host(dB)[:n_out], "folded B, round %d" % k)
+        c0, c1, c2 = br.fr_unpack(want)
+        vk = br.fr_unpack(v[k:k + 1])[0]
+        assert (2 * c0 + c1 + c2) % R == claim
+        claim = (c0 + c1 * vk + c2 * vk * vk) % R
+        assert br.fr_unpack(ops.fr_to_host(d_claim)) == [claim]
+        n_in, n_out = n_out, n_out // 2
