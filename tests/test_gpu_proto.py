@@ -28,7 +28,9 @@ def _oracle_round2(A, B, in_size, out_size, v):
     return A, B, a, b, c
 
 
-@pytest.mark.parametrize("in_size,out_size", [(2, 1), (8, 4), (6, 4), (5, 4), (4096, 2048), (3000, 2048), (1 << 17, 1 << 16), (100000, 65536)])
+@pytest.mark.parametrize("in_size,out_size", [(2, 1), (8, 4), (6, 4), (5, 4), (4096, 2048), (3000, 2048), (1 << 17, 1 << 16), (100000, 65536),
+                                              # long rounds: several indices per thread, upper halves that end inside a workgroup's range
+                                              (1 << 22, 1 << 21), (3000001, 1 << 21), ((1 << 22) - 700, (1 << 21) - 300)])
 def test_sumcheck_round2(ops, in_size, out_size):
     A, B = rand_fr(in_size, 1 + in_size), rand_fr(in_size, 2 + in_size)
     v = rand_fr(1, 3)
@@ -373,7 +375,7 @@ def test_weighted_sums_of_one_tensor_against_several_tables(ops):
             assert_same(got[2 * j + 1], orc.mle_eval(d, us[j]), "claim %d, X1 - X0" % j)
 
 
-@pytest.mark.parametrize("in_size", [1 << 18, (1 << 18) - 3000, 5000])
+@pytest.mark.parametrize("in_size", [1 << 18, (1 << 18) - 3000, 5000, (1 << 22) - 12345])
 def test_sumcheck_rounds_chained_through_their_claim(ops, in_size):
     """grape_sumcheck_round2_claim over four rounds in a row against grape_sumcheck_round2: the same
     three sums and folded tensors in every round (the middle coefficient comes from the claim), and the
