@@ -451,6 +451,29 @@ def commit_i32(scalars, rowlen, table, N, c, nw, K, out=None):
     return out
 
 
+def stream_create():
+    """a stream of the library's own (default priority, its own scratch memory); returns the handle"""
+    h = ctypes.c_void_p()
+    _capi.check(init().grape_stream_create(ctypes.byref(h)))
+    return h
+
+
+def stream_destroy(h):
+    _capi.check(init().grape_stream_destroy(h))
+
+
+def stream_sync(h):
+    _capi.check(init().grape_stream_sync(h))
+
+
+def commit_i32_nowait(scalars, rowlen, table, N, c, nw, K, out, flag, stream):
+    """queues the commitment on `stream` (a handle from stream_create) and returns; `flag` is a device
+    int32 the caller has cleared, set when a scalar does not fit the table's digits"""
+    lib = init()
+    _capi.check(lib.grape_commit_i32_nowait(_p(out), _p(scalars), scalars.numel(), rowlen, _p(table), N, c, nw, K, _p(flag), stream))
+    return out
+
+
 def commit_fr(scalars, rowlen, table, N, c, nw, K, out=None):
     lib = init()
     size = scalars.shape[0]
