@@ -93,6 +93,44 @@ def test_commit_i32_small_vs_oracle_and_bigint(ops, gens64):
     assert got[0] is None and got[1] == br.g1_neg(br.g1_unpack(host[3:4])[0])
 
 
+def test_commitments_queued_on_three_streams(ops, gens64):
+    """grape_commit_i32_nowait on three streams of the library in turn (each stream with its own scratch,
+    output and digit-range flag): nine commitments of different matrices against the oracle, and a
+    flag that is raised by the one commitment whose scalars do not fit"""
+    import torch
+    k, host, dev = gens64
+    n, rows = 32, 300
+    wide = ops.g1_wide_table_gen(dev[:n].contiguous(), 16, 1, 32768)
+    tab = orc.g1_table(host[:n], 256)
+    mats = [gaussian_i16((rows, n), 60 + i) for i in range(9)]
+    dmats = [torch.from_numpy(m).cuda() for m in mats]
+    streams = [ops.stream_create() for _ in range(3)]
+    outs = [ops.g1_empty(rows) for _ in range(9)]
+    flags = torch.zeros(9, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    try:
+        for i in range(9):
+            ops.commit_i32_nowait(dmats[i], n, wide, n, 16, 1, 32768, outs[i], flags[i:i + 1], streams[i % 3])
+        for h in streams:
+            ops.stream_sync(h)
+        assert flags.tolist() == [0] * 9
+        for i in range(9):
+            assert_same(ops.g1_to_host(outs[i]), orc.commit_i32(mats[i], tab, n, n), "queued commitment %d" % i)
+        bad = mats[4].copy()
+        bad[7, 5] = 40000
+        dbad = torch.from_numpy(bad).cuda()
+        flags.zero_()
+        torch.cuda.synchronize()
+        for i in range(3):
+            ops.commit_i32_nowait(dbad if i == 1 else dmats[i], n, wide, n, 16, 1, 32768, outs[i], flags[i:i + 1], streams[i])
+        for h in streams:
+            ops.stream_sync(h)
+        assert flags.tolist()[:3] == [0, 1, 0]
+    finally:
+        for h in streams:
+            ops.stream_destroy(h)
+
+
 def test_commit_int16_fast_path(ops, gens64):
     import torch
     k, host, dev = gens64
