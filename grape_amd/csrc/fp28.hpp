@@ -720,4 +720,60 @@ GRAPE_HD G1Affine xyzz28_to_affine(const Xyzz28& a) {
     return r;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Affine + affine with the inversion supplied by the caller (Montgomery's trick over many
+// independent additions: table generation).  Inputs are finite points with canonical coordinates.
+// ------------------------------------------------------------------------------------------------
+// a normalised value in [0, 2^k p) -> the representative in [0, p)
+template <int K>
+GRAPE_HD Fp28 fp28_below_p(Fp28 t) {
+#pragma unroll
+    for (int s = K - 1; s >= 0; s--) {
+        Fp28 d;
+#pragma unroll
+        for (int i = 0; i < fp28::N; i++) d.v[i] = t.v[i] - fp28::P(i) * (1 << s);
+        d = fp28::normalize(d);
+        const bool ok = d.v[fp28::N - 1] >= 0;
+#pragma unroll
+        for (int i = 0; i < fp28::N; i++) t.v[i] = ok ? d.v[i] : t.v[i];
+    }
+    return t;
+}
+// denominator of the slope of e + f (x_e - x_f), or of 2 f (2 y_f) when `dbl`; a value congruent
+// to zero means that the sum is no finite affine addition (e = +-f, or a point of order two)
+GRAPE_HD Fp28 affine28_slope_den(const Affine28& e, const Affine28& f, bool dbl) {
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < fp28::N; i++) r.v[i] = dbl ? 2 * f.y.v[i] : e.x.v[i] - f.x.v[i];
+    return r;
+}
+// e + f (2 f when `dbl`; then e must equal f) given dinv = 1 / affine28_slope_den(e, f, dbl), a
+// product output in (0, 3p): 3M + 1S (one more S for the doubling), coordinates canonical
+GRAPE_HD Affine28 affine28_add_given_inverse(const Affine28& e, const Affine28& f, bool dbl, const Fp28& dinv) {
+    using namespace fp28;
+    Fp28 num;
+    if (dbl) {
+        const Fp28 xx = sqr(f.x);                       // (0, 3p)
+#pragma unroll
+        for (int i = 0; i < N; i++) num.v[i] = 3 * xx.v[i];
+        num = normalize(num);                           // (0, 9p)
+    } else {
+        num = sub(e.y, f.y);                            // (-p, p)
+    }
+    const Fp28 lam = mul(num, dinv);                    // 9 * 3 = 27 <= 2^11
+    const Fp28 ll = sqr(lam);                           // (0, 3p)
+    Fp28 x3;
+#pragma unroll
+    for (int i = 0; i < N; i++) x3.v[i] = ll.v[i] - e.x.v[i] - f.x.v[i] + P2(i);   // (0, 5p)
+    x3 = fp28_below_p<3>(normalize(x3));
+    const Fp28 ly = mul(lam, sub(e.x, x3));             // 3 * 1
+    Fp28 y3;
+#pragma unroll
+    for (int i = 0; i < N; i++) y3.v[i] = ly.v[i] - e.y.v[i] + P(i);               // (0, 4p)
+    Affine28 r;
+    r.x = x3;
+    r.y = fp28_below_p<2>(normalize(y3));
+    return r;
+}
+
 }  // namespace grape

@@ -397,6 +397,112 @@ __global__ void __launch_bounds__(64) wide_normalize_kernel(uint32_t* table, con
 }
 
 // ------------------------------------------------------------------------------------------------
+// Table generation by levels: once the multiples 1..have of every base are in the table, the next
+// cnt <= have are E[have + k] = E[k] + E[have] (k = have is the doubling of E[have]) - additions
+// of two AFFINE entries that are already final, all independent.  An affine addition is 3M + 1S
+// once the inverse of its slope's denominator is known, and Montgomery's trick shares one
+// inversion over a thread's run of consecutive k: a forward pass multiplies the denominators up,
+// parking every prefix product in the destination entry it belongs to (free until the backward
+// pass fills it), one divstep inversion, and a backward pass that peels the inverses off and
+// writes the sums.  About 6 products and 0.5 KB of traffic per entry, where a chain of mixed
+// XYZZ additions plus the normalisation of every entry costs 17 products and an inversion per 8.
+// A run whose denominators multiply to zero (a base that is the identity or has small order: no
+// generator of the prime-order group) raises *degenerate and leaves its entries to
+// wide_extend_exact_kernel.
+// ------------------------------------------------------------------------------------------------
+constexpr uint32_t kExtendRun = 64;   // additions that share one inversion
+constexpr int kFp28Quads = (L28 + 3) / 4;
+__device__ __forceinline__ Fp28 ld_fp28(const uint32_t* p) {
+    const uint4* q = reinterpret_cast<const uint4*>(p);
+    uint4 w[kFp28Quads];
+#pragma unroll
+    for (int i = 0; i < kFp28Quads; i++) w[i] = q[i];
+    const uint32_t* f = reinterpret_cast<const uint32_t*>(w);
+    Fp28 r;
+#pragma unroll
+    for (int i = 0; i < L28; i++) r.v[i] = (int32_t)f[i];
+    return r;
+}
+__device__ __forceinline__ void st_fp28(uint32_t* p, const Fp28& a) {
+    uint32_t f[4 * kFp28Quads];
+#pragma unroll
+    for (int i = 0; i < 4 * kFp28Quads; i++) f[i] = i < L28 ? (uint32_t)a.v[i] : 0u;
+    uint4* q = reinterpret_cast<uint4*>(p);
+#pragma unroll
+    for (int i = 0; i < kFp28Quads; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+}
+static_assert(4 * kFp28Quads <= kWideEntryWords, "a prefix product must fit the entry it is parked in");
+__device__ __forceinline__ void st_entry28_raw(uint32_t* table, size_t e, const Affine28& a) {
+    uint32_t f[kWideEntryWords];
+#pragma unroll
+    for (int i = 0; i < L28; i++) {
+        f[i] = (uint32_t)a.x.v[i];
+        f[L28 + i] = (uint32_t)a.y.v[i];
+    }
+#pragma unroll
+    for (int i = 2 * L28; i < kWideEntryWords; i++) f[i] = 0;
+    uint4* q = reinterpret_cast<uint4*>(table + (size_t)kWideEntryWords * e);
+#pragma unroll
+    for (int i = 0; i < kWideEntryWords / 4; i++) q[i] = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+}
+
+// One thread per (run of `run` consecutive k, window w, generator i); i is the fastest index, so a
+// wave reads and writes adjacent entries.
+__global__ void __launch_bounds__(kBlock) wide_extend_kernel(uint32_t* table, size_t N, uint32_t nw, uint32_t K, uint32_t have,
+                                                             uint32_t cnt, uint32_t run, int* degenerate) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t per = (size_t)nw * N;
+    const uint32_t nruns = (cnt + run - 1) / run;
+    if (t >= per * nruns) return;
+    const uint32_t r = (uint32_t)(t / per);
+    const size_t wi = t - (size_t)r * per;
+    const size_t w = wi / N, i = wi - w * N;
+    const uint32_t k0 = r * run + 1;                              // first k of the run
+    const uint32_t k1 = k0 + run < cnt + 1 ? k0 + run : cnt + 1;  // one past its last
+    const size_t e0 = w * K * N + i;                              // entry of the multiple k: e0 + (k-1) N
+    const Affine28 f = ld_entry28(table, e0 + (size_t)(have - 1) * N);
+    bool bad = entry_is_inf(f);
+    Fp28 acc = fp28::one();
+    for (uint32_t k = k0; k < k1; k++) {
+        const Affine28 e = ld_entry28(table, e0 + (size_t)(k - 1) * N);
+        bad |= entry_is_inf(e);
+        st_fp28(table + (size_t)kWideEntryWords * (e0 + (size_t)(have + k - 1) * N), acc);
+        acc = fp28::mul(acc, affine28_slope_den(e, f, k == have));
+    }
+    bad |= fp28::is_zero_mod_p(acc);
+    if (bad) {
+        *degenerate = 1;
+        return;
+    }
+    Fp28 inv = fp28::inverse_by(acc);
+    for (uint32_t k = k1 - 1; k >= k0; k--) {
+        const size_t dst = e0 + (size_t)(have + k - 1) * N;
+        const Affine28 e = ld_entry28(table, e0 + (size_t)(k - 1) * N);
+        const Fp28 dinv = fp28::mul(inv, ld_fp28(table + (size_t)kWideEntryWords * dst));
+        inv = fp28::mul(inv, affine28_slope_den(e, f, k == have));
+        st_entry28_raw(table, dst, affine28_add_given_inverse(e, f, k == have, dinv));
+    }
+}
+
+// The same level through the general addition, one thread per entry, every exceptional case
+// handled (identity, equal and opposite points): runs only when the level met a degenerate run.
+__global__ void __launch_bounds__(64) wide_extend_exact_kernel(uint32_t* table, size_t N, uint32_t nw, uint32_t K, uint32_t have,
+                                                               uint32_t cnt, const int* degenerate) {
+    if (*degenerate == 0) return;
+    const size_t per = (size_t)nw * N;
+    for (size_t t = (size_t)blockIdx.x * 64 + threadIdx.x; t < per * cnt; t += (size_t)gridDim.x * 64) {
+        const uint32_t k = (uint32_t)(t / per) + 1;
+        const size_t wi = t - (size_t)(k - 1) * per;
+        const size_t w = wi / N, i = wi - w * N;
+        const size_t e0 = w * K * N + i;
+        Xyzz28 acc = xyzz28_inf();
+        madd28(acc, ld_entry28(table, e0 + (size_t)(k - 1) * N), false);
+        madd28(acc, ld_entry28(table, e0 + (size_t)(have - 1) * N), false);
+        st_entry28(table, e0 + (size_t)(have + k - 1) * N, xyzz28_to_affine(acc));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // commitment, wide table
 // ------------------------------------------------------------------------------------------------
 // Each wave owns one row segment of `seg` columns; lane l takes columns l, l+64, ...
@@ -954,33 +1060,39 @@ size_t grape_g1_wide_table_bytes(size_t N, uint32_t nw, uint32_t K) { return (si
 static int wide_table_gen_impl(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     hipStream_t s = as_stream(st);
     const size_t per_chunk = (size_t)nw * N;
-    // chunk length: long enough to amortise the start-up scalar multiplication, short enough
-    // to expose nw*N*(K/CH) threads
+    // the first CH multiples of every base as a chain of mixed additions, normalised together;
+    // everything above them level by level from the entries below (wide_extend_kernel)
     uint32_t CH = 64;
     if (K < CH) CH = K;
-    const uint32_t nchunks = (K + CH - 1) / CH;
-    // slab the chunk index so that the XYZZ staging buffer stays below ~1.5 GiB
-    size_t slab_chunks = ((size_t)3 << 29) / (per_chunk * CH * (16 * FW));
-    if (slab_chunks < 1) slab_chunks = 1;
-    if (slab_chunks > nchunks) slab_chunks = nchunks;
     void* ws;
     const size_t bases_bytes = per_chunk * (8 * FW);
-    const size_t tmp_bytes = slab_chunks * CH * per_chunk * (16 * FW);
-    int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes, &ws, s);
+    const size_t tmp_bytes = (size_t)CH * per_chunk * (16 * FW);
+    int rc = scratch_get(kSlotMsm, bases_bytes + tmp_bytes + 256, &ws, s);
     if (rc) return rc;
     uint32_t* bases = (uint32_t*)ws;
     uint32_t* tmp = (uint32_t*)((char*)ws + bases_bytes);
+    int* degenerate = (int*)((char*)ws + bases_bytes + tmp_bytes);
+    rc = zero_fill(degenerate, sizeof(int), s);
+    if (rc) return rc;
     window_bases_kernel<<<blocks_for(N, 64), 64, 0, s>>>(bases, gens, N, c, nw);
     GRAPE_LAUNCH_CHECK();
-    for (uint32_t j0 = 0; j0 < nchunks; j0 += (uint32_t)slab_chunks) {
-        uint32_t nj = nchunks - j0 < slab_chunks ? nchunks - j0 : (uint32_t)slab_chunks;
-        size_t nthreads = per_chunk * nj;
-        wide_chain_kernel<<<blocks_for(nthreads, 64), 64, 0, s>>>(tmp, bases, N, nw, K, CH, j0, nj);
-        size_t k_hi = (size_t)(j0 + nj) * CH < K ? (size_t)(j0 + nj) * CH : K;
-        size_t n_entries = (k_hi - (size_t)j0 * CH) * per_chunk;
-        size_t nthr2 = (n_entries + kNormChunk - 1) / kNormChunk;
-        wide_normalize_kernel<<<blocks_for(nthr2, 64), 64, 0, s>>>(table, tmp, N, nw, K, CH, j0, n_entries);
+    {
+        wide_chain_kernel<<<blocks_for(per_chunk, 64), 64, 0, s>>>(tmp, bases, N, nw, K, CH, 0, 1);
+        const size_t n_entries = (size_t)CH * per_chunk;
+        const size_t nthr2 = (n_entries + kNormChunk - 1) / kNormChunk;
+        wide_normalize_kernel<<<blocks_for(nthr2, 64), 64, 0, s>>>(table, tmp, N, nw, K, CH, 0, n_entries);
         GRAPE_LAUNCH_CHECK();
+    }
+    for (uint32_t have = CH; have < K;) {
+        const uint32_t cnt = K - have < have ? K - have : have;
+        const uint32_t run = cnt < kExtendRun ? cnt : kExtendRun;
+        const size_t nthreads = per_chunk * ((cnt + run - 1) / run);
+        const size_t exact_want = (per_chunk * cnt + 63) / 64;
+        const unsigned exact_blocks = (unsigned)(exact_want < 16384 ? exact_want : 16384);   // a no-op unless the flag is up
+        wide_extend_kernel<<<blocks_for(nthreads), kBlock, 0, s>>>(table, N, nw, K, have, cnt, run, degenerate);
+        wide_extend_exact_kernel<<<exact_blocks, 64, 0, s>>>(table, N, nw, K, have, cnt, degenerate);
+        GRAPE_LAUNCH_CHECK();
+        have += cnt;
     }
     return GRAPE_OK;
 }

@@ -1,6 +1,7 @@
 // Host build of the 28-bit-limb Fp arithmetic (grape_amd/csrc/fp28.hpp) behind a few C entry
 // points, so that the CPU test-suite can check it against Python integers and the oracle.
 #include <cstring>
+#include <vector>
 #include "../../grape_amd/csrc/fp28.hpp"
 using namespace grape;
 static constexpr int FW = FpParams::N;     // 32-bit words of an Fp element in memory
@@ -145,5 +146,46 @@ void t28_horner(const uint32_t* points, int n, int dbl, uint32_t* out_affine) {
     }
     G1Affine r = xyzz28_to_affine(acc);
     memcpy(out_affine, &r, 2 * FB);
+}
+// The table generator's step: out[k] = pts[k] + base for k < n (pts[k] == base is the doubling), as
+// affine additions that share ONE inversion - forward pass of prefix products of the slope
+// denominators, one inversion, backward pass.  Canonical affine points in and out (2 FW x u32).
+// Returns 1 when the product of the denominators is congruent to zero (no finite affine addition
+// for some k; nothing is written then).
+int t28_affine_batch(const uint32_t* pts, const int* dbl, int n, const uint32_t* base, uint32_t* out) {
+    auto load = [](const uint32_t* src) {
+        G1Affine p;
+        memcpy(&p, src, 2 * FB);
+        Affine28 q;
+        q.x = fp28::from_canonical(p.x);
+        q.y = fp28::from_canonical(p.y);
+        return q;
+    };
+    const Affine28 f = load(base);
+    std::vector<Fp28> pre(n);
+    Fp28 acc = fp28::one();
+    for (int k = 0; k < n; k++) {
+        pre[k] = acc;
+        acc = fp28::mul(acc, affine28_slope_den(load(pts + 2 * FW * k), f, dbl[k] != 0));
+    }
+    if (fp28::is_zero_mod_p(acc)) return 1;
+    Fp28 inv = fp28::inverse_by(acc);
+    for (int k = n - 1; k >= 0; k--) {
+        const Affine28 e = load(pts + 2 * FW * k);
+        const Fp28 dinv = fp28::mul(inv, pre[k]);
+        inv = fp28::mul(inv, affine28_slope_den(e, f, dbl[k] != 0));
+        const Affine28 r = affine28_add_given_inverse(e, f, dbl[k] != 0, dinv);
+        // the entry format wants canonical coordinates: check that here, limb by limb
+        for (int i = 0; i < fp28::N - 1; i++)
+            if (r.x.v[i] < 0 || r.x.v[i] > (int32_t)fp28::MASK || r.y.v[i] < 0 || r.y.v[i] > (int32_t)fp28::MASK) return 2;
+        Fp28 dx = fp28::normalize(fp28::sub(r.x, [] { Fp28 p; for (int i = 0; i < fp28::N; i++) p.v[i] = fp28::P(i); return p; }()));
+        Fp28 dy = fp28::normalize(fp28::sub(r.y, [] { Fp28 p; for (int i = 0; i < fp28::N; i++) p.v[i] = fp28::P(i); return p; }()));
+        if (dx.v[fp28::N - 1] >= 0 || dy.v[fp28::N - 1] >= 0 || r.x.v[fp28::N - 1] < 0 || r.y.v[fp28::N - 1] < 0) return 3;
+        G1Affine o;
+        o.x = fp28::to_canonical(r.x);
+        o.y = fp28::to_canonical(r.y);
+        memcpy(out + 2 * FW * k, &o, 2 * FB);
+    }
+    return 0;
 }
 }

@@ -185,3 +185,41 @@ def test_doubling_chain_horner(lib):
             want = br.g1_mul(1 << d, want) if want is not None else None
             want = br.g1_add(want, p)
         assert got == want, (n, d)
+
+
+def _affine_batch(lib, pts, dbl, base):
+    arr = np.ascontiguousarray(br.g1_pack(pts).view(np.uint32).reshape(len(pts), 2 * FW))
+    b = np.ascontiguousarray(br.g1_pack([base]).view(np.uint32).reshape(2 * FW))
+    flags = np.array(dbl, dtype=np.int32)
+    out = np.zeros((len(pts), 2 * FW), dtype=np.uint32)
+    rc = lib.t28_affine_batch(_u32(arr), flags.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), len(pts), _u32(b), _u32(out))
+    return rc, br.g1_unpack(out.view(np.uint64).reshape(len(pts), br.G1_WORDS))
+
+
+def test_affine_additions_sharing_one_inversion(lib):
+    """The table generator's level step - multiples k*B + h*B for a run of k, the doubling h*B + h*B
+    among them - as affine additions behind one shared inversion, against the textbook group law;
+    coordinates come out canonical (checked inside the host twin: codes 2 and 3); a run that holds
+    a pair without a finite affine sum (equal points not flagged as a doubling, opposite points) is
+    reported instead of computed"""
+    rng = random.Random(8)
+    B = br.g1_mul(rng.randrange(1, br.R_MOD), br.G1)
+    h = 64
+    base = br.g1_mul(h, B)
+    ks = list(range(1, 41)) + [h]
+    pts = [br.g1_mul(k, B) for k in ks]
+    rc, got = _affine_batch(lib, pts, [k == h for k in ks], base)
+    assert rc == 0
+    assert got == [br.g1_mul(k + h, B) for k in ks]
+    # one element, and the doubling alone
+    rc, got = _affine_batch(lib, pts[:1], [False], base)
+    assert rc == 0 and got == [br.g1_mul(1 + h, B)]
+    rc, got = _affine_batch(lib, [base], [True], base)
+    assert rc == 0 and got == [br.g1_mul(2 * h, B)]
+    # random pairs of unrelated points
+    qs = _points([rng.randrange(1, br.R_MOD) for _ in range(12)])
+    rc, got = _affine_batch(lib, qs, [False] * len(qs), base)
+    assert rc == 0 and got == [br.g1_add(q, base) for q in qs]
+    # no finite affine sum: the same point without the doubling flag, and the opposite point
+    assert _affine_batch(lib, pts[:3] + [base], [False] * 4, base)[0] == 1
+    assert _affine_batch(lib, [br.g1_neg(base)] + pts[:3], [False] * 4, base)[0] == 1

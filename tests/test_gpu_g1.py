@@ -65,6 +65,43 @@ def test_wide_table_entries(ops, gens64):
         assert pt == br.g1_mul(kk << (c * w), pts[i])
 
 
+def _table_case(ops, pts, c, nw, K, ks):
+    import torch
+    n = len(pts)
+    dev = torch.from_numpy(br.g1_pack(pts)).cuda()
+    table = ops.g1_wide_table_gen(dev, c, nw, K)
+    cases = [(w, kk, i) for w in range(nw) for kk in ks for i in range(n)]
+    idx = [(w * K + (kk - 1)) * n + i for (w, kk, i) in cases]
+    got = ops.wide_table_entries_to_host(table, idx)
+    for (w, kk, i), pt in zip(cases, got):
+        assert pt == br.g1_mul(kk << (c * w), pts[i]), (c, nw, K, w, kk, i)
+
+
+def test_wide_table_levels(ops, gens64):
+    """entries above the first 64 multiples come from the level step (E[h + k] = E[k] + E[h], affine
+    additions behind shared inversions): every level's first and last entry, the doubling
+    E[2h] and entries inside runs, for power-of-two and ragged K, against Python integers"""
+    k, host, dev = gens64
+    pts = br.g1_unpack(host[:5])
+    _table_case(ops, pts, 9, 2, 256, [1, 2, 63, 64, 65, 66, 100, 127, 128, 129, 191, 192, 193, 255, 256])
+    _table_case(ops, pts, 9, 2, 200, [64, 65, 128, 129, 130, 192, 193, 199, 200])
+    _table_case(ops, pts[:2], 12, 1, 2048, [64, 65, 1024, 1025, 1088, 1089, 1537, 2047, 2048])
+    _table_case(ops, pts[:3], 6, 3, 32, [1, 31, 32])          # below the first chain's length: no level at all
+
+
+def test_wide_table_with_degenerate_bases(ops, gens64):
+    """a generator set that holds the identity (and, where the curve has one, a point of order three):
+    their multiples repeat or vanish, no affine sum exists for some of them, and the level step
+    hands such levels to the general addition - all entries still equal the multiples"""
+    k, host, dev = gens64
+    pts = br.g1_unpack(host[:3])
+    pts.insert(1, None)
+    if br.CURVE != "bn254":
+        assert br.g1_on_curve((0, 2)) and br.g1_mul(3, (0, 2)) is None
+        pts.append((0, 2))
+    _table_case(ops, pts, 8, 2, 256, [1, 2, 3, 64, 65, 66, 128, 129, 130, 131, 255, 256])
+
+
 def test_commit_i32_small_vs_oracle_and_bigint(ops, gens64):
     import torch
     k, host, dev = gens64
