@@ -52,7 +52,7 @@ static inline unsigned blocks_for(size_t n, int per_block = kBlock) {
 // Scratch pool: one growing device allocation per (stream, slot), reused across calls so the hot
 // path never allocates once warm.  Slots are independent buffers (a call may use several at once);
 // the buffer belongs to `stream`: only kernels launched on that stream may touch it.
-enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kSlotWitA = 8, kSlotWitB = 9, kNumSlots = 10 };
+enum ScratchSlot { kSlotReduce = 0, kSlotFold = 1, kSlotInv = 2, kSlotMsm = 3, kSlotMisc = 4, kSlotFoldW = 5, kSlotHistIdx = 6, kSlotHistPart = 7, kSlotWitA = 8, kSlotWitB = 9, kSlotTable = 10, kNumSlots = 11 };
 int scratch_get(ScratchSlot slot, size_t bytes, void** out, hipStream_t stream);
 // Zeroes device memory with a small fill kernel (word-sized regions) so that a caller who captures
 // the stream into a graph records a kernel node, not a memset node.

@@ -308,18 +308,6 @@ __global__ void __launch_bounds__(64) scalar_mul_base_kernel(uint32_t* out, cons
     st_affine(out, i, to_affine(scalar_mul(p, kk, 255)));
 }
 
-// reference-format table: out[w*N + i] = w*G_i (naive_msm)
-__global__ void __launch_bounds__(64) ref_table_kernel(uint32_t* out, const uint32_t* gens, size_t N, uint32_t W) {
-    size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
-    if (i >= N) return;
-    G1Affine g = ld_affine(gens, i);
-    G1Xyzz res = G1Xyzz::inf();
-    for (uint32_t w = 0; w < W; w++) {
-        st_affine(out, (size_t)w * N + i, to_affine(res));
-        madd(res, g, false);
-    }
-}
-
 // bases[w*N + i] = 2^(c*w) * G_i, affine
 __global__ void __launch_bounds__(64) window_bases_kernel(uint32_t* bases, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw) {
     size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
@@ -411,6 +399,7 @@ __global__ void __launch_bounds__(64) wide_normalize_kernel(uint32_t* table, con
 // wide_extend_exact_kernel.
 // ------------------------------------------------------------------------------------------------
 constexpr uint32_t kExtendRun = 64;   // additions that share one inversion
+constexpr uint32_t kFirstChain = 16;  // multiples of a base made by the chain of mixed additions before the levels start
 constexpr int kFp28Quads = (L28 + 3) / 4;
 __device__ __forceinline__ Fp28 ld_fp28(const uint32_t* p) {
     const uint4* q = reinterpret_cast<const uint4*>(p);
@@ -500,6 +489,22 @@ __global__ void __launch_bounds__(64) wide_extend_exact_kernel(uint32_t* table, 
         madd28(acc, ld_entry28(table, e0 + (size_t)(have - 1) * N), false);
         st_entry28(table, e0 + (size_t)(have + k - 1) * N, xyzz28_to_affine(acc));
     }
+}
+
+// Reference-format table from a one-window wide table over the generators i0 .. i0+ns:
+// out[w*N + i0 + i] = w * G_(i0+i) in the canonical memory form (w = 0: the identity), one product
+// per coordinate to change the limb form and the Montgomery radix.
+__global__ void __launch_bounds__(kBlock) ref_from_wide_kernel(uint32_t* out, const uint32_t* wide, size_t N, size_t i0, size_t ns, uint32_t W) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= ns * W) return;
+    const size_t w = t / ns, i = t - w * ns;
+    G1Affine a = G1Affine::inf();
+    if (w > 0) {
+        const Affine28 e = ld_entry28(wide, (w - 1) * ns + i);
+        a.x = fp28::to_canonical(e.x);
+        a.y = fp28::to_canonical(e.y);
+    }
+    st_affine(out, w * N + i0 + i, a);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1046,11 +1051,32 @@ int grape_g1_scalar_mul_base(uint32_t* out, const uint32_t* k, const uint32_t* b
     return GRAPE_OK;
 }
 
+static int wide_table_gen_impl(uint32_t* table, const uint32_t* gens, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st);
+
+// The multiples come from the level-wise generator of the wide tables (one window, K = W - 1), a
+// slab of generators at a time through a staging table of at most 1 GiB, and are then rewritten in
+// the reference's layout and limb form.
 int grape_g1_table_gen(uint32_t* table, const uint32_t* gens, size_t N, uint32_t W, grape_stream_t st) {
     if (N == 0 || W == 0) return GRAPE_OK;
     CHECK_PTR16(table); CHECK_PTR16(gens);
-    ref_table_kernel<<<blocks_for(N, 64), 64, 0, as_stream(st)>>>(table, gens, N, W);
-    GRAPE_LAUNCH_CHECK();
+    GRAPE_REQUIRE(W <= (1u << 16), "bad table shape");
+    hipStream_t s = as_stream(st);
+    const uint32_t K = W > 1 ? W - 1 : 1;
+    size_t slab = ((size_t)1 << 30) / ((size_t)K * 4 * kWideEntryWords);
+    if (slab < 64) slab = 64;
+    if (slab > N) slab = N;
+    void* stage;
+    int rc = scratch_get(kSlotTable, slab * K * 4 * kWideEntryWords, &stage, s);
+    if (rc) return rc;
+    for (size_t i0 = 0; i0 < N; i0 += slab) {
+        const size_t ns = N - i0 < slab ? N - i0 : slab;
+        if (W > 1) {
+            rc = wide_table_gen_impl((uint32_t*)stage, gens + i0 * (size_t)(2 * FW), ns, 1, 1, K, st);
+            if (rc) return rc;
+        }
+        ref_from_wide_kernel<<<blocks_for(ns * W), kBlock, 0, s>>>(table, (const uint32_t*)stage, N, i0, ns, W);
+        GRAPE_LAUNCH_CHECK();
+    }
     return GRAPE_OK;
 }
 
@@ -1062,7 +1088,7 @@ static int wide_table_gen_impl(uint32_t* table, const uint32_t* gens, size_t N, 
     const size_t per_chunk = (size_t)nw * N;
     // the first CH multiples of every base as a chain of mixed additions, normalised together;
     // everything above them level by level from the entries below (wide_extend_kernel)
-    uint32_t CH = 64;
+    uint32_t CH = kFirstChain;
     if (K < CH) CH = K;
     void* ws;
     const size_t bases_bytes = per_chunk * (8 * FW);

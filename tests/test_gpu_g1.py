@@ -78,15 +78,16 @@ def _table_case(ops, pts, c, nw, K, ks):
 
 
 def test_wide_table_levels(ops, gens64):
-    """entries above the first 64 multiples come from the level step (E[h + k] = E[k] + E[h], affine
+    """entries above the first 16 multiples come from the level step (E[h + k] = E[k] + E[h], affine
     additions behind shared inversions): every level's first and last entry, the doubling
     E[2h] and entries inside runs, for power-of-two and ragged K, against Python integers"""
     k, host, dev = gens64
     pts = br.g1_unpack(host[:5])
-    _table_case(ops, pts, 9, 2, 256, [1, 2, 63, 64, 65, 66, 100, 127, 128, 129, 191, 192, 193, 255, 256])
+    _table_case(ops, pts, 9, 2, 256, [1, 2, 15, 16, 17, 18, 31, 32, 33, 63, 64, 65, 66, 100, 127, 128, 129, 191, 192, 193, 255, 256])
     _table_case(ops, pts, 9, 2, 200, [64, 65, 128, 129, 130, 192, 193, 199, 200])
     _table_case(ops, pts[:2], 12, 1, 2048, [64, 65, 1024, 1025, 1088, 1089, 1537, 2047, 2048])
-    _table_case(ops, pts[:3], 6, 3, 32, [1, 31, 32])          # below the first chain's length: no level at all
+    _table_case(ops, pts[:3], 6, 3, 32, [1, 16, 17, 31, 32])
+    _table_case(ops, pts[:3], 4, 3, 8, [1, 7, 8])              # below the first chain's length: no level at all
 
 
 def test_wide_table_with_degenerate_bases(ops, gens64):
@@ -99,7 +100,7 @@ def test_wide_table_with_degenerate_bases(ops, gens64):
     if br.CURVE != "bn254":
         assert br.g1_on_curve((0, 2)) and br.g1_mul(3, (0, 2)) is None
         pts.append((0, 2))
-    _table_case(ops, pts, 8, 2, 256, [1, 2, 3, 64, 65, 66, 128, 129, 130, 131, 255, 256])
+    _table_case(ops, pts, 8, 2, 256, [1, 2, 3, 16, 17, 18, 19, 32, 33, 64, 65, 66, 128, 129, 130, 131, 255, 256])
 
 
 def test_commit_i32_small_vs_oracle_and_bigint(ops, gens64):
