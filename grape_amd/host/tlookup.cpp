@@ -137,6 +137,9 @@ bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& h
 }
 
 namespace {
+// A witness round over at least this many index pairs runs before the commitments of its proof, a
+// shorter one (launch-bound) beside them.
+constexpr uint kLongRoundPairs = 1u << 16;
 // A stream beside the default one (two per process, created on first use) and the two events that order it against
 // the default stream: begin() makes it wait for what the default stream has queued, end() makes the
 // default stream wait for it.  If the scope is left by an exception the destructor waits for the
@@ -331,16 +334,35 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         // small kernels per round on the table side, two on the witness side).
         SideChain side(0), witness(1);
         side.begin();                       // the second stream waits for everything queued so far
-        grape_stream_t ws = nullptr;        // where the witness side runs: the default stream, or one of its own beside the commitments
+        grape_stream_t ws = nullptr;        // where the short witness rounds run: the default stream, or one of its own beside the commitments
+        uint cur = D;
+        uint k = 0;
+        int vi = (int)rounds - 1;
+        // A and S: five sums and the fold of both tensors in one pass
+        auto witness_round = [&](grape_stream_t st) {
+            const uint half = cur / 2;
+            fr_t* slot = sums.gpu_data + 13 * (size_t)k;
+            const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
+            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), st), "grape_wround2");
+            A.set_size(half);
+            S.set_size(half);
+            cur = half;
+            vi--;
+            k++;
+        };
+        // overlap: the commitments are queued without waiting (their digit-range flags are read after
+        // the rounds have been queued too), so the chip works on them while the host issues the
+        // rounds' launches; everything that needs the host to wait on the default stream (the sums
+        // above) is behind us.  The long witness rounds go first, on the default stream and so
+        // BEFORE the commitments, not beside them: a round kernel and the commitment kernel each
+        // fill the chip with two waves per SIMD, and side by side a SIMD holds one wave of each -
+        // the commitment's wave then issues at the rate of a lone wave (half) while the round's
+        // wave waits for memory, which made the pair slower than one after the other.  The short
+        // rounds (launch-bound) do run beside the commitments, on a stream of their own.
         if (overlap) {
-            witness.begin();                // both streams wait for what is queued so far - not for the commitments, queued next
+            while (vi >= 0 && cur / 2 >= kLongRoundPairs) witness_round(nullptr);
+            witness.begin();                // waits for what is queued so far (the long rounds) - not for the commitments, queued next
             ws = witness.stream;
-        }
-        // overlap: the commitments are queued now, without waiting (their digit-range flags are read
-        // after the rounds have been queued too), so the chip works on them while the host issues
-        // the rounds' launches; everything that needs the host to wait on the default stream (the
-        // sums above) is behind us
-        if (overlap) {
             check(grape_malloc((void**)&d_flags, 2 * sizeof(int)), "grape_malloc");
             check(grape_memset_zero(d_flags, 2 * sizeof(int), nullptr), "grape_memset_zero");
             // commit_time of this mode: what the commitment kernels take on the default stream, between two events
@@ -358,19 +380,7 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             });
             check(grape_event_record(commit_events().second, nullptr), "grape_event_record");
         }
-        uint cur = D;
-        uint k = 0;
-        for (int vi = (int)rounds - 1; vi >= 0; vi--, k++) {
-            const uint half = cur / 2;
-            fr_t* slot = sums.gpu_data + 13 * (size_t)k;
-            const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
-            // A and S: five sums and the fold of both tensors in one pass
-            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), ws),
-                  "grape_wround2");
-            A.set_size(half);
-            S.set_size(half);
-            cur = half;
-        }
+        while (vi >= 0) witness_round(ws);
         // the table side is queued second: its many small launches reach the chip while it works on the
         // first, long rounds of the witness side
         {
