@@ -351,8 +351,24 @@ int grape_alloc_cache_release(size_t* bytes_released) {
     if (bytes_released) *bytes_released = n;
     return GRAPE_OK;
 }
+// A payload of at most 1 KiB travels as the argument of a kernel that writes it: queued on the
+// stream like any other work, nothing to wait for, and the host buffer is free at once (the
+// launch has copied the argument).  A copy from pageable host memory would make the host wait for
+// everything the stream still holds - once per scalar handed to a kernel.
+struct SmallPayload { uint32_t w[256]; };
+__global__ void __launch_bounds__(256) poke_kernel(uint32_t* dst, SmallPayload p, uint32_t words) {
+    if (threadIdx.x < words) dst[threadIdx.x] = p.w[threadIdx.x];
+}
 int grape_memcpy_h2d(void* d, const void* s, size_t bytes, grape_stream_t st) {
     if (!bytes) return GRAPE_OK;
+    if (bytes <= sizeof(SmallPayload) && (bytes & 3) == 0 && (reinterpret_cast<uintptr_t>(d) & 3) == 0) {
+        GRAPE_REQUIRE(d != nullptr && s != nullptr, "null pointer");
+        SmallPayload p;
+        memcpy(p.w, s, bytes);
+        poke_kernel<<<1, 256, 0, as_stream(st)>>>((uint32_t*)d, p, (uint32_t)(bytes / 4));
+        GRAPE_LAUNCH_CHECK();
+        return GRAPE_OK;
+    }
     GRAPE_HIP_CHECK(hipMemcpyAsync(d, s, bytes, hipMemcpyHostToDevice, as_stream(st)));
     GRAPE_HIP_CHECK(hipStreamSynchronize(as_stream(st)));   // the host buffer may be reused at once
     return GRAPE_OK;

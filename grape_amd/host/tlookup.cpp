@@ -39,13 +39,11 @@ void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
     int* padded = nullptr;
     check(grape_malloc((void**)&padded, sizeof(int) * (size_t)pad_size), "grape_malloc");
     check(grape_i32_pad_fill(padded, d_idx_, N, pad_N, pad_size, fill, nullptr), "grape_i32_pad_fill");
-    check(grape_stream_sync(nullptr), "sync");
-    grape_free(d_idx_);
+    grape_free(d_idx_);                       // grape_free hands a block out again only after the work queued so far
     d_idx_ = padded;
 }
 void tLookup::drop_index() {
     if (d_idx_ || d_hist_) {
-        check(grape_stream_sync(nullptr), "sync");
         grape_free(d_idx_);
         grape_free(d_hist_);
         d_idx_ = nullptr;
@@ -66,7 +64,6 @@ void tLookup::index_to_m(uint witness_size, int low_) {
         check(grape_memcpy_h2d(hist + (-low_), &zero_count, sizeof(uint32_t), nullptr), "h2d");
     }
     m.get_data(m.size, hist);
-    check(grape_stream_sync(nullptr), "sync");
     grape_free(d_hist_);
     d_hist_ = hist;                           // kept for the proof in flight: the commitment of A picks its table entries by count
 }
@@ -302,7 +299,6 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     FrTensor Bm(B);
     Bm *= m;
     Fr alpha_sq = alpha * alpha;
-    Fr C = alpha_sq - Bm.sum(N);
     Fr claim = alpha + alpha_sq;
     Fr N_div_D = Fr((long)N) * Fr((long)D).invert();
     const Fr two_inv = Fr(2).invert();
@@ -315,15 +311,16 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     {
         fr_t* d_u = grape_host::upload(u);
         check(grape_eq_pyramid(W(E.gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_pyramid");
-        check(grape_stream_sync(nullptr), "sync");
-        grape_free(d_u);
+        grape_free(d_u);                    // no wait: the block is handed out again only after what is queued here
     }
     // The prover's challenges are all known before the first round, so the rounds are queued
     // back to back: every round leaves its 13 sums in its own slot of one device buffer, which
     // is read once after the last round; the polynomials and the running claim follow on the
     // host.  (The reference interleaves a device-to-host copy and a sync with every round.)
+    // (The sum of B * m, which only the host's constant term needs, travels with them.)
     const uint rounds = (uint)v.size();
-    FrTensor sums(13 * (rounds ? rounds : 1));
+    FrTensor sums(13 * (rounds ? rounds : 1) + 1);
+    check(grape_fr_sum(W(sums.gpu_data + 13 * (size_t)(rounds ? rounds : 1)), W(Bm.gpu_data), N, nullptr), "grape_fr_sum");
     fr_t* d_v = grape_host::upload(v);
     int* d_flags = nullptr;
     FrTensor Bw(B), Tw(T), mw(m);          // phase 2 binds copies; T, B, m of this object stay intact
@@ -410,8 +407,9 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             check(grape_event_elapsed_ms(&ms, commit_events().first, commit_events().second), "grape_event_elapsed_ms");
             commit_time += ms * 1e-3;
         }
-        std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1));
-        check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * 13 * (size_t)rounds, nullptr), "d2h");
+        std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1) + 1);
+        check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * h.size(), nullptr), "d2h");
+        Fr C = alpha_sq - h.back();
         grape_free(d_v);
         d_v = nullptr;
 

@@ -60,6 +60,9 @@ int grape_free(void *d_ptr);
  * cost tens of microseconds for small blocks and milliseconds and more for multi-GiB ones.  This gives every kept block back to the
  * driver (it also happens by itself when an allocation fails).  No counterpart in the reference. */
 int grape_alloc_cache_release(size_t *bytes_released);
+/* Host to device, ordered like any other work on `stream`; the host buffer may be reused as soon as
+ * the call returns.  At most 1 KiB (a scalar, a vector of challenges) is carried by a small kernel
+ * as its argument and the call does not wait; a longer copy waits for the stream. */
 int grape_memcpy_h2d(void *d_dst, const void *src, size_t bytes, grape_stream_t stream);
 int grape_memcpy_d2h(void *dst, const void *d_src, size_t bytes, grape_stream_t stream); /* syncs */
 int grape_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, grape_stream_t stream);
