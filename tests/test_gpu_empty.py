@@ -128,3 +128,37 @@ def test_memset_zero_of_any_size_and_alignment(ops):
         torch.cuda.synchronize()
         h = buf.cpu().numpy()
         assert not h[off:off + n].any() and (h[:off] == 0x5a).all() and (h[off + n:] == 0x5a).all(), (off, n)
+
+
+def test_host_to_device_copies_of_every_size_class(ops):
+    """grape_memcpy_h2d carries payloads of at most 1 KiB as a kernel argument and copies longer or
+    unaligned ones: 4 bytes to 1 KiB, just above it, odd lengths and odd destinations all arrive,
+    neighbours stay untouched, and the host buffer may be overwritten as soon as the call returns"""
+    import ctypes
+    import torch
+    from grape_amd import _capi
+    lib = ops.init()
+    rng = np.random.default_rng(11)
+    for nbytes, off in ((4, 0), (32, 0), (32, 64), (1020, 4), (1024, 0), (1028, 0), (4096, 0), (30, 0), (32, 2), (1, 5)):
+        dst = torch.full((8192,), 0xA5, dtype=torch.uint8, device="cuda")
+        src = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+        keep = src.copy()
+        _capi.check(lib.grape_memcpy_h2d(ctypes.c_void_p(dst.data_ptr() + off), src.ctypes.data_as(ctypes.c_void_p), nbytes, None))
+        src[:] = 0                                   # the call has taken what it needs
+        torch.cuda.synchronize()
+        got = dst.cpu().numpy()
+        assert np.array_equal(got[off:off + nbytes], keep), (nbytes, off)
+        assert (got[:off] == 0xA5).all() and (got[off + nbytes:] == 0xA5).all(), (nbytes, off)
+    # stream order: a value written, used and overwritten on the same stream
+    a = ops.to_dev(rand_fr(4, 3))
+    one = rand_fr(1, 4)
+    two = rand_fr(1, 5)
+    slot = torch.zeros(8, dtype=torch.int32, device="cuda")
+    outs = []
+    for val in (one, two):
+        buf = np.ascontiguousarray(val).view(np.uint32).copy()
+        _capi.check(lib.grape_memcpy_h2d(ctypes.c_void_p(slot.data_ptr()), buf.ctypes.data_as(ctypes.c_void_p), 32, None))
+        outs.append(slot.clone())
+    torch.cuda.synchronize()
+    assert np.array_equal(outs[0].cpu().numpy().view(np.uint32), np.ascontiguousarray(one).view(np.uint32).reshape(-1))
+    assert np.array_equal(outs[1].cpu().numpy().view(np.uint32), np.ascontiguousarray(two).view(np.uint32).reshape(-1))
