@@ -163,18 +163,20 @@ size_t Hyrax::table_bytes_in_use() const {
     return used;
 }
 
-// A small per-window table for full-width scalars (every window has its own set of multiples, so a
-// scalar multiple needs additions only): what the scaled table B[t] * G_i of a lookup object is built
-// through, one-off, at 24 additions per entry (c = 11: 13 GB for 4096 generators).  Commitments do
-// not use it when a strided table exists.
+// A per-window table for full-width scalars (every window has its own set of multiples, so a
+// scalar multiple needs additions only and one accumulator per lane): what the scaled table
+// B[t] * G_i of a lookup object is built through and what the sparse commitment reads, at one
+// addition per window (c = 13: 20 additions from 43 GB for 4096 generators; the widest window whose
+// table stays below 48 GB and inside the budget is taken - the table itself is generated in a tenth
+// of a second).  Multi-row commitments do not use it when a strided table exists.
 bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
     if (!build) return false;
     const size_t used = table_bytes_in_use();
-    for (uint c = 11; c >= 8; c--) {
+    for (uint c = 13; c >= 8; c--) {
         const uint nw = (255 + c - 1) / c, K = 1u << (c - 1);
         const size_t bytes = grape_g1_wide_table_bytes(rowlen, nw, K);
-        if (bytes <= ((size_t)16 << 30) && used + bytes <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
+        if (bytes <= ((size_t)48 << 30) && used + bytes <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }
     return false;
 }
