@@ -69,9 +69,10 @@ void tLookup::index_to_m(uint witness_size, int low_) {
 }
 
 // com(A) through the entries that occur often.  A[i] = B[index_i]; an entry t that occurs n_t times
-// costs n_t full-width scalars (16 additions each with the strided table) on the plain path, or one
-// row B[t]*G_i of the scaled table (rowlen entries at about 27 additions each, built for this proof
-// only) plus n_t single additions.  So an entry is worth a row when n_t > 1.8 rowlen; with the
+// costs n_t full-width scalars (16 to 20 additions each) on the plain path, or one row B[t]*G_i of
+// the scaled table (rowlen entries at 20 additions and a normalisation each, built for this proof
+// only) plus n_t single additions.  So an entry is worth a row when n_t exceeds rowlen by a factor
+// somewhat above one; 1.8 is taken (the proof's time is flat from 1.2 to 2.2), and with the
 // activations of a transformer layer nearly all elements sit on such entries.  Elements of the
 // other entries keep their scalars and are committed on the plain path; the two sums are added.
 // Returns false (nothing committed) when no entry qualifies or the table does not fit.
