@@ -167,8 +167,8 @@ size_t Hyrax::table_bytes_in_use() const {
 // scalar multiple needs additions only and one accumulator per lane): what the scaled table
 // B[t] * G_i of a lookup object is built through and what the sparse commitment reads, at one
 // addition per window (c = 13: 20 additions from 43 GB for 4096 generators; the widest window whose
-// table stays below 48 GB and inside the budget is taken - the table itself is generated in a tenth
-// of a second).  Multi-row commitments do not use it when a strided table exists.
+// table stays below its cap and inside the budget is taken - the table itself is generated in a
+// tenth of a second).  Multi-row commitments do not use it when a strided table exists.
 bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     if (fr_table_.d && fr_table_.ngen >= rowlen) return true;
     if (!build) return false;
@@ -176,7 +176,9 @@ bool Hyrax::ensure_fr_table(uint rowlen, bool build) {
     for (uint c = 13; c >= 8; c--) {
         const uint nw = (255 + c - 1) / c, K = 1u << (c - 1);
         const size_t bytes = grape_g1_wide_table_bytes(rowlen, nw, K);
-        if (bytes <= ((size_t)48 << 30) && used + bytes <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
+        // wide windows may take 48 GB, narrow ones (which lose to the strided table anyway) 16 GB
+        const size_t cap = (size_t)(c >= 12 ? 48 : 16) << 30;
+        if (bytes <= cap && used + bytes <= table_budget_) return ensure_table(fr_table_, rowlen, c, nw, K);
     }
     return false;
 }
@@ -272,8 +274,9 @@ affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
 
 affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
     if (ncols > npoints) throw std::runtime_error("row longer than the generator set");
-    if (!ensure_fr_table(ncols)) return nullptr;
     size_t bytes = grape_g1_wide_table_bytes(ncols, 1, scalars.size);   // one entry per (scalar, column)
+    if (table_bytes_in_use() + bytes > table_budget_) return nullptr;      // before the per-window table is built for nothing
+    if (!ensure_fr_table(ncols)) return nullptr;
     if (table_bytes_in_use() + bytes > table_budget_) return nullptr;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, bytes), "grape_malloc");
