@@ -52,6 +52,15 @@ def test_reference_table(ops, gens64):
     assert not got[:n].any()                  # w = 0 row is infinity
 
 
+def test_reference_table_edge_shapes(ops, gens64):
+    """the reference-format table for one generator and for few, with one multiple (the identity row only),
+    two, an odd count, one more than the first chain of the generator and the reference's 256"""
+    k, host, dev = gens64
+    for n, W in ((1, 1), (1, 2), (3, 3), (5, 17), (2, 18), (64, 33), (7, 256)):
+        got = ops.g1_to_host(ops.g1_table_gen(dev[:n].contiguous(), W))
+        assert_same(got, orc.g1_table(host[:n], W), "table n=%d W=%d" % (n, W))
+
+
 def test_wide_table_entries(ops, gens64):
     k, host, dev = gens64
     n, c, nw, K = 8, 8, 3, 128
