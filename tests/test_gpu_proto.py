@@ -151,6 +151,18 @@ def test_histogram_long_witness(ops):
     pre = torch.full((length,), 3, dtype=torch.int32, device="cuda")
     h2 = ops.tlookup_hist(vals, low, length, hist=pre).cpu().numpy().view(np.uint32)
     assert np.array_equal(h2, want + 3)
+    # a large table of which the witness touches little: most (chunk of the witness, range of bins)
+    # pairs are empty and are skipped; stray values put single elements into otherwise empty pairs
+    low2, length2 = -(1 << 19), 1 << 20
+    n2 = (1 << 21) + 5
+    t = np.rint(rng.normal(0.0, 181.0, size=n2)).astype(np.int64)
+    t[3] = low2
+    t[n2 // 2] = low2 + length2 - 1
+    t[n2 - 2] = 300000
+    t[n2 - 1] = low2 + length2                                  # just outside
+    want2 = np.bincount(t[:-1] - low2, minlength=length2).astype(np.uint32)
+    h4 = ops.tlookup_hist(ops.fr_from_i32(torch.from_numpy(t.astype(np.int32)).cuda()), low2, length2).cpu().numpy().view(np.uint32)
+    assert np.array_equal(h4, want2) and int(h4.sum()) == n2 - 1
     # small table, everything in one bin
     same = ops.fr_from_i32(torch.full(((1 << 20) + 1,), 5, dtype=torch.int32, device="cuda"))
     h3 = ops.tlookup_hist(same, 0, 16).cpu().numpy()
