@@ -747,48 +747,56 @@ __global__ void __launch_bounds__(64) strided_horner_kernel(uint32_t* out, const
 // ------------------------------------------------------------------------------------------------
 // commitment of the few elements of a tensor that a flag array lets through (full-width scalars)
 // ------------------------------------------------------------------------------------------------
-// One wave per row.  The wave sweeps the row's flags 64 columns at a time and queues the columns
-// whose flag is zero in LDS; whenever 64 are queued (and once more at the end of the row) every lane
-// takes one queued column, loads its scalar and adds scalar * G_col through the per-window table.
-// Lanes therefore work on dense batches however thinly the live elements are spread: sweeping the
-// whole tensor with the dense kernel costs a recoding per element and an addition slot per WAVE
-// that holds one live element - 80 ms for 2^27 elements of which 0.7 % are live, against 3 ms here.
+// G lanes per row, 64 / G rows per wave.  Every lane group sweeps its row's flags G columns at a
+// time and queues the columns whose flag is zero in LDS; whenever some group has G queued (and once
+// more at the end of the rows) every lane takes one queued column of its row, loads its scalar and
+// adds scalar * G_col through the per-window table.  Lanes therefore work on dense batches however
+// thinly the live elements are spread: sweeping the whole tensor with the dense kernel costs a
+// recoding per element and an addition slot per WAVE that holds one live element - 80 ms for 2^27
+// elements of which 0.7 % are live, against 3 ms here.  With many rows G = 32: a row of 4096 with
+// 27 live elements fills 27 of 32 lanes of its batch instead of 27 of 64.
+template <int G>
 __global__ void __launch_bounds__(64) commit_sparse_fr_kernel(uint32_t* partial, const uint32_t* scalars, const int32_t* __restrict__ skip,
                                                               uint32_t rowlen, size_t rows, const uint32_t* table, size_t N,
                                                               uint32_t c, uint32_t nw, uint32_t K, int* err_flag) {
-    __shared__ uint32_t queue[128];
+    constexpr int R = 64 / G;                            // rows per wave
+    __shared__ uint32_t queue[R][2 * G];
     const int lane = threadIdx.x;
-    const size_t row = blockIdx.x;
-    if (row >= rows) return;
+    const int grp = lane / G, sub = lane % G;
+    const size_t row = (size_t)blockIdx.x * R + grp;
+    const bool have_row = row < rows;
+    const unsigned long long gmask = (G == 64 ? ~0ull : ((1ull << (G & 63)) - 1ull)) << (grp * G);
     Xyzz28 acc = xyzz28_inf();
-    uint32_t qn = 0;                                     // queued columns (wave-uniform)
-    for (uint32_t base = 0;; base += 64) {
+    uint32_t qn = 0;                                     // queued columns of this lane's row (uniform within the group)
+    for (uint32_t base = 0;; base += G) {
         const bool last = base >= rowlen;
         if (!last) {
-            const uint32_t col = base + lane;
-            const bool take = col < rowlen && skip[geom::scalar_index(row, rowlen, col)] == 0;
-            const unsigned long long m = __ballot(take);
-            if (take) queue[qn + __popcll(m & ((1ull << lane) - 1ull))] = col;
+            const uint32_t col = base + sub;
+            const bool take = have_row && col < rowlen && skip[geom::scalar_index(row, rowlen, col)] == 0;
+            const unsigned long long m = __ballot(take) & gmask;
+            if (take) queue[grp][qn + __popcll(m & ((1ull << lane) - 1ull))] = col;
             qn += (uint32_t)__popcll(m);
             __syncthreads();
         }
-        if (qn >= 64 || (last && qn > 0)) {
-            const uint32_t n = qn < 64 ? qn : 64;
-            if ((uint32_t)lane < n) {
-                const uint32_t col = queue[lane];
+        // wave-uniform trigger: some group's batch is full, or the rows have ended with something queued
+        const bool go = last ? __any(qn > 0) : __any(qn >= (uint32_t)G);
+        if (go) {
+            const uint32_t n = qn < (uint32_t)G ? qn : (uint32_t)G;
+            if ((uint32_t)sub < n) {
+                const uint32_t col = queue[grp][sub];
                 const Fr k = from_mont(ld_fr8(scalars, geom::scalar_index(row, rowlen, col)));
                 madd_scalar_fr(acc, k, table, N, col, c, nw, K, err_flag);
             }
             __syncthreads();
-            const uint32_t moved = (uint32_t)lane + 64 < qn ? queue[lane + 64] : 0u;
+            const uint32_t moved = (uint32_t)sub + G < qn ? queue[grp][sub + G] : 0u;
             __syncthreads();
-            if ((uint32_t)lane + 64 < qn) queue[lane] = moved;
+            if ((uint32_t)sub + G < qn) queue[grp][sub] = moved;
             qn -= n;
             __syncthreads();
         }
         if (last) break;
     }
-    st_partial28(partial, row * 64 + lane, acc);
+    if (have_row) st_partial28(partial, row * G + sub, acc);
 }
 
 // Row epilogue: 2^lg_lpr lanes per row, each sums its share of the partials serially, then a
@@ -1235,10 +1243,16 @@ int grape_commit_fr_sparse(uint32_t* out, const uint32_t* scalars, const int32_t
         const size_t nr = rows - r0 < slab ? rows - r0 : slab;
         const uint32_t lg_lpr = reduce_lanes_log2(nr);
         const size_t rows_per_wave = (size_t)64 >> lg_lpr;
-        commit_sparse_fr_kernel<<<(unsigned)nr, 64, 0, s>>>((uint32_t*)ws, scalars + r0 * rowlen * 8, skip + r0 * rowlen, rowlen, nr, table, N,
-                                                           c, nw, K, err);
+        // many rows: half a wave per row, so that a thinly populated row still fills its batch
+        const bool narrow = nr >= 4096;
+        if (narrow)
+            commit_sparse_fr_kernel<32><<<(unsigned)((nr + 1) / 2), 64, 0, s>>>((uint32_t*)ws, scalars + r0 * rowlen * 8, skip + r0 * rowlen, rowlen, nr,
+                                                                              table, N, c, nw, K, err);
+        else
+            commit_sparse_fr_kernel<64><<<(unsigned)nr, 64, 0, s>>>((uint32_t*)ws, scalars + r0 * rowlen * 8, skip + r0 * rowlen, rowlen, nr, table, N,
+                                                                   c, nw, K, err);
         commit_reduce_kernel<true><<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW),
-                                                                                                  (const uint32_t*)ws, nr, 64, lg_lpr);
+                                                                                                  (const uint32_t*)ws, nr, narrow ? 32 : 64, lg_lpr);
     }
     GRAPE_LAUNCH_CHECK();
     int h_err = 0;

@@ -389,11 +389,13 @@ def test_reference_table_path_in_every_launch_shape(ops):
         assert_same(got, want, "i32 ref table %dx%d" % (rows, rowlen))
 
 
-@pytest.mark.parametrize("rowlen,rows,live", [(16, 5, 0.3), (200, 7, 0.02), (200, 7, 0.9), (64, 3, 0.0), (1000, 4, 0.07)])
+@pytest.mark.parametrize("rowlen,rows,live", [(16, 5, 0.3), (200, 7, 0.02), (200, 7, 0.9), (64, 3, 0.0), (1000, 4, 0.07),
+                                              (48, 4097, 0.3), (100, 5000, 0.02), (70, 4096, 0.9)])
 def test_commit_fr_sparse_against_dense_commitment_of_masked_tensor(ops, rowlen, rows, live):
-    """the commitment of the flagged-in elements only (queued per row, dense batches of 64, a last
-    partial batch, rows with none) equals the dense commitment of the tensor with the others zeroed,
-    and the oracle's on a few rows"""
+    """the commitment of the flagged-in elements only (queued per row, dense batches of 64 - of 32 with
+    two rows per wave when the rows are many, an odd number of them included - a last partial batch,
+    rows with none) equals the dense commitment of the tensor with the others zeroed, and the
+    oracle's on a few rows"""
     import torch
     k = _scalars(rowlen, 131)
     dev = ops.g1_make_generators(k)
