@@ -566,6 +566,8 @@ def rounds_workload(args):
         ("sumcheck2_kernel<three sums> + final_sum (grape_sumcheck_round2)", 192, h, lambda: ops.sumcheck_round2(A, B, n, h, v)),
         ("wround2_kernel<beta, plain sums> + final (grape_wround2, logUp round)", 224, h,
          lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True)),
+        ("wround2_kernel<beta, plain sums, inverse pair> + final (grape_wround2, first logUp round over A = 1/(S + beta))", 224, h,
+         lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True, inverse_pair=True)),
         ("wround2_kernel<no beta> + final (grape_wround2, element-product round)", 224, h,
          lambda: ops.wround2(A, B, None, e, n, h, v)),
         ("tl_round_kernel + final_sum (grape_tlookup_round_sums, read only)", 160, h, lambda: ops.tlookup_round_sums(A, B, beta, e, h)),

@@ -59,7 +59,11 @@ __device__ __forceinline__ Fr reduce_to_fr(fr26::Acc& C, int lo_r) {
     return fr26::unpack(fr26::canon_wide(fr26::reduce(C, lo_r)));
 }
 
-template <bool BETA, bool PLAIN>
+// UNIT: the caller states that A[i] * (S[i] + beta) = 1 at every index (the first round of a logUp
+// proof, where A was made as the inverse of S + beta).  Then the constant coefficient is the sum of
+// the weights and the value at t = 1 equals it, so only the top coefficient sum_g e * dA * dS is
+// taken: one weight product and one accumulation per index instead of two and three.
+template <bool BETA, bool PLAIN, bool UNIT = false>
 __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E,
                                                          uint32_t in_size, uint32_t n_out, uint32_t rowlen, uint32_t rowpad,
                                                          const uint32_t* v, uint32_t* partial) {
@@ -85,9 +89,12 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         const fr26::Limbs da = fr26::sub(a1, a0);
         st_fr(A, g, fold1(w1, a0, da));
         fr26::Acc T;
-        fr26::acc_zero(T);
-        fr26::mac(T, e16, a0);
-        const fr26::Limbs ea0 = fr26::reduce(T, 0);
+        fr26::Limbs ea0;
+        if (!UNIT) {
+            fr26::acc_zero(T);
+            fr26::mac(T, e16, a0);
+            ea0 = fr26::reduce(T, 0);
+        }
         fr26::acc_zero(T);
         fr26::mac(T, e16, da);
         const fr26::Limbs ead = fr26::reduce(T, 1);
@@ -100,7 +107,9 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         const fr26::Limbs ds = fr26::sub(s1r, s0r);
         st_fr(S, g, fold1(w1, s0r, ds));
         fr26::mac(W2, ead, ds);
-        if (BETA) {
+        if (UNIT) {
+            // W0 and WQ stay zero: the finishing kernel writes the coefficients they would give
+        } else if (BETA) {
             fr26::mac(W0, ea0, fr26::add(s0r, bt));
             fr26::mac(WQ, fr26::add(ea0, ead), fr26::add(s1r, bt));
         } else {
@@ -125,7 +134,8 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
 }
 
 // sums[0..2] = 16 * (W0, WQ - W0 - W2, W2); with PLAIN sums[3] = sum A0, sums[4] = sum A1 - sum A0
-template <bool PLAIN>
+// UNIT (weights that sum to one, A * (S + beta) = 1 everywhere): sums[0] = 1, sums[1] = -sums[2]
+template <bool PLAIN, bool UNIT = false>
 __global__ void __launch_bounds__(kBlock) wround2_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
     constexpr int NV = PLAIN ? 5 : 3;
     __shared__ Fr lds[NV * (kBlock / 64)];
@@ -144,8 +154,14 @@ __global__ void __launch_bounds__(kBlock) wround2_final_kernel(uint32_t* out, co
             Fr t = w[k];
 #pragma unroll
             for (int d = 0; d < 4; d++) t = add(t, t);
-            st_fr(out, k, t);
+            w[k] = t;
         }
+        if (UNIT) {
+            w[0] = Fr::one();
+            w[1] = sub(Fr::zero(), w[2]);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; k++) st_fr(out, k, w[k]);
         if (PLAIN) {
             st_fr(out, 3, acc[3]);
             st_fr(out, 4, sub(acc[4], acc[3]));
@@ -294,7 +310,13 @@ int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t
     int rc = scratch_get(kSlotReduce, (size_t)nb * nv * 32, &ws, s);
     if (rc) return rc;
     uint32_t* partial = (uint32_t*)ws;
-    if (beta && plain_sums) {
+    if (plain_sums == 2) {
+        GRAPE_REQUIRE(rowlen == rowpad && in_size == 2 * (uint64_t)n_out,
+                      "the inverse-pair round needs whole pairs and unpadded rows (weights that sum to one)");
+        if (beta) wround2_kernel<true, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        else wround2_kernel<false, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
+        wround2_final_kernel<true, true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    } else if (beta && plain_sums) {
         wround2_kernel<true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
         wround2_final_kernel<true><<<1, kBlock, 0, s>>>(sums, partial, nb);
     } else if (beta) {

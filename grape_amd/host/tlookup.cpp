@@ -341,7 +341,12 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             const uint half = cur / 2;
             fr_t* slot = sums.gpu_data + 13 * (size_t)k;
             const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
-            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), 1, W(slot), st), "grape_wround2");
+            // first round of a witness that sits on its table: A = B[index] is the exact inverse of S + beta at
+            // every index (B holds the inverses of T + beta, none of which is zero for a range table and, for
+            // a mapping table with its random r, except with probability 2^-235), and the weights of a full
+            // level sum to one - the round then needs its top coefficient only
+            const int mode = (k == 0 && from_table && cur == 2 * half && (cur & (cur - 1)) == 0) ? 2 : 1;
+            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), mode, W(slot), st), "grape_wround2");
             A.set_size(half);
             S.set_size(half);
             cur = half;

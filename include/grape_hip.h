@@ -182,6 +182,11 @@ int grape_eq_pyramid(uint32_t *d_pyr, const uint32_t *d_u, uint32_t nu, grape_st
  * When the tensors' rows hold rowlen elements but the weights live on rows padded to rowpad entries
  * (rows of 11008 with weights over 16384), g' = g + (g / rowlen) * (rowpad - rowlen); otherwise pass
  * rowlen = rowpad and g' = g.  d_sums holds 3 (5 with plain_sums) elements.
+ * plain_sums == 2 (with rowlen == rowpad and in_size == 2 n_out) is the round of a caller that knows
+ * A[i] * (S[i] + beta) = 1 at every index and weights that sum to one - the first round of a logUp
+ * proof over A = 1/(S + beta): d_sums[0] = 1 and d_sums[1] = -d_sums[2] then follow without being
+ * summed, and the pass takes one weight product per index instead of two.  The five sums equal those
+ * of plain_sums == 1 whenever the statement holds.
  * One pass replaces sumcheck_kernel + three folds of coefficient arrays per round in eleMul_sumcheck
  * (src/prove.cu:119-172) and tLookup_poly_kernel + three multilinear evaluations +
  * tLookup_poly_sum_kernel + two sums + the reduce kernel in tLookup_phase1 (src/tlookup.cu:117-151,216-244).

@@ -326,6 +326,32 @@ def test_weighted_round_with_fused_fold(ops, in_size, n_out, beta, plain):
     assert_same(ops.fr_to_host(dS)[:n_out], orc.partial_eval(Sp, 2 * n_out, v, 2, 0, n_out)[:n_out], "folded S")
 
 
+@pytest.mark.parametrize("n_out,beta", [(1, True), (4096, True), (1 << 17, True), ((1 << 18), False)])
+def test_weighted_round_of_an_inverse_pair(ops, n_out, beta):
+    """the first round of a logUp proof, where A = 1/(S + beta): the variant that takes only the top
+    coefficient (and writes 1 and its negative for the other two) gives the five sums and the folds
+    of the general round, which in turn match the oracle's coefficients"""
+    in_size = 2 * n_out
+    logh = br.log2ceil(n_out)
+    S = rand_fr(in_size, 281 + n_out)
+    bt, v, u = rand_fr(1, 283), rand_fr(1, 284), rand_fr(max(logh, 1), 285)
+    zero = np.zeros((1, 4), dtype=np.uint64)
+    dbt = ops.to_dev(bt) if beta else None
+    A = ops.fr_to_host(ops.fr_shift_inverse(ops.to_dev(S), ops.to_dev(bt if beta else zero)))
+    e = ops.eq_pyramid(ops.to_dev(u), logh)[n_out - 1:2 * n_out - 1].contiguous()
+    dA1, dS1, dA2, dS2 = ops.to_dev(A), ops.to_dev(S), ops.to_dev(A), ops.to_dev(S)
+    general = ops.fr_to_host(ops.wround2(dA1, dS1, dbt, e, in_size, n_out, ops.to_dev(v), plain_sums=True))
+    short = ops.fr_to_host(ops.wround2(dA2, dS2, dbt, e, in_size, n_out, ops.to_dev(v), plain_sums=True, inverse_pair=True))
+    assert_same(short, general, "five sums")
+    assert br.fr_unpack(short[:1]) == [1]
+    assert_same(ops.fr_to_host(dA2)[:n_out], ops.fr_to_host(dA1)[:n_out], "folded A")
+    assert_same(ops.fr_to_host(dS2)[:n_out], ops.fr_to_host(dS1)[:n_out], "folded S")
+    if n_out <= 4096:
+        o = [ops.fr_to_host(t) for t in ops.tlookup_poly(ops.to_dev(A), ops.to_dev(S), dbt, n_out)]
+        for k in range(3):
+            assert_same(short[k], orc.mle_eval(o[k], u[:logh]), "weighted coefficient %d" % k)
+
+
 def test_weighted_round_on_padded_rows(ops):
     """rows of 11 elements whose weights live on rows padded to 16: row f, column j takes e[16 f + j]"""
     rows, rl, rp = 64, 11, 16
