@@ -69,6 +69,7 @@ SIGNATURES = {
     "grape_fr_axpy": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_hot_select": [c_void_p, c_u32, c_u32, c_u32, c_void_p, c_void_p, ctypes.POINTER(ctypes.c_uint64), c_void_p],
     "grape_tlookup_hot_index": [c_void_p, c_void_p, c_size_t, c_void_p, c_u32, c_void_p],
+    "grape_tlookup_hot_coverage": [c_void_p, c_u32, c_void_p, ctypes.POINTER(ctypes.c_uint64), c_void_p],
     "grape_fr_mask_cold": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_fr_gather": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_commit_fr_sparse": [c_void_p, c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],

@@ -189,7 +189,8 @@ def tlookup_mapping_prove(dS_in, dS_out, D, low, length, table, alpha, r, u, v, 
 
 def tlookup_mapping_prove_ex(dS_in, dS_out, D, low, length, table, alpha, r, u, v, d_table, npoints, com_scale, msm_size,
                              hot_min_count=0):
-    """returns (transcript, S(v), com_A, entries with a table row, elements committed as full-width scalars)"""
+    """returns (transcript, S(v), com_A, entries with a table row, elements committed as full-width scalars,
+    whether the rows were found in place from an earlier proof of the same lookup object)"""
     lib = load()
     alpha, r, u, v = _fr(alpha, 1), _fr(r, 1), _fr(u), _fr(v)
     table = np.ascontiguousarray(table, dtype=np.int32)
@@ -198,11 +199,11 @@ def tlookup_mapping_prove_ex(dS_in, dS_out, D, low, length, table, alpha, r, u, 
     sc = np.zeros(4, dtype=np.uint64)
     Dp = 1 << max(0, (D - 1).bit_length())
     com_a = np.zeros((Dp // (msm_size * com_scale), G1W), dtype=np.uint64)
-    stats = (ctypes.c_uint64 * 2)()
+    stats = (ctypes.c_uint64 * 3)()
     _check(lib.grape_host_tlookup_mapping_prove_ex(_dp(dS_in), _dp(dS_out), D, low, length, _hp(table), _hp(alpha), _hp(r),
                                                    _hp(u), _hp(v), u.shape[0], _dp(d_table), npoints, com_scale, msm_size,
                                                    _hp(tr), ctypes.byref(nr), _hp(sc), hot_min_count, _hp(com_a), stats))
-    return tr[: nr.value].copy(), sc, com_a, int(stats[0]), int(stats[1])
+    return tr[: nr.value].copy(), sc, com_a, int(stats[0]), int(stats[1]), bool(stats[2])
 
 
 def fr_op(op, a, b=None):

@@ -963,6 +963,40 @@ int grape_tlookup_hot_select(const uint32_t* hist, uint32_t len, uint32_t min_co
     return GRAPE_OK;
 }
 
+// what a slot assignment made for an earlier witness leaves uncovered in this one
+__global__ void __launch_bounds__(kBlock) hot_coverage_kernel(const uint32_t* __restrict__ hist, uint32_t len, const int32_t* __restrict__ slot1,
+                                                              unsigned long long* info) {
+    __shared__ unsigned long long part[kBlock / 64];
+    unsigned long long cold = 0;
+    for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < len; t += gridDim.x * kBlock)
+        if (slot1[t] == 0) cold += hist[t];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) cold += __shfl_xor(cold, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = cold;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long sum = 0;
+        for (int w = 0; w < kBlock / 64; w++) sum += part[w];
+        if (sum) atomicAdd(info, sum);               // one atomic per workgroup
+    }
+}
+int grape_tlookup_hot_coverage(const uint32_t* hist, uint32_t len, const int32_t* slot1, uint64_t* cold_elements, grape_stream_t st) {
+    GRAPE_REQUIRE(hist != nullptr && slot1 != nullptr && cold_elements != nullptr && len > 0, "bad arguments");
+    hipStream_t s = as_stream(st);
+    void* ws;
+    int rc = scratch_get(kSlotMisc, 64, &ws, s);
+    if (rc) return rc;
+    rc = zero_fill(ws, 8, s);
+    if (rc) return rc;
+    unsigned nb = blocks_for(len);
+    if (nb > 256) nb = 256;
+    hot_coverage_kernel<<<nb, kBlock, 0, s>>>(hist, len, slot1, (unsigned long long*)ws);
+    GRAPE_LAUNCH_CHECK();
+    GRAPE_HIP_CHECK(hipMemcpyAsync(cold_elements, ws, sizeof(uint64_t), hipMemcpyDeviceToHost, s));
+    GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+    return GRAPE_OK;
+}
+
 int grape_tlookup_hot_index(int32_t* out, const int32_t* idx1, size_t n, const int32_t* slot1, uint32_t len, grape_stream_t st) {
     if (n == 0) return GRAPE_OK;
     GRAPE_REQUIRE(out != nullptr && idx1 != nullptr && slot1 != nullptr && len > 0, "bad arguments");

@@ -37,10 +37,12 @@ struct ProveTimer {
     return 0;
 
 #include <map>
+#include <array>
 #include <memory>
 #include <tuple>
 // Hyrax objects persist across calls (keyed by their table), so the wide fixed-base tables
 // they build are generated once per generator set, as in a long-running prover.
+static void drop_lookup_objects();   // they hold tables tied to a Hyrax object: gone before it goes
 static Hyrax& hyrax_for(const uint32_t* d_table, uint32_t npoints, uint32_t com_scale, uint32_t layer_num) {
     typedef std::tuple<const uint32_t*, uint32_t, uint32_t, uint32_t> Key;
     static std::map<Key, std::unique_ptr<Hyrax>> cache;
@@ -48,7 +50,10 @@ static Hyrax& hyrax_for(const uint32_t* d_table, uint32_t npoints, uint32_t com_
     Key k(d_table, npoints, com_scale, layer_num);
     auto it = cache.find(k);
     if (it == cache.end()) {
-        if (cache.size() >= 4) cache.clear();   // bounded: drop old tables
+        if (cache.size() >= 4) {                // bounded: drop old tables
+            drop_lookup_objects();
+            cache.clear();
+        }
         it = cache.emplace(k, std::unique_ptr<Hyrax>(new Hyrax(layer_num, npoints / com_scale, (affine_t*)d_table, G, com_scale))).first;
     }
     return *it->second;
@@ -191,6 +196,39 @@ int grape_host_hyrax_open_verify(const uint32_t* d_tensor, uint32_t size, uint32
     GUARD_END
 }
 
+extern "C++" {
+// Lookup objects persist across calls like the reference's driver keeps them across the layers of a
+// model (test/llm.cu:57-64): the tables tied to them (B[t]*G_i over every entry of a range table,
+// over the occupied entries of a mapping table) are built by the first proof.
+typedef std::tuple<int32_t, uint32_t, Hyrax*> LKey;
+static std::map<LKey, std::unique_ptr<tLookupRange>> g_range_lookups;
+// a mapping lookup with its r pinned (the constructor draws r; the table is rebuilt with the given one)
+struct PinnedMapping : tLookupRangeMapping {
+    PinnedMapping(int low, uint len, const int* map, const Fr& r_) : tLookupRangeMapping(low, len, map) {
+        r = r_;
+        grape_host::check(grape_tlookup_init((uint32_t*)T.gpu_data, (uint32_t*)B.gpu_data, low, len,
+                                             (uint32_t*)grape_host::device_scalar(beta), (uint32_t*)mapped_vals.gpu_data,
+                                             (uint32_t*)grape_host::device_scalar(r), nullptr),
+                          "grape_tlookup_init");
+    }
+};
+// keyed by range, r, a hash of the mapped values and the Hyrax object
+typedef std::tuple<int32_t, uint32_t, std::array<uint64_t, 4>, uint64_t, Hyrax*> MKey;
+static std::map<MKey, std::unique_ptr<PinnedMapping>> g_mapping_lookups;
+static void drop_lookup_objects() {
+    g_range_lookups.clear();
+    g_mapping_lookups.clear();
+}
+static uint64_t hash_ints(const int32_t* p, size_t n) {
+    uint64_t h = 1469598103934665603ull;                 // FNV-1a over the words
+    for (size_t i = 0; i < n; i++) {
+        h ^= (uint32_t)p[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+}  // extern "C++"
+
 int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low, uint32_t len, const uint32_t* alpha,
                                    const uint32_t* u, const uint32_t* v, uint32_t nuv, const uint32_t* d_table, uint32_t npoints,
                                    uint32_t com_scale, uint32_t msm_size, uint32_t* m_out, uint32_t* transcript, uint32_t* n_rounds,
@@ -198,13 +236,11 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
     GUARD_BEGIN
     Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
     // lookup objects persist like Hyrax objects: their scaled table is built once
-    typedef std::tuple<int32_t, uint32_t, Hyrax*> LKey;
-    static std::map<LKey, std::unique_ptr<tLookupRange>> lcache;
     LKey lkey(low, len, &hyrax);
-    auto lit = lcache.find(lkey);
-    if (lit == lcache.end()) {
-        if (lcache.size() >= 2) lcache.clear();
-        lit = lcache.emplace(lkey, std::unique_ptr<tLookupRange>(new tLookupRange(low, len))).first;
+    auto lit = g_range_lookups.find(lkey);
+    if (lit == g_range_lookups.end()) {
+        if (g_range_lookups.size() >= 2) g_range_lookups.clear();
+        lit = g_range_lookups.emplace(lkey, std::unique_ptr<tLookupRange>(new tLookupRange(low, len))).first;
     }
     tLookupRange& lk = *lit->second;
     lk.set_indexed_commit(g_indexed_commit);
@@ -235,16 +271,15 @@ static void mapping_prove_impl(const uint32_t* d_S_in, const uint32_t* d_S_out, 
                                uint32_t msm_size, uint32_t* transcript, uint32_t* n_rounds, uint32_t* S_claim,
                                uint32_t hot_min_count, uint32_t* com_A_out, uint64_t* hot_stats) {
     Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, 1);
-    // r is drawn in the constructor; to pin it, seed-independent, rebuild the table with the given r
-    struct Pinned : tLookupRangeMapping {
-        Pinned(int low, uint len, const int* map, const Fr& r_) : tLookupRangeMapping(low, len, map) {
-            r = r_;
-            grape_host::check(grape_tlookup_init((uint32_t*)T.gpu_data, (uint32_t*)B.gpu_data, low, len,
-                                                 (uint32_t*)grape_host::device_scalar(beta), (uint32_t*)mapped_vals.gpu_data,
-                                                 (uint32_t*)grape_host::device_scalar(r), nullptr),
-                              "grape_tlookup_init");
-        }
-    } lk(low, len, map, fr_from(r));
+    std::array<uint64_t, 4> rk;
+    std::memcpy(rk.data(), r, 32);
+    MKey mkey(low, len, rk, hash_ints(map, len), &hyrax);
+    auto mit = g_mapping_lookups.find(mkey);
+    if (mit == g_mapping_lookups.end()) {
+        if (g_mapping_lookups.size() >= 4) g_mapping_lookups.clear();
+        mit = g_mapping_lookups.emplace(mkey, std::unique_ptr<PinnedMapping>(new PinnedMapping(low, len, map, fr_from(r)))).first;
+    }
+    PinnedMapping& lk = *mit->second;
     lk.set_indexed_commit(g_indexed_commit);
     lk.set_hot_min_count(hot_min_count);
     lk.alpha = fr_from(alpha);
@@ -266,6 +301,7 @@ static void mapping_prove_impl(const uint32_t* d_S_in, const uint32_t* d_S_out, 
     if (hot_stats) {
         hot_stats[0] = lk.hot_entries();
         hot_stats[1] = lk.cold_elements();
+        hot_stats[2] = lk.hot_rows_reused() ? 1 : 0;
     }
 }
 

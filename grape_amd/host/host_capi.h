@@ -70,7 +70,11 @@ int grape_host_tlookup_mapping_prove(const uint32_t *d_S_in, const uint32_t *d_S
 /* The same, with the count from which a table entry gets a row of the per-proof table B[t]*G_i
  * (0 = the break-even count), the commitment of A (affine, D / (msm_size*com_scale) points) and
  * hot_stats[0] = entries that got a row, hot_stats[1] = elements committed as full-width scalars
- * (both zero when the plain path was taken). */
+ * (both zero when the plain path was taken), hot_stats[2] = 1 when the rows were found in place:
+ * lookup objects persist across calls (keyed by range, r, the mapped values and the generators) as the
+ * reference's driver keeps them across the layers of a model, and the rows of an earlier proof serve
+ * a later one while they cover its witness; a call with hot_min_count != 0 builds its own rows and
+ * keeps none. */
 int grape_host_tlookup_mapping_prove_ex(const uint32_t *d_S_in, const uint32_t *d_S_out, uint32_t D, int32_t low,
                                         uint32_t len, const int32_t *map, const uint32_t *alpha, const uint32_t *r,
                                         const uint32_t *u, const uint32_t *v, uint32_t nuv, const uint32_t *d_table,

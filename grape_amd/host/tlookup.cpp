@@ -15,6 +15,8 @@ tLookup::~tLookup() {
     grape_free(com_A);
     grape_free(com_m);
     Hyrax::release_scaled_table(scaled_table_);
+    Hyrax::release_scaled_table(hot_table_);
+    grape_free(hot_slot1_);
     grape_free(d_idx_);
 }
 
@@ -76,62 +78,93 @@ void tLookup::index_to_m(uint witness_size, int low_) {
 // activations of a transformer layer nearly all elements sit on such entries.  Elements of the
 // other entries keep their scalars and are committed on the plain path; the two sums are added.
 // Returns false (nothing committed) when no entry qualifies or the table does not fit.
+void tLookup::drop_hot_rows() {
+    Hyrax::release_scaled_table(hot_table_);
+    grape_free(hot_slot1_);
+    hot_table_ = nullptr;
+    hot_slot1_ = nullptr;
+    hot_rows_ = hot_cols_ = 0;
+    hot_for_ = nullptr;
+}
+
 bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& hyrax) {
     const uint N = T.size;
     const uint rowlen = msm_size * hyrax.com_scale;
     const uint rows = D / rowlen;
     const uint min_count = hot_min_count_ ? hot_min_count_ : (uint)(1.8 * rowlen) + 1;
-    const size_t row_bytes = grape_g1_wide_table_bytes(rowlen, 1, 1);
-    const size_t free_bytes = hyrax.table_bytes_free();
-    size_t max_hot = free_bytes / row_bytes;
-    if (max_hot > N) max_hot = N;
-    if (max_hot == 0) return false;
-    int* d_slot1 = nullptr;
-    uint32_t* d_list = nullptr;
-    int* d_hot = nullptr;
-    affine_t* table = nullptr;
-    affine_t* com_cold = nullptr;
-    bool done = false;
-    try {
-        check(grape_malloc((void**)&d_slot1, sizeof(int) * (size_t)N), "grape_malloc");
-        check(grape_malloc((void**)&d_list, sizeof(uint32_t) * (size_t)N), "grape_malloc");
-        uint64_t info[2] = {0, 0};
-        check(grape_tlookup_hot_select(d_hist_, N, min_count, (uint32_t)max_hot, d_slot1, d_list, info, nullptr), "grape_tlookup_hot_select");
-        const uint n_hot = (uint)info[0];
-        if (n_hot != 0) {
-            FrTensor Bhot(n_hot);
-            check(grape_fr_gather(W(Bhot.gpu_data), W(B.gpu_data), d_list, n_hot, nullptr), "grape_fr_gather");
-            table = hyrax.build_scaled_table(Bhot, rowlen);
-        }
-        if (table) {
-            check(grape_malloc((void**)&d_hot, sizeof(int) * (size_t)D), "grape_malloc");
-            check(grape_tlookup_hot_index(d_hot, d_idx_, D, d_slot1, N, nullptr), "grape_tlookup_hot_index");
-            com_A = hyrax.commit_indexed_affine(d_hot, D, msm_size, table, rowlen, n_hot);
-            if (info[1] != 0) {
-                // the elements without a table row: queued per row and committed as full-width scalars
-                com_cold = hyrax.commit_sparse_affine(A, d_hot, D, msm_size);
-                if (!com_cold) {
-                    FrTensor Acold(D);
-                    check(grape_fr_mask_cold(W(Acold.gpu_data), W(A.gpu_data), d_hot, D, nullptr), "grape_fr_mask_cold");
-                    com_cold = hyrax.commit_affine(Acold, D, msm_size);
-                }
-                check(grape_g1_affine_add((uint32_t*)com_A, (const uint32_t*)com_A, (const uint32_t*)com_cold, rows, nullptr),
-                      "grape_g1_affine_add");
+    hot_reused_ = false;
+    uint64_t cold = 0;
+    // rows kept from an earlier proof: used again when the elements they leave out (20 additions
+    // each instead of one) cost less than building rows anew (rowlen entries of 20 additions and a
+    // normalisation per row)
+    if (hot_table_ && (hot_for_ != &hyrax || hot_cols_ != rowlen)) drop_hot_rows();
+    if (hot_table_ && hot_min_count_ == 0) {
+        check(grape_tlookup_hot_coverage(d_hist_, N, hot_slot1_, &cold, nullptr), "grape_tlookup_hot_coverage");
+        if ((double)cold * 19.0 <= (double)hot_rows_ * rowlen * 23.0) hot_reused_ = true;
+    }
+    if (!hot_reused_) {
+        drop_hot_rows();
+        const size_t row_bytes = grape_g1_wide_table_bytes(rowlen, 1, 1);
+        size_t max_hot = hyrax.table_bytes_free() / row_bytes;
+        if (max_hot > N) max_hot = N;
+        if (max_hot == 0) return false;
+        uint32_t* d_list = nullptr;
+        try {
+            check(grape_malloc((void**)&hot_slot1_, sizeof(int) * (size_t)N), "grape_malloc");
+            check(grape_malloc((void**)&d_list, sizeof(uint32_t) * (size_t)N), "grape_malloc");
+            uint64_t info[2] = {0, 0};
+            check(grape_tlookup_hot_select(d_hist_, N, min_count, (uint32_t)max_hot, hot_slot1_, d_list, info, nullptr), "grape_tlookup_hot_select");
+            const uint n_hot = (uint)info[0];
+            cold = info[1];
+            if (n_hot != 0) {
+                FrTensor Bhot(n_hot);
+                check(grape_fr_gather(W(Bhot.gpu_data), W(B.gpu_data), d_list, n_hot, nullptr), "grape_fr_gather");
+                hot_table_ = hyrax.build_scaled_table(Bhot, rowlen);
             }
-            hot_entries_ = n_hot;
-            cold_elements_ = info[1];
-            done = true;
+            hot_rows_ = n_hot;
+            hot_cols_ = rowlen;
+            hot_for_ = &hyrax;
+        } catch (...) {
+            grape_stream_sync(nullptr);
+            grape_free(d_list);
+            drop_hot_rows();
+            throw;
         }
+        grape_free(d_list);
+        if (!hot_table_) {
+            drop_hot_rows();
+            return false;
+        }
+    }
+    int* d_hot = nullptr;
+    affine_t* com_cold = nullptr;
+    try {
+        check(grape_malloc((void**)&d_hot, sizeof(int) * (size_t)D), "grape_malloc");
+        check(grape_tlookup_hot_index(d_hot, d_idx_, D, hot_slot1_, N, nullptr), "grape_tlookup_hot_index");
+        com_A = hyrax.commit_indexed_affine(d_hot, D, msm_size, hot_table_, rowlen, hot_rows_);
+        if (cold != 0) {
+            // the elements without a table row: queued per row and committed as full-width scalars
+            com_cold = hyrax.commit_sparse_affine(A, d_hot, D, msm_size);
+            if (!com_cold) {
+                FrTensor Acold(D);
+                check(grape_fr_mask_cold(W(Acold.gpu_data), W(A.gpu_data), d_hot, D, nullptr), "grape_fr_mask_cold");
+                com_cold = hyrax.commit_affine(Acold, D, msm_size);
+            }
+            check(grape_g1_affine_add((uint32_t*)com_A, (const uint32_t*)com_A, (const uint32_t*)com_cold, rows, nullptr),
+                  "grape_g1_affine_add");
+        }
+        hot_entries_ = hot_rows_;
+        cold_elements_ = cold;
         check(grape_stream_sync(nullptr), "sync");
     } catch (...) {
         grape_stream_sync(nullptr);
-        grape_free(d_slot1); grape_free(d_list); grape_free(d_hot); grape_free(com_cold);
-        Hyrax::release_scaled_table(table);
+        grape_free(d_hot); grape_free(com_cold);
         throw;
     }
-    grape_free(d_slot1); grape_free(d_list); grape_free(d_hot); grape_free(com_cold);
-    Hyrax::release_scaled_table(table);
-    return done;
+    grape_free(d_hot); grape_free(com_cold);
+    // a caller that pins the count threshold is measuring one selection: nothing is kept for the next proof
+    if (hot_min_count_ != 0) drop_hot_rows();
+    return true;
 }
 
 namespace {
@@ -231,6 +264,9 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     if (D % msm_size != 0) throw std::runtime_error("D % msm_size != 0");
     if (N > D) throw std::runtime_error("tLookup: the table is longer than the witness");   // phase 2 binds log2(N) of the log2(D) variables
     last_transcript = SumcheckTranscript();
+    hot_entries_ = 0;                       // what THIS proof does with the occupied entries
+    cold_elements_ = 0;
+    hot_reused_ = false;
 
     fr_t* d_beta = grape_host::device_scalar(beta);
     // A = 1/(S + beta): read from B where the witness matches its table entry (every element of

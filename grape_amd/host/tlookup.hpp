@@ -35,11 +35,14 @@ public:
     // The commitment is the same group element either way.
     void set_indexed_commit(bool on) { indexed_commit_ = on; }
     // Where no table over every entry fits (mapping lookups), A is committed through a table of
-    // the entries that occur at least `n` times in the witness, built for that proof (0 = the
-    // break-even count, 1.8 times the row length).  What the last prove() did is reported below.
+    // the entries that occur at least `n` times in the witness (0 = the break-even count, 1.8 times
+    // the row length), built by the first proof that needs it and kept: a later proof uses the rows
+    // again unless its elements outside them would cost more than new rows.  What the last prove()
+    // did is reported below (hot_rows_reused: it found its rows in place).
     void set_hot_min_count(uint n) { hot_min_count_ = n; }
     uint hot_entries() const { return hot_entries_; }
     uint64_t cold_elements() const { return cold_elements_; }
+    bool hot_rows_reused() const { return hot_reused_; }
 
 protected:
     Fr run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
@@ -63,7 +66,17 @@ protected:
     uint hot_min_count_ = 0;
     uint hot_entries_ = 0;
     uint64_t cold_elements_ = 0;
+    bool hot_reused_ = false;
     bool commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& hyrax);
+    // Rows B[t]*G_i of the entries that were occupied in an earlier witness, with their slot
+    // assignment: B is fixed for the object's life (the reference keeps one lookup object for all
+    // layers of a model, test/llm.cu:57-64), so the rows serve later proofs as long as they cover
+    // the witness well enough.
+    affine_t* hot_table_ = nullptr;
+    int* hot_slot1_ = nullptr;          // entry -> slot + 1 (0 = no row), T.size entries
+    uint hot_rows_ = 0, hot_cols_ = 0;
+    Hyrax* hot_for_ = nullptr;
+    void drop_hot_rows();
     affine_t* scaled_table_ = nullptr;  // B[t]*G_i, built on first use
     uint scaled_cols_ = 0;
     Hyrax* scaled_for_ = nullptr;

@@ -259,6 +259,12 @@ int grape_tlookup_inverse_by_table(uint32_t *d_A, const uint32_t *d_S, const int
  */
 int grape_tlookup_hot_select(const uint32_t *d_hist, uint32_t len, uint32_t min_count, uint32_t max_hot, int32_t *d_slot1,
                              uint32_t *d_hot_list, uint64_t *info, grape_stream_t stream);
+/* A slot assignment kept from an earlier witness of the same table (the rows of B[t]*G_i it stands
+ * for are kept with it): *cold_elements (HOST; the call synchronises) = number of elements of the
+ * witness counted in d_hist whose entry has no slot in d_slot1, i.e. what would have to be
+ * committed as full-width scalars if the rows were used again.  No counterpart in the reference. */
+int grape_tlookup_hot_coverage(const uint32_t *d_hist, uint32_t len, const int32_t *d_slot1, uint64_t *cold_elements,
+                               grape_stream_t stream);
 /* out[i] = d_slot1[d_idx1[i] - 1] (0 when d_idx1[i] is 0 or above len). */
 int grape_tlookup_hot_index(int32_t *d_out, const int32_t *d_idx1, size_t n, const int32_t *d_slot1, uint32_t len,
                             grape_stream_t stream);

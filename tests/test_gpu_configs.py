@@ -224,14 +224,15 @@ def test_configs4_softmax_mapping_lookup_through_occupied_entries(ops, host, gen
     host.set_indexed_commit(True)
     dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
     dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
-    tr, sc, com_a, n_hot, n_cold = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    tr, sc, com_a, n_hot, n_cold, reused = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    assert not reused
     counts = np.bincount(S_in.astype(np.int64) - low, minlength=N)
     thr = int(1.8 * 4096) + 1
     assert n_hot == int((counts >= thr).sum()) and n_hot > 100
     assert n_cold == int(counts[counts < thr].sum()) and 0 < n_cold < D // 5
     # the plain path on the same witness
     host.set_indexed_commit(False)
-    tr2, sc2, com_a2, h2, c2 = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    tr2, sc2, com_a2, h2, c2, _ = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
     host.set_indexed_commit(True)
     assert h2 == 0 and c2 == 0
     assert_same(com_a, com_a2, "com(A): occupied-entry table == full-width commitment")

@@ -420,6 +420,60 @@ def test_cpp_reference_programs_run(ops, tmp_path):
     assert "programs_flow OK" in res.stdout
 
 
+def test_tlookup_mapping_keeps_its_rows_between_proofs(ops, host, gens):
+    """a mapping lookup object proves several witnesses (the reference keeps one object for all layers):
+    the rows B[t]*G_i built for the first are used again while they cover the witness, and are
+    rebuilt when the occupied entries have moved; com(A) and the transcript always equal those of
+    the plain full-width path"""
+    import torch
+    hg, dg = gens
+    logN, low, msm = 12, -2048, 64
+    N, D = 1 << logN, 1 << 13
+    rng = np.random.default_rng(771)
+    fmap = rng.integers(-1000, 1000, size=N).astype(np.int32)
+    table = ops.g1_table_gen(dg[:msm].contiguous(), 256)
+    alpha, r, u, v = rand_fr(1, 772), rand_fr(1, 773), rand_fr(13, 774), rand_fr(13, 775)
+
+    def witness(centre, seed):
+        g = np.random.default_rng(seed)
+        s = np.clip(np.rint(g.normal(centre, 6.0, size=D)), low, low + N - 1).astype(np.int32)
+        spread = g.random(D) < 0.05
+        s[spread] = g.integers(low, low + N, size=int(spread.sum()))
+        return s
+
+    def prove(s_in, indexed=True):
+        host.set_indexed_commit(indexed)
+        dSi = ops.fr_from_i32(torch.from_numpy(s_in).cuda())
+        dSo = ops.fr_from_i32(torch.from_numpy(fmap[s_in - low]).cuda())
+        out = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, msm, 1, msm)
+        host.set_indexed_commit(True)
+        return out
+
+    w1, w2, w3 = witness(0.0, 1), witness(0.0, 2), witness(700.0, 3)
+    tr1, sc1, com1, hot1, cold1, reused1 = prove(w1)
+    assert not reused1 and hot1 > 0 and cold1 > 0
+    tr1b, sc1b, com1b, hot1b, cold1b, reused1b = prove(w1)
+    assert reused1b and hot1b == hot1 and cold1b == cold1
+    assert_same(com1b, com1, "same witness, rows in place")
+    assert_same(tr1b, tr1, "transcript")
+    # another witness on the same entries: the rows serve it, its own elements outside them are counted
+    tr2, sc2, com2, hot2, cold2, reused2 = prove(w2)
+    assert reused2 and hot2 == hot1
+    slot = np.bincount(w1.astype(np.int64) - low, minlength=N) >= int(1.8 * msm) + 1
+    assert cold2 == int((~slot[w2.astype(np.int64) - low]).sum())
+    tr2p, sc2p, com2p, h, c, _ = prove(w2, indexed=False)
+    assert h == 0 and c == 0
+    assert_same(com2, com2p, "com(A) through kept rows == full-width commitment")
+    assert_same(tr2, tr2p, "transcript")
+    # the occupied entries have moved: the kept rows cover almost nothing and are replaced
+    tr3, sc3, com3, hot3, cold3, reused3 = prove(w3)
+    assert not reused3 and hot3 > 0
+    tr3p, sc3p, com3p, _, _, _ = prove(w3, indexed=False)
+    assert_same(com3, com3p, "com(A) after the rows were rebuilt")
+    assert_same(tr3, tr3p, "transcript")
+    assert prove(w3)[5]
+
+
 @pytest.mark.parametrize("hot_min_count,pad", [(0, False), (1, False), (40, False), (300, False), (40, True)])
 def test_tlookup_mapping_commits_A_through_occupied_entries(ops, host, gens, hot_min_count, pad):
     """com(A) of a mapping lookup through a per-proof table of the entries that occur often: the
@@ -455,7 +509,7 @@ def test_tlookup_mapping_commits_A_through_occupied_entries(ops, host, gens, hot
     table = ops.g1_table_gen(dg[:msm].contiguous(), 256)
     dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
     dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
-    tr, sc, com_a, n_hot, n_cold = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, msm, 1, msm,
+    tr, sc, com_a, n_hot, n_cold, _ = host.tlookup_mapping_prove_ex(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, msm, 1, msm,
                                                                  hot_min_count=hot_min_count)
     assert_same(tr, wtr, "transcript")
     assert_same(sc, wsc, "S(v)")
