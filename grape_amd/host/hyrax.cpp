@@ -298,6 +298,11 @@ void Hyrax::release_scaled_table(affine_t* table) {
     grape_free(table);
 }
 
+bool Hyrax::owns_scaled_table(const affine_t* table) const {
+    auto it = scaled_registry().find(table);
+    return it != scaled_registry().end() && it->second.first == this;
+}
+
 affine_t* Hyrax::commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len, int* d_flag) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;

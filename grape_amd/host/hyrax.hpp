@@ -68,6 +68,9 @@ public:
     // frees a table that build_scaled_table returned and gives its bytes back to the budget of the
     // Hyrax object that built it, if that object still exists
     static void release_scaled_table(affine_t* table);
+    // is `table` one that THIS object built and still accounts for?  (false once the object that
+    // built it is gone, even if a new object sits at the same address)
+    bool owns_scaled_table(const affine_t* table) const;
     // idx_plus1[j] = idx_j + 1 (0 = contributes nothing); rows of N*com_scale, affine output.
     affine_t* commit_indexed_affine(int* idx_plus1, uint size, uint N, affine_t* scaled_table, uint ncols, uint len, int* d_flag = nullptr);
 

@@ -97,7 +97,7 @@ bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& h
     // rows kept from an earlier proof: used again when the elements they leave out (20 additions
     // each instead of one) cost less than building rows anew (rowlen entries of 20 additions and a
     // normalisation per row)
-    if (hot_table_ && (hot_for_ != &hyrax || hot_cols_ != rowlen)) drop_hot_rows();
+    if (hot_table_ && (hot_for_ != &hyrax || hot_cols_ != rowlen || !hyrax.owns_scaled_table(hot_table_))) drop_hot_rows();
     if (hot_table_ && hot_min_count_ == 0) {
         check(grape_tlookup_hot_coverage(d_hist_, N, hot_slot1_, &cold, nullptr), "grape_tlookup_hot_coverage");
         if ((double)cold * 19.0 <= (double)hot_rows_ * rowlen * 23.0) hot_reused_ = true;
@@ -295,7 +295,8 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         commit_time += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     };
     timed([&] {
-        if (indexed_commit_ && index_known_ && (scaled_for_ != &hyrax || scaled_cols_ < rowlen)) {
+        if (indexed_commit_ && index_known_ &&
+            (scaled_for_ != &hyrax || scaled_cols_ < rowlen || (scaled_table_ && !hyrax.owns_scaled_table(scaled_table_)))) {
             Hyrax::release_scaled_table(scaled_table_);
             scaled_table_ = hyrax.build_scaled_table(B, rowlen);   // nullptr when over budget
             scaled_cols_ = scaled_table_ ? rowlen : 0;
