@@ -163,6 +163,41 @@ int main(int argc, char** argv) {
         }
         require(rejected, "out-of-range witness was not rejected");
 
+        // ---- a lookup object outlives the Hyrax object whose table it holds: with another Hyrax object
+        // (other generators, possibly at the same address) it builds its table again, and the commitment
+        // of A it leaves is the new object's commitment of 1/(S + beta)
+        {
+            h_s[5] = (int)((5 * 37 + 11) % 1024) - 512;
+            require(grape_memcpy_h2d(d_s, h_s.data(), sizeof(int) * D, nullptr) == 0, "h2d");
+            tLookupRange kept(-512, 1024);
+            {
+                Hyrax first(layer_num, npoints / com_scale, points, cpu_points[0]);
+                FrTensor Sa(D, d_s), Aa(D);
+                kept.prove(Sa, Aa, v2, first, N, commit_time);
+            }
+            affine_t* points2 = nullptr;
+            require(grape_malloc((void**)&points2, sizeof(affine_t) * 256 * npoints) == 0, "grape_malloc");
+            std::vector<bn128> cpu_points2 = precompute_generators(npoints, 256, points2);
+            require(!(cpu_points2[0] == cpu_points[0]), "second generator set equals the first");
+            {
+                Hyrax second(layer_num, npoints / com_scale, points2, cpu_points2[0]);
+                FrTensor Sb(D, d_s), Ab(D);
+                kept.prove(Sb, Ab, v2, second, N, commit_time);
+                FrTensor A_ref(D, d_s);
+                A_ref += 1024;                  // beta is the table size
+                A_ref.inverse();
+                affine_t* want = second.commit_affine(A_ref, D, N);
+                const uint arows = D / N / com_scale;
+                require(kept.com_A_rows == arows, "rows of com(A)");
+                std::vector<unsigned char> got_b(sizeof(affine_t) * arows), want_b(sizeof(affine_t) * arows);
+                require(grape_memcpy_d2h(got_b.data(), kept.com_A, got_b.size(), nullptr) == 0, "d2h");
+                require(grape_memcpy_d2h(want_b.data(), want, want_b.size(), nullptr) == 0, "d2h");
+                require(got_b == want_b, "com(A) after the Hyrax object changed is not the new object's commitment");
+                grape_free(want);
+            }
+            grape_free(points2);
+        }
+
         // ---- Fr_partial_me: the fold without compaction leaves value (o, g) at o * c * w + g
         {
             const uint c = 6, w = 5, outer = 3, n = outer * c * w;     // an odd tail in the second round
