@@ -495,7 +495,9 @@ def witness_workload(args):
     layer_mads = float(T) * D * (4 * D + 3 * F) + 2.0 * T * T * D
     if on_matrix_cores:
         int8_ops = 2.0 * planes_a * planes_b * mads
-        roofline = {"bound": "mfma", "kernel": "wit_matmul_mfma_kernel<%d,%d> (%d x %d x %d, int8 byte planes)" % (planes_a, planes_b, T, F, D),
+        # the library takes its 128 x 128 tile kernel when the product has a tile per CU
+        kname = "wit_matmul_mfma_big_kernel" if ((T + 127) // 128) * ((F + 127) // 128) >= 256 else "wit_matmul_mfma_kernel"
+        roofline = {"bound": "mfma", "kernel": "%s<%d,%d> (%d x %d x %d, int8 byte planes)" % (kname, planes_a, planes_b, T, F, D),
                     "achieved": int8_ops / (kern_ms * 1e-3) / 1e12, "peak": 5000.0, "unit": "TOP/s",
                     "frac": int8_ops / (kern_ms * 1e-3) / 1e12 / 5000.0, "traffic": None, "kernel_ms": kern_ms,
                     "plane_split_ms": split_ms,

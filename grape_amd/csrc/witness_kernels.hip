@@ -174,12 +174,15 @@ __global__ void __launch_bounds__(kBlock) wit_matmul_simple_kernel(MatmulArgs p,
 // recombined as 64-bit integers in the epilogue and rescaled like in the kernel above.
 //
 // Workgroup tile 64 (rows of a) x 128 (rows of b), K step 64 bytes; four waves, each 32 x 64 (two
-// MFMA tiles); LDS rows are padded to 80 bytes so that 16 consecutive rows' 16-byte fragments
-// fall in disjoint banks; the next K step travels through registers while this one multiplies.
+// MFMA tiles); the 16-byte chunks of an LDS row are permuted by the row number so that fragment
+// reads and staging writes are both free of bank conflicts; the next K step travels through
+// registers while this one multiplies.  Products with at least one 128 x 128 tile per CU take
+// the eight-wave kernel further down.
 // ------------------------------------------------------------------------------------------------
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
-constexpr int kMfTN = 64, kMfTM = 128, kMfK = 64, kMfLd = 80;
+constexpr int kMfTN = 64, kMfTM = 128, kMfK = 64, kMfLd = 64;
+constexpr int kBgT = 128;      // rows of a and rows of b per workgroup of the large-tile kernel
 
 // largest magnitude of n values (n a multiple of 4, 16-byte aligned), folded into *out with an atomic maximum
 __global__ void __launch_bounds__(kBlock) wit_maxabs_kernel(uint32_t* out, const int32_t* x, size_t n) {
@@ -249,33 +252,60 @@ struct MfmaArgs {
     uint32_t N, M, Kp;
     int64_t scale;
     int shift, transpose_out;
-    uint32_t tiles_m;
+    uint32_t tiles_n, tiles_m;
     uint32_t* status;
 };
+
+// Which tile a workgroup takes.  Workgroups are dealt to the eight XCDs in turn, so workgroup b is the
+// (b / 8)-th of XCD b % 8; every XCD gets a contiguous run of the tile order, and the order walks
+// panels of eight tile columns row by row: the 64 workgroups an XCD runs at a time then share the
+// operand rows of 8 x 8 tiles (a step's distinct bytes are an eighth of what they request) and find
+// them in that XCD's L2 instead of streaming whole rows of tiles past it.
+__device__ __forceinline__ void mfma_tile_of(uint32_t b, uint32_t nb, uint32_t tiles_n, uint32_t tiles_m, uint32_t& tn, uint32_t& tm) {
+    constexpr uint32_t W = 8;
+    const uint32_t x = b & 7u, per = nb >> 3, extra = nb & 7u;
+    uint32_t l = x * per + (x < extra ? x : extra) + (b >> 3);
+    const uint32_t full = tiles_m / W, in_full = full * tiles_n * W;
+    if (l < in_full) {
+        const uint32_t pnl = l / (tiles_n * W), r = l - pnl * tiles_n * W;
+        tn = r / W;
+        tm = pnl * W + (r - tn * W);
+    } else {
+        l -= in_full;
+        const uint32_t wr = tiles_m - full * W;
+        tn = l / wr;
+        tm = full * W + (l - tn * wr);
+    }
+}
 
 template <int PA, int PB>
 __global__ void __launch_bounds__(256, 2) wit_matmul_mfma_kernel(MfmaArgs p) {
     constexpr int G = PA + PB - 1;
+    constexpr int CR = kMfK / 16;                     // 16-byte chunks in a row of one K step
+    constexpr int RP = 256 / CR;                      // rows one staging pass of the workgroup covers
+    constexpr int NA = kMfTN / RP, NB = kMfTM / RP;   // passes per plane
     __shared__ __attribute__((aligned(16))) int8_t As[PA * kMfTN * kMfLd];
     __shared__ __attribute__((aligned(16))) int8_t Bs[PB * kMfTM * kMfLd];
-    uint32_t bid = blockIdx.x;
-    const uint32_t nb = gridDim.x;
-    if ((nb & 7u) == 0) bid = (bid & 7u) * (nb >> 3) + (bid >> 3);
-    const uint32_t tn = bid / p.tiles_m, tm = bid - tn * p.tiles_m;
+    uint32_t tn, tm;
+    mfma_tile_of(blockIdx.x, gridDim.x, p.tiles_n, p.tiles_m, tn, tm);
     const uint32_t n0 = tn * kMfTN, m0 = tm * kMfTM;
     const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
     const uint32_t wn = (wave & 1u) * 32u, wm = (wave >> 1) * 64u;
 
-    // staging: 16-byte chunks; a: row t/4, chunk t%4 of every plane; b: rows (t + 256 h)/4, h = 0, 1
-    // named registers (planes beyond PA / PB are never touched)
-    uint4 sa0, sa1, sa2 = make_uint4(0, 0, 0, 0), sb00, sb01, sb10, sb11, sb20 = make_uint4(0, 0, 0, 0), sb21 = make_uint4(0, 0, 0, 0);
-    const uint32_t ra = (n0 + (t >> 2) < p.N) ? n0 + (t >> 2) : p.N - 1;
-    const uint32_t rb0 = (m0 + (t >> 2) < p.M) ? m0 + (t >> 2) : p.M - 1;
-    const uint32_t rb1 = (m0 + 64u + (t >> 2) < p.M) ? m0 + 64u + (t >> 2) : p.M - 1;
-    const uint32_t ck = 16u * (t & 3u);
-    const int8_t* ga = p.a + (size_t)ra * p.Kp + ck;
-    const int8_t* gb0 = p.b + (size_t)rb0 * p.Kp + ck;
-    const int8_t* gb1 = p.b + (size_t)rb1 * p.Kp + ck;
+    // staging: thread t carries chunk t % CR of rows t / CR + RP h of every plane (fully unrolled: registers)
+    const uint32_t lr = t / CR, ck = 16u * (t % CR);
+    v4i_t sa[PA][NA], sb[PB][NB];
+    const int8_t *ga[NA], *gb[NB];
+#pragma unroll
+    for (int h = 0; h < NA; h++) {
+        const uint32_t r = n0 + lr + RP * h;
+        ga[h] = p.a + (size_t)(r < p.N ? r : p.N - 1) * p.Kp + ck;
+    }
+#pragma unroll
+    for (int h = 0; h < NB; h++) {
+        const uint32_t r = m0 + lr + RP * h;
+        gb[h] = p.b + (size_t)(r < p.M ? r : p.M - 1) * p.Kp + ck;
+    }
     const size_t pla = (size_t)p.N * p.Kp, plb = (size_t)p.M * p.Kp;     // plane strides
     v16i_t acc[G][2];
 #pragma unroll
@@ -285,59 +315,50 @@ __global__ void __launch_bounds__(256, 2) wit_matmul_mfma_kernel(MfmaArgs p) {
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[g][tt][i] = 0;
 
-    const uint32_t frow = lane & 31u, fk = 16u * (lane >> 5);
-#define WIT_LD16(ptr) (*reinterpret_cast<const uint4*>(ptr))
-#define WIT_ST16(arr, row, v) (*reinterpret_cast<uint4*>(&arr[(row) * kMfLd + ck]) = (v))
-    sa0 = WIT_LD16(ga);
-    sa1 = WIT_LD16(ga + pla);
-    if (PA > 2) sa2 = WIT_LD16(ga + 2 * pla);
-    sb00 = WIT_LD16(gb0);
-    sb01 = WIT_LD16(gb1);
-    sb10 = WIT_LD16(gb0 + plb);
-    sb11 = WIT_LD16(gb1 + plb);
-    if (PB > 2) {
-        sb20 = WIT_LD16(gb0 + 2 * plb);
-        sb21 = WIT_LD16(gb1 + 2 * plb);
-    }
-    const uint32_t lr = t >> 2;
+    // LDS rows are kMfK bytes with no padding; the 16-byte chunk c of row r sits at chunk position
+    // c ^ ((r / RL) % CR) (RL = rows per 128 bytes), so that eight consecutive rows' equal chunks
+    // (the fragment reads) and the consecutive chunks of one or two rows (the staging writes) both
+    // spread over all banks
+    constexpr int RL = 8 / CR;
+    const uint32_t frow = lane & 31u;
+    const uint32_t fx = 16u * ((lane >> 5) ^ ((frow / RL) % CR));     // fragment of k offset kk + 16 (lane / 32): byte kk ^ fx
+    const uint32_t wx = 16u * ((t % CR) ^ ((lr / RL) % CR));
+#define WIT_LD16(ptr) (*reinterpret_cast<const v4i_t*>(ptr))
+#define WIT_ST16(arr, row, v) (*reinterpret_cast<v4i_t*>(&arr[(row) * kMfLd + wx]) = (v))
+    auto fetch = [&](uint32_t k) {
+#pragma unroll
+        for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+            for (int h = 0; h < NA; h++) sa[pa][h] = WIT_LD16(ga[h] + pa * pla + k);
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int h = 0; h < NB; h++) sb[pb][h] = WIT_LD16(gb[h] + pb * plb + k);
+    };
+    fetch(0);
     for (uint32_t k0 = 0; k0 < p.Kp; k0 += kMfK) {
         __syncthreads();
-        WIT_ST16(As, lr, sa0);
-        WIT_ST16(As, kMfTN + lr, sa1);
-        if (PA > 2) WIT_ST16(As, 2 * kMfTN + lr, sa2);
-        WIT_ST16(Bs, lr, sb00);
-        WIT_ST16(Bs, 64 + lr, sb01);
-        WIT_ST16(Bs, kMfTM + lr, sb10);
-        WIT_ST16(Bs, kMfTM + 64 + lr, sb11);
-        if (PB > 2) {
-            WIT_ST16(Bs, 2 * kMfTM + lr, sb20);
-            WIT_ST16(Bs, 2 * kMfTM + 64 + lr, sb21);
-        }
+#pragma unroll
+        for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+            for (int h = 0; h < NA; h++) WIT_ST16(As, pa * kMfTN + RP * h + lr, sa[pa][h]);
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int h = 0; h < NB; h++) WIT_ST16(Bs, pb * kMfTM + RP * h + lr, sb[pb][h]);
         __syncthreads();
-        if (k0 + kMfK < p.Kp) {
-            const uint32_t kn = k0 + kMfK;
-            sa0 = WIT_LD16(ga + kn);
-            sa1 = WIT_LD16(ga + pla + kn);
-            if (PA > 2) sa2 = WIT_LD16(ga + 2 * pla + kn);
-            sb00 = WIT_LD16(gb0 + kn);
-            sb01 = WIT_LD16(gb1 + kn);
-            sb10 = WIT_LD16(gb0 + plb + kn);
-            sb11 = WIT_LD16(gb1 + plb + kn);
-            if (PB > 2) {
-                sb20 = WIT_LD16(gb0 + 2 * plb + kn);
-                sb21 = WIT_LD16(gb1 + 2 * plb + kn);
-            }
-        }
+        if (k0 + kMfK < p.Kp) fetch(k0 + kMfK);
 #pragma unroll
         for (int kk = 0; kk < kMfK; kk += 32) {
             v4i_t fa[PA], fb[PB][2];
 #pragma unroll
-            for (int pa = 0; pa < PA; pa++) fa[pa] = *reinterpret_cast<const v4i_t*>(&As[(pa * kMfTN + wn + frow) * kMfLd + kk + fk]);
+            for (int pa = 0; pa < PA; pa++)
+                fa[pa] = *reinterpret_cast<const v4i_t*>(&As[(pa * kMfTN + wn + frow) * kMfLd + (kk ^ fx)]);
 #pragma unroll
             for (int pb = 0; pb < PB; pb++)
 #pragma unroll
                 for (int tt = 0; tt < 2; tt++)
-                    fb[pb][tt] = *reinterpret_cast<const v4i_t*>(&Bs[(pb * kMfTM + wm + 32 * tt + frow) * kMfLd + kk + fk]);
+                    fb[pb][tt] = *reinterpret_cast<const v4i_t*>(&Bs[(pb * kMfTM + wm + 32 * tt + frow) * kMfLd + (kk ^ fx)]);
 #pragma unroll
             for (int pa = 0; pa < PA; pa++)
 #pragma unroll
@@ -351,6 +372,121 @@ __global__ void __launch_bounds__(256, 2) wit_matmul_mfma_kernel(MfmaArgs p) {
 #undef WIT_LD16
 #undef WIT_ST16
     // accumulator register i of lane l holds row 8 (i / 4) + 4 (l / 32) + i % 4, column l % 32
+    uint32_t bad = 0;
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) {
+        const uint32_t m = m0 + wm + 32 * tt + (lane & 31u);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t n = n0 + wn + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
+            int64_t y = 0;
+#pragma unroll
+            for (int g = G - 1; g >= 0; g--) y = y * 256 + (int64_t)acc[g][tt][i];
+            if (n < p.N && m < p.M) {
+                int32_t q, r;
+                rescale64(y, p.scale, p.shift, q, r, bad);
+                const size_t o = p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m;
+                p.q[o] = q;
+                if (p.r) p.r[o] = r;
+            }
+        }
+    }
+    if (bad) atomicOr(p.status, bad);
+}
+
+// The same product with a workgroup tile of 128 x 128 and eight waves (4 x 2, each 32 x 64 as above):
+// a workgroup then asks L2 for 40 KB per K step and 192 matrix instructions where two workgroups of
+// the kernel above ask for 56 KB, and L2 bandwidth is what the smaller tile runs into.  One workgroup
+// fills a CU (two waves per SIMD), so the K steps alternate between two LDS stages with one barrier
+// per step: a wave writes the operands of step k + 1 (in registers since step k - 1) to the other
+// stage, requests those of step k + 2, and multiplies step k.  Launched when the product has at
+// least one such tile per CU.
+template <int PA, int PB>
+__global__ void __launch_bounds__(512, 2) wit_matmul_mfma_big_kernel(MfmaArgs p) {
+    constexpr int G = PA + PB - 1;
+    constexpr int CR = kMfK / 16, RL = 8 / CR;
+    static_assert(512 / CR == kBgT, "one staging pass covers the tile's rows");
+    constexpr int kStageA = PA * kBgT * kMfK, kStageB = PB * kBgT * kMfK;
+    __shared__ __attribute__((aligned(16))) int8_t As[2 * kStageA];
+    __shared__ __attribute__((aligned(16))) int8_t Bs[2 * kStageB];
+    uint32_t tn, tm;
+    mfma_tile_of(blockIdx.x, gridDim.x, p.tiles_n, p.tiles_m, tn, tm);
+    const uint32_t n0 = tn * kBgT, m0 = tm * kBgT;
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+    const uint32_t wn = (wave & 3u) * 32u, wm = (wave >> 2) * 64u;
+
+    const uint32_t lr = t / CR, ck = 16u * (t % CR);
+    v4i_t sa[PA], sb[PB];
+    const uint32_t ra = n0 + lr, rb = m0 + lr;
+    const int8_t* ga = p.a + (size_t)(ra < p.N ? ra : p.N - 1) * p.Kp + ck;
+    const int8_t* gb = p.b + (size_t)(rb < p.M ? rb : p.M - 1) * p.Kp + ck;
+    const size_t pla = (size_t)p.N * p.Kp, plb = (size_t)p.M * p.Kp;
+    v16i_t acc[G][2];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[g][tt][i] = 0;
+
+    // same chunk positions in LDS as in the kernel above
+    const uint32_t frow = lane & 31u;
+    const uint32_t fx = 16u * ((lane >> 5) ^ ((frow / RL) % CR));
+    const uint32_t wx = 16u * ((t % CR) ^ ((lr / RL) % CR));
+#define WIT_FETCH(k)                                                                                          \
+    {                                                                                                         \
+        _Pragma("unroll") for (int pa = 0; pa < PA; pa++) sa[pa] = *reinterpret_cast<const v4i_t*>(ga + pa * pla + (k)); \
+        _Pragma("unroll") for (int pb = 0; pb < PB; pb++) sb[pb] = *reinterpret_cast<const v4i_t*>(gb + pb * plb + (k)); \
+    }
+#define WIT_STAGE(st)                                                                                         \
+    {                                                                                                         \
+        _Pragma("unroll") for (int pa = 0; pa < PA; pa++)                                                     \
+            *reinterpret_cast<v4i_t*>(&As[(st) * kStageA + (pa * kBgT + lr) * kMfK + wx]) = sa[pa];           \
+        _Pragma("unroll") for (int pb = 0; pb < PB; pb++)                                                     \
+            *reinterpret_cast<v4i_t*>(&Bs[(st) * kStageB + (pb * kBgT + lr) * kMfK + wx]) = sb[pb];           \
+    }
+    WIT_FETCH(0);
+    WIT_STAGE(0);
+    if (kMfK < p.Kp) WIT_FETCH(kMfK);
+    __syncthreads();
+    uint32_t cur = 0;
+#define WIT_FRAGS(fa_, fb_, kk)                                                                               \
+    {                                                                                                         \
+        _Pragma("unroll") for (int pa = 0; pa < PA; pa++)                                                     \
+            fa_[pa] = *reinterpret_cast<const v4i_t*>(&Ac[(pa * kBgT + wn + frow) * kMfK + ((kk) ^ fx)]);     \
+        _Pragma("unroll") for (int pb = 0; pb < PB; pb++)                                                     \
+            _Pragma("unroll") for (int tt = 0; tt < 2; tt++)                                                  \
+                fb_[pb][tt] = *reinterpret_cast<const v4i_t*>(&Bc[(pb * kBgT + wm + 32 * tt + frow) * kMfK + ((kk) ^ fx)]); \
+    }
+#define WIT_PRODUCTS(fa_, fb_)                                                                                \
+    {                                                                                                         \
+        _Pragma("unroll") for (int pa = 0; pa < PA; pa++)                                                     \
+            _Pragma("unroll") for (int pb = 0; pb < PB; pb++)                                                 \
+                _Pragma("unroll") for (int tt = 0; tt < 2; tt++)                                              \
+                    acc[pa + pb][tt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_[pa], fb_[pb][tt], acc[pa + pb][tt], 0, 0, 0); \
+    }
+    static_assert(kMfK == 64, "two fragment reads per K step");
+    for (uint32_t k0 = 0; k0 < p.Kp; k0 += kMfK) {
+        const int8_t* Ac = As + cur * kStageA;
+        const int8_t* Bc = Bs + cur * kStageB;
+        v4i_t fa0[PA], fb0[PB][2], fa1[PA], fb1[PB][2];
+        // this step's first fragments are requested before the staging writes, which would otherwise queue ahead of them
+        WIT_FRAGS(fa0, fb0, 0);
+        if (k0 + kMfK < p.Kp) {
+            WIT_STAGE(cur ^ 1u);
+            if (k0 + 2 * kMfK < p.Kp) WIT_FETCH(k0 + 2 * kMfK);
+        }
+        WIT_FRAGS(fa1, fb1, 32);
+        WIT_PRODUCTS(fa0, fb0);
+        WIT_PRODUCTS(fa1, fb1);
+        __syncthreads();
+        cur ^= 1u;
+    }
+#undef WIT_FRAGS
+#undef WIT_PRODUCTS
+#undef WIT_FETCH
+#undef WIT_STAGE
+
     uint32_t bad = 0;
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
@@ -623,13 +759,25 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
         m.q = d_q; m.r = d_r; m.a = (const int8_t*)pa; m.b = (const int8_t*)pb;
         m.N = N; m.M = M; m.Kp = Kp;
         m.scale = scale; m.shift = p.shift; m.transpose_out = p.transpose_out;
-        m.tiles_m = (M + kMfTM - 1) / kMfTM;
         m.status = p.status;
-        const unsigned grid = ((N + kMfTN - 1) / kMfTN) * m.tiles_m;
-        if (PA == 2 && PB == 2) wit_matmul_mfma_kernel<2, 2><<<grid, 256, 0, s>>>(m);
-        else if (PA == 3 && PB == 2) wit_matmul_mfma_kernel<3, 2><<<grid, 256, 0, s>>>(m);
-        else if (PA == 2 && PB == 3) wit_matmul_mfma_kernel<2, 3><<<grid, 256, 0, s>>>(m);
-        else wit_matmul_mfma_kernel<3, 3><<<grid, 256, 0, s>>>(m);
+        const uint64_t big_tiles = (uint64_t)((N + kBgT - 1) / kBgT) * ((M + kBgT - 1) / kBgT);
+        if (big_tiles >= (uint64_t)kNumCU) {
+            m.tiles_n = (N + kBgT - 1) / kBgT;
+            m.tiles_m = (M + kBgT - 1) / kBgT;
+            const unsigned grid = (unsigned)big_tiles;
+            if (PA == 2 && PB == 2) wit_matmul_mfma_big_kernel<2, 2><<<grid, 512, 0, s>>>(m);
+            else if (PA == 3 && PB == 2) wit_matmul_mfma_big_kernel<3, 2><<<grid, 512, 0, s>>>(m);
+            else if (PA == 2 && PB == 3) wit_matmul_mfma_big_kernel<2, 3><<<grid, 512, 0, s>>>(m);
+            else wit_matmul_mfma_big_kernel<3, 3><<<grid, 512, 0, s>>>(m);
+        } else {
+            m.tiles_n = (N + kMfTN - 1) / kMfTN;
+            m.tiles_m = (M + kMfTM - 1) / kMfTM;
+            const unsigned grid = m.tiles_n * m.tiles_m;
+            if (PA == 2 && PB == 2) wit_matmul_mfma_kernel<2, 2><<<grid, 256, 0, s>>>(m);
+            else if (PA == 3 && PB == 2) wit_matmul_mfma_kernel<3, 2><<<grid, 256, 0, s>>>(m);
+            else if (PA == 2 && PB == 3) wit_matmul_mfma_kernel<2, 3><<<grid, 256, 0, s>>>(m);
+            else wit_matmul_mfma_kernel<3, 3><<<grid, 256, 0, s>>>(m);
+        }
     } else if (aligned && L <= 65535) {
         dim3 grid(p.tiles_n * p.tiles_m, L);
         wit_matmul_tiled_kernel<<<grid, 256, 0, s>>>(p);

@@ -78,6 +78,29 @@ def test_matrix_core_path_over_every_plane_count(ops, amax, bmax):
     assert ops.wit_status() == 0
 
 
+@pytest.mark.parametrize("amax,bmax,K,tr", [(60, 60, 132, False), ((1 << 22) - 1, (1 << 14) - 1, 132, False), ((1 << 14) - 1, (1 << 22) - 1, 68, True),
+                                            ((1 << 22) - 1, (1 << 22) - 1, 132, False), ((1 << 20), (1 << 15) - 1, 64, True)])
+def test_matrix_core_path_with_a_tile_per_cu(ops, amax, bmax, K, tr):
+    """a product of 17 x 16 tiles of 128 x 128 (ragged on both sides) takes the large-tile kernel: one, two and
+    three K steps, every plane count, both output orders"""
+    rng = np.random.default_rng(amax % 1000 + bmax % 777 + K)
+    N, M = 2061, 1925
+    a = rng.integers(-amax, amax + 1, (N, K)).astype(np.int32)
+    b = rng.integers(-bmax, bmax + 1, (M, K)).astype(np.int32)
+    a[N - 1, :] = amax
+    b[M - 1, :] = -bmax
+    ops.wit_set_matmul_method(2)
+    try:
+        q, r = ops.wit_matmul_rescale(dev(a), dev(b), 1 << 31, transpose_out=tr)
+    finally:
+        ops.wit_set_matmul_method(0)
+    wq, wr = wo.rescale(wo.matmul_t(a, b), 1 << 31)
+    if tr:
+        wq, wr = wq.T, wr.T
+    assert np.array_equal(host(q), wq) and np.array_equal(host(r), wr)
+    assert ops.wit_status() == 0
+
+
 def test_matrix_core_path_refuses_what_it_cannot_do(ops):
     from grape_amd import _capi
     a = np.full((8, 64), 1 << 22, dtype=np.int32)      # four byte planes
