@@ -399,8 +399,11 @@ __global__ void __launch_bounds__(256, 2) wit_matmul_mfma_kernel(MfmaArgs p) {
 // the kernel above ask for 56 KB, and L2 bandwidth is what the smaller tile runs into.  One workgroup
 // fills a CU (two waves per SIMD), so the K steps alternate between two LDS stages with one barrier
 // per step: a wave writes the operands of step k + 1 (in registers since step k - 1) to the other
-// stage, requests those of step k + 2, and multiplies step k.  Launched when the product has at
-// least one such tile per CU.
+// stage, requests those of step k + 2, and multiplies step k.  The products are v_mfma_i32_16x16x64_i8
+// (2 x 4 tiles of 16 x 16 per wave, one instruction per tile, plane pair and K step): same
+// fragments, registers and operations as with the 32 x 32 x 32 form, but the chip holds a higher
+// clock under it (2.0 against 1.76 GHz in a loop of nothing else on random bytes).  Launched when
+// the product has at least one such tile per CU.
 template <int PA, int PB>
 __global__ void __launch_bounds__(512, 2) wit_matmul_mfma_big_kernel(MfmaArgs p) {
     constexpr int G = PA + PB - 1;
@@ -421,17 +424,20 @@ __global__ void __launch_bounds__(512, 2) wit_matmul_mfma_big_kernel(MfmaArgs p)
     const int8_t* ga = p.a + (size_t)(ra < p.N ? ra : p.N - 1) * p.Kp + ck;
     const int8_t* gb = p.b + (size_t)(rb < p.M ? rb : p.M - 1) * p.Kp + ck;
     const size_t pla = (size_t)p.N * p.Kp, plb = (size_t)p.M * p.Kp;
-    v16i_t acc[G][2];
+    // v_mfma_i32_16x16x64_i8: one K step is one instruction deep; 2 x 4 tiles of 16 x 16 per wave
+    v4i_t acc[G][2][4];
 #pragma unroll
     for (int g = 0; g < G; g++)
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
+        for (int ti = 0; ti < 2; ti++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc[g][tt][i] = 0;
+            for (int tj = 0; tj < 4; tj++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[g][ti][tj][i] = 0;
 
     // same chunk positions in LDS as in the kernel above
-    const uint32_t frow = lane & 31u;
-    const uint32_t fx = 16u * ((lane >> 5) ^ ((frow / RL) % CR));
+    const uint32_t frow = lane & 15u;
+    const uint32_t fx = 16u * ((lane >> 4) ^ ((frow / RL) % CR));      // lane l holds row l % 16, bytes 16 (l / 16) .. + 16 of the step
     const uint32_t wx = 16u * ((t % CR) ^ ((lr / RL) % CR));
 #define WIT_FETCH(k)                                                                                          \
     {                                                                                                         \
@@ -450,62 +456,86 @@ __global__ void __launch_bounds__(512, 2) wit_matmul_mfma_big_kernel(MfmaArgs p)
     if (kMfK < p.Kp) WIT_FETCH(kMfK);
     __syncthreads();
     uint32_t cur = 0;
-#define WIT_FRAGS(fa_, fb_, kk)                                                                               \
-    {                                                                                                         \
-        _Pragma("unroll") for (int pa = 0; pa < PA; pa++)                                                     \
-            fa_[pa] = *reinterpret_cast<const v4i_t*>(&Ac[(pa * kBgT + wn + frow) * kMfK + ((kk) ^ fx)]);     \
-        _Pragma("unroll") for (int pb = 0; pb < PB; pb++)                                                     \
-            _Pragma("unroll") for (int tt = 0; tt < 2; tt++)                                                  \
-                fb_[pb][tt] = *reinterpret_cast<const v4i_t*>(&Bc[(pb * kBgT + wm + 32 * tt + frow) * kMfK + ((kk) ^ fx)]); \
-    }
-#define WIT_PRODUCTS(fa_, fb_)                                                                                \
-    {                                                                                                         \
-        _Pragma("unroll") for (int pa = 0; pa < PA; pa++)                                                     \
-            _Pragma("unroll") for (int pb = 0; pb < PB; pb++)                                                 \
-                _Pragma("unroll") for (int tt = 0; tt < 2; tt++)                                              \
-                    acc[pa + pb][tt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa_[pa], fb_[pb][tt], acc[pa + pb][tt], 0, 0, 0); \
-    }
-    static_assert(kMfK == 64, "two fragment reads per K step");
+    static_assert(kMfK == 64, "a K step is one matrix instruction deep");
     for (uint32_t k0 = 0; k0 < p.Kp; k0 += kMfK) {
         const int8_t* Ac = As + cur * kStageA;
         const int8_t* Bc = Bs + cur * kStageB;
-        v4i_t fa0[PA], fb0[PB][2], fa1[PA], fb1[PB][2];
-        // this step's first fragments are requested before the staging writes, which would otherwise queue ahead of them
-        WIT_FRAGS(fa0, fb0, 0);
-        if (k0 + kMfK < p.Kp) {
-            WIT_STAGE(cur ^ 1u);
-            if (k0 + 2 * kMfK < p.Kp) WIT_FETCH(k0 + 2 * kMfK);
+        // this step's fragments are requested before the staging writes, which would otherwise queue ahead of them
+        v4i_t fa[PA][2];
+#pragma unroll
+        for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++)
+                fa[pa][ti] = *reinterpret_cast<const v4i_t*>(&Ac[(pa * kBgT + wn + 16 * ti + frow) * kMfK + fx]);
+        if constexpr (PA + PB < 6) {
+            v4i_t fb[PB][4];
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int tj = 0; tj < 4; tj++)
+                    fb[pb][tj] = *reinterpret_cast<const v4i_t*>(&Bc[(pb * kBgT + wm + 16 * tj + frow) * kMfK + fx]);
+            if (k0 + kMfK < p.Kp) {
+                WIT_STAGE(cur ^ 1u);
+                if (k0 + 2 * kMfK < p.Kp) WIT_FETCH(k0 + 2 * kMfK);
+            }
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+                for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+                    for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                        for (int tj = 0; tj < 4; tj++)
+                            acc[pa + pb][ti][tj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[pa][ti], fb[pb][tj], acc[pa + pb][ti][tj], 0, 0, 0);
+        } else {
+            // three planes on both sides: the fragments of b one tile column at a time, or the 160 accumulator
+            // registers and 18 fragments do not fit
+            if (k0 + kMfK < p.Kp) {
+                WIT_STAGE(cur ^ 1u);
+                if (k0 + 2 * kMfK < p.Kp) WIT_FETCH(k0 + 2 * kMfK);
+            }
+#pragma unroll
+            for (int tj = 0; tj < 4; tj++) {
+                v4i_t fb[PB];
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++) fb[pb] = *reinterpret_cast<const v4i_t*>(&Bc[(pb * kBgT + wm + 16 * tj + frow) * kMfK + fx]);
+#pragma unroll
+                for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+                    for (int pa = 0; pa < PA; pa++)
+#pragma unroll
+                        for (int pb = 0; pb < PB; pb++)
+                            acc[pa + pb][ti][tj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[pa][ti], fb[pb], acc[pa + pb][ti][tj], 0, 0, 0);
+            }
         }
-        WIT_FRAGS(fa1, fb1, 32);
-        WIT_PRODUCTS(fa0, fb0);
-        WIT_PRODUCTS(fa1, fb1);
         __syncthreads();
         cur ^= 1u;
     }
-#undef WIT_FRAGS
-#undef WIT_PRODUCTS
 #undef WIT_FETCH
 #undef WIT_STAGE
 
+    // accumulator register i of lane l holds row 4 (l / 16) + i, column l % 16 of its tile
     uint32_t bad = 0;
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++) {
-        const uint32_t m = m0 + wm + 32 * tt + (lane & 31u);
+    for (int ti = 0; ti < 2; ti++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const uint32_t n = n0 + wn + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
-            int64_t y = 0;
+        for (int tj = 0; tj < 4; tj++) {
+            const uint32_t m = m0 + wm + 16 * tj + (lane & 15u);
 #pragma unroll
-            for (int g = G - 1; g >= 0; g--) y = y * 256 + (int64_t)acc[g][tt][i];
-            if (n < p.N && m < p.M) {
-                int32_t q, r;
-                rescale64(y, p.scale, p.shift, q, r, bad);
-                const size_t o = p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m;
-                p.q[o] = q;
-                if (p.r) p.r[o] = r;
+            for (int i = 0; i < 4; i++) {
+                const uint32_t n = n0 + wn + 16 * ti + 4 * (lane >> 4) + i;
+                int64_t y = 0;
+#pragma unroll
+                for (int g = G - 1; g >= 0; g--) y = y * 256 + (int64_t)acc[g][ti][tj][i];
+                if (n < p.N && m < p.M) {
+                    int32_t q, r;
+                    rescale64(y, p.scale, p.shift, q, r, bad);
+                    const size_t o = p.transpose_out ? (size_t)m * p.N + n : (size_t)n * p.M + m;
+                    p.q[o] = q;
+                    if (p.r) p.r[o] = r;
+                }
             }
         }
-    }
     if (bad) atomicOr(p.status, bad);
 }
 
