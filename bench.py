@@ -488,7 +488,7 @@ def witness_workload(args):
         ops.wit_matmul_rescale(h2, weights["gate"], 1 << 20)
         ms.append(ops.profile_last())
     ops.profile_enable(False)
-    on_matrix_cores = len(ms[-1]) == 2
+    on_matrix_cores = len(ms[-1]) == 3      # plane split, the host's read of the operand magnitudes, the product
     kern_ms = float(np.median([m[-1] for m in ms[1:]]))
     split_ms = float(np.median([m[0] for m in ms[1:]])) if on_matrix_cores else 0.0
     mads = float(T) * D * F

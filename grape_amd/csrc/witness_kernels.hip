@@ -184,26 +184,39 @@ typedef int v16i_t __attribute__((ext_vector_type(16)));
 constexpr int kMfTN = 64, kMfTM = 128, kMfK = 64, kMfLd = 64;
 constexpr int kBgT = 128;      // rows of a and rows of b per workgroup of the large-tile kernel
 
-// largest magnitude of n values (n a multiple of 4, 16-byte aligned), folded into *out with an atomic maximum
-__global__ void __launch_bounds__(kBlock) wit_maxabs_kernel(uint32_t* out, const int32_t* x, size_t n) {
-    const int4* x4 = reinterpret_cast<const int4*>(x);
-    const size_t n4 = n / 4;
-    const size_t stride = (size_t)gridDim.x * kBlock;
+// planes[p][row][k] for k < Kp (zero beyond K) for three planes, and the largest magnitude of x folded
+// into *mx with an atomic maximum (one per workgroup): the caller learns from it how many of the
+// planes are non-zero.  A thread takes 4 consecutive k at a time, the grid strides over the tensor.
+__global__ void __launch_bounds__(kBlock) wit_split_kernel(int8_t* planes, uint32_t* mx, const int32_t* x, uint32_t R, uint32_t K, uint32_t Kp) {
+    const uint32_t per_row = Kp / 4;
+    const size_t total = (size_t)R * per_row, stride = (size_t)gridDim.x * kBlock;
+    const size_t plane = (size_t)R * Kp;
     uint32_t m = 0;
-    auto fold = [&](const int4& v) {
-        const int32_t e[4] = {v.x, v.y, v.z, v.w};
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += stride) {
+        const uint32_t row = (uint32_t)(idx / per_row), k = 4u * (uint32_t)(idx - (size_t)row * per_row);
+        int32_t v[4] = {0, 0, 0, 0};
+        if (k < K) {      // K is a multiple of 4
+            const int4 t = *reinterpret_cast<const int4*>(x + (size_t)row * K + k);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t a = e[j] < 0 ? 0u - (uint32_t)e[j] : (uint32_t)e[j];
+            const uint32_t a = v[j] < 0 ? 0u - (uint32_t)v[j] : (uint32_t)v[j];
             m = a > m ? a : m;
         }
-    };
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    for (; i + 3 * stride < n4; i += 4 * stride) {      // four loads in flight
-        const int4 v0 = x4[i], v1 = x4[i + stride], v2 = x4[i + 2 * stride], v3 = x4[i + 3 * stride];
-        fold(v0); fold(v1); fold(v2); fold(v3);
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int32_t d = (int32_t)(int8_t)(v[j] & 0xff);
+                // (v - d) is a multiple of 256; the subtraction cannot wrap (|d| <= 128 towards zero)
+                v[j] = (int32_t)(((int64_t)v[j] - d) >> 8);
+                w |= ((uint32_t)d & 0xffu) << (8 * j);
+            }
+            *reinterpret_cast<uint32_t*>(planes + p * plane + (size_t)row * Kp + k) = w;
+        }
     }
-    for (; i < n4; i += stride) fold(x4[i]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
         const uint32_t o = __shfl_xor(m, off, 64);
@@ -216,31 +229,7 @@ __global__ void __launch_bounds__(kBlock) wit_maxabs_kernel(uint32_t* out, const
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int w = 1; w < kBlock / 64; w++) m = sh[w] > m ? sh[w] : m;
-        if (m) atomicMax(out, m);
-    }
-}
-
-// planes[p][row][k] for k < Kp (zero beyond K); one thread per 4 consecutive k
-__global__ void __launch_bounds__(kBlock) wit_split_kernel(int8_t* planes, const int32_t* x, uint32_t R, uint32_t K, uint32_t Kp, int P) {
-    const size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t per_row = Kp / 4;
-    if (idx >= (size_t)R * per_row) return;
-    const uint32_t row = (uint32_t)(idx / per_row), k = 4u * (uint32_t)(idx - (size_t)row * per_row);
-    int32_t v[4] = {0, 0, 0, 0};
-    if (k < K) {      // K is a multiple of 4
-        const int4 t = *reinterpret_cast<const int4*>(x + (size_t)row * K + k);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    }
-    for (int p = 0; p < P; p++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int32_t d = (int32_t)(int8_t)(v[j] & 0xff);
-            // (v - d) is a multiple of 256; the subtraction cannot wrap (|d| <= 128 towards zero)
-            v[j] = (int32_t)(((int64_t)v[j] - d) >> 8);
-            w |= ((uint32_t)d & 0xffu) << (8 * j);
-        }
-        *reinterpret_cast<uint32_t*>(planes + ((size_t)p * R + row) * Kp + k) = w;
+        if (m) atomicMax(mx, m);
     }
 }
 
@@ -743,26 +732,38 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
     int rc = status_word(&p.status, s);
     if (rc) return rc;
     const bool aligned = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_a) | reinterpret_cast<uintptr_t>(d_b)) & 15) == 0;
-    // matrix-core path: one batch, aligned rows, operands of at most three byte planes each
+    // matrix-core path: one batch, aligned rows, operands of at most three byte planes each.  The split into
+    // three planes also reports the operands' largest magnitudes; planes that turn out to be zero are left
+    // out of the product, and operands beyond three planes go to the multiply-add kernel.
     bool use_mfma = false;
     int PA = 0, PB = 0;
     const uint32_t Kp = (K + kMfK - 1) / kMfK * kMfK;
+    void *pa = nullptr, *pb = nullptr;
     if (g_matmul_method != 1 && L == 1 && aligned && (g_matmul_method == 2 || (uint64_t)N * M * K >= ((uint64_t)1 << 26))) {
         void* mx;
         rc = scratch_get(kSlotMisc, 64, &mx, s);
         if (rc) return rc;
+        rc = scratch_get(kSlotWitA, (size_t)3 * N * Kp, &pa, s);
+        if (rc) return rc;
+        rc = scratch_get(kSlotWitB, (size_t)3 * M * Kp, &pb, s);
+        if (rc) return rc;
         uint32_t* d_mx = (uint32_t*)mx;
+        if (profiling()) {
+            profile_begin();
+            profile_mark(s);
+        }
         wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx);
         wit_status_clear_kernel<<<1, 1, 0, s>>>(d_mx + 1);
-        const size_t na = (size_t)N * K, nbb = (size_t)M * K;
-        // K is a multiple of 4, so both element counts are; at least 8 vectors of 4 per thread, at most 1024 workgroups
-        const size_t ga_ = (na / 4 + kBlock * 8 - 1) / (kBlock * 8), gb_ = (nbb / 4 + kBlock * 8 - 1) / (kBlock * 8);
-        wit_maxabs_kernel<<<(unsigned)(ga_ < 1024 ? ga_ : 1024), kBlock, 0, s>>>(d_mx, d_a, na);
-        wit_maxabs_kernel<<<(unsigned)(gb_ < 1024 ? gb_ : 1024), kBlock, 0, s>>>(d_mx + 1, d_b, nbb);
+        // at least 8 groups of 4 per thread, at most 2048 workgroups (one atomic each)
+        const size_t ga_ = ((size_t)N * (Kp / 4) + kBlock * 8 - 1) / (kBlock * 8), gb_ = ((size_t)M * (Kp / 4) + kBlock * 8 - 1) / (kBlock * 8);
+        wit_split_kernel<<<(unsigned)(ga_ < 2048 ? ga_ : 2048), kBlock, 0, s>>>((int8_t*)pa, d_mx, d_a, N, K, Kp);
+        wit_split_kernel<<<(unsigned)(gb_ < 2048 ? gb_ : 2048), kBlock, 0, s>>>((int8_t*)pb, d_mx + 1, d_b, M, K, Kp);
         GRAPE_LAUNCH_CHECK();
+        if (profiling()) profile_mark(s);
         uint32_t h_mx[2] = {0, 0};
         GRAPE_HIP_CHECK(hipMemcpyAsync(h_mx, d_mx, sizeof(h_mx), hipMemcpyDeviceToHost, s));
         GRAPE_HIP_CHECK(hipStreamSynchronize(s));
+        if (profiling()) profile_mark(s);      // intervals: the split, the host's read of the magnitudes, the product
         PA = planes_for(h_mx[0]);
         PB = planes_for(h_mx[1]);
         if (PA < 2) PA = 2;
@@ -771,20 +772,11 @@ int grape_wit_matmul_rescale(int32_t* d_q, int32_t* d_r, const int32_t* d_a, con
         use_mfma = PA <= 3 && PB <= 3 && (uint64_t)Kp * pmin < 131072;   // a group stays below 2^31
     }
     GRAPE_REQUIRE(!(g_matmul_method == 2 && !use_mfma), "the matrix-core path needs one batch, K a multiple of 4, 16-byte aligned rows and operands below 2^22");
-    if (profiling()) {
+    if (profiling() && !use_mfma) {
         profile_begin();
         profile_mark(s);
     }
     if (use_mfma) {
-        void *pa, *pb;
-        rc = scratch_get(kSlotWitA, (size_t)PA * N * Kp, &pa, s);
-        if (rc) return rc;
-        rc = scratch_get(kSlotWitB, (size_t)PB * M * Kp, &pb, s);
-        if (rc) return rc;
-        wit_split_kernel<<<blocks_for((size_t)N * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pa, d_a, N, K, Kp, PA);
-        wit_split_kernel<<<blocks_for((size_t)M * (Kp / 4)), kBlock, 0, s>>>((int8_t*)pb, d_b, M, K, Kp, PB);
-        GRAPE_LAUNCH_CHECK();
-        if (profiling()) profile_mark(s);
         MfmaArgs m;
         m.q = d_q; m.r = d_r; m.a = (const int8_t*)pa; m.b = (const int8_t*)pb;
         m.N = N; m.M = M; m.Kp = Kp;
