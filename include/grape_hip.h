@@ -425,7 +425,8 @@ int grape_wit_matmul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, con
  * matrix-core products of signed byte planes (this path reads the operands' ranges back and so
  * synchronises the stream).  method 0 = choose (matrix cores from 2^26 multiply-adds), 1 = multiply-add
  * kernels only, 2 = matrix cores or GRAPE_EINVAL.  With grape_profile_enable, grape_profile_last()
- * gives [0] the product kernel, or [0] the plane split and [1] the product kernel on the matrix cores. */
+ * gives [0] the product kernel, or, on the matrix cores, [0] the plane split of both operands (which also
+ * finds their ranges), [1] the host's read of the ranges and [2] the product kernel. */
 int grape_wit_set_matmul_method(int method);
 /* q, r of a[i] * b[i] (d_r may be NULL).  model.py:673-675. */
 int grape_wit_elemul_rescale(int32_t *d_q, int32_t *d_r, const int32_t *d_a, const int32_t *d_b, size_t n, int64_t scale,
