@@ -9,9 +9,9 @@ LIB_PATH = os.path.join(_HERE, "host", "libgrape_host_bn254.so" if CURVE == "bn2
 G1W = FP_WORDS              # u64 words of an affine point (2 coordinates of FP_WORDS / 2)
 _lib = None
 
-NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_prove_matmul", "grape_host_prove_elemul",
+NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_set_input_format", "grape_host_prove_matmul", "grape_host_prove_elemul",
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
-         "grape_host_hyrax_open_verify", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove", "grape_host_tlookup_mapping_prove_ex",
+         "grape_host_hyrax_open_verify", "grape_host_hyrax_open", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove", "grape_host_tlookup_mapping_prove_ex",
          "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
          "grape_host_generate_data", "grape_host_single_commit", "grape_host_layer_witness_new", "grape_host_layer_witness_generate",
          "grape_host_layer_witness_names", "grape_host_layer_witness_tensor", "grape_host_layer_witness_save",
@@ -49,6 +49,12 @@ def load():
 
 def set_indexed_commit(on):
     load().grape_host_set_indexed_commit(1 if on else 0)
+
+
+def set_input_format(fmt):
+    """0: tensor arguments are field elements (default); 1: int32 values that each call embeds itself"""
+    if load().grape_host_set_input_format({"fr": 0, "i32": 1}[fmt]) != 0:
+        raise HostError("unknown input format")
 
 
 def last_commit_seconds():
@@ -154,11 +160,23 @@ def hyrax_open_verify(d_tensor, size, N, d_table, npoints, eval_point, c, com_sc
     return res, bool(ok.value)
 
 
-def tlookup_range_prove(dS, D, low, length, alpha, u, v, d_table, npoints, com_scale, msm_size, want_commitments=False):
+def hyrax_open(d_tensor, size, N, d_table, npoints, eval_point, c, com_scale=16, layer_num=1):
+    """Hyrax::open of a copy of the tensor; returns the opened evaluation"""
+    lib = load()
+    pt = _fr(eval_point)
+    c = _fr(c, 1)
+    res = np.zeros(4, dtype=np.uint64)
+    _check(lib.grape_host_hyrax_open(_dp(d_tensor), size, N, _dp(d_table), npoints, com_scale, layer_num, _hp(pt), pt.shape[0],
+                                     _hp(c), _hp(res)))
+    return res
+
+
+def tlookup_range_prove(dS, D, low, length, alpha, u, v, d_table, npoints, com_scale, msm_size, want_commitments=False,
+                        want_m=True):
     lib = load()
     alpha, u, v = _fr(alpha, 1), _fr(u), _fr(v)
     size = 1 << max(0, (length - 1).bit_length())
-    m = np.zeros((size, 4), dtype=np.uint64)
+    m = np.zeros((size, 4), dtype=np.uint64) if want_m else None
     tr = np.zeros((64, 4, 4), dtype=np.uint64)
     nr = ctypes.c_uint32(0)
     sc = np.zeros(4, dtype=np.uint64)

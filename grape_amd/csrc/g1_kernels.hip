@@ -944,6 +944,28 @@ using geom::reduce_lanes_log2;
 // largest size the GPU tests run; the host classes split longer tensors by rows.
 constexpr size_t kMaxCommitScalars = (size_t)1 << 28;
 
+// Row reduction of `rows` rows of `nparts` partial sums each.  With few rows the chain of additions of
+// the reducing lanes is what takes the time (one row of 4096 partial sums on 64 lanes: 64 + 6 additions
+// one after the other, 1 ms), so those go through two levels: every 256 partial sums of a row become
+// one (4 + 6 additions, one wave per group), then the groups of a row are folded (`tmp`: one
+// accumulator of 256 bytes per group).
+constexpr uint32_t kReduceGroup = 256;
+static size_t reduce_tmp_bytes(size_t rows, uint32_t nparts) { return rows * (size_t)(nparts / kReduceGroup + 1) * (4 * kPartialWords); }
+template <bool AFFINE>
+static void launch_reduce(uint32_t* out, const uint32_t* partial, size_t rows, uint32_t nparts, uint32_t lg_lpr, uint32_t* tmp, hipStream_t s) {
+    if (tmp && lg_lpr == 6 && nparts >= 4 * kReduceGroup && nparts % kReduceGroup == 0) {
+        const uint32_t groups = nparts / kReduceGroup;
+        commit_reduce_kernel<false><<<(unsigned)(rows * groups), 64, 0, s>>>(tmp, partial, rows * groups, kReduceGroup, 6);
+        uint32_t lg2 = 0;
+        while ((1u << lg2) < groups && lg2 < 6) lg2++;
+        const size_t per_wave = (size_t)64 >> lg2;
+        commit_reduce_kernel<AFFINE><<<(unsigned)((rows + per_wave - 1) / per_wave), 64, 0, s>>>(out, tmp, rows, groups, lg2);
+        return;
+    }
+    const size_t per_wave = (size_t)64 >> lg_lpr;
+    commit_reduce_kernel<AFFINE><<<(unsigned)((rows + per_wave - 1) / per_wave), 64, 0, s>>>(out, partial, rows, nparts, lg_lpr);
+}
+
 template <bool FR>
 static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
                             uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st, int* caller_flag = nullptr) {
@@ -966,17 +988,18 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
     const uint32_t lg_lpr = plan.lg_lpr, nseg = plan.nseg, seg = plan.seg;
     const size_t slab = plan.slab, partial_bytes = plan.partial_bytes;
     void* ws;
-    int rc = scratch_get(kSlotMsm, partial_bytes + 64, &ws, s);
+    const size_t tmp_bytes = reduce_tmp_bytes(slab, nseg * 64);
+    int rc = scratch_get(kSlotMsm, partial_bytes + tmp_bytes + 64, &ws, s);
     if (rc) return rc;
+    uint32_t* red_tmp = (uint32_t*)((char*)ws + partial_bytes);
     // the digit-range flag: the call's own (cleared here, read back at the end), or one the caller
     // owns, has cleared and reads when it likes - then nothing here waits for the stream
-    int* err = caller_flag ? caller_flag : (int*)((char*)ws + partial_bytes);
+    int* err = caller_flag ? caller_flag : (int*)((char*)ws + partial_bytes + tmp_bytes);
     if (!caller_flag) {
         rc = zero_fill(err, sizeof(int), s);
         if (rc) return rc;
     }
     const size_t elem_words = FR ? 8 : 1;
-    const size_t rows_per_wave = (size_t)64 >> lg_lpr;
     profile_begin();
     for (size_t r0 = 0; r0 < rows; r0 += slab) {
         const size_t nr = rows - r0 < slab ? rows - r0 : slab;
@@ -984,8 +1007,7 @@ static int commit_wide_impl(uint32_t* out, const void* scalars, size_t size, uin
         profile_mark(s);
         commit_wide_kernel<FR><<<blocks_for(nr * nseg * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, N, c, nw, K, err);
         profile_mark(s);
-        commit_reduce_kernel<true><<<(unsigned)((nr + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), (const uint32_t*)ws, nr,
-                                                                                                 nseg * 64, lg_lpr);
+        launch_reduce<true>(out + r0 * (size_t)(2 * FW), (const uint32_t*)ws, nr, nseg * 64, lg_lpr, red_tmp, s);
         profile_mark(s);
     }
     GRAPE_LAUNCH_CHECK();
@@ -1023,17 +1045,18 @@ static int commit_ref_impl(uint32_t* out, const void* scalars, size_t size, uint
     if (slab > rows) slab = rows;
     const size_t partial_bytes = slab * nwin * nseg * 64 * (size_t)(4 * kPartialWords);
     void* ws;
-    int rc = scratch_get(kSlotMsm, partial_bytes + slab * nwin * (size_t)(8 * FW) + 64, &ws, s);
+    const size_t sums_bytes = (slab * nwin * (size_t)(8 * FW) + 255) & ~(size_t)255;
+    int rc = scratch_get(kSlotMsm, partial_bytes + sums_bytes + reduce_tmp_bytes(slab * nwin, nseg * 64) + 64, &ws, s);
     if (rc) return rc;
     uint32_t* sums = (uint32_t*)((char*)ws + partial_bytes);
+    uint32_t* red_tmp = (uint32_t*)((char*)ws + partial_bytes + sums_bytes);
     const size_t elem_words = FR ? 8 : 1;
     for (size_t r0 = 0; r0 < rows; r0 += slab) {
         const size_t nr = rows - r0 < slab ? rows - r0 : slab;
         const size_t units = nr * nwin * nseg;
         const uint32_t* sc = (const uint32_t*)scalars + r0 * rowlen * elem_words;
         commit_ref28_kernel<FR><<<blocks_for(units * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, npoints);
-        const size_t per_wave = (size_t)64 >> lg_lpr, rw = nr * nwin;
-        commit_reduce_kernel<true><<<(unsigned)((rw + per_wave - 1) / per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rw, nseg * 64, lg_lpr);
+        launch_reduce<true>(sums, (const uint32_t*)ws, nr * nwin, nseg * 64, lg_lpr, red_tmp, s);
         commit_ref_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, nwin);
     }
     GRAPE_LAUNCH_CHECK();
@@ -1166,10 +1189,10 @@ int grape_commit_fr_strided(uint32_t* out, const uint32_t* scalars, size_t size,
     const size_t partial_bytes = slab * J * nseg * 64 * (size_t)(4 * kPartialWords);
     const size_t sums_bytes = slab * J * (size_t)(4 * kPartialWords);
     void* ws;
-    int rc = scratch_get(kSlotMsm, partial_bytes + sums_bytes, &ws, s);
+    int rc = scratch_get(kSlotMsm, partial_bytes + sums_bytes + reduce_tmp_bytes(slab * J, nseg * 64), &ws, s);
     if (rc) return rc;
     uint32_t* sums = (uint32_t*)((char*)ws + partial_bytes);
-    const size_t rows_per_wave = (size_t)64 >> lg_lpr;
+    uint32_t* red_tmp = (uint32_t*)((char*)ws + partial_bytes + sums_bytes);
     profile_begin();
     for (size_t r0 = 0; r0 < rows; r0 += slab) {
         const size_t nr = rows - r0 < slab ? rows - r0 : slab;
@@ -1177,8 +1200,7 @@ int grape_commit_fr_strided(uint32_t* out, const uint32_t* scalars, size_t size,
         profile_mark(s);
         commit_strided_kernel<<<blocks_for(nr * J * nseg * 64), kBlock, 0, s>>>((uint32_t*)ws, sc, rowlen, nr, seg, nseg, table, N, c, nw, K, J, nsets);
         profile_mark(s);
-        const size_t rj = nr * J;
-        commit_reduce_kernel<false><<<(unsigned)((rj + rows_per_wave - 1) / rows_per_wave), 64, 0, s>>>(sums, (const uint32_t*)ws, rj, nseg * 64, lg_lpr);
+        launch_reduce<false>(sums, (const uint32_t*)ws, nr * J, nseg * 64, lg_lpr, red_tmp, s);
         strided_horner_kernel<<<blocks_for(nr, 64), 64, 0, s>>>(out + r0 * (size_t)(2 * FW), sums, nr, J, c);
         profile_mark(s);
     }

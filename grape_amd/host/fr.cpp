@@ -188,3 +188,29 @@ G1 operator*(const Fr& k, const G1& pt) {
     }
     return G1(grape::xyzz_to_jac(acc));
 }
+
+G1FixedBase::G1FixedBase(const G1& base) : table_((size_t)kWindows * kPerWindow) {
+    grape::G1Xyzz b = grape::jac_to_xyzz(base.p);
+    for (int w = 0; w < kWindows; w++) {
+        grape::G1Xyzz acc = b;
+        for (int k = 1; k <= kPerWindow; k++) {
+            table_[(size_t)w * kPerWindow + (k - 1)] = acc;
+            grape::xyzz_add(acc, b);                       // after the last entry: 2^kBits * b, the next window's base
+        }
+        b = acc;
+    }
+}
+
+G1 G1FixedBase::mul(const Fr& k) const {
+    uint32_t w[9];
+    k.to_plain(w);
+    w[8] = 0;
+    grape::G1Xyzz acc = grape::G1Xyzz::inf();
+    for (int i = 0; i < kWindows; i++) {
+        const int bit = i * kBits;
+        const uint64_t two = (uint64_t)w[bit >> 5] | ((uint64_t)w[(bit >> 5) + 1] << 32);
+        const uint32_t d = (uint32_t)(two >> (bit & 31)) & (uint32_t)kPerWindow;
+        if (d) grape::xyzz_add(acc, table_[(size_t)i * kPerWindow + (d - 1)]);
+    }
+    return G1(grape::xyzz_to_jac(acc));
+}

@@ -70,8 +70,14 @@ static Fr fr_from(const uint32_t* p) {
     return x;
 }
 static void fr_to(uint32_t* p, const Fr& x) { std::memcpy(p, &x, 32); }
+static int g_input_format = 0;      // 0: field elements, 1: int32 values (grape_host_set_input_format)
 static FrTensor tensor_from_device(const uint32_t* d, uint32_t n, uint32_t capacity = 0) {
     FrTensor t(capacity > n ? capacity : n);
+    if (g_input_format == 1) {
+        // as the reference's drivers hand integers to a tensor: FrTensor::get_data (test/llm.cu:77)
+        t.get_data(n, reinterpret_cast<int*>(const_cast<uint32_t*>(d)));
+        return t;
+    }
     t.set_size(n);
     grape_host::check(grape_memcpy_d2d(t.gpu_data, d, 32 * (size_t)n, nullptr), "grape_memcpy_d2d");
     return t;
@@ -92,6 +98,11 @@ double grape_host_last_prove_seconds(void) { return g_last_prove_s; }
 double grape_host_last_commit_seconds(void) { return g_last_commit_s; }
 void grape_host_seed(uint64_t seed) { Fr::seed(seed); }
 void grape_host_set_indexed_commit(int on) { g_indexed_commit = on != 0; }
+int grape_host_set_input_format(int fmt) {
+    if (fmt != 0 && fmt != 1) return 1;
+    g_input_format = fmt;
+    return 0;
+}
 
 int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int N, int M, int K, const uint32_t* u, uint32_t nu,
                             const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
@@ -193,6 +204,19 @@ int grape_host_hyrax_open_verify(const uint32_t* d_tensor, uint32_t size, uint32
     fr_to(result, proof.result);
     *verified = hyrax.verify(proof, com, pt, fr_from(c), size, N) ? 1 : 0;
     grape_free(com);
+    GUARD_END
+}
+
+// Hyrax::open alone (src/Hyrax.cu:237-305): the opening a prover runs after a sub-proof, timed like the provers
+int grape_host_hyrax_open(const uint32_t* d_tensor, uint32_t size, uint32_t N, const uint32_t* d_table, uint32_t npoints,
+                          uint32_t com_scale, uint32_t layer_num, const uint32_t* eval_point, uint32_t n_eval, const uint32_t* c,
+                          uint32_t* result) {
+    GUARD_BEGIN
+    Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, layer_num);
+    FrTensor t = tensor_from_device(d_tensor, size);
+    ProveTimer timer;
+    Hyrax_proof proof = hyrax.open(t, vec_from(eval_point, n_eval), fr_from(c), size, N);
+    fr_to(result, proof.result);
     GUARD_END
 }
 

@@ -18,6 +18,11 @@ void grape_host_seed(uint64_t seed);
 /* tLookupRange objects made by the wrappers below commit A through the scaled table (1) or as a
  * full-width tensor (0); default 1. */
 void grape_host_set_indexed_commit(int on);
+/* What the tensor arguments d_A, d_B, d_T, d_S, d_S_in, d_S_out, d_tensor of the calls below point
+ * to: 0 (default) field elements of 32 bytes; 1 int32 values, which the call embeds into a tensor of
+ * its own with FrTensor::get_data as the reference's drivers do (test/llm.cu:77).  Returns 1 for an
+ * unknown format. */
+int grape_host_set_input_format(int fmt);
 
 /* prove_matmul on copies of the device tensors d_A (L*N*K) and d_B (L*M*K).  transcript receives
  * 4 coefficients (8 u32 each) per round. */
@@ -49,6 +54,11 @@ int grape_host_hyrax_commit_fr(const uint32_t *d_scalars, uint32_t size, uint32_
 int grape_host_hyrax_open_verify(const uint32_t *d_tensor, uint32_t size, uint32_t N, const uint32_t *d_table,
                                  uint32_t npoints, uint32_t com_scale, uint32_t layer_num, const uint32_t *eval_point,
                                  uint32_t n_eval, const uint32_t *c, uint32_t *result, int *verified);
+/* Hyrax::open alone on a copy of the tensor: result = the opened evaluation.  The time of the
+ * opening (between two device synchronisations) is what grape_host_last_prove_seconds() returns. */
+int grape_host_hyrax_open(const uint32_t *d_tensor, uint32_t size, uint32_t N, const uint32_t *d_table, uint32_t npoints,
+                          uint32_t com_scale, uint32_t layer_num, const uint32_t *eval_point, uint32_t n_eval,
+                          const uint32_t *c, uint32_t *result);
 
 /*
  * tLookupRange(low, len).prove on a copy of the witness d_S (D elements).  alpha, u, v are host

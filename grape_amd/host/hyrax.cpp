@@ -241,8 +241,14 @@ bool Hyrax::ensure_strided_table(uint rowlen, bool build) {
 }
 
 void Hyrax::commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build) {
-    // one row only (an opening's blinding row): a table that is already there is used, none is built for it
-    if (ensure_strided_table(rowlen, may_build)) {
+    // one row only (an opening's blinding row): a table that is already there is used, none is built for it,
+    // and the per-window table is preferred - its 20 additions per scalar are nothing for one row, while the
+    // strided table's (J-1)*c doublings per row are a chain of half a millisecond on one lane
+    const bool single = size == rowlen;
+    if (single && ensure_fr_table(rowlen, false)) {
+        const WideTable& t = fr_table_;
+        check(grape_commit_fr(W(out), W(scalars), size, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, nullptr), "grape_commit_fr");
+    } else if (ensure_strided_table(rowlen, may_build)) {
         const StridedTable& t = fr_strided_;
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
                   return grape_commit_fr_strided(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.J, t.nsets, nullptr);
@@ -398,7 +404,8 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
 
     d.partial_eval(d.size, eval_point, new_N, 0, 1);
     Fr sum_ad = grape_host::download(d.gpu_data);
-    bn128 commit_ad = sum_ad * G;
+    if (!G_multiples_) G_multiples_.reset(new G1FixedBase(G));
+    bn128 commit_ad = G_multiples_->mul(sum_ad);
 
     affine_t host_com_d;
     check(grape_memcpy_d2h(&host_com_d, com_d_dev, sizeof(affine_t), nullptr), "d2h");

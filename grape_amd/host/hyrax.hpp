@@ -1,5 +1,6 @@
 // Hyrax row commitments: the interface of the reference's include/Hyrax.cuh:57-86.
 #pragma once
+#include <memory>
 #include <vector>
 #include "ec_operation.hpp"
 #include "fr_tensor.hpp"
@@ -110,5 +111,6 @@ private:
     bool int16_ok_ = true;
     size_t scaled_bytes_ = 0;
     std::vector<Fr> last_open_point_;
+    std::unique_ptr<G1FixedBase> G_multiples_;      // built by the first opening
     size_t table_budget_ = (size_t)128 << 30;
 };
