@@ -79,6 +79,7 @@ SIGNATURES = {
     "grape_tlookup_poly_sum": [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_round_sums": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p],
     "grape_tlookup_mb_sums": [c_void_p, c_void_p, c_size_t, c_void_p, c_void_p],
+    "grape_tlookup_table_round": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p],
     "grape_eq_table": [c_void_p, c_void_p, c_u32, c_void_p],
     "grape_eq_table_halve": [c_void_p, c_size_t, c_void_p],
     "grape_fr_fold_msb_multi": [ctypes.POINTER(c_void_p), c_u32, c_size_t, c_void_p, c_void_p],

@@ -119,22 +119,146 @@ __device__ __forceinline__ void block_sum(Fr* vals, Fr* lds) {
     }
 }
 
-// NV interleaved partial arrays: partial[b*NV + k]; out[k] = sum_b partial[b*NV + k]
-template <int NV>
-__global__ void __launch_bounds__(kBlock) final_sum_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
-    __shared__ Fr lds[NV * (kBlock / 64)];
-    Fr acc[NV];
+// ---- finishing kernels: ONE workgroup adds up the partial sums that the workgroups of a round left.
+// A long round leaves up to eleven thousand partial sums per coefficient; read one at a time by 256
+// threads that is a chain of 43 dependent loads (30-60 us, as much as the whole round of a short
+// proof), so long lists go to a workgroup of 1024 threads, and every thread keeps two groups of loads
+// in flight.  (Letting the last workgroup of the round kernel do this instead - an arrival counter
+// behind a device-scope fence - was built and measured: the fence makes every workgroup write the
+// folded tensors' dirty cache lines back before it may take its ticket, and the round kernels lost
+// 5-12 % at 2^24 index pairs, more than the saved launch is worth.)
+constexpr int kFinalBlock = 1024;
+constexpr unsigned kFinalWideMin = 4 * kBlock;     // partial sums per coefficient from which the wide workgroup is used
+
+// Plain integer sum of canonical elements (nine words: room for 2^32 terms): a step of a sum tree costs
+// nine add-with-carry instead of the 24 instructions of a modular addition, and ONE reduction ends it.
+struct Sum9 {
+    uint32_t w[9];
+};
+__device__ __forceinline__ void sum9_zero(Sum9& s) {
 #pragma unroll
-    for (int k = 0; k < NV; k++) acc[k] = Fr::zero();
-    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
+    for (int i = 0; i < 9; i++) s.w[i] = 0;
+}
+__device__ __forceinline__ void sum9_add_fr(Sum9& s, const Fr& a) {
+    uint32_t c = 0;
 #pragma unroll
-        for (int k = 0; k < NV; k++) acc[k] = add(acc[k], ld_fr(partial, (size_t)b * NV + k));
+    for (int i = 0; i < 8; i++) s.w[i] = detail::adc32(s.w[i], a.v[i], c);
+    s.w[8] += c;
+}
+__device__ __forceinline__ void sum9_add(Sum9& s, const Sum9& t) {
+    uint32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < 9; i++) s.w[i] = detail::adc32(s.w[i], t.w[i], c);
+}
+__device__ __forceinline__ Sum9 shfl_down_sum9(const Sum9& a, int off) {
+    Sum9 r;
+#pragma unroll
+    for (int i = 0; i < 9; i++) r.w[i] = __shfl_down(a.w[i], off, 64);
+    return r;
+}
+// lo + hi * 2^256 mod r: lo < 2^256 < 6 r loses r up to five times, and hi * 2^256 mod r is the memory
+// form of the integer hi
+__device__ __forceinline__ Fr sum9_to_fr(const Sum9& s) {
+    Fr lo;
+#pragma unroll
+    for (int i = 0; i < 8; i++) lo.v[i] = s.w[i];
+#pragma unroll
+    for (int rep = 0; rep < 5; rep++) {
+        Fr d;
+        detail::final_sub<FrParams>(d.v, lo.v, 0);
+        lo = d;
     }
-    block_sum<NV>(acc, lds);
+    return add(lo, fr26::from_u32c(s.w[8]));
+}
+
+// tot[k] = sum over b < nblocks of partial[b*NV + k] for every k whose bit in SKIP is clear (the others
+// are left zero), valid in thread 0 of a workgroup of BLOCK threads; lds9 holds NV * (BLOCK/64) * 9 words
+template <int NV, int BLOCK, unsigned SKIP = 0>
+__device__ __forceinline__ void workgroup_totals(Fr* tot, const uint32_t* partial, unsigned nblocks, uint32_t* lds9) {
+    constexpr int NW = BLOCK / 64;
+    Sum9 s[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) sum9_zero(s[k]);
+    unsigned b = threadIdx.x;
+    for (; b + BLOCK < nblocks; b += 2 * BLOCK) {
+        Fr t0[NV], t1[NV];
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            if (SKIP & (1u << k)) continue;
+            t0[k] = ld_fr(partial, (size_t)b * NV + k);
+            t1[k] = ld_fr(partial, (size_t)(b + BLOCK) * NV + k);
+        }
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            if (SKIP & (1u << k)) continue;
+            sum9_add_fr(s[k], t0[k]);
+            sum9_add_fr(s[k], t1[k]);
+        }
+    }
+    if (b < nblocks) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            if (SKIP & (1u << k)) continue;
+            sum9_add_fr(s[k], ld_fr(partial, (size_t)b * NV + k));
+        }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        if (SKIP & (1u << k)) continue;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) sum9_add(s[k], shfl_down_sum9(s[k], off));
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < 9; i++) lds9[(k * NW + wave) * 9 + i] = s[k].w[i];
+        }
+    }
+    __syncthreads();
+    // thread k folds the waves' sums of value k and reduces it (the reductions side by side, not one
+    // after the other on one thread), then thread 0 collects the NV results
+    Fr mine = Fr::zero();
+    const int k = threadIdx.x;
+    if (k < NV && !((SKIP >> k) & 1u)) {
+        Sum9 t;
+        sum9_zero(t);
+        for (int w = 0; w < NW; w++) {
+            Sum9 o;
+#pragma unroll
+            for (int i = 0; i < 9; i++) o.w[i] = lds9[(k * NW + w) * 9 + i];
+            sum9_add(t, o);
+        }
+        mine = sum9_to_fr(t);
+    }
+    __syncthreads();
+    if (k < NV) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) lds9[k * 8 + i] = mine.v[i];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) tot[j].v[i] = lds9[j * 8 + i];
+        }
+    }
+}
+
+// NV interleaved partial arrays: partial[b*NV + k]; out[k] = sum_b partial[b*NV + k]
+template <int NV, int BLOCK = kBlock>
+__global__ void __launch_bounds__(BLOCK) final_sum_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
+    __shared__ uint32_t lds9[NV * (BLOCK / 64) * 9];
+    Fr acc[NV];
+    workgroup_totals<NV, BLOCK>(acc, partial, nblocks, lds9);
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < NV; k++) st_fr(out, k, acc[k]);
     }
+}
+template <int NV>
+static inline void launch_final_sum(uint32_t* out, const uint32_t* partial, unsigned nblocks, hipStream_t s) {
+    if (nblocks >= kFinalWideMin) final_sum_kernel<NV, kFinalBlock><<<1, kFinalBlock, 0, s>>>(out, partial, nblocks);
+    else final_sum_kernel<NV, kBlock><<<1, kBlock, 0, s>>>(out, partial, nblocks);
 }
 
 #define CHECK_PTR16(p) GRAPE_REQUIRE((p) != nullptr && (reinterpret_cast<uintptr_t>(p) & 15) == 0, #p " must be a 16-byte aligned device pointer")

@@ -500,7 +500,7 @@ int grape_fr_sum(uint32_t* out, const uint32_t* in, size_t n, grape_stream_t st)
         int rc = scratch_get(kSlotReduce, (size_t)nb * 32, &ws, s);
         if (rc) return rc;
         sum_kernel<<<nb, kBlock, 0, s>>>((uint32_t*)ws, in, n);
-        final_sum_kernel<1><<<1, kBlock, 0, s>>>(out, (const uint32_t*)ws, nb);
+        launch_final_sum<1>(out, (const uint32_t*)ws, nb, s);
     }
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;

@@ -125,15 +125,12 @@ __global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint3
 
 // Finishes a round that was summed without its middle coefficient: out = (c0, claim - 2 c0 - c2, c2),
 // and the claim of the next round, the polynomial's value at the challenge v, replaces *claim.
-__global__ void __launch_bounds__(kBlock) sumcheck2_claim_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks,
-                                                                       uint32_t* claim, const uint32_t* v) {
-    __shared__ Fr lds[3 * (kBlock / 64)];
-    Fr acc[3] = {Fr::zero(), Fr::zero(), Fr::zero()};
-    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
-        acc[0] = add(acc[0], ld_fr(partial, (size_t)b * 3));
-        acc[2] = add(acc[2], ld_fr(partial, (size_t)b * 3 + 2));
-    }
-    block_sum<3>(acc, lds);
+template <int BLOCK>
+__global__ void __launch_bounds__(BLOCK) sumcheck2_claim_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks,
+                                                                      uint32_t* claim, const uint32_t* v) {
+    __shared__ uint32_t lds9[3 * (BLOCK / 64) * 9];
+    Fr acc[3];
+    workgroup_totals<3, BLOCK, 2u>(acc, partial, nblocks, lds9);       // the middle slot is not written by the round kernel
     if (threadIdx.x == 0) {
         const Fr c0 = acc[0], c2 = acc[2];
         const Fr c1 = sub(sub(sub(ld_fr(claim, 0), c0), c0), c2);
@@ -546,10 +543,10 @@ __global__ void __launch_bounds__(kBlock) tl_poly_sum_kernel(const uint32_t* A, 
 
 // 5 sums per round: eq-weighted coefficients of (A0+tA1)(S0+beta+tS1), and plain sums of A0, A1.
 // e*A0 and e*A1 are reduced products; the three second-level products are accumulated
-// double-width over the thread's iterations and reduced once.
-__global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
-                                                          const uint32_t* eq, size_t n_out, uint32_t* partial) {
-    __shared__ Fr lds[5 * (kBlock / 64)];
+// double-width over the thread's iterations and reduced once.  This thread's share (the indices
+// t = first, first + stride, ...; at most kLogUpIters of them) is left in acc[0..4].
+__device__ __forceinline__ void tl_round_thread_sums(Fr* acc, const uint32_t* A, const uint32_t* S, const uint32_t* beta,
+                                                     const uint32_t* eq, size_t n_out, size_t first, size_t stride) {
     const Fr btc = beta ? ld_fr(beta, 0) : Fr::zero();
     const fr26::Limbs bt = fr26::pack(btc);
     fr26::Acc C0, Q, C2;
@@ -560,8 +557,7 @@ __global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, 
     fr26::Limbs sa0, sa1;
 #pragma unroll
     for (int k = 0; k < fr26::N; k++) sa0.v[k] = sa1.v[k] = 0;
-    const size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
+    for (size_t t = first; t < n_out; t += stride) {
         // operands are consumed as early as possible so that few of them are live beside the
         // three double-width accumulators
         const fr26::Limbs e16 = fr26::pack16(ld_fr(eq, t));         // limbs < 2^30: one product per column set
@@ -588,7 +584,17 @@ __global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, 
     // per iteration |Q| grows by at most 3.92 * 3 r^2 = 11.8 r^2; 16 iterations -> below 189 r^2,
     // i.e. within 5.4 r of zero after the reduction: finish_sum's window of 34 r holds with lo_r = 6
     const Fr c0 = fr26::finish_sum(C0, 4), c2 = fr26::finish_sum(C2, 4), q1 = fr26::finish_sum(Q, 6);
-    Fr acc[5] = {c0, sub(sub(q1, c0), c2), c2, fr26::limb_sum_to_fr(sa0, 0), fr26::limb_sum_to_fr(sa1, 16)};
+    acc[0] = c0;
+    acc[1] = sub(sub(q1, c0), c2);
+    acc[2] = c2;
+    acc[3] = fr26::limb_sum_to_fr(sa0, 0);
+    acc[4] = fr26::limb_sum_to_fr(sa1, 16);
+}
+__global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, const uint32_t* S, const uint32_t* beta,
+                                                          const uint32_t* eq, size_t n_out, uint32_t* partial) {
+    __shared__ Fr lds[5 * (kBlock / 64)];
+    Fr acc[5];
+    tl_round_thread_sums(acc, A, S, beta, eq, n_out, (size_t)blockIdx.x * kBlock + threadIdx.x, (size_t)gridDim.x * kBlock);
     block_sum<5>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
@@ -596,14 +602,13 @@ __global__ void __launch_bounds__(kBlock, 2) tl_round_kernel(const uint32_t* A, 
     }
 }
 
-__global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* partial) {
-    __shared__ Fr lds[3 * (kBlock / 64)];
+// the coefficient sums of (m0 + t m1)(B0 + t B1) over this thread's indices, left in acc[0..2]
+__device__ __forceinline__ void tl_mb_thread_sums(Fr* acc, const uint32_t* m, const uint32_t* B, size_t n_out, size_t first, size_t stride) {
     fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
     fr26::acc_zero(Q);
     fr26::acc_zero(C2);
-    const size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n_out; t += stride) {
+    for (size_t t = first; t < n_out; t += stride) {
         const fr26::Limbs m0 = ld_l26(m, t), b0 = ld_l26(B, t);
         const fr26::Limbs mh = ld_l26(m, t + n_out), bh = ld_l26(B, t + n_out);
         const fr26::Limbs m1 = fr26::sub(mh, m0), b1 = fr26::sub(bh, b0);
@@ -612,11 +617,47 @@ __global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const 
         fr26::mac(C2, m1, b1);
     }
     const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2), q1 = fr26::finish_sum(Q, 2);
-    Fr acc[3] = {c0, sub(sub(q1, c0), c2), c2};
+    acc[0] = c0;
+    acc[1] = sub(sub(q1, c0), c2);
+    acc[2] = c2;
+}
+__global__ void __launch_bounds__(kBlock) tl_mb_kernel(const uint32_t* m, const uint32_t* B, size_t n_out, uint32_t* partial) {
+    __shared__ Fr lds[3 * (kBlock / 64)];
+    Fr acc[3];
+    tl_mb_thread_sums(acc, m, B, n_out, (size_t)blockIdx.x * kBlock + threadIdx.x, (size_t)gridDim.x * kBlock);
     block_sum<3>(acc, lds);
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < 3; k++) st_fr(partial, (size_t)blockIdx.x * 3 + k, acc[k]);
+    }
+}
+
+// One round of the table side of a logUp proof (src/tlookup.cu:153-190: the terms over B, T and m of
+// phase 2) as ONE launch: the five sums over (B, T + beta) with the round's weights, the three sums
+// over (m, B), then the fold of the three tensors by the round's challenge - every index is read and
+// folded by the thread that owns it, so the three steps need no barrier between them.  One finishing
+// kernel adds up the workgroups' eight sums.  (The round was five launches: two sum kernels, their two
+// finishing kernels and the fold.)
+__global__ void __launch_bounds__(kBlock, 2) tl_table_round_kernel(uint32_t* B, uint32_t* T, uint32_t* m, const uint32_t* beta,
+                                                                const uint32_t* eq, size_t n_out, const uint32_t* v, uint32_t* partial) {
+    __shared__ Fr lds[8 * (kBlock / 64)];
+    const size_t first = (size_t)blockIdx.x * kBlock + threadIdx.x, stride = (size_t)gridDim.x * kBlock;
+    Fr acc[8];
+    tl_round_thread_sums(acc, B, T, beta, eq, n_out, first, stride);
+    tl_mb_thread_sums(acc + 5, m, B, n_out, first, stride);
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    for (size_t t = first; t < n_out; t += stride) {
+        uint32_t* X[3] = {B, T, m};
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const fr26::Limbs lo = ld_l26(X[j], t);
+            st_fr(X[j], t, fold1(w1, lo, fr26::sub(ld_l26(X[j], t + n_out), lo)));
+        }
+    }
+    block_sum<8>(acc, lds);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) st_fr(partial, (size_t)blockIdx.x * 8 + k, acc[k]);
     }
 }
 
@@ -729,7 +770,7 @@ static int sumcheck2_impl(uint32_t* A, uint32_t* B, uint32_t* a, uint32_t* b, ui
     } else {
         sumcheck2_kernel<COEFFS, false><<<nb, kBlock, 0, s>>>(A, B, a, b, c, in_size, out_size, v, nullptr, partial);
     }
-    if (sums) final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    if (sums) launch_final_sum<3>(sums, partial, nb, s);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
@@ -771,7 +812,8 @@ int grape_sumcheck_round2_claim(uint32_t* A, uint32_t* B, uint32_t in_size, uint
     } else {
         sumcheck2_kernel<false, false, true><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, nullptr, partial);
     }
-    sumcheck2_claim_final_kernel<<<1, kBlock, 0, s>>>(sums, partial, nb, claim, v);
+    if (nb >= kFinalWideMin) sumcheck2_claim_final_kernel<kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb, claim, v);
+    else sumcheck2_claim_final_kernel<kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb, claim, v);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
@@ -799,7 +841,7 @@ int grape_sumcheck_round2_noalloc(uint32_t* A, uint32_t* B, uint32_t in_size, ui
     } else {
         sumcheck2_kernel<false, false><<<nb, kBlock, 0, s>>>(A, B, nullptr, nullptr, nullptr, in_size, out_size, v, nullptr, partial);
     }
-    final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    launch_final_sum<3>(sums, partial, nb, s);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
@@ -1059,7 +1101,7 @@ int grape_tlookup_round_sums(const uint32_t* A, const uint32_t* S, const uint32_
     int rc = scratch_get(kSlotReduce, (size_t)nb * 5 * 32, &ws, s);
     if (rc) return rc;
     tl_round_kernel<<<nb, kBlock, 0, s>>>(A, S, beta, eq, n_out, (uint32_t*)ws);
-    final_sum_kernel<5><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
+    launch_final_sum<5>(sums, (const uint32_t*)ws, nb, s);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
@@ -1072,7 +1114,23 @@ int grape_tlookup_mb_sums(const uint32_t* m, const uint32_t* B, size_t n_out, ui
     int rc = scratch_get(kSlotReduce, (size_t)nb * 3 * 32, &ws, s);
     if (rc) return rc;
     tl_mb_kernel<<<nb, kBlock, 0, s>>>(m, B, n_out, (uint32_t*)ws);
-    final_sum_kernel<3><<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, nb);
+    launch_final_sum<3>(sums, (const uint32_t*)ws, nb, s);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_table_round(uint32_t* B, uint32_t* T, uint32_t* m, const uint32_t* beta, const uint32_t* eq, size_t n_out,
+                              const uint32_t* v, uint32_t* sums, grape_stream_t st) {
+    CHECK_PTR16(B); CHECK_PTR16(T); CHECK_PTR16(m); CHECK_PTR16(eq); CHECK_PTR16(v); CHECK_PTR16(sums);
+    if (beta) CHECK_PTR16(beta);
+    GRAPE_REQUIRE(n_out >= 1, "empty round");
+    hipStream_t s = as_stream(st);
+    const unsigned nb = reduce_grid(n_out, kLogUpIters);
+    void* ws;
+    int rc = scratch_get(kSlotReduce, (size_t)nb * 8 * 32, &ws, s);
+    if (rc) return rc;
+    tl_table_round_kernel<<<nb, kBlock, 0, s>>>(B, T, m, beta, eq, n_out, v, (uint32_t*)ws);
+    launch_final_sum<8>(sums, (const uint32_t*)ws, nb, s);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

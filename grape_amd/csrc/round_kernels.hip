@@ -59,6 +59,30 @@ __device__ __forceinline__ Fr reduce_to_fr(fr26::Acc& C, int lo_r) {
     return fr26::unpack(fr26::canon_wide(fr26::reduce(C, lo_r)));
 }
 
+// sums[0..2] = 16 * (W0, WQ - W0 - W2, W2); with PLAIN sums[3] = sum A0, sums[4] = sum A1 - sum A0
+// UNIT (weights that sum to one, A * (S + beta) = 1 everywhere): sums[0] = 1, sums[1] = -sums[2]
+template <bool PLAIN, bool UNIT>
+__device__ __forceinline__ void wround2_result(uint32_t* out, const Fr* acc) {
+    Fr w[3] = {acc[0], sub(sub(acc[1], acc[0]), acc[2]), acc[2]};
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        Fr t = w[k];
+#pragma unroll
+        for (int d = 0; d < 4; d++) t = add(t, t);
+        w[k] = t;
+    }
+    if (UNIT) {
+        w[0] = Fr::one();
+        w[1] = sub(Fr::zero(), w[2]);
+    }
+#pragma unroll
+    for (int k = 0; k < 3; k++) st_fr(out, k, w[k]);
+    if (PLAIN) {
+        st_fr(out, 3, acc[3]);
+        st_fr(out, 4, sub(acc[4], acc[3]));
+    }
+}
+
 // UNIT: the caller states that A[i] * (S[i] + beta) = 1 at every index (the first round of a logUp
 // proof, where A was made as the inverse of S + beta).  Then the constant coefficient is the sum of
 // the weights and the value at t = 1 equals it, so only the top coefficient sum_g e * dA * dS is
@@ -132,41 +156,13 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         for (int k = 0; k < NV; k++) st_fr(partial, (size_t)blockIdx.x * NV + k, acc[k]);
     }
 }
-
-// sums[0..2] = 16 * (W0, WQ - W0 - W2, W2); with PLAIN sums[3] = sum A0, sums[4] = sum A1 - sum A0
-// UNIT (weights that sum to one, A * (S + beta) = 1 everywhere): sums[0] = 1, sums[1] = -sums[2]
-template <bool PLAIN, bool UNIT = false>
-__global__ void __launch_bounds__(kBlock) wround2_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
+template <bool PLAIN, bool UNIT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK) wround2_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
     constexpr int NV = PLAIN ? 5 : 3;
-    __shared__ Fr lds[NV * (kBlock / 64)];
-    Fr acc[NV];
-#pragma unroll
-    for (int k = 0; k < NV; k++) acc[k] = Fr::zero();
-    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) {
-#pragma unroll
-        for (int k = 0; k < NV; k++) acc[k] = add(acc[k], ld_fr(partial, (size_t)b * NV + k));
-    }
-    block_sum<NV>(acc, lds);
-    if (threadIdx.x == 0) {
-        Fr w[3] = {acc[0], sub(sub(acc[1], acc[0]), acc[2]), acc[2]};
-#pragma unroll
-        for (int k = 0; k < 3; k++) {
-            Fr t = w[k];
-#pragma unroll
-            for (int d = 0; d < 4; d++) t = add(t, t);
-            w[k] = t;
-        }
-        if (UNIT) {
-            w[0] = Fr::one();
-            w[1] = sub(Fr::zero(), w[2]);
-        }
-#pragma unroll
-        for (int k = 0; k < 3; k++) st_fr(out, k, w[k]);
-        if (PLAIN) {
-            st_fr(out, 3, acc[3]);
-            st_fr(out, 4, sub(acc[4], acc[3]));
-        }
-    }
+    __shared__ uint32_t lds9[NV * (BLOCK / 64) * 9];
+    Fr tot[NV];
+    workgroup_totals<NV, BLOCK>(tot, partial, nblocks, lds9);
+    if (threadIdx.x == 0) wround2_result<PLAIN, UNIT>(out, tot);
 }
 
 // ---------------------------------------------------------------- matmul phase 1: weights per segment
@@ -310,25 +306,27 @@ int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t
     int rc = scratch_get(kSlotReduce, (size_t)nb * nv * 32, &ws, s);
     if (rc) return rc;
     uint32_t* partial = (uint32_t*)ws;
+#define GRAPE_WROUND2(B, P, U)                                                                                        \
+    do {                                                                                                              \
+        wround2_kernel<B, P, U><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);     \
+        if (nb >= kFinalWideMin) wround2_final_kernel<P, U, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb); \
+        else wround2_final_kernel<P, U, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);                               \
+    } while (0)
     if (plain_sums == 2) {
         GRAPE_REQUIRE(rowlen == rowpad && in_size == 2 * (uint64_t)n_out,
                       "the inverse-pair round needs whole pairs and unpadded rows (weights that sum to one)");
-        if (beta) wround2_kernel<true, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        else wround2_kernel<false, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        wround2_final_kernel<true, true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+        if (beta) GRAPE_WROUND2(true, true, true);
+        else GRAPE_WROUND2(false, true, true);
     } else if (beta && plain_sums) {
-        wround2_kernel<true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        wround2_final_kernel<true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+        GRAPE_WROUND2(true, true, false);
     } else if (beta) {
-        wround2_kernel<true, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        wround2_final_kernel<false><<<1, kBlock, 0, s>>>(sums, partial, nb);
+        GRAPE_WROUND2(true, false, false);
     } else if (plain_sums) {
-        wround2_kernel<false, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        wround2_final_kernel<true><<<1, kBlock, 0, s>>>(sums, partial, nb);
+        GRAPE_WROUND2(false, true, false);
     } else {
-        wround2_kernel<false, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);
-        wround2_final_kernel<false><<<1, kBlock, 0, s>>>(sums, partial, nb);
+        GRAPE_WROUND2(false, false, false);
     }
+#undef GRAPE_WROUND2
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

@@ -107,6 +107,7 @@ int scratch_get(ScratchSlot slot, size_t bytes, void** out, hipStream_t stream) 
     return GRAPE_OK;
 }
 
+
 // 16-byte-per-lane streaming copy, grid-stride
 __global__ void __launch_bounds__(256) copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

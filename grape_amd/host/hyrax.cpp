@@ -129,29 +129,33 @@ affine_t* Hyrax::commit_affine(int* tensor, uint size, uint N) {
 
 // any int32 scalars: five signed 8-bit digits per scalar through a small table, or the reference's
 // byte windows when even that table is over budget
-void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag) {
+void Hyrax::commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag, void* stream) {
+    if (!d_flag) stream = nullptr;                       // a call that waits for its result runs on the default stream
+    const affine_t* had = int32_table_.d;
     if (ensure_table(int32_table_, rowlen, 8, 5, 128)) {
+        // a table built just now was built on the default stream: another stream may read it only once it is there
+        if (stream && int32_table_.d != had) check(grape_stream_sync(nullptr), "sync");
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
                   if (d_flag)
                       return grape_commit_i32_nowait(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128,
-                                                     d_flag, nullptr);
+                                                     d_flag, stream);
                   return grape_commit_i32(W(out + r0), tensor + e0, n, rowlen, W(int32_table_.d), int32_table_.ngen, 8, 5, 128, nullptr);
               }),
               "grape_commit_i32");
     } else {
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
-                  return grape_commit_i32_ref_table(W(out + r0), tensor + e0, n, rowlen, W(g_affine), npoints, nullptr);
+                  return grape_commit_i32_ref_table(W(out + r0), tensor + e0, n, rowlen, W(g_affine), npoints, stream);
               }),
               "grape_commit_i32_ref_table");
     }
 }
 
-affine_t* Hyrax::commit_affine_i32(int* tensor, uint size, uint N, int* d_flag) {
+affine_t* Hyrax::commit_affine_i32(int* tensor, uint size, uint N, int* d_flag, void* stream) {
     check_shape(size, N);
     const uint rowlen = N * com_scale;
     affine_t* out = nullptr;
     check(grape_malloc((void**)&out, sizeof(affine_t) * (size_t)(size / rowlen)), "grape_malloc");
-    commit_i32_rows(out, tensor, size, rowlen, d_flag);
+    commit_i32_rows(out, tensor, size, rowlen, d_flag, stream);
     return out;
 }
 

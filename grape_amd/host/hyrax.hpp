@@ -50,7 +50,8 @@ public:
     // table up for this object when a value does not fit it): lookup multiplicities.
     // With d_flag (a device int the caller owns and has cleared) the call queues its kernels and returns
     // without waiting; the flag is 1 afterwards if a scalar did not fit the table's digits.
-    affine_t* commit_affine_i32(int* tensor, uint size, uint N, int* d_flag = nullptr);
+    // `stream` (a grape_stream_t; with d_flag only) is where the kernels are queued instead of the default stream.
+    affine_t* commit_affine_i32(int* tensor, uint size, uint N, int* d_flag = nullptr, void* stream = nullptr);
 
     Hyrax_proof open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
     // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
@@ -104,7 +105,7 @@ private:
     size_t table_bytes_in_use() const;
     // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
     void commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build);
-    void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag);
+    void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag, void* stream = nullptr);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;
     StridedTable fr_strided_;

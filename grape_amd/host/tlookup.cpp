@@ -192,6 +192,13 @@ struct SideChain {
         ev_begin = g_side_event[which][0];
         ev_end = g_side_event[which][1];
     }
+    // `waiter` does not start what is queued on it from now on before what `other` holds at this moment is done
+    static void order(grape_stream_t waiter, grape_stream_t other) {
+        static void* ev = nullptr;
+        if (!ev) check(grape_event_create(&ev), "grape_event_create");
+        check(grape_event_record(ev, other), "grape_event_record");
+        check(grape_stream_wait_event(waiter, ev), "grape_stream_wait_event");
+    }
     void begin() {
         check(grape_event_record(ev_begin, nullptr), "grape_event_record");
         check(grape_stream_wait_event(stream, ev_begin), "grape_stream_wait_event");
@@ -390,6 +397,21 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             vi--;
             k++;
         };
+        // the table side of phase 2: per round one launch for the five sums over (B, T), the three over
+        // (m, B) and the fold of all three, and one finishing launch
+        auto table_side = [&] {
+            uint cur_t = N;
+            for (int vt = (int)logN - 1; vt >= 0 && vt < (int)rounds; vt--) {
+                const uint kt = rounds - 1 - (uint)vt;
+                const uint half = cur_t / 2;
+                fr_t* slot = sums.gpu_data + 13 * (size_t)kt;
+                const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - kt)) - 1);
+                check(grape_tlookup_table_round(W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data), W(d_beta), W(e), half, W(d_v + vt),
+                                                W(slot + 5), side.stream),
+                      "grape_tlookup_table_round");
+                cur_t = half;
+            }
+        };
         // overlap: the commitments are queued without waiting (their digit-range flags are read after
         // the rounds have been queued too), so the chip works on them while the host issues the
         // rounds' launches; everything that needs the host to wait on the default stream (the sums
@@ -401,43 +423,39 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         // rounds (launch-bound) do run beside the commitments, on a stream of their own.
         if (overlap) {
             while (vi >= 0 && cur / 2 >= kLongRoundPairs) witness_round(nullptr);
-            witness.begin();                // waits for what is queued so far (the long rounds) - not for the commitments, queued next
-            ws = witness.stream;
+            // The table side and the commitment of m (a few rows: a short accumulation and a latency chain of a
+            // row reduction) go to the second stream now, so that they run beside the long rounds and the
+            // commitment of A instead of after them; the host gets through these launches while the chip
+            // still works on the long rounds.
             check(grape_malloc((void**)&d_flags, 2 * sizeof(int)), "grape_malloc");
             check(grape_memset_zero(d_flags, 2 * sizeof(int), nullptr), "grape_memset_zero");
-            // commit_time of this mode: what the commitment kernels take on the default stream, between two events
+            grape_free(com_A);
+            grape_free(com_m);
+            com_A = com_m = nullptr;
+            table_side();
+            const uint m_N = 1u << (Log2(N) / 2);
+            com_m_rows = N / (m_N * hyrax.com_scale);
+            const bool m_aside = d_hist_ && D < (1u << 31);
+            if (m_aside) {
+                // d_flags was cleared on the default stream: the second stream meets that point first
+                SideChain::order(side.stream, nullptr);
+                com_m = hyrax.commit_affine_i32(reinterpret_cast<int*>(d_hist_), N, m_N, d_flags + 1, side.stream);
+            }
+            witness.begin();                // waits for what is queued so far (the long rounds) - not for the commitments, queued next
+            ws = witness.stream;
+            // commit_time of this mode: what the commitment of A takes on the default stream, between two events
             check(grape_event_record(commit_events().first, nullptr), "grape_event_record");
             timed([&] {
-                grape_free(com_A);
-                grape_free(com_m);
-                com_A = com_m = nullptr;
                 com_A = hyrax.commit_indexed_affine(d_idx_, D, msm_size, scaled_table_, scaled_cols_, N, d_flags);
                 com_A_rows = D / (msm_size * hyrax.com_scale);
-                uint m_N = 1u << (Log2(N) / 2);
-                if (d_hist_ && D < (1u << 31)) com_m = hyrax.commit_affine_i32(reinterpret_cast<int*>(d_hist_), N, m_N, d_flags + 1);
-                else com_m = hyrax.commit_affine(m, N, m_N);
-                com_m_rows = N / (m_N * hyrax.com_scale);
+                if (!m_aside) com_m = hyrax.commit_affine(m, N, m_N);
             });
             check(grape_event_record(commit_events().second, nullptr), "grape_event_record");
         }
         while (vi >= 0) witness_round(ws);
-        // the table side is queued second: its many small launches reach the chip while it works on the
-        // first, long rounds of the witness side
-        {
-            uint cur_t = N;
-            for (int vi = (int)logN - 1; vi >= 0 && vi < (int)rounds; vi--) {
-                const uint k = rounds - 1 - (uint)vi;
-                const uint half = cur_t / 2;
-                fr_t* slot = sums.gpu_data + 13 * (size_t)k;
-                const fr_t* e = E.gpu_data + (((size_t)1 << (nu - 1 - k)) - 1);
-                check(grape_tlookup_round_sums(W(Bw.gpu_data), W(Tw.gpu_data), W(d_beta), W(e), half, W(slot + 5), side.stream),
-                      "grape_tlookup_round_sums");
-                check(grape_tlookup_mb_sums(W(mw.gpu_data), W(Bw.gpu_data), half, W(slot + 10), side.stream), "grape_tlookup_mb_sums");
-                uint32_t* ptrs[3] = {W(Bw.gpu_data), W(Tw.gpu_data), W(mw.gpu_data)};
-                check(grape_fr_fold_msb_multi(ptrs, 3, half, W(d_v + vi), side.stream), "grape_fr_fold_msb_multi");
-                cur_t = half;
-            }
-        }
+        // without the overlap the table side is queued last: its small launches reach the chip while it
+        // works on the first, long rounds of the witness side
+        if (!overlap) table_side();
         if (overlap) witness.end();
         side.end();                         // the default stream waits for the table side
         if (overlap) {

@@ -327,6 +327,14 @@ def tlookup_round_sums(A, S, beta, eq, n_out):
     return sums
 
 
+def tlookup_table_round(B, T, m, beta, eq, n_out, v):
+    """one launch: 5 weighted sums over (B, T + beta), 3 sums over (m, B), then B, T, m folded in place by v"""
+    lib = init()
+    sums = fr_empty(8)
+    _capi.check(lib.grape_tlookup_table_round(_p(B), _p(T), _p(m), _p(beta), _p(eq), n_out, _p(v), _p(sums), _s()))
+    return sums
+
+
 def tlookup_mb_sums(m, B, n_out):
     lib = init()
     sums = fr_empty(3)

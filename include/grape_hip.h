@@ -294,6 +294,14 @@ int grape_tlookup_round_sums(const uint32_t *d_A, const uint32_t *d_S, const uin
                              size_t n_out, uint32_t *d_sums, grape_stream_t stream);
 /* d_sums[0..2] = sums of the coefficients of (m0 + t m1)(B0 + t B1) (src/tlookup.cu:180-185). */
 int grape_tlookup_mb_sums(const uint32_t *d_m, const uint32_t *d_B, size_t n_out, uint32_t *d_sums, grape_stream_t stream);
+/*
+ * One round of the table side of the logUp sumcheck (the terms over B, T and m of tLookup_phase2,
+ * src/tlookup.cu:153-190) in one launch: d_sums[0..4] as grape_tlookup_round_sums(B, T, beta, eq),
+ * d_sums[5..7] as grape_tlookup_mb_sums(m, B), then B, T and m are folded in place by the challenge
+ * d_v as grape_fr_fold_msb_multi does (their first n_out elements are the folded tensors).
+ */
+int grape_tlookup_table_round(uint32_t *d_B, uint32_t *d_T, uint32_t *d_m, const uint32_t *d_beta, const uint32_t *d_eq,
+                              size_t n_out, const uint32_t *d_v, uint32_t *d_sums, grape_stream_t stream);
 /* e[i] = prod_j (u_j if bit_j(i) else 1 - u_j) for i < 2^nu; u is a device array of nu challenges. */
 int grape_eq_table(uint32_t *d_eq, const uint32_t *d_u, uint32_t nu, grape_stream_t stream);
 /* e'[x] = e[x] + e[x + n_out] for x < n_out: the table of the remaining variables after the

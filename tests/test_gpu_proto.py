@@ -259,6 +259,29 @@ def test_fused_round_sums_equal_reference_steps(ops):
         assert_same(mb[k], orc.fr_sum(o[k]), "m*B coefficient %d" % k)
 
 
+@pytest.mark.parametrize("n_out", [1, 3, 256, 5000, 1 << 16, (1 << 19) + 77])
+def test_table_side_round_in_one_launch_equals_its_steps(ops, n_out):
+    """grape_tlookup_table_round (sums over (B, T), sums over (m, B) and the fold of the three tensors, finished by the
+    last workgroup of the launch) against the separate entry points; two rounds in a row on one stream, so that the
+    second one finds the arrival counter as the first one left it"""
+    logh = max(1, (n_out - 1).bit_length())
+    beta, v = rand_fr(1, 163), rand_fr(2, 164)
+    eq = ops.eq_table(ops.to_dev(rand_fr(logh, 165)))
+    for rnd in range(2):
+        B, T, m = rand_fr(2 * n_out, 160 + 10 * rnd), rand_fr(2 * n_out, 161 + 10 * rnd), rand_fr(2 * n_out, 162 + 10 * rnd)
+        dB, dT, dm = ops.to_dev(B), ops.to_dev(T), ops.to_dev(m)
+        want5 = ops.fr_to_host(ops.tlookup_round_sums(dB, dT, ops.to_dev(beta), eq, n_out))[:5]
+        want3 = ops.fr_to_host(ops.tlookup_mb_sums(dm, dB, n_out))
+        fB, fT, fm = ops.to_dev(B), ops.to_dev(T), ops.to_dev(m)
+        dv = ops.to_dev(v[rnd:rnd + 1])
+        ops.fr_fold_msb_multi([fB, fT, fm], n_out, dv)
+        got = ops.fr_to_host(ops.tlookup_table_round(dB, dT, dm, ops.to_dev(beta), eq, n_out, dv))
+        assert_same(got[:5], want5, "sums over (B, T)")
+        assert_same(got[5:8], want3, "sums over (m, B)")
+        for name, a, b in (("B", dB, fB), ("T", dT, fT), ("m", dm, fm)):
+            assert_same(ops.fr_to_host(a)[:n_out], ops.fr_to_host(b)[:n_out], "folded " + name)
+
+
 def test_eq_table_and_halving(ops):
     u = rand_fr(10, 71)
     ui = br.fr_unpack(u)
