@@ -373,6 +373,7 @@ def layer_workload(args):
                    "provers_only_s": float(np.mean([r["provers_only_s"] for r in runs])),
                    "provers_breakdown_s": last["provers_breakdown_s"],
                    "step_s": [r["value"] for r in runs],
+                   "step_wall_breakdown_s": [r["wall_breakdown_s"] for r in runs],
                    "cold_s": cold["value"] if cold else None, "cold": cold,
                    "spread_s": spread["value"] if spread else None, "spread": spread,
                    "hbm_in_use_gib": (total_b - free_b) / 2**30, "hbm_total_gib": total_b / 2**30,
@@ -669,6 +670,8 @@ def rounds_workload(args):
          lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True)),
         ("wround2_kernel<beta, plain sums, inverse pair> + final (grape_wround2, first logUp round over A = 1/(S + beta))", 224, h,
          lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True, inverse_pair=True)),
+        ("wround2_kernel<beta, plain sums, middle coefficient from the claim> + final (grape_wround2, long logUp rounds after the first)", 224, h,
+         lambda: ops.wround2(A, B, beta, e, n, h, v, plain_sums=True, no_middle=True)),
         ("wround2_kernel<no beta> + final (grape_wround2, element-product round)", 224, h,
          lambda: ops.wround2(A, B, None, e, n, h, v)),
         ("tl_round_kernel + final_sum (grape_tlookup_round_sums, read only)", 160, h, lambda: ops.tlookup_round_sums(A, B, beta, e, h)),
@@ -689,6 +692,122 @@ def rounds_workload(args):
         "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["frac_of_hbm_peak"],
                      "traffic": None, "kernel": head["kernel"]},
         "kernels": out,
+        "hbm_copy": {"kernel": "copy_kernel", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "GBps": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9}}))
+    return 0
+
+
+def plumbing_workload(args):
+    """Benchmark configuration configs[0] and the reduce-type kernels the other configurations lean on.
+    configs[0]: 2^16 seeded Fr elements times a second such tensor, the full sum of the product, and the
+    Hyrax commitment of the product as a 256 x 256 matrix (256 MSMs of 256 full-width scalars) - checked
+    against the CPU oracle, which is also timed.  Then, at sizes that stream from HBM: element-wise
+    product, full sum, batched inversion (tlookup's A = 1/(S + beta)), the index + inverse-by-table pass
+    of a lookup and its LDS-counted multiplicity histogram.  Every kernel is timed with events on the
+    launch stream over `steps` launches; bytes per element are the operands read once and the result
+    written once.  One JSON line."""
+    import torch
+    import orc
+    from grape_amd import ops
+    from gpuutil import rand_fr
+    ops.init(0)
+
+    def timed(fn, steps=None):
+        steps = steps or args.steps
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    # ---- configs[0]
+    n0, side = 1 << 16, 256
+    a, b = rand_fr(n0, 101), rand_fr(n0, 102)
+    dA, dB = ops.to_dev(a), ops.to_dev(b)
+    k = rand_fr(side, 103)
+    gens = ops.g1_make_generators(k)
+    c_bits = 13
+    nw = (255 + c_bits - 1) // c_bits
+    table = ops.g1_wide_table_gen(gens, c_bits, nw, 1 << (c_bits - 1))
+    prod = ops.fr_mul(dA, dB)
+    total = ops.fr_sum(prod)
+    com = ops.commit_fr(prod, side, table, side, c_bits, nw, 1 << (c_bits - 1))
+    t0 = time.perf_counter()
+    h_prod = orc.vec2("orc_fr_vec_mul", a, b)
+    h_sum = orc.fr_sum(h_prod)
+    h_gens = orc.g1_make_generators(k)
+    t1 = time.perf_counter()
+    h_com = orc.commit_fr(h_prod, orc.g1_table(h_gens, 256), side, side)
+    t2 = time.perf_counter()
+    if not (np.array_equal(ops.fr_to_host(prod), h_prod) and np.array_equal(ops.fr_to_host(total)[0], h_sum)
+            and np.array_equal(ops.g1_to_host(com), h_com)):
+        print("bench.py: configs[0] differs from the CPU oracle", file=sys.stderr)
+        return 1
+    cfg0 = {
+        "mul_ms": timed(lambda: ops.fr_mul(dA, dB, out=prod)),
+        "sum_ms": timed(lambda: ops.fr_sum(prod)),
+        "commit_ms": timed(lambda: ops.commit_fr(prod, side, table, side, c_bits, nw, 1 << (c_bits - 1), out=com)),
+    }
+    cfg0["commit_Mpoints_per_s"] = n0 / (cfg0["commit_ms"] * 1e-3) / 1e6
+    cfg0["note"] = ("2^16 elements are launch-bound (4 MiB of operands); the commitment is 256 rows of 256 full-width scalars through "
+                    "a %d-bit per-window table (%d additions per scalar)" % (c_bits, nw))
+    cpu = {"value": n0 / (t2 - t1) / 1e6, "unit": "Mpoints/s", "cores": orc.lib().orc_num_threads(), "kind": "port",
+           "sample": "the whole of configs[0]: 256 x 256 full-width commitment %.2f s (product, sum and generators %.3f s)" % (t2 - t1, t1 - t0)}
+    del table
+
+    # ---- streaming sizes
+    lg = args.log_elems
+    n = 1 << lg
+    seeds = rand_fr(3, 104)
+    X = ops.fr_from_i32(torch.arange(n, dtype=torch.int32, device="cuda") + 1)
+    ops.fr_bcast_mul(X, ops.to_dev(seeds[0:1]), out=X)             # full-width, all non-zero
+    Y = ops.fr_from_i32(torch.arange(n, dtype=torch.int32, device="cuda") * 5 + 3)
+    ops.fr_bcast_mul(Y, ops.to_dev(seeds[1:2]), out=Y)
+    out = ops.fr_empty(n)
+    beta = ops.to_dev(seeds[2:3])
+    lgw, tab_len, low = lg - 1, 1 << 16, -(1 << 15)
+    nwit = 1 << lgw
+    wit = torch.randint(low, low + tab_len, (nwit,), dtype=torch.int32, device="cuda")
+    S = ops.fr_from_i32(wit)
+    T, Btab = ops.tlookup_init(low, tab_len, ops.to_dev(rand_fr(1, 105)))
+    idx1, A, mism = ops.tlookup_index_inverse(S, low, Btab)
+    if mism != 0:
+        print("bench.py: the witness is off its table", file=sys.stderr)
+        return 1
+    hist = torch.zeros(tab_len, dtype=torch.int32, device="cuda")
+    cases = [
+        ("ew_kernel<mul> (grape_fr_mul)", 96, n, lambda: ops.fr_mul(X, Y, out=out)),
+        ("sum_kernel + final_sum (grape_fr_sum)", 32, n, lambda: ops.fr_sum(X)),
+        ("inv_*_kernel, three-level batched inversion (grape_fr_shift_inverse, A = 1/(S + beta))", 64, n,
+         lambda: ops.fr_shift_inverse(X, beta, out=out)),
+        ("index_inverse_kernel (grape_tlookup_index_inverse: index, A = B[index])", 68, nwit,
+         lambda: ops.tlookup_index_inverse(S, low, Btab)),
+        ("hist_ranges + hist_lds<32768> + hist_merge (grape_tlookup_hist_index, 2^16 bins)", 4, nwit,
+         lambda: ops.tlookup_hist_index(idx1, tab_len, hist=hist)),
+    ]
+    kernels = []
+    for name, bytes_per, units, fn in cases:
+        ms = timed(fn)
+        gbps = bytes_per * units / (ms * 1e-3) / 1e9
+        kernels.append({"kernel": name, "bytes_per_unit": bytes_per, "units": units, "ms": ms, "GBps": gbps,
+                        "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS, "units_per_s": units / (ms * 1e-3)})
+    copy_ms = ops.bench_copy(1 << 30, 5)
+    head = kernels[1]
+    print(json.dumps({
+        "metric": "fr_sum_bandwidth", "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "configs[0] (2^16 Fr mul + sum + 256x256 Fr-path commit) and the reduce-type kernels at 2^%d elements "
+                               "(lookup kernels at 2^%d)" % (lg, lgw),
+                   "configs0": cfg0},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["frac_of_hbm_peak"],
+                     "traffic": None, "kernel": head["kernel"]},
+        "kernels": kernels,
+        "inversions_per_s": kernels[2]["units_per_s"],
+        "cpu_baseline": cpu,
         "hbm_copy": {"kernel": "copy_kernel", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "GBps": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9}}))
     return 0
 
@@ -714,11 +833,12 @@ def main():
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
     ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")
-    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "mapping", "witness", "rounds"], default="commit",
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "mapping", "witness", "rounds", "plumbing"], default="commit",
                     help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
                          "lookup: configs[3]; layer: configs[4]; mapping: the layer's softmax lookup on its own; "
                          "witness: the layer's witness generator; "
-                         "rounds: the streaming kernels of the sumcheck / logUp rounds")
+                         "rounds: the streaming kernels of the sumcheck / logUp rounds; "
+                         "plumbing: configs[0] and the reduce-type kernels (sum, batched inversion, lookup index and histogram)")
     ap.add_argument("--plain-commit", action="store_true",
                     help="mapping workload: commit A as full-width scalars instead of through its occupied entries")
     ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer and witness workloads")
@@ -731,10 +851,10 @@ def main():
         print("bench.py: this build runs the proving hot path on ONE GPU; --gpus %d is not supported "
               "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
         return 2
-    if args.workload == "rounds":
+    if args.workload in ("rounds", "plumbing"):
         args.steps = 10 if args.steps is None else args.steps
         args.warmup = 2 if args.warmup is None else args.warmup
-        return rounds_workload(args)
+        return rounds_workload(args) if args.workload == "rounds" else plumbing_workload(args)
     if args.workload == "witness":
         args.steps = 3 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
@@ -935,10 +1055,11 @@ def main():
 
 
 def layer_in_child():
-    """`bench.py --workload layer` (one warm-up layer, two timed) as a child process; returns its
+    """`bench.py --workload layer` (two warm-up layers - the cold one that builds the tables and one more, after which the
+    block cache holds every size a layer asks for - and two timed) as a child process; returns its
     figures, or the reason why there are none - the commit figure above does not depend on it."""
     import subprocess
-    cmd = [sys.executable, os.path.abspath(__file__), "--workload", "layer", "--steps", "2", "--warmup", "1"]
+    cmd = [sys.executable, os.path.abspath(__file__), "--workload", "layer", "--steps", "2", "--warmup", "2"]
     try:
         res = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
         lines = [l for l in res.stdout.splitlines() if l.startswith("{")]

@@ -65,6 +65,27 @@ __device__ __forceinline__ void foldt2(const int32_t* tab, const fr26::Limbs& lo
     out_b = fr26::foldt_finish(cb);
 }
 
+// The table fold of ONE element, rows through scalar loads as in foldt2 (for kernels whose registers
+// do not hold two sets of fold columns beside their accumulators).
+__device__ __forceinline__ Fr foldt1(const int32_t* tab, const fr26::Limbs& lo, const fr26::Limbs& d) {
+    constexpr int N = fr26::N;
+    int64_t c[N + 2];
+    c[0] = c[1] = 0;
+#pragma unroll
+    for (int k = 0; k < N; k++) c[k + 2] = (int64_t)(uint32_t)lo.v[k];
+    FoldTabPtr row[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) row[j] = (FoldTabPtr)(uintptr_t)(tab + j * N);
+    asm volatile("" : "+s"(row[0]), "+s"(row[1]));
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+#pragma unroll
+        for (int k = 0; k < N; k++) c[k] += (int64_t)d.v[j] * (int64_t)row[j][k];
+        if (j + 2 < N) asm volatile("" : "+s"(row[j + 2]) : "v"((uint32_t)c[0]));
+    }
+    return fr26::foldt_finish(c);
+}
+
 // The ten multiples of a round's challenge that the table fold multiplies by (fr26::fold_table), for
 // `count` <= 64 challenges: thread t writes the table of v[t] at tabs + 100 t.  (static: every
 // source file that launches it gets its own copy)

@@ -533,6 +533,10 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
         if (c0 + 128 < col_end) sc2 = ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, c0 + 128)];
     }
     int32_t sc0 = (!FR && s * seg + lane < col_end) ? ((const int32_t*)scalars)[geom::scalar_index(row, rowlen, s * seg + lane)] : 0;
+    // destination of the look-ahead touches: one register for the whole loop, read only after it.  (Declared
+    // inside the loop it is free again at the top of the next iteration, the compiler reuses it for an
+    // address there and has to wait for every outstanding load first - 1.5 % of the kernel's time.)
+    uint32_t touch = 0;
     for (uint32_t col = s * seg + lane; col < col_end; col += 64) {
         if (FR) {
             const Fr k = from_mont(ld_fr8((const uint32_t*)scalars, geom::scalar_index(row, rowlen, col)));
@@ -561,7 +565,6 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                 if (have_next) next_entry = geom::table_entry(0, K, magn, N, col + 64);
             }
             const uint32_t* touch_ptr = table + (size_t)kWideEntryWords * next_entry;
-            uint32_t touch = 0;
             for (uint32_t w = 0; w < nw; w++) {
                 int64_t d = v & (int64_t)mask;
                 v >>= c;                            // arithmetic shift keeps the sign
@@ -581,10 +584,10 @@ __global__ void __launch_bounds__(kBlock) commit_wide_kernel(uint32_t* partial, 
                     madd28(acc, e, neg);
                 }
             }
-            asm volatile("" ::"v"(touch));          // keeps the touch alive until here
             if (v != 0) *err_flag = 1;              // scalar does not fit nw windows
         }
     }
+    asm volatile("" ::"v"(touch));                  // keeps the touches alive until here
     st_partial28(partial, wave * 64 + lane, acc);
 }
 

@@ -61,9 +61,10 @@ __device__ __forceinline__ Fr reduce_to_fr(fr26::Acc& C, int lo_r) {
 
 // sums[0..2] = 16 * (W0, WQ - W0 - W2, W2); with PLAIN sums[3] = sum A0, sums[4] = sum A1 - sum A0
 // UNIT (weights that sum to one, A * (S + beta) = 1 everywhere): sums[0] = 1, sums[1] = -sums[2]
-template <bool PLAIN, bool UNIT>
+// NOMID (the caller takes the middle coefficient from its running claim): sums[1] = 0
+template <bool PLAIN, bool UNIT, bool NOMID>
 __device__ __forceinline__ void wround2_result(uint32_t* out, const Fr* acc) {
-    Fr w[3] = {acc[0], sub(sub(acc[1], acc[0]), acc[2]), acc[2]};
+    Fr w[3] = {acc[0], NOMID ? Fr::zero() : sub(sub(acc[1], acc[0]), acc[2]), acc[2]};
 #pragma unroll
     for (int k = 0; k < 3; k++) {
         Fr t = w[k];
@@ -87,13 +88,18 @@ __device__ __forceinline__ void wround2_result(uint32_t* out, const Fr* acc) {
 // proof, where A was made as the inverse of S + beta).  Then the constant coefficient is the sum of
 // the weights and the value at t = 1 equals it, so only the top coefficient sum_g e * dA * dS is
 // taken: one weight product and one accumulation per index instead of two and three.
-template <bool BETA, bool PLAIN, bool UNIT = false>
+// TAB: the folds go through the table of the challenge's multiples (fr26::fold_table; long rounds).
+// NOMID: the sum of the round polynomial over {0, 1} is known to the caller (the value the previous
+// round's polynomial took at its challenge), which fixes the middle coefficient: the value at t = 1
+// is not accumulated - one product and one double-width accumulator less per index.
+template <bool BETA, bool PLAIN, bool UNIT, bool TAB, bool NOMID = false>
 __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E,
                                                          uint32_t in_size, uint32_t n_out, uint32_t rowlen, uint32_t rowpad,
-                                                         const uint32_t* v, uint32_t* partial) {
+                                                         const uint32_t* v, const int32_t* __restrict__ tab, uint32_t* partial) {
     constexpr int NV = PLAIN ? 5 : 3;
     __shared__ Fr lds[NV * (kBlock / 64)];
-    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    fr26::Limbs w1;
+    if (!TAB) w1 = fr26::weight16(ld_fr(v, 0));
     fr26::Limbs bt;
     if (BETA) bt = fr26::pack(ld_fr(beta, 0));
     fr26::Acc W0, WQ, W2;
@@ -111,7 +117,6 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         const fr26::Limbs a0 = ld_l26(A, g);
         const fr26::Limbs a1 = ld_hi26(A, g, n_out, in_size);
         const fr26::Limbs da = fr26::sub(a1, a0);
-        st_fr(A, g, fold1(w1, a0, da));
         fr26::Acc T;
         fr26::Limbs ea0;
         if (!UNIT) {
@@ -126,25 +131,26 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
             sa0 = fr26::add(sa0, a0);
             sa1 = fr26::add(sa1, a1);
         }
+        st_fr(A, g, TAB ? foldt1(tab, a0, da) : fold1(w1, a0, da));
         const fr26::Limbs s0r = ld_l26(S, g);
         const fr26::Limbs s1r = ld_hi26(S, g, n_out, in_size);
         const fr26::Limbs ds = fr26::sub(s1r, s0r);
-        st_fr(S, g, fold1(w1, s0r, ds));
+        st_fr(S, g, TAB ? foldt1(tab, s0r, ds) : fold1(w1, s0r, ds));
         fr26::mac(W2, ead, ds);
         if (UNIT) {
             // W0 and WQ stay zero: the finishing kernel writes the coefficients they would give
         } else if (BETA) {
             fr26::mac(W0, ea0, fr26::add(s0r, bt));
-            fr26::mac(WQ, fr26::add(ea0, ead), fr26::add(s1r, bt));
+            if (!NOMID) fr26::mac(WQ, fr26::add(ea0, ead), fr26::add(s1r, bt));
         } else {
             fr26::mac(W0, ea0, s0r);
-            fr26::mac(WQ, fr26::add(ea0, ead), s1r);
+            if (!NOMID) fr26::mac(WQ, fr26::add(ea0, ead), s1r);
         }
     }
     // offsets: |W0| < 71 r^2 -> within 2 r, |W2| < 60 r^2 -> within 1.7 r, |WQ| < 189 r^2 -> within 5.4 r
     Fr acc[NV];
     acc[0] = reduce_to_fr(W0, 3);
-    acc[1] = reduce_to_fr(WQ, 6);
+    acc[1] = NOMID ? Fr::zero() : reduce_to_fr(WQ, 6);
     acc[2] = reduce_to_fr(W2, 3);
     if (PLAIN) {
         acc[3] = fr26::limb_sum_to_fr(sa0, 0);      // below 24 r
@@ -156,13 +162,13 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         for (int k = 0; k < NV; k++) st_fr(partial, (size_t)blockIdx.x * NV + k, acc[k]);
     }
 }
-template <bool PLAIN, bool UNIT, int BLOCK>
+template <bool PLAIN, bool UNIT, bool NOMID, int BLOCK>
 __global__ void __launch_bounds__(BLOCK) wround2_final_kernel(uint32_t* out, const uint32_t* partial, unsigned nblocks) {
     constexpr int NV = PLAIN ? 5 : 3;
     __shared__ uint32_t lds9[NV * (BLOCK / 64) * 9];
     Fr tot[NV];
-    workgroup_totals<NV, BLOCK>(tot, partial, nblocks, lds9);
-    if (threadIdx.x == 0) wround2_result<PLAIN, UNIT>(out, tot);
+    workgroup_totals<NV, BLOCK, NOMID ? 2u : 0u>(tot, partial, nblocks, lds9);
+    if (threadIdx.x == 0) wround2_result<PLAIN, UNIT, NOMID>(out, tot);
 }
 
 // ---------------------------------------------------------------- matmul phase 1: weights per segment
@@ -303,16 +309,31 @@ int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t
     }
     const int nv = plain_sums ? 5 : 3;
     void* ws;
-    int rc = scratch_get(kSlotReduce, (size_t)nb * nv * 32, &ws, s);
+    const size_t partial_bytes = (size_t)nb * nv * 32;
+    int rc = scratch_get(kSlotReduce, partial_bytes + kFoldTableBytes, &ws, s);
     if (rc) return rc;
     uint32_t* partial = (uint32_t*)ws;
+    // long rounds fold through the table of the challenge's multiples (one more small launch)
+    const bool use_tab = n_out >= kTableFoldMinOut;
+    int32_t* tab = (int32_t*)((char*)ws + partial_bytes);
+    if (use_tab) fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+// five sums and three accumulators leave no registers for the table fold's columns (it spills: 1.16 against
+    // 1.10 ms at 2^24 index pairs), so that form keeps the single-product fold at every size
 #define GRAPE_WROUND2(B, P, U)                                                                                        \
     do {                                                                                                              \
-        wround2_kernel<B, P, U><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, partial);     \
-        if (nb >= kFinalWideMin) wround2_final_kernel<P, U, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb); \
-        else wround2_final_kernel<P, U, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);                               \
+        if (use_tab && !((P) && !(U)))                                                                                \
+            wround2_kernel<B, P, U, !((P) && !(U))><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, tab, partial); \
+        else wround2_kernel<B, P, U, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, nullptr, partial);    \
+        if (nb >= kFinalWideMin) wround2_final_kernel<P, U, false, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb); \
+        else wround2_final_kernel<P, U, false, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);                               \
     } while (0)
-    if (plain_sums == 2) {
+    if (plain_sums == 3) {
+        // the middle coefficient is left to the caller (sums[1] = 0); long rounds of a logUp proof
+        GRAPE_REQUIRE(beta != nullptr && use_tab, "the round without its middle coefficient is built for logUp rounds of 2^16 index pairs and more");
+        wround2_kernel<true, true, false, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, tab, partial);
+        if (nb >= kFinalWideMin) wround2_final_kernel<true, false, true, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb);
+        else wround2_final_kernel<true, false, true, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);
+    } else if (plain_sums == 2) {
         GRAPE_REQUIRE(rowlen == rowpad && in_size == 2 * (uint64_t)n_out,
                       "the inverse-pair round needs whole pairs and unpadded rows (weights that sum to one)");
         if (beta) GRAPE_WROUND2(true, true, true);

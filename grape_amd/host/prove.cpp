@@ -145,6 +145,14 @@ void matmul_sumcheck_phase2(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, 
 // src/prove.cu:175-210
 std::pair<Fr, Fr> prove_matmul(FrTensor& A, FrTensor& B, int L, int N, int M, int K, const std::vector<Fr> u,
                                const std::vector<Fr> v, Fr& claim, SumcheckTranscript* transcript) {
+    // The point u is read as log2(M) variables of the column index, log2(N) of the row index and log2(L)
+    // of the batch index, while the reference finds the end of the batch variables at Log2(L*N*M)
+    // (src/prove.cu:198): the two agree only when the padded extents multiply to the padded product.
+    // A shape like N = 3, M = 5 (Log2(15) = 4, but 2 + 3 variables) has no defined reading - the
+    // reference's folds would run past the end of u - and is refused, as is a point that is too short.
+    const uint lu = Log2((uint)L) + Log2((uint)N) + Log2((uint)M);
+    if (L < 1 || N < 1 || M < 1 || K < 1 || Log2((uint)(L * N * M)) != lu || u.size() < lu || v.size() < Log2((uint)(L * K)))
+        throw std::runtime_error("prove_matmul: Incompatible dimensions");
     fr_t* U = grape_host::upload(u);
     fr_t* V = grape_host::upload(v);
     std::pair<Fr, Fr> ret;

@@ -375,6 +375,7 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         // beside the rounds over A and S (the short rounds are launch- and latency-bound: five
         // small kernels per round on the table side, two on the witness side).
         SideChain side(0), witness(1);
+        std::vector<char> mid_from_claim(rounds ? rounds : 1, 0);    // rounds whose middle coefficient follows from the claim
         side.begin();                       // the second stream waits for everything queued so far
         grape_stream_t ws = nullptr;        // where the short witness rounds run: the default stream, or one of its own beside the commitments
         uint cur = D;
@@ -389,7 +390,13 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             // every index (B holds the inverses of T + beta, none of which is zero for a range table and, for
             // a mapping table with its random r, except with probability 2^-235), and the weights of a full
             // level sum to one - the round then needs its top coefficient only
-            const int mode = (k == 0 && from_table && cur == 2 * half && (cur & (cur - 1)) == 0) ? 2 : 1;
+            int mode = (k == 0 && from_table && cur == 2 * half && (cur & (cur - 1)) == 0) ? 2 : 1;
+            // a long round after the first: its middle coefficient is left to the host, which holds the
+            // round's claim when it assembles the polynomials (one limb product per index pair less)
+            if (mode == 1 && half >= kLongRoundPairs) {
+                mode = 3;
+                mid_from_claim[k] = 1;
+            }
             check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), mode, W(slot), st), "grape_wround2");
             A.set_size(half);
             S.set_size(half);
@@ -478,25 +485,35 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         int ui = (int)nu - 1;      // index of the variable bound in this round (u.back())
         k = 0;
         for (int vi = (int)rounds - 1; vi >= 0; vi--, ui--, k++) {
-            const Fr* a3 = &h[13 * (size_t)k];
+            Fr* a3 = &h[13 * (size_t)k];
             const Fr* b3 = a3 + 5;
             const Fr* c3 = a3 + 10;
-            Polynomial p0({a3[0], a3[1], a3[2]});
-            p0 = p0 * alpha_run;
-            Polynomial p1({a3[3], a3[4]});
-            Polynomial p;
-            if (vi >= (int)logN) {
-                p0 *= Polynomial::eq(u[ui]);
-                p = p0 + p1 + Polynomial(C * two_inv);
-                if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase1: claim != p(0) + p(1)");
-                C = C * two_inv;
-            } else {
+            const bool phase1 = vi >= (int)logN;
+            // the round polynomial from the 13 sums (src/tlookup.cu:117-151, :153-190)
+            auto round_poly = [&]() {
+                Polynomial p0({a3[0], a3[1], a3[2]});
+                p0 = p0 * alpha_run;
+                Polynomial p1({a3[3], a3[4]});
+                if (phase1) {
+                    p0 *= Polynomial::eq(u[ui]);
+                    return p0 + p1 + Polynomial(C * two_inv);
+                }
                 Fr coef = N_div_D * alpha_sq_run;
                 p0 += Polynomial({b3[0] * coef, b3[1] * coef, b3[2] * coef});
                 Polynomial p2({c3[0], c3[1], c3[2]});
-                p = Polynomial::eq(u[ui]) * p0 + p1 - p2 * N_div_D;
-                if (claim != p(0) + p(1)) throw std::runtime_error("tLookup_phase2: claim != p(0) + p(1)");
+                return Polynomial::eq(u[ui]) * p0 + p1 - p2 * N_div_D;
+            };
+            if (mid_from_claim[k]) {
+                // the kernel left a3[1] = 0.  p(0) + p(1) is linear in it with slope eq(u, 1) * alpha_run = u * alpha_run
+                // (only the value at t = 1 of the weighted term contains it), and must equal the claim
+                const Fr slope = u[ui] * alpha_run;
+                if (slope.is_zero()) throw std::runtime_error("tLookup: a challenge is zero, the round's middle coefficient is not determined by its claim");
+                const Polynomial p_without = round_poly();
+                a3[1] = (claim - (p_without(0) + p_without(1))) * slope.inverse();
             }
+            Polynomial p = round_poly();
+            if (claim != p(0) + p(1)) throw std::runtime_error(phase1 ? "tLookup_phase1: claim != p(0) + p(1)" : "tLookup_phase2: claim != p(0) + p(1)");
+            if (phase1) C = C * two_inv;
             claim = p(v[vi]);
             last_transcript.rounds.push_back(p);
             last_transcript.claims.push_back(claim);

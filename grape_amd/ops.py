@@ -364,11 +364,12 @@ def eq_pyramid(u, nu=None):
     return pyr
 
 
-def wround2(A, S, beta, e, in_size, n_out, v, plain_sums=False, rowlen=1, rowpad=1, inverse_pair=False):
-    """inverse_pair: the caller states A * (S + beta) = 1 at every index and weights that sum to one"""
+def wround2(A, S, beta, e, in_size, n_out, v, plain_sums=False, rowlen=1, rowpad=1, inverse_pair=False, no_middle=False):
+    """inverse_pair: the caller states A * (S + beta) = 1 at every index and weights that sum to one;
+    no_middle: the middle coefficient is left out (sums[1] = 0) for a caller that takes it from the round's claim"""
     lib = init()
     sums = fr_empty(5 if plain_sums else 3)
-    mode = 2 if inverse_pair else (1 if plain_sums else 0)
+    mode = 3 if no_middle else (2 if inverse_pair else (1 if plain_sums else 0))
     _capi.check(lib.grape_wround2(_p(A), _p(S), _p(beta), _p(e), in_size, n_out, rowlen, rowpad, _p(v), mode,
                                   _p(sums), _s()))
     return sums

@@ -187,6 +187,9 @@ int grape_eq_pyramid(uint32_t *d_pyr, const uint32_t *d_u, uint32_t nu, grape_st
  * proof over A = 1/(S + beta): d_sums[0] = 1 and d_sums[1] = -d_sums[2] then follow without being
  * summed, and the pass takes one weight product per index instead of two.  The five sums equal those
  * of plain_sums == 1 whenever the statement holds.
+ * plain_sums == 3 (d_beta given, n_out >= 2^16) leaves the middle coefficient out: d_sums[1] = 0 and the
+ * other four sums as with plain_sums == 1.  It is for a caller that holds the round's claim - the sum of
+ * the round polynomial over {0, 1}, src/tlookup.cu:228 - from which the middle coefficient follows.
  * One pass replaces sumcheck_kernel + three folds of coefficient arrays per round in eleMul_sumcheck
  * (src/prove.cu:119-172) and tLookup_poly_kernel + three multilinear evaluations +
  * tLookup_poly_sum_kernel + two sums + the reduce kernel in tLookup_phase1 (src/tlookup.cu:117-151,216-244).

@@ -349,6 +349,27 @@ def test_weighted_round_with_fused_fold(ops, in_size, n_out, beta, plain):
     assert_same(ops.fr_to_host(dS)[:n_out], orc.partial_eval(Sp, 2 * n_out, v, 2, 0, n_out)[:n_out], "folded S")
 
 
+@pytest.mark.parametrize("in_size,n_out", [(1 << 17, 1 << 16), ((1 << 18) - 1000, 1 << 17), (1 << 22, 1 << 21)])
+def test_weighted_round_without_its_middle_coefficient(ops, in_size, n_out):
+    """the long logUp rounds after the first: the variant that leaves the middle coefficient to the caller gives the other
+    four sums and the folds of the general round (whose sums the tests above pin against the oracle), and writes zero
+    in the middle slot; both fold through the table of the challenge's multiples at this size"""
+    logh = br.log2ceil(n_out)
+    A, S = rand_fr(in_size, 291 + n_out), rand_fr(in_size, 292 + n_out)
+    bt, v, u = rand_fr(1, 293), rand_fr(1, 294), rand_fr(logh, 295)
+    e = ops.eq_pyramid(ops.to_dev(u), logh)[n_out - 1:2 * n_out - 1].contiguous()
+    dA1, dS1, dA2, dS2 = ops.to_dev(A), ops.to_dev(S), ops.to_dev(A), ops.to_dev(S)
+    general = ops.fr_to_host(ops.wround2(dA1, dS1, ops.to_dev(bt), e, in_size, n_out, ops.to_dev(v), plain_sums=True))
+    short = ops.fr_to_host(ops.wround2(dA2, dS2, ops.to_dev(bt), e, in_size, n_out, ops.to_dev(v), plain_sums=True, no_middle=True))
+    assert_same(short[[0, 2, 3, 4]], general[[0, 2, 3, 4]], "the four sums")
+    assert br.fr_unpack(short[1:2]) == [0]
+    assert_same(ops.fr_to_host(dA2)[:n_out], ops.fr_to_host(dA1)[:n_out], "folded A")
+    assert_same(ops.fr_to_host(dS2)[:n_out], ops.fr_to_host(dS1)[:n_out], "folded S")
+    # the folds through the table against the oracle's fold
+    assert_same(ops.fr_to_host(dA2)[:1000], orc.partial_eval(np.concatenate([A, np.zeros((2 * n_out - in_size, 4), dtype=np.uint64)]),
+                                                               2 * n_out, v, 2, 0, n_out)[:1000], "folded A against the oracle")
+
+
 @pytest.mark.parametrize("n_out,beta", [(1, True), (4096, True), (1 << 17, True), ((1 << 18), False)])
 def test_weighted_round_of_an_inverse_pair(ops, n_out, beta):
     """the first round of a logUp proof, where A = 1/(S + beta): the variant that takes only the top
