@@ -110,7 +110,7 @@ __global__ void __launch_bounds__(kBlock, 2) sumcheck2_kernel(uint32_t* A, uint3
         }
     }
     if (partial) {
-        // |sum| < 16 r^2 -> within (-0.46 r, 1.46 r) after reduction
+        // at most kRoundIters = 64 products below r^2 in size: |sum| < 64 r^2 -> within (-1.82 r, 2.82 r) after the reduction
         const Fr c0 = fr26::finish_sum(C0, 2), c2 = fr26::finish_sum(C2, 2);
         Fr acc[3] = {c0, Fr::zero(), c2};
         if (!CLAIM) acc[1] = sub(sub(fr26::finish_sum(Q, 2), c0), c2);

@@ -175,14 +175,14 @@ __global__ void __launch_bounds__(BLOCK) wround2_final_kernel(uint32_t* out, con
 // Indices g = seg * seglen + k; every index of a segment shares the weight e[seg], so the three
 // sums are taken per (segment, chunk) without weights and the finishing kernel applies e[seg].
 __global__ void __launch_bounds__(kBlock) sumcheck2_seg_kernel(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size,
-                                                               uint32_t seglen, const uint32_t* v, uint32_t* partial) {
+                                                               uint32_t seglen, uint32_t seg0, const uint32_t* v, uint32_t* partial) {
     __shared__ Fr lds[3 * (kBlock / 64)];
     const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
     fr26::Acc C0, Q, C2;
     fr26::acc_zero(C0);
     fr26::acc_zero(Q);
     fr26::acc_zero(C2);
-    const uint32_t seg = blockIdx.y;
+    const uint32_t seg = seg0 + blockIdx.y;            // a launch covers at most 65535 segments (the grid's y extent)
     const uint32_t stride = gridDim.x * kBlock;      // the host keeps seglen / stride <= 64
     for (uint32_t k = blockIdx.x * kBlock + threadIdx.x; k < seglen; k += stride) {
         const size_t g = (size_t)seg * seglen + k;
@@ -358,7 +358,6 @@ int grape_sumcheck_round2_seg(uint32_t* A, uint32_t* B, uint32_t in_size, uint32
     GRAPE_REQUIRE(out_size >= 1 && in_size >= out_size && in_size <= 2 * (uint64_t)out_size, "need out_size <= in_size <= 2*out_size");
     GRAPE_REQUIRE(seglen >= 1 && out_size % seglen == 0, "out_size must be a whole number of segments");
     const uint32_t nseg = out_size / seglen;
-    GRAPE_REQUIRE(nseg <= 65535, "too many segments");
     hipStream_t s = as_stream(st);
     // chunks per segment: one index per thread until the grid is large, never more than 64 per thread
     uint32_t nchunk = blocks_for(seglen);
@@ -369,7 +368,10 @@ int grape_sumcheck_round2_seg(uint32_t* A, uint32_t* B, uint32_t in_size, uint32
     void* ws;
     int rc = scratch_get(kSlotReduce, (size_t)nseg * nchunk * 3 * 32, &ws, s);
     if (rc) return rc;
-    sumcheck2_seg_kernel<<<dim3(nchunk, nseg), kBlock, 0, s>>>(A, B, in_size, out_size, seglen, v, (uint32_t*)ws);
+    for (uint32_t seg0 = 0; seg0 < nseg; seg0 += 65535) {
+        const uint32_t ns = nseg - seg0 < 65535 ? nseg - seg0 : 65535;
+        sumcheck2_seg_kernel<<<dim3(nchunk, ns), kBlock, 0, s>>>(A, B, in_size, out_size, seglen, seg0, v, (uint32_t*)ws);
+    }
     seg_final_kernel<<<1, kBlock, 0, s>>>(sums, (const uint32_t*)ws, e, nseg, nchunk);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;

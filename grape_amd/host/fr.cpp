@@ -1,4 +1,5 @@
 #include "fr.hpp"
+#include <atomic>
 #include <errno.h>
 #include <sys/random.h>
 #include <iomanip>
@@ -31,7 +32,7 @@ struct Xoshiro {
 // (one generator behind a mutex, so OpenMP callers stay safe, though their interleaving is not
 // reproducible); Fr::seed_from_os() switches back.
 std::mutex g_rng_mu;
-bool g_seeded = false;
+std::atomic<bool> g_seeded{false};
 Xoshiro g_xo;
 
 // 64 random bits from the OS, buffered per thread
@@ -55,12 +56,16 @@ uint64_t os_random64() {
     buf[have] = 0;                       // a word is handed out once and not kept
     return w;
 }
-uint64_t next64() {
-    {
+// four words of one draw: one lock per element in the reproducible mode, none in the default mode
+void next256(uint64_t w[4]) {
+    if (g_seeded.load(std::memory_order_acquire)) {
         std::lock_guard<std::mutex> lock(g_rng_mu);
-        if (g_seeded) return g_xo.next();
+        if (g_seeded.load(std::memory_order_relaxed)) {
+            for (int i = 0; i < 4; i++) w[i] = g_xo.next();
+            return;
+        }
     }
-    return os_random64();
+    for (int i = 0; i < 4; i++) w[i] = os_random64();
 }
 bool below_modulus(const uint32_t* a) {
     for (int i = 7; i >= 0; i--) {
@@ -84,24 +89,22 @@ Fr::Fr(long x) {
 void Fr::seed(uint64_t s) {
     std::lock_guard<std::mutex> lock(g_rng_mu);
     g_xo.seed(s);
-    g_seeded = true;
+    g_seeded.store(true, std::memory_order_release);
 }
 void Fr::seed_from_os() {
     std::lock_guard<std::mutex> lock(g_rng_mu);
-    g_seeded = false;
+    g_seeded.store(false, std::memory_order_release);
 }
-bool Fr::seeded() {
-    std::lock_guard<std::mutex> lock(g_rng_mu);
-    return g_seeded;
-}
+bool Fr::seeded() { return g_seeded.load(std::memory_order_acquire); }
 
 Fr Fr::random_element() {
     for (;;) {
         fr_t raw;
+        uint64_t w[4];
+        next256(w);
         for (int i = 0; i < 4; i++) {
-            uint64_t w = next64();
-            raw.v[2 * i] = (uint32_t)w;
-            raw.v[2 * i + 1] = (uint32_t)(w >> 32);
+            raw.v[2 * i] = (uint32_t)w[i];
+            raw.v[2 * i + 1] = (uint32_t)(w[i] >> 32);
         }
         raw.v[7] &= 0x7fffffffu;
         if (below_modulus(raw.v)) return Fr(raw);   // a uniform residue read as Montgomery form is uniform

@@ -18,18 +18,33 @@ void ensure_init() {
 }
 
 static constexpr int kSlots = 64;
+namespace {
+// the ring of one host thread, given back when the thread ends
+struct ScalarRing {
+    fr_t* p = nullptr;
+    ~ScalarRing() { grape_free(p); }
+};
+}  // namespace
 fr_t* device_scalar(const Fr& x) {
     // one ring per host thread: a slot is rewritten after kSlots further calls of the same thread,
     // never by another thread
-    thread_local fr_t* ring = nullptr;
+    thread_local ScalarRing holder;
     thread_local int next = 0;
     ensure_init();
-    if (!ring) check(grape_malloc((void**)&ring, sizeof(fr_t) * kSlots), "grape_malloc");
+    if (!holder.p) check(grape_malloc((void**)&holder.p, sizeof(fr_t) * kSlots), "grape_malloc");
+    fr_t* const ring = holder.p;
     fr_t* slot = ring + next;
     next = (next + 1) % kSlots;
     check(grape_memcpy_h2d(slot, &x, sizeof(fr_t), nullptr), "grape_memcpy_h2d");
     return slot;
 }
+DeviceFr::DeviceFr(const Fr& x) {
+    ensure_init();
+    check(grape_malloc((void**)&p_, sizeof(fr_t)), "grape_malloc");
+    check(grape_memcpy_h2d(p_, &x, sizeof(fr_t), nullptr), "grape_memcpy_h2d");
+}
+DeviceFr::~DeviceFr() { grape_free(p_); }
+
 fr_t* upload(const std::vector<Fr>& v) {
     ensure_init();
     fr_t* d = nullptr;

@@ -12,8 +12,22 @@ namespace grape_host {
 void check(int rc, const char* what);
 // Uploads one scalar into a small ring of device slots and returns its device address
 // (replaces the cudaMalloc + cudaMemcpy + cudaFree of a 32-byte scalar per call,
-// src/fr-tensor.cu:212-218).
+// src/fr-tensor.cu:212-218).  The slot is rewritten, on the default stream, once the calling thread has
+// asked for 64 further scalars: the address is for kernels queued on the default stream right away.
+// A scalar that other streams read, or that is read for long, gets a DeviceFr of its own.
 fr_t* device_scalar(const Fr& x);
+// One scalar in a device buffer of its own, freed when the object goes.
+class DeviceFr {
+public:
+    explicit DeviceFr(const Fr& x);
+    ~DeviceFr();
+    DeviceFr(const DeviceFr&) = delete;
+    DeviceFr& operator=(const DeviceFr&) = delete;
+    fr_t* get() const { return p_; }
+
+private:
+    fr_t* p_ = nullptr;
+};
 // Uploads a challenge vector; the caller frees with grape_free.
 fr_t* upload(const std::vector<Fr>& v);
 Fr download(const fr_t* d_ptr);

@@ -68,7 +68,9 @@ void Hyrax::check_shape(uint size, uint N) const {
 bool Hyrax::ensure_table(WideTable& t, uint rowlen, uint c, uint nw, uint K) {
     if (t.d && t.ngen >= rowlen && t.c == c && t.nw == nw) return true;
     size_t bytes = grape_g1_wide_table_bytes(rowlen, nw, K);
-    if (bytes > table_budget_) return false;
+    // against what every other table of this object holds (the one being replaced gives its bytes back)
+    const size_t others = table_bytes_in_use() - (t.d ? grape_g1_wide_table_bytes(t.ngen, t.nw, t.K) : 0);
+    if (others + bytes > table_budget_) return false;
     if (rowlen > npoints) throw std::runtime_error("row longer than the generator set");
     grape_free(t.d);
     t = WideTable();
@@ -281,6 +283,8 @@ affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
     commit_fr_rows(out, tensor.gpu_data, size, rowlen, rows > 1);
     return out;
 }
+
+bool Hyrax::prepare_scaled_tables(uint ncols) { return ensure_fr_table(ncols); }
 
 affine_t* Hyrax::build_scaled_table(const FrTensor& scalars, uint ncols) {
     if (ncols > npoints) throw std::runtime_error("row longer than the generator set");

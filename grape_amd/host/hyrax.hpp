@@ -67,6 +67,10 @@ public:
     // owned by the caller, freed with grape_free); nullptr when it would not fit the budget.
     // With it, a tensor whose elements are scalars[idx] commits at one addition per element:
     affine_t* build_scaled_table(const FrTensor& scalars, uint ncols);
+    // Builds what build_scaled_table reads (the per-window table over the first ncols generators) if it is
+    // not there yet, so that table_bytes_free() afterwards is what a scaled table may really take; false when
+    // it does not fit the budget (build_scaled_table would return nullptr).
+    bool prepare_scaled_tables(uint ncols);
     // frees a table that build_scaled_table returned and gives its bytes back to the budget of the
     // Hyrax object that built it, if that object still exists
     static void release_scaled_table(affine_t* table);

@@ -262,7 +262,6 @@ Fr combine_claims(FrTensor& X, const std::vector<Fr>& claims, const std::vector<
     const uint rounds = (uint)v.size();
     std::vector<Fr> eq_accumulate(num, Fr::one());
     if (rounds > 0 && num > 0) {
-        if (num > 16) throw std::runtime_error("combine_claims: at most 16 claims");
         fr_t* d_v = grape_host::upload(v);
         std::vector<std::unique_ptr<EqPyramid>> eq;
         std::vector<fr_t*> d_u(num, nullptr);
@@ -275,10 +274,14 @@ Fr combine_claims(FrTensor& X, const std::vector<Fr>& claims, const std::vector<
             uint in = size;
             for (uint i = 0; i < rounds; i++) {
                 const uint out = in / 2;
-                const uint32_t* tables[16];
-                for (uint j = 0; j < num; j++) tables[j] = W(eq[j]->level(rounds - 1 - i));
-                check(grape_wsum1_multi(W(X.gpu_data), tables, num, in, out, W(sums.gpu_data + 2 * (size_t)num * i), nullptr),
-                      "grape_wsum1_multi");
+                // one launch weighs the tensor against up to 16 tables: more claims go in groups of 16
+                for (uint j0 = 0; j0 < num; j0 += 16) {
+                    const uint nj = num - j0 < 16 ? num - j0 : 16;
+                    const uint32_t* tables[16];
+                    for (uint j = 0; j < nj; j++) tables[j] = W(eq[j0 + j]->level(rounds - 1 - i));
+                    check(grape_wsum1_multi(W(X.gpu_data), tables, nj, in, out, W(sums.gpu_data + 2 * ((size_t)num * i + j0)), nullptr),
+                          "grape_wsum1_multi");
+                }
                 uint32_t* ptrs[1] = {W(X.gpu_data)};
                 check(grape_fr_fold_msb_multi(ptrs, 1, out, W(d_v + (rounds - 1 - i)), nullptr), "grape_fr_fold_msb_multi");
                 in = out;

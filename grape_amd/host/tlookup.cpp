@@ -105,6 +105,8 @@ bool tLookup::commit_A_by_occupancy(FrTensor& A, uint D, uint msm_size, Hyrax& h
     if (!hot_reused_) {
         drop_hot_rows();
         const size_t row_bytes = grape_g1_wide_table_bytes(rowlen, 1, 1);
+        // the per-window table the rows are built through comes first: it takes its share of the budget
+        if (!hyrax.prepare_scaled_tables(rowlen)) return false;
         size_t max_hot = hyrax.table_bytes_free() / row_bytes;
         if (max_hot > N) max_hot = N;
         if (max_hot == 0) return false;
@@ -275,7 +277,10 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     cold_elements_ = 0;
     hot_reused_ = false;
 
-    fr_t* d_beta = grape_host::device_scalar(beta);
+    // beta is read by kernels on the side streams until the end of the proof: a buffer of its own, not a
+    // slot of the ring of grape_host::device_scalar (which is rewritten after 64 further scalars)
+    grape_host::DeviceFr beta_buf(beta);
+    fr_t* d_beta = beta_buf.get();
     // A = 1/(S + beta): read from B where the witness matches its table entry (every element of
     // a valid witness does), computed by batched inversion otherwise (tlookup_inv_kernel,
     // src/tlookup.cu:52-62, inverts per element)

@@ -308,7 +308,7 @@ def test_prove_elemul_vs_oracle(ops, host, L, M, N):
         host.prove_elemul(ops.to_dev(pA), ops.to_dev(pB), L, M, N, pu, pv, br.fr_pack([claim0 + 1])[0])
 
 
-@pytest.mark.parametrize("nv,num", [(4, 3), (3, 1), (1, 2), (10, 4)])
+@pytest.mark.parametrize("nv,num", [(4, 3), (3, 1), (1, 2), (10, 4), (5, 17)])      # 17 claims: two launches of the multi-table kernel per round
 def test_combine_claims_vs_oracle(ops, host, nv, num):
     X = rand_fr(1 << nv, 90 + nv)
     us = [rand_fr(nv, 91 + nv + j) for j in range(num)]

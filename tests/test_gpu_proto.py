@@ -418,7 +418,8 @@ def test_weighted_round_on_padded_rows(ops):
     assert sums == [x % R for x in want]
 
 
-@pytest.mark.parametrize("nseg,seglen,ragged", [(1, 8, 0), (4, 96, 0), (32, 128, 0), (2, 20000, 0), (8, 300, 1000)])
+@pytest.mark.parametrize("nseg,seglen,ragged", [(1, 8, 0), (4, 96, 0), (32, 128, 0), (2, 20000, 0), (8, 300, 1000),
+                                                (70000, 2, 3)])      # more segments than one launch's grid holds
 def test_segment_weighted_round(ops, nseg, seglen, ragged):
     """grape_sumcheck_round2_seg: the three sums of every segment of seglen indices times that segment's
     weight, and the folds - against the plain round kernel run per segment"""
