@@ -952,23 +952,34 @@ int grape_tlookup_inverse_by_table(uint32_t* A, const uint32_t* S, const int32_t
     return GRAPE_OK;
 }
 
+int grape_tlookup_index_inverse_nowait(int32_t* idx1, uint32_t* A, const uint32_t* key, size_t n, int32_t low, uint32_t len,
+                                       const uint32_t* B, const uint32_t* cmp, const uint32_t* cmp_table, uint32_t* d_mismatches,
+                                       grape_stream_t st) {
+    GRAPE_REQUIRE(d_mismatches != nullptr && idx1 != nullptr && len > 0, "bad arguments");
+    hipStream_t s = as_stream(st);
+    int rc = zero_fill(d_mismatches, sizeof(uint32_t), s);
+    if (rc) return rc;
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(A); CHECK_PTR16(key); CHECK_PTR16(B);
+    GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr), "cmp and cmp_table go together");
+    if (cmp) { CHECK_PTR16(cmp); CHECK_PTR16(cmp_table); }
+    index_inverse_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, key, n, low, len, B, cmp, cmp_table, (unsigned int*)d_mismatches);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
 int grape_tlookup_index_inverse(int32_t* idx1, uint32_t* A, const uint32_t* key, size_t n, int32_t low, uint32_t len,
                                 const uint32_t* B, const uint32_t* cmp, const uint32_t* cmp_table, size_t* mismatches,
                                 grape_stream_t st) {
     GRAPE_REQUIRE(mismatches != nullptr && idx1 != nullptr && len > 0, "bad arguments");
     *mismatches = 0;
     if (n == 0) return GRAPE_OK;
-    CHECK_PTR16(A); CHECK_PTR16(key); CHECK_PTR16(B);
-    GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr), "cmp and cmp_table go together");
-    if (cmp) { CHECK_PTR16(cmp); CHECK_PTR16(cmp_table); }
     hipStream_t s = as_stream(st);
     void* cnt;
     int rc = scratch_get(kSlotMisc, 64, &cnt, s);
     if (rc) return rc;
-    rc = zero_fill(cnt, sizeof(unsigned int), s);
+    rc = grape_tlookup_index_inverse_nowait(idx1, A, key, n, low, len, B, cmp, cmp_table, (uint32_t*)cnt, st);
     if (rc) return rc;
-    index_inverse_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, key, n, low, len, B, cmp, cmp_table, (unsigned int*)cnt);
-    GRAPE_LAUNCH_CHECK();
     unsigned int h = 0;
     GRAPE_HIP_CHECK(hipMemcpyAsync(&h, cnt, sizeof h, hipMemcpyDeviceToHost, s));
     GRAPE_HIP_CHECK(hipStreamSynchronize(s));

@@ -29,11 +29,24 @@ void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const
     drop_index();
     a_ready_ = false;
     check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(key.size ? key.size : 1)), "grape_malloc");
-    size_t mismatches = 0;
-    check(grape_tlookup_index_inverse(d_idx_, W(A.gpu_data), W(key.gpu_data), key.size, low_, T.size, W(B.gpu_data),
-                                      cmp ? W(cmp->gpu_data) : nullptr, cmp_table ? W(cmp_table->gpu_data) : nullptr, &mismatches,
-                                      nullptr),
-          "grape_tlookup_index_inverse");
+    // The pass over the witness is queued first and its count of unmatched elements read last: in between the
+    // host queues the proof's weights (a dozen small launches on the second stream) while the chip is busy.
+    uint32_t* d_count = nullptr;
+    check(grape_malloc((void**)&d_count, sizeof(uint32_t)), "grape_malloc");
+    uint32_t mismatches = 1;
+    try {
+        check(grape_tlookup_index_inverse_nowait(d_idx_, W(A.gpu_data), W(key.gpu_data), key.size, low_, T.size, W(B.gpu_data),
+                                                 cmp ? W(cmp->gpu_data) : nullptr, cmp_table ? W(cmp_table->gpu_data) : nullptr, d_count,
+                                                 nullptr),
+              "grape_tlookup_index_inverse_nowait");
+        start_weights(1u << Log2(key.size));
+        check(grape_memcpy_d2h(&mismatches, d_count, sizeof(uint32_t), nullptr), "grape_memcpy_d2h");
+    } catch (...) {
+        grape_stream_sync(nullptr);
+        grape_free(d_count);
+        throw;
+    }
+    grape_free(d_count);
     a_ready_ = mismatches == 0;
 }
 void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
@@ -227,6 +240,20 @@ std::pair<void*, void*> commit_events() {
 }
 }  // namespace
 
+void tLookup::start_weights(uint D) {
+    const uint nu = Log2(D);
+    u_ready_ = forced_u_.empty() ? random_vec(nu) : forced_u_;
+    forced_u_.clear();
+    E_ready_.reset();
+    if (u_ready_.size() != nu) return;          // run() reports the mismatch
+    E_ready_.reset(new FrTensor((uint)grape_eq_pyramid_elems(nu ? nu - 1 : 0)));
+    fr_t* d_u = grape_host::upload(u_ready_);
+    SideChain side(0);
+    SideChain::order(side.stream, nullptr);     // the point's upload before the pyramid
+    check(grape_eq_pyramid(W(E_ready_->gpu_data), W(d_u), nu ? nu - 1 : 0, side.stream), "grape_eq_pyramid");
+    grape_free(d_u);                            // handed out again only after what is queued here
+}
+
 static void histogram_to_m(FrTensor& m, const FrTensor& vals, int low) {
     uint32_t* hist = nullptr;
     check(grape_malloc((void**)&hist, sizeof(uint32_t) * (size_t)m.size), "grape_malloc");
@@ -266,8 +293,17 @@ void tLookupRange::prep(const FrTensor& vals) { histogram_to_m(m, vals, low); }
 Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
     const uint D = S.size;
     const uint N = T.size;
-    std::vector<Fr> u = forced_u_.empty() ? random_vec(Log2(D)) : forced_u_;
-    forced_u_.clear();
+    // the point and its eq pyramid may have been started by prove() (start_weights)
+    std::unique_ptr<FrTensor> E_early = std::move(E_ready_);
+    std::vector<Fr> u;
+    if (!u_ready_.empty() || E_early) {
+        u = std::move(u_ready_);
+        u_ready_.clear();
+    } else {
+        u = forced_u_.empty() ? random_vec(Log2(D)) : forced_u_;
+        forced_u_.clear();
+    }
+    if (u.size() != Log2(D)) E_early.reset();
     if (u.size() != v.size()) throw std::runtime_error("u.size() != v.size()");
     if (v.size() != Log2(D)) throw std::runtime_error("u.size() != ceilLog2(D)");
     if (D % msm_size != 0) throw std::runtime_error("D % msm_size != 0");
@@ -357,12 +393,17 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     // eq tables of every prefix of u[0 .. nu-2]: round k (which binds variable nu-1-k) weights its
     // D / 2^(k+1) index pairs with level nu-1-k; nothing is halved between rounds
     const uint nu = (uint)u.size();
-    FrTensor E((uint)grape_eq_pyramid_elems(nu ? nu - 1 : 0));
-    {
+    std::unique_ptr<FrTensor> E_own;
+    if (E_early) {
+        SideChain early(0);
+        SideChain::order(nullptr, early.stream);     // the default stream meets the finished pyramid
+    } else {
+        E_own.reset(new FrTensor((uint)grape_eq_pyramid_elems(nu ? nu - 1 : 0)));
         fr_t* d_u = grape_host::upload(u);
-        check(grape_eq_pyramid(W(E.gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_pyramid");
+        check(grape_eq_pyramid(W(E_own->gpu_data), W(d_u), nu ? nu - 1 : 0, nullptr), "grape_eq_pyramid");
         grape_free(d_u);                    // no wait: the block is handed out again only after what is queued here
     }
+    FrTensor& E = E_early ? *E_early : *E_own;
     // The prover's challenges are all known before the first round, so the rounds are queued
     // back to back: every round leaves its 13 sums in its own slot of one device buffer, which
     // is read once after the last round; the polynomials and the running claim follow on the
@@ -537,8 +578,12 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
 Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
     uint D = S.size;
     a_ready_ = false;
-    if (D == (1u << Log2(D)) && A.size >= D) make_index_and_A(S, low, A, nullptr, nullptr);   // no padding: index and A = B[index] together
-    else make_index(S, low);
+    if (D == (1u << Log2(D)) && A.size >= D) {
+        make_index_and_A(S, low, A, nullptr, nullptr);   // no padding: index and A = B[index] together (starts the weights too)
+    } else {
+        start_weights(1u << Log2(D));
+        make_index(S, low);
+    }
     index_to_m(D, low);                       // what prep(S) computes, from the shared indices
     if (D != (1u << Log2(D))) {
         // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
@@ -595,9 +640,13 @@ Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, cons
     uint D = S_in.size;
     a_ready_ = false;
     if (S_out.size != D) throw std::runtime_error("tLookupRangeMapping: S_in.size != S_out.size");
-    // no padding: index, the check S_out = f(S_in) and A = B[index] in one pass
-    if (D == (1u << Log2(D)) && A.size >= D) make_index_and_A(S_in, low, A, &S_out, &mapped_vals);
-    else make_index(S_in, low);
+    // no padding: index, the check S_out = f(S_in) and A = B[index] in one pass (starts the weights too)
+    if (D == (1u << Log2(D)) && A.size >= D) {
+        make_index_and_A(S_in, low, A, &S_out, &mapped_vals);
+    } else {
+        start_weights(1u << Log2(D));
+        make_index(S_in, low);
+    }
     index_to_m(D, low);                       // what prep(S_in) computes, from the shared indices
     FrTensor S(1u << Log2(D));
     S.set_size(D);

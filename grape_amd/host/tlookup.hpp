@@ -2,6 +2,7 @@
 // include/tlookup.cuh:37-79.
 #pragma once
 #include <string>
+#include <memory>
 #include <vector>
 #include "fr_tensor.hpp"
 #include "hyrax.hpp"
@@ -47,6 +48,12 @@ public:
 protected:
     Fr run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
     std::vector<Fr> forced_u_;
+    // The weights of a proof over a witness of D (padded) elements - the object's random point u and the pyramid of
+    // its eq tables - started on the second stream before the witness is indexed and counted, so that they are
+    // built beside those passes; run() takes them over.
+    void start_weights(uint D);
+    std::vector<Fr> u_ready_;
+    std::unique_ptr<FrTensor> E_ready_;
     bool indexed_commit_ = true;
     bool index_known_ = false;          // set by tLookupRange: A's index is S - low
     int index_low_ = 0;

@@ -235,6 +235,11 @@ int grape_tlookup_index(int32_t *d_out, const uint32_t *d_vals, size_t n, int32_
 int grape_tlookup_index_inverse(int32_t *d_idx1, uint32_t *d_A, const uint32_t *d_key, size_t n, int32_t low, uint32_t len,
                                 const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table, size_t *mismatches,
                                 grape_stream_t stream);
+/* The same pass queued without waiting: the count of unmatched elements is left in the device word
+ * d_mismatches (cleared by the call), for a caller that has more to queue before it reads the count. */
+int grape_tlookup_index_inverse_nowait(int32_t *d_idx1, uint32_t *d_A, const uint32_t *d_key, size_t n, int32_t low, uint32_t len,
+                                       const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table,
+                                       uint32_t *d_mismatches, grape_stream_t stream);
 /* The same histogram from indices already made by grape_tlookup_index (d_idx1[i] = index + 1,
  * 0 = outside the table): hist[d_idx1[i] - 1] += 1. */
 int grape_tlookup_hist_index(uint32_t *d_hist, const int32_t *d_idx1, size_t n, uint32_t len, grape_stream_t stream);
