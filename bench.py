@@ -54,7 +54,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch read from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # same counter reads for the 1 GiB copy kernel below); the counters cannot be read from inside this
 # process, so these are the figures of the committed counter summary of this same command.
-COMMIT_KERNEL_TRAFFIC_BYTES = 2.580e9
+COMMIT_KERNEL_TRAFFIC_BYTES = 2.627e9
 FOLD_KERNEL_TRAFFIC_BYTES = 1.110e9
 
 
@@ -466,6 +466,53 @@ def lookup_workload(args):
     return 0
 
 
+def claims_workload(args):
+    """The two remaining sub-provers of the layer at its largest shapes: prove_eleMul on the gated
+    feed-forward product (2048 rows of 11008 columns, padded to 16384: 2^25 index pairs, 25 rounds) and
+    combine_claims of three claims on one 4096 x 4096 weight (24 rounds).  One step = one proof of each;
+    the final evaluations are checked against independent multilinear evaluations on the GPU."""
+    import torch
+    from grape_amd import ops, _host as host
+    from gpuutil import rand_fr
+    ops.init(0)
+    host.load()
+    L, M, N, Np = 1, 2048, 11008, 16384
+    rng = np.random.default_rng(61)
+    dA = ops.fr_from_i32(torch.from_numpy(rng.integers(-(1 << 15), 1 << 15, M * N).astype(np.int32)).cuda())
+    dB = ops.fr_from_i32(torch.from_numpy(rng.integers(-(1 << 15), 1 << 15, M * N).astype(np.int32)).cuda())
+    u, v = rand_fr(25, 62), rand_fr(25, 63)
+    zero = ops.to_dev(np.zeros((1, 4), dtype=np.uint64))
+    pa, pb = ops.fr_pad(dA, N, Np, M * Np, zero), ops.fr_pad(dB, N, Np, M * Np, zero)
+    claim = host.mle_eval(ops.fr_mul(pa, pb), M * Np, u)
+    nv, num = 24, 3
+    X = ops.fr_from_i32(torch.from_numpy(gaussian_i16((4096, 4096), 64)).cuda())
+    us = np.stack([rand_fr(nv, 65 + j) for j in range(num)])
+    vv = rand_fr(nv, 69)
+    claims = np.stack([host.mle_eval(X, 1 << nv, us[j]) for j in range(num)])
+    t_mul, t_comb = [], []
+    for i in range(args.warmup + args.steps):
+        _, _, ac, bc = host.prove_elemul(dA, dB, L, M, N, u, v, claim)
+        t1 = host.last_prove_seconds()
+        _, res = host.combine_claims(X, 1 << nv, claims, us, vv)
+        t2 = host.last_prove_seconds()
+        if i >= args.warmup:
+            t_mul.append(t1)
+            t_comb.append(t2)
+    if not (np.array_equal(host.mle_eval(pa, M * Np, v), ac) and np.array_equal(host.mle_eval(pb, M * Np, v), bc)
+            and np.array_equal(host.mle_eval(X, 1 << nv, vv), res)):
+        print("bench.py: final evaluations differ from independent evaluations", file=sys.stderr)
+        return 1
+    t1, t2 = float(np.mean(t_mul)), float(np.mean(t_comb))
+    print(json.dumps({
+        "metric": "elemul_sumcheck_time", "value": t1, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t1 * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "prove_eleMul 2048 x 11008 (padded to 2^25 index pairs) and combine_claims of 3 claims on 2^24 elements",
+                   "elemul_operand_read_GBps": 2 * 32.0 * M * N / t1 / 1e9,
+                   "combine_claims_s": t2, "combine_claims_operand_read_GBps": 32.0 * (1 << nv) / t2 / 1e9}}))
+    return 0
+
+
 def mapping_workload(args):
     """The layer's largest single proof on its own: the softmax exponential's mapping lookup, 2^27 scores
     (32 heads x 2048 x 2048) into the 2^20-entry table, 4096 generators, scores distributed as the layer's
@@ -833,12 +880,13 @@ def main():
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
     ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")
-    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "mapping", "witness", "rounds", "plumbing"], default="commit",
+    ap.add_argument("--workload", choices=["commit", "layer", "matmul", "lookup", "mapping", "witness", "rounds", "plumbing", "claims"], default="commit",
                     help="commit: configs[1], the metric's headline (default); matmul: configs[2]; "
                          "lookup: configs[3]; layer: configs[4]; mapping: the layer's softmax lookup on its own; "
                          "witness: the layer's witness generator; "
                          "rounds: the streaming kernels of the sumcheck / logUp rounds; "
-                         "plumbing: configs[0] and the reduce-type kernels (sum, batched inversion, lookup index and histogram)")
+                         "plumbing: configs[0] and the reduce-type kernels (sum, batched inversion, lookup index and histogram); "
+                         "claims: prove_eleMul and combine_claims at the layer's largest shapes")
     ap.add_argument("--plain-commit", action="store_true",
                     help="mapping workload: commit A as full-width scalars instead of through its occupied entries")
     ap.add_argument("--seq", type=int, default=2048, help="sequence length of the layer and witness workloads")
@@ -863,10 +911,10 @@ def main():
         args.steps = 3 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
         return mapping_workload(args)
-    if args.workload in ("matmul", "lookup"):
+    if args.workload in ("matmul", "lookup", "claims"):
         args.steps = 5 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
-        return matmul_workload(args) if args.workload == "matmul" else lookup_workload(args)
+        return {"matmul": matmul_workload, "lookup": lookup_workload, "claims": claims_workload}[args.workload](args)
     if args.workload == "layer":
         args.steps = 1 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup

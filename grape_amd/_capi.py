@@ -59,6 +59,11 @@ SIGNATURES = {
     "grape_eq_pyramid_elems": [c_u32],
     "grape_eq_pyramid": [c_void_p, c_void_p, c_u32, c_void_p],
     "grape_wround2": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_u32, c_u32, c_void_p, c_int, c_void_p, c_void_p],
+    "grape_wround2_partial_bytes": [c_u32],
+    "grape_fold_tables": [c_void_p, c_void_p, c_u32, c_void_p],
+    "grape_wround2_queue": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_u32, c_u32, c_u32, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    "grape_wround2_queue_indexed": [c_void_p, c_void_p, c_void_p, c_void_p, c_u32, c_void_p, c_void_p, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
+    "grape_wround2_finish": [c_void_p, c_void_p, c_u32, c_int, c_void_p],
     "grape_sumcheck_round2_seg": [c_void_p, c_void_p, c_u32, c_u32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_wsum1_multi": [c_void_p, ctypes.POINTER(c_void_p), c_u32, c_u32, c_u32, c_void_p, c_void_p],
     "grape_tlookup_hist": [c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p],
@@ -122,7 +127,8 @@ SIGNATURES = {
     "grape_event_record": [c_void_p, c_void_p],
     "grape_event_elapsed_ms": [ctypes.POINTER(ctypes.c_float), c_void_p, c_void_p],
 }
-_RESTYPES = {"grape_last_error": ctypes.c_char_p, "grape_g1_wide_table_bytes": c_size_t, "grape_eq_pyramid_elems": c_size_t}
+_RESTYPES = {"grape_last_error": ctypes.c_char_p, "grape_g1_wide_table_bytes": c_size_t, "grape_eq_pyramid_elems": c_size_t,
+             "grape_wround2_partial_bytes": c_size_t}
 
 _lib = None
 

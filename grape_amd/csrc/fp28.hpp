@@ -21,6 +21,7 @@
 // case: BN254 leaves R'/p = 2^26 of head-room instead of 2^11 and sums 10 limb products.
 #pragma once
 #include "curve.hpp"
+#include "divstep.hpp"
 
 namespace grape {
 
@@ -374,14 +375,15 @@ GRAPE_HD Fp28 inverse(const Fp28& a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Modular inversion by divsteps (Bernstein-Yang "safegcd"), batched 30 steps at a time on
-// signed 30-bit limbs.  About 800 divsteps for a 381-bit modulus, i.e. some 27 batches of a few
-// hundred instructions each - an order of magnitude fewer sequential instructions than the
-// a^(p-2) ladder, which matters because one inversion sits on the critical path of every row
-// epilogue.  The reference inverts with the same family of algorithm
-// (include/field/mont_t.cuh:1058-1120, ct_inverse_mod_x).
+// Modular inversion by divsteps (divstep.hpp) for the 28-bit form: about 800 divsteps for a 381-bit
+// modulus, i.e. some 27 batches of a few hundred instructions each - one inversion sits on the
+// critical path of every row epilogue.
 // ------------------------------------------------------------------------------------------------
 namespace by {
+
+using divstep::M30;
+using divstep::Mat;
+using divstep::divsteps30;
 
 #if defined(GRAPE_CURVE_BN254)
 constexpr int L = 9;                        // 9 x 30 = 270 bits
@@ -400,86 +402,15 @@ GRAPE_HD int32_t P30(int i) {
     return t[i];
 }
 #endif
-constexpr int32_t M30 = (1 << 30) - 1;
-// floor((49 d + 57) / 17) divsteps always suffice for d-bit inputs (Bernstein-Yang, d >= 46):
-// 1110 for 384 bits, 741 for 256 bits; taken 30 at a time
-constexpr int kBatches = ((49 * 32 * FpParams::N + 57) / 17 + 29) / 30;
+struct PMod {
+    static constexpr uint32_t INV30 = PINV30;
+    static GRAPE_HD int32_t limb(int i) { return P30(i); }
+};
+// 1110 divsteps at most for 384 bits, 741 for 256 bits
+constexpr int kBatches = divstep::batches_for_bits(32 * FpParams::N);
 
-struct Mat { int32_t u, v, q, r; };
-
-// 30 divsteps on the low words; returns the transition matrix scaled by 2^30:
-//   u*f + v*g = 2^30 * f',   q*f + r*g = 2^30 * g'
-GRAPE_HD int32_t divsteps30(int32_t delta, uint32_t f, uint32_t g, Mat& t) {
-    int32_t u = 1, v = 0, q = 0, r = 1;
-    for (int i = 0; i < 30; i++) {
-        const bool swap = (delta > 0) & ((g & 1u) != 0);
-        // (f, g) <- (g, -f), rows of the matrix alike, delta <- -delta
-        const uint32_t nf = swap ? g : f;
-        const uint32_t ng = swap ? (0u - f) : g;
-        const int32_t nu = swap ? q : u, nv = swap ? r : v;
-        const int32_t nq = swap ? -u : q, nr = swap ? -v : r;
-        delta = swap ? -delta : delta;
-        f = nf; g = ng; u = nu; v = nv; q = nq; r = nr;
-        // make g even
-        const bool odd = (g & 1u) != 0;
-        g += odd ? f : 0u;
-        q += odd ? u : 0;
-        r += odd ? v : 0;
-        delta += 1;
-        g >>= 1;
-        u <<= 1;
-        v <<= 1;
-    }
-    t.u = u; t.v = v; t.q = q; t.r = r;
-    return delta;
-}
-
-// (f, g) <- t * (f, g) / 2^30, exact
-GRAPE_HD void update_fg(int32_t* f, int32_t* g, const Mat& t) {
-    int64_t cf = (int64_t)t.u * f[0] + (int64_t)t.v * g[0];
-    int64_t cg = (int64_t)t.q * f[0] + (int64_t)t.r * g[0];
-    cf >>= 30;   // the low 30 bits are zero by construction
-    cg >>= 30;
-#pragma unroll
-    for (int i = 1; i < L; i++) {
-        cf += (int64_t)t.u * f[i] + (int64_t)t.v * g[i];
-        cg += (int64_t)t.q * f[i] + (int64_t)t.r * g[i];
-        f[i - 1] = (int32_t)cf & M30;
-        g[i - 1] = (int32_t)cg & M30;
-        cf >>= 30;
-        cg >>= 30;
-    }
-    f[L - 1] = (int32_t)cf;
-    g[L - 1] = (int32_t)cg;
-}
-
-// (d, e) <- t * (d, e) / 2^30 mod p, keeping both in (-2p, p)
-GRAPE_HD void update_de(int32_t* d, int32_t* e, const Mat& t) {
-    const int32_t sd = d[L - 1] >> 31, se = e[L - 1] >> 31;   // all-ones when negative
-    // a negative d (e) is replaced by d + p (e + p): that adds u*p (v*p) to the first row
-    int32_t md = (t.u & sd) + (t.v & se);
-    int32_t me = (t.q & sd) + (t.r & se);
-    int64_t cd = (int64_t)t.u * d[0] + (int64_t)t.v * e[0];
-    int64_t ce = (int64_t)t.q * d[0] + (int64_t)t.r * e[0];
-    // choose the multiple of p that clears the low 30 bits
-    md -= (int32_t)((PINV30 * (uint32_t)cd + (uint32_t)md) & (uint32_t)M30);
-    me -= (int32_t)((PINV30 * (uint32_t)ce + (uint32_t)me) & (uint32_t)M30);
-    cd += (int64_t)P30(0) * md;
-    ce += (int64_t)P30(0) * me;
-    cd >>= 30;
-    ce >>= 30;
-#pragma unroll
-    for (int i = 1; i < L; i++) {
-        cd += (int64_t)t.u * d[i] + (int64_t)t.v * e[i] + (int64_t)P30(i) * md;
-        ce += (int64_t)t.q * d[i] + (int64_t)t.r * e[i] + (int64_t)P30(i) * me;
-        d[i - 1] = (int32_t)cd & M30;
-        e[i - 1] = (int32_t)ce & M30;
-        cd >>= 30;
-        ce >>= 30;
-    }
-    d[L - 1] = (int32_t)cd;
-    e[L - 1] = (int32_t)ce;
-}
+GRAPE_HD void update_fg(int32_t* f, int32_t* g, const Mat& t) { divstep::update_fg<L>(f, g, t); }
+GRAPE_HD void update_de(int32_t* d, int32_t* e, const Mat& t) { divstep::update_de<L, PMod>(d, e, t); }
 
 }  // namespace by
 

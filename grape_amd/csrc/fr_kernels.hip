@@ -5,6 +5,7 @@
 // one element with two 16-byte vector accesses, so a wave64 covers 2 KiB of contiguous memory per
 // element index and both halves of every 128-byte line are consumed back to back.
 #include "fr_device.hpp"
+#include "divstep.hpp"
 
 namespace grape {
 
@@ -137,37 +138,40 @@ __global__ void __launch_bounds__(kBlock) inv_prod_kernel(uint32_t* prod, const 
     }
     st_fr(prod, t, acc);
 }
-// given inv_prod[t] = 1/prod[t], write the individual inverses
+// given inv_prod[t] = 1/prod[t], write the individual inverses.  Only the prefix products stay in
+// registers (8 elements = 64 registers); the elements themselves are read again on the way back -
+// holding both sets spilled to scratch memory, which cost 2.5 times the traffic of the second read.
 __global__ void __launch_bounds__(kBlock) inv_back_kernel(uint32_t* out, const uint32_t* in, const uint32_t* beta,
                                                           const uint32_t* inv_prod, size_t n) {
     size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
     size_t nchunks = (n + kInvChunk - 1) / kInvChunk;
     if (t >= nchunks) return;
     Fr bt = beta ? ld_fr(beta, 0) : Fr::zero();
-    Fr x[kInvChunk];
     Fr pre[kInvChunk];   // pre[k] = product of non-zero x[0..k-1]
     Fr acc = Fr::one();
-#pragma unroll
+#pragma clang loop unroll(full)
     for (int k = 0; k < kInvChunk; k++) {
         size_t i = t + (size_t)k * nchunks;
-        x[k] = Fr::zero();
+        Fr x = Fr::zero();
         if (i < n) {
-            x[k] = ld_fr(in, i);
-            if (beta) x[k] = add(x[k], bt);
+            x = ld_fr(in, i);
+            if (beta) x = add(x, bt);
         }
         pre[k] = acc;
-        if (!x[k].is_zero()) acc = fr26::mulc(acc, x[k]);
+        if (!x.is_zero()) acc = fr26::mulc(acc, x);
     }
     Fr inv = ld_fr(inv_prod, t);   // 1 / product of all non-zero x
-#pragma unroll
+#pragma clang loop unroll(full)
     for (int k = kInvChunk - 1; k >= 0; k--) {
         size_t i = t + (size_t)k * nchunks;
         if (i < n) {
-            if (x[k].is_zero()) {
+            Fr x = ld_fr(in, i);          // (out may be in: element i is read before it is written, by this thread only)
+            if (beta) x = add(x, bt);
+            if (x.is_zero()) {
                 st_fr(out, i, Fr::zero());
             } else {
                 st_fr(out, i, fr26::mulc(inv, pre[k]));
-                inv = fr26::mulc(inv, x[k]);
+                inv = fr26::mulc(inv, x);
             }
         }
     }
@@ -178,7 +182,7 @@ __global__ void __launch_bounds__(kBlock) inv_direct_kernel(uint32_t* out, const
     if (i >= n) return;
     Fr x = ld_fr(in, i);
     if (beta) x = add(x, ld_fr(beta, 0));
-    st_fr(out, i, inverse(x));
+    st_fr(out, i, divstep::inverse_by(x));
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -496,7 +496,7 @@ __global__ void __launch_bounds__(kBlock) index_inverse_kernel(int32_t* idx1, ui
             for (int k = 0; k < 8; k++) diff |= a.v[k] ^ b.v[k];
             bad = diff != 0;
         }
-        if (!bad) st_fr(A, i, ld_fr(B, d.v[0]));
+        if (!bad && A) st_fr(A, i, ld_fr(B, d.v[0]));
     }
     const unsigned long long b = __ballot(bad);
     if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
@@ -642,22 +642,36 @@ __global__ void __launch_bounds__(kBlock, 2) tl_table_round_kernel(uint32_t* B, 
                                                                 const uint32_t* eq, size_t n_out, const uint32_t* v, uint32_t* partial) {
     __shared__ Fr lds[8 * (kBlock / 64)];
     const size_t first = (size_t)blockIdx.x * kBlock + threadIdx.x, stride = (size_t)gridDim.x * kBlock;
-    Fr acc[8];
-    tl_round_thread_sums(acc, B, T, beta, eq, n_out, first, stride);
-    tl_mb_thread_sums(acc + 5, m, B, n_out, first, stride);
-    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
-    for (size_t t = first; t < n_out; t += stride) {
-        uint32_t* X[3] = {B, T, m};
+    // the two groups of sums one after the other, each handed to the workgroup's sum before the next starts,
+    // so that neither is held in registers beside the other's accumulators
+    {
+        Fr acc3[3];
+        tl_mb_thread_sums(acc3, m, B, n_out, first, stride);
+        block_sum<3>(acc3, lds);
+        if (threadIdx.x == 0) {
 #pragma unroll
-        for (int j = 0; j < 3; j++) {
-            const fr26::Limbs lo = ld_l26(X[j], t);
-            st_fr(X[j], t, fold1(w1, lo, fr26::sub(ld_l26(X[j], t + n_out), lo)));
+            for (int k = 0; k < 3; k++) st_fr(partial, (size_t)blockIdx.x * 8 + 5 + k, acc3[k]);
+        }
+        __syncthreads();                   // lds is reused below
+    }
+    {
+        Fr acc5[5];
+        tl_round_thread_sums(acc5, B, T, beta, eq, n_out, first, stride);
+        block_sum<5>(acc5, lds);
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int k = 0; k < 5; k++) st_fr(partial, (size_t)blockIdx.x * 8 + k, acc5[k]);
         }
     }
-    block_sum<8>(acc, lds);
-    if (threadIdx.x == 0) {
-#pragma unroll
-        for (int k = 0; k < 8; k++) st_fr(partial, (size_t)blockIdx.x * 8 + k, acc[k]);
+    const fr26::Limbs w1 = fr26::weight16(ld_fr(v, 0));
+    auto fold_one = [&](uint32_t* X, size_t t) __attribute__((always_inline)) {
+        const fr26::Limbs lo = ld_l26(X, t);
+        st_fr(X, t, fold1(w1, lo, fr26::sub(ld_l26(X, t + n_out), lo)));
+    };
+    for (size_t t = first; t < n_out; t += stride) {
+        fold_one(B, t);
+        fold_one(T, t);
+        fold_one(m, t);
     }
 }
 
@@ -960,7 +974,8 @@ int grape_tlookup_index_inverse_nowait(int32_t* idx1, uint32_t* A, const uint32_
     int rc = zero_fill(d_mismatches, sizeof(uint32_t), s);
     if (rc) return rc;
     if (n == 0) return GRAPE_OK;
-    CHECK_PTR16(A); CHECK_PTR16(key); CHECK_PTR16(B);
+    CHECK_PTR16(key);
+    if (A) { CHECK_PTR16(A); CHECK_PTR16(B); }       // A == nullptr: indices and the count only
     GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr), "cmp and cmp_table go together");
     if (cmp) { CHECK_PTR16(cmp); CHECK_PTR16(cmp_table); }
     index_inverse_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, key, n, low, len, B, cmp, cmp_table, (unsigned int*)d_mismatches);

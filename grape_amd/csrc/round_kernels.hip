@@ -92,10 +92,13 @@ __device__ __forceinline__ void wround2_result(uint32_t* out, const Fr* acc) {
 // NOMID: the sum of the round polynomial over {0, 1} is known to the caller (the value the previous
 // round's polynomial took at its challenge), which fixes the middle coefficient: the value at t = 1
 // is not accumulated - one product and one double-width accumulator less per index.
-template <bool BETA, bool PLAIN, bool UNIT, bool TAB, bool NOMID = false>
+// IDX: A is not read but gathered, A[i] = Bt[idx1[i] - 1] (in_size == 2 n_out): the first round of a lookup whose
+// logUp tensor was never written out - the pass over the witness left the table indices only.
+template <bool BETA, bool PLAIN, bool UNIT, bool TAB, bool NOMID = false, bool IDX = false>
 __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E,
                                                          uint32_t in_size, uint32_t n_out, uint32_t rowlen, uint32_t rowpad,
-                                                         const uint32_t* v, const int32_t* __restrict__ tab, uint32_t* partial) {
+                                                         const uint32_t* v, const int32_t* __restrict__ tab, uint32_t* partial,
+                                                         const int32_t* __restrict__ idx1 = nullptr, const uint32_t* Bt = nullptr) {
     constexpr int NV = PLAIN ? 5 : 3;
     __shared__ Fr lds[NV * (kBlock / 64)];
     fr26::Limbs w1;
@@ -114,8 +117,15 @@ __global__ void __launch_bounds__(kBlock, 2) wround2_kernel(uint32_t* A, uint32_
         // weights live on rows of `rowpad` entries when the tensors' rows hold `rowlen` < rowpad
         const size_t ei = rowlen == rowpad ? g : g + (size_t)((uint32_t)g / rowlen) * (rowpad - rowlen);
         const fr26::Limbs e16 = fr26::pack16(ld_fr(E, ei));
-        const fr26::Limbs a0 = ld_l26(A, g);
-        const fr26::Limbs a1 = ld_hi26(A, g, n_out, in_size);
+        fr26::Limbs a0, a1;
+        if (IDX) {
+            const uint32_t j0 = (uint32_t)idx1[g], j1 = (uint32_t)idx1[g + n_out];     // 0 marks an element outside the table
+            a0 = ld_l26(Bt, j0 ? j0 - 1 : 0);
+            a1 = ld_l26(Bt, j1 ? j1 - 1 : 0);
+        } else {
+            a0 = ld_l26(A, g);
+            a1 = ld_hi26(A, g, n_out, in_size);
+        }
         const fr26::Limbs da = fr26::sub(a1, a0);
         fr26::Acc T;
         fr26::Limbs ea0;
@@ -295,28 +305,23 @@ int grape_eq_pyramid(uint32_t* pyr, const uint32_t* u, uint32_t nu, grape_stream
     return GRAPE_OK;
 }
 
-int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E, uint32_t in_size, uint32_t n_out,
-                  uint32_t rowlen, uint32_t rowpad, const uint32_t* v, int plain_sums, uint32_t* sums, grape_stream_t st) {
-    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(E); CHECK_PTR16(v); CHECK_PTR16(sums);
-    GRAPE_REQUIRE(n_out >= 1 && in_size >= n_out && in_size <= 2 * (uint64_t)n_out, "need n_out <= in_size <= 2*n_out");
-    GRAPE_REQUIRE(rowlen >= 1 && rowlen <= rowpad, "need 1 <= rowlen <= rowpad");
-    if (beta) CHECK_PTR16(beta);
-    hipStream_t s = as_stream(st);
+// workgroups of a weighted round over n_out index pairs
+static unsigned wround2_blocks(uint32_t n_out) {
     unsigned nb = blocks_for(n_out);
     if (nb > (unsigned)kNumCU * 4) {
         const unsigned need = blocks_for(n_out, kBlock * kWIters);
         nb = need > (unsigned)kNumCU * 4 ? need : (unsigned)kNumCU * 4;
     }
-    const int nv = plain_sums ? 5 : 3;
-    void* ws;
-    const size_t partial_bytes = (size_t)nb * nv * 32;
-    int rc = scratch_get(kSlotReduce, partial_bytes + kFoldTableBytes, &ws, s);
-    if (rc) return rc;
-    uint32_t* partial = (uint32_t*)ws;
-    // long rounds fold through the table of the challenge's multiples (one more small launch)
-    const bool use_tab = n_out >= kTableFoldMinOut;
-    int32_t* tab = (int32_t*)((char*)ws + partial_bytes);
-    if (use_tab) fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+    return nb;
+}
+
+// The two launches of a weighted round: the pass over the operands (partial sums per workgroup; `tab`: the table of
+// the challenge's multiples, or nullptr for the single-product fold) and the kernel that finishes the sums.
+static int wround2_main(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E, uint32_t in_size, uint32_t n_out,
+                        uint32_t rowlen, uint32_t rowpad, const uint32_t* v, int plain_sums, const int32_t* tab, uint32_t* partial,
+                        hipStream_t s) {
+    const unsigned nb = wround2_blocks(n_out);
+    const bool use_tab = tab != nullptr;
 // five sums and three accumulators leave no registers for the table fold's columns (it spills: 1.16 against
     // 1.10 ms at 2^24 index pairs), so that form keeps the single-product fold at every size
 #define GRAPE_WROUND2(B, P, U)                                                                                        \
@@ -324,15 +329,11 @@ int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t
         if (use_tab && !((P) && !(U)))                                                                                \
             wround2_kernel<B, P, U, !((P) && !(U))><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, tab, partial); \
         else wround2_kernel<B, P, U, false><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, nullptr, partial);    \
-        if (nb >= kFinalWideMin) wround2_final_kernel<P, U, false, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb); \
-        else wround2_final_kernel<P, U, false, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);                               \
     } while (0)
     if (plain_sums == 3) {
         // the middle coefficient is left to the caller (sums[1] = 0); long rounds of a logUp proof
         GRAPE_REQUIRE(beta != nullptr && use_tab, "the round without its middle coefficient is built for logUp rounds of 2^16 index pairs and more");
         wround2_kernel<true, true, false, true, true><<<nb, kBlock, 0, s>>>(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, tab, partial);
-        if (nb >= kFinalWideMin) wround2_final_kernel<true, false, true, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb);
-        else wround2_final_kernel<true, false, true, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);
     } else if (plain_sums == 2) {
         GRAPE_REQUIRE(rowlen == rowpad && in_size == 2 * (uint64_t)n_out,
                       "the inverse-pair round needs whole pairs and unpadded rows (weights that sum to one)");
@@ -348,9 +349,94 @@ int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t
         GRAPE_WROUND2(false, false, false);
     }
 #undef GRAPE_WROUND2
+    return GRAPE_OK;
+}
+static void wround2_final(uint32_t* sums, const uint32_t* partial, uint32_t n_out, int plain_sums, hipStream_t s) {
+    const unsigned nb = wround2_blocks(n_out);
+#define GRAPE_WFINAL(P, U, M)                                                                                    \
+    do {                                                                                                         \
+        if (nb >= kFinalWideMin) wround2_final_kernel<P, U, M, kFinalBlock><<<1, kFinalBlock, 0, s>>>(sums, partial, nb); \
+        else wround2_final_kernel<P, U, M, kBlock><<<1, kBlock, 0, s>>>(sums, partial, nb);                      \
+    } while (0)
+    if (plain_sums == 3) GRAPE_WFINAL(true, false, true);
+    else if (plain_sums == 2) GRAPE_WFINAL(true, true, false);
+    else if (plain_sums) GRAPE_WFINAL(true, false, false);
+    else GRAPE_WFINAL(false, false, false);
+#undef GRAPE_WFINAL
+}
+#define GRAPE_WROUND2_CHECKS()                                                                                              \
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(E); CHECK_PTR16(v);                                                        \
+    GRAPE_REQUIRE(n_out >= 1 && in_size >= n_out && in_size <= 2 * (uint64_t)n_out, "need n_out <= in_size <= 2*n_out"); \
+    GRAPE_REQUIRE(rowlen >= 1 && rowlen <= rowpad, "need 1 <= rowlen <= rowpad");                                        \
+    if (beta) CHECK_PTR16(beta)
+
+int grape_wround2(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E, uint32_t in_size, uint32_t n_out,
+                  uint32_t rowlen, uint32_t rowpad, const uint32_t* v, int plain_sums, uint32_t* sums, grape_stream_t st) {
+    GRAPE_WROUND2_CHECKS();
+    CHECK_PTR16(sums);
+    hipStream_t s = as_stream(st);
+    void* ws;
+    const size_t partial_bytes = (size_t)wround2_blocks(n_out) * (plain_sums ? 5 : 3) * 32;
+    int rc = scratch_get(kSlotReduce, partial_bytes + kFoldTableBytes, &ws, s);
+    if (rc) return rc;
+    uint32_t* partial = (uint32_t*)ws;
+    // long rounds fold through the table of the challenge's multiples (one more small launch)
+    int32_t* tab = nullptr;
+    if (n_out >= kTableFoldMinOut) {
+        tab = (int32_t*)((char*)ws + partial_bytes);
+        fold_tables_kernel<<<1, 64, 0, s>>>(tab, v, 1);
+    }
+    rc = wround2_main(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, plain_sums, tab, partial, s);
+    if (rc) return rc;
+    wround2_final(sums, partial, n_out, plain_sums, s);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
+
+size_t grape_wround2_partial_bytes(uint32_t n_out) { return (size_t)wround2_blocks(n_out ? n_out : 1) * 5 * 32; }
+
+static_assert(GRAPE_FOLD_TABLE_WORDS == fr26::kFoldTableWords, "the header's table size is the kernels'");
+int grape_fold_tables(int32_t* tabs, const uint32_t* v, uint32_t count, grape_stream_t st) {
+    GRAPE_REQUIRE(tabs != nullptr && (reinterpret_cast<uintptr_t>(tabs) & 3) == 0, "tabs must be 4-byte aligned");
+    GRAPE_REQUIRE(count >= 1 && count <= 64, "1..64 challenges");
+    CHECK_PTR16(v);
+    fold_tables_kernel<<<1, 64, 0, as_stream(st)>>>(tabs, v, count);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wround2_queue(uint32_t* A, uint32_t* S, const uint32_t* beta, const uint32_t* E, uint32_t in_size, uint32_t n_out,
+                        uint32_t rowlen, uint32_t rowpad, const uint32_t* v, int plain_sums, const int32_t* tab, uint32_t* partial,
+                        grape_stream_t st) {
+    GRAPE_WROUND2_CHECKS();
+    CHECK_PTR16(partial);
+    GRAPE_REQUIRE(tab == nullptr || n_out >= kTableFoldMinOut, "the table fold is built for rounds of 2^16 index pairs and more");
+    int rc = wround2_main(A, S, beta, E, in_size, n_out, rowlen, rowpad, v, plain_sums, tab, partial, as_stream(st));
+    if (rc) return rc;
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wround2_queue_indexed(uint32_t* A, uint32_t* S, const int32_t* idx1, const uint32_t* Bt, uint32_t len, const uint32_t* beta,
+                                const uint32_t* E, uint32_t n_out, const uint32_t* v, const int32_t* tab, uint32_t* partial,
+                                grape_stream_t st) {
+    CHECK_PTR16(A); CHECK_PTR16(S); CHECK_PTR16(E); CHECK_PTR16(v); CHECK_PTR16(Bt); CHECK_PTR16(beta); CHECK_PTR16(partial);
+    GRAPE_REQUIRE(idx1 != nullptr && len >= 1, "bad arguments");
+    GRAPE_REQUIRE(tab != nullptr && n_out >= kTableFoldMinOut && n_out <= (1u << 30), "built for first rounds of 2^16 index pairs and more");
+    wround2_kernel<true, true, true, true, false, true><<<wround2_blocks(n_out), kBlock, 0, as_stream(st)>>>(
+        A, S, beta, E, 2 * n_out, n_out, 1, 1, v, tab, partial, idx1, Bt);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_wround2_finish(uint32_t* sums, const uint32_t* partial, uint32_t n_out, int plain_sums, grape_stream_t st) {
+    CHECK_PTR16(sums); CHECK_PTR16(partial);
+    GRAPE_REQUIRE(n_out >= 1, "need n_out >= 1");
+    wround2_final(sums, partial, n_out, plain_sums, as_stream(st));
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+#undef GRAPE_WROUND2_CHECKS
 
 int grape_sumcheck_round2_seg(uint32_t* A, uint32_t* B, uint32_t in_size, uint32_t out_size, uint32_t seglen, const uint32_t* e,
                               const uint32_t* v, uint32_t* sums, grape_stream_t st) {

@@ -45,11 +45,11 @@ DeviceFr::DeviceFr(const Fr& x) {
 }
 DeviceFr::~DeviceFr() { grape_free(p_); }
 
-fr_t* upload(const std::vector<Fr>& v) {
+fr_t* upload(const std::vector<Fr>& v, void* stream) {
     ensure_init();
     fr_t* d = nullptr;
     check(grape_malloc((void**)&d, sizeof(fr_t) * std::max<size_t>(v.size(), 1)), "grape_malloc");
-    check(grape_memcpy_h2d(d, v.data(), sizeof(fr_t) * v.size(), nullptr), "grape_memcpy_h2d");
+    check(grape_memcpy_h2d(d, v.data(), sizeof(fr_t) * v.size(), stream), "grape_memcpy_h2d");
     return d;
 }
 Fr download(const fr_t* d_ptr) {

@@ -29,7 +29,7 @@ private:
     fr_t* p_ = nullptr;
 };
 // Uploads a challenge vector; the caller frees with grape_free.
-fr_t* upload(const std::vector<Fr>& v);
+fr_t* upload(const std::vector<Fr>& v, void* stream = nullptr);   // queued on `stream` (nullptr: the default stream)
 Fr download(const fr_t* d_ptr);
 void ensure_init();
 }  // namespace grape_host

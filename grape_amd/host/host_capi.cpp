@@ -151,7 +151,11 @@ int grape_host_combine_claims(const uint32_t* d_X, uint32_t size, const uint32_t
     std::vector<std::vector<Fr>> us(num);
     for (uint32_t j = 0; j < num; j++) us[j] = vec_from(u + 8 * (size_t)j * nv, nv);
     SumcheckTranscript tr;
-    Fr r = combine_claims(X, vec_from(claims, num), us, vec_from(v, nv), size, &tr);
+    Fr r;
+    {
+        ProveTimer timer;
+        r = combine_claims(X, vec_from(claims, num), us, vec_from(v, nv), size, &tr);
+    }
     fr_to(result, r);
     put_transcript(tr, transcript, n_rounds);
     GUARD_END

@@ -25,9 +25,10 @@ void tLookup::make_index(const FrTensor& vals, int low_) {
     check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(vals.size ? vals.size : 1)), "grape_malloc");
     check(grape_tlookup_index(d_idx_, W(vals.gpu_data), vals.size, low_, T.size, nullptr), "grape_tlookup_index");
 }
-void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table) {
+void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table, bool write_A) {
     drop_index();
     a_ready_ = false;
+    a_deferred_ = false;
     check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(key.size ? key.size : 1)), "grape_malloc");
     // The pass over the witness is queued first and its count of unmatched elements read last: in between the
     // host queues the proof's weights (a dozen small launches on the second stream) while the chip is busy.
@@ -35,7 +36,7 @@ void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const
     check(grape_malloc((void**)&d_count, sizeof(uint32_t)), "grape_malloc");
     uint32_t mismatches = 1;
     try {
-        check(grape_tlookup_index_inverse_nowait(d_idx_, W(A.gpu_data), W(key.gpu_data), key.size, low_, T.size, W(B.gpu_data),
+        check(grape_tlookup_index_inverse_nowait(d_idx_, write_A ? W(A.gpu_data) : nullptr, W(key.gpu_data), key.size, low_, T.size, W(B.gpu_data),
                                                  cmp ? W(cmp->gpu_data) : nullptr, cmp_table ? W(cmp_table->gpu_data) : nullptr, d_count,
                                                  nullptr),
               "grape_tlookup_index_inverse_nowait");
@@ -47,7 +48,8 @@ void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const
         throw;
     }
     grape_free(d_count);
-    a_ready_ = mismatches == 0;
+    a_ready_ = write_A && mismatches == 0;
+    a_deferred_ = !write_A && mismatches == 0;
 }
 void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
     if (!d_idx_ || N == pad_N) return;
@@ -67,18 +69,19 @@ void tLookup::drop_index() {
 }
 // multiplicities from the indices (get_histogram_kernel, src/tlookup.cu:5-14, with the padding
 // rule of :276-281)
-void tLookup::index_to_m(uint witness_size, int low_) {
+void tLookup::index_to_m(uint witness_size, int low_, void* stream) {
+    m_pending_ = false;
     uint32_t* hist = nullptr;
     check(grape_malloc((void**)&hist, sizeof(uint32_t) * (size_t)m.size), "grape_malloc");
-    check(grape_memset_zero(hist, sizeof(uint32_t) * (size_t)m.size, nullptr), "grape_memset_zero");
-    check(grape_tlookup_hist_index(hist, d_idx_, witness_size, m.size, nullptr), "grape_tlookup_hist_index");
+    check(grape_memset_zero(hist, sizeof(uint32_t) * (size_t)m.size, stream), "grape_memset_zero");
+    check(grape_tlookup_hist_index(hist, d_idx_, witness_size, m.size, stream), "grape_tlookup_hist_index");
     if (witness_size != (1u << Log2(witness_size))) {
         uint32_t zero_count = 0;
-        check(grape_memcpy_d2h(&zero_count, hist + (-low_), sizeof(uint32_t), nullptr), "d2h");
+        check(grape_memcpy_d2h(&zero_count, hist + (-low_), sizeof(uint32_t), stream), "d2h");
         zero_count += (1u << Log2(witness_size)) - witness_size;
-        check(grape_memcpy_h2d(hist + (-low_), &zero_count, sizeof(uint32_t), nullptr), "h2d");
+        check(grape_memcpy_h2d(hist + (-low_), &zero_count, sizeof(uint32_t), stream), "h2d");
     }
-    m.get_data(m.size, hist);
+    check(grape_fr_from_u32(W(m.gpu_data), hist, m.size, stream), "grape_fr_from_u32");
     grape_free(d_hist_);
     d_hist_ = hist;                           // kept for the proof in flight: the commitment of A picks its table entries by count
 }
@@ -247,9 +250,10 @@ void tLookup::start_weights(uint D) {
     E_ready_.reset();
     if (u_ready_.size() != nu) return;          // run() reports the mismatch
     E_ready_.reset(new FrTensor((uint)grape_eq_pyramid_elems(nu ? nu - 1 : 0)));
-    fr_t* d_u = grape_host::upload(u_ready_);
+    // the point travels on the second stream too: on the default stream it would queue behind the pass over the
+    // witness, and the pyramid with it
     SideChain side(0);
-    SideChain::order(side.stream, nullptr);     // the point's upload before the pyramid
+    fr_t* d_u = grape_host::upload(u_ready_, side.stream);
     check(grape_eq_pyramid(W(E_ready_->gpu_data), W(d_u), nu ? nu - 1 : 0, side.stream), "grape_eq_pyramid");
     grape_free(d_u);                            // handed out again only after what is queued here
 }
@@ -317,20 +321,6 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     // slot of the ring of grape_host::device_scalar (which is rewritten after 64 further scalars)
     grape_host::DeviceFr beta_buf(beta);
     fr_t* d_beta = beta_buf.get();
-    // A = 1/(S + beta): read from B where the witness matches its table entry (every element of
-    // a valid witness does), computed by batched inversion otherwise (tlookup_inv_kernel,
-    // src/tlookup.cu:52-62, inverts per element)
-    bool from_table = a_ready_;
-    a_ready_ = false;
-    if (!from_table && d_idx_) {
-        size_t mismatches = 0;
-        check(grape_tlookup_inverse_by_table(W(A.gpu_data), W(S.gpu_data), d_idx_, W(T.gpu_data), W(B.gpu_data), D, N, &mismatches, nullptr),
-              "grape_tlookup_inverse_by_table");
-        from_table = mismatches == 0;
-    }
-    if (!from_table) check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
-    A.set_size(D);
-
     // Commitments of A and m (kept, not dropped).  With the scaled table of a range lookup the
     // commitment of A reads only the indices, so it does not have to finish before the rounds start
     // folding A: the rounds are then queued first, on streams of their own, and the commitments run
@@ -353,6 +343,32 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     });
     const bool indexed = indexed_commit_ && index_known_ && scaled_table_;
     const bool overlap = indexed && d_idx_ != nullptr;
+    // A = 1/(S + beta): read from B where the witness matches its table entry (every element of
+    // a valid witness does), computed by batched inversion otherwise (tlookup_inv_kernel,
+    // src/tlookup.cu:52-62, inverts per element).  When prove() found every element in the table and
+    // left A unwritten, the first round gathers it from B - if that round is one of the long ones queued
+    // beside the commitments; otherwise A is written out now.
+    bool from_table = a_ready_;
+    const bool gather_first = a_deferred_ && overlap && D == (1u << Log2(D)) && D / 2 >= kLongRoundPairs && A.size >= D;
+    a_ready_ = false;
+    a_deferred_ = false;
+    if (gather_first) from_table = true;
+    if (!from_table && d_idx_) {
+        size_t mismatches = 0;
+        check(grape_tlookup_inverse_by_table(W(A.gpu_data), W(S.gpu_data), d_idx_, W(T.gpu_data), W(B.gpu_data), D, N, &mismatches, nullptr),
+              "grape_tlookup_inverse_by_table");
+        from_table = mismatches == 0;
+    }
+    if (!from_table) check(grape_fr_shift_inverse(W(A.gpu_data), W(S.gpu_data), W(d_beta), D, nullptr), "grape_fr_shift_inverse");
+    A.set_size(D);
+    if (overlap) {
+        // The previous proof's commitments go now, while the streams are idle: a block that is freed takes the
+        // marks of what the streams hold at that moment, and the allocation that takes it over waits for those -
+        // freed behind the long rounds, the commitments' output buffers would make the host wait for them.
+        grape_free(com_A);
+        grape_free(com_m);
+        com_A = com_m = nullptr;
+    }
     auto commit_all = [&] {
         grape_free(com_A);
         grape_free(com_m);
@@ -380,10 +396,15 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         com_m_rows = N / (m_N * hyrax.com_scale);
         check(grape_stream_sync(nullptr), "sync");
     };
+    // multiplicities that prove() left to this point: counted now, on the default stream, unless the
+    // commitments run beside the rounds - then the count, B * m and its sum follow the long rounds on the
+    // second stream (whose table side and commitment of m are their only readers)
+    if (m_pending_ && !overlap) index_to_m(m_pending_size_, m_pending_low_);
+    const bool m_late = m_pending_;
     if (!overlap) timed(commit_all);
 
     FrTensor Bm(B);
-    Bm *= m;
+    if (!m_late) Bm *= m;
     Fr alpha_sq = alpha * alpha;
     Fr claim = alpha + alpha_sq;
     Fr N_div_D = Fr((long)N) * Fr((long)D).invert();
@@ -410,11 +431,19 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
     // host.  (The reference interleaves a device-to-host copy and a sync with every round.)
     // (The sum of B * m, which only the host's constant term needs, travels with them.)
     const uint rounds = (uint)v.size();
-    FrTensor sums(13 * (rounds ? rounds : 1) + 1);
-    check(grape_fr_sum(W(sums.gpu_data + 13 * (size_t)(rounds ? rounds : 1)), W(Bm.gpu_data), N, nullptr), "grape_fr_sum");
+    // (Three more slots travel with them: the sum of B * m, the last element left of S - the value the proof
+    // returns - and the two digit-range flags of the commitments queued beside the rounds.)
+    const size_t n_sums = 13 * (size_t)(rounds ? rounds : 1);
+    FrTensor sums((uint)n_sums + 3);
+    fr_t* const d_sum_Bm = sums.gpu_data + n_sums;
+    fr_t* const d_S_last = sums.gpu_data + n_sums + 1;
+    int* const d_flags = reinterpret_cast<int*>(sums.gpu_data + n_sums + 2);
+    if (!m_late) check(grape_fr_sum(W(d_sum_Bm), W(Bm.gpu_data), N, nullptr), "grape_fr_sum");
     fr_t* d_v = grape_host::upload(v);
-    int* d_flags = nullptr;
-    FrTensor Bw(B), Tw(T), mw(m);          // phase 2 binds copies; T, B, m of this object stay intact
+    Fr S_last;
+    char* long_work = nullptr;             // partial sums of the long rounds and the challenges' tables (overlap mode)
+    FrTensor Bw(B), Tw(T), mw(N);          // phase 2 binds copies; T, B, m of this object stay intact
+    if (!m_late) check(grape_memcpy_d2d(mw.gpu_data, m.gpu_data, sizeof(fr_t) * (size_t)N, nullptr), "grape_memcpy_d2d");
     try {
         // The table side of phase 2 (B, T, m: sums and folds of the last log2(N) rounds) depends on
         // nothing the witness side produces, so it runs as a chain of its own on a second stream,
@@ -427,6 +456,8 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         uint cur = D;
         uint k = 0;
         int vi = (int)rounds - 1;
+        size_t long_used = 0;
+        int32_t* d_tabs = nullptr;
         // A and S: five sums and the fold of both tensors in one pass
         auto witness_round = [&](grape_stream_t st) {
             const uint half = cur / 2;
@@ -443,7 +474,24 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
                 mode = 3;
                 mid_from_claim[k] = 1;
             }
-            check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), mode, W(slot), st), "grape_wround2");
+            if (long_work && half >= kLongRoundPairs) {
+                // long round beside the commitments: only the pass over the operands stays on the chain of rounds; its
+                // sums are finished on the stream of the short rounds, from a work buffer of the round's own
+                uint32_t* partial = reinterpret_cast<uint32_t*>(long_work + long_used);
+                long_used += grape_wround2_partial_bytes(half);
+                if (k == 0 && gather_first)
+                    check(grape_wround2_queue_indexed(W(A.gpu_data), W(S.gpu_data), d_idx_, W(B.gpu_data), N, W(d_beta), W(e), half, W(d_v + vi),
+                                                      d_tabs + (size_t)GRAPE_FOLD_TABLE_WORDS * (size_t)vi, partial, st),
+                          "grape_wround2_queue_indexed");
+                else
+                    check(grape_wround2_queue(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), mode,
+                                              d_tabs + (size_t)GRAPE_FOLD_TABLE_WORDS * (size_t)vi, partial, st),
+                          "grape_wround2_queue");
+                SideChain::order(witness.stream, st);
+                check(grape_wround2_finish(W(slot), partial, half, mode, witness.stream), "grape_wround2_finish");
+            } else {
+                check(grape_wround2(W(A.gpu_data), W(S.gpu_data), W(d_beta), W(e), cur, half, 1, 1, W(d_v + vi), mode, W(slot), st), "grape_wround2");
+            }
             A.set_size(half);
             S.set_size(half);
             cur = half;
@@ -475,16 +523,27 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         // wave waits for memory, which made the pair slower than one after the other.  The short
         // rounds (launch-bound) do run beside the commitments, on a stream of their own.
         if (overlap) {
+            // work memory of the long rounds (every round its own partial sums) and the tables of all challenges' multiples
+            size_t need = 0;
+            for (uint c = D; c / 2 >= kLongRoundPairs; c /= 2) need += grape_wround2_partial_bytes(c / 2);
+            if (need) {
+                check(grape_malloc((void**)&long_work, need + sizeof(int32_t) * GRAPE_FOLD_TABLE_WORDS * (size_t)rounds), "grape_malloc");
+                d_tabs = reinterpret_cast<int32_t*>(long_work + need);
+                for (uint k0 = 0; k0 < rounds; k0 += 64)
+                    check(grape_fold_tables(d_tabs + (size_t)GRAPE_FOLD_TABLE_WORDS * k0, W(d_v + k0), std::min(64u, rounds - k0), nullptr), "grape_fold_tables");
+            }
             while (vi >= 0 && cur / 2 >= kLongRoundPairs) witness_round(nullptr);
             // The table side and the commitment of m (a few rows: a short accumulation and a latency chain of a
             // row reduction) go to the second stream now, so that they run beside the long rounds and the
             // commitment of A instead of after them; the host gets through these launches while the chip
             // still works on the long rounds.
-            check(grape_malloc((void**)&d_flags, 2 * sizeof(int)), "grape_malloc");
             check(grape_memset_zero(d_flags, 2 * sizeof(int), nullptr), "grape_memset_zero");
-            grape_free(com_A);
-            grape_free(com_m);
-            com_A = com_m = nullptr;
+            if (m_late) {
+                index_to_m(m_pending_size_, m_pending_low_, side.stream);
+                check(grape_fr_mul(W(Bm.gpu_data), W(Bm.gpu_data), W(m.gpu_data), N, side.stream), "grape_fr_mul");
+                check(grape_fr_sum(W(d_sum_Bm), W(Bm.gpu_data), N, side.stream), "grape_fr_sum");
+                check(grape_memcpy_d2d(mw.gpu_data, m.gpu_data, sizeof(fr_t) * (size_t)N, side.stream), "grape_memcpy_d2d");
+            }
             table_side();
             const uint m_N = 1u << (Log2(N) / 2);
             com_m_rows = N / (m_N * hyrax.com_scale);
@@ -506,26 +565,29 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
             check(grape_event_record(commit_events().second, nullptr), "grape_event_record");
         }
         while (vi >= 0) witness_round(ws);
+        check(grape_memcpy_d2d(d_S_last, S.gpu_data, sizeof(fr_t), ws), "grape_memcpy_d2d");   // S(v), behind the last round
         // without the overlap the table side is queued last: its small launches reach the chip while it
         // works on the first, long rounds of the witness side
         if (!overlap) table_side();
         if (overlap) witness.end();
         side.end();                         // the default stream waits for the table side
+        // one copy brings everything the host still needs (and is where it waits for the proof's work)
+        std::vector<Fr> h(n_sums + 3);
+        check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * h.size(), nullptr), "d2h");
         if (overlap) {
-            int flags[2] = {0, 0};
-            check(grape_memcpy_d2h(flags, d_flags, sizeof flags, nullptr), "d2h");
-            grape_free(d_flags);
-            d_flags = nullptr;
+            int flags[2];
+            std::memcpy(flags, &h[n_sums + 2], sizeof flags);
             if (flags[0] || flags[1]) throw std::runtime_error("tLookup: a commitment inside the proof met a scalar outside its table's digits");
             float ms = 0;
             check(grape_event_elapsed_ms(&ms, commit_events().first, commit_events().second), "grape_event_elapsed_ms");
             commit_time += ms * 1e-3;
         }
-        std::vector<Fr> h(13 * (size_t)(rounds ? rounds : 1) + 1);
-        check(grape_memcpy_d2h(h.data(), sums.gpu_data, sizeof(fr_t) * h.size(), nullptr), "d2h");
-        Fr C = alpha_sq - h.back();
+        S_last = h[n_sums + 1];
+        Fr C = alpha_sq - h[n_sums];
         grape_free(d_v);
         d_v = nullptr;
+        grape_free(long_work);
+        long_work = nullptr;
 
         Fr alpha_run = alpha, alpha_sq_run = alpha_sq;
         int ui = (int)nu - 1;      // index of the variable bound in this round (u.back())
@@ -569,22 +631,32 @@ Fr tLookup::run(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax
         }
     } catch (...) {
         grape_free(d_v);
-        grape_free(d_flags);
+        grape_free(long_work);
         throw;
     }
-    return S(0u);
+    return S_last;
 }
 
 Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time) {
     uint D = S.size;
     a_ready_ = false;
     if (D == (1u << Log2(D)) && A.size >= D) {
-        make_index_and_A(S, low, A, nullptr, nullptr);   // no padding: index and A = B[index] together (starts the weights too)
+        // no padding: index and A = B[index] in one pass (starts the weights too); A stays unwritten where the
+        // first round can gather it from B (a witness of 2^17 elements and more, committed through its indices)
+        const bool gather = indexed_commit_ && index_known_ && D / 2 >= (1u << 16);
+        make_index_and_A(S, low, A, nullptr, nullptr, !gather);
     } else {
         start_weights(1u << Log2(D));
         make_index(S, low);
     }
-    index_to_m(D, low);                       // what prep(S) computes, from the shared indices
+    // what prep(S) computes, from the shared indices; a witness that needs no padding leaves it to run()
+    if (D == (1u << Log2(D)) && d_idx_) {
+        m_pending_ = true;
+        m_pending_size_ = D;
+        m_pending_low_ = low;
+    } else {
+        index_to_m(D, low);
+    }
     if (D != (1u << Log2(D))) {
         // src/tlookup.cu:299-305: rows of 11008 padded to 16384 with zeros
         Fr pad_value = Fr::zero();
@@ -595,6 +667,7 @@ Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax
     try {
         ret = run(S, A, v, hyrax, msm_size, commit_time);
     } catch (...) {
+        m_pending_ = false;
         drop_index();
         throw;
     }

@@ -64,11 +64,20 @@ protected:
     void make_index(const FrTensor& vals, int low_);
     // index and A = B[index] in one pass over a witness that needs no padding; cmp / cmp_table: the
     // second component of a mapping lookup and the table's.  Sets a_ready_ when every element matched.
-    void make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table);
+    // write_A = false: the indices and the check only (a_deferred_ when every element matched); the first round then
+    // gathers A from B, or run() writes it out where that round cannot.
+    void make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table, bool write_A = true);
     bool a_ready_ = false;              // A of the proof in flight already holds B[index]
+    bool a_deferred_ = false;           // every element sits in the table, A not written yet
     void drop_index();
     void pad_index(uint N, uint pad_N, uint pad_size, int fill);   // rows of N indices -> rows of pad_N
-    void index_to_m(uint witness_size, int low_);
+    void index_to_m(uint witness_size, int low_, void* stream = nullptr);
+    // prove() may leave the multiplicities to run(): when the commitments are queued beside the rounds, the
+    // counting pass goes to the second stream (where everything that reads m runs) instead of standing between
+    // the pass over the witness and the first round
+    bool m_pending_ = false;
+    uint m_pending_size_ = 0;
+    int m_pending_low_ = 0;
     uint32_t* d_hist_ = nullptr;        // counts per table entry of the proof in flight (made by index_to_m)
     uint hot_min_count_ = 0;
     uint hot_entries_ = 0;

@@ -223,12 +223,12 @@ def tlookup_hist_index(idx1, length, hist=None):
     return hist
 
 
-def tlookup_index_inverse(key, low, B, cmp=None, cmp_table=None):
-    """returns (idx1, A, mismatches)"""
+def tlookup_index_inverse(key, low, B, cmp=None, cmp_table=None, write_A=True):
+    """returns (idx1, A, mismatches); write_A=False: indices and the count only (A is None)"""
     lib = init()
     n = key.shape[0]
     idx1 = torch.empty(n, dtype=torch.int32, device="cuda")
-    A = fr_empty(n)
+    A = fr_empty(n) if write_A else None
     mm = ctypes.c_size_t(0)
     _capi.check(lib.grape_tlookup_index_inverse(_p(idx1), _p(A), _p(key), n, low, B.shape[0], _p(B),
                                                 _p(cmp) if cmp is not None else None, _p(cmp_table) if cmp_table is not None else None,
@@ -373,6 +373,38 @@ def wround2(A, S, beta, e, in_size, n_out, v, plain_sums=False, rowlen=1, rowpad
     _capi.check(lib.grape_wround2(_p(A), _p(S), _p(beta), _p(e), in_size, n_out, rowlen, rowpad, _p(v), mode,
                                   _p(sums), _s()))
     return sums
+
+
+def wround2_split(A, S, beta, e, in_size, n_out, v, plain_sums=False, rowlen=1, rowpad=1, inverse_pair=False, no_middle=False,
+                  table=True):
+    """wround2 through its two halves: the table of the challenge's multiples (table=True and n_out >= 2^16), the
+    pass over the operands into a work buffer of the caller, the finishing of the sums"""
+    lib = init()
+    sums = fr_empty(5 if plain_sums else 3)
+    mode = 3 if no_middle else (2 if inverse_pair else (1 if plain_sums else 0))
+    partial = torch.empty(lib.grape_wround2_partial_bytes(n_out) // 4, dtype=torch.int32, device="cuda")
+    tab = None
+    if table and n_out >= (1 << 16):
+        tab = torch.empty(100, dtype=torch.int32, device="cuda")
+        _capi.check(lib.grape_fold_tables(_p(tab), _p(v), 1, _s()))
+    _capi.check(lib.grape_wround2_queue(_p(A), _p(S), _p(beta), _p(e), in_size, n_out, rowlen, rowpad, _p(v), mode,
+                                        _p(tab), _p(partial), _s()))
+    _capi.check(lib.grape_wround2_finish(_p(sums), _p(partial), n_out, mode, _s()))
+    return sums
+
+
+def wround2_first_indexed(S, idx1, B, beta, e, n_out, v):
+    """first round of a lookup whose logUp tensor A = B[idx1 - 1] was never written out; returns (sums, folded A)"""
+    lib = init()
+    sums = fr_empty(5)
+    A = fr_empty(n_out)
+    partial = torch.empty(lib.grape_wround2_partial_bytes(n_out) // 4, dtype=torch.int32, device="cuda")
+    tab = torch.empty(100, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_fold_tables(_p(tab), _p(v), 1, _s()))
+    _capi.check(lib.grape_wround2_queue_indexed(_p(A), _p(S), _p(idx1), _p(B), B.shape[0], _p(beta), _p(e), n_out, _p(v), _p(tab),
+                                                _p(partial), _s()))
+    _capi.check(lib.grape_wround2_finish(_p(sums), _p(partial), n_out, 2, _s()))
+    return sums, A
 
 
 def sumcheck_round2_seg(A, B, in_size, out_size, seglen, e, v):

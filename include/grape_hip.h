@@ -197,6 +197,37 @@ int grape_eq_pyramid(uint32_t *d_pyr, const uint32_t *d_u, uint32_t nu, grape_st
 int grape_wround2(uint32_t *d_A, uint32_t *d_S, const uint32_t *d_beta, const uint32_t *d_e, uint32_t in_size, uint32_t n_out,
                   uint32_t rowlen, uint32_t rowpad, const uint32_t *d_v, int plain_sums, uint32_t *d_sums, grape_stream_t stream);
 /*
+ * grape_wround2 in two halves, for a prover that queues all rounds of a proof and reads their sums once at the
+ * end (the reference's tLookup_phase1 loop, src/tlookup.cu:216-244, copies and waits once per round): the finishing of
+ * a round's sums is then not part of the chain of rounds and may run on another stream, and the tables of the
+ * challenges' multiples are made by one launch for the whole proof.
+ *   grape_fold_tables:  d_tabs + GRAPE_FOLD_TABLE_WORDS * k (int32 words) receives the table of d_v[k], k < count <= 64.
+ *   grape_wround2_queue: the pass over the operands of grape_wround2 (same arguments and folds); the round's
+ *     per-workgroup sums go to d_partial (grape_wround2_partial_bytes(n_out) bytes, 16-byte aligned, the
+ *     caller's own for as long as the round is unfinished).  d_tab: the table of *d_v made by grape_fold_tables
+ *     (rounds of n_out >= 2^16; plain_sums == 3 requires it) or NULL for the single-product fold.
+ *   grape_wround2_finish: d_sums[0..4] (d_sums[0..2] with plain_sums == 0) from d_partial, as grape_wround2 leaves
+ *     them; n_out and plain_sums as given to grape_wround2_queue.
+ */
+#define GRAPE_FOLD_TABLE_WORDS 100 /* int32 words of one challenge's table */
+size_t grape_wround2_partial_bytes(uint32_t n_out);
+int grape_fold_tables(int32_t *d_tabs, const uint32_t *d_v, uint32_t count, grape_stream_t stream);
+int grape_wround2_queue(uint32_t *d_A, uint32_t *d_S, const uint32_t *d_beta, const uint32_t *d_e, uint32_t in_size, uint32_t n_out,
+                        uint32_t rowlen, uint32_t rowpad, const uint32_t *d_v, int plain_sums, const int32_t *d_tab,
+                        uint32_t *d_partial, grape_stream_t stream);
+int grape_wround2_finish(uint32_t *d_sums, const uint32_t *d_partial, uint32_t n_out, int plain_sums, grape_stream_t stream);
+/*
+ * grape_wround2_queue with plain_sums == 2 for a logUp tensor that was never written out: the first round of a
+ * lookup over 2 n_out elements reads d_A[i] as d_B[d_idx1[i] - 1] (d_idx1 as grape_tlookup_index_inverse leaves it with
+ * d_A == NULL and no unmatched element; an index 0 reads entry 0) and writes the folded tensor to d_A[0 .. n_out);
+ * d_S is folded in place.  d_tab is required (n_out >= 2^16).  Finished by grape_wround2_finish(.., plain_sums = 2).
+ * Together with the pass over the witness this leaves out one write and one read of the whole tensor
+ * (tlookup_inv_kernel's output, src/tlookup.cu:52-62, as the first round's input, :117-151).
+ */
+int grape_wround2_queue_indexed(uint32_t *d_A, uint32_t *d_S, const int32_t *d_idx1, const uint32_t *d_B, uint32_t len,
+                                const uint32_t *d_beta, const uint32_t *d_e, uint32_t n_out, const uint32_t *d_v, const int32_t *d_tab,
+                                uint32_t *d_partial, grape_stream_t stream);
+/*
  * One round of matmul_sumcheck_phase1 (src/prove.cu:49-85): grape_sumcheck_round2 on indices
  * g = seg * seglen + k where every index of a segment carries the weight d_e[seg]
  * (out_size / seglen segments): d_sums[t] = sum_seg d_e[seg] * sum_k coefficient_t(seg, k); A and B
@@ -236,7 +267,9 @@ int grape_tlookup_index_inverse(int32_t *d_idx1, uint32_t *d_A, const uint32_t *
                                 const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table, size_t *mismatches,
                                 grape_stream_t stream);
 /* The same pass queued without waiting: the count of unmatched elements is left in the device word
- * d_mismatches (cleared by the call), for a caller that has more to queue before it reads the count. */
+ * d_mismatches (cleared by the call), for a caller that has more to queue before it reads the count.
+ * d_A == NULL: indices and the count only (a caller whose first round gathers d_B[index] itself,
+ * grape_wround2_queue_indexed). */
 int grape_tlookup_index_inverse_nowait(int32_t *d_idx1, uint32_t *d_A, const uint32_t *d_key, size_t n, int32_t low, uint32_t len,
                                        const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table,
                                        uint32_t *d_mismatches, grape_stream_t stream);

@@ -2,12 +2,16 @@
 // points, for the CPU test-suite.
 #include <cstring>
 #include "../../grape_amd/csrc/fr26.hpp"
+#include "../../grape_amd/csrc/divstep.hpp"
 using namespace grape;
 
 static Fr ld(const uint32_t* p) { Fr x; memcpy(&x, p, 32); return x; }
 static void st(uint32_t* p, const Fr& x) { memcpy(p, &x, 32); }
 
 extern "C" {
+// 1/a by divsteps and by the a^(r-2) ladder, memory form in and out
+void t26_inverse_by(const uint32_t* a, uint32_t* out) { st(out, divstep::inverse_by(ld(a))); }
+void t26_inverse_ladder(const uint32_t* a, uint32_t* out) { st(out, inverse(ld(a))); }
 void t26_mulc(const uint32_t* a, const uint32_t* b, uint32_t* out) { st(out, fr26::mulc(ld(a), ld(b))); }
 void t26_from_mont(const uint32_t* a, uint32_t* out) { st(out, fr26::from_montc(ld(a))); }
 void t26_to_mont(const uint32_t* a, uint32_t* out) { st(out, fr26::to_montc(ld(a))); }

@@ -18,7 +18,7 @@ R = br.R_MOD
 
 @pytest.fixture(scope="module")
 def lib():
-    deps = [SRC] + [os.path.join(HERE, "..", "grape_amd", "csrc", f) for f in ("fr26.hpp", "field.hpp")]
+    deps = [SRC] + [os.path.join(HERE, "..", "grape_amd", "csrc", f) for f in ("fr26.hpp", "field.hpp", "divstep.hpp")]
     if not os.path.exists(LIB) or any(os.path.getmtime(d) > os.path.getmtime(LIB) for d in deps):
         subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-unknown-pragmas"]
                               + (["-DGRAPE_CURVE_BN254"] if BN else []) + ["-o", LIB, SRC])
@@ -55,6 +55,20 @@ def test_mulc_and_montgomery(lib):
         assert np.array_equal(out, plain)
         lib.t26_to_mont(_u32(plain), _u32(out))
         assert np.array_equal(out, pa)
+
+
+def test_inverse_by_divsteps(lib):
+    """1/a through batched divsteps on 30-bit limbs against pow(a, -1, r) and against the a^(r-2) ladder it
+    replaces at the top level of a batched inversion; 1/0 = 0 as in the reference"""
+    rng = random.Random(7)
+    vals = EDGE + [rng.randrange(R) for _ in range(300)] + [rng.randrange(1 << k) for k in (1, 5, 30, 31, 60, 61, 90, 200)]
+    out, out2 = np.zeros(8, dtype=np.uint32), np.zeros(8, dtype=np.uint32)
+    for a in vals:
+        lib.t26_inverse_by(_u32(_p([a])[0]), _u32(out))
+        lib.t26_inverse_ladder(_u32(_p([a])[0]), _u32(out2))
+        want = pow(a, -1, R) if a % R else 0
+        assert _val(out) == want, hex(a)
+        assert _val(out2) == want, hex(a)
 
 
 def test_integer_embedding(lib):

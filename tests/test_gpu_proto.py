@@ -370,6 +370,69 @@ def test_weighted_round_without_its_middle_coefficient(ops, in_size, n_out):
                                                                2 * n_out, v, 2, 0, n_out)[:1000], "folded A against the oracle")
 
 
+@pytest.mark.parametrize("in_size,n_out,mode", [(1 << 17, 1 << 16, "no_middle"), ((1 << 18) - 1000, 1 << 17, "plain"), (1 << 19, 1 << 18, "three"),
+                                                 (6000, 4096, "plain"), (1 << 18, 1 << 17, "no_table")])
+def test_weighted_round_in_two_halves(ops, in_size, n_out, mode):
+    """grape_fold_tables + grape_wround2_queue + grape_wround2_finish (work buffer and table of the caller's, finishing
+    apart from the pass) against grape_wround2 on the same operands: sums and folds bit for bit"""
+    logh = br.log2ceil(n_out)
+    A, S = rand_fr(in_size, 301 + n_out), rand_fr(in_size, 302 + n_out)
+    bt, v, u = rand_fr(1, 303), rand_fr(1, 304), rand_fr(logh, 305)
+    e = ops.eq_pyramid(ops.to_dev(u), logh)[n_out - 1:2 * n_out - 1].contiguous()
+    kw = dict(plain_sums=mode != "three", no_middle=mode == "no_middle")
+    dA1, dS1, dA2, dS2 = ops.to_dev(A), ops.to_dev(S), ops.to_dev(A), ops.to_dev(S)
+    whole = ops.fr_to_host(ops.wround2(dA1, dS1, ops.to_dev(bt), e, in_size, n_out, ops.to_dev(v), **kw))
+    halves = ops.fr_to_host(ops.wround2_split(dA2, dS2, ops.to_dev(bt), e, in_size, n_out, ops.to_dev(v), table=mode != "no_table", **kw))
+    assert_same(halves, whole, "sums")
+    assert_same(ops.fr_to_host(dA2)[:n_out], ops.fr_to_host(dA1)[:n_out], "folded A")
+    assert_same(ops.fr_to_host(dS2)[:n_out], ops.fr_to_host(dS1)[:n_out], "folded S")
+
+
+@pytest.mark.parametrize("n_out", [1 << 16, 1 << 18])
+def test_first_round_gathers_the_logup_tensor_from_its_table(ops, n_out):
+    """a witness whose pass left only the table indices (A unwritten): the first round reads A[i] = B[index_i] itself and
+    gives the sums, the folded A and the folded S of the round over the written-out tensor"""
+    import torch
+    low, length = -20000, 1 << 16
+    n = 2 * n_out
+    s = np.random.default_rng(311 + n_out).integers(low, low + length, size=n).astype(np.int32)
+    vals = ops.fr_from_i32(torch.from_numpy(s).cuda())
+    beta = ops.to_dev(br.fr_pack([length]))
+    T, B = ops.tlookup_init(low, length, beta)
+    idx_a, A, mism = ops.tlookup_index_inverse(vals, low, B)
+    idx_b, none, mism_b = ops.tlookup_index_inverse(vals, low, B, write_A=False)
+    assert mism == 0 and mism_b == 0 and none is None and torch.equal(idx_a, idx_b)
+    logh = br.log2ceil(n_out)
+    v, u = rand_fr(1, 312), rand_fr(logh, 313)
+    e = ops.eq_pyramid(ops.to_dev(u), logh)[n_out - 1:2 * n_out - 1].contiguous()
+    S1, S2 = vals.clone(), vals.clone()
+    whole = ops.fr_to_host(ops.wround2(A, S1, beta, e, n, n_out, ops.to_dev(v), plain_sums=True, inverse_pair=True))
+    sums, A2 = ops.wround2_first_indexed(S2, idx_b, B, beta, e, n_out, ops.to_dev(v))
+    assert_same(ops.fr_to_host(sums), whole, "five sums")
+    assert_same(ops.fr_to_host(A2), ops.fr_to_host(A)[:n_out], "folded A")
+    assert_same(ops.fr_to_host(S2)[:n_out], ops.fr_to_host(S1)[:n_out], "folded S")
+    # an element outside the table is counted by the index-only pass too
+    s[5] = low + length + 9
+    _, _, mism_c = ops.tlookup_index_inverse(ops.fr_from_i32(torch.from_numpy(s).cuda()), low, B, write_A=False)
+    assert mism_c == 1
+
+
+def test_fold_tables_of_several_challenges(ops):
+    """one launch makes the tables of up to 64 challenges: table k equals the table made for challenge k alone"""
+    import torch
+    from grape_amd import _capi
+    lib = ops.init()
+    v = ops.to_dev(rand_fr(24, 306))
+    many = torch.zeros(24 * 100, dtype=torch.int32, device="cuda")
+    _capi.check(lib.grape_fold_tables(ops._p(many), ops._p(v), 24, None))
+    for k in (0, 7, 23):
+        one = torch.zeros(100, dtype=torch.int32, device="cuda")
+        _capi.check(lib.grape_fold_tables(ops._p(one), ops._p(v[k:k + 1].contiguous()), 1, None))
+        assert torch.equal(many[100 * k:100 * k + 100], one)
+    with pytest.raises(_capi.GrapeError):
+        _capi.check(lib.grape_fold_tables(ops._p(many), ops._p(v), 65, None))
+
+
 @pytest.mark.parametrize("n_out,beta", [(1, True), (4096, True), (1 << 17, True), ((1 << 18), False)])
 def test_weighted_round_of_an_inverse_pair(ops, n_out, beta):
     """the first round of a logUp proof, where A = 1/(S + beta): the variant that takes only the top
