@@ -98,6 +98,7 @@ SIGNATURES = {
     "grape_commit_i32": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_i32_nowait": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p, c_void_p],
     "grape_commit_fr": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
+    "grape_commit_fr_nowait": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p, c_void_p],
     "grape_g1_strided_table_gen": [c_void_p, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_fr_strided": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_u32, c_u32, c_u32, c_void_p],
     "grape_commit_i32_ref_table": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p, c_size_t, c_void_p],

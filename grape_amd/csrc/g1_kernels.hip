@@ -1303,6 +1303,11 @@ int grape_commit_fr(uint32_t* out, const uint32_t* scalars, size_t size, uint32_
                     uint32_t c, uint32_t nw, uint32_t K, grape_stream_t st) {
     return commit_wide_impl<true>(out, scalars, size, rowlen, table, N, c, nw, K, st);
 }
+int grape_commit_fr_nowait(uint32_t* out, const uint32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table, size_t N,
+                           uint32_t c, uint32_t nw, uint32_t K, int32_t* d_flag, grape_stream_t st) {
+    GRAPE_REQUIRE(d_flag != nullptr, "the caller's flag is required");
+    return commit_wide_impl<true>(out, scalars, size, rowlen, table, N, c, nw, K, st, d_flag);
+}
 
 int grape_commit_i32_ref_table(uint32_t* out, const int32_t* scalars, size_t size, uint32_t rowlen, const uint32_t* table,
                                size_t npoints, grape_stream_t st) {

@@ -246,32 +246,37 @@ bool Hyrax::ensure_strided_table(uint rowlen, bool build) {
     return true;
 }
 
-void Hyrax::commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build) {
+bool Hyrax::commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build, void* stream, int* d_flag) {
     // one row only (an opening's blinding row): a table that is already there is used, none is built for it,
     // and the per-window table is preferred - its 20 additions per scalar are nothing for one row, while the
     // strided table's (J-1)*c doublings per row are a chain of half a millisecond on one lane
     const bool single = size == rowlen;
     if (single && ensure_fr_table(rowlen, false)) {
         const WideTable& t = fr_table_;
-        check(grape_commit_fr(W(out), W(scalars), size, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, nullptr), "grape_commit_fr");
+        if (d_flag) {
+            check(grape_commit_fr_nowait(W(out), W(scalars), size, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, d_flag, stream), "grape_commit_fr_nowait");
+            return true;
+        }
+        check(grape_commit_fr(W(out), W(scalars), size, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, stream), "grape_commit_fr");
     } else if (ensure_strided_table(rowlen, may_build)) {
         const StridedTable& t = fr_strided_;
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
-                  return grape_commit_fr_strided(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.J, t.nsets, nullptr);
+                  return grape_commit_fr_strided(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.J, t.nsets, stream);
               }),
               "grape_commit_fr_strided");
     } else if (ensure_fr_table(rowlen, false)) {
         const WideTable& t = fr_table_;
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
-                  return grape_commit_fr(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, nullptr);
+                  return grape_commit_fr(W(out + r0), W(scalars + e0), n, rowlen, W(t.d), t.ngen, t.c, t.nw, t.K, stream);
               }),
               "grape_commit_fr");
     } else {
         check(for_row_chunks(size, rowlen, [&](size_t e0, size_t n, size_t r0) {
-                  return grape_commit_fr_ref_table(W(out + r0), W(scalars + e0), n, rowlen, W(g_affine), npoints, nullptr);
+                  return grape_commit_fr_ref_table(W(out + r0), W(scalars + e0), n, rowlen, W(g_affine), npoints, stream);
               }),
               "grape_commit_fr_ref_table");
     }
+    return false;
 }
 
 affine_t* Hyrax::commit_affine(FrTensor& tensor, uint size, uint N) {
@@ -391,10 +396,23 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     for (uint i = 0; i < new_N; i++) host_d[i] = Fr::random_element();
     FrTensor d = FrTensor::from_host(host_d);
 
-    // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185)
+    // commitment of d: one row of new_N full-width scalars (single_commit, src/Hyrax.cu:176-185).  A short
+    // accumulation and then a latency chain (the row's reduction), so it runs on a stream of its own beside the folds
+    // of the tensor below; nothing below writes to d.
+    static grape_stream_t open_stream = nullptr;      // lives as long as the process
+    static void* d_uploaded = nullptr;
+    if (!open_stream) {
+        check(grape_stream_create(&open_stream), "grape_stream_create");
+        check(grape_event_create(&d_uploaded), "grape_event_create");
+    }
+    check(grape_event_record(d_uploaded, nullptr), "grape_event_record");        // a short d travels as a queued launch
+    check(grape_stream_wait_event(open_stream, d_uploaded), "grape_stream_wait_event");
+    // (the point and, behind it, the digit-range flag of a commitment queued without waiting)
     affine_t* com_d_dev = nullptr;
-    check(grape_malloc((void**)&com_d_dev, sizeof(affine_t)), "grape_malloc");
-    commit_fr_rows(com_d_dev, d.gpu_data, new_N, new_N, false);
+    check(grape_malloc((void**)&com_d_dev, sizeof(affine_t) + 16), "grape_malloc");
+    int* d_flag = reinterpret_cast<int*>(com_d_dev + 1);
+    check(grape_memset_zero(d_flag, sizeof(int), open_stream), "grape_memset_zero");
+    const bool flag_used = commit_fr_rows(com_d_dev, d.gpu_data, new_N, new_N, false, open_stream, d_flag);
 
     FrTensor x(new_N);
     tensor.partial_eval(size, eval_point, (size / layer_num) / (N * com_scale), Log2(N * com_scale), N * com_scale);
@@ -410,13 +428,21 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     z *= c;
     z += d;
 
-    d.partial_eval(d.size, eval_point, new_N, 0, 1);
-    Fr sum_ad = grape_host::download(d.gpu_data);
+    FrTensor d_fold(d);                         // folded in place: a copy, the commitment may still be reading d
+    d_fold.partial_eval(d_fold.size, eval_point, new_N, 0, 1);
+    Fr sum_ad = grape_host::download(d_fold.gpu_data);
     if (!G_multiples_) G_multiples_.reset(new G1FixedBase(G));
     bn128 commit_ad = G_multiples_->mul(sum_ad);
 
-    affine_t host_com_d;
-    check(grape_memcpy_d2h(&host_com_d, com_d_dev, sizeof(affine_t), nullptr), "d2h");
+    struct { affine_t p; int flag[4]; } com_d_host;
+    static_assert(sizeof(com_d_host) == sizeof(affine_t) + 16, "point and flag travel together");
+    check(grape_memcpy_d2h(&com_d_host, com_d_dev, sizeof(com_d_host), open_stream), "d2h");     // waits for the commitment
+    if (flag_used && com_d_host.flag[0]) {
+        grape_free(com_d_dev);
+        grape_free(eval_point);
+        throw std::runtime_error("Hyrax::open: a blinding scalar does not fit the table's digit range");
+    }
+    const affine_t& host_com_d = com_d_host.p;
     Hyrax_proof proof(result, new_N, bn128(host_com_d), commit_ad);
     check(grape_memcpy_d2h(proof.z, z.gpu_data, sizeof(fr_t) * (size_t)new_N, nullptr), "d2h");
     grape_free(com_d_dev);

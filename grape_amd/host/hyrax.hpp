@@ -108,7 +108,9 @@ private:
     bool ensure_strided_table(uint rowlen, bool build = true);  // the table full-width commitments go through
     size_t table_bytes_in_use() const;
     // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
-    void commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build);
+    // d_flag (single rows through the per-window table only): queued without waiting, digit-range check left in *d_flag;
+    // returns whether it was queued that way (false: the call has waited and checked)
+    bool commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build, void* stream = nullptr, int* d_flag = nullptr);
     void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag, void* stream = nullptr);
     void check_shape(uint size, uint N) const;
     WideTable int16_table_, int16x2_table_, int32_table_, fr_table_;

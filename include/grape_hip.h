@@ -419,6 +419,11 @@ int grape_commit_i32_nowait(uint32_t *d_out_affine, const int32_t *d_scalars, si
  * never carries out. */
 int grape_commit_fr(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
                     const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, grape_stream_t stream);
+/* grape_commit_fr without the wait at its end, *d_flag as in grape_commit_i32_nowait: for Hyrax::open
+ * (src/Hyrax.cu:237-305), whose blinding row is committed beside the folds of the opened tensor. */
+int grape_commit_fr_nowait(uint32_t *d_out_affine, const uint32_t *d_scalars_mont, size_t size, uint32_t rowlen,
+                           const uint32_t *d_wide_table, size_t N, uint32_t c, uint32_t nw, uint32_t K, int32_t *d_flag,
+                           grape_stream_t stream);
 /*
  * Strided fixed-base table: table[(q*K + (k-1))*N + i] = k * 2^(c*J*q) * G_i, k = 1..K = 2^(c-1), q < nsets
  * (the same entry format as the wide table; size grape_g1_wide_table_bytes(N, nsets, K)), and the
