@@ -120,6 +120,7 @@ def layer_workload(args):
     host.load()
     host.load().grape_host_seed(12345)          # seeds the host classes' challenge generator
     host.set_input_format("i32")                # the host calls embed the integer tensors themselves (FrTensor::get_data)
+    host.set_int_folds(not args.no_int_folds)   # ... except where an opening or an evaluation can fold the integers directly
     T, D, H, HD, F = args.seq, 4096, 32, 128, 11008
     FP = 16384                                  # rows of 11008 are padded to 16384 (src/tlookup.cu:301)
     SH = 16
@@ -369,6 +370,10 @@ def layer_workload(args):
                    "scope": "wall clock of every proof block between two device synchronisations, as the reference's "
                             "total_prove_time (test/llm.cu:69-125): integer tensors -> Fr, copies, claim evaluation, sub-proof, "
                             "Hyrax openings; plus the 7 weight commitments; witness generation outside",
+                   "integer_tensors": ("openings and claim evaluations fold their integer tensors directly (Hyrax::open(const int*), "
+                                       "FrTensor::eval_ints): same values, the embedded tensor is never written; the sub-provers embed theirs "
+                                       "with FrTensor::get_data") if not args.no_int_folds else
+                                      "every integer tensor is embedded with FrTensor::get_data before its proof step (--no-int-folds)",
                    "wall_breakdown_s": last["wall_breakdown_s"],
                    "provers_only_s": float(np.mean([r["provers_only_s"] for r in runs])),
                    "provers_breakdown_s": last["provers_breakdown_s"],
@@ -877,6 +882,9 @@ def main():
                     help="commit workload: skip the second measurement (the same steps queued without waiting on three streams)")
     ap.add_argument("--no-spread", action="store_true",
                     help="layer workload: skip the two extra layers whose softmax scores are spread over the whole table")
+    ap.add_argument("--no-int-folds", action="store_true",
+                    help="layer workload: openings and claim evaluations embed their integer tensors first (get_data + open / operator()) "
+                         "instead of folding the integers directly")
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
     ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")
@@ -1116,7 +1124,7 @@ def layer_in_child():
         d = json.loads(lines[-1])
         c = d["config"]
         return {"value": d["value"], "unit": "s", "steps": d["steps"], "warmup": d["warmup"], "workload": c["workload"],
-                "scope": c["scope"], "wall_breakdown_s": c["wall_breakdown_s"], "provers_only_s": c["provers_only_s"],
+                "scope": c["scope"], "integer_tensors": c["integer_tensors"], "wall_breakdown_s": c["wall_breakdown_s"], "provers_only_s": c["provers_only_s"],
                 "provers_breakdown_s": c["provers_breakdown_s"], "step_s": c["step_s"],
                 "cold_s": c["cold_s"], "cold_wall_breakdown_s": c["cold"]["wall_breakdown_s"] if c["cold"] else None,
                 "spread_s": c["spread_s"], "spread_wall_breakdown_s": c["spread"]["wall_breakdown_s"] if c["spread"] else None,

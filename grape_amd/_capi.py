@@ -50,6 +50,8 @@ SIGNATURES = {
     "grape_i32_pad": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_void_p],
     "grape_i32_pad_fill": [c_void_p, c_void_p, c_u32, c_u32, c_size_t, c_i32, c_void_p],
     "grape_fr_fold": [c_void_p, c_size_t, c_void_p, c_u32, c_u32, c_u32, c_void_p],
+    "grape_fr_fold_i32_elems": [c_size_t, c_u32, c_u32],
+    "grape_fr_fold_i32": [c_void_p, c_void_p, c_size_t, c_void_p, c_u32, c_u32, c_u32, c_void_p],
     "grape_sumcheck_round2": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_claim": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_sumcheck_round2_noalloc": [c_void_p, c_void_p, c_u32, c_u32, c_void_p, c_void_p, c_void_p],
@@ -129,7 +131,7 @@ SIGNATURES = {
     "grape_event_elapsed_ms": [ctypes.POINTER(ctypes.c_float), c_void_p, c_void_p],
 }
 _RESTYPES = {"grape_last_error": ctypes.c_char_p, "grape_g1_wide_table_bytes": c_size_t, "grape_eq_pyramid_elems": c_size_t,
-             "grape_wround2_partial_bytes": c_size_t}
+             "grape_wround2_partial_bytes": c_size_t, "grape_fr_fold_i32_elems": c_size_t}
 
 _lib = None
 

@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(_HERE, "host", "libgrape_host_bn254.so" if CURVE == "bn2
 G1W = FP_WORDS              # u64 words of an affine point (2 coordinates of FP_WORDS / 2)
 _lib = None
 
-NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_set_input_format", "grape_host_prove_matmul", "grape_host_prove_elemul",
+NAMES = ["grape_host_last_error", "grape_host_seed", "grape_host_last_prove_seconds", "grape_host_last_commit_seconds", "grape_host_set_indexed_commit", "grape_host_set_input_format", "grape_host_set_int_folds", "grape_host_prove_matmul", "grape_host_prove_elemul",
          "grape_host_combine_claims", "grape_host_mle_eval", "grape_host_hyrax_commit_i32", "grape_host_hyrax_commit_fr",
          "grape_host_hyrax_open_verify", "grape_host_hyrax_open", "grape_host_tlookup_range_prove", "grape_host_tlookup_mapping_prove", "grape_host_tlookup_mapping_prove_ex",
          "grape_host_fr_op", "grape_host_g1_mul_generator", "grape_host_bin_io", "grape_host_findsize", "grape_host_load_data",
@@ -55,6 +55,11 @@ def set_input_format(fmt):
     """0: tensor arguments are field elements (default); 1: int32 values that each call embeds itself"""
     if load().grape_host_set_input_format({"fr": 0, "i32": 1}[fmt]) != 0:
         raise HostError("unknown input format")
+
+
+def set_int_folds(on):
+    """with int32 inputs: openings and evaluations fold the integers directly (default) or embed them first"""
+    load().grape_host_set_int_folds(1 if on else 0)
 
 
 def last_commit_seconds():

@@ -199,6 +199,8 @@ struct FoldPlan {
     uint32_t lo[kFoldMaxPasses];      // the pass binds challenges lo .. lo+b-1
     uint32_t b[kFoldMaxPasses];
     uint32_t off[kFoldMaxPasses];     // first weight of the pass in the weight buffer
+    uint32_t first_plain;             // pass 0 reads plain integers: its weights carry the factor 2^256 that brings
+                                      // a product with a plain value into memory form
 };
 
 // Weights of every pass of a fold, in the 26-bit working form with the radix factor 16 folded
@@ -219,7 +221,8 @@ __global__ void __launch_bounds__(kBlock) fold_weights_kernel(int32_t* wts, cons
 #pragma unroll
         for (int k = 0; k < width; k++) f[k] = fr26::mulc(f[2 * k], f[2 * k + 1]);
     }
-    const Fr acc = f[0];
+    Fr acc = f[0];
+    if (p == 0 && plan.first_plain) acc = fr26::mulc(acc, Fr::rr());
     const fr26::Limbs w = fr26::weight16(acc);
     int32_t* dst = wts + (size_t)fr26::N * (plan.off[p] + threadIdx.x);
 #pragma unroll
@@ -229,7 +232,10 @@ __global__ void __launch_bounds__(kBlock) fold_weights_kernel(int32_t* wts, cons
 // One pass.  A workgroup is 4 waves: 4/S groups of 64 outputs, each output summed by S waves
 // that take every S-th term; the partial sums meet in LDS.  The weight index is wave-uniform, so
 // the weights arrive through scalar loads and cost no vector registers.
-template <int S>
+// I32: the input is a tensor of 32-bit integers (the value x stands for the field element x, negative values for
+// r - |x|): an element is two signed limbs, a product 20 multiply-adds, and 4 bytes are read where the embedded
+// tensor has 32 - the pass that folds an integer tensor without first writing it out as field elements.
+template <int S, bool I32 = false>
 __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* __restrict__ out, const uint32_t* __restrict__ in,
                                                            const int32_t* __restrict__ wts, uint32_t n_hi_max,
                                                            uint32_t outer, uint32_t c, uint32_t lg_c_lo, uint32_t gap) {
@@ -247,7 +253,8 @@ __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* __restrict_
     const uint32_t o = live ? tid / inner : 0;
     const uint32_t p = live ? tid - o * inner : 0;  // i_lo*gap + g
     const uint32_t i_lo = p / gap;
-    const uint32_t* src = in + 8 * ((size_t)o * c * gap + p);
+    const uint32_t* src = in + (I32 ? 1 : 8) * ((size_t)o * c * gap + p);
+    const int32_t* isrc = reinterpret_cast<const int32_t*>(src);
     const size_t hi_stride = (size_t)c_lo * gap;    // elements between consecutive i_hi
     // number of i_hi with i_hi*c_lo + i_lo < c (zero for a dead lane)
     const uint32_t n_hi = live ? (c - i_lo + c_lo - 1) >> lg_c_lo : 0;
@@ -259,19 +266,33 @@ __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* __restrict_
     // wave-uniform offsets and four loads in flight per lane (a dead lane reads the terms of
     // output 0 and stores nothing).  A ragged last term (c not a multiple of c_lo) follows
     // under a lane predicate, in the part whose turn it is.
-    constexpr int U = 4;
+    constexpr int U = I32 ? 8 : 4;
     const uint32_t n_full = c >> lg_c_lo;
     uint32_t h = (uint32_t)part;
-    for (; h + (U - 1) * S < n_full; h += U * S) {
-        Fr t[U];
+    // an integer x = l0 + 2^26 l1 with 0 <= l0 < 2^26, -32 <= l1 < 32: a column grows by < 2^53 per term
+    auto mac_int = [&](const fr26::Limbs& w, int32_t xv) {
+        const int64_t l0 = (int64_t)(xv & (int32_t)fr26::MASK), l1 = (int64_t)(xv >> fr26::W);
 #pragma unroll
-        for (int k = 0; k < U; k++) t[k] = ld_fr(src, (size_t)(h + k * S) * hi_stride);
+        for (int j = 0; j < fr26::N; j++) {
+            C.c[j] += (int64_t)w.v[j] * l0;
+            C.c[j + 1] += (int64_t)w.v[j] * l1;
+        }
+    };
+    for (; h + (U - 1) * S < n_full; h += U * S) {
+        Fr t[I32 ? 1 : U];
+        int32_t ti[I32 ? U : 1];
+#pragma unroll
+        for (int k = 0; k < U; k++) {
+            if (I32) ti[k] = isrc[(size_t)(h + k * S) * hi_stride];
+            else t[k] = ld_fr(src, (size_t)(h + k * S) * hi_stride);
+        }
 #pragma unroll
         for (int k = 0; k < U; k++) {
             fr26::Limbs w;
 #pragma unroll
             for (int j = 0; j < fr26::N; j++) w.v[j] = wts[(size_t)fr26::N * (h + k * S) + j];
-            fr26::mac(C, w, fr26::pack(t[k]));
+            if (I32) mac_int(w, ti[k]);
+            else fr26::mac(C, w, fr26::pack(t[k]));
         }
     }
     for (; h < n_hi_max; h += S) {
@@ -279,7 +300,8 @@ __global__ void __launch_bounds__(kBlock) fold_pass_kernel(uint32_t* __restrict_
             fr26::Limbs w;
 #pragma unroll
             for (int j = 0; j < fr26::N; j++) w.v[j] = wts[(size_t)fr26::N * h + j];
-            fr26::mac(C, w, ld_l26(src, (size_t)h * hi_stride));
+            if (I32) mac_int(w, isrc[(size_t)h * hi_stride]);
+            else fr26::mac(C, w, ld_l26(src, (size_t)h * hi_stride));
         }
     }
     fr26::Limbs r = fr26::reduce(C, 0);
@@ -541,69 +563,83 @@ int grape_i32_pad_fill(int32_t* out, const int32_t* in, uint32_t N, uint32_t pad
     return GRAPE_OK;
 }
 
-int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
+// Plan of a fold's passes: each binds as many top bits as possible (6, or more when the outputs are
+// too few to fill the chip and S waves share one output), until the slab of one outer index
+// fits the LDS finish kernel.
+struct FoldPass { uint32_t b, S, off; };
+static int plan_fold(size_t outer, uint32_t c, uint32_t gap, uint32_t id, FoldPass* passes, FoldPlan& plan) {
+    plan.npass = 0;
+    plan.first_plain = 0;
+    uint32_t l = log2ceil(c), off = 0;
+    size_t cc = c;
+    while (l > 0 && !fold_small_fits(outer, cc, gap)) {
+        // Measured on MI355X: a pass streams fastest with one thread per output, 16 to 64
+        // terms per thread and 2^20 threads; 2^19 threads come close.  Failing that, up to
+        // four waves share an output to reach 2^19 threads.
+        uint32_t S = 0, b = 0;
+        auto items = [&](uint32_t tb) { return outer * gap * ((size_t)1 << (l - tb)); };
+        for (uint32_t want = 20; want >= 19 && S == 0; want--) {
+            for (uint32_t tb = l < 6 ? l : 6; tb >= 4 && S == 0; tb--) {
+                if (items(tb) >= ((size_t)1 << want)) { S = 1; b = tb; }
+            }
+        }
+        for (uint32_t tb = l < 8 ? l : 8; tb >= 4 && S == 0; tb--) {
+            const uint32_t ts = items(tb) * 2 >= ((size_t)1 << 19) ? 2 : 4;
+            if (items(tb) * ts >= ((size_t)1 << 19) && (1u << tb) <= 64 * ts) { S = ts; b = tb; }
+        }
+        if (S == 0) {
+            // too few outputs to fill the chip whatever the split: four waves per output and
+            // at most 32 terms per thread keep the pass short
+            S = 4; b = l <= 7 ? l : 6;
+            // few, short slabs: stop as soon as the LDS finish kernel can take over
+            if (outer <= (size_t)kFoldSmallMaxOuter && gap <= (size_t)kFoldSmallElems) {
+                uint32_t keep = 0;      // bits the finish kernel can bind
+                while (keep < l && (((size_t)2 << keep) * gap) <= (size_t)kFoldSmallElems) keep++;
+                if (l > keep && l - keep < b) b = l - keep;
+            }
+        }
+        GRAPE_REQUIRE(plan.npass < (uint32_t)kFoldMaxPasses, "fold: too many passes");
+        passes[plan.npass] = {b, S, off};
+        plan.lo[plan.npass] = id + (l - b);
+        plan.b[plan.npass] = b;
+        plan.off[plan.npass] = off;
+        plan.npass++;
+        off += 1u << b;
+        l -= b;
+        const size_t c_lo = (size_t)1 << l;
+        cc = cc < c_lo ? cc : c_lo;
+    }
+    return GRAPE_OK;
+}
+
+// grape_fr_fold on t, or - with `ints` - the fold of the integer tensor `ints` left in t: the first pass reads the
+// integers (4 bytes per element) and writes field elements, the later passes work on those as before.
+static int fold_impl(uint32_t* t, const int32_t* ints, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
     if (N == 0) return GRAPE_OK;
     CHECK_PTR16(t); CHECK_PTR16(x);
     GRAPE_REQUIRE(c >= 1 && gap >= 1 && N >= (size_t)c * gap && N % ((size_t)c * gap) == 0, "N must be a multiple of c*gap");
     hipStream_t s = as_stream(st);
     const size_t outer = N / ((size_t)c * gap);
     uint32_t L = log2ceil(c);
+    FoldPass passes[kFoldMaxPasses];
+    FoldPlan plan;
+    int prc = plan_fold(outer, c, gap, id, passes, plan);
+    if (prc) return prc;
+    if (ints && (L == 0 || plan.npass == 0)) {
+        // nothing to bind, or a tensor small enough for the finish kernel alone: embedded first (N elements of t)
+        from_i32_kernel<<<blocks_for(N), kBlock, 0, s>>>(t, ints, N);
+        GRAPE_LAUNCH_CHECK();
+        ints = nullptr;
+    }
     if (L == 0) return GRAPE_OK;   // c == 1: nothing to bind, data already compact
+    plan.first_plain = ints ? 1u : 0u;
     const uint32_t* xs = x + 8 * (size_t)id;
     size_t cur_c = c;
-    const uint32_t* src = t;
+    const uint32_t* src = ints ? reinterpret_cast<const uint32_t*>(ints) : t;
     // With a single outer index a pass can run in place (thread p reads p + k*stride only).
     // Otherwise passes ping-pong through scratch and the result is copied to the front.
     uint32_t* ws[2] = {nullptr, nullptr};
     int which = 0;
-    // Plan the passes: each binds as many top bits as possible (6, or more when the outputs are
-    // too few to fill the chip and S waves share one output), until the slab of one outer index
-    // fits the LDS finish kernel.
-    struct FoldPass { uint32_t b, S, off; };
-    FoldPass passes[kFoldMaxPasses];
-    FoldPlan plan;
-    plan.npass = 0;
-    {
-        uint32_t l = L, off = 0;
-        size_t cc = c;
-        while (l > 0 && !fold_small_fits(outer, cc, gap)) {
-            // Measured on MI355X: a pass streams fastest with one thread per output, 16 to 64
-            // terms per thread and 2^20 threads; 2^19 threads come close.  Failing that, up to
-            // four waves share an output to reach 2^19 threads.
-            uint32_t S = 0, b = 0;
-            auto items = [&](uint32_t tb) { return outer * gap * ((size_t)1 << (l - tb)); };
-            for (uint32_t want = 20; want >= 19 && S == 0; want--) {
-                for (uint32_t tb = l < 6 ? l : 6; tb >= 4 && S == 0; tb--) {
-                    if (items(tb) >= ((size_t)1 << want)) { S = 1; b = tb; }
-                }
-            }
-            for (uint32_t tb = l < 8 ? l : 8; tb >= 4 && S == 0; tb--) {
-                const uint32_t ts = items(tb) * 2 >= ((size_t)1 << 19) ? 2 : 4;
-                if (items(tb) * ts >= ((size_t)1 << 19) && (1u << tb) <= 64 * ts) { S = ts; b = tb; }
-            }
-            if (S == 0) {
-                // too few outputs to fill the chip whatever the split: four waves per output and
-                // at most 32 terms per thread keep the pass short
-                S = 4; b = l <= 7 ? l : 6;
-                // few, short slabs: stop as soon as the LDS finish kernel can take over
-                if (outer <= (size_t)kFoldSmallMaxOuter && gap <= (size_t)kFoldSmallElems) {
-                    uint32_t keep = 0;      // bits the finish kernel can bind
-                    while (keep < l && (((size_t)2 << keep) * gap) <= (size_t)kFoldSmallElems) keep++;
-                    if (l > keep && l - keep < b) b = l - keep;
-                }
-            }
-            GRAPE_REQUIRE(plan.npass < (uint32_t)kFoldMaxPasses, "fold: too many passes");
-            passes[plan.npass] = {b, S, off};
-            plan.lo[plan.npass] = id + (l - b);
-            plan.b[plan.npass] = b;
-            plan.off[plan.npass] = off;
-            plan.npass++;
-            off += 1u << b;
-            l -= b;
-            const size_t c_lo = (size_t)1 << l;
-            cc = cc < c_lo ? cc : c_lo;
-        }
-    }
     const int32_t* wts = nullptr;
     if (plan.npass) {
         void* p;
@@ -656,12 +692,16 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
         GRAPE_REQUIRE(total < ((size_t)1 << 32) - 256, "fold: more than 2^32 outputs in one pass");
         const uint32_t n_hi_max = (uint32_t)((cur_c + c_lo - 1) / c_lo);
         const int32_t* w = wts + (size_t)fr26::N * ps.off;
-        if (ps.S == 1)
-            fold_pass_kernel<1><<<blocks_for(total, 256), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
-        else if (ps.S == 2)
-            fold_pass_kernel<2><<<blocks_for(total, 128), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
-        else
-            fold_pass_kernel<4><<<blocks_for(total, 64), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);
+        const bool plain = ints != nullptr && pi == 1;      // the first pass of a fold of integers
+#define GRAPE_FOLD_PASS(SS, PER)                                                                                                    \
+    do {                                                                                                                            \
+        if (plain) fold_pass_kernel<SS, true><<<blocks_for(total, PER), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap); \
+        else fold_pass_kernel<SS, false><<<blocks_for(total, PER), kBlock, 0, s>>>(dst, src, w, n_hi_max, (uint32_t)outer, (uint32_t)cur_c, L - b, gap);     \
+    } while (0)
+        if (ps.S == 1) GRAPE_FOLD_PASS(1, 256);
+        else if (ps.S == 2) GRAPE_FOLD_PASS(2, 128);
+        else GRAPE_FOLD_PASS(4, 64);
+#undef GRAPE_FOLD_PASS
         GRAPE_LAUNCH_CHECK();
         profile_mark(s);
         src = dst;
@@ -670,6 +710,26 @@ int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t
     }
     if (src != t) GRAPE_HIP_CHECK(hipMemcpyAsync(t, src, outer * gap * 32, hipMemcpyDeviceToDevice, s));
     return GRAPE_OK;
+}
+
+int grape_fr_fold(uint32_t* t, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
+    return fold_impl(t, nullptr, N, x, c, id, gap, st);
+}
+
+size_t grape_fr_fold_i32_elems(size_t N, uint32_t c, uint32_t gap) {
+    if (N == 0 || c == 0 || gap == 0 || N % ((size_t)c * gap) != 0) return N;
+    const size_t outer = N / ((size_t)c * gap);
+    FoldPass passes[kFoldMaxPasses];
+    FoldPlan plan;
+    if (plan_fold(outer, c, gap, 0, passes, plan) != GRAPE_OK || plan.npass == 0) return N;
+    if (outer > 1) return outer * gap;                 // the passes go through work memory of the library
+    const size_t c_lo = (size_t)1 << (log2ceil(c) - passes[0].b);
+    return (c < c_lo ? c : c_lo) * gap;                // one outer index: the first pass writes into d_out
+}
+
+int grape_fr_fold_i32(uint32_t* out, const int32_t* in, size_t N, const uint32_t* x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t st) {
+    GRAPE_REQUIRE(in != nullptr || N == 0, "null input");
+    return fold_impl(out, in, N, x, c, id, gap, st);
 }
 
 }  // extern "C"

@@ -202,6 +202,26 @@ FrTensor FrTensor::random(uint size) {
     for (uint i = 0; i < size; i++) tmp[i] = Fr::random_element();
     return from_host(tmp);
 }
+FrTensor FrTensor::folded_from_ints(const int* device_int_data, uint N, fr_t* x, uint c, uint id, uint gap) {
+    grape_host::ensure_init();
+    const size_t elems = grape_fr_fold_i32_elems(N, c, gap);
+    FrTensor out((uint)(elems ? elems : 1));
+    check(grape_fr_fold_i32(W(out.gpu_data), device_int_data, N, W(x), c, id, gap, nullptr), "grape_fr_fold_i32");
+    out.set_size(c && gap ? N / (c * gap) * gap : 0);
+    return out;
+}
+Fr FrTensor::eval_ints(const int* device_int_data, uint size, const std::vector<Fr>& u) {
+    if ((uint64_t)size != ((uint64_t)1 << u.size())) {
+        // the rows-of-11008 reading of a short tensor (src/fr-tensor.cu:346-369) goes through the embedded tensor
+        FrTensor t(size, const_cast<int*>(device_int_data));
+        return t(u);
+    }
+    fr_t* d_u = grape_host::upload(u);
+    FrTensor t = folded_from_ints(device_int_data, size, d_u, size, 0, 1);
+    Fr ret = grape_host::download(t.gpu_data);
+    grape_free(d_u);
+    return ret;
+}
 FrTensor FrTensor::from_host(const std::vector<Fr>& v) {
     FrTensor out((uint)v.size());
     check(grape_memcpy_h2d(out.gpu_data, v.data(), sizeof(fr_t) * v.size(), nullptr), "grape_memcpy_h2d");

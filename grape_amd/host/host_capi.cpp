@@ -71,6 +71,7 @@ static Fr fr_from(const uint32_t* p) {
 }
 static void fr_to(uint32_t* p, const Fr& x) { std::memcpy(p, &x, 32); }
 static int g_input_format = 0;      // 0: field elements, 1: int32 values (grape_host_set_input_format)
+static bool g_int_folds = true;     // integer inputs of an opening or an evaluation are folded from the integers (grape_host_set_int_folds)
 static FrTensor tensor_from_device(const uint32_t* d, uint32_t n, uint32_t capacity = 0) {
     FrTensor t(capacity > n ? capacity : n);
     if (g_input_format == 1) {
@@ -103,6 +104,7 @@ int grape_host_set_input_format(int fmt) {
     g_input_format = fmt;
     return 0;
 }
+void grape_host_set_int_folds(int on) { g_int_folds = on != 0; }
 
 int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int N, int M, int K, const uint32_t* u, uint32_t nu,
                             const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
@@ -163,8 +165,12 @@ int grape_host_combine_claims(const uint32_t* d_X, uint32_t size, const uint32_t
 
 int grape_host_mle_eval(const uint32_t* d_T, uint32_t size, const uint32_t* u, uint32_t nu, uint32_t* out) {
     GUARD_BEGIN
-    FrTensor T = tensor_from_device(d_T, size);
-    fr_to(out, T(vec_from(u, nu)));
+    if (g_input_format == 1 && g_int_folds) {
+        fr_to(out, FrTensor::eval_ints(reinterpret_cast<const int*>(d_T), size, vec_from(u, nu)));
+    } else {
+        FrTensor T = tensor_from_device(d_T, size);
+        fr_to(out, T(vec_from(u, nu)));
+    }
     GUARD_END
 }
 
@@ -217,10 +223,16 @@ int grape_host_hyrax_open(const uint32_t* d_tensor, uint32_t size, uint32_t N, c
                           uint32_t* result) {
     GUARD_BEGIN
     Hyrax& hyrax = hyrax_for(d_table, npoints, com_scale, layer_num);
-    FrTensor t = tensor_from_device(d_tensor, size);
-    ProveTimer timer;
-    Hyrax_proof proof = hyrax.open(t, vec_from(eval_point, n_eval), fr_from(c), size, N);
-    fr_to(result, proof.result);
+    if (g_input_format == 1 && g_int_folds) {
+        ProveTimer timer;
+        Hyrax_proof proof = hyrax.open(reinterpret_cast<const int*>(d_tensor), vec_from(eval_point, n_eval), fr_from(c), size, N);
+        fr_to(result, proof.result);
+    } else {
+        FrTensor t = tensor_from_device(d_tensor, size);
+        ProveTimer timer;
+        Hyrax_proof proof = hyrax.open(t, vec_from(eval_point, n_eval), fr_from(c), size, N);
+        fr_to(result, proof.result);
+    }
     GUARD_END
 }
 

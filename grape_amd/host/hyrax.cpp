@@ -385,6 +385,14 @@ jacob_t* Hyrax::commit(FrTensor& tensor, uint size, uint N) {
 // outer variables of the point, blind it as z = c*x + d with a random row d, commit d, and send
 // <a,d>*G where a is the eq-vector of the inner variables.
 Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N) {
+    return open_impl(&tensor, nullptr, eval_point_, c, size, N);
+}
+Hyrax_proof Hyrax::open(const int* device_int_data, const std::vector<Fr> eval_point_, Fr c, uint size, uint N) {
+    return open_impl(nullptr, device_int_data, eval_point_, c, size, N);
+}
+// tensor_in, or the integer tensor `ints` read as FrTensor::get_data would embed it: its fold over the rows then reads the
+// integers directly (4 bytes per element where embedding and folding move 68)
+Hyrax_proof Hyrax::open_impl(FrTensor* tensor_in, const int* ints, const std::vector<Fr>& eval_point_, Fr c, uint size, uint N) {
     if (size / N / com_scale < layer_num) throw std::runtime_error("Size too small: size < N * com_scale * layer_num");
     uint pad_N = 1u << Log2(N);
     uint new_N = pad_N * com_scale;
@@ -415,7 +423,14 @@ Hyrax_proof Hyrax::open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr 
     const bool flag_used = commit_fr_rows(com_d_dev, d.gpu_data, new_N, new_N, false, open_stream, d_flag);
 
     FrTensor x(new_N);
-    tensor.partial_eval(size, eval_point, (size / layer_num) / (N * com_scale), Log2(N * com_scale), N * com_scale);
+    std::unique_ptr<FrTensor> rows_of_ints;
+    if (ints) {
+        rows_of_ints.reset(new FrTensor(FrTensor::folded_from_ints(ints, size, eval_point, (size / layer_num) / (N * com_scale),
+                                                                    Log2(N * com_scale), N * com_scale)));
+    } else {
+        tensor_in->partial_eval(size, eval_point, (size / layer_num) / (N * com_scale), Log2(N * com_scale), N * com_scale);
+    }
+    FrTensor& tensor = ints ? *rows_of_ints : *tensor_in;
     tensor.partial_eval((N * com_scale) * layer_num, eval_point, layer_num, Log2(size / layer_num), N * com_scale);
     x = tensor;
     if (pad_N != N) x.pad(tensor, N, pad_N, new_N, Fr::zero());

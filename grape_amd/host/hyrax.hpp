@@ -54,6 +54,9 @@ public:
     affine_t* commit_affine_i32(int* tensor, uint size, uint N, int* d_flag = nullptr, void* stream = nullptr);
 
     Hyrax_proof open(FrTensor& tensor, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
+    // addition: the opening of the tensor that FrTensor::get_data would make of `size` device integers (the reference's
+    // drivers embed an integer tensor and open it, test/llm.cu:99-104) - same proof, the integers are read directly
+    Hyrax_proof open(const int* device_int_data, const std::vector<Fr> eval_point_, Fr c, uint size, uint N);
     // Checks an opening against row commitments (the equations of test/HyraxTest.cu:87-125);
     // the reference's own verify is an empty stub (src/Hyrax.cu:307-310).
     bool verify(Hyrax_proof& proof, jacob_t* commitment, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
@@ -110,6 +113,7 @@ private:
     // commits `size` full-width scalars in rows of rowlen into out[0 .. size/rowlen)
     // d_flag (single rows through the per-window table only): queued without waiting, digit-range check left in *d_flag;
     // returns whether it was queued that way (false: the call has waited and checked)
+    Hyrax_proof open_impl(FrTensor* tensor, const int* ints, const std::vector<Fr>& eval_point, Fr c, uint size, uint N);
     bool commit_fr_rows(affine_t* out, fr_t* scalars, size_t size, uint rowlen, bool may_build, void* stream = nullptr, int* d_flag = nullptr);
     void commit_i32_rows(affine_t* out, int* tensor, size_t size, uint rowlen, int* d_flag, void* stream = nullptr);
     void check_shape(uint size, uint N) const;

@@ -163,6 +163,14 @@ def fr_fold(t, N, x, c, idx, gap):
 
 
 # ------------------------------------------------------------------ sumcheck / tlookup
+def fr_fold_i32(ints, N, x, c, idx, gap):
+    """fold of the integer tensor `ints` (as its embedding into Fr); returns the [N/(c*gap)][gap] result"""
+    lib = init()
+    out = fr_empty(max(1, lib.grape_fr_fold_i32_elems(N, c, gap)))
+    _capi.check(lib.grape_fr_fold_i32(_p(out), _p(ints), N, _p(x), c, idx, gap, _s()))
+    return out[: N // (c * gap) * gap]
+
+
 def sumcheck_round2_claim(A, B, in_size, out_size, v, claim):
     """claim (device, one element) is replaced by the next round's claim; returns the three sums"""
     lib = init()

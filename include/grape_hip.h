@@ -114,6 +114,17 @@ int grape_i32_pad_fill(int32_t *d_out, const int32_t *d_in, uint32_t N, uint32_t
  * Fr_partial_eval_kernel :53-72.  x is a device array of challenges.
  */
 int grape_fr_fold(uint32_t *d_t, size_t N, const uint32_t *d_x, uint32_t c, uint32_t id, uint32_t gap, grape_stream_t stream);
+/*
+ * The same fold of a tensor of N 32-bit integers, i.e. of the field tensor that FrTensor::get_data
+ * (src/fr-tensor.cu:30-39: |x| as a residue, negated for x < 0) would make of d_in - without making it:
+ * the first pass reads the integers and writes field elements into d_out, the later passes work there.
+ * The [N/(c*gap)][gap] result is left at the front of d_out, which must hold
+ * grape_fr_fold_i32_elems(N, c, gap) elements; d_in is not modified.  For the reference's drivers'
+ * get_data + partial_eval / operator() / Hyrax::open on an integer tensor (test/llm.cu:99-125).
+ */
+size_t grape_fr_fold_i32_elems(size_t N, uint32_t c, uint32_t gap);
+int grape_fr_fold_i32(uint32_t *d_out, const int32_t *d_in, size_t N, const uint32_t *d_x, uint32_t c, uint32_t id, uint32_t gap,
+                      grape_stream_t stream);
 
 /* ------------------------------------------------------------------ sumcheck ----------------- */
 /*

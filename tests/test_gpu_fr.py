@@ -169,6 +169,31 @@ def test_fold_large_shapes_vs_oracle(ops, outer, c, gap):
     assert_same(got, want, "fold")
 
 
+@pytest.mark.parametrize("outer,c,gap", [
+    (1, 16, 1 << 19), (1, 16, 1 << 17), (1, 13, 1 << 17), (300, 4096, 1), (1, 1 << 21, 1),    # every pass variant
+    (1, 2048, 4096),          # an opening's fold over the rows of a 2048 x 4096 tensor
+    (3, 8, 5), (1, 1, 77), (2, 37, 16), (1, 1024, 2),                                          # finish kernel alone, nothing to bind
+])
+def test_fold_of_an_integer_tensor(ops, outer, c, gap):
+    """grape_fr_fold_i32 against the fold of the embedded tensor (grape_fr_from_i32 + grape_fr_fold, itself pinned
+    against the oracle above), bit for bit; integers over the whole int32 range, both signs"""
+    import torch
+    n = outer * c * gap
+    rng = np.random.default_rng(101 + c + gap)
+    ints = rng.integers(-(1 << 31), 1 << 31, size=n, dtype=np.int64).astype(np.int32)
+    ints[:4] = [-(1 << 31), (1 << 31) - 1, 0, -1]
+    di = torch.from_numpy(ints).cuda()
+    x = ops.to_dev(rand_fr(br.log2ceil(c) + 3, 102 + c))
+    want = ops.fr_from_i32(di)
+    ops.fr_fold(want, n, x, c, 2, gap)
+    got = ops.fr_fold_i32(di, n, x, c, 2, gap)
+    assert_same(ops.fr_to_host(got), ops.fr_to_host(want)[: outer * gap], "fold of integers")
+    assert np.array_equal(di.cpu().numpy(), ints)            # the input is left alone
+    if n <= 1 << 16:
+        assert_same(ops.fr_to_host(got), orc.partial_eval(ops.fr_to_host(ops.fr_from_i32(di)), n, ops.fr_to_host(x), c, 2, gap)[: outer * gap],
+                    "fold of integers against the oracle")
+
+
 def test_fold_full_eval_config3_shape_slice(ops):
     # the two folds of BASELINE config 3 at reduced token/feature counts but the real K = 4096
     # stride: A [N=64][K=4096] over N with id = log2(M), B [M=128][K=4096] over M with id = 0

@@ -284,6 +284,38 @@ def test_hyrax_open_and_verify(ops, host, gens):
     assert_same(res, orc.mle_eval(t, pt), "opened value = T(point)")
 
 
+@pytest.mark.parametrize("rows,N", [(8, 4), (2048, 256)])
+def test_opening_and_evaluation_of_integer_tensors(ops, host, gens, rows, N):
+    """Hyrax::open(const int*, ...) and FrTensor::eval_ints (the fold reads the integers) against get_data + open /
+    operator() on the embedded tensor, and against the oracle's evaluation of that tensor"""
+    import torch
+    hg, dg = gens
+    npoints = max(64, N)
+    if npoints > dg.shape[0]:
+        dg = ops.g1_make_generators(rand_fr(npoints, 74))
+    table = ops.g1_table_gen(dg[:npoints].contiguous(), 256)
+    size = rows * N
+    ints = np.random.default_rng(75 + rows).integers(-(1 << 31), 1 << 31, size=size, dtype=np.int64).astype(np.int32)
+    di = torch.from_numpy(ints).cuda()
+    pt, c = rand_fr(br.log2ceil(size), 76), rand_fr(1, 77)
+    want = orc.mle_eval(ops.fr_to_host(ops.fr_from_i32(di)), pt) if size <= 4096 else None
+    host.set_input_format("i32")
+    try:
+        results = {}
+        for folds in (True, False):
+            host.set_int_folds(folds)
+            results[folds] = (host.hyrax_open(di, size, N, table, npoints, pt, c, com_scale=1), host.mle_eval(di, size, pt))
+    finally:
+        host.set_int_folds(True)
+        host.set_input_format("fr")
+    assert_same(results[True][0], results[False][0], "opened value, integers folded directly")
+    assert_same(results[True][1], results[False][1], "evaluation, integers folded directly")
+    assert_same(results[True][0], results[True][1], "opening = evaluation")
+    assert np.array_equal(di.cpu().numpy(), ints)
+    if want is not None:
+        assert_same(results[True][0], want, "against the oracle")
+
+
 @pytest.mark.parametrize("L,M,N", [(1, 4, 8), (2, 2, 4), (1, 4, 6), (2, 1, 5), (1, 32, 64), (1, 2, 1)])
 def test_prove_elemul_vs_oracle(ops, host, L, M, N):
     rng = random.Random(81 + L + M + N)
