@@ -371,8 +371,9 @@ def layer_workload(args):
                             "total_prove_time (test/llm.cu:69-125): integer tensors -> Fr, copies, claim evaluation, sub-proof, "
                             "Hyrax openings; plus the 7 weight commitments; witness generation outside",
                    "integer_tensors": ("openings and claim evaluations fold their integer tensors directly (Hyrax::open(const int*), "
-                                       "FrTensor::eval_ints): same values, the embedded tensor is never written; the sub-provers embed theirs "
-                                       "with FrTensor::get_data") if not args.no_int_folds else
+                                       "FrTensor::eval_ints) and the lookup provers index and embed their integer witnesses in one pass "
+                                       "(tLookupRange::prove(const int*, ...), tLookupRangeMapping::prove(const int*, const int*, ...)): same "
+                                       "proofs; the matmul provers embed their operands with FrTensor::get_data") if not args.no_int_folds else
                                       "every integer tensor is embedded with FrTensor::get_data before its proof step (--no-int-folds)",
                    "wall_breakdown_s": last["wall_breakdown_s"],
                    "provers_only_s": float(np.mean([r["provers_only_s"] for r in runs])),
@@ -883,8 +884,8 @@ def main():
     ap.add_argument("--no-spread", action="store_true",
                     help="layer workload: skip the two extra layers whose softmax scores are spread over the whole table")
     ap.add_argument("--no-int-folds", action="store_true",
-                    help="layer workload: openings and claim evaluations embed their integer tensors first (get_data + open / operator()) "
-                         "instead of folding the integers directly")
+                    help="layer workload: openings, claim evaluations and lookups embed their integer tensors first (FrTensor::get_data) "
+                         "instead of reading the integers directly")
     ap.add_argument("--no-layer", action="store_true",
                     help="commit workload: skip the configs[4] layer proof that is measured afterwards in a child process")
     ap.add_argument("--log-elems", type=int, default=25, help="rounds workload: log2 of the tensors' element count")

@@ -73,6 +73,7 @@ SIGNATURES = {
     "grape_tlookup_hist_index": [c_void_p, c_void_p, c_size_t, c_u32, c_void_p],
     "grape_tlookup_inverse_by_table": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_u32, ctypes.POINTER(c_size_t), c_void_p],
     "grape_tlookup_index_inverse": [c_void_p, c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p, c_void_p, c_void_p, ctypes.POINTER(c_size_t), c_void_p],
+    "grape_tlookup_index_embed_i32_nowait": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_tlookup_index_inverse_nowait": [c_void_p, c_void_p, c_void_p, c_size_t, c_i32, c_u32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "grape_fr_axpy": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     "grape_tlookup_hot_select": [c_void_p, c_u32, c_u32, c_u32, c_void_p, c_void_p, ctypes.POINTER(ctypes.c_uint64), c_void_p],

@@ -502,6 +502,36 @@ __global__ void __launch_bounds__(kBlock) index_inverse_kernel(int32_t* idx1, ui
     if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
 }
 
+// The same pass over an INTEGER witness (the tensors a driver would first embed with FrTensor::get_data): besides the
+// index, the check and A it leaves the witness itself as field elements - S[i] = key_i for a range lookup,
+// S[i] = key_i + r * cmp_i (the combined witness, src/tlookup.cu:407-410) for a mapping lookup, whose table of second
+// components is an integer table too.  8 bytes per element are read where embedding two tensors, indexing them and
+// combining them move 270.
+__global__ void __launch_bounds__(kBlock) index_embed_i32_kernel(int32_t* idx1, uint32_t* A, uint32_t* S, const int32_t* __restrict__ key,
+                                                                  const int32_t* __restrict__ cmp, size_t n, int32_t low, uint32_t len,
+                                                                  const uint32_t* B, const int32_t* __restrict__ cmp_table, const uint32_t* r,
+                                                                  unsigned int* mismatches) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    bool bad = false;
+    if (i < n) {
+        const int32_t k = key[i];
+        const int64_t d = (int64_t)k - (int64_t)low;
+        const bool inside = d >= 0 && d < (int64_t)len;
+        idx1[i] = inside ? (int32_t)(d + 1) : 0;
+        bad = !inside;
+        Fr s = fr26::from_i32c(k);
+        if (cmp) {
+            const int32_t c = cmp[i];
+            if (inside) bad = c != cmp_table[d];
+            s = add(s, fr26::mulc(fr26::from_i32c(c), ld_fr(r, 0)));
+        }
+        st_fr(S, i, s);
+        if (!bad && A) st_fr(A, i, ld_fr(B, (size_t)d));
+    }
+    const unsigned long long b = __ballot(bad);
+    if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
+}
+
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
 __global__ void __launch_bounds__(kBlock) index_kernel(int32_t* out, const uint32_t* vals, size_t n, int32_t low, uint32_t len) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -979,6 +1009,24 @@ int grape_tlookup_index_inverse_nowait(int32_t* idx1, uint32_t* A, const uint32_
     GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr), "cmp and cmp_table go together");
     if (cmp) { CHECK_PTR16(cmp); CHECK_PTR16(cmp_table); }
     index_inverse_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, key, n, low, len, B, cmp, cmp_table, (unsigned int*)d_mismatches);
+    GRAPE_LAUNCH_CHECK();
+    return GRAPE_OK;
+}
+
+int grape_tlookup_index_embed_i32_nowait(int32_t* idx1, uint32_t* A, uint32_t* S, const int32_t* key, const int32_t* cmp, size_t n, int32_t low,
+                                         uint32_t len, const uint32_t* B, const int32_t* cmp_table, const uint32_t* r, uint32_t* d_mismatches,
+                                         grape_stream_t st) {
+    GRAPE_REQUIRE(d_mismatches != nullptr && idx1 != nullptr && len > 0, "bad arguments");
+    hipStream_t s = as_stream(st);
+    int rc = zero_fill(d_mismatches, sizeof(uint32_t), s);
+    if (rc) return rc;
+    if (n == 0) return GRAPE_OK;
+    CHECK_PTR16(S);
+    GRAPE_REQUIRE(key != nullptr, "null witness");
+    if (A) { CHECK_PTR16(A); CHECK_PTR16(B); }       // A == nullptr: no logUp tensor written
+    GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr) && (cmp == nullptr) == (r == nullptr), "cmp, cmp_table and r go together");
+    if (r) CHECK_PTR16(r);
+    index_embed_i32_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, S, key, cmp, n, low, len, B, cmp_table, r, (unsigned int*)d_mismatches);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }

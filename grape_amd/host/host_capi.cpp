@@ -287,11 +287,17 @@ int grape_host_tlookup_range_prove(const uint32_t* d_S, uint32_t D, int32_t low,
     lk.alpha = fr_from(alpha);
     lk.set_u(vec_from(u, nuv));
     uint32_t Dp = 1u << Log2(D);
-    FrTensor S = tensor_from_device(d_S, D, Dp);
     FrTensor A(Dp);
     double ct = 0;
     Fr sc;
-    {
+    if (g_input_format == 1 && g_int_folds) {
+        // the witness stays a tensor of integers: the prover's pass over it embeds it on the way
+        FrTensor S(Dp);
+        S.set_size(D);
+        ProveTimer timer;
+        sc = lk.prove(reinterpret_cast<const int*>(d_S), S, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    } else {
+        FrTensor S = tensor_from_device(d_S, D, Dp);
         ProveTimer timer;
         sc = lk.prove(S, A, vec_from(v, nuv), hyrax, msm_size, ct);
     }
@@ -325,12 +331,15 @@ static void mapping_prove_impl(const uint32_t* d_S_in, const uint32_t* d_S_out, 
     lk.alpha = fr_from(alpha);
     lk.set_u(vec_from(u, nuv));
     uint32_t Dp = 1u << Log2(D);
-    FrTensor S_in = tensor_from_device(d_S_in, D);
-    FrTensor S_out = tensor_from_device(d_S_out, D);
     FrTensor A(Dp);
     double ct = 0;
     Fr sc;
-    {
+    if (g_input_format == 1 && g_int_folds) {
+        ProveTimer timer;
+        sc = lk.prove(reinterpret_cast<const int*>(d_S_in), reinterpret_cast<const int*>(d_S_out), D, A, vec_from(v, nuv), hyrax, msm_size, ct);
+    } else {
+        FrTensor S_in = tensor_from_device(d_S_in, D);
+        FrTensor S_out = tensor_from_device(d_S_out, D);
         ProveTimer timer;
         sc = lk.prove(S_in, S_out, A, vec_from(v, nuv), hyrax, msm_size, ct);
     }

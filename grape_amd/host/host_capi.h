@@ -23,8 +23,9 @@ void grape_host_set_indexed_commit(int on);
  * its own with FrTensor::get_data as the reference's drivers do (test/llm.cu:77).  Returns 1 for an
  * unknown format. */
 int grape_host_set_input_format(int fmt);
-/* With int32 inputs, grape_host_hyrax_open and grape_host_mle_eval fold the integers directly (1, default:
- * Hyrax::open(const int*, ...), FrTensor::eval_ints) or embed them first and fold the field tensor (0). */
+/* With int32 inputs, grape_host_hyrax_open and grape_host_mle_eval fold the integers directly and the lookup provers
+ * index the integer witness (1, default: Hyrax::open(const int*, ...), FrTensor::eval_ints, tLookupRange::prove(const int*, ...),
+ * tLookupRangeMapping::prove(const int*, const int*, ...)), or every call embeds its tensors first (0). */
 void grape_host_set_int_folds(int on);
 
 /* prove_matmul on copies of the device tensors d_A (L*N*K) and d_B (L*M*K).  transcript receives

@@ -51,6 +51,31 @@ void tLookup::make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const
     a_ready_ = write_A && mismatches == 0;
     a_deferred_ = !write_A && mismatches == 0;
 }
+void tLookup::make_index_and_A_from_ints(const int* key, const int* cmp, uint n, int low_, FrTensor& S, FrTensor& A, const int* cmp_table,
+                                         const Fr* r, bool write_A) {
+    drop_index();
+    a_ready_ = false;
+    a_deferred_ = false;
+    check(grape_malloc((void**)&d_idx_, sizeof(int) * (size_t)(n ? n : 1)), "grape_malloc");
+    uint32_t* d_count = nullptr;
+    check(grape_malloc((void**)&d_count, sizeof(uint32_t)), "grape_malloc");
+    uint32_t mismatches = 1;
+    try {
+        check(grape_tlookup_index_embed_i32_nowait(d_idx_, write_A ? W(A.gpu_data) : nullptr, W(S.gpu_data), key, cmp, n, low_, T.size,
+                                                   W(B.gpu_data), cmp_table, r ? W(grape_host::device_scalar(*r)) : nullptr, d_count, nullptr),
+              "grape_tlookup_index_embed_i32_nowait");
+        S.set_size(n);
+        start_weights(1u << Log2(n));
+        check(grape_memcpy_d2h(&mismatches, d_count, sizeof(uint32_t), nullptr), "grape_memcpy_d2h");
+    } catch (...) {
+        grape_stream_sync(nullptr);
+        grape_free(d_count);
+        throw;
+    }
+    grape_free(d_count);
+    a_ready_ = write_A && mismatches == 0;
+    a_deferred_ = !write_A && mismatches == 0;
+}
 void tLookup::pad_index(uint N, uint pad_N, uint pad_size, int fill) {
     if (!d_idx_ || N == pad_N) return;
     int* padded = nullptr;
@@ -675,6 +700,32 @@ Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax
     return ret;
 }
 
+Fr tLookupRange::prove(const int* device_int_S, FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size,
+                       double& commit_time) {
+    const uint D = S.size;
+    if (!(D == (1u << Log2(D)) && A.size >= D)) {
+        // a witness that needs padding goes the ordinary way
+        S.get_data(D, const_cast<int*>(device_int_S));
+        return prove(S, A, v, hyrax, msm_size, commit_time);
+    }
+    a_ready_ = false;
+    const bool gather = indexed_commit_ && index_known_ && D / 2 >= (1u << 16);
+    make_index_and_A_from_ints(device_int_S, nullptr, D, low, S, A, nullptr, nullptr, !gather);
+    m_pending_ = true;
+    m_pending_size_ = D;
+    m_pending_low_ = low;
+    Fr ret;
+    try {
+        ret = run(S, A, v, hyrax, msm_size, commit_time);
+    } catch (...) {
+        m_pending_ = false;
+        drop_index();
+        throw;
+    }
+    drop_index();
+    return ret;
+}
+
 // ------------------------------------------------------------------ mapping lookup
 void tLookupRangeMapping::init_from_host(const int* host_table, uint len) {
     if (len != (1u << Log2(len))) throw std::runtime_error("tLookupRangeMapping: len must be a power of two");
@@ -686,8 +737,10 @@ void tLookupRangeMapping::init_from_host(const int* host_table, uint len) {
                              W(grape_host::device_scalar(r)), nullptr),
           "grape_tlookup_init");
     check(grape_stream_sync(nullptr), "sync");
-    grape_free(d_int);
+    grape_free(d_map_int_);
+    d_map_int_ = d_int;                   // kept: a witness handed over as integers is checked against it
 }
+tLookupRangeMapping::~tLookupRangeMapping() { grape_free(d_map_int_); }
 
 // src/tlookup.cu:350-372
 tLookupRangeMapping::tLookupRangeMapping(const int low_, const uint len, const std::string& filename)
@@ -729,6 +782,29 @@ Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, cons
         S.pad(A, 11008, 16384, 1u << Log2(D), pad_value);
         pad_index(11008, 16384, 1u << Log2(D), -low + 1);      // the padding value sits at table index -low
     }
+    Fr ret;
+    try {
+        ret = run(S, A, v, hyrax, msm_size, commit_time);
+    } catch (...) {
+        drop_index();
+        throw;
+    }
+    drop_index();
+    return ret;
+}
+
+Fr tLookupRangeMapping::prove(const int* device_int_S_in, const int* device_int_S_out, uint D, FrTensor& A, const std::vector<Fr>& v,
+                              Hyrax& hyrax, uint msm_size, double& commit_time) {
+    if (!(D == (1u << Log2(D)) && A.size >= D)) {
+        FrTensor S_in(D, const_cast<int*>(device_int_S_in)), S_out(D, const_cast<int*>(device_int_S_out));
+        return prove(S_in, S_out, A, v, hyrax, msm_size, commit_time);
+    }
+    a_ready_ = false;
+    // index, the check S_out = f(S_in) against the integer table, A = B[index] and the combined witness S_in + r * S_out in one
+    // pass over the integers
+    FrTensor S(D);
+    make_index_and_A_from_ints(device_int_S_in, device_int_S_out, D, low, S, A, d_map_int_, &r, true);
+    index_to_m(D, low);
     Fr ret;
     try {
         ret = run(S, A, v, hyrax, msm_size, commit_time);

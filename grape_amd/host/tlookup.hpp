@@ -67,6 +67,10 @@ protected:
     // write_A = false: the indices and the check only (a_deferred_ when every element matched); the first round then
     // gathers A from B, or run() writes it out where that round cannot.
     void make_index_and_A(const FrTensor& key, int low_, FrTensor& A, const FrTensor* cmp, const FrTensor* cmp_table, bool write_A = true);
+    // the same pass over a witness that is still a tensor of integers: also leaves the witness as field elements in S
+    // (key, or key + r * cmp with the integer table cmp_table of a mapping lookup)
+    void make_index_and_A_from_ints(const int* key, const int* cmp, uint n, int low_, FrTensor& S, FrTensor& A, const int* cmp_table,
+                                    const Fr* r, bool write_A);
     bool a_ready_ = false;              // A of the proof in flight already holds B[index]
     bool a_deferred_ = false;           // every element sits in the table, A not written yet
     void drop_index();
@@ -108,6 +112,10 @@ public:
     void prep(const FrTensor& vals);
     // Proves every element of S lies in [low, low+len); returns S(v).  S and A are scratch-mutated.
     Fr prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
+    // addition: the proof for the tensor that FrTensor::get_data would make of S.size device integers (the reference's
+    // drivers embed the witness and prove it, test/llm.cu:77-104).  S is work memory of at least the padded size; the
+    // pass that indexes the witness reads the integers and writes S.
+    Fr prove(const int* device_int_S, FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size, double& commit_time);
 };
 
 class tLookupRangeMapping : public tLookup {
@@ -124,9 +132,14 @@ public:
     void prep(const FrTensor& vals);
     Fr prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size,
              double& commit_time);
+    // addition: the same for two tensors of D device integers (see tLookupRange::prove)
+    Fr prove(const int* device_int_S_in, const int* device_int_S_out, uint D, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax,
+             uint msm_size, double& commit_time);
+    ~tLookupRangeMapping();
 
 private:
     void init_from_host(const int* host_table, uint len);
+    int* d_map_int_ = nullptr;          // the table's second components as integers (for witnesses handed over as integers)
 };
 
 // The round-by-round form of the logUp sumcheck, as the reference exposes it

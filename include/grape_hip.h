@@ -284,6 +284,14 @@ int grape_tlookup_index_inverse(int32_t *d_idx1, uint32_t *d_A, const uint32_t *
 int grape_tlookup_index_inverse_nowait(int32_t *d_idx1, uint32_t *d_A, const uint32_t *d_key, size_t n, int32_t low, uint32_t len,
                                        const uint32_t *d_B, const uint32_t *d_cmp, const uint32_t *d_cmp_table,
                                        uint32_t *d_mismatches, grape_stream_t stream);
+/* The pass over a witness that is still a tensor of 32-bit integers (what a driver would embed with
+ * FrTensor::get_data first, test/llm.cu:77): indices, check, count and d_A as above (d_A may be NULL), and the
+ * witness as field elements in d_S: d_S[i] = key_i for a range lookup (d_cmp = d_cmp_table = d_r = NULL),
+ * d_S[i] = key_i + r * cmp_i for a mapping lookup (src/tlookup.cu:407-410), whose second components are
+ * compared with the INTEGER table d_cmp_table[index].  Queued without waiting, as the call above. */
+int grape_tlookup_index_embed_i32_nowait(int32_t *d_idx1, uint32_t *d_A, uint32_t *d_S, const int32_t *d_key, const int32_t *d_cmp,
+                                         size_t n, int32_t low, uint32_t len, const uint32_t *d_B, const int32_t *d_cmp_table,
+                                         const uint32_t *d_r, uint32_t *d_mismatches, grape_stream_t stream);
 /* The same histogram from indices already made by grape_tlookup_index (d_idx1[i] = index + 1,
  * 0 = outside the table): hist[d_idx1[i] - 1] += 1. */
 int grape_tlookup_hist_index(uint32_t *d_hist, const int32_t *d_idx1, size_t n, uint32_t len, grape_stream_t stream);

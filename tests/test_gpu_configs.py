@@ -102,7 +102,16 @@ def test_configs3_tlookup_range_2p24_in_2p16_indexed(ops, host, gens4096):
     table = ops.g1_table_gen(dg, 256)
     dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
     res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, NGEN, 1, 4096, want_commitments=True)
-    del dS, table
+    del dS
+    # the same proof from the witness as integers (the prover's pass over it embeds it; the first round gathers A)
+    host.set_input_format("i32")
+    try:
+        res_i = host.tlookup_range_prove(torch.from_numpy(S).cuda(), D, low, N, alpha, u, v, table, NGEN, 1, 4096, want_commitments=True)
+    finally:
+        host.set_input_format("fr")
+    for key in ("m", "transcript", "S_claim", "com_A", "com_m"):
+        assert_same(res_i[key], res[key], "integer witness: " + key)
+    del table
     torch.cuda.empty_cache()
     assert br.fr_unpack(res["m"]) == [int(x) for x in np.bincount(S.astype(np.int64) - low, minlength=N)]
     Sp = orc.from_i32(S)
@@ -237,7 +246,19 @@ def test_configs4_softmax_mapping_lookup_through_occupied_entries(ops, host, gen
     assert h2 == 0 and c2 == 0
     assert_same(com_a, com_a2, "com(A): occupied-entry table == full-width commitment")
     assert_same(tr, tr2, "transcripts")
-    del dSi, dSo, table
+    del dSi, dSo
+    # the same proof from the two tensors as integers (one pass indexes, checks and combines them)
+    host.set_input_format("i32")
+    try:
+        tr3, sc3, com_a3, h3, c3, _ = host.tlookup_mapping_prove_ex(torch.from_numpy(S_in).cuda(), torch.from_numpy(S_out).cuda(), D, low, N,
+                                                                    exp_map, alpha, r, u, v, table, NGEN, 1, 4096)
+    finally:
+        host.set_input_format("fr")
+    assert_same(tr3, tr, "integer witness: transcript")
+    assert_same(sc3, sc, "integer witness: S(v)")
+    assert_same(com_a3, com_a, "integer witness: com(A)")
+    assert (h3, c3) == (n_hot, n_cold)
+    del table
     torch.cuda.empty_cache()
     T, B = orc.tlookup_init(low, N, beta, orc.from_i32(exp_map), r[0])
     m = orc.tlookup_prep(orc.from_i32(S_in), low, N)

@@ -36,6 +36,25 @@ def gens(ops):
     return h, d
 
 
+class _witness_as:
+    """hands integer witnesses to the host calls as field tensors ("fr") or as the integers themselves ("i32": the
+    provers then index and embed them in one pass)"""
+    def __init__(self, host, ops, fmt):
+        self.host, self.ops, self.fmt = host, ops, fmt
+
+    def __enter__(self):
+        self.host.set_input_format(self.fmt)
+        return self
+
+    def __exit__(self, *exc):
+        self.host.set_input_format("fr")
+
+    def dev(self, ints):
+        import torch
+        d = torch.from_numpy(np.ascontiguousarray(ints, dtype=np.int32)).cuda()
+        return d if self.fmt == "i32" else self.ops.fr_from_i32(d)
+
+
 def _int_tensor(shape, seed):
     rng = np.random.default_rng(seed)
     return rng.integers(-2**15, 2**15, size=shape).astype(np.int32)
@@ -106,10 +125,13 @@ def test_mle_eval_operator(ops, host):
     assert_same(host.mle_eval(ops.to_dev(t), 2 * 11008, u), orc.mle_eval(t, u), "T(u), 11008 columns")
 
 
+@pytest.mark.parametrize("fmt", ["fr", "i32"])
 @pytest.mark.parametrize("indexed", [True, False])
 @pytest.mark.parametrize("logD,logN,low", [(4, 2, -2), (5, 3, -4), (3, 3, 0), (12, 6, -32), (14, 8, -128), (16, 16, -32768)])
-def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed):
+def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed, fmt):
     import torch
+    if fmt == "i32" and logD in (5, 14):
+        pytest.skip("the integer-witness path is covered at the other sizes")
     host.set_indexed_commit(indexed)
     hg, dg = gens
     D, N = 1 << logD, 1 << logN
@@ -123,9 +145,9 @@ def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed
     st, wtr, wsc = orc.tlookup_prove(Sp, T, B, m, alpha[0], beta, u, v)
     assert st == 0
     table = ops.g1_table_gen(dg, 256)               # 256 generators: com(m) uses rows of 2^(logN/2)
-    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
     msm = min(D, 16)
-    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 256, 1, msm, want_commitments=True)
+    with _witness_as(host, ops, fmt) as w:
+        res = host.tlookup_range_prove(w.dev(S), D, low, N, alpha, u, v, table, 256, 1, msm, want_commitments=True)
     assert_same(res["m"], m, "multiplicities")
     assert_same(res["transcript"], wtr, "transcript")
     assert_same(res["S_claim"], wsc, "S(v)")
@@ -145,17 +167,18 @@ def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed
     assert_same(res["com_m"], orc.commit_fr(m, tab, mN, 256), "com(m)")
 
 
-def test_tlookup_range_rejects_out_of_range(ops, host, gens):
-    import torch
+@pytest.mark.parametrize("fmt", ["fr", "i32"])
+def test_tlookup_range_rejects_out_of_range(ops, host, gens, fmt):
     hg, dg = gens
     S = np.array([0, 1, 2, 3, 9, 1, 2, 3, 0, 0, 1, 1, 2, 2, 3, 3], dtype=np.int32)
     table = ops.g1_table_gen(dg[:16].contiguous(), 256)
-    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
-    with pytest.raises(host.HostError, match="tLookup_phase"):
-        host.tlookup_range_prove(dS, 16, 0, 4, rand_fr(1, 31), rand_fr(4, 32), rand_fr(4, 33), table, 16, 1, 16)
+    with _witness_as(host, ops, fmt) as w:
+        with pytest.raises(host.HostError, match="tLookup_phase"):
+            host.tlookup_range_prove(w.dev(S), 16, 0, 4, rand_fr(1, 31), rand_fr(4, 32), rand_fr(4, 33), table, 16, 1, 16)
 
 
-def test_tlookup_pads_11008_rows(ops, host, gens):
+@pytest.mark.parametrize("fmt", ["fr", "i32"])
+def test_tlookup_pads_11008_rows(ops, host, gens, fmt):
     # a witness of 2 x 11008 values is padded to 2 x 16384 with zeros, which are counted in m
     import torch
     hg, dg = gens
@@ -172,14 +195,15 @@ def test_tlookup_pads_11008_rows(ops, host, gens):
     st, wtr, wsc = orc.tlookup_prove(Spad, T, B, m, alpha[0], beta, u, v)
     assert st == 0
     table = ops.g1_table_gen(dg[:16].contiguous(), 256)
-    dS = ops.fr_from_i32(torch.from_numpy(S).cuda())
-    res = host.tlookup_range_prove(dS, D, low, N, alpha, u, v, table, 16, 1, 16)
+    with _witness_as(host, ops, fmt) as w:
+        res = host.tlookup_range_prove(w.dev(S), D, low, N, alpha, u, v, table, 16, 1, 16)
     assert_same(res["m"], m, "multiplicities with pad fix-up")
     assert_same(res["transcript"], wtr, "transcript")
     assert_same(res["S_claim"], wsc, "S(v)")
 
 
-def test_tlookup_mapping_prove_vs_oracle(ops, host, gens):
+@pytest.mark.parametrize("fmt", ["fr", "i32"])
+def test_tlookup_mapping_prove_vs_oracle(ops, host, gens, fmt):
     import torch
     hg, dg = gens
     logD, logN, low = 10, 6, -32
@@ -196,17 +220,16 @@ def test_tlookup_mapping_prove_vs_oracle(ops, host, gens):
     st, wtr, wsc = orc.tlookup_prove(S, T, B, m, alpha[0], beta, u, v)
     assert st == 0
     table = ops.g1_table_gen(dg[:16].contiguous(), 256)
-    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
-    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
-    tr, sc = host.tlookup_mapping_prove(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
-    assert_same(tr, wtr, "transcript")
-    assert_same(sc, wsc, "S(v)")
-    # a wrong output value is caught
-    S_out2 = S_out.copy()
-    S_out2[5] += 1
-    with pytest.raises(host.HostError, match="tLookup_phase"):
-        host.tlookup_mapping_prove(dSi, ops.fr_from_i32(torch.from_numpy(S_out2).cuda()), D, low, N, fmap, alpha, r, u, v,
-                                   table, 16, 1, 16)
+    with _witness_as(host, ops, fmt) as w:
+        dSi, dSo = w.dev(S_in), w.dev(S_out)
+        tr, sc = host.tlookup_mapping_prove(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
+        assert_same(tr, wtr, "transcript")
+        assert_same(sc, wsc, "S(v)")
+        # a wrong output value is caught
+        S_out2 = S_out.copy()
+        S_out2[5] += 1
+        with pytest.raises(host.HostError, match="tLookup_phase"):
+            host.tlookup_mapping_prove(dSi, w.dev(S_out2), D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
 
 
 def test_tlookup_mapping_pads_11008_rows(ops, host, gens):
