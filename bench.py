@@ -373,7 +373,7 @@ def layer_workload(args):
                    "integer_tensors": ("openings and claim evaluations fold their integer tensors directly (Hyrax::open(const int*), "
                                        "FrTensor::eval_ints) and the lookup provers index and embed their integer witnesses in one pass "
                                        "(tLookupRange::prove(const int*, ...), tLookupRangeMapping::prove(const int*, const int*, ...)): same "
-                                       "proofs; the matmul provers embed their operands with FrTensor::get_data") if not args.no_int_folds else
+                                       "proofs; prove_matmul(const int*, const int*, ...) folds the row variables of its operands from the integers") if not args.no_int_folds else
                                       "every integer tensor is embedded with FrTensor::get_data before its proof step (--no-int-folds)",
                    "wall_breakdown_s": last["wall_breakdown_s"],
                    "provers_only_s": float(np.mean([r["provers_only_s"] for r in runs])),

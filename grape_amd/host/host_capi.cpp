@@ -110,12 +110,16 @@ int grape_host_prove_matmul(const uint32_t* d_A, const uint32_t* d_B, int L, int
                             const uint32_t* v, uint32_t nv, uint32_t* claim_inout, uint32_t* transcript, uint32_t* n_rounds,
                             uint32_t* A_claim, uint32_t* B_claim) {
     GUARD_BEGIN
-    FrTensor A = tensor_from_device(d_A, (uint32_t)(L * N * K));
-    FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * K));
     Fr claim = fr_from(claim_inout);
     SumcheckTranscript tr;
     std::pair<Fr, Fr> res;
-    {
+    if (g_input_format == 1 && g_int_folds) {
+        ProveTimer timer;
+        res = prove_matmul(reinterpret_cast<const int*>(d_A), reinterpret_cast<const int*>(d_B), L, N, M, K, vec_from(u, nu), vec_from(v, nv),
+                           claim, &tr);
+    } else {
+        FrTensor A = tensor_from_device(d_A, (uint32_t)(L * N * K));
+        FrTensor B = tensor_from_device(d_B, (uint32_t)(L * M * K));
         ProveTimer timer;
         res = prove_matmul(A, B, L, N, M, K, vec_from(u, nu), vec_from(v, nv), claim, &tr);
     }

@@ -153,12 +153,33 @@ std::pair<Fr, Fr> prove_matmul(FrTensor& A, FrTensor& B, int L, int N, int M, in
     const uint lu = Log2((uint)L) + Log2((uint)N) + Log2((uint)M);
     if (L < 1 || N < 1 || M < 1 || K < 1 || Log2((uint)(L * N * M)) != lu || u.size() < lu || v.size() < Log2((uint)(L * K)))
         throw std::runtime_error("prove_matmul: Incompatible dimensions");
+    return prove_matmul_impl(&A, &B, nullptr, nullptr, L, N, M, K, u, v, claim, transcript);
+}
+std::pair<Fr, Fr> prove_matmul(const int* device_int_A, const int* device_int_B, int L, int N, int M, int K, const std::vector<Fr> u,
+                               const std::vector<Fr> v, Fr& claim, SumcheckTranscript* transcript) {
+    const uint lu = Log2((uint)L) + Log2((uint)N) + Log2((uint)M);
+    if (L < 1 || N < 1 || M < 1 || K < 1 || Log2((uint)(L * N * M)) != lu || u.size() < lu || v.size() < Log2((uint)(L * K)))
+        throw std::runtime_error("prove_matmul: Incompatible dimensions");
+    return prove_matmul_impl(nullptr, nullptr, device_int_A, device_int_B, L, N, M, K, u, v, claim, transcript);
+}
+// A_in / B_in, or the integer tensors read as FrTensor::get_data would embed them: the folds over the row variables, which
+// read each operand once, then read the integers themselves
+std::pair<Fr, Fr> prove_matmul_impl(FrTensor* A_in, FrTensor* B_in, const int* A_ints, const int* B_ints, int L, int N, int M, int K,
+                                    const std::vector<Fr>& u, const std::vector<Fr>& v, Fr& claim, SumcheckTranscript* transcript) {
     fr_t* U = grape_host::upload(u);
     fr_t* V = grape_host::upload(v);
     std::pair<Fr, Fr> ret;
     try {
-        A.partial_eval(A.size, U, N, Log2(M), K);
-        B.partial_eval(B.size, U, M, 0, K);
+        std::unique_ptr<FrTensor> A_own, B_own;
+        if (A_ints) {
+            A_own.reset(new FrTensor(FrTensor::folded_from_ints(A_ints, (uint)(L * N * K), U, N, Log2(M), K)));
+            B_own.reset(new FrTensor(FrTensor::folded_from_ints(B_ints, (uint)(L * M * K), U, M, 0, K)));
+        } else {
+            A_in->partial_eval(A_in->size, U, N, Log2(M), K);
+            B_in->partial_eval(B_in->size, U, M, 0, K);
+        }
+        FrTensor& A = A_ints ? *A_own : *A_in;
+        FrTensor& B = A_ints ? *B_own : *B_in;
         FrTensor a(1), b(1), c(1);      // the reference's coefficient arrays (src/prove.cu:190-192): not used by the fused rounds
         Fr eq_accumulate = matmul_sumcheck_phase1(A, B, a, b, c, U + Log2(L * N * M), V + Log2(L * K), K, K * L, claim, transcript);
         matmul_sumcheck_phase2(A, B, a, b, c, V + Log2(K), K, claim, eq_accumulate, transcript);

@@ -39,6 +39,12 @@ Fr eleMul_sumcheck(FrTensor& A, FrTensor& B, FrTensor& a, FrTensor& b, FrTensor&
 // v = (k bits | l bits), claim in/out.  Returns (A(v_k,u_n,v_l), B(v_k,u_m,v_l)).
 std::pair<Fr, Fr> prove_matmul(FrTensor& A, FrTensor& B, int L, int N, int M, int K, const std::vector<Fr> u,
                                const std::vector<Fr> v, Fr& claim, SumcheckTranscript* transcript = nullptr);
+// addition: prove_matmul for the tensors FrTensor::get_data would make of the device integers (the reference's drivers embed
+// the operands and prove, test/llm.cu:85-95): the folds over the row variables read the integers
+std::pair<Fr, Fr> prove_matmul(const int* device_int_A, const int* device_int_B, int L, int N, int M, int K, const std::vector<Fr> u,
+                               const std::vector<Fr> v, Fr& claim, SumcheckTranscript* transcript = nullptr);
+std::pair<Fr, Fr> prove_matmul_impl(FrTensor* A, FrTensor* B, const int* A_ints, const int* B_ints, int L, int N, int M, int K,
+                                    const std::vector<Fr>& u, const std::vector<Fr>& v, Fr& claim, SumcheckTranscript* transcript);
 std::pair<Fr, Fr> prove_eleMul(FrTensor& A, FrTensor& B, int L, int M, int N, const std::vector<Fr> u,
                                const std::vector<Fr> v, Fr& claim, SumcheckTranscript* transcript = nullptr);
 Fr combine_claims(FrTensor& X, const std::vector<Fr>& claims, const std::vector<std::vector<Fr>>& u,

@@ -103,6 +103,13 @@ def test_prove_matmul_vs_oracle(ops, host, L, N, M, K):
     assert_same(claim, wclaim, "final claim")
     assert_same(ac, wac, "A(v)")
     assert_same(bc, wbc, "B(v)")
+    # the same proof from the operands as integers (the folds over the rows read them directly)
+    with _witness_as(host, ops, "i32") as w:
+        tr2, claim2, ac2, bc2 = host.prove_matmul(w.dev(A), w.dev(B), L, N, M, K, u, v, claim0)
+    assert_same(tr2, wtr, "integer operands: transcript")
+    assert_same(claim2, wclaim, "integer operands: final claim")
+    assert_same(ac2, wac, "integer operands: A(v)")
+    assert_same(bc2, wbc, "integer operands: B(v)")
 
 
 @pytest.mark.parametrize("K", [4, 1 << 17])      # the long case starts with a round that takes its middle coefficient from the claim
