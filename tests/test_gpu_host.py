@@ -132,13 +132,15 @@ def test_mle_eval_operator(ops, host):
     assert_same(host.mle_eval(ops.to_dev(t), 2 * 11008, u), orc.mle_eval(t, u), "T(u), 11008 columns")
 
 
-@pytest.mark.parametrize("fmt", ["fr", "i32"])
-@pytest.mark.parametrize("indexed", [True, False])
-@pytest.mark.parametrize("logD,logN,low", [(4, 2, -2), (5, 3, -4), (3, 3, 0), (12, 6, -32), (14, 8, -128), (16, 16, -32768)])
+_RANGE_SHAPES = [(4, 2, -2), (5, 3, -4), (3, 3, 0), (12, 6, -32), (14, 8, -128), (16, 16, -32768)]
+
+
+# every shape with the witness as a field tensor; four of them again with the witness handed over as integers
+@pytest.mark.parametrize("logD,logN,low,indexed,fmt",
+                         [s + (i, "fr") for s in _RANGE_SHAPES for i in (True, False)] +
+                         [s + (i, "i32") for s in _RANGE_SHAPES if s[0] not in (5, 14) for i in (True, False)])
 def test_tlookup_range_prove_vs_oracle(ops, host, gens, logD, logN, low, indexed, fmt):
     import torch
-    if fmt == "i32" and logD in (5, 14):
-        pytest.skip("the integer-witness path is covered at the other sizes")
     host.set_indexed_commit(indexed)
     hg, dg = gens
     D, N = 1 << logD, 1 << logN
