@@ -703,8 +703,29 @@ Fr tLookupRange::prove(FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax
 Fr tLookupRange::prove(const int* device_int_S, FrTensor& S, FrTensor& A, const std::vector<Fr>& v, Hyrax& hyrax, uint msm_size,
                        double& commit_time) {
     const uint D = S.size;
-    if (!(D == (1u << Log2(D)) && A.size >= D)) {
-        // a witness that needs padding goes the ordinary way
+    const uint Dp = 1u << Log2(D);
+    if (D != Dp && D % 11008 == 0 && (uint64_t)(D / 11008) * 16384 <= Dp && low <= 0 && (int64_t)low + (int64_t)T.size > 0 && A.size >= Dp &&
+        S.capacity() >= Dp) {
+        // rows of 11008 (src/tlookup.cu:299-305): the INTEGERS are padded to rows of 16384 with zeros - the witness the reference
+        // proves after its own padding, whose multiplicities are those of the unpadded one plus the padding's zeros
+        // (:276-281) - and proved as a witness that needs none
+        int* padded = nullptr;
+        check(grape_malloc((void**)&padded, sizeof(int) * (size_t)Dp), "grape_malloc");
+        Fr ret;
+        try {
+            check(grape_i32_pad(padded, device_int_S, 11008, 16384, Dp, nullptr), "grape_i32_pad");
+            S.set_size(Dp);
+            ret = prove(padded, S, A, v, hyrax, msm_size, commit_time);
+        } catch (...) {
+            grape_stream_sync(nullptr);
+            grape_free(padded);
+            throw;
+        }
+        grape_free(padded);
+        return ret;
+    }
+    if (!(D == Dp && A.size >= D)) {
+        // any other witness that needs padding goes the ordinary way
         S.get_data(D, const_cast<int*>(device_int_S));
         return prove(S, A, v, hyrax, msm_size, commit_time);
     }
@@ -739,6 +760,8 @@ void tLookupRangeMapping::init_from_host(const int* host_table, uint len) {
     check(grape_stream_sync(nullptr), "sync");
     grape_free(d_map_int_);
     d_map_int_ = d_int;                   // kept: a witness handed over as integers is checked against it
+    have_map_zero_ = low <= 0 && (int64_t)low + (int64_t)len > 0;
+    map_zero_ = have_map_zero_ ? host_table[-low] : 0;
 }
 tLookupRangeMapping::~tLookupRangeMapping() { grape_free(d_map_int_); }
 
@@ -795,7 +818,29 @@ Fr tLookupRangeMapping::prove(FrTensor& S_in, FrTensor& S_out, FrTensor& A, cons
 
 Fr tLookupRangeMapping::prove(const int* device_int_S_in, const int* device_int_S_out, uint D, FrTensor& A, const std::vector<Fr>& v,
                               Hyrax& hyrax, uint msm_size, double& commit_time) {
-    if (!(D == (1u << Log2(D)) && A.size >= D)) {
+    const uint Dp = 1u << Log2(D);
+    if (D != Dp && D % 11008 == 0 && (uint64_t)(D / 11008) * 16384 <= Dp && have_map_zero_ && A.size >= Dp) {
+        // rows of 11008: both integer tensors are padded to rows of 16384 with the pair (0, f(0)) the reference pads with
+        // (src/tlookup.cu:411-420) and proved as a witness that needs no padding
+        int *pin = nullptr, *pout = nullptr;
+        Fr ret;
+        try {
+            check(grape_malloc((void**)&pin, sizeof(int) * (size_t)Dp), "grape_malloc");
+            check(grape_malloc((void**)&pout, sizeof(int) * (size_t)Dp), "grape_malloc");
+            check(grape_i32_pad(pin, device_int_S_in, 11008, 16384, Dp, nullptr), "grape_i32_pad");
+            check(grape_i32_pad_fill(pout, device_int_S_out, 11008, 16384, Dp, map_zero_, nullptr), "grape_i32_pad_fill");
+            ret = prove(pin, pout, Dp, A, v, hyrax, msm_size, commit_time);
+        } catch (...) {
+            grape_stream_sync(nullptr);
+            grape_free(pin);
+            grape_free(pout);
+            throw;
+        }
+        grape_free(pin);
+        grape_free(pout);
+        return ret;
+    }
+    if (!(D == Dp && A.size >= D)) {
         FrTensor S_in(D, const_cast<int*>(device_int_S_in)), S_out(D, const_cast<int*>(device_int_S_out));
         return prove(S_in, S_out, A, v, hyrax, msm_size, commit_time);
     }

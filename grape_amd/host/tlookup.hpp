@@ -140,6 +140,8 @@ public:
 private:
     void init_from_host(const int* host_table, uint len);
     int* d_map_int_ = nullptr;          // the table's second components as integers (for witnesses handed over as integers)
+    bool have_map_zero_ = false;        // 0 is a table key ...
+    int map_zero_ = 0;                  // ... and this its image f(0): the pair a padded witness is filled with
 };
 
 // The round-by-round form of the logUp sumcheck, as the reference exposes it

@@ -241,7 +241,8 @@ def test_tlookup_mapping_prove_vs_oracle(ops, host, gens, fmt):
             host.tlookup_mapping_prove(dSi, w.dev(S_out2), D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
 
 
-def test_tlookup_mapping_pads_11008_rows(ops, host, gens):
+@pytest.mark.parametrize("fmt", ["fr", "i32"])
+def test_tlookup_mapping_pads_11008_rows(ops, host, gens, fmt):
     # mapping lookup of 2 x 11008 pairs: padded to 2 x 16384 with the pair (0, f(0)), counted in m
     import torch
     hg, dg = gens
@@ -261,9 +262,8 @@ def test_tlookup_mapping_pads_11008_rows(ops, host, gens):
     st, wtr, wsc = orc.tlookup_prove(Spad, T, B, m, alpha[0], beta, u, v)
     assert st == 0
     table = ops.g1_table_gen(dg[:16].contiguous(), 256)
-    dSi = ops.fr_from_i32(torch.from_numpy(S_in).cuda())
-    dSo = ops.fr_from_i32(torch.from_numpy(S_out).cuda())
-    tr, sc = host.tlookup_mapping_prove(dSi, dSo, D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
+    with _witness_as(host, ops, fmt) as w:
+        tr, sc = host.tlookup_mapping_prove(w.dev(S_in), w.dev(S_out), D, low, N, fmap, alpha, r, u, v, table, 16, 1, 16)
     assert_same(tr, wtr, "transcript")
     assert_same(sc, wsc, "S(v)")
 
