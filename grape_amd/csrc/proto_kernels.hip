@@ -507,29 +507,52 @@ __global__ void __launch_bounds__(kBlock) index_inverse_kernel(int32_t* idx1, ui
 // S[i] = key_i + r * cmp_i (the combined witness, src/tlookup.cu:407-410) for a mapping lookup, whose table of second
 // components is an integer table too.  8 bytes per element are read where embedding two tensors, indexing them and
 // combining them move 270.
+constexpr int kEmbedPerThread = 4;
 __global__ void __launch_bounds__(kBlock) index_embed_i32_kernel(int32_t* idx1, uint32_t* A, uint32_t* S, const int32_t* __restrict__ key,
                                                                   const int32_t* __restrict__ cmp, size_t n, int32_t low, uint32_t len,
                                                                   const uint32_t* B, const int32_t* __restrict__ cmp_table, const uint32_t* r,
                                                                   unsigned int* mismatches) {
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    bool bad = false;
-    if (i < n) {
-        const int32_t k = key[i];
-        const int64_t d = (int64_t)k - (int64_t)low;
-        const bool inside = d >= 0 && d < (int64_t)len;
-        idx1[i] = inside ? (int32_t)(d + 1) : 0;
-        bad = !inside;
-        Fr s = fr26::from_i32c(k);
-        if (cmp) {
-            const int32_t c = cmp[i];
-            if (inside) bad = c != cmp_table[d];
-            s = add(s, fr26::mulc(fr26::from_i32c(c), ld_fr(r, 0)));
+    // The witness element is ONE reduction of a two-term sum of plain integers against constants that carry the factors:
+    // key * W + cmp * Wr with W = 16 * 2^512 and Wr = 16 * r * 2^512 (mod the modulus) reduces to (key + r * cmp) * 2^256,
+    // the memory form.  An integer is two signed limbs, so a term is 20 multiply-adds.
+    const fr26::Limbs w = fr26::weight16(Fr::rr());
+    fr26::Limbs wr;
+    if (cmp) wr = fr26::weight16(fr26::mulc(ld_fr(r, 0), Fr::rr()));
+    auto mac_int = [](fr26::Acc& C, const fr26::Limbs& x, int32_t v) {
+        const int64_t l0 = (int64_t)(v & (int32_t)fr26::MASK), l1 = (int64_t)(v >> fr26::W);
+#pragma unroll
+        for (int j = 0; j < fr26::N; j++) {
+            C.c[j] += (int64_t)x.v[j] * l0;
+            C.c[j + 1] += (int64_t)x.v[j] * l1;
         }
-        st_fr(S, i, s);
-        if (!bad && A) st_fr(A, i, ld_fr(B, (size_t)d));
+    };
+    const size_t base = (size_t)blockIdx.x * (kBlock * kEmbedPerThread) + threadIdx.x;
+    unsigned int nbad = 0;
+#pragma unroll
+    for (int q = 0; q < kEmbedPerThread; q++) {
+        const size_t i = base + (size_t)q * kBlock;
+        bool bad = false;
+        if (i < n) {
+            const int32_t k = key[i];
+            const int64_t d = (int64_t)k - (int64_t)low;
+            const bool inside = d >= 0 && d < (int64_t)len;
+            idx1[i] = inside ? (int32_t)(d + 1) : 0;
+            bad = !inside;
+            fr26::Acc C;
+            fr26::acc_zero(C);
+            mac_int(C, w, k);
+            if (cmp) {
+                const int32_t c = cmp[i];
+                if (inside) bad = c != cmp_table[d];
+                mac_int(C, wr, c);
+            }
+            // |sum| < 2^32 * modulus: the reduced value plus one modulus lies in [0, 2 * modulus)
+            st_fr(S, i, fr26::unpack(fr26::canon(fr26::reduce(C, 1), 1)));
+            if (!bad && A) st_fr(A, i, ld_fr(B, (size_t)d));
+        }
+        nbad += (unsigned int)__popcll(__ballot(bad));
     }
-    const unsigned long long b = __ballot(bad);
-    if (b != 0ull && (threadIdx.x & 63) == 0) atomicAdd(mismatches, (unsigned int)__popcll(b));
+    if (nbad != 0 && (threadIdx.x & 63) == 0) atomicAdd(mismatches, nbad);
 }
 
 // out[i] = (v_i - low) + 1 for an in-range value, 0 otherwise
@@ -1026,7 +1049,8 @@ int grape_tlookup_index_embed_i32_nowait(int32_t* idx1, uint32_t* A, uint32_t* S
     if (A) { CHECK_PTR16(A); CHECK_PTR16(B); }       // A == nullptr: no logUp tensor written
     GRAPE_REQUIRE((cmp == nullptr) == (cmp_table == nullptr) && (cmp == nullptr) == (r == nullptr), "cmp, cmp_table and r go together");
     if (r) CHECK_PTR16(r);
-    index_embed_i32_kernel<<<blocks_for(n), kBlock, 0, s>>>(idx1, A, S, key, cmp, n, low, len, B, cmp_table, r, (unsigned int*)d_mismatches);
+    index_embed_i32_kernel<<<blocks_for(n, kBlock * kEmbedPerThread), kBlock, 0, s>>>(idx1, A, S, key, cmp, n, low, len, B, cmp_table, r,
+                                                                                     (unsigned int*)d_mismatches);
     GRAPE_LAUNCH_CHECK();
     return GRAPE_OK;
 }
