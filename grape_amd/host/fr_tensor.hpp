@@ -76,12 +76,12 @@ public:
 
     static FrTensor random(uint size);
 
-    // additions: host <-> device transfer of whole tensors
     // additions: an integer tensor folded or evaluated as the tensor get_data would make of it, without making
     // it (the first pass reads the integers): partial_eval(N, x, c, id, gap) of that tensor, compacted, and
     // operator()(u) for a power-of-two size
     static FrTensor folded_from_ints(const int* device_int_data, uint N, fr_t* x, uint c, uint id, uint gap);
     static Fr eval_ints(const int* device_int_data, uint size, const std::vector<Fr>& u);
+    // additions: host <-> device transfer of whole tensors
     static FrTensor from_host(const std::vector<Fr>& v);
     std::vector<Fr> to_host() const;
     uint capacity() const { return capacity_; }
