@@ -54,7 +54,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch read from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # same counter reads for the 1 GiB copy kernel below); the counters cannot be read from inside this
 # process, so these are the figures of the committed counter summary of this same command.
-COMMIT_KERNEL_TRAFFIC_BYTES = 2.626e9
+COMMIT_KERNEL_TRAFFIC_BYTES = 2.627e9
 FOLD_KERNEL_TRAFFIC_BYTES = 1.110e9
 
 
@@ -1063,7 +1063,7 @@ def main():
     ops.profile_enable(False)
     fold_pass_ms = float(np.median(fold_ms))
     fold_bytes = 32.0 * n_fold                                   # every element read once (writes: 1/32 more, not counted)
-    roofline_streaming = {"bound": "hbm", "kernel": "fold_pass_kernel<1> (first pass of grape_fr_fold, c=64)",
+    roofline_streaming = {"bound": "hbm", "kernel": "fold_pass_kernel<1, false> (first pass of grape_fr_fold, c=64)",
                           "achieved": fold_bytes / (fold_pass_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                           "frac": fold_bytes / (fold_pass_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": FOLD_KERNEL_TRAFFIC_BYTES,
                           "kernel_ms": fold_pass_ms, "elements": n_fold}

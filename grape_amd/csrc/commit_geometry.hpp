@@ -14,10 +14,12 @@ constexpr int kPartialWords = 64;      // one lane's partial accumulator: 256 by
 constexpr int kWaveLanes = 64;
 constexpr size_t kSlabSegments = 32768;   // row segments per launch: 512 MiB of partial sums
 
-// Lanes that share a row in the row-reduction kernel: 8 when rows alone fill the chip (measured best
-// for 4096 rows of 64 partials: 4 lanes +6 %, 16 +33 %, 32 +65 % - idle lanes of the tree steps cost
+// Lanes that share a row in the one-wave row-reduction kernel: 8 when rows alone fill the chip (measured
+// best for 4096 rows of 64 partials: 4 lanes +6 %, 16 +33 %, 32 +65 % - idle lanes of the tree steps cost
 // more than shorter chains save), up to a whole wave when rows are few and the chain per lane is
-// what takes the time (one row of 32768 partials: 150 ms with 8 lanes).
+// what takes the time (one row of 32768 partials: 150 ms with 8 lanes).  With 512 rows and more (a value
+// below 6) a call that waits for its result takes the four-wave kernel instead, which hands partial sums
+// between waves through LDS (tree_row / tree_share below); the value still bounds the column segments of a row.
 GRAPE_HD uint32_t reduce_lanes_log2(size_t rows) {
     if (rows >= 2048) return 3;
     if (rows >= 1024) return 4;
@@ -72,6 +74,13 @@ GRAPE_HD size_t table_entry(uint32_t w, uint32_t K, uint32_t mag, size_t N, uint
 GRAPE_HD size_t partial_word(size_t i) { return (size_t)kPartialWords * i; }
 // reduction kernel: row of lane `lane` of workgroup `block`
 GRAPE_HD size_t reduce_row(size_t block, int lane, uint32_t lg_lpr) { return block * (size_t)(kWaveLanes >> lg_lpr) + (size_t)(lane >> lg_lpr); }
+// four-wave reduction kernel: a workgroup of 256 threads takes kTreeRows rows, 32 lanes a row; thread t works
+// on row tree_row(block, t) and starts from partial sums tree_share(t), tree_share(t) + 32, ... of that row
+constexpr int kTreeRows = 8;
+constexpr int kTreeThreads = 256;
+GRAPE_HD size_t tree_row(size_t block, int t) { return block * (size_t)kTreeRows + (size_t)(t & (kTreeRows - 1)); }
+GRAPE_HD uint32_t tree_share(int t) { return (uint32_t)t >> 3; }
+GRAPE_HD bool tree_reduction(uint32_t lg_lpr, uint32_t nparts) { return lg_lpr <= 5 && nparts <= 4096; }
 // workgroups of a launch of `threads` threads in groups of `per_block`
 GRAPE_HD size_t blocks_needed(size_t threads, size_t per_block) { return (threads + per_block - 1) / per_block; }
 

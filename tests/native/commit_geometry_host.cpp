@@ -70,6 +70,25 @@ extern "C" long long commit_geometry_check(size_t size, uint32_t rowlen, size_t 
         ck.le("reduction grid (workgroups)", rblocks, 0x7fffffffull);
         ck.le("reduction grid (threads)", rblocks * 64, 0xffffffffull);
         const uint32_t nparts = plan.nseg * 64;
+        if (geom::tree_reduction(plan.lg_lpr, nparts)) {
+            // four-wave kernel (calls that wait for their result): every thread's row and the last partial sum of its share
+            const size_t tblocks = (nr + geom::kTreeRows - 1) / geom::kTreeRows;
+            ck.le("tree reduction grid (workgroups)", tblocks, 0x7fffffffull);
+            for (size_t b = 0; b < tblocks; b++) {
+                for (int t = 0; t < geom::kTreeThreads; t++) {
+                    const size_t row = geom::tree_row(b, t);
+                    if (row >= nr) continue;
+                    const uint32_t share = geom::tree_share(t);
+                    ck.lt("share of a thread", share, 32);
+                    if (share >= nparts) continue;
+                    const uint32_t last = share + ((nparts - 1 - share) / 32) * 32;
+                    ck.lt("partial sum of a row", last, nparts);
+                    ck.lt("partial word (load)", geom::partial_word(row * nparts + last) + geom::kPartialWords - 1, partial_words);
+                    ck.lt("output word", (r0 + row + 1) * point_words - 1, out_words);
+                }
+            }
+        }
+        // one-wave kernel (queued calls, and every call with few rows)
         for (size_t b = 0; b < rblocks; b++) {
             for (int lane = 0; lane < 64; lane++) {
                 const size_t row = geom::reduce_row(b, lane, plan.lg_lpr);

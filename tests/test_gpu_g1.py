@@ -178,6 +178,37 @@ def test_commitments_queued_on_three_streams(ops, gens64):
             ops.stream_destroy(h)
 
 
+@pytest.mark.parametrize("rows,n", [(515, 64), (600, 256), (1100, 128), (2051, 64), (4100, 256)])
+def test_waiting_and_queued_commitments_agree(ops, rows, n):
+    """with 512 rows and more a call that waits for its result (grape_commit_i32) and a queued one
+    (grape_commit_i32_nowait) take different row reductions - four waves per eight rows with partial sums handed
+    on through LDS, one wave per eight to two rows - over 64 to 256 partial sums per row: the same affine points
+    bit for bit, and the oracle's"""
+    import torch
+    k = _scalars(n, 300 + n)
+    host = orc.g1_make_generators(k)
+    dev = ops.g1_make_generators(k)
+    wide = ops.g1_wide_table_gen(dev, 8, 1, 128)
+    rng = np.random.default_rng(rows * 7 + n)
+    m = rng.integers(-100, 101, size=(rows, n), dtype=np.int32)
+    m[3] = 0                                   # a row that sums to the identity
+    m[5, 1:] = 0                               # a row of one term
+    d = torch.from_numpy(m).cuda()
+    waited = ops.g1_to_host(ops.commit_i32(d, n, wide, n, 8, 1, 128))
+    h = ops.stream_create()
+    out = ops.g1_empty(rows)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    try:
+        ops.commit_i32_nowait(d, n, wide, n, 8, 1, 128, out, flag, h)
+        ops.stream_sync(h)
+    finally:
+        ops.stream_destroy(h)
+    assert flag.tolist() == [0]
+    assert_same(ops.g1_to_host(out), waited, "queued against waiting")
+    assert_same(waited, orc.commit_i32(m, orc.g1_table(host, 256), n, n), "against the oracle")
+
+
 def test_commit_int16_fast_path(ops, gens64):
     import torch
     k, host, dev = gens64
