@@ -80,7 +80,10 @@ constexpr int kTreeRows = 8;
 constexpr int kTreeThreads = 256;
 GRAPE_HD size_t tree_row(size_t block, int t) { return block * (size_t)kTreeRows + (size_t)(t & (kTreeRows - 1)); }
 GRAPE_HD uint32_t tree_share(int t) { return (uint32_t)t >> 3; }
-GRAPE_HD bool tree_reduction(uint32_t lg_lpr, uint32_t nparts) { return lg_lpr <= 5 && nparts <= 4096; }
+// taken for 512 to 4096 rows: up to 512 workgroups, which the chip holds all at once (two per compute unit) - with more
+// rows the waves that idle at the kernel's barriers keep later workgroups out, and the one-wave kernel is faster
+// (32 768 rows: 0.8 against 1.5 ms)
+GRAPE_HD bool tree_reduction(size_t rows, uint32_t lg_lpr, uint32_t nparts) { return lg_lpr <= 5 && rows <= 4096 && nparts <= 4096; }
 // workgroups of a launch of `threads` threads in groups of `per_block`
 GRAPE_HD size_t blocks_needed(size_t threads, size_t per_block) { return (threads + per_block - 1) / per_block; }
 

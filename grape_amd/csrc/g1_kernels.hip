@@ -1043,7 +1043,7 @@ static void launch_reduce(uint32_t* out, const uint32_t* partial, size_t rows, u
     // chain is the gain (0.29 against 0.35 ms for 4096 rows of 64).  Beside other kernels it is the loss: its
     // waves hold half as many wave slots again while they wait at the barriers, and a commitment queued
     // behind this one runs slower for it (three streams of 4096 x 4096 commitments: 6220 against 6550 Mpoints/s)
-    if (alone && geom::tree_reduction(lg_lpr, nparts)) {
+    if (alone && geom::tree_reduction(rows, lg_lpr, nparts)) {
         commit_reduce_tree_kernel<AFFINE><<<(unsigned)((rows + kTreeRows - 1) / kTreeRows), geom::kTreeThreads, 0, s>>>(out, partial, rows, nparts);
         return;
     }

@@ -70,7 +70,7 @@ extern "C" long long commit_geometry_check(size_t size, uint32_t rowlen, size_t 
         ck.le("reduction grid (workgroups)", rblocks, 0x7fffffffull);
         ck.le("reduction grid (threads)", rblocks * 64, 0xffffffffull);
         const uint32_t nparts = plan.nseg * 64;
-        if (geom::tree_reduction(plan.lg_lpr, nparts)) {
+        if (geom::tree_reduction(nr, plan.lg_lpr, nparts)) {
             // four-wave kernel (calls that wait for their result): every thread's row and the last partial sum of its share
             const size_t tblocks = (nr + geom::kTreeRows - 1) / geom::kTreeRows;
             ck.le("tree reduction grid (workgroups)", tblocks, 0x7fffffffull);

@@ -178,9 +178,9 @@ def test_commitments_queued_on_three_streams(ops, gens64):
             ops.stream_destroy(h)
 
 
-@pytest.mark.parametrize("rows,n", [(515, 64), (600, 256), (1100, 128), (2051, 64), (4100, 256)])
+@pytest.mark.parametrize("rows,n", [(515, 64), (600, 256), (1100, 128), (2051, 64), (4096, 256)])
 def test_waiting_and_queued_commitments_agree(ops, rows, n):
-    """with 512 rows and more a call that waits for its result (grape_commit_i32) and a queued one
+    """with 512 to 4096 rows a call that waits for its result (grape_commit_i32) and a queued one
     (grape_commit_i32_nowait) take different row reductions - four waves per eight rows with partial sums handed
     on through LDS, one wave per eight to two rows - over 64 to 256 partial sums per row: the same affine points
     bit for bit, and the oracle's"""
